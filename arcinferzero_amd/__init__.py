@@ -1,0 +1,10 @@
+"""MI355X-native GGUF block-quantized matmul (prefill GEMM, decode GEMV, MoE grouped GEMM) behind a C ABI.
+
+The compute path is the in-tree shared library ``libarcz_hip.so`` (hand-written HIP for gfx950 plus the C++ host
+dispatch); this package is a thin ctypes binding over ``include/arcz_hip.h`` and ``include/arcz_engine.h`` with numpy
+in and out.  There is no fallback: if the library is missing, importing :mod:`arcinferzero_amd.binding` raises.
+"""
+from .binding import (  # noqa: F401
+    Q4_K, Q6_K, Q8_0, ArczError, Buffer, Engine, Runtime, Weight, MoeLayer, gen_normal, gen_weights, gguf_bytes,
+    lib, lib_path, planes_bytes, quantize_rows, repack_planes,
+)

@@ -1,0 +1,114 @@
+// C ABI of include/arcz_engine.h over the Engine class (engine_hip.h).
+#include "../../include/arcz_engine.h"
+
+#include <string>
+
+#include "engine_hip.h"
+
+struct arcz_engine { Engine* e; };
+struct arcz_weight { GpuWeight w; };
+struct arcz_moe_layer { Engine::MoeLayer L; };
+
+namespace {
+std::string g_err;
+template <class F> int guarded(F&& f) {
+  try {
+    f();
+    return ARCZ_OK;
+  } catch (const std::exception& ex) {
+    g_err = ex.what();
+    fprintf(stderr, "arcz engine: %s\n", ex.what());
+    return ARCZ_E_ENGINE;
+  }
+}
+}  // namespace
+
+extern "C" {
+
+const char* arcz_engine_error(void) { return g_err.c_str(); }
+
+arcz_engine* arcz_engine_create(int max_chunk, int max_k) {
+  Engine* e = nullptr;
+  if (guarded([&] { e = new Engine(max_chunk, max_k); }) != ARCZ_OK) return nullptr;
+  return new arcz_engine{e};
+}
+void arcz_engine_destroy(arcz_engine* e) {
+  if (!e) return;
+  guarded([&] { delete e->e; });
+  delete e;
+}
+
+arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, const void* gguf, size_t bytes) {
+  arcz_weight* w = new arcz_weight;
+  if (guarded([&] { w->w = e->e->make_weight(type, (const uint8_t*)gguf, bytes, N, K); }) != ARCZ_OK) {
+    delete w;
+    return nullptr;
+  }
+  return w;
+}
+int arcz_weight_free(arcz_engine* e, arcz_weight* w) {
+  if (!w) return ARCZ_OK;
+  const int r = guarded([&] { e->e->free_weight(w->w); });
+  delete w;
+  return r;
+}
+arcz_mem* arcz_weight_raw(const arcz_weight* w) { return w ? w->w.raw : nullptr; }
+
+int arcz_engine_quantize(arcz_engine* e, arcz_mem* x, int ldx, int K, int Mp, int T, int act32) {
+  return guarded([&] { e->e->quantize_rows(x, ldx, K, Mp, T, act32); });
+}
+int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp,
+                                int T) {
+  return guarded([&] { e->e->set_activations(aq, asc, absum, K, Mp, T); });
+}
+arcz_mem* arcz_engine_aq(arcz_engine* e) { return e->e->aq_; }
+arcz_mem* arcz_engine_asc(arcz_engine* e) { return e->e->asc_; }
+arcz_mem* arcz_engine_absum(arcz_engine* e) { return e->e->absum_; }
+
+int arcz_engine_matmul(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off, int acc,
+                       int act32) {
+  return guarded([&] {
+    if (!w) throw std::runtime_error("matmul: no weight");
+    e->e->matmul(name ? name : "matmul", w->w, Mp, C, ldc, c_off, acc, act32 != 0);
+  });
+}
+
+arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, const void* up, const void* down,
+                                      int NE, int NU, int E, int F) {
+  arcz_moe_layer* L = new arcz_moe_layer;
+  if (guarded([&] {
+        L->L = e->e->make_moe_layer(type, (const uint8_t*)gate, (const uint8_t*)up, (const uint8_t*)down, NE, NU, E, F);
+      }) != ARCZ_OK) {
+    delete L;
+    return nullptr;
+  }
+  return L;
+}
+int arcz_engine_layer_moe(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp) {
+  return guarded([&] { e->e->layer_moe(L->L, logits, ldl, x, T, Mp); });
+}
+int arcz_engine_moe_route(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, int T, int tm) {
+  return guarded([&] { e->e->moe_route(L->L, logits, ldl, T, tm); });
+}
+arcz_mem* arcz_engine_moe_buffer(arcz_engine* e, int which) {
+  Engine& E = *e->e;
+  cl_mem b[12] = {E.mids_, E.mwts_, E.moffs_, E.mtiles_, E.mtstart_, E.stok_, E.swt_, E.minv_, E.mh_, E.mhq_, E.mhsc_, E.my_};
+  return which >= 0 && which < 12 ? b[which] : nullptr;
+}
+int arcz_engine_moe_slots(arcz_engine* e) { return e->e->slots_; }
+
+void arcz_engine_profile(arcz_engine* e, int on) { e->e->profile = on != 0; }
+int arcz_engine_profile_collect(arcz_engine* e) {
+  return guarded([&] { e->e->collect_profile(); });
+}
+int arcz_engine_profile_get(arcz_engine* e, const char* name, double* ms, int* launches) {
+  auto it = e->e->prof_ms.find(name);
+  if (it == e->e->prof_ms.end()) return -1;
+  if (ms) *ms = it->second;
+  if (launches) *launches = e->e->prof_n[name];
+  return ARCZ_OK;
+}
+void arcz_engine_profile_reset(arcz_engine* e) { e->e->prof_ms.clear(); e->e->prof_n.clear(); }
+uint64_t arcz_engine_rd_bytes(arcz_engine* e) { return e->e->rd_bytes; }
+
+}  // extern "C"

@@ -1,0 +1,261 @@
+// Host-side helpers of the library that need no GPU: the regrouping of GGUF rows into the device planes (the place of
+// the reference's gpu_raw_sb / upload_padded, src/quants.h:728-761, zero/engine_load.h:84-130), the f32 -> Q8_0 row
+// quantizer the reference uses for small f32 matrices (src/quants.h:429-442), and the seeded generators of synthetic
+// tensors (weights ~ N(0, 0.02) quantized to Q4_K / Q6_K / Q8_0, activations ~ N(0, 1)) that the benchmark and the
+// tests share.  The Q4_K / Q6_K quantizers have no counterpart in the reference (it only reads those types): they
+// make valid blocks from random values and are input generators, not part of the compute path.
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "kernels/common.h"
+
+namespace {
+
+// IEEE binary16 conversions, round to nearest even, subnormals kept (the reference's own are src/quants.h:17-52)
+float f16_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1Fu, m = h & 0x3FFu, bits;
+  if (e == 0) {
+    if (m == 0) bits = sign;
+    else {
+      int ex = 113;
+      while (!(m & 0x400u)) { m <<= 1; --ex; }
+      bits = sign | ((uint32_t)ex << 23) | ((m & 0x3FFu) << 13);
+    }
+  } else if (e == 31) bits = sign | 0x7F800000u | (m << 13);
+  else bits = sign | ((e + 112) << 23) | (m << 13);
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+uint16_t f32_to_f16(float x) {
+  uint32_t f;
+  memcpy(&f, &x, 4);
+  const uint32_t sign = (f >> 16) & 0x8000u, e8 = (f >> 23) & 0xFFu;
+  uint32_t mant = f & 0x7FFFFFu;
+  const int e = (int)e8 - 112;
+  if (e8 == 0xFF) return (uint16_t)(sign | 0x7C00u | (mant ? 0x200u : 0u));
+  if (e >= 31) return (uint16_t)(sign | 0x7C00u);
+  if (e <= 0) {
+    if (e < -10) return (uint16_t)sign;
+    mant |= 0x800000u;
+    const uint32_t shift = (uint32_t)(14 - e);
+    uint32_t h = mant >> shift;
+    const uint32_t rem = mant & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (h & 1u))) ++h;
+    return (uint16_t)(sign | h);
+  }
+  uint32_t h = sign | ((uint32_t)e << 10) | (mant >> 13);
+  const uint32_t rem = mant & 0x1FFFu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;
+  return (uint16_t)h;
+}
+
+inline uint64_t splitmix64(uint64_t& s) {
+  uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
+  const size_t u = rows * (size_t)(K / 256);
+  return type == QT_Q4_K ? u * 144 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : 0;
+}
+size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) { return raw_planes_bytes((int)type, rows, K / 256); }
+
+// GGUF rows -> device planes (layout: kernels/common.h).  0 or -1 (unsupported type / K).
+int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, uint8_t* dst) {
+  if (K <= 0 || K % 256) return -1;
+  const int nsb = K / 256;
+  const int64_t u = (int64_t)rows * nsb;
+  if (type == QT_Q4_K) {
+    const PlanesQ4K pl = planes_q4k(rows, nsb);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i) {
+      memcpy(dst + pl.hdr + i * 16, src + i * 144, 16);
+      memcpy(dst + pl.qs + i * 128, src + i * 144 + 16, 128);
+    }
+    return 0;
+  }
+  if (type == QT_Q6_K) {
+    const PlanesQ6K pl = planes_q6k(rows, nsb);
+    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_Q6_K, rows, nsb) - (pl.d + u * 2));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i) {
+      memcpy(dst + pl.ql + i * 128, src + i * 210, 128);
+      memcpy(dst + pl.qh + i * 64, src + i * 210 + 128, 64);
+      memcpy(dst + pl.sc + i * 16, src + i * 210 + 192, 16);
+      memcpy(dst + pl.d + i * 2, src + i * 210 + 208, 2);
+    }
+    return 0;
+  }
+  if (type == QT_Q8_0) {
+    const PlanesQ80 pl = planes_q80(rows, nsb);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i)
+      for (int b = 0; b < 8; ++b) {
+        memcpy(dst + pl.d + i * 16 + 2 * b, src + i * 272 + 34 * b, 2);
+        memcpy(dst + pl.qs + i * 256 + 32 * b, src + i * 272 + 34 * b + 2, 32);
+      }
+    return 0;
+  }
+  return -1;
+}
+
+// n values ~ N(mean, std): SplitMix64 -> two uniforms -> Box-Muller in f32, element i from the stream position i / 2
+// (so any sub-range can be generated alone).  The same seed gives the same tensor on every machine.
+void arcz_gen_normal(uint64_t seed, size_t n, float mean, float std, float* out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t p = 0; p < (int64_t)((n + 1) / 2); ++p) {
+    uint64_t s = seed * 0xD1342543DE82EF95ull + (uint64_t)p * 0x9E3779B97F4A7C15ull * 2;
+    const uint64_t a = splitmix64(s), b = splitmix64(s);
+    const float u1 = ((float)((a >> 40) + 1)) * (1.0f / 16777216.0f);  // (0, 1]
+    const float u2 = (float)(b >> 40) * (1.0f / 16777216.0f);          // [0, 1)
+    const float r = sqrtf(-2.0f * logf(u1)), th = 6.28318530717958647692f * u2;
+    out[2 * p] = mean + std * r * cosf(th);
+    if ((size_t)(2 * p + 1) < n) out[2 * p + 1] = mean + std * r * sinf(th);
+  }
+}
+
+// f32 rows [N][K] -> GGUF Q8_0 (34-byte blocks): d = amax / 127 kept as fp16, q = rte(v * (1 / d)) with the f32 d
+// (reference src/quants.h:429-442).
+void arcz_quantize_q8_0(const float* src, size_t N, int K, uint8_t* out) {
+  const int64_t nb = (int64_t)N * (K / 32);
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < nb; ++b) {
+    const float* v = src + b * 32;
+    float amax = 0;
+    for (int i = 0; i < 32; ++i) amax = std::fmax(amax, std::fabs(v[i]));
+    const float d = amax / 127.0f, inv = d > 0 ? 1.0f / d : 0.0f;
+    uint8_t* blk = out + b * 34;
+    const uint16_t dh = f32_to_f16(d);
+    memcpy(blk, &dh, 2);
+    for (int i = 0; i < 32; ++i) blk[2 + i] = (uint8_t)(int8_t)std::lrintf(v[i] * inv);
+  }
+}
+
+// f32 rows -> GGUF Q4_K superblocks (144 bytes per 256 values).  Per 32-block: offset lo = min(v, 0), step
+// (max - lo) / 15; the eight steps and offsets are rounded to 6 bits against d = max step / 63, dmin = max offset / 63
+// (both kept as fp16); quants re-rounded against the stored scales.  Layout as GGUF (reference src/quants.h:61-69,
+// 91-113).
+void arcz_quantize_q4_k(const float* src, size_t N, int K, uint8_t* out) {
+  const int64_t nsbt = (int64_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < nsbt; ++s) {
+    const float* v = src + s * 256;
+    uint8_t* p = out + s * 144;
+    float step[8], off[8], smax = 0, omax = 0;
+    for (int b = 0; b < 8; ++b) {
+      float lo = 0, hi = 0;
+      for (int i = 0; i < 32; ++i) { lo = std::fmin(lo, v[32 * b + i]); hi = std::fmax(hi, v[32 * b + i]); }
+      step[b] = (hi - lo) / 15.0f;
+      off[b] = -lo;
+      smax = std::fmax(smax, step[b]);
+      omax = std::fmax(omax, off[b]);
+    }
+    const uint16_t dh = f32_to_f16(smax / 63.0f), mh = f32_to_f16(omax / 63.0f);
+    const float d = f16_to_f32(dh), dmin = f16_to_f32(mh);
+    int sc[8], mn[8];
+    for (int b = 0; b < 8; ++b) {
+      sc[b] = d > 0 ? std::min(63, std::max(0, (int)std::lrintf(step[b] / d))) : 0;
+      mn[b] = dmin > 0 ? std::min(63, std::max(0, (int)std::lrintf(off[b] / dmin))) : 0;
+    }
+    memcpy(p, &dh, 2);
+    memcpy(p + 2, &mh, 2);
+    uint8_t* q = p + 4;
+    memset(q, 0, 12);
+    for (int j = 0; j < 8; ++j) {
+      if (j < 4) {
+        q[j] |= sc[j] & 63;
+        q[j + 4] |= mn[j] & 63;
+      } else {
+        q[j + 4] = (uint8_t)((sc[j] & 0xF) | ((mn[j] & 0xF) << 4));
+        q[j - 4] |= (uint8_t)((sc[j] >> 4) << 6);
+        q[j] |= (uint8_t)((mn[j] >> 4) << 6);
+      }
+    }
+    uint8_t* qs = p + 16;
+    for (int j = 0; j < 4; ++j)
+      for (int l = 0; l < 32; ++l) {
+        int qq[2];
+        for (int h = 0; h < 2; ++h) {
+          const int b = 2 * j + h;
+          const float sd = d * (float)sc[b], x = v[64 * j + 32 * h + l] + dmin * (float)mn[b];
+          qq[h] = sd > 0 ? std::min(15, std::max(0, (int)std::lrintf(x / sd))) : 0;
+        }
+        qs[32 * j + l] = (uint8_t)(qq[0] | (qq[1] << 4));
+      }
+  }
+}
+
+// f32 rows -> GGUF Q6_K superblocks (210 bytes per 256 values): per 16 values a step amax / 31, rounded to int8
+// against d = max step / 127 (fp16); q = rte(v / (d * sc)) in -32..31, stored + 32 (reference src/quants.h:115-134).
+void arcz_quantize_q6_k(const float* src, size_t N, int K, uint8_t* out) {
+  const int64_t nsbt = (int64_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < nsbt; ++s) {
+    const float* v = src + s * 256;
+    uint8_t* p = out + s * 210;
+    float step[16], smax = 0;
+    for (int b = 0; b < 16; ++b) {
+      float amax = 0;
+      for (int i = 0; i < 16; ++i) amax = std::fmax(amax, std::fabs(v[16 * b + i]));
+      step[b] = amax / 31.0f;
+      smax = std::fmax(smax, step[b]);
+    }
+    const uint16_t dh = f32_to_f16(smax / 127.0f);
+    const float d = f16_to_f32(dh);
+    int8_t sc[16];
+    int q[256];
+    for (int b = 0; b < 16; ++b) {
+      sc[b] = (int8_t)(d > 0 ? std::min(127, std::max(1, (int)std::lrintf(step[b] / d))) : 0);
+      const float sd = d * (float)sc[b];
+      for (int i = 0; i < 16; ++i)
+        q[16 * b + i] = 32 + (sd > 0 ? std::min(31, std::max(-32, (int)std::lrintf(v[16 * b + i] / sd))) : 0);
+    }
+    uint8_t *ql = p, *qh = p + 128;
+    memset(p, 0, 192);
+    for (int n = 0; n < 2; ++n)
+      for (int l = 0; l < 32; ++l) {
+        const int q0 = q[128 * n + l], q1 = q[128 * n + l + 32], q2 = q[128 * n + l + 64], q3 = q[128 * n + l + 96];
+        ql[64 * n + l] = (uint8_t)((q0 & 0xF) | ((q2 & 0xF) << 4));
+        ql[64 * n + l + 32] = (uint8_t)((q1 & 0xF) | ((q3 & 0xF) << 4));
+        qh[32 * n + l] = (uint8_t)((q0 >> 4) | ((q1 >> 4) << 2) | ((q2 >> 4) << 4) | ((q3 >> 4) << 6));
+      }
+    memcpy(p + 192, sc, 16);
+    memcpy(p + 208, &dh, 2);
+  }
+}
+
+// Quantizes f32 rows to `type` (8, 12, 14).  0 or -1.
+int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
+  if (K <= 0 || K % 256) return -1;
+  if (type == QT_Q8_0) arcz_quantize_q8_0(src, N, K, out);
+  else if (type == QT_Q4_K) arcz_quantize_q4_k(src, N, K, out);
+  else if (type == QT_Q6_K) arcz_quantize_q6_k(src, N, K, out);
+  else return -1;
+  return 0;
+}
+
+// Synthetic weights: rows [row0, row0 + N) of a matrix ~ N(0, std) with the given seed, quantized to `type`, written
+// as GGUF blocks.  Generated in slabs so that a 150k-row matrix needs no f32 copy of itself.
+int arcz_gen_weights(uint32_t type, uint64_t seed, size_t N, int K, float std, uint8_t* out) {
+  if (K <= 0 || K % 256 || !arcz_gguf_bytes(type, 1, K)) return -1;
+  const size_t slab = 4096, rb = arcz_gguf_bytes(type, 1, K);
+  std::vector<float> f(slab * (size_t)K);
+  for (size_t r0 = 0; r0 < N; r0 += slab) {
+    const size_t nr = std::min(slab, N - r0);
+    arcz_gen_normal(seed + 0x1000003ull * (r0 / slab + 1), nr * K, 0.0f, std, f.data());
+    arcz_quantize_rows(type, f.data(), nr, K, out + r0 * rb);
+  }
+  return 0;
+}
+
+}  // extern "C"

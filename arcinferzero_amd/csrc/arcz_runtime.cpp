@@ -1,0 +1,417 @@
+// HIP backend behind include/arcz_hip.h: buffers, one stream, ahead-of-time kernel variants looked up by the
+// reference's (which, defs, name) key, checked launches, events.  It replaces the reference's zero/clrt.h +
+// zero/ze_min.h (hipMalloc / hipModuleLaunchKernel / one hipStream_t).
+#include "../../include/arcz_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "kernel_table.h"
+
+struct arcz_mem {
+  char* ptr;
+  size_t size;
+  bool owner;
+};
+struct arcz_kernel {
+  hipFunction_t fn;
+  const KernelSpec* spec;
+  std::string symbol;
+  std::vector<int> hidden;  // the -D values that ride along as trailing int arguments
+};
+struct arcz_event {
+  hipEvent_t start, stop;
+  bool pair;
+};
+
+namespace {
+struct Runtime {
+  bool up = false;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t prop;
+  std::string name;
+  std::set<arcz_mem*> mems;
+  size_t device_bytes = 0;
+  std::map<std::string, hipModule_t> modules;
+  std::map<std::string, arcz_kernel*> kernels;
+  int (*oom_hook)(void) = nullptr;
+  long fake_oom = 0, allocs = 0;
+  uint64_t launches = 0;
+  std::string err;
+};
+Runtime R;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  R.err = buf;
+  fprintf(stderr, "arcz: %s\n", buf);
+  return code;
+}
+#define HIP_TRY(x)                                                                                          \
+  do {                                                                                                      \
+    hipError_t e_ = (x);                                                                                    \
+    if (e_ != hipSuccess) return fail(ARCZ_E_DEVICE, "%s failed: %s", #x, hipGetErrorString(e_));           \
+  } while (0)
+
+bool out_of_bounds(const char* what, const arcz_mem* b, size_t off, size_t n) {
+  if (b && R.mems.count(const_cast<arcz_mem*>(b)) && off <= b->size && n <= b->size - off) return false;
+  fail(ARCZ_E_BOUNDS, "%s of %zu bytes at offset %zu past the end of a %zu-byte buffer (refused)", what, n, off,
+       b && R.mems.count(const_cast<arcz_mem*>(b)) ? b->size : (size_t)0);
+  return true;
+}
+}  // namespace
+
+extern "C" {
+
+// the code objects, linked in by kernel_blobs.S
+extern const unsigned char arcz_blob_ops[], arcz_blob_decode[], arcz_blob_gemm[], arcz_blob_moe[];
+
+int arcz_init(int device) {
+  if (R.up) return ARCZ_OK;
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return fail(ARCZ_E_DEVICE, "no HIP device");
+  if (device < 0 || device >= n) return fail(ARCZ_E_DEVICE, "device %d of %d", device, n);
+  HIP_TRY(hipSetDevice(device));
+  HIP_TRY(hipGetDeviceProperties(&R.prop, device));
+  R.name = std::string(R.prop.gcnArchName) + " " + R.prop.name;
+  if (R.name.rfind("gfx950", 0) != 0 && !getenv("ARCZ_ANY_ARCH"))
+    return fail(ARCZ_E_DEVICE, "device %d is %s: the kernels are built for gfx950 only", device, R.name.c_str());
+  HIP_TRY(hipStreamCreate(&R.stream));
+  R.device = device;
+  R.up = true;
+  return ARCZ_OK;
+}
+
+void arcz_shutdown(void) {
+  if (!R.up) return;
+  hipStreamSynchronize(R.stream);
+  for (auto& kv : R.kernels) delete kv.second;
+  R.kernels.clear();
+  for (auto& kv : R.modules) hipModuleUnload(kv.second);
+  R.modules.clear();
+  for (arcz_mem* m : R.mems) {
+    if (m->owner) hipFree(m->ptr);
+    delete m;
+  }
+  R.mems.clear();
+  R.device_bytes = 0;
+  hipStreamDestroy(R.stream);
+  R.stream = nullptr;
+  R.up = false;
+}
+
+const char* arcz_last_error(void) { return R.err.c_str(); }
+const char* arcz_device_name(void) { return R.name.c_str(); }
+int arcz_device_cus(void) { return R.up ? R.prop.multiProcessorCount : 0; }
+size_t arcz_device_mem(void) { return R.up ? R.prop.totalGlobalMem : 0; }
+size_t arcz_device_bytes(void) { return R.device_bytes; }
+
+arcz_mem* arcz_alloc(size_t bytes) {
+  if (!R.up) { fail(ARCZ_E_DEVICE, "arcz_alloc before arcz_init"); return nullptr; }
+  const size_t n = bytes < 64 ? 64 : bytes;
+  void* p = nullptr;
+  hipError_t e = hipSuccess;
+  ++R.allocs;
+  for (int attempt = 0; attempt <= 8; ++attempt) {
+    const bool fake = R.fake_oom > 0 && attempt == 0 && R.allocs % R.fake_oom == 0;
+    e = fake ? hipErrorOutOfMemory : hipMalloc(&p, n);
+    if (e == hipSuccess) break;
+    if (!fake) (void)hipGetLastError();
+    if (e != hipErrorOutOfMemory) break;
+    if (!(R.oom_hook && R.oom_hook())) break;  // nothing was freed: give up (clrt.h:474-487)
+  }
+  if (e != hipSuccess || !p) {
+    fail(ARCZ_E_OOM, "allocation of %zu bytes failed: %s", n, hipGetErrorString(e));
+    return nullptr;
+  }
+  arcz_mem* m = new arcz_mem{(char*)p, bytes, true};
+  R.mems.insert(m);
+  R.device_bytes += bytes;
+  return m;
+}
+
+arcz_mem* arcz_view(arcz_mem* parent, size_t offset, size_t bytes) {
+  if (!parent || !R.mems.count(parent) || offset > parent->size || bytes > parent->size - offset) {
+    fail(ARCZ_E_SUBBUFFER, "view of %zu bytes at %zu past its parent's end", bytes, offset);
+    return nullptr;
+  }
+  arcz_mem* m = new arcz_mem{parent->ptr + offset, bytes, false};
+  R.mems.insert(m);
+  return m;
+}
+
+int arcz_free(arcz_mem* m) {
+  if (!m) return ARCZ_OK;
+  if (!R.mems.count(m)) return fail(ARCZ_E_ARG_VALUE, "arcz_free of a handle that is not live");
+  if (m->owner) {
+    HIP_TRY(hipStreamSynchronize(R.stream));
+    HIP_TRY(hipFree(m->ptr));
+    R.device_bytes -= m->size;
+  }
+  R.mems.erase(m);
+  delete m;
+  return ARCZ_OK;
+}
+
+size_t arcz_mem_size(const arcz_mem* m) { return m && R.mems.count(const_cast<arcz_mem*>(m)) ? m->size : 0; }
+void* arcz_mem_ptr(const arcz_mem* m) { return m && R.mems.count(const_cast<arcz_mem*>(m)) ? m->ptr : nullptr; }
+
+int arcz_h2d(arcz_mem* dst, size_t offset, const void* src, size_t bytes) {
+  if (out_of_bounds("write", dst, offset, bytes)) return ARCZ_E_BOUNDS;
+  if (!bytes) return ARCZ_OK;
+  HIP_TRY(hipMemcpyAsync(dst->ptr + offset, src, bytes, hipMemcpyHostToDevice, R.stream));
+  HIP_TRY(hipStreamSynchronize(R.stream));
+  return ARCZ_OK;
+}
+int arcz_d2h(void* dst, const arcz_mem* src, size_t offset, size_t bytes) {
+  if (out_of_bounds("read", src, offset, bytes)) return ARCZ_E_BOUNDS;
+  if (!bytes) return ARCZ_OK;
+  HIP_TRY(hipMemcpyAsync(dst, src->ptr + offset, bytes, hipMemcpyDeviceToHost, R.stream));
+  HIP_TRY(hipStreamSynchronize(R.stream));
+  return ARCZ_OK;
+}
+int arcz_d2d(arcz_mem* dst, size_t dst_offset, const arcz_mem* src, size_t src_offset, size_t bytes) {
+  if (out_of_bounds("copy (source)", src, src_offset, bytes) || out_of_bounds("copy (destination)", dst, dst_offset, bytes))
+    return ARCZ_E_BOUNDS;
+  if (!bytes) return ARCZ_OK;
+  HIP_TRY(hipMemcpyAsync(dst->ptr + dst_offset, src->ptr + src_offset, bytes, hipMemcpyDeviceToDevice, R.stream));
+  return ARCZ_OK;
+}
+
+static arcz_kernel* fill_kernel();
+
+int arcz_fill(arcz_mem* dst, const void* pattern, size_t ps, size_t offset, size_t bytes) {
+  if (out_of_bounds("fill", dst, offset, bytes)) return ARCZ_E_BOUNDS;
+  if (!bytes) return ARCZ_OK;
+  if ((ps != 1 && ps != 2 && ps != 4) || bytes % ps || offset % ps)
+    return fail(ARCZ_E_BOUNDS, "fill pattern of %zu bytes over %zu bytes at %zu", ps, bytes, offset);
+  uint32_t v = 0;
+  memcpy(&v, pattern, ps);
+  if (ps == 1) v |= v << 8;
+  if (ps <= 2) v |= v << 16;
+  if (bytes % 4 == 0 && offset % 4 == 0) {
+    // a small kernel rather than a memset node: callers may be under stream capture
+    arcz_kernel* k = fill_kernel();
+    if (!k) return ARCZ_E_BUILD;
+    void* p = dst->ptr + offset;
+    size_t n = bytes / 4;
+    void* params[3] = {&p, &v, &n};
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    HIP_TRY(hipModuleLaunchKernel(k->fn, blocks, 1, 1, 256, 1, 1, 0, R.stream, params, nullptr));
+  } else {
+    if (ps == 1) HIP_TRY(hipMemsetAsync(dst->ptr + offset, (int)(v & 0xFF), bytes, R.stream));
+    else HIP_TRY(hipMemsetD16Async((hipDeviceptr_t)(dst->ptr + offset), (unsigned short)(v & 0xFFFF), bytes / 2, R.stream));
+  }
+  HIP_TRY(hipStreamSynchronize(R.stream));
+  return ARCZ_OK;
+}
+
+// ---- kernels
+
+static const unsigned char* blob_of(const std::string& which) {
+  if (which == "ops") return arcz_blob_ops;
+  if (which == "decode") return arcz_blob_decode;
+  if (which == "gemm") return arcz_blob_gemm;
+  if (which == "moe") return arcz_blob_moe;
+  return nullptr;
+}
+
+// "-DQT=12 -DGROWS=2 -cl-whatever" -> {QT: 12, GROWS: 2}; a -D without a value is 1
+static std::map<std::string, long> parse_defs(const char* defs) {
+  std::map<std::string, long> out;
+  const std::string s = defs ? defs : "";
+  size_t i = 0;
+  while (i < s.size()) {
+    while (i < s.size() && s[i] == ' ') ++i;
+    size_t j = i;
+    while (j < s.size() && s[j] != ' ') ++j;
+    const std::string tok = s.substr(i, j - i);
+    if (tok.size() > 2 && tok[0] == '-' && tok[1] == 'D') {
+      const size_t eq = tok.find('=');
+      const std::string name = tok.substr(2, eq == std::string::npos ? std::string::npos : eq - 2);
+      out[name] = eq == std::string::npos ? 1 : strtol(tok.c_str() + eq + 1, nullptr, 0);
+    }
+    i = j;
+  }
+  return out;
+}
+
+arcz_kernel* arcz_kernel_get(const char* which, const char* defs, const char* name) {
+  if (!R.up) { fail(ARCZ_E_DEVICE, "arcz_kernel_get before arcz_init"); return nullptr; }
+  const std::string w = which ? which : "", d = defs ? defs : "", nm = name ? name : "";
+  const std::string key = w + d + "|" + nm;  // the reference's cache key (engine_setup.h:318)
+  auto it = R.kernels.find(key);
+  if (it != R.kernels.end()) return it->second;
+  const std::map<std::string, long> dv = parse_defs(defs);
+  const KernelSpec* spec = nullptr;
+  for (const KernelSpec& s : kKernelTable)
+    if (!spec && w == s.which && nm == s.name && (!s.requires_def || dv.count(s.requires_def))) spec = &s;
+  if (!spec) { fail(ARCZ_E_BUILD, "no kernel %s in module %s", nm.c_str(), w.c_str()); return nullptr; }
+  std::string symbol = nm;
+  for (int i = 0; spec->variant[i]; ++i) {
+    auto f = dv.find(spec->variant[i]);
+    if (f == dv.end()) { fail(ARCZ_E_BUILD, "%s: -D%s is required", nm.c_str(), spec->variant[i]); return nullptr; }
+    symbol += (i == 0 ? "__" : "_") + std::string(spec->variant[i]) + std::to_string(f->second);
+  }
+  std::vector<int> hidden;
+  for (int i = 0; spec->hidden[i].name; ++i) {
+    auto f = dv.find(spec->hidden[i].name);
+    if (f == dv.end() && spec->hidden[i].required) {
+      fail(ARCZ_E_BUILD, "%s: -D%s is required", nm.c_str(), spec->hidden[i].name);
+      return nullptr;
+    }
+    hidden.push_back(f == dv.end() ? spec->hidden[i].def : (int)f->second);
+  }
+  hipModule_t mod;
+  auto mi = R.modules.find(w);
+  if (mi == R.modules.end()) {
+    const unsigned char* blob = blob_of(w);
+    if (!blob) { fail(ARCZ_E_BUILD, "no module %s", w.c_str()); return nullptr; }
+    hipError_t e = hipModuleLoadData(&mod, blob);
+    if (e != hipSuccess) { fail(ARCZ_E_BUILD, "module %s does not load: %s", w.c_str(), hipGetErrorString(e)); return nullptr; }
+    R.modules[w] = mod;
+  } else {
+    mod = mi->second;
+  }
+  hipFunction_t fn;
+  hipError_t e = hipModuleGetFunction(&fn, mod, symbol.c_str());
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    fail(ARCZ_E_BUILD, "module %s has no variant %s (defs \"%s\")", w.c_str(), symbol.c_str(), d.c_str());
+    return nullptr;
+  }
+  arcz_kernel* k = new arcz_kernel{fn, spec, symbol, hidden};
+  R.kernels[key] = k;
+  return k;
+}
+
+static arcz_kernel* fill_kernel() { return arcz_kernel_get("ops", "", "fill32"); }
+
+const char* arcz_kernel_symbol(const arcz_kernel* k) { return k ? k->symbol.c_str() : ""; }
+
+int arcz_launch(arcz_kernel* k, unsigned dim, const size_t* global, const size_t* local, const void* const* args,
+                const size_t* sizes, unsigned nargs, arcz_event** event) {
+  if (event) *event = nullptr;
+  if (!R.up || !k) return fail(ARCZ_E_DEVICE, "arcz_launch without a runtime or kernel");
+  if (dim < 1 || dim > 3) return fail(ARCZ_E_GLOBAL_SIZE, "%s: %u dimensions", k->symbol.c_str(), dim);
+  unsigned gs[3] = {1, 1, 1}, ls[3] = {1, 1, 1};
+  for (unsigned d = 0; d < dim; ++d) {
+    if (global[d] == 0) return ARCZ_OK;  // nothing to run (clrt.h:942)
+    if (global[d] > 0xFFFFFFFFull)
+      return fail(ARCZ_E_GLOBAL_SIZE, "%s: global size %zu past 32 bits (refused)", k->symbol.c_str(), global[d]);
+    gs[d] = (unsigned)global[d];
+  }
+  if (local) {
+    for (unsigned d = 0; d < dim; ++d) ls[d] = (unsigned)local[d];
+  } else {
+    ls[0] = 256;
+    while (ls[0] > 1 && gs[0] % ls[0]) --ls[0];
+  }
+  for (unsigned d = 0; d < 3; ++d)
+    if (ls[d] == 0 || gs[d] % ls[d])
+      return fail(ARCZ_E_WORK_GROUP, "%s: global size %u x %u x %u is not a multiple of the work-group %u x %u x %u",
+                  k->symbol.c_str(), gs[0], gs[1], gs[2], ls[0], ls[1], ls[2]);
+  if ((size_t)ls[0] * ls[1] * ls[2] > 1024 || (k->spec->local_x && ls[0] * ls[1] * ls[2] != (unsigned)k->spec->local_x))
+    return fail(ARCZ_E_WORK_GROUP, "%s: work-group %u x %u x %u (the kernel is written for %d threads)",
+                k->symbol.c_str(), ls[0], ls[1], ls[2], k->spec->local_x ? k->spec->local_x : 1024);
+  // arguments: count, sizes, pointers
+  const size_t nsig = strlen(k->spec->args);
+  if (nargs != nsig)
+    return fail(ARCZ_E_ARG_INDEX, "%s takes %zu arguments, %u given", k->symbol.c_str(), nsig, nargs);
+  unsigned char store[64][8];
+  void* params[64 + 8];
+  if (nsig + k->hidden.size() > 64) return fail(ARCZ_E_ARG_INDEX, "%s: too many arguments", k->symbol.c_str());
+  for (unsigned i = 0; i < nargs; ++i) {
+    const char c = k->spec->args[i];
+    const size_t want = (c == 'p' || c == 'z') ? 8 : 4;
+    if (sizes[i] != want || !args[i])
+      return fail(ARCZ_E_ARG_SIZE, "%s: argument %u has %zu bytes, the kernel takes %zu", k->symbol.c_str(), i, sizes[i], want);
+    memcpy(store[i], args[i], want);
+    if (c == 'p') {
+      arcz_mem* m;
+      memcpy(&m, args[i], 8);
+      if (m) {
+        if (!R.mems.count(m))
+          return fail(ARCZ_E_ARG_VALUE, "%s: argument %u is not a live buffer", k->symbol.c_str(), i);
+        memcpy(store[i], &m->ptr, 8);
+      }
+    }
+    params[i] = store[i];
+  }
+  for (size_t h = 0; h < k->hidden.size(); ++h) params[nargs + h] = &k->hidden[h];
+  arcz_event* ev = nullptr;
+  if (event) {
+    ev = new arcz_event{nullptr, nullptr, true};
+    HIP_TRY(hipEventCreate(&ev->start));
+    HIP_TRY(hipEventCreate(&ev->stop));
+    HIP_TRY(hipEventRecord(ev->start, R.stream));
+  }
+  hipError_t e = hipModuleLaunchKernel(k->fn, gs[0] / ls[0], gs[1] / ls[1], gs[2] / ls[2], ls[0], ls[1], ls[2], 0,
+                                       R.stream, params, nullptr);
+  if (e != hipSuccess) {
+    if (ev) { hipEventDestroy(ev->start); hipEventDestroy(ev->stop); delete ev; }
+    return fail(ARCZ_E_DEVICE, "launch of %s (global %u x %u x %u, local %u x %u x %u) failed: %s", k->symbol.c_str(),
+                gs[0], gs[1], gs[2], ls[0], ls[1], ls[2], hipGetErrorString(e));
+  }
+  ++R.launches;
+  if (ev) {
+    HIP_TRY(hipEventRecord(ev->stop, R.stream));
+    *event = ev;
+  }
+  return ARCZ_OK;
+}
+
+int arcz_sync(void) {
+  if (!R.up) return fail(ARCZ_E_DEVICE, "arcz_sync before arcz_init");
+  HIP_TRY(hipStreamSynchronize(R.stream));
+  return ARCZ_OK;
+}
+
+double arcz_event_ms(arcz_event* e) {
+  if (!e || !e->pair) return -1.0;
+  if (hipEventSynchronize(e->stop) != hipSuccess) return -1.0;
+  float ms = 0;
+  if (hipEventElapsedTime(&ms, e->start, e->stop) != hipSuccess) return -1.0;
+  return ms;
+}
+void arcz_event_release(arcz_event* e) {
+  if (!e) return;
+  hipEventDestroy(e->start);
+  if (e->pair) hipEventDestroy(e->stop);
+  delete e;
+}
+arcz_event* arcz_event_record(void) {
+  if (!R.up) return nullptr;
+  arcz_event* ev = new arcz_event{nullptr, nullptr, false};
+  if (hipEventCreate(&ev->start) != hipSuccess || hipEventRecord(ev->start, R.stream) != hipSuccess) {
+    delete ev;
+    return nullptr;
+  }
+  return ev;
+}
+double arcz_event_elapsed_ms(arcz_event* start, arcz_event* stop) {
+  if (!start || !stop) return -1.0;
+  if (hipEventSynchronize(stop->start) != hipSuccess) return -1.0;
+  float ms = 0;
+  if (hipEventElapsedTime(&ms, start->start, stop->start) != hipSuccess) return -1.0;
+  return ms;
+}
+
+void arcz_set_oom_hook(int (*hook)(void)) { R.oom_hook = hook; }
+void arcz_set_fake_oom(long n) { R.fake_oom = n; R.allocs = 0; }
+uint64_t arcz_launch_count(void) { return R.launches; }
+
+}  // extern "C"

@@ -1,0 +1,159 @@
+// The OpenCL-subset names the reference engine is written against (zero/clrt.h), on top of the C ABI of
+// include/arcz_hip.h.  Engine code that says clCreateBuffer / clSetKernelArg / clEnqueueNDRangeKernel / CL_CHECK /
+// set_args compiles against this header unchanged; underneath there is hipMalloc, hipModuleLaunchKernel and one
+// stream instead of Level Zero.
+#pragma once
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/arcz_hip.h"
+
+typedef int cl_int;
+typedef unsigned cl_uint;
+typedef unsigned cl_bool;
+typedef unsigned long cl_ulong;
+typedef cl_ulong cl_mem_flags;
+typedef cl_ulong cl_map_flags;
+typedef cl_uint cl_buffer_create_type;
+typedef arcz_mem* cl_mem;
+typedef arcz_event* cl_event;
+typedef struct _arcz_queue* cl_command_queue;
+typedef struct _arcz_context* cl_context;
+struct cl_buffer_region { size_t origin, size; };
+
+// cl_kernel: the backend's kernel handle plus the argument values set so far (clSetKernelArg keeps them per kernel,
+// zero/clrt.h:47-57; a launch sends them all).
+struct ArczKernelArgs {
+  arcz_kernel* k = nullptr;
+  std::string name;
+  struct Arg { size_t sz = 0; unsigned char v[8] = {}; };
+  std::vector<Arg> args;
+};
+typedef ArczKernelArgs* cl_kernel;
+
+#define CL_SUCCESS 0
+#define CL_TRUE 1
+#define CL_FALSE 0
+#define CL_MEM_READ_WRITE (1 << 0)
+#define CL_MEM_WRITE_ONLY (1 << 1)
+#define CL_MEM_READ_ONLY (1 << 2)
+#define CL_MEM_COPY_HOST_PTR (1 << 5)
+#define CL_BUFFER_CREATE_TYPE_REGION 0x1220
+
+// Any failure ends the process with a message, unless the owner asked for exceptions (the reference's CL_CHECK,
+// zero/clrt.h:85-93, and soft_fail, :1050).
+namespace arcz {
+inline bool& soft_fail() { static bool v = false; return v; }
+inline void check(int err, const char* what, const char* file, int line) {
+  if (err == CL_SUCCESS) return;
+  char msg[640];
+  snprintf(msg, sizeof msg, "%s failed with %d at %s:%d: %s", what, err, file, line, arcz_last_error());
+  if (soft_fail()) throw std::runtime_error(msg);
+  fprintf(stderr, "arcz: %s\n", msg);
+  fflush(stderr);
+  _Exit(1);
+}
+}  // namespace arcz
+#define CL_CHECK(x) arcz::check((x), #x, __FILE__, __LINE__)
+
+inline cl_int clFinish(cl_command_queue) { return arcz_sync(); }
+inline cl_int clFlush(cl_command_queue) { return CL_SUCCESS; }
+inline cl_mem clCreateBuffer(cl_context, cl_mem_flags flags, size_t n, void* host, cl_int* err) {
+  cl_mem m = arcz_alloc(n);
+  cl_int e = m ? CL_SUCCESS : ARCZ_E_OOM;
+  if (m && (flags & CL_MEM_COPY_HOST_PTR) && host) e = arcz_h2d(m, 0, host, n);
+  if (err) *err = e;
+  return m;
+}
+inline cl_mem clCreateSubBuffer(cl_mem parent, cl_mem_flags, cl_buffer_create_type, const void* region, cl_int* err) {
+  const cl_buffer_region* r = (const cl_buffer_region*)region;
+  cl_mem m = arcz_view(parent, r->origin, r->size);
+  if (err) *err = m ? CL_SUCCESS : ARCZ_E_SUBBUFFER;
+  return m;
+}
+inline cl_int clReleaseMemObject(cl_mem m) { return arcz_free(m); }
+inline cl_int clEnqueueReadBuffer(cl_command_queue, cl_mem b, cl_bool, size_t off, size_t n, void* host, cl_uint,
+                                  const cl_event*, cl_event* ev) {
+  if (ev) *ev = nullptr;
+  return arcz_d2h(host, b, off, n);
+}
+inline cl_int clEnqueueWriteBuffer(cl_command_queue, cl_mem b, cl_bool, size_t off, size_t n, const void* host, cl_uint,
+                                   const cl_event*, cl_event* ev) {
+  if (ev) *ev = nullptr;
+  return arcz_h2d(b, off, host, n);
+}
+inline cl_int clEnqueueCopyBuffer(cl_command_queue, cl_mem src, cl_mem dst, size_t so, size_t doff, size_t n, cl_uint,
+                                  const cl_event*, cl_event* ev) {
+  if (ev) *ev = nullptr;
+  return arcz_d2d(dst, doff, src, so, n);
+}
+inline cl_int clEnqueueFillBuffer(cl_command_queue, cl_mem b, const void* pattern, size_t ps, size_t off, size_t n,
+                                  cl_uint, const cl_event*, cl_event* ev) {
+  if (ev) *ev = nullptr;
+  return arcz_fill(b, pattern, ps, off, n);
+}
+inline cl_int clSetKernelArg(cl_kernel k, cl_uint i, size_t sz, const void* v) {
+  if (!k || sz > 8 || !v) return ARCZ_E_ARG_SIZE;
+  if (k->args.size() <= i) k->args.resize(i + 1);
+  k->args[i].sz = sz;
+  memcpy(k->args[i].v, v, sz);
+  return CL_SUCCESS;
+}
+inline cl_int clEnqueueNDRangeKernel(cl_command_queue, cl_kernel k, cl_uint dim, const size_t*, const size_t* g,
+                                     const size_t* l, cl_uint, const cl_event*, cl_event* ev) {
+  const void* ptrs[64];
+  size_t sizes[64];
+  const size_t n = k->args.size();
+  if (n > 64) return ARCZ_E_ARG_INDEX;
+  for (size_t i = 0; i < n; ++i) { ptrs[i] = k->args[i].v; sizes[i] = k->args[i].sz; }
+  return arcz_launch(k->k, dim, g, l, ptrs, sizes, (unsigned)n, ev);
+}
+inline cl_int clReleaseEvent(cl_event e) { arcz_event_release(e); return CL_SUCCESS; }
+inline cl_int clReleaseKernel(cl_kernel k) { delete k; return CL_SUCCESS; }
+
+// set_args(k, first index, values...) (zero/clrt.h:1363-1367)
+inline void set_args(cl_kernel, cl_uint) {}
+template <class T, class... Rest>
+inline void set_args(cl_kernel k, cl_uint i, const T& v, const Rest&... rest) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "kernel arguments are 4 or 8 bytes");
+  CL_CHECK(clSetKernelArg(k, i, sizeof(T), &v));
+  set_args(k, i + 1, rest...);
+}
+
+// ClRt: start-up and kernel lookup (zero/clrt.h:1025-1333).  build() + kernel() of the reference compile a program
+// per option string; here both are one lookup in the ahead-of-time variants.
+struct ClRt {
+  std::string device_id;
+  bool soft_fail = false;
+  cl_context ctx = (cl_context)1;
+  cl_command_queue queue = (cl_command_queue)1;
+  bool init(bool = false) {
+    if (arcz_init(0) != ARCZ_OK) return false;
+    device_id = arcz_device_name();
+    return true;
+  }
+  cl_kernel kernel(const std::string& which, const std::string& defs, const std::string& name) {
+    arcz_kernel* h = arcz_kernel_get(which.c_str(), defs.c_str(), name.c_str());
+    if (!h) {
+      const std::string msg = "no kernel " + which + " " + defs + " | " + name + ": " + arcz_last_error();
+      if (soft_fail || arcz::soft_fail()) throw std::runtime_error(msg);
+      fprintf(stderr, "arcz: %s\n", msg.c_str());
+      _Exit(1);
+    }
+    cl_kernel k = new ArczKernelArgs;
+    k->k = h;
+    k->name = name;
+    return k;
+  }
+  cl_mem buffer(cl_mem_flags flags, size_t n, const void* host = nullptr) {
+    cl_int err;
+    cl_mem m = clCreateBuffer(ctx, flags | (host ? CL_MEM_COPY_HOST_PTR : 0), n, const_cast<void*>(host), &err);
+    CL_CHECK(err);
+    return m;
+  }
+  static double event_ms(cl_event e) { return arcz_event_ms(e); }
+};

@@ -1,0 +1,359 @@
+// The matmul dispatch of the reference engine (zero/engine.h:936-1251: run, matmul, matmul1, gemv1_rows; the weight
+// upload of zero/engine_load.h:84-196; the MoE layer of zero/engine_moe.h:8-470), re-hosted on the HIP backend.
+// Same entry points, argument meaning and error behaviour; launch shapes and tuning rules are gfx950's own.
+#pragma once
+#include <algorithm>
+#include <cstdint>
+#include <map>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "clrt_hip.h"
+#include "kernels/common.h"
+
+#define GGML_Q8_0 8u
+#define GGML_Q4_K 12u
+#define GGML_Q6_K 14u
+
+extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
+extern "C" size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
+
+// (zero/engine.h:27-34) raw = the device planes of all `rows` rows (an expert tensor holds n_expert * N rows)
+struct GpuWeight {
+  uint32_t type = 0;
+  int N = 0, K = 0;
+  cl_mem raw = nullptr;
+  size_t rows = 0;
+};
+
+inline const char* ggml_type_name(uint32_t t) {
+  return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q6_K ? "Q6_K" : "?";
+}
+
+class Engine {
+ public:
+  ClRt cl_;
+  bool profile = false;
+  std::map<std::string, double> prof_ms;
+  std::map<std::string, int> prof_n;
+  uint64_t rd_bytes = 0;  // GGUF bytes of the weights the GEMVs read (zero/engine.h:150-151)
+
+  // max_chunk token rows of at most max_k values each (alloc_buffers, zero/engine_alloc.h:4-41)
+  Engine(int max_chunk_, int max_k_) : max_chunk(max_chunk_), max_k(max_k_) {
+    arcz::soft_fail() = true;
+    cl_.soft_fail = true;
+    if (!cl_.init()) throw std::runtime_error(std::string("no GPU runtime: ") + arcz_last_error());
+    if (max_chunk <= 0 || max_k <= 0 || max_k % 256) throw std::invalid_argument("Engine: max_k must be a positive multiple of 256");
+    const size_t M = (size_t)max_chunk;
+    aq_ = buf(M * max_k);
+    asc_ = buf(M * (max_k / 32) * 4);
+    absum_ = buf(M * (max_k / 16) * 2);
+  }
+  ~Engine() {
+    for (auto& kv : kernels_) clReleaseKernel(kv.second);
+    for (auto it = mems_.rbegin(); it != mems_.rend(); ++it) clReleaseMemObject(*it);  // views before parents
+  }
+  Engine(const Engine&) = delete;
+
+  int max_chunk, max_k;
+  cl_mem aq_ = nullptr, asc_ = nullptr, absum_ = nullptr;
+  int cur_T_ = 0, cur_K_ = 0, cur_Mp_ = 0;
+
+  cl_mem buf(size_t bytes, const void* host = nullptr) {
+    cl_mem m = cl_.buffer(CL_MEM_READ_WRITE, bytes, host);
+    mems_.push_back(m);
+    return m;
+  }
+  void release(cl_mem m) {
+    auto it = std::find(mems_.begin(), mems_.end(), m);
+    if (it != mems_.end()) mems_.erase(it);
+    CL_CHECK(clReleaseMemObject(m));
+  }
+
+  // (zero/engine_setup.h:317-362) one kernel object per (source, -D string, name)
+  cl_kernel kernel(const std::string& which, const std::string& defs, const std::string& name) {
+    const std::string key = which + defs + "|" + name;
+    auto it = kernels_.find(key);
+    if (it != kernels_.end()) return it->second;
+    cl_kernel k = cl_.kernel(which, defs, name);
+    kernels_[key] = k;
+    return k;
+  }
+  // (zero/engine.h:936-950)
+  void run(const char* name, cl_kernel k, int dims, const size_t* gws, const size_t* lws) {
+    cl_event e = nullptr;
+    CL_CHECK(clEnqueueNDRangeKernel(cl_.queue, k, dims, nullptr, gws, lws, 0, nullptr, profile ? &e : nullptr));
+    if (profile && e) events_.push_back({name, e});
+  }
+  void collect_profile() {
+    if (!profile) return;
+    clFinish(cl_.queue);
+    for (auto& [n, e] : events_) {
+      prof_ms[n] += ClRt::event_ms(e);
+      prof_n[n]++;
+      clReleaseEvent(e);
+    }
+    events_.clear();
+  }
+
+  // ---- weights (zero/engine_load.h:84-130 upload_padded, :157-196 make_weight): the GGUF rows regrouped into the
+  // device planes on the host, then one upload.  rows = N for a matrix, n_expert * N for an expert tensor.
+  GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
+    if (rows == 0) rows = (size_t)N;
+    if (type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q6_K)
+      throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
+    if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
+    if (nbytes != arcz_gguf_bytes(type, rows, K))
+      throw std::runtime_error("make_weight: " + std::to_string(nbytes) + " bytes given, " +
+                               std::to_string(arcz_gguf_bytes(type, rows, K)) + " expected");
+    GpuWeight w;
+    w.type = type;
+    w.N = N;
+    w.K = K;
+    w.rows = rows;
+    const size_t pb = raw_planes_bytes((int)type, rows, K / 256);
+    std::vector<uint8_t> planes(pb);
+    if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
+    w.raw = buf(pb, planes.data());
+    return w;
+  }
+  void free_weight(GpuWeight& w) {
+    if (w.raw) release(w.raw);
+    w.raw = nullptr;
+  }
+  static uint64_t raw_bytes(const GpuWeight& w) { return arcz_gguf_bytes(w.type, w.rows, w.K); }  // (zero/engine.h:209)
+
+  // ---- activations.  The reference quantizes inside its norm / SwiGLU kernels (quant_store16, zero/kernels/ops.cl:
+  // 38-72, launched by rmsnorm_quant, zero/engine.h:1256-1267); quantize_rows is that step alone: rows [0, T) of x
+  // (row stride ldx floats) into aq_ / asc_ / absum_ laid out for Mp rows, rows [T, Mp) zero.  Sets the form the next
+  // matmul takes (cur_T_).
+  void quantize_rows(cl_mem x, int ldx, int K, int Mp, int T, int act32) {
+    check_chunk(K, Mp, T);
+    if (!act32) throw std::runtime_error("quantize_rows: the matmul kernels take per-32 activation scales (act32)");
+    if (ldx < K || arcz_mem_size(x) < ((size_t)(T - 1) * ldx + K) * 4) throw std::runtime_error("quantize_rows: x is too small");
+    cl_kernel k = kernel("ops", "", "quant_rows");
+    set_args(k, 0, x, ldx, K, Mp, T, aq_, asc_, absum_, act32);
+    size_t gws[2] = {(size_t)256 * (K / 256), (size_t)(Mp + 63) / 64}, lws[2] = {256, 1};
+    run("quant_rows", k, 2, gws, lws);
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
+  }
+  // Activations quantized elsewhere (the reference's benches quantize on the host, bench/gemv_bench.cpp:103-129).
+  void set_activations(const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp, int T) {
+    check_chunk(K, Mp, T);
+    CL_CHECK(clEnqueueWriteBuffer(cl_.queue, aq_, CL_TRUE, 0, (size_t)Mp * K, aq, 0, nullptr, nullptr));
+    CL_CHECK(clEnqueueWriteBuffer(cl_.queue, asc_, CL_TRUE, 0, (size_t)Mp * (K / 32) * 4, asc, 0, nullptr, nullptr));
+    CL_CHECK(clEnqueueWriteBuffer(cl_.queue, absum_, CL_TRUE, 0, (size_t)Mp * (K / 16) * 2, absum, 0, nullptr, nullptr));
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
+  }
+
+  // ---- matmul (zero/engine.h:1080-1112 without the two-pass mode): C[:, c_off : c_off+N] (+)= act * W^T for the
+  // current chunk.  acc: 0 = store, 1 = accumulate into C, 2 = C = silu(C) * result (GEMM path only).
+  void matmul(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
+    matmul1(name, w, Mp, C, ldc, c_off, acc, act32);
+  }
+
+  // rows per half wave of the one-token GEMV (the place of the reference's gemv1_rows, zero/engine.h:1119-1123)
+  static int gemv1_rows(const GpuWeight& w) {
+    static const int force = getenv("ARCZ_GROWS") ? atoi(getenv("ARCZ_GROWS")) : 0;
+    if (force == 1 || force == 2 || force == 4) return force <= w.N ? force : 1;
+    return w.N <= 4096 ? 1 : 2;
+  }
+  static int gemv_mt_rows(const GpuWeight& w) {
+    static const int force = getenv("ARCZ_GROWS_MT") ? atoi(getenv("ARCZ_GROWS_MT")) : 0;
+    if (force == 1 || force == 2) return force;
+    return w.N <= 4096 ? 1 : 2;
+  }
+
+  void matmul1(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
+    if (!w.raw) throw std::runtime_error(std::string("matmul ") + name + ": the weight is not loaded");
+    if (!act32) throw std::runtime_error(std::string("matmul ") + name + ": per-256 activation scales are not built");
+    if (cur_T_ <= 0 || w.K != cur_K_ || Mp != cur_Mp_)
+      throw std::runtime_error(std::string("matmul ") + name + ": the activations hold " + std::to_string(cur_Mp_) + " x " +
+                               std::to_string(cur_K_) + ", the matrix takes " + std::to_string(Mp) + " x " + std::to_string(w.K));
+    if (acc < 0 || acc > 2) throw std::runtime_error(std::string("matmul ") + name + ": accumulate mode");
+    const int rows_out = cur_T_ > 8 ? Mp : cur_T_;
+    if (c_off < 0 || (cur_T_ > 1 && c_off + w.N > ldc) ||
+        arcz_mem_size(C) < ((size_t)(rows_out - 1) * (cur_T_ == 1 ? 0 : ldc) + c_off + w.N) * 4)
+      throw std::runtime_error(std::string("matmul ") + name + ": the output does not fit C");
+    int a = acc;
+    cl_mem tabs = nullptr;  // (the reference's codebook tables: none of the three types has one)
+    if (cur_T_ == 1) {
+      if (a > 1) throw std::logic_error(std::string("GEMV with a fused epilogue: ") + name);
+      const int grows = gemv1_rows(w);
+      int N = w.N, K = w.K, M = Mp;
+      rd_bytes += raw_bytes(w);
+      cl_kernel k = kernel("decode", "-DQT=" + std::to_string(w.type) + " -DGROWS=" + std::to_string(grows), "gemv");
+      set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
+      const size_t hws = (size_t)(N + grows - 1) / grows, l1 = 256;
+      size_t g1 = (hws * 32 + l1 - 1) / l1 * l1;
+      run(name, k, 1, &g1, &l1);
+      return;
+    }
+    if (cur_T_ > 1 && cur_T_ <= 8) {
+      if (a > 1) throw std::logic_error(std::string("GEMV with a fused epilogue: ") + name);
+      const int gr = gemv_mt_rows(w);
+      cl_kernel k = kernel("decode", "-DQT=" + std::to_string(w.type) + " -DGROWS=" + std::to_string(gr) + " -DTB=" +
+                                         std::to_string(cur_T_), "gemv_mt");
+      int N = w.N, K = w.K, M = Mp, T = cur_T_;
+      rd_bytes += raw_bytes(w);
+      set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a);
+      size_t g1 = ((size_t)(N + gr - 1) / gr * 32 + 255) / 256 * 256, l1 = 256;
+      run(name, k, 1, &g1, &l1);
+      return;
+    }
+    gemm_dense(name, w, Mp, C, ldc, c_off, a);
+  }
+
+  // The prefill GEMM (zero/engine.h:1205-1250).  Token rows come in whole tiles (the reference pads a chunk to 128
+  // rows from 128 tokens on, :521-522).
+  void gemm_dense(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int a) {
+    cl_kernel k = gemm_kernel(w.type, false);
+    int M = Mp, N = w.N, K = w.K;
+    // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
+    //  registers over the whole of K.  The reference splits rows longer than 8192 into 17-superblock pieces for its
+    //  cache, zero/engine.h:1236-1250; pieces after the first accumulate into C and are not bit-identical to one pass.)
+    static const int sk_sb = getenv("ARCZ_GEMM_SPLIT") ? std::max(0, atoi(getenv("ARCZ_GEMM_SPLIT"))) : 0;
+    const int nsb = K / 256, splits = a != 2 && sk_sb > 0 ? (nsb + sk_sb - 1) / sk_sb : 1, rgroup = 1;
+    cl_mem unused = nullptr;
+    const size_t tiles = (size_t)((Mp + 127) / 128) * ((N + 127) / 128);
+    size_t gws[1] = {tiles * 256}, lws[1] = {256};
+    for (int sp = 0; sp < splits; ++sp) {
+      int s0 = nsb * sp / splits, s1 = nsb * (sp + 1) / splits, ac = sp == 0 ? a : 1;
+      set_args(k, 0, w.raw, unused, aq_, asc_, absum_, C, M, N, K, ldc, c_off, ac, rgroup, s0, s1);
+      run(name, k, 1, gws, lws);
+    }
+  }
+  // (zero/engine_setup.h:384-420 gemm_kernel / moe_gemm_kernel)
+  cl_kernel gemm_kernel(uint32_t qtype, bool tiles, int ne = 0) {
+    std::string defs = "-DQTYPE=" + std::to_string(qtype) + " -DACT32";
+    if (tiles) defs += " -DMOE_TILES -DNE=" + std::to_string(ne);
+    return kernel("gemm", defs, "gemm");
+  }
+
+  // ---------------------------------------------------------------- mixture of experts (zero/engine_moe.h)
+  struct MoeLayer {
+    GpuWeight ex[3];  // gate, up [NE][F][E]; down [NE][E][F]
+    int NE = 0, NU = 0, E = 0, F = 0;
+  };
+  // buffers of the layer (zero/engine_alloc.h:109-159): sized for max_chunk tokens
+  cl_mem mids_ = nullptr, mwts_ = nullptr, sgate_ = nullptr, mcount_ = nullptr, moffs_ = nullptr, mcursor_ = nullptr,
+         mtiles_ = nullptr, mtstart_ = nullptr, stok_ = nullptr, swt_ = nullptr, minv_ = nullptr, mh_ = nullptr,
+         mhq_ = nullptr, mhsc_ = nullptr, my_ = nullptr;
+  int slots_ = 0, moe_ne_ = 0, moe_nu_ = 0, moe_e_ = 0, moe_f_ = 0;
+
+  void moe_alloc(int NE, int NU, int E, int F) {
+    if (moe_ne_ == NE && moe_nu_ == NU && moe_e_ == E && moe_f_ == F) return;
+    if (moe_ne_) throw std::runtime_error("moe_alloc: one expert geometry per engine");
+    if (NE <= 0 || NE > 512 || NU <= 0 || NU > 64 || NU > NE || E % 256 || F % 256)
+      throw std::runtime_error("moe_alloc: unsupported expert geometry");
+    moe_ne_ = NE; moe_nu_ = NU; moe_e_ = E; moe_f_ = F;
+    slots_ = max_chunk * NU;
+    const size_t S = (size_t)slots_;
+    mids_ = buf(S * 4); mwts_ = buf(S * 4); sgate_ = buf((size_t)max_chunk * 4);
+    mcount_ = buf((size_t)NE * 4); moffs_ = buf((size_t)NE * 4); mcursor_ = buf((size_t)NE * 4);
+    mtiles_ = buf((1 + 3 * (S + NE)) * 4); mtstart_ = buf((size_t)(NE + 1) * 4);
+    stok_ = buf(S * 4); swt_ = buf(S * 4); minv_ = buf(S * 4);
+    mh_ = buf(S * F * 4); mhq_ = buf(S * F); mhsc_ = buf(S * (F / 32) * 4); my_ = buf(S * E * 4);
+    const uint32_t zero = 0;
+    CL_CHECK(clEnqueueFillBuffer(cl_.queue, mcount_, &zero, 4, 0, (size_t)NE * 4, 0, nullptr, nullptr));
+  }
+
+  MoeLayer make_moe_layer(uint32_t type, const uint8_t* gate, const uint8_t* up, const uint8_t* down, int NE, int NU,
+                          int E, int F) {
+    moe_alloc(NE, NU, E, F);
+    MoeLayer L;
+    L.NE = NE; L.NU = NU; L.E = E; L.F = F;
+    L.ex[0] = make_weight(type, gate, arcz_gguf_bytes(type, (size_t)NE * F, E), F, E, (size_t)NE * F);
+    L.ex[1] = make_weight(type, up, arcz_gguf_bytes(type, (size_t)NE * F, E), F, E, (size_t)NE * F);
+    L.ex[2] = make_weight(type, down, arcz_gguf_bytes(type, (size_t)NE * E, F), E, F, (size_t)NE * E);
+    return L;
+  }
+
+  // routing -> slots grouped by expert -> tiles (zero/engine_moe.h:95-134).  rl: router logits [T][ldl] f32.
+  // tm: slots per tile.
+  void moe_route(const MoeLayer& L, cl_mem rl, int ldl, int T, int tm) {
+    const int NE = L.NE, NU = L.NU, n = T * NU;
+    if (T <= 0 || T > max_chunk || ldl < NE || arcz_mem_size(rl) < ((size_t)(T - 1) * ldl + NE) * 4)
+      throw std::runtime_error("moe_route: router logits do not fit");
+    const std::string defs = "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DTM=" + std::to_string(tm);
+    {
+      cl_kernel k = kernel("moe", defs, "moe_route");
+      int NR = ldl, TT = T;
+      set_args(k, 0, rl, NR, TT, mids_, mwts_, sgate_, mcount_);
+      size_t g1 = (size_t)(T + 3) / 4 * 256, l1 = 256;
+      run("moe_route", k, 1, &g1, &l1);
+    }
+    {
+      cl_kernel k = kernel("moe", defs, "moe_scan");
+      set_args(k, 0, mcount_, moffs_, mcursor_, mtiles_, mtstart_);
+      size_t g1 = 1024, l1 = 1024;
+      run("moe_scan", k, 1, &g1, &l1);
+    }
+    {
+      cl_kernel k = kernel("moe", defs, "moe_scatter");
+      int nn = n;
+      set_args(k, 0, mids_, mwts_, nn, mcursor_, stok_, swt_, minv_);
+      size_t g1 = (size_t)NE * 256, l1 = 256;
+      run("moe_scatter", k, 1, &g1, &l1);
+    }
+  }
+
+  // The experts of a chunk through the tile GEMM (zero/engine_moe.h:433-470 moe_gemm, without its decode pass: the
+  // kernel decodes the raw rows itself): part 0 = gate, then up with the fused SwiGLU into mh_; part 2 = down,
+  // routing-weighted, into my_.
+  void moe_gemm(const MoeLayer& L, int part, int Mp, size_t max_tiles) {
+    const int E = L.E, F = L.F, NE = L.NE;
+    for (int i = part; i < (part == 0 ? 2 : 3); ++i) {
+      const int N = i == 2 ? E : F, K = i == 2 ? F : E;
+      cl_kernel k = gemm_kernel(L.ex[i].type, true, NE);
+      int M = i == 2 ? slots_ : Mp, NN = N, KK = K, ldc = N, acc = i == 1 ? 2 : 0, e0 = 0, e1 = NE, um = i == 2 ? 0 : 1,
+          us = i == 2 ? 1 : 0;
+      cl_mem unused = nullptr;
+      set_args(k, 0, L.ex[i].raw, unused, i == 2 ? mhq_ : aq_, i == 2 ? mhsc_ : asc_, absum_, i == 2 ? my_ : mh_, M, NN, KK,
+               ldc, acc, mtiles_, mtstart_, e0, e1, stok_, um, swt_, us);
+      size_t gws[2] = {(size_t)(N + 127) / 128 * 256, max_tiles}, lws[2] = {256, 1};
+      run(i == 2 ? "moe_down" : "moe_gateup", k, 2, gws, lws);
+    }
+  }
+
+  // x[t] += sum_k w_k * expert_k(h[t]) for the T tokens whose quantized h is the current activation chunk
+  // (zero/engine_moe.h:8-361 layer_moe: standard experts, no shared expert).  x: [T][E] f32.
+  void layer_moe(const MoeLayer& L, cl_mem rl, int ldl, cl_mem x, int T, int Mp) {
+    const int E = L.E, F = L.F, NU = L.NU, n = T * NU;
+    if (cur_T_ != T || cur_K_ != E || cur_Mp_ != Mp) throw std::runtime_error("layer_moe: the activations are not this chunk's");
+    if (arcz_mem_size(x) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: x is too small");
+    const int tm = 128;  // slots per tile: the token rows of one work-group of the tile GEMM
+    moe_route(L, rl, ldl, T, tm);
+    // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)
+    const size_t max_tiles = (size_t)(n + tm - 1) / tm + std::min(n, L.NE);
+    moe_gemm(L, 0, Mp, max_tiles);
+    {
+      cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_quant");
+      int FF = F, S = slots_;
+      set_args(k, 0, mh_, FF, S, mhq_, mhsc_);
+      size_t gws[2] = {(size_t)256 * (F / 256), (size_t)(n + 63) / 64}, lws[2] = {256, 1};
+      run("moe_quant", k, 2, gws, lws);
+    }
+    moe_gemm(L, 2, Mp, max_tiles);
+    {
+      cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_combine");
+      cl_mem sh = nullptr;
+      int EE = E;
+      set_args(k, 0, x, sh, sgate_, my_, minv_, EE);
+      size_t gws[2] = {((size_t)E + 255) / 256 * 256, (size_t)T}, lws[2] = {256, 1};
+      run("moe_combine", k, 2, gws, lws);
+    }
+  }
+
+ private:
+  void check_chunk(int K, int Mp, int T) {
+    if (K <= 0 || K % 256 || K > max_k || Mp <= 0 || Mp > max_chunk || T <= 0 || T > Mp)
+      throw std::runtime_error("activation chunk " + std::to_string(T) + " of " + std::to_string(Mp) + " rows x " +
+                               std::to_string(K) + " does not fit the engine's buffers (" + std::to_string(max_chunk) + " x " +
+                               std::to_string(max_k) + ")");
+  }
+  std::map<std::string, cl_kernel> kernels_;
+  std::vector<cl_mem> mems_;
+  std::vector<std::pair<std::string, cl_event>> events_;
+};

@@ -1,0 +1,43 @@
+// The kernels of the embedded code objects: for each (module, name) the argument signature the launch checks, the
+// -D names that select a compiled variant, and the -D names whose values ride along as trailing int arguments.
+// Signature letters: p = device buffer (8 bytes), i = int / uint (4), f = float (4), z = size_t by value (8).
+#pragma once
+
+struct HiddenDef {
+  const char* name;  // nullptr ends the list
+  int def;
+  bool required;
+};
+struct KernelSpec {
+  const char* which;
+  const char* name;
+  const char* requires_def;  // this entry is taken only when the -D string holds this name (nullptr: always)
+  const char* args;
+  const char* variant[5];  // nullptr-terminated
+  HiddenDef hidden[6];     // {nullptr} terminated
+  int local_x;             // threads per work-group the kernel is written for (0 = any)
+};
+
+// Entries with requires_def come before the plain entry of the same name.
+static const KernelSpec kKernelTable[] = {
+    // ---- ops
+    {"ops", "quant_rows", nullptr, "piiiipppi", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},
+    // ---- decode
+    {"decode", "gemv", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{nullptr, 0, false}}, 256},
+    {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{nullptr, 0, false}}, 256},
+    // ---- gemm
+    {"gemm", "gemm", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
+     {{"NE", 0, true}, {nullptr, 0, false}}, 256},
+    {"gemm", "gemm", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
+    // ---- moe
+    {"moe", "moe_route", nullptr, "piipppp", {nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_route1", nullptr, "pppppp", {nullptr},
+     {{"NE", 0, true}, {"NU", 0, true}, {"HAS_GATE", 0, false}, {nullptr, 0, false}}, 64},
+    {"moe", "moe_scan", nullptr, "ppppp", {nullptr}, {{"NE", 0, true}, {"TM", 16, false}, {nullptr, 0, false}}, 1024},
+    {"moe", "moe_scatter", nullptr, "ppipppp", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_quant", nullptr, "piipp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_combine", nullptr, "pppppi", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},
+};

@@ -1,0 +1,100 @@
+// Shared device helpers for the gfx950 kernels: vector types, GGUF type ids, the device weight layout, scale decoding.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#ifdef __HIPCC__
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v32f __attribute__((ext_vector_type(32)));
+#endif
+
+// GGUF type ids (reference src/gguf.h:18-22)
+#define QT_Q8_0 8
+#define QT_Q4_K 12
+#define QT_Q6_K 14
+
+// ---- device weight layout ("raw planes").  A matrix of R rows x K columns (K % 256 == 0, nsb = K / 256) is held
+// as separate planes, each row-major over (row, superblock), so that every field is 16-byte aligned and a wave's
+// consecutive lanes read consecutive 16-byte units.  The byte count equals the GGUF byte count except Q6_K's 2-byte
+// scale per superblock, which keeps its size (the plane as a whole is padded to 16 bytes).
+//   Q4_K : qs  [R][nsb][128]  (GGUF order: byte l of chunk j = element 64j+l low nibble, 64j+32+l high nibble)
+//          hdr [R][nsb][16]   (f16 d, f16 dmin, 12 bytes of packed 6-bit scales / mins, as in GGUF)
+//   Q6_K : ql  [R][nsb][128], qh [R][nsb][64], sc [R][nsb][16] (int8), d [R][nsb] (f16)
+//   Q8_0 : qs  [R][nsb][256] (int8), d [R][nsb][8] (f16)
+// Plane offsets from the start of the buffer, in bytes (each a multiple of 256 when R * nsb is a multiple of 16;
+// always a multiple of 16 otherwise except as noted).
+struct PlanesQ4K { size_t qs, hdr; };
+struct PlanesQ6K { size_t ql, qh, sc, d; };
+struct PlanesQ80 { size_t qs, d; };
+
+__host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
+__host__ __device__ inline PlanesQ4K planes_q4k(size_t rows, int nsb) {
+  PlanesQ4K p;
+  p.qs = 0;
+  p.hdr = rows * (size_t)nsb * 128;
+  return p;
+}
+__host__ __device__ inline PlanesQ6K planes_q6k(size_t rows, int nsb) {
+  PlanesQ6K p;
+  const size_t u = rows * (size_t)nsb;
+  p.ql = 0;
+  p.qh = u * 128;
+  p.sc = p.qh + u * 64;
+  p.d = p.sc + u * 16;
+  return p;
+}
+__host__ __device__ inline PlanesQ80 planes_q80(size_t rows, int nsb) {
+  PlanesQ80 p;
+  p.qs = 0;
+  p.d = rows * (size_t)nsb * 256;
+  return p;
+}
+__host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb) {
+  const size_t u = rows * (size_t)nsb;
+  if (qt == QT_Q4_K) return u * 144;
+  if (qt == QT_Q6_K) return align16(u * 208 + u * 2);
+  if (qt == QT_Q8_0) return u * 272;
+  return 0;
+}
+
+#ifdef __HIPCC__
+__device__ inline float f16_bits_to_f32(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)(h & 0xFFFFu));
+}
+
+// Per-byte (q - 32) for four 6-bit unsigned values packed in a word, without borrows between bytes.
+__device__ inline uint32_t sub32_bytes(uint32_t q) { return ((q | 0x80808080u) - 0x20202020u) ^ 0x80808080u; }
+
+// 6-bit scale and min of Q4_K sub-blocks 2j and 2j+1 from the three words of packed scale bytes (bytes 0-3, 4-7,
+// 8-11 of the 12: the GGUF packing, reference src/quants.h:61-69).
+__device__ inline void q4k_scales_pair(uint32_t s0, uint32_t s1, uint32_t s2, int j, int& sc0, int& sc1, int& mn0,
+                                       int& mn1) {
+  const int sh = 16 * (j & 1);
+  const uint32_t x0 = s0 >> sh, x1 = s1 >> sh, y = s2 >> sh;
+  if (j < 2) {
+    sc0 = x0 & 63; sc1 = (x0 >> 8) & 63;
+    mn0 = x1 & 63; mn1 = (x1 >> 8) & 63;
+  } else {
+    sc0 = (y & 0xF) | (((x0 >> 6) & 3) << 4);
+    sc1 = ((y >> 8) & 0xF) | (((x0 >> 14) & 3) << 4);
+    mn0 = ((y >> 4) & 0xF) | (((x1 >> 6) & 3) << 4);
+    mn1 = ((y >> 12) & 0xF) | (((x1 >> 14) & 3) << 4);
+  }
+}
+
+__device__ inline int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
+
+// Sum over the 32 lanes of a half wave (lanes 0-31 and 32-63 separately), same value in every lane; a fixed tree,
+// so results do not depend on anything but the inputs.
+__device__ inline float half_wave_sum(float v) {
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 8, 64);
+  v += __shfl_xor(v, 4, 64);
+  v += __shfl_xor(v, 2, 64);
+  v += __shfl_xor(v, 1, 64);
+  return v;
+}
+#endif

@@ -1,0 +1,197 @@
+// "decode" module: the bandwidth-bound matrix-vector products on the raw weight planes, for 1 token (gemv) and for
+// 2..8 tokens that share one read of the weights (gemv_mt).
+//
+// Arithmetic per 16-element half block h of weight row n and token t, as the reference's gemv
+// (zero/kernels/decode.cl:992-1003):  I = sum of 16 int8 x int8 products (v_dot4_i32_i8, exact int32);
+//   Q4_K : acc += sa * (d * (float)(sc * I) - dmin * (float)(mn * bs))      sa: the token's scale of the 32-block,
+//   Q6_K : acc += sa * d * (float)(sc16 * I)                                bs: its int16 sum of the 16 activations
+//   Q8_0 : acc += sa * d * (float)I
+// (the reference groups the two halves of a 32-block inside the int -> float conversion; here each half is converted
+// alone, because a lane's 16-byte unit of Q4_K nibbles holds halves of two different blocks: the same real number,
+// rounded at another place).  Lanes add their terms in unit order; a row's 32 lanes are summed by a fixed tree.
+//
+// Mapping: a half wave (32 lanes) takes GROWS consecutive rows; lane l reads the 16-byte units l, l+32, ... of a
+// row's quant plane, so a wave's load instruction covers two contiguous 512-byte runs.  The token's int8 values,
+// scales and sums of a unit are loaded once and used for all GROWS rows.
+#include "common.h"
+
+template <int QT> struct UnitsPerSb { static constexpr int v = QT == QT_Q8_0 ? 16 : 8; };
+
+template <int QT, int TB, int GROWS>
+__device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ aq,
+                                 const float* __restrict__ asc, const short* __restrict__ absum, int M, int T,
+                                 float* __restrict__ C, int ldc, int c_off, int accumulate, size_t plane_rows) {
+  const int nsb = K >> 8, units = nsb * UnitsPerSb<QT>::v;
+  const int hl = threadIdx.x & 31;
+  const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
+  const int r0 = hw * GROWS;
+  if (r0 >= N) return;
+  float acc[GROWS][TB];
+#pragma unroll
+  for (int r = 0; r < GROWS; ++r)
+#pragma unroll
+    for (int t = 0; t < TB; ++t) acc[r][t] = 0.0f;
+
+  if constexpr (QT == QT_Q4_K) {
+    const PlanesQ4K pl = planes_q4k(plane_rows, nsb);
+    const int j = (hl >> 1) & 3, half = hl & 1;
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 3;
+      const int e_lo = sb * 256 + 64 * j + 16 * half;
+      uint4 alo[TB], ahi[TB];
+      float salo[TB], sahi[TB];
+      int bslo[TB], bshi[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) {
+        const int tt = t < T ? t : 0;
+        alo[t] = *(const uint4*)(aq + (size_t)tt * K + e_lo);
+        ahi[t] = *(const uint4*)(aq + (size_t)tt * K + e_lo + 32);
+        salo[t] = asc[(size_t)(sb * 8 + 2 * j) * M + tt];
+        sahi[t] = asc[(size_t)(sb * 8 + 2 * j + 1) * M + tt];
+        bslo[t] = absum[(size_t)(sb * 16 + 4 * j + half) * M + tt];
+        bshi[t] = absum[(size_t)(sb * 16 + 4 * j + 2 + half) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const int n = min(r0 + r, N - 1);
+        const uint4 w = *(const uint4*)(raw + pl.qs + (size_t)n * nsb * 128 + (size_t)u * 16);
+        const uint4 h = *(const uint4*)(raw + pl.hdr + ((size_t)n * nsb + sb) * 16);
+        const float d = f16_bits_to_f32(h.x), dmin = f16_bits_to_f32(h.x >> 16);
+        int sc0, sc1, mn0, mn1;
+        q4k_scales_pair(h.y, h.z, h.w, j, sc0, sc1, mn0, mn1);
+        const uint32_t wl[4] = {w.x & 0x0F0F0F0Fu, w.y & 0x0F0F0F0Fu, w.z & 0x0F0F0F0Fu, w.w & 0x0F0F0F0Fu};
+        const uint32_t wh[4] = {(w.x >> 4) & 0x0F0F0F0Fu, (w.y >> 4) & 0x0F0F0F0Fu, (w.z >> 4) & 0x0F0F0F0Fu,
+                                (w.w >> 4) & 0x0F0F0F0Fu};
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+          int ilo = dot4(wl[0], alo[t].x, 0);
+          ilo = dot4(wl[1], alo[t].y, ilo);
+          ilo = dot4(wl[2], alo[t].z, ilo);
+          ilo = dot4(wl[3], alo[t].w, ilo);
+          int ihi = dot4(wh[0], ahi[t].x, 0);
+          ihi = dot4(wh[1], ahi[t].y, ihi);
+          ihi = dot4(wh[2], ahi[t].z, ihi);
+          ihi = dot4(wh[3], ahi[t].w, ihi);
+          acc[r][t] += salo[t] * (d * (float)(sc0 * ilo) - dmin * (float)(mn0 * bslo[t]));
+          acc[r][t] += sahi[t] * (d * (float)(sc1 * ihi) - dmin * (float)(mn1 * bshi[t]));
+        }
+      }
+    }
+  } else if constexpr (QT == QT_Q6_K) {
+    const PlanesQ6K pl = planes_q6k(plane_rows, nsb);
+    const int idx = hl & 7, n2 = idx >> 2, l0 = (idx & 3) * 16, q1 = l0 >> 5;
+    const int hsh1 = 2 * q1, hsh2 = 2 * q1 + 4;
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 3;
+      const int e1 = sb * 256 + 128 * n2 + l0, e2 = e1 + 64;
+      uint4 a1[TB], a2[TB];
+      float sa1[TB], sa2[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) {
+        const int tt = t < T ? t : 0;
+        a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
+        a2[t] = *(const uint4*)(aq + (size_t)tt * K + e2);
+        sa1[t] = asc[(size_t)(e1 >> 5) * M + tt];
+        sa2[t] = asc[(size_t)(e2 >> 5) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const int n = min(r0 + r, N - 1);
+        const size_t rs = (size_t)n * nsb + sb;
+        const uint4 L = *(const uint4*)(raw + pl.ql + (size_t)n * nsb * 128 + (size_t)u * 16);
+        const uint4 H = *(const uint4*)(raw + pl.qh + rs * 64 + 32 * n2 + (l0 & 31));
+        const signed char* scp = (const signed char*)(raw + pl.sc + rs * 16 + 8 * n2 + (idx & 3));
+        const int sc1 = scp[0], sc2 = scp[4];
+        const float d = f16_bits_to_f32(*(const unsigned short*)(raw + pl.d + rs * 2));
+        const uint32_t Lw[4] = {L.x, L.y, L.z, L.w}, Hw[4] = {H.x, H.y, H.z, H.w};
+        uint32_t w1[4], w2[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          w1[k] = sub32_bytes((Lw[k] & 0x0F0F0F0Fu) | (((Hw[k] >> hsh1) & 0x03030303u) << 4));
+          w2[k] = sub32_bytes(((Lw[k] >> 4) & 0x0F0F0F0Fu) | (((Hw[k] >> hsh2) & 0x03030303u) << 4));
+        }
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+          int i1 = dot4(w1[0], a1[t].x, 0);
+          i1 = dot4(w1[1], a1[t].y, i1);
+          i1 = dot4(w1[2], a1[t].z, i1);
+          i1 = dot4(w1[3], a1[t].w, i1);
+          int i2 = dot4(w2[0], a2[t].x, 0);
+          i2 = dot4(w2[1], a2[t].y, i2);
+          i2 = dot4(w2[2], a2[t].z, i2);
+          i2 = dot4(w2[3], a2[t].w, i2);
+          acc[r][t] += sa1[t] * d * (float)(sc1 * i1);
+          acc[r][t] += sa2[t] * d * (float)(sc2 * i2);
+        }
+      }
+    }
+  } else {
+    const PlanesQ80 pl = planes_q80(plane_rows, nsb);
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 4, b = (u >> 1) & 7;
+      const int e = u * 16;
+      uint4 a[TB];
+      float sa[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) {
+        const int tt = t < T ? t : 0;
+        a[t] = *(const uint4*)(aq + (size_t)tt * K + e);
+        sa[t] = asc[(size_t)(e >> 5) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const int n = min(r0 + r, N - 1);
+        const uint4 w = *(const uint4*)(raw + pl.qs + (size_t)n * nsb * 256 + (size_t)u * 16);
+        const float d = f16_bits_to_f32(*(const unsigned short*)(raw + pl.d + (((size_t)n * nsb + sb) * 8 + b) * 2));
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+          int i = dot4(w.x, a[t].x, 0);
+          i = dot4(w.y, a[t].y, i);
+          i = dot4(w.z, a[t].z, i);
+          i = dot4(w.w, a[t].w, i);
+          acc[r][t] += sa[t] * d * (float)i;
+        }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < GROWS; ++r)
+#pragma unroll
+    for (int t = 0; t < TB; ++t) {
+      const float v = half_wave_sum(acc[r][t]);
+      const int n = r0 + r;
+      if (hl == 0 && n < N && t < T) {
+        float* cp = C + (size_t)t * ldc + c_off + n;
+        *cp = accumulate ? *cp + v : v;
+      }
+    }
+}
+
+// gemv: one token.  Arguments as the reference's gemv (zero/kernels/decode.cl:913-915); `tabs` (its codebook
+// tables) is unused by these three types.  grid: ceil(N / GROWS) half waves in work-groups of 256.
+#define GEMV_INST(QT, GROWS)                                                                                         \
+  extern "C" __global__ __launch_bounds__(256) void gemv__QT##QT##_GROWS##GROWS(                                      \
+      const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
+      const short* absum, int M, float* C, int c_off, int accumulate) {                                               \
+    gemv_body<QT, 1, GROWS>(raw, N, K, aq, asc, absum, M, 1, C, 0, c_off, accumulate, (size_t)N);                    \
+  }
+
+// gemv_mt: T = TB tokens (reference zero/kernels/decode.cl:1581-1583).
+#define GEMV_MT_INST(QT, GROWS, TB)                                                                                  \
+  extern "C" __global__ __launch_bounds__(256) void gemv_mt__QT##QT##_GROWS##GROWS##_TB##TB(                          \
+      const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
+      const short* absum, int M, int T, float* C, int ldc, int c_off, int accumulate) {                               \
+    gemv_body<QT, TB, GROWS>(raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, (size_t)N);                 \
+  }
+
+#define GEMV_ALL(QT)                                                                                                 \
+  GEMV_INST(QT, 1) GEMV_INST(QT, 2) GEMV_INST(QT, 4)                                                                  \
+  GEMV_MT_INST(QT, 1, 2) GEMV_MT_INST(QT, 1, 3) GEMV_MT_INST(QT, 1, 4) GEMV_MT_INST(QT, 1, 5)                         \
+  GEMV_MT_INST(QT, 1, 6) GEMV_MT_INST(QT, 1, 7) GEMV_MT_INST(QT, 1, 8)                                                \
+  GEMV_MT_INST(QT, 2, 2) GEMV_MT_INST(QT, 2, 3) GEMV_MT_INST(QT, 2, 4) GEMV_MT_INST(QT, 2, 5)                         \
+  GEMV_MT_INST(QT, 2, 6) GEMV_MT_INST(QT, 2, 7) GEMV_MT_INST(QT, 2, 8)
+
+GEMV_ALL(8)
+GEMV_ALL(12)
+GEMV_ALL(14)

@@ -1,0 +1,235 @@
+// "moe" module: routing, grouping of the (token, expert) pairs by expert, the expert-input quantizer and the final
+// combine of a mixture-of-experts FFN (reference zero/kernels/moe.cl:50-179, 258-290, 344-352).  The reference
+// compiles these with -DNE (experts), -DNU (experts per token), -DTM (slots per tile); here they are trailing
+// arguments.
+#include "quant.h"
+
+#define MAX_PER_LANE 8  // NE <= 512
+
+// moe_route: one wave per token.  The NU largest of NE logits (ties: the lower expert), p = exp(l - max),
+// weights p / sum of the selected p; counts[e]++ per selection; sgate[t] = sigmoid(logit NE) when the row holds one.
+// grid: ceil(T / 4) work-groups of 256 threads.
+extern "C" __global__ __launch_bounds__(256) void moe_route(const float* __restrict__ logits, int ldl, int T,
+                                                            int* __restrict__ ids, float* __restrict__ wts,
+                                                            float* __restrict__ sgate, int* __restrict__ counts,
+                                                            int NE, int NU) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const float* lg = logits + (size_t)t * ldl;
+  float v[MAX_PER_LANE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < MAX_PER_LANE; ++i) {
+    const int e = i * 64 + lane;
+    v[i] = e < NE ? lg[e] : -INFINITY;
+    mx = fmaxf(mx, v[i]);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+  float sum = 0.0f, myp = 0.0f;
+  int mysel = 0;
+  for (int k = 0; k < NU; ++k) {
+    float bv = -INFINITY;
+    int bi = NE;
+#pragma unroll
+    for (int i = 0; i < MAX_PER_LANE; ++i)
+      if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
+    // wave arg-max, the lower index among equal values
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const float ov = __shfl_xor(bv, d, 64);
+      const int oi = __shfl_xor(bi, d, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+#pragma unroll
+    for (int i = 0; i < MAX_PER_LANE; ++i)
+      if (i * 64 + lane == bi) v[i] = -INFINITY;
+    const int sel = min(bi, NE - 1);  // (a row of NaN picks no lane: keep the index inside the tables)
+    const float p = expf(bv - mx);
+    sum += p;
+    if (lane == k) { mysel = sel; myp = p; }
+  }
+  if (lane < NU) {
+    ids[(size_t)t * NU + lane] = mysel;
+    wts[(size_t)t * NU + lane] = myp / sum;
+    atomicAdd(&counts[mysel], 1);
+  }
+  if (lane == 0 && sgate) sgate[t] = ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
+}
+
+// moe_route1: a single token straight into NU one-slot tiles (no counts, scan or scatter).  One wave.
+extern "C" __global__ __launch_bounds__(64) void moe_route1(const float* __restrict__ logits, float* __restrict__ sgate,
+                                                            int* __restrict__ tiles, int* __restrict__ stok,
+                                                            float* __restrict__ swt, int* __restrict__ inv, int NE,
+                                                            int NU, int has_gate) {
+  const int lane = threadIdx.x & 63;
+  float v[MAX_PER_LANE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < MAX_PER_LANE; ++i) {
+    const int e = i * 64 + lane;
+    v[i] = e < NE ? logits[e] : -INFINITY;
+    mx = fmaxf(mx, v[i]);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+  float sum = 0.0f, myp = 0.0f;
+  int mysel = 0;
+  for (int k = 0; k < NU; ++k) {
+    float bv = -INFINITY;
+    int bi = NE;
+#pragma unroll
+    for (int i = 0; i < MAX_PER_LANE; ++i)
+      if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const float ov = __shfl_xor(bv, d, 64);
+      const int oi = __shfl_xor(bi, d, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+#pragma unroll
+    for (int i = 0; i < MAX_PER_LANE; ++i)
+      if (i * 64 + lane == bi) v[i] = -INFINITY;
+    const float p = expf(bv - mx);
+    sum += p;
+    if (lane == k) { mysel = min(bi, NE - 1); myp = p; }
+  }
+  if (lane < NU) {
+    tiles[1 + 3 * lane] = mysel;
+    tiles[2 + 3 * lane] = lane;
+    tiles[3 + 3 * lane] = 1;
+    stok[lane] = 0;
+    swt[lane] = myp / sum;
+    inv[lane] = lane;
+  }
+  if (lane == 0) {
+    tiles[0] = NU;
+    if (sgate) sgate[0] = has_gate ? 1.0f / (1.0f + expf(-logits[NE])) : 0.0f;
+  }
+}
+
+// moe_scan: exclusive scan of the counts -> offs / cursor; the tile list tiles[0] = number of tiles, then (expert,
+// first slot, rows <= TM) per tile; tstart[e] = first tile of expert e, tstart[NE] = the tile count; counts reset.
+// One work-group of 1024 threads (NE <= 1024).
+extern "C" __global__ __launch_bounds__(1024) void moe_scan(int* __restrict__ counts, int* __restrict__ offs,
+                                                            int* __restrict__ cursor, int* __restrict__ tiles,
+                                                            int* __restrict__ tstart, int NE, int TM) {
+  __shared__ int a[1024], b[1024];
+  const int e = threadIdx.x;
+  const int c = e < NE ? counts[e] : 0, nt = (c + TM - 1) / TM;
+  a[e] = c;
+  b[e] = nt;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int x = e >= d ? a[e - d] : 0, y = e >= d ? b[e - d] : 0;
+    __syncthreads();
+    a[e] += x;
+    b[e] += y;
+    __syncthreads();
+  }
+  if (e >= NE) return;
+  const int off = a[e] - c, toff = b[e] - nt;
+  offs[e] = off;
+  cursor[e] = off;
+  tstart[e] = toff;
+  if (e == NE - 1) tiles[0] = tstart[NE] = b[e];
+  for (int i = 0; i < nt; ++i) {
+    int* tp = tiles + 1 + 3 * (toff + i);
+    tp[0] = e;
+    tp[1] = off + i * TM;
+    tp[2] = min(TM, c - i * TM);
+  }
+  counts[e] = 0;
+}
+
+// moe_scatter: places pair i = (token i / NU, expert ids[i]) in a slot of its expert's range, in pair order: the
+// k-th pair of expert e (counting i upwards) gets slot offs[e] + k, so the layout is the same on every run (the
+// reference draws slots from an atomic counter; its results do not depend on the order, its layout does).
+// One work-group of 256 threads per expert, each scanning all n pairs.  `cursor` holds offs (as moe_scan wrote it).
+extern "C" __global__ __launch_bounds__(256) void moe_scatter(const int* __restrict__ ids, const float* __restrict__ wts,
+                                                              int n, int* __restrict__ cursor, int* __restrict__ stok,
+                                                              float* __restrict__ swt, int* __restrict__ inv, int NU) {
+  __shared__ int wsum[4];
+  __shared__ int base_s;
+  const int e = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  if (t == 0) base_s = cursor[e];
+  __syncthreads();
+  for (int i0 = 0; i0 < n; i0 += 256) {
+    const int i = i0 + t;
+    const bool mine = i < n && ids[i] == e;
+    const unsigned long long bal = __ballot(mine);
+    const int rank = __popcll(bal & ((1ull << lane) - 1));
+    if (lane == 0) wsum[wave] = __popcll(bal);
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += wsum[w];
+    const int total = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+    const int base = base_s;
+    if (mine) {
+      const int s = base + before + rank;
+      stok[s] = i / NU;
+      swt[s] = wts[i];
+      inv[i] = s;
+    }
+    __syncthreads();
+    if (t == 0) base_s = base + total;
+    __syncthreads();
+  }
+}
+
+// moe_quant: h [S][F] f32 (S slot rows, the first n in use) -> hq [S][F] int8, hsc [F/32][S] f32 with row stride S;
+// no sums (reference zero/kernels/moe.cl:258-274; FV: columns >= FV quantize as zeros).  The grid covers the rows in
+// use in tiles of 64; rows of a tile at or past S are skipped.  grid (F/256, ceil(n/64)), local 256.
+extern "C" __global__ __launch_bounds__(256) void moe_quant(const float* __restrict__ h, int F, int S,
+                                                            signed char* __restrict__ hq, float* __restrict__ hsc,
+                                                            int FV) {
+  __shared__ float lasc[8][64];
+  const int s = blockIdx.x, m0 = blockIdx.y * 64;
+  const int lane16 = threadIdx.x & 15, rg = threadIdx.x >> 4;
+#pragma unroll 1
+  for (int p = 0; p < 4; ++p) {
+    const int r = p * 16 + rg, m = m0 + r;
+    float v[16];
+    const int base = s * 256 + 16 * lane16;
+    if (m < S) {
+      const float4* src = (const float4*)(h + (size_t)m * F + base);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 f = src[i];
+        v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (base + i >= FV) v[i] = 0.0f;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) v[i] = 0.0f;
+    }
+    const float amax = block_amax(v, 1);
+    uint4 pk;
+    int sum;
+    quant16(v, amax, pk, sum);
+    if (m < S) *(uint4*)(hq + (size_t)m * F + base) = pk;
+    if ((lane16 & 1) == 0) lasc[lane16 >> 1][r] = amax / 127.0f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = threadIdx.x + 256 * i, b = idx >> 6, r = idx & 63;
+    if (m0 + r < S) hsc[((size_t)s * 8 + b) * S + m0 + r] = lasc[b][r];
+  }
+}
+
+// moe_combine: x[t][c] += sum over k (in order) of y[inv[t * NU + k]][c]  (+ sgate[t] * sh[t][c] when there is a
+// shared expert: sh non-null).  grid (ceil(N / 256) * 256, T), local (256, 1).
+extern "C" __global__ __launch_bounds__(256) void moe_combine(float* __restrict__ x, const float* __restrict__ sh,
+                                                              const float* __restrict__ sgate, const float* __restrict__ y,
+                                                              const int* __restrict__ inv, int N, int NU) {
+  const int c = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+  if (c >= N) return;
+  float v = 0.0f;
+  for (int k = 0; k < NU; ++k) v += y[(size_t)inv[t * NU + k] * N + c];
+  if (sh) v += sgate[t] * sh[(size_t)t * N + c];
+  x[(size_t)t * N + c] += v;
+}

@@ -1,0 +1,101 @@
+// "ops" module: the activation quantizer that feeds every block-quantized matmul, alone and fused into the two
+// producers the matmul path uses (RMS norm, SwiGLU).
+//
+// Arithmetic per block of 32 (act32) or 256 values, as the reference's quant_store16 (zero/kernels/ops.cl:38-72,
+// CPU twin src/quants.h:626-643):  amax = max |v|;  inv = amax > 0 ? 127 / amax : 0;  q = rte(v * inv) (one f32
+// multiply, then round to nearest even);  scale = amax / 127 (a true division);  absum = int16 sum of each 16 q.
+// Layouts: aq [M][K] int8, asc [K/32][M] (or [K/256][M]) f32, absum [K/16][M] int16.  Rows m >= T are written as
+// zeros with scale 0 (the padding rows of a prompt chunk).
+//
+// Mapping: a work-group of 256 threads takes one superblock (256 values) of 64 token rows.  Thread t holds 16
+// consecutive values of one row (16 threads = one row's superblock, read as one contiguous KiB); the two threads of a
+// 32-block exchange their maxima with one cross-lane move.  Scales and sums go through LDS so that they leave as
+// runs of 64 consecutive tokens (the token-minor layout the matmuls read).
+#include "quant.h"
+
+// Shared tail of the row kernels: stores one tile's scales and sums token-minor.
+struct QuantTile {
+  float asc[8][64];
+  short sum[16][64];
+};
+
+__device__ inline void store_tile_scales(const QuantTile& lds, int s, int m0, int M, int act32, float* asc,
+                                         short* absum) {
+  const int t = threadIdx.x;
+  if (act32) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = t + 256 * i, b = idx >> 6, r = idx & 63;
+      if (m0 + r < M) asc[((size_t)s * 8 + b) * M + m0 + r] = lds.asc[b][r];
+    }
+  } else if (t < 64) {
+    if (m0 + t < M) asc[(size_t)s * M + m0 + t] = lds.asc[0][t];
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = t + 256 * i, h = idx >> 6, r = idx & 63;
+    if (m0 + r < M) absum[((size_t)s * 16 + h) * M + m0 + r] = lds.sum[h][r];
+  }
+}
+
+// quant_rows: x [T][ldx] f32 -> aq / asc / absum for M rows (rows >= T zero).  grid (K/256, ceil(M/64)), local 256.
+extern "C" __global__ __launch_bounds__(256) void quant_rows(const float* __restrict__ x, int ldx, int K, int M, int T,
+                                                             signed char* __restrict__ aq, float* __restrict__ asc,
+                                                             short* __restrict__ absum, int act32) {
+  __shared__ QuantTile lds;
+  const int s = blockIdx.x, m0 = blockIdx.y * 64;
+  const int lane16 = threadIdx.x & 15, rg = threadIdx.x >> 4;
+#pragma unroll 1
+  for (int p = 0; p < 4; ++p) {
+    const int r = p * 16 + rg, m = m0 + r;
+    float v[16];
+    if (m < T) {
+      const float4* src = (const float4*)(x + (size_t)m * ldx + s * 256 + 16 * lane16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 f = src[i];
+        v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) v[i] = 0.0f;
+    }
+    const float amax = block_amax(v, act32);
+    uint4 pk;
+    int sum;
+    quant16(v, amax, pk, sum);
+    if (m < M) *(uint4*)(aq + (size_t)m * K + s * 256 + 16 * lane16) = pk;
+    lds.sum[lane16][r] = (short)sum;
+    if (act32) {
+      if ((lane16 & 1) == 0) lds.asc[lane16 >> 1][r] = amax / 127.0f;
+    } else if (lane16 == 0) {
+      lds.asc[0][r] = amax / 127.0f;
+    }
+  }
+  __syncthreads();
+  store_tile_scales(lds, s, m0, M, act32, asc, absum);
+}
+
+// fill32: p[i] = v for i < n (the fill used where a captured graph must not hold a memset node).
+extern "C" __global__ void fill32(uint32_t* p, uint32_t v, size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// copy128: dst[i] = src[i] over n 16-byte units; the plain streaming copy the bandwidth probe and the counter
+// calibration use.
+extern "C" __global__ void copy128(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+// read_probe: streams n 16-byte units and folds them into one word per thread (written only if it is the impossible
+// value, so the loads cannot be dropped): the read-bandwidth probe (the reference's Engine::read_gbs pattern,
+// zero/engine.h:154-208).
+extern "C" __global__ void read_probe(const uint4* __restrict__ src, size_t n, uint32_t* sink) {
+  uint32_t acc = 0;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const uint4 v = src[i];
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == 0x9E3779B9u) sink[0] = acc;
+}

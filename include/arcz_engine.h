@@ -1,0 +1,84 @@
+/*
+ * arcz_engine.h -- the C ABI of the matmul dispatch: what the reference's Engine (zero/engine.h) offers for this
+ * path, callable from any language.  The C++ class behind it (arcinferzero_amd/csrc/engine_hip.h) keeps the
+ * reference's method names and argument meaning; a C++ caller can use that class directly.
+ *
+ * Every call returns 0 or a negative status; arcz_engine_error() gives the message of the last failure (the C++
+ * methods throw std::runtime_error / std::logic_error as the reference's do; the exceptions stop here).
+ * One engine per process is the expected use; all engines share the one stream of arcz_hip.h.
+ */
+#ifndef ARCZ_ENGINE_H
+#define ARCZ_ENGINE_H
+#include "arcz_hip.h"
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ARCZ_E_ENGINE (-100) /* an exception of the dispatch code: bad shapes, unsupported type, unloaded weight */
+
+typedef struct arcz_engine arcz_engine;
+typedef struct arcz_weight arcz_weight;       /* GpuWeight (zero/engine.h:27-34) */
+typedef struct arcz_moe_layer arcz_moe_layer; /* the expert tensors of one layer (zero/engine_stream.h:285-306) */
+
+const char* arcz_engine_error(void);
+
+/* Engine::Engine + alloc_buffers (zero/engine.h:268, zero/engine_alloc.h:4-41): activation buffers for chunks of up
+ * to max_chunk token rows of up to max_k values (aq int8 [M][K], asc f32 [K/32][M], absum int16 [K/16][M]). */
+arcz_engine* arcz_engine_create(int max_chunk, int max_k);
+void arcz_engine_destroy(arcz_engine* e);
+
+/* make_weight + upload_padded (zero/engine_load.h:84-130, 157-196): N rows of K values as GGUF blocks of `type`
+ * (8 = Q8_0, 12 = Q4_K, 14 = Q6_K), regrouped into the device layout and uploaded. */
+arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, const void* gguf, size_t bytes);
+int arcz_weight_free(arcz_engine* e, arcz_weight* w);
+arcz_mem* arcz_weight_raw(const arcz_weight* w);
+
+/* The activation quantizer as a step of its own (quant_store16 of zero/kernels/ops.cl:38-72 inside the launch of
+ * zero/engine.h:1256-1267): rows [0, T) of x (f32, row stride ldx) -> the engine's aq / asc / absum laid out for
+ * Mp rows; rows [T, Mp) are zero.  The next matmul takes its form from T: 1 GEMV, 2..8 multi-token GEMV, else GEMM. */
+int arcz_engine_quantize(arcz_engine* e, arcz_mem* x, int ldx, int K, int Mp, int T, int act32);
+/* Activations quantized by the caller, as the reference's benches do (bench/gemv_bench.cpp:103-129). */
+int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp,
+                                int T);
+/* The engine's activation buffers (Engine::aq_, asc_, absum_; zero/engine_sessions.h:571). */
+arcz_mem* arcz_engine_aq(arcz_engine* e);
+arcz_mem* arcz_engine_asc(arcz_engine* e);
+arcz_mem* arcz_engine_absum(arcz_engine* e);
+
+/* Engine::matmul(name, w, Mp, C, ldc, c_off, acc, act32) (zero/engine.h:1080): C[:, c_off : c_off + N] (+)= act W^T
+ * for the current chunk.  acc 0 = store, 1 = add to C, 2 = C = silu(C) * result (GEMM form only). */
+int arcz_engine_matmul(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off, int acc,
+                       int act32);
+
+/* Expert tensors of one MoE layer: gate, up [NE][F][E] and down [NE][E][F] as GGUF blocks of `type`. */
+arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, const void* up, const void* down,
+                                      int NE, int NU, int E, int F);
+/* Engine::layer_moe (zero/engine_moe.h:8-361, standard experts, no shared expert): x[t] += sum_k w_k expert_k(h[t]) for
+ * the T tokens whose quantized h is the current activation chunk; logits: router logits [T][ldl] f32. */
+int arcz_engine_layer_moe(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp);
+/* The routing step alone (moe_route + moe_scan + moe_scatter, zero/engine_moe.h:111-133) with tiles of tm slots, and
+ * its buffers: which = 0 ids, 1 wts, 2 offs, 3 tiles, 4 tstart, 5 stok, 6 swt, 7 inv, 8 h (f32), 9 hq, 10 hsc, 11 y. */
+int arcz_engine_moe_route(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, int T, int tm);
+arcz_mem* arcz_engine_moe_buffer(arcz_engine* e, int which);
+int arcz_engine_moe_slots(arcz_engine* e);
+
+/* Engine::profile / collect_profile (zero/engine.h:936-950): per-launch device time summed by name. */
+void arcz_engine_profile(arcz_engine* e, int on);
+int arcz_engine_profile_collect(arcz_engine* e);
+int arcz_engine_profile_get(arcz_engine* e, const char* name, double* ms, int* launches);
+void arcz_engine_profile_reset(arcz_engine* e);
+uint64_t arcz_engine_rd_bytes(arcz_engine* e);
+
+/* Host helpers (no GPU): byte counts, the GGUF -> device planes regrouping, quantizers and seeded generators. */
+size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
+size_t arcz_planes_bytes(uint32_t type, size_t rows, int K);
+int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* planes);
+/* quantize_rows_q8_0 (src/quants.h:429-442) and this library's own Q4_K / Q6_K block makers (input generators). */
+int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out);
+void arcz_gen_normal(uint64_t seed, size_t n, float mean, float std, float* out);
+int arcz_gen_weights(uint32_t type, uint64_t seed, size_t N, int K, float std, uint8_t* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

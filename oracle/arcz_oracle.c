@@ -1,0 +1,540 @@
+/*
+ * CPU oracle for the GGUF block-quantized matmul path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain C, the arithmetic of the reference engine for the path this repository accelerates.
+ * It is the checker that tests, the smoke check and the bench's cpu_baseline leg compare the HIP kernels with;
+ * nothing in the shipped library links, loads or calls it.
+ *
+ * Every function names the reference lines it follows (paths relative to the reference tree).
+ *
+ * Pin status (what holds each function to the reference, see tests/test_oracle_*.py):
+ *   orc_fp16_to_f32 / orc_f32_to_fp16   all 65,536 patterns vs numpy.float16; random + tie f32 inputs vs numpy and
+ *                                       vs the compiled reference header (oracle/_ref)
+ *   orc_decode_sb / orc_dequant_row     closed-form blocks with exact binary fractions; pack/unpack brute force;
+ *                                       golden vectors and live comparison with the compiled reference header
+ *   orc_quantize_act                    closed forms (max -> +-127, zero block, ties to even); golden + compiled ref
+ *   orc_quantize_rows_q8_0              golden + compiled ref; round trip bound
+ *   orc_block_sums                      brute-force integer sums in numpy (int64)
+ *   orc_matmul_ref                      numpy float64 dot of dequantized rows; unit-scale known answer
+ *   orc_matmul_formula                  against orc_matmul_ref within float rounding; unit-scale known answer (exact)
+ *   orc_moe_route                       stable-sort top-k in numpy (the reference's own CPU check, tests/test_route.cpp:28-44)
+ *   orc_moe_scan / orc_moe_scatter      invariants (bijection, contiguity, counts) + numpy restatement
+ *   orc_moe_layer                       composition of the above, compared with a numpy float64 composition
+ * The f32 -> Q4_K / Q6_K quantizers used to make synthetic weights are not part of the reference (it has none) and
+ * not part of this file: they are input generators of the product's bench/test utilities; parity unpinned by design.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_Q8_0 8u
+#define ORC_Q4_K 12u
+#define ORC_Q6_K 14u
+
+/* ---------------------------------------------------------------- fp16 (src/quants.h:17-52) */
+
+/* IEEE binary16 -> f32, exact; subnormals normalized (src/quants.h:17-31). */
+float orc_fp16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1Fu, m = h & 0x3FFu, bits;
+  if (e == 0) {
+    if (m == 0) {
+      bits = sign;
+    } else {
+      int ex = 127 - 15 + 1;
+      while (!(m & 0x400u)) { m <<= 1; --ex; }
+      bits = sign | ((uint32_t)ex << 23) | ((m & 0x3FFu) << 13);
+    }
+  } else if (e == 31) {
+    bits = sign | 0x7F800000u | (m << 13);
+  } else {
+    bits = sign | ((e + 127 - 15) << 23) | (m << 13);
+  }
+  float r;
+  memcpy(&r, &bits, 4);
+  return r;
+}
+
+/* f32 -> binary16, round to nearest even, NaN -> quiet, overflow -> inf, below 2^-25 -> signed zero
+ * (src/quants.h:33-52). */
+uint16_t orc_f32_to_fp16(float x) {
+  uint32_t f;
+  memcpy(&f, &x, 4);
+  const uint32_t sign = (f >> 16) & 0x8000u;
+  const uint32_t e8 = (f >> 23) & 0xFFu;
+  uint32_t mant = f & 0x7FFFFFu;
+  const int32_t e = (int32_t)e8 - 127 + 15;
+  if (e8 == 0xFF) return (uint16_t)(sign | 0x7C00u | (mant ? 0x200u : 0u));
+  if (e >= 31) return (uint16_t)(sign | 0x7C00u);
+  if (e <= 0) {
+    if (e < -10) return (uint16_t)sign;
+    mant |= 0x800000u;
+    const uint32_t shift = (uint32_t)(14 - e);
+    uint32_t h = mant >> shift;
+    const uint32_t rem = mant & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (h & 1u))) ++h;
+    return (uint16_t)(sign | h);
+  }
+  uint32_t h = sign | ((uint32_t)e << 10) | (mant >> 13);
+  const uint32_t rem = mant & 0x1FFFu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;
+  return (uint16_t)h;
+}
+
+/* ---------------------------------------------------------------- block formats (src/gguf.h:48-79) */
+
+/* Bytes of one 256-element superblock in GGUF (src/gguf.h:59,62,64; src/quants.h:327-331). 0 = unsupported. */
+int orc_sb_bytes(uint32_t type) {
+  switch (type) {
+    case ORC_Q8_0: return 34 * 8;
+    case ORC_Q4_K: return 144;
+    case ORC_Q6_K: return 210;
+    default: return 0;
+  }
+}
+
+/* 6-bit scale / min of sub-block j of a Q4_K superblock from its 12 packed bytes (src/quants.h:61-69). */
+static void scale_min_k4(int j, const uint8_t* q, int* sc, int* mn) {
+  if (j < 4) {
+    *sc = q[j] & 63;
+    *mn = q[j + 4] & 63;
+  } else {
+    *sc = (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4);
+    *mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+  }
+}
+
+/*
+ * One decoded superblock (the fields of the reference's DecodedSB that the three types use, src/quants.h:72-84).
+ *   Q4_K: q 0..15, sc[8], mn[8], d, dmin        (src/quants.h:91-113)
+ *   Q6_K: q 0..63 (offset 32 NOT removed), sc6[16], d   (src/quants.h:115-134)
+ *   Q8_0: q -128..127, d8[8]                    (src/quants.h:149-157)
+ */
+typedef struct {
+  float d, dmin;
+  int sc[8], mn[8];
+  int sc6[16];
+  float d8[8];
+  int16_t q[256];
+} orc_sb;
+
+static uint16_t rd16(const uint8_t* p) { uint16_t v; memcpy(&v, p, 2); return v; }
+
+int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
+  memset(o, 0, sizeof *o);
+  if (type == ORC_Q4_K) {
+    o->d = orc_fp16_to_f32(rd16(p));
+    o->dmin = orc_fp16_to_f32(rd16(p + 2));
+    for (int b = 0; b < 8; ++b) scale_min_k4(b, p + 4, &o->sc[b], &o->mn[b]);
+    const uint8_t* qs = p + 16;
+    for (int j = 0; j < 4; ++j)
+      for (int l = 0; l < 32; ++l) {
+        o->q[64 * j + l] = (int16_t)(qs[32 * j + l] & 0xF);
+        o->q[64 * j + 32 + l] = (int16_t)(qs[32 * j + l] >> 4);
+      }
+    return 0;
+  }
+  if (type == ORC_Q6_K) {
+    const uint8_t *ql = p, *qh = p + 128;
+    const int8_t* sc = (const int8_t*)(p + 192);
+    o->d = orc_fp16_to_f32(rd16(p + 208));
+    for (int i = 0; i < 16; ++i) o->sc6[i] = sc[i];
+    for (int n = 0; n < 2; ++n)
+      for (int l = 0; l < 32; ++l) {
+        const uint8_t *L = ql + 64 * n, *H = qh + 32 * n;
+        o->q[128 * n + l + 0] = (int16_t)((L[l] & 0xF) | (((H[l] >> 0) & 3) << 4));
+        o->q[128 * n + l + 32] = (int16_t)((L[l + 32] & 0xF) | (((H[l] >> 2) & 3) << 4));
+        o->q[128 * n + l + 64] = (int16_t)((L[l] >> 4) | (((H[l] >> 4) & 3) << 4));
+        o->q[128 * n + l + 96] = (int16_t)((L[l + 32] >> 4) | (((H[l] >> 6) & 3) << 4));
+      }
+    return 0;
+  }
+  if (type == ORC_Q8_0) {
+    for (int b = 0; b < 8; ++b) {
+      const uint8_t* blk = p + 34 * b;
+      o->d8[b] = orc_fp16_to_f32(rd16(blk));
+      for (int i = 0; i < 32; ++i) o->q[32 * b + i] = (int8_t)blk[2 + i];
+    }
+    return 0;
+  }
+  return -1;
+}
+
+/* Value of element e of a decoded superblock, f32, evaluated left to right as written (src/quants.h:317-324). */
+static float sb_value(uint32_t type, const orc_sb* o, int e) {
+  if (type == ORC_Q4_K) return o->d * (float)o->sc[e / 32] * (float)o->q[e] - o->dmin * (float)o->mn[e / 32];
+  if (type == ORC_Q6_K) return o->d * (float)o->sc6[e / 16] * (float)(o->q[e] - 32);
+  return o->d8[e / 32] * (float)o->q[e];
+}
+
+/* The signed integer the int8 dot product sees for element e: Q4_K q (0..15), Q6_K q - 32, Q8_0 q
+ * (zero/kernels/decode.cl:221-260). */
+static int sb_int(uint32_t type, const orc_sb* o, int e) { return type == ORC_Q6_K ? o->q[e] - 32 : o->q[e]; }
+
+/* One row of K elements to f32 (src/quants.h:519, generic tail 617-621).  K % 256 == 0. */
+int orc_dequant_row(uint32_t type, const uint8_t* row, int K, float* out) {
+  const int bb = orc_sb_bytes(type);
+  if (!bb || K % 256) return -1;
+  orc_sb o;
+  for (int s = 0; s < K / 256; ++s) {
+    orc_decode_sb(type, row + (size_t)s * bb, &o);
+    for (int e = 0; e < 256; ++e) out[s * 256 + e] = sb_value(type, &o, e);
+  }
+  return 0;
+}
+
+/* Decoded integer fields of one row, for tests: q [K] (as the dot product sees them), isc [K/16] integer sub-scale
+ * per 16 elements (Q4_K: the block's 6-bit scale twice, Q6_K: the int8 scales, Q8_0: 1), imn [K/16] (Q4_K mins twice,
+ * else 0), d [K/32] f32 scale per 32-block (Q4_K / Q6_K: the superblock's d repeated), dmin [K/32]. */
+int orc_decode_row_fields(uint32_t type, const uint8_t* row, int K, int8_t* q, int32_t* isc, int32_t* imn, float* d,
+                          float* dmin) {
+  const int bb = orc_sb_bytes(type);
+  if (!bb || K % 256) return -1;
+  orc_sb o;
+  for (int s = 0; s < K / 256; ++s) {
+    orc_decode_sb(type, row + (size_t)s * bb, &o);
+    for (int e = 0; e < 256; ++e) q[s * 256 + e] = (int8_t)sb_int(type, &o, e);
+    for (int h = 0; h < 16; ++h) {
+      isc[s * 16 + h] = type == ORC_Q4_K ? o.sc[h / 2] : type == ORC_Q6_K ? o.sc6[h] : 1;
+      imn[s * 16 + h] = type == ORC_Q4_K ? o.mn[h / 2] : 0;
+    }
+    for (int b = 0; b < 8; ++b) {
+      d[s * 8 + b] = type == ORC_Q8_0 ? o.d8[b] : o.d;
+      dmin[s * 8 + b] = type == ORC_Q4_K ? o.dmin : 0.0f;
+    }
+  }
+  return 0;
+}
+
+/* ---------------------------------------------------------------- quantizers */
+
+/* Activation quantizer: int8 per block of 32 (act32) or 256 with an absmax scale, and the int16 sum of every 16
+ * int8 values.  aq [M][K], asc [K/B][M], absum [K/16][M]  (src/quants.h:626-643 == zero/kernels/ops.cl:38-72).
+ * inv = 127/amax, q = lrintf(v * inv) under round-to-nearest-even, scale = amax / 127. */
+void orc_quantize_act(const float* x, int M, int K, int8_t* aq, float* asc, int16_t* absum, int act32) {
+  const int B = act32 ? 32 : 256;
+  for (int m = 0; m < M; ++m)
+    for (int b0 = 0; b0 < K; b0 += B) {
+      const float* v = x + (size_t)m * K + b0;
+      float amax = 0;
+      for (int i = 0; i < B; ++i) amax = fmaxf(amax, fabsf(v[i]));
+      const float inv = amax > 0 ? 127.0f / amax : 0.0f;
+      asc[(size_t)(b0 / B) * M + m] = amax / 127.0f;
+      for (int i = 0; i < B; ++i) {
+        const float p = v[i] * inv; /* one f32 multiply, no fma */
+        aq[(size_t)m * K + b0 + i] = (int8_t)lrintf(p);
+      }
+    }
+  for (int m = 0; m < M; ++m)
+    for (int b = 0; b < K / 16; ++b) {
+      int sum = 0;
+      for (int i = 0; i < 16; ++i) sum += aq[(size_t)m * K + b * 16 + i];
+      absum[(size_t)b * M + m] = (int16_t)sum;
+    }
+}
+
+/* The expert input quantizer (zero/kernels/moe.cl:258-274): as orc_quantize_act with act32, rows of F values, scales
+ * hsc [(F/32)][S] with row stride S (the slot count), no sums. */
+void orc_moe_quant(const float* h, int n, int F, int S, int8_t* hq, float* hsc) {
+  for (int r = 0; r < n; ++r)
+    for (int b = 0; b < F / 32; ++b) {
+      const float* v = h + (size_t)r * F + 32 * b;
+      float amax = 0;
+      for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
+      const float inv = amax > 0 ? 127.0f / amax : 0.0f;
+      hsc[(size_t)b * S + r] = amax / 127.0f;
+      for (int i = 0; i < 32; ++i) {
+        const float p = v[i] * inv;
+        hq[(size_t)r * F + 32 * b + i] = (int8_t)lrintf(p);
+      }
+    }
+}
+
+/* f32 rows [N][K] -> GGUF Q8_0 blocks: d = amax / 127 (stored as fp16 of that f32), q = lrintf(v * (1 / d)) with the
+ * f32 d, not the rounded one (src/quants.h:429-442). out: N * K/32 * 34 bytes. */
+void orc_quantize_rows_q8_0(const float* src, int N, int K, uint8_t* out) {
+  for (size_t b = 0; b < (size_t)N * (size_t)(K / 32); ++b) {
+    const float* v = src + b * 32;
+    float amax = 0;
+    for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    const float d = amax / 127.0f, inv = d > 0 ? 1.0f / d : 0.0f;
+    uint8_t* blk = out + b * 34;
+    const uint16_t dh = orc_f32_to_fp16(d);
+    memcpy(blk, &dh, 2);
+    for (int i = 0; i < 32; ++i) {
+      const float p = v[i] * inv;
+      blk[2 + i] = (uint8_t)(int8_t)lrintf(p);
+    }
+  }
+}
+
+/* ---------------------------------------------------------------- integer block sums */
+
+/* I [M][N][K/16]: the int32 dot product of every 16-element half block of weight row n with token row m
+ * (zero/kernels/decode.cl:992-999: lo / hi).  A 32-block's sum is the sum of its two halves. */
+int orc_block_sums(uint32_t type, const uint8_t* W, int N, int K, const int8_t* aq, int M, int32_t* I) {
+  const int bb = orc_sb_bytes(type), nsb = K / 256;
+  if (!bb || K % 256) return -1;
+#pragma omp parallel for schedule(dynamic, 16)
+  for (int n = 0; n < N; ++n) {
+    orc_sb o;
+    for (int s = 0; s < nsb; ++s) {
+      orc_decode_sb(type, W + ((size_t)n * nsb + s) * bb, &o);
+      for (int m = 0; m < M; ++m)
+        for (int h = 0; h < 16; ++h) {
+          int32_t acc = 0;
+          for (int i = 0; i < 16; ++i) acc += sb_int(type, &o, 16 * h + i) * (int32_t)aq[(size_t)m * K + s * 256 + 16 * h + i];
+          I[((size_t)m * N + n) * (K / 16) + s * 16 + h] = acc;
+        }
+    }
+  }
+  return 0;
+}
+
+/* ---------------------------------------------------------------- f32 references */
+
+/* Y[m][n] = (float) sum_k (double)dequant(W)[n][k] * (double)((float)aq[m][k] * asc[k/32][m]): the reference's CPU
+ * matmul (tools/ref_forward.cpp:268-303: OpenMP over output rows, schedule(dynamic, 16), dequant_row once per row,
+ * double-accumulated dot per token) on activations rounded as the engine rounds them
+ * (tools/ref_forward.cpp:109-126 round_int8 with B = 32; bench/gemv_bench.cpp:121-123, 203-207: xq = q * sc).
+ * asc has row stride Ms (>= M).  Y row stride ldy. */
+int orc_matmul_ref(uint32_t type, const uint8_t* W, int N, int K, const int8_t* aq, const float* asc, int Ms, int M,
+                   float* Y, int ldy) {
+  const int bb = orc_sb_bytes(type), nsb = K / 256;
+  if (!bb || K % 256) return -1;
+  float* X = (float*)malloc((size_t)M * K * sizeof(float));
+  if (!X) return -2;
+  for (int m = 0; m < M; ++m)
+    for (int k = 0; k < K; ++k) X[(size_t)m * K + k] = (float)aq[(size_t)m * K + k] * asc[(size_t)(k / 32) * Ms + m];
+#pragma omp parallel
+  {
+    float* w = (float*)malloc((size_t)K * sizeof(float));
+#pragma omp for schedule(dynamic, 16)
+    for (int n = 0; n < N; ++n) {
+      orc_dequant_row(type, W + (size_t)n * nsb * bb, K, w);
+      for (int m = 0; m < M; ++m) {
+        double acc = 0;
+        const float* x = X + (size_t)m * K;
+        for (int k = 0; k < K; ++k) acc += (double)w[k] * x[k];
+        Y[(size_t)m * ldy + n] = (float)acc;
+      }
+    }
+    free(w);
+  }
+  free(X);
+  return 0;
+}
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+/* The engine's own arithmetic, in f32, from the integer block sums.
+ *   form 0 (GEMV, zero/kernels/decode.cl:1000-1003), per 32-block b in order:
+ *     Q4_K: acc += sa * (d * (float)(sc*lo + sc*hi) - dmin * (float)(mn*bs0 + mn*bs1))
+ *     Q6_K / Q8_0: acc += sa * d * (float)(sc0*lo + sc1*hi)
+ *   form 1 (GEMM with per-32 activation scales, zero/kernels/gemm.cl:439-488), per superblock, block pairs (2j, 2j+1):
+ *     Q4_K: tq = fma(avl,(float)plo, fma(avh,(float)phi,tq)); tmn likewise; res = fma(d,tq, fma(-dmin,tmn,res))
+ *     Q6_K: plo = acc0*sc0 + acc1*sc1; tq as above; res = fma(d,tq,res)
+ *     Q8_0: res = fma(avl*dlo,(float)acc0, fma(avh*dhi,(float)acc1,res))
+ * The reference's lanes add their partial sums in an implementation-defined tree (sub_group_reduce_add); this
+ * restatement adds in block order, so it is a second f32 evaluation to compare within rounding, not bit for bit. */
+int orc_matmul_formula(uint32_t type, int form, const uint8_t* W, int N, int K, const int8_t* aq, const float* asc,
+                       const int16_t* absum, int Ms, int M, float* Y, int ldy) {
+  const int bb = orc_sb_bytes(type), nsb = K / 256;
+  if (!bb || K % 256) return -1;
+#pragma omp parallel for schedule(dynamic, 16)
+  for (int n = 0; n < N; ++n) {
+    orc_sb o;
+    for (int m = 0; m < M; ++m) {
+      float res = 0.0f;
+      for (int s = 0; s < nsb; ++s) {
+        orc_decode_sb(type, W + ((size_t)n * nsb + s) * bb, &o);
+        int32_t h16[16];
+        for (int h = 0; h < 16; ++h) {
+          int32_t acc = 0;
+          for (int i = 0; i < 16; ++i) acc += sb_int(type, &o, 16 * h + i) * (int32_t)aq[(size_t)m * K + s * 256 + 16 * h + i];
+          h16[h] = acc;
+        }
+        float tq = 0.0f, tmn = 0.0f;
+        for (int j = 0; j < 4; ++j) {
+          float t2[2], m2[2], sa2[2];
+          for (int u = 0; u < 2; ++u) {
+            const int b = 2 * j + u;
+            const float sa = asc[(size_t)(s * 8 + b) * Ms + m];
+            const int lo = h16[2 * b], hi = h16[2 * b + 1];
+            const int bs0 = absum[(size_t)(s * 16 + 2 * b) * Ms + m], bs1 = absum[(size_t)(s * 16 + 2 * b + 1) * Ms + m];
+            sa2[u] = sa;
+            if (type == ORC_Q4_K) {
+              t2[u] = (float)(o.sc[b] * lo + o.sc[b] * hi);
+              m2[u] = (float)(o.mn[b] * bs0 + o.mn[b] * bs1);
+              if (form == 0) res += sa * (o.d * t2[u] - o.dmin * m2[u]);
+            } else if (type == ORC_Q6_K) {
+              t2[u] = (float)(o.sc6[2 * b] * lo + o.sc6[2 * b + 1] * hi);
+              m2[u] = 0.0f;
+              if (form == 0) res += sa * o.d * t2[u];
+            } else {
+              t2[u] = (float)(lo + hi);
+              m2[u] = 0.0f;
+              if (form == 0) res += sa * o.d8[b] * t2[u];
+            }
+          }
+          if (form == 1) {
+            if (type == ORC_Q8_0) {
+              res = fmaf(sa2[0] * o.d8[2 * j], t2[0], fmaf(sa2[1] * o.d8[2 * j + 1], t2[1], res));
+            } else {
+              tq = fmaf(sa2[0], t2[0], fmaf(sa2[1], t2[1], tq));
+              tmn = fmaf(sa2[0], m2[0], fmaf(sa2[1], m2[1], tmn));
+            }
+          }
+        }
+        if (form == 1 && type == ORC_Q4_K) res = fmaf(o.d, tq, fmaf(-o.dmin, tmn, res));
+        if (form == 1 && type == ORC_Q6_K) res = fmaf(o.d, tq, res);
+      }
+      Y[(size_t)m * ldy + n] = res;
+    }
+  }
+  return 0;
+}
+
+/* ---------------------------------------------------------------- mixture of experts */
+
+/* silu as the CPU reference evaluates it (tools/ref_forward.cpp:321): below -80 the result is 0. */
+float orc_silu(float x) { return x < -80.0f ? 0.0f : x / (1.0f + expf(-x)); }
+
+/* Routing of T tokens (zero/kernels/moe.cl:50-89): the NU largest of NE logits (ties: the lower expert id),
+ * p_k = exp(l_k - max l), weights p_k / sum of the selected p; per-expert counts; sgate = sigmoid(l[NE]) when the
+ * row has a shared-expert logit at column NE (ldl > NE), else 0.5 is NOT written: sgate may be NULL. */
+void orc_moe_route(const float* logits, int ldl, int T, int NE, int NU, int32_t* ids, float* wts, float* sgate,
+                   int32_t* counts) {
+  for (int e = 0; e < NE; ++e) counts[e] = 0;
+  float* v = (float*)malloc((size_t)NE * sizeof(float));
+  for (int t = 0; t < T; ++t) {
+    const float* lg = logits + (size_t)t * ldl;
+    float mx = -INFINITY;
+    for (int e = 0; e < NE; ++e) { v[e] = lg[e]; mx = fmaxf(mx, v[e]); }
+    float p[64], sum = 0.0f;
+    int sel[64];
+    for (int k = 0; k < NU; ++k) {
+      float bv = -INFINITY;
+      int bi = NE;
+      for (int e = 0; e < NE; ++e)
+        if (v[e] > bv) { bv = v[e]; bi = e; } /* strict >: the lowest index of equal values wins */
+      if (bi < NE) v[bi] = -INFINITY;
+      sel[k] = bi < NE - 1 ? bi : NE - 1; /* (a row of NaN picks nothing: clamped as moe.cl:77) */
+      p[k] = expf(bv - mx);
+      sum += p[k];
+    }
+    for (int k = 0; k < NU; ++k) {
+      ids[(size_t)t * NU + k] = sel[k];
+      wts[(size_t)t * NU + k] = p[k] / sum;
+      counts[sel[k]]++;
+    }
+    if (sgate) sgate[t] = ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
+  }
+  free(v);
+}
+
+/* Exclusive scan of the counts and the tile list (zero/kernels/moe.cl:141-168): offs[e], tstart[e] (first tile of
+ * expert e), tstart[NE] = tile count, tiles[0] = tile count then (expert, first slot, rows <= TM) per tile. */
+void orc_moe_scan(const int32_t* counts, int NE, int TM, int32_t* offs, int32_t* tiles, int32_t* tstart) {
+  int off = 0, toff = 0;
+  for (int e = 0; e < NE; ++e) {
+    const int c = counts[e], nt = (c + TM - 1) / TM;
+    offs[e] = off;
+    tstart[e] = toff;
+    for (int i = 0; i < nt; ++i) {
+      tiles[1 + 3 * (toff + i) + 0] = e;
+      tiles[1 + 3 * (toff + i) + 1] = off + i * TM;
+      tiles[1 + 3 * (toff + i) + 2] = c - i * TM < TM ? c - i * TM : TM;
+    }
+    off += c;
+    toff += nt;
+  }
+  tiles[0] = tstart[NE] = toff;
+}
+
+/* Slots in pair order (zero/kernels/moe.cl:171-179 with its atomic counter replaced by the serial order; the
+ * reference's slot order inside an expert is not deterministic, its results are). */
+void orc_moe_scatter(const int32_t* ids, const float* wts, int n, int NU, const int32_t* offs, int NE, int32_t* stok,
+                     float* swt, int32_t* inv) {
+  int32_t* cur = (int32_t*)malloc((size_t)NE * sizeof(int32_t));
+  memcpy(cur, offs, (size_t)NE * sizeof(int32_t));
+  for (int i = 0; i < n; ++i) {
+    const int s = cur[ids[i]]++;
+    stok[s] = i / NU;
+    swt[s] = wts[i];
+    inv[i] = s;
+  }
+  free(cur);
+}
+
+/* One MoE FFN over T tokens (zero/engine_moe.h:8-361 with standard expert tensors and no shared expert;
+ * tools/ref_forward.cpp:333-364 expert_mv per (token, expert)):
+ *   route -> per pair: g = Wg_e x, u = Wu_e x (x = the token's int8-rounded input), h = silu(g) * u,
+ *   h rounded to int8 per 32 (zero/kernels/moe.cl:258-274), v = Wd_e h, y = w * v; out[t] = sum_k y (k order,
+ *   zero/kernels/moe.cl:349-351).
+ * Dot products as orc_matmul_ref (double accumulation of dequantized weights).  The gate / up sums are rounded to
+ * f32 before the SwiGLU, as the engine stores them.  Wg, Wu: [NE][F][E] rows, Wd: [NE][E][F] rows, GGUF blocks.
+ * Also returns h [T*NU][F] (pair order) when h_out is not NULL. */
+int orc_moe_layer(uint32_t type, const uint8_t* Wg, const uint8_t* Wu, const uint8_t* Wd, int NE, int NU, int E, int F,
+                  const int8_t* aq, const float* asc, int Ms, int T, const float* logits, int ldl, float* out,
+                  float* h_out) {
+  const int bb = orc_sb_bytes(type);
+  if (!bb || E % 256 || F % 256) return -1;
+  const size_t rbE = (size_t)(E / 256) * bb, rbF = (size_t)(F / 256) * bb;
+  int32_t* ids = (int32_t*)malloc((size_t)T * NU * 4);
+  float* wts = (float*)malloc((size_t)T * NU * 4);
+  int32_t* counts = (int32_t*)malloc((size_t)NE * 4);
+  orc_moe_route(logits, ldl, T, NE, NU, ids, wts, NULL, counts);
+  memset(out, 0, (size_t)T * E * sizeof(float));
+  float* Y = (float*)malloc((size_t)T * NU * E * sizeof(float));
+#pragma omp parallel
+  {
+    float* w = (float*)malloc((size_t)(E > F ? E : F) * sizeof(float));
+    float* x = (float*)malloc((size_t)E * sizeof(float));
+    float* h = (float*)malloc((size_t)F * sizeof(float));
+    int8_t* hq = (int8_t*)malloc((size_t)F);
+    float* hs = (float*)malloc((size_t)(F / 32) * sizeof(float));
+    float* hx = (float*)malloc((size_t)F * sizeof(float));
+#pragma omp for schedule(dynamic, 4)
+    for (int i = 0; i < T * NU; ++i) {
+      const int t = i / NU, e = ids[i];
+      for (int k = 0; k < E; ++k) x[k] = (float)aq[(size_t)t * E + k] * asc[(size_t)(k / 32) * Ms + t];
+      for (int f = 0; f < F; ++f) {
+        double g = 0, u = 0;
+        orc_dequant_row(type, Wg + ((size_t)e * F + f) * rbE, E, w);
+        for (int k = 0; k < E; ++k) g += (double)w[k] * x[k];
+        orc_dequant_row(type, Wu + ((size_t)e * F + f) * rbE, E, w);
+        for (int k = 0; k < E; ++k) u += (double)w[k] * x[k];
+        h[f] = orc_silu((float)g) * (float)u;
+      }
+      if (h_out) memcpy(h_out + (size_t)i * F, h, (size_t)F * sizeof(float));
+      orc_moe_quant(h, 1, F, 1, hq, hs);
+      for (int f = 0; f < F; ++f) hx[f] = (float)hq[f] * hs[f / 32];
+      for (int c = 0; c < E; ++c) {
+        double v = 0;
+        orc_dequant_row(type, Wd + ((size_t)e * E + c) * rbF, F, w);
+        for (int f = 0; f < F; ++f) v += (double)w[f] * hx[f];
+        Y[(size_t)i * E + c] = wts[i] * (float)v;
+      }
+    }
+    free(w); free(x); free(h); free(hq); free(hs); free(hx);
+  }
+  for (int t = 0; t < T; ++t)
+    for (int c = 0; c < E; ++c) {
+      float v = 0.0f;
+      for (int k = 0; k < NU; ++k) v += Y[((size_t)t * NU + k) * E + c];
+      out[(size_t)t * E + c] += v;
+    }
+  free(ids); free(wts); free(counts); free(Y);
+  return 0;
+}

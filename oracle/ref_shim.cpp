@@ -1,0 +1,41 @@
+// Thin extern "C" window onto the reference's own CPU code (src/quants.h), compiled from the reference tree where it
+// lies (see oracle/Makefile: -I$(REF)).  TEST INFRASTRUCTURE ONLY: it exists to validate oracle/arcz_oracle.c and,
+// optionally, to time the reference's CPU path; the output goes to oracle/_ref/ and is never committed.
+// Nothing of the reference is copied here: every function below only forwards to the header's functions.
+#include <cstdint>
+#include <cstring>
+#include <vector>
+#include "src/gguf.h"
+#include "src/quants.h"
+
+extern "C" {
+float ref_fp16_to_f32(uint16_t h) { return fp16_to_f32(h); }
+uint16_t ref_f32_to_fp16(float x) { return f32_to_fp16(x); }
+int ref_sb_bytes(uint32_t type) { return gguf_sb_bytes(type); }
+int ref_dequant_row(uint32_t type, const uint8_t* row, int K, float* out) {
+  try { dequant_row(type, row, K, out); } catch (...) { return -1; }
+  return 0;
+}
+// q[256], sc[8], mn[8], sc6[16], d8[8], d, dmin of one superblock
+int ref_decode_sb(uint32_t type, const uint8_t* p, int16_t* q, int32_t* sc, int32_t* mn, int32_t* sc6, float* d8,
+                  float* d, float* dmin) {
+  DecodedSB o;
+  try { decode_sb(type, p, o); } catch (...) { return -1; }
+  for (int i = 0; i < 256; ++i) q[i] = o.q[i];
+  for (int i = 0; i < 8; ++i) { sc[i] = o.sc[i]; mn[i] = o.mn[i]; d8[i] = o.d8[i]; }
+  for (int i = 0; i < 16; ++i) sc6[i] = o.sc6[i];
+  *d = o.d;
+  *dmin = o.dmin;
+  return 0;
+}
+void ref_quantize_act_cpu(const float* x, int M, int K, int8_t* aq, float* asc, uint16_t* absum, int act32) {
+  quantize_act_cpu(x, M, K, aq, asc, absum, act32 != 0);
+}
+void ref_quantize_rows_q8_0(const float* src, int N, int K, uint8_t* out) {
+  const std::vector<uint8_t> v = quantize_rows_q8_0(src, N, K);
+  memcpy(out, v.data(), v.size());
+}
+// the reference's GPU raw form of one superblock (src/quants.h gpu_raw_sb), to compare layouts in tests
+int ref_raw_padded_sb_bytes(uint32_t type) { return raw_padded_sb_bytes(type); }
+void ref_gpu_raw_sb(uint32_t type, const uint8_t* src, uint8_t* dst) { gpu_raw_sb(type, src, dst); }
+}

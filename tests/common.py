@@ -1,0 +1,90 @@
+"""Shared builders of test inputs: seeded synthetic tensors (the library's generators), hand-made blocks with unit
+scales, and the error measures the reference's own harness uses."""
+import numpy as np
+
+import arcinferzero_amd as az
+import oracle_lib as orc
+
+Q8_0, Q4_K, Q6_K = az.Q8_0, az.Q4_K, az.Q6_K
+TYPES = (Q8_0, Q4_K, Q6_K)
+TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+
+
+def make_weights(qtype, N, K, seed):
+    return az.gen_weights(qtype, seed, N, K, 0.02)
+
+
+def make_acts(M, K, seed, outliers=False):
+    x = az.gen_normal(seed, (M, K))
+    if outliers:  # the reference's bench multiplies one value in 97 by 4 (bench/gemv_bench.cpp:112)
+        rng = np.random.default_rng(seed)
+        x = x * (1.0 + 3.0 * (rng.integers(0, 97, size=x.shape) == 0)).astype(np.float32)
+    return x
+
+
+def pad_rows(a, Mp):
+    """[M][K] -> [Mp][K] with zero rows."""
+    out = np.zeros((Mp,) + a.shape[1:], a.dtype)
+    out[:a.shape[0]] = a
+    return out
+
+
+def quantize_padded(x, Mp):
+    """Oracle quantization of x [T][K] laid out for Mp rows (rows >= T zero, scale 0)."""
+    return orc.quantize_act(pad_rows(x, Mp))
+
+
+def rel_err_rows(y, ref):
+    """Per token row: max_n |y - ref| / max_n |ref| (bench/gemv_bench.cpp:199-214)."""
+    y = np.asarray(y, np.float64)
+    ref = np.asarray(ref, np.float64)
+    return np.abs(y - ref).max(axis=1) / np.maximum(np.abs(ref).max(axis=1), 1e-30)
+
+
+def mixed_err(y, ref):
+    """Per element |y - ref| / (|ref| + rms(ref)): shows that the row normalization is not doing the work."""
+    y = np.asarray(y, np.float64)
+    ref = np.asarray(ref, np.float64)
+    return (np.abs(y - ref) / (np.abs(ref) + np.sqrt((ref ** 2).mean()))).max()
+
+
+def unit_scale_weights(qtype, N, K, seed):
+    """GGUF blocks whose scales are exactly 1 (d = 1.0, sub-scales 1, mins 0) over random quants, and the integer
+    matrix [N][K] they decode to: with activations whose scales are exactly 1 the f32 output is the integer sum."""
+    rng = np.random.default_rng(seed)
+    nsb = K // 256
+    one = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    if qtype == Q4_K:
+        q = rng.integers(0, 16, size=(N, nsb, 256), dtype=np.int64)
+        blk = np.zeros((N, nsb, 144), np.uint8)
+        blk[..., 0:2] = one
+        blk[..., 4:8] = 1      # sc[0..3] = 1, mn = 0
+        blk[..., 12:16] = 1    # sc[4..7] low nibble = 1
+        for j in range(4):
+            blk[..., 16 + 32 * j:16 + 32 * j + 32] = (q[..., 64 * j:64 * j + 32] | (q[..., 64 * j + 32:64 * j + 64] << 4)).astype(np.uint8)
+        return blk.reshape(-1), q.reshape(N, K)
+    if qtype == Q6_K:
+        q = rng.integers(0, 64, size=(N, nsb, 256), dtype=np.int64)
+        blk = np.zeros((N, nsb, 210), np.uint8)
+        blk[..., 192:208] = 1
+        blk[..., 208:210] = one
+        for n in range(2):
+            b = q[..., 128 * n:128 * n + 128]
+            q0, q1, q2, q3 = b[..., 0:32], b[..., 32:64], b[..., 64:96], b[..., 96:128]
+            blk[..., 64 * n:64 * n + 32] = ((q0 & 15) | ((q2 & 15) << 4)).astype(np.uint8)
+            blk[..., 64 * n + 32:64 * n + 64] = ((q1 & 15) | ((q3 & 15) << 4)).astype(np.uint8)
+            blk[..., 128 + 32 * n:128 + 32 * n + 32] = ((q0 >> 4) | ((q1 >> 4) << 2) | ((q2 >> 4) << 4) | ((q3 >> 4) << 6)).astype(np.uint8)
+        return blk.reshape(-1), (q - 32).reshape(N, K)
+    q = rng.integers(-128, 128, size=(N, K // 32, 32), dtype=np.int64)
+    blk = np.zeros((N, K // 32, 34), np.uint8)
+    blk[..., 0:2] = one
+    blk[..., 2:] = q.astype(np.int8).view(np.uint8)
+    return blk.reshape(-1), q.reshape(N, K)
+
+
+def unit_scale_acts(M, K, seed):
+    """Integer-valued activations whose every 32-block has |max| = 127: they quantize to themselves with scale 1."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-127, 128, size=(M, K // 32, 32)).astype(np.float32)
+    x[..., 0] = np.where(rng.integers(0, 2, size=(M, K // 32)) == 0, 127.0, -127.0)
+    return x.reshape(M, K)

@@ -1,0 +1,105 @@
+"""Prefill GEMM (int8 MFMA) on the GPU against the oracle: tolerance 1e-3 of the f32 reference per token row, exact
+integer block sums through unit scales, the three epilogues, agreement with the GEMV on the same inputs, determinism."""
+import numpy as np
+import pytest
+
+import arcinferzero_amd as az
+import oracle_lib as orc
+from common import (TYPES, TYPE_NAMES, make_acts, make_weights, mixed_err, quantize_padded, rel_err_rows,
+                    unit_scale_acts, unit_scale_weights)
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+TIGHT = 2e-5
+
+
+@pytest.fixture(scope="module")
+def eng(rt):
+    e = az.Engine(512, 5120)
+    yield e
+    e.close()
+
+
+def run_gemm(eng, qtype, W, N, K, x, Mp, acc=0, c_init=None, ldc=None, c_off=0):
+    T = x.shape[0]
+    ldc = N + c_off if ldc is None else ldc
+    w = eng.make_weight(qtype, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, Mp, T)
+    cb = az.Runtime.alloc(Mp * ldc * 4)
+    if c_init is None:
+        cb.fill(0xFFFFFFFF)
+    else:
+        cb.write(c_init)
+    eng.matmul("test", w, Mp, cb, ldc, c_off, acc)
+    y = cb.read(np.float32, Mp * ldc).reshape(Mp, ldc)
+    for b in (cb, xb):
+        b.free()
+    w.free()
+    return y
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("T,Mp,N,K", [(16, 16, 64, 256), (100, 112, 272, 512), (128, 128, 128, 1024), (300, 384, 384, 768)])
+def test_gemm_vs_oracle(eng, qtype, T, Mp, N, K):
+    print(f"gemm {TYPE_NAMES[qtype]} T={T} Mp={Mp} N={N} K={K}", flush=True)
+    W = make_weights(qtype, N, K, seed=31 + qtype)
+    x = make_acts(T, K, seed=41 + T, outliers=True)
+    y = run_gemm(eng, qtype, W, N, K, x, Mp)
+    aq, asc, absum = quantize_padded(x, Mp)
+    ref = orc.matmul_ref(qtype, W, N, K, aq[:T], asc)
+    assert np.isfinite(y).all()
+    assert not y[T:].any()                      # padding rows: zero activations give exact zeros
+    err = rel_err_rows(y[:T], ref)
+    form = orc.matmul_formula(qtype, 1, W, N, K, aq[:T], asc, absum)
+    print(f"  rel {err.max():.2e} mixed {mixed_err(y[:T], ref):.2e} vs formula {rel_err_rows(y[:T], form).max():.2e}")
+    assert err.max() <= TOL
+    assert rel_err_rows(y[:T], form).max() <= TIGHT
+    y2 = run_gemm(eng, qtype, W, N, K, x, Mp)
+    assert np.array_equal(y.view(np.uint32), y2.view(np.uint32))   # bit-identical run to run
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_gemm_block_sums_exact(eng, qtype):
+    T, N, K = 160, 160, 512
+    W, wi = unit_scale_weights(qtype, N, K, seed=15)
+    x = unit_scale_acts(T, K, seed=16)
+    y = run_gemm(eng, qtype, W, N, K, x, 160)
+    exact = x.astype(np.int64) @ wi.T
+    assert np.abs(exact).max() < 2 ** 24
+    assert np.array_equal(y, exact.astype(np.float32))
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_gemm_matches_gemv(eng, qtype):
+    """Rows 0..7 of a 16-row GEMM against the 8-token GEMV on the same inputs: both within tolerance of the same
+    reference and of each other."""
+    N, K, T = 192, 1024, 16
+    W = make_weights(qtype, N, K, seed=51)
+    x = make_acts(T, K, seed=52)
+    yg = run_gemm(eng, qtype, W, N, K, x, 16)
+    w = eng.make_weight(qtype, N, K, W)
+    xb = az.Runtime.from_numpy(x[:8])
+    eng.quantize(xb, K, K, 16, 8)
+    cb = az.Runtime.alloc(8 * N * 4)
+    eng.matmul("test", w, 16, cb, N, 0, 0)
+    yv = cb.read(np.float32, 8 * N).reshape(8, N)
+    cb.free(); xb.free(); w.free()
+    assert rel_err_rows(yg[:8], yv).max() <= TIGHT
+
+
+def test_gemm_epilogues(eng):
+    qtype, T, Mp, N, K = az.Q4_K, 64, 64, 128, 512
+    W = make_weights(qtype, N, K, seed=61)
+    x = make_acts(T, K, seed=62)
+    ldc, c_off = 300, 100
+    c0 = az.gen_normal(63, (Mp, ldc))
+    y0 = run_gemm(eng, qtype, W, N, K, x, Mp)
+    ya = run_gemm(eng, qtype, W, N, K, x, Mp, acc=1, c_init=c0, ldc=ldc, c_off=c_off)
+    assert np.array_equal(ya[:, :c_off], c0[:, :c_off]) and np.array_equal(ya[:, c_off + N:], c0[:, c_off + N:])
+    assert np.array_equal(ya[:, c_off:c_off + N], y0 + c0[:, c_off:c_off + N])
+    ys = run_gemm(eng, qtype, W, N, K, x, Mp, acc=2, c_init=c0, ldc=ldc, c_off=c_off)
+    g = c0[:, c_off:c_off + N].astype(np.float64)
+    want = y0.astype(np.float64) * (g / (1.0 + np.exp(-g)))   # C = silu(C) * result (gemm.cl:562-565)
+    assert np.abs(ys[:, c_off:c_off + N] - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.array_equal(ys[:, :c_off], c0[:, :c_off])

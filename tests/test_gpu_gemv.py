@@ -1,0 +1,107 @@
+"""Decode GEMV (1 token) and multi-token GEMV (2..8 tokens) on the GPU against the oracle.
+
+f32 outputs: per token row max|y - ref| / max|ref| <= 1e-3 against the double-accumulated dequantized reference
+(tools/ref_forward.cpp:268-303 semantics; the measure of bench/gemv_bench.cpp:199-214) -- the stated tolerance; the
+observed error is float rounding only, so a much tighter bound against the engine-formula restatement is checked too.
+int32 block sums: exact, through unit scales (every scale 1: the f32 output is the integer sum itself).
+"""
+import numpy as np
+import pytest
+
+import arcinferzero_amd as az
+import oracle_lib as orc
+from common import (TYPES, TYPE_NAMES, make_acts, make_weights, mixed_err, quantize_padded, rel_err_rows,
+                    unit_scale_acts, unit_scale_weights)
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3        # the tolerance the path is specified to
+TIGHT = 2e-5      # what float rounding alone allows against the same-formula restatement
+
+
+@pytest.fixture(scope="module")
+def eng(rt):
+    e = az.Engine(16, 17408)
+    yield e
+    e.close()
+
+
+def run_gemv(eng, qtype, W, N, K, x, Mp, acc=0, c_init=None, ldc=None, c_off=0):
+    T = x.shape[0]
+    ldc = N + c_off if ldc is None else ldc
+    w = eng.make_weight(qtype, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, Mp, T)
+    cb = az.Runtime.alloc(T * ldc * 4)
+    if c_init is None:
+        cb.fill(0xFFFFFFFF)  # NaN poison (bench/gemv_bench.cpp:154-157)
+    else:
+        cb.write(c_init)
+    eng.matmul("test", w, Mp, cb, ldc, c_off, acc)
+    y = cb.read(np.float32, T * ldc).reshape(T, ldc)
+    for b in (cb, xb):
+        b.free()
+    w.free()
+    return y
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("T", [1, 2, 3, 5, 8])
+def test_gemv_small_vs_oracle(eng, qtype, T):
+    N, K, Mp = 264, 512, 16   # N not a multiple of the rows per work-group
+    print(f"gemv {TYPE_NAMES[qtype]} T={T} N={N} K={K}", flush=True)
+    W = make_weights(qtype, N, K, seed=11 + qtype)
+    x = make_acts(T, K, seed=21 + T, outliers=True)
+    y = run_gemv(eng, qtype, W, N, K, x, Mp)
+    aq, asc, absum = quantize_padded(x, Mp)
+    ref = orc.matmul_ref(qtype, W, N, K, aq[:T], asc)
+    assert np.isfinite(y).all()
+    assert rel_err_rows(y, ref).max() <= TOL
+    form = orc.matmul_formula(qtype, 0, W, N, K, aq[:T], asc, absum)
+    assert rel_err_rows(y, form).max() <= TIGHT
+    print(f"  rel {rel_err_rows(y, ref).max():.2e} mixed {mixed_err(y, ref):.2e} vs formula {rel_err_rows(y, form).max():.2e}")
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("T", [1, 2, 7])
+def test_gemv_block_sums_exact(eng, qtype, T):
+    """Unit scales: the f32 output must be the exact integer dot product (all partial sums stay below 2^24)."""
+    N, K = 96, 768
+    W, wi = unit_scale_weights(qtype, N, K, seed=5)
+    x = unit_scale_acts(T, K, seed=6)
+    y = run_gemv(eng, qtype, W, N, K, x, 16)
+    exact = x.astype(np.int64) @ wi.T
+    assert np.abs(exact).max() < 2 ** 24
+    assert np.array_equal(y.astype(np.int64), exact) and np.array_equal(y, exact.astype(np.float32))
+
+
+@pytest.mark.parametrize("qtype,N,K,T", [(az.Q4_K, 17408, 5120, 1), (az.Q4_K, 5120, 17408, 2), (az.Q6_K, 4096, 5120, 1),
+                                         (az.Q8_0, 4096, 4096, 4)])
+def test_gemv_config_shapes_sampled(eng, qtype, N, K, T):
+    """The decode shapes of the configs, checked on ~512 sampled rows (the reference samples ~4096, gemv_bench.cpp:202)
+    plus determinism: two runs give the same bits."""
+    print(f"gemv config {TYPE_NAMES[qtype]} N={N} K={K} T={T}", flush=True)
+    W = make_weights(qtype, N, K, seed=3)
+    x = make_acts(T, K, seed=4)
+    y = run_gemv(eng, qtype, W, N, K, x, 16)
+    y2 = run_gemv(eng, qtype, W, N, K, x, 16)
+    assert np.array_equal(y.view(np.uint32), y2.view(np.uint32))
+    rows = np.arange(0, N, max(1, N // 512))
+    rb = az.gguf_bytes(qtype, 1, K)
+    Wr = np.concatenate([W[r * rb:(r + 1) * rb] for r in rows])
+    aq, asc, _ = quantize_padded(x, 16)
+    ref = orc.matmul_ref(qtype, Wr, len(rows), K, aq[:T], asc)
+    err = rel_err_rows(y[:, rows], ref)
+    print(f"  rel {err.max():.2e}")
+    assert err.max() <= TOL
+
+
+def test_gemv_accumulate_and_offset(eng):
+    N, K, T, Mp = 128, 512, 3, 16
+    W = make_weights(az.Q4_K, N, K, seed=8)
+    x = make_acts(T, K, seed=9)
+    ldc, c_off = 200, 40
+    c0 = az.gen_normal(77, (T, ldc))
+    y0 = run_gemv(eng, az.Q4_K, W, N, K, x, Mp)
+    y = run_gemv(eng, az.Q4_K, W, N, K, x, Mp, acc=1, c_init=c0, ldc=ldc, c_off=c_off)
+    assert np.array_equal(y[:, :c_off], c0[:, :c_off]) and np.array_equal(y[:, c_off + N:], c0[:, c_off + N:])
+    assert np.array_equal(y[:, c_off:c_off + N], c0[:, c_off:c_off + N] + y0)
