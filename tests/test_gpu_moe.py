@@ -1,0 +1,115 @@
+"""Mixture-of-experts path on the GPU against the oracle: routing (ids and counts equal, weights < 1e-6, the bar of
+the reference's own tests/test_route.cpp:28-96), the counting sort (invariants, and equality with the oracle's serial
+order: the GPU scatter is deterministic), the expert-input quantizer (bit-exact on the GPU's own h), the grouped GEMM
+and the whole layer (1e-3 of the f32 reference)."""
+import numpy as np
+import pytest
+
+import arcinferzero_amd as az
+import oracle_lib as orc
+from common import TYPE_NAMES, make_acts, make_weights, quantize_padded, rel_err_rows
+
+pytestmark = pytest.mark.gpu
+
+
+def route_on_gpu(eng, L, logits, tm):
+    T = logits.shape[0]
+    lb = az.Runtime.from_numpy(logits)
+    eng.moe_route(L, lb, logits.shape[1], T, tm)
+    n = T * L.NU
+    out = {
+        "ids": eng.moe_buffer("ids").read(np.int32, n).reshape(T, L.NU),
+        "wts": eng.moe_buffer("wts").read(np.float32, n).reshape(T, L.NU),
+        "offs": eng.moe_buffer("offs").read(np.int32, L.NE),
+        "tstart": eng.moe_buffer("tstart").read(np.int32, L.NE + 1),
+        "stok": eng.moe_buffer("stok").read(np.int32, n),
+        "swt": eng.moe_buffer("swt").read(np.float32, n),
+        "inv": eng.moe_buffer("inv").read(np.int32, n),
+    }
+    nt = int(out["tstart"][-1])
+    out["tiles"] = eng.moe_buffer("tiles").read(np.int32, 1 + 3 * nt)
+    lb.free()
+    return out
+
+
+@pytest.mark.parametrize("NE,NU,T,tm", [(8, 2, 40, 16), (128, 8, 300, 128), (256, 6, 7, 16), (64, 8, 1, 128)])
+def test_routing_and_sort(rt, NE, NU, T, tm):
+    print(f"route NE={NE} NU={NU} T={T}", flush=True)
+    eng = az.Engine(512, 256)
+    try:
+        dummy = np.zeros(az.gguf_bytes(az.Q8_0, NE * 256, 256), np.uint8)
+        L = eng.make_moe_layer(az.Q8_0, dummy, dummy, dummy, NE, NU, 256, 256)
+        rng = np.random.default_rng(11)
+        logits = (rng.standard_normal((T, NE + 1)) * 2.0).astype(np.float32)
+        logits[0, 3] = logits[0, 5] = logits[0].max() + 1.0       # a tie: the lower expert first
+        g = route_on_gpu(eng, L, logits, tm)
+        # the reference's CPU check: stable sort by descending logit
+        for t in range(T):
+            idx = np.argsort(-logits[t, :NE], kind="stable")[:NU]
+            assert np.array_equal(g["ids"][t], idx)
+            p = np.exp(logits[t, idx].astype(np.float64) - float(logits[t, idx[0]]))
+            assert np.abs(g["wts"][t] - p / p.sum()).max() < 1e-6
+        ids, wts, _, counts = orc.moe_route(logits, NE, NU)
+        assert np.array_equal(g["ids"], ids) and np.abs(g["wts"] - wts).max() < 1e-6
+        offs, tiles, tstart = orc.moe_scan(counts, tm)
+        assert np.array_equal(g["offs"], offs) and np.array_equal(g["tstart"], tstart)
+        assert np.array_equal(g["tiles"], tiles[:g["tiles"].size])
+        # invariants of the sort
+        n = T * NU
+        assert counts.sum() == n and sorted(g["inv"].tolist()) == list(range(n))
+        assert np.array_equal(g["stok"][g["inv"]], np.arange(n) // NU)
+        assert np.array_equal(g["swt"][g["inv"]], g["wts"].reshape(-1))
+        e_of_slot = np.repeat(np.arange(NE), counts)
+        assert np.array_equal(e_of_slot[g["inv"]], g["ids"].reshape(-1))
+        # and the deterministic order: equal to the oracle's serial scatter
+        stok, swt, inv = orc.moe_scatter(g["ids"], g["wts"], offs)
+        assert np.array_equal(g["inv"], inv) and np.array_equal(g["stok"], stok)
+        # a second layer call must start from zeroed counts
+        g2 = route_on_gpu(eng, L, logits, tm)
+        assert np.array_equal(g2["offs"], offs) and np.array_equal(g2["inv"], inv)
+    finally:
+        eng.close()
+
+
+@pytest.mark.parametrize("qtype,NE,NU,E,F,T,Mp", [(az.Q4_K, 8, 2, 256, 256, 40, 48), (az.Q8_0, 4, 2, 256, 512, 20, 32),
+                                                   (az.Q6_K, 6, 3, 512, 256, 33, 48), (az.Q4_K, 16, 4, 512, 768, 300, 384)])
+def test_moe_layer_vs_oracle(rt, qtype, NE, NU, E, F, T, Mp):
+    print(f"moe layer {TYPE_NAMES[qtype]} NE={NE} NU={NU} E={E} F={F} T={T}", flush=True)
+    eng = az.Engine(Mp, max(E, F))
+    try:
+        Wg = make_weights(qtype, NE * F, E, seed=1)
+        Wu = make_weights(qtype, NE * F, E, seed=2)
+        Wd = make_weights(qtype, NE * E, F, seed=3)
+        L = eng.make_moe_layer(qtype, Wg, Wu, Wd, NE, NU, E, F)
+        x = make_acts(T, E, seed=4)
+        rng = np.random.default_rng(5)
+        logits = rng.standard_normal((T, NE)).astype(np.float32)
+        logits[:, 1] -= 50.0                                  # an expert that gets no token
+        xb = az.Runtime.from_numpy(x)
+        eng.quantize(xb, E, E, Mp, T)
+        lb = az.Runtime.from_numpy(logits)
+        x0 = az.gen_normal(9, (T, E))
+        ob = az.Runtime.from_numpy(x0)
+        eng.layer_moe(L, lb, NE, ob, T, Mp)
+        out = ob.read(np.float32, T * E).reshape(T, E)
+        aq, asc, _ = quantize_padded(x, Mp)
+        ref, href = orc.moe_layer(qtype, Wg, Wu, Wd, NE, NU, E, F, aq[:T], asc, logits)
+        err = rel_err_rows(out - x0, ref)
+        print(f"  layer rel err {err.max():.2e}")
+        assert np.isfinite(out).all() and err.max() <= 1e-3
+        # h on the GPU (slot order) against the oracle's (pair order), then the second quantization bit for bit
+        n = T * NU
+        S = eng.moe_slots
+        inv = eng.moe_buffer("inv").read(np.int32, n)
+        h = eng.moe_buffer("h").read(np.float32, S * F).reshape(S, F)
+        assert rel_err_rows(h[inv], href).max() <= 1e-3
+        hq = eng.moe_buffer("hq").read(np.int8, S * F).reshape(S, F)
+        hsc = eng.moe_buffer("hsc").read(np.float32, (F // 32) * S).reshape(F // 32, S)
+        used = np.sort(inv)
+        rq, rsc = orc.moe_quant(h[used])
+        assert np.array_equal(hq[used], rq)
+        assert np.array_equal(hsc[:, used].view(np.uint32), rsc.view(np.uint32))
+        for b in (xb, lb, ob):
+            b.free()
+    finally:
+        eng.close()
