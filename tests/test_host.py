@@ -1,0 +1,111 @@
+"""What can be checked without a GPU: the C-ABI library loads and exports every symbol its headers declare, fails
+loudly (not silently) when there is no device, and its host-side helpers -- the GGUF -> device planes regrouping,
+the Q8_0 row quantizer, the synthetic generators -- do what they say."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import arcinferzero_amd as az
+import oracle_lib as orc
+from common import TYPES, make_weights
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = []
+    for hdr in ("arcz_hip.h", "arcz_engine.h"):
+        src = open(os.path.join(ROOT, "include", hdr)).read()
+        src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+        names += re.findall(r"\b(arcz_[a-z0-9_]+)\s*\(", src)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_symbols()
+    assert len(names) > 50
+    missing = [n for n in names if not hasattr(az.lib, n)]
+    assert not missing, missing
+
+
+def test_no_device_fails_loudly():
+    """Without a GPU nothing computes: init reports an error, allocation and engine creation return NULL."""
+    import subprocess, sys
+    code = ("import arcinferzero_amd as az, sys\n"
+            "r = az.lib.arcz_init(0)\n"
+            "if r == 0: sys.exit(77)\n"
+            "assert r < 0 and az.lib.arcz_last_error()\n"
+            "assert not az.lib.arcz_alloc(1024)\n"
+            "try:\n    az.Engine(16, 256)\nexcept az.ArczError as e:\n    print('engine refused:', e)\nelse:\n    sys.exit(1)\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=ROOT, timeout=120)
+    if r.returncode == 77:
+        pytest.skip("a GPU is present")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "engine refused" in r.stdout
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_repack_planes_layout(qtype):
+    rows, K = 6, 768
+    nsb = K // 256
+    W = make_weights(qtype, rows, K, seed=21)
+    P = az.repack_planes(qtype, rows, K, W)
+    assert P.size == az.planes_bytes(qtype, rows, K)
+    u = rows * nsb
+    if qtype == az.Q4_K:
+        sb = W.reshape(u, 144)
+        assert P.size == W.size
+        assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 16:]) and np.array_equal(P[u * 128:].reshape(u, 16), sb[:, :16])
+    elif qtype == az.Q6_K:
+        sb = W.reshape(u, 210)
+        o = 0
+        for lo, n in ((0, 128), (128, 64), (192, 16), (208, 2)):
+            assert np.array_equal(P[o:o + u * n].reshape(u, n), sb[:, lo:lo + n])
+            o += u * n
+        assert not P[o:].any() and P.size % 16 == 0
+    else:
+        blk = W.reshape(u, 8, 34)
+        assert np.array_equal(P[:u * 256].reshape(u, 8, 32), blk[:, :, 2:]) and np.array_equal(P[u * 256:].reshape(u, 8, 2), blk[:, :, :2])
+
+
+def test_q8_0_quantizer_is_the_reference_one():
+    w = az.gen_normal(5, (32, 512), std=0.02)
+    w[3, 64:96] = 0
+    assert np.array_equal(az.quantize_rows(az.Q8_0, w), orc.quantize_rows_q8_0(w))
+
+
+@pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q6_K, 0.02), (az.Q8_0, 0.006)])
+def test_block_makers_make_valid_close_blocks(qtype, rel):
+    """The Q4_K / Q6_K block makers are input generators (the reference has none): valid fields and a round-trip
+    error of the size the bit width allows."""
+    N, K = 64, 1024
+    w = az.gen_normal(6, (N, K), std=0.02)
+    B = az.quantize_rows(qtype, w)
+    back = orc.dequant_rows(qtype, B, N, K)
+    assert np.isfinite(back).all()
+    err = np.sqrt(((back - w) ** 2).mean()) / np.sqrt((w ** 2).mean())
+    assert err < rel, err
+    q, isc, imn, d, dmin = orc.decode_row_fields(qtype, B[:az.gguf_bytes(qtype, 1, K)], K)
+    if qtype == az.Q4_K:
+        assert q.min() >= 0 and q.max() <= 15 and isc.max() <= 63 and imn.max() <= 63 and len(np.unique(q)) == 16
+    elif qtype == az.Q6_K:
+        assert q.min() >= -32 and q.max() <= 31 and isc.max() <= 127 and isc.min() >= 1
+
+
+def test_generators_are_seeded_and_normal():
+    a, b = az.gen_normal(42, (1000, 256)), az.gen_normal(42, (1000, 256))
+    assert np.array_equal(a, b) and not np.array_equal(a, az.gen_normal(43, (1000, 256)))
+    assert abs(a.mean()) < 0.01 and abs(a.std() - 1.0) < 0.01 and abs((a ** 4).mean() - 3.0) < 0.1
+    w1, w2 = az.gen_weights(az.Q4_K, 1, 5000, 256), az.gen_weights(az.Q4_K, 1, 5000, 256)
+    assert np.array_equal(w1, w2)
+
+
+def test_byte_counts_match_the_formats():
+    assert az.gguf_bytes(az.Q4_K, 17408, 5120) == 50135040       # the figures the roofline uses
+    assert az.gguf_bytes(az.Q6_K, 151936, 5120) == 638131200
+    assert az.gguf_bytes(az.Q8_0, 4096, 4096) == 17825792
+    assert az.gguf_bytes(az.Q4_K, 128 * 768, 2048) * 2 + az.gguf_bytes(az.Q4_K, 128 * 2048, 768) == 339738624
+    assert az.gguf_bytes(5, 1, 256) == 0

@@ -1,0 +1,311 @@
+"""Pins the CPU oracle (oracle/arcz_oracle.c) before anything is compared with it: golden vectors taken from the
+reference's own header, the compiled reference itself where it is built (oracle/_ref), and what the mathematics
+fixes -- closed forms, brute force in numpy, exhaustive fp16 -- chosen so that a dropped term, a wrong index or a
+transposed operand fails."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from common import TYPES, make_acts, make_weights, rel_err_rows, unit_scale_acts, unit_scale_weights
+
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz"))
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+NAMES = {Q4_K: "q4k", Q6_K: "q6k", Q8_0: "q80"}
+
+
+# ---------------------------------------------------------------- fp16
+def test_fp16_to_f32_exhaustive():
+    h = np.arange(65536, dtype=np.uint16)
+    got = np.array([np.float32(orc.orc.orc_fp16_to_f32(int(v))).view(np.uint32) for v in h], np.uint32)
+    want = h.view(np.float16).astype(np.float32).view(np.uint32)
+    nan = np.isnan(h.view(np.float16))
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.isnan(got[nan].view(np.float32)).all()
+    assert np.array_equal(got, G["fp16_all_to_f32_bits"])          # the reference, bit for bit (NaN payloads too)
+
+
+def test_f32_to_fp16_golden_and_numpy():
+    f = G["f32_in"]
+    got = np.array([orc.orc.orc_f32_to_fp16(C.c_float(float(v))) for v in f], np.uint16)
+    assert np.array_equal(got, G["f32_to_fp16"])
+    ok = ~np.isnan(f)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got[ok], f[ok].astype(np.float16).view(np.uint16))   # IEEE round to nearest even
+
+
+def test_fp16_round_trip_all_finite():
+    h = np.arange(65536, dtype=np.uint16)
+    fin = np.isfinite(h.view(np.float16))
+    back = np.array([orc.orc.orc_f32_to_fp16(C.c_float(orc.orc.orc_fp16_to_f32(int(v)))) for v in h[fin]], np.uint16)
+    assert np.array_equal(back, h[fin])
+
+
+# ---------------------------------------------------------------- decoders
+@pytest.mark.parametrize("qtype", TYPES)
+def test_dequant_golden(qtype):
+    nm = NAMES[qtype]
+    got = orc.dequant_rows(qtype, G[f"{nm}_raw"], 4, 512)
+    assert np.array_equal(got.view(np.uint32), G[f"{nm}_dequant"].view(np.uint32))
+    q, isc, imn, d, dmin = orc.decode_row_fields(qtype, G[f"{nm}_raw"][:512 // 256 * orc.SB_BYTES[qtype]], 512)
+    gq = G[f"{nm}_sb0_q"].astype(np.int32) - (32 if qtype == Q6_K else 0)
+    assert np.array_equal(q[:256], gq)
+    if qtype == Q4_K:
+        assert np.array_equal(isc[:16:2], G[f"{nm}_sb0_sc"]) and np.array_equal(imn[:16:2], G[f"{nm}_sb0_mn"])
+        assert d[0] == G[f"{nm}_sb0_d"][0] and dmin[0] == G[f"{nm}_sb0_d"][1]
+    elif qtype == Q6_K:
+        assert np.array_equal(isc[:16], G[f"{nm}_sb0_sc6"]) and d[0] == G[f"{nm}_sb0_d"][0]
+    else:
+        assert np.array_equal(d[:8], G[f"{nm}_sb0_d8"])
+
+
+@pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
+@pytest.mark.parametrize("qtype", TYPES)
+def test_dequant_vs_compiled_reference(qtype):
+    W = make_weights(qtype, 16, 1024, seed=3)
+    assert np.array_equal(orc.dequant_rows(qtype, W, 16, 1024).view(np.uint32),
+                          orc.dequant_rows(qtype, W, 16, 1024, lib=orc.ref).view(np.uint32))
+
+
+def test_q4k_closed_form():
+    """Exact binary fractions, expected values without the decoder (the pattern of tests/test_quant_rows.cpp:17-29)."""
+    K = 512
+    blk = np.zeros((2, 144), np.uint8)
+    exp = np.zeros(K, np.float32)
+    for s in range(2):
+        d, dmin = (0.25, 0.5) if s == 0 else (2.0, 0.125)
+        blk[s, 0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+        blk[s, 2:4] = np.frombuffer(np.float16(dmin).tobytes(), np.uint8)
+        sc = [(7 * b + 3 + 11 * s) % 64 for b in range(8)]
+        mn = [(13 * b + 5 + 17 * s) % 64 for b in range(8)]
+        sb = blk[s, 4:16]
+        for j in range(8):                       # the packing of get_scale_min_k4, written out from its definition
+            if j < 4:
+                sb[j] |= sc[j]; sb[j + 4] |= mn[j]
+            else:
+                sb[j + 4] |= (sc[j] & 15) | ((mn[j] & 15) << 4)
+                sb[j - 4] |= (sc[j] >> 4) << 6
+                sb[j] |= (mn[j] >> 4) << 6
+        for e in range(256):
+            q = (e * 5 + 3 * s) % 16
+            j, r = divmod(e, 64)
+            if r < 32: blk[s, 16 + 32 * j + r] |= q
+            else: blk[s, 16 + 32 * j + r - 32] |= q << 4
+            exp[256 * s + e] = d * sc[e // 32] * q - dmin * mn[e // 32]
+    got = orc.dequant_rows(Q4_K, blk.reshape(-1), 1, K)[0]
+    assert np.array_equal(got, exp)
+
+
+def test_q6k_closed_form():
+    K = 256
+    blk = np.zeros(210, np.uint8)
+    d = 0.125
+    blk[208:210] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+    sc = np.array([(9 * i) % 31 - 15 for i in range(16)], np.int8)
+    blk[192:208] = sc.view(np.uint8)
+    exp = np.zeros(K, np.float32)
+    for e in range(256):
+        q = (e * 7 + 1) % 64
+        n, r = divmod(e, 128)
+        quarter, l = divmod(r, 32)
+        lb = 64 * n + l + (32 if quarter & 1 else 0)
+        blk[lb] |= (q & 15) << (4 if quarter >= 2 else 0)
+        blk[128 + 32 * n + l] |= (q >> 4) << (2 * quarter)
+        exp[e] = d * sc[e // 16] * (q - 32)
+    assert np.array_equal(orc.dequant_rows(Q6_K, blk, 1, K)[0], exp)
+
+
+def test_q80_closed_form():
+    K = 256
+    blk = np.zeros((8, 34), np.uint8)
+    exp = np.zeros(K, np.float32)
+    for b in range(8):
+        d = [0.0, 0.25, 0.5, 2.0][b % 4]
+        blk[b, 0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+        for i in range(32):
+            q = (i * 13 + b * 7) % 256 - 128
+            blk[b, 2 + i] = np.int8(q).view(np.uint8)
+            exp[32 * b + i] = d * q
+    assert np.array_equal(orc.dequant_rows(Q8_0, blk.reshape(-1), 1, K)[0], exp)
+
+
+# ---------------------------------------------------------------- quantizers
+def test_quantize_act_golden():
+    for a32 in (1, 0):
+        aq, asc, absum = orc.quantize_act(G["act_x"], act32=bool(a32))
+        assert np.array_equal(aq, G[f"act{a32}_aq"])
+        assert np.array_equal(asc.view(np.uint32), G[f"act{a32}_asc"].view(np.uint32))
+        assert np.array_equal(absum, G[f"act{a32}_absum"].view(np.int16))
+
+
+def test_quantize_act_closed_forms():
+    x = np.zeros((3, 64), np.float32)
+    x[0, :32] = np.linspace(-2.0, 2.0, 32)
+    x[1, :32] = np.array([127.0] + [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5] * 4 + [0.0] * 3)
+    x[2, 32:] = -5.0
+    aq, asc, absum = orc.quantize_act(x)
+    assert aq[0, 0] == -127 and aq[0, 31] == 127 and np.array_equal(aq[0, :32], -aq[0, :32][::-1])   # sign symmetry
+    assert asc[0, 0] == np.float32(2.0) / np.float32(127.0)
+    assert asc[1, 0] == 0.0 and not aq[0, 32:].any()                                               # zero block
+    assert aq[1, 1:8].tolist() == [0, 2, 2, 0, -2, -2, 4]                                           # ties to even
+    assert (aq[2, 32:] == -127).all() and absum[2, 2] == -127 * 16
+    assert np.array_equal(aq.reshape(3, 4, 16).astype(np.int32).sum(axis=2).T, absum.astype(np.int32))
+
+
+@pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
+def test_quantizers_vs_compiled_reference():
+    x = make_acts(32, 1024, seed=5, outliers=True)
+    for a32 in (True, False):
+        a, b = orc.quantize_act(x, act32=a32), orc.quantize_act(x, act32=a32, lib=orc.ref)
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+        assert np.array_equal(a[2], b[2])
+    w = (make_acts(16, 512, seed=6) * 0.02).astype(np.float32)
+    assert np.array_equal(orc.quantize_rows_q8_0(w), orc.quantize_rows_q8_0(w, lib=orc.ref))
+
+
+def test_quantize_rows_q8_0_golden_and_roundtrip():
+    w = G["q80_rows_in"]
+    out = orc.quantize_rows_q8_0(w)
+    assert np.array_equal(out, G["q80_rows_out"])
+    back = orc.dequant_rows(Q8_0, out, 8, 256)
+    amax = np.abs(w.reshape(8, 8, 32)).max(axis=2, keepdims=True)
+    # half a step of the block's scale, plus the fp16 rounding of the scale itself
+    assert (np.abs(back.reshape(8, 8, 32) - w.reshape(8, 8, 32)) <= amax / 127.0 * 0.5 + amax * 2.0 ** -11 + 1e-12).all()
+
+
+# ---------------------------------------------------------------- integer sums and the f32 references
+@pytest.mark.parametrize("qtype", TYPES)
+def test_block_sums_brute_force(qtype):
+    N, K, M = 5, 512, 3
+    W = make_weights(qtype, N, K, seed=7)
+    aq, asc, absum = orc.quantize_act(make_acts(M, K, seed=8))
+    I = orc.block_sums(qtype, W, N, K, aq)
+    q = np.stack([orc.decode_row_fields(qtype, W[n * (K // 256) * orc.SB_BYTES[qtype]:(n + 1) * (K // 256) * orc.SB_BYTES[qtype]], K)[0]
+                  for n in range(N)]).astype(np.int64)
+    want = np.einsum("nhk,mhk->mnh", q.reshape(N, K // 16, 16), aq.astype(np.int64).reshape(M, K // 16, 16))
+    assert np.array_equal(I, want)
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_matmul_ref_is_a_float64_dot(qtype):
+    N, K, M = 24, 768, 5
+    W = make_weights(qtype, N, K, seed=9)
+    aq, asc, absum = orc.quantize_act(make_acts(M, K, seed=10, outliers=True))
+    Y = orc.matmul_ref(qtype, W, N, K, aq, asc)
+    w = orc.dequant_rows(qtype, W, N, K).astype(np.float64)
+    x = (aq.astype(np.float32) * np.repeat(asc.T, 32, axis=1)).astype(np.float64)
+    want = x @ w.T
+    assert np.abs(Y - want).max() <= 2e-7 * np.abs(want).max()       # one rounding to f32 (summation order aside)
+    for form in (0, 1):
+        F = orc.matmul_formula(qtype, form, W, N, K, aq, asc, absum)
+        assert rel_err_rows(F, want).max() <= 5e-6                      # the engine's f32 formulas: rounding only
+
+
+@pytest.mark.parametrize("qtype", TYPES)
+def test_unit_scale_known_answer(qtype):
+    """All scales 1: both f32 evaluations must give the exact integer sum (catches a dropped min term, a wrong
+    sub-scale index, a swapped nibble)."""
+    N, K, M = 12, 512, 4
+    W, wi = unit_scale_weights(qtype, N, K, seed=11)
+    x = unit_scale_acts(M, K, seed=12)
+    aq, asc, absum = orc.quantize_act(x)
+    assert np.array_equal(aq.astype(np.float32), x) and (asc == 1.0).all()
+    exact = (x.astype(np.int64) @ wi.T).astype(np.float32)
+    assert np.array_equal(orc.matmul_ref(qtype, W, N, K, aq, asc), exact)
+    for form in (0, 1):
+        assert np.array_equal(orc.matmul_formula(qtype, form, W, N, K, aq, asc, absum), exact)
+
+
+def test_q4k_min_term_matters():
+    """A Q4_K matrix with zero quants and non-zero mins: the output is -dmin * mn * sum(a), nothing else."""
+    K, N = 256, 1
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[2:4] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    blk[4:8] = 1
+    blk[8:12] = [2, 3, 4, 5]               # mn[0..3]
+    blk[12:16] = 1 | (6 << 4)              # sc[4..7] = 1, mn[4..7] = 6
+    x = unit_scale_acts(2, K, seed=13)
+    aq, asc, absum = orc.quantize_act(x)
+    mn = np.array([2, 3, 4, 5, 6, 6, 6, 6], np.float64)
+    want = -(0.5 * mn * x.reshape(2, 8, 32).sum(axis=2)).sum(axis=1)
+    for Y in (orc.matmul_ref(Q4_K, blk, N, K, aq, asc), orc.matmul_formula(Q4_K, 0, blk, N, K, aq, asc, absum),
+              orc.matmul_formula(Q4_K, 1, blk, N, K, aq, asc, absum)):
+        assert np.array_equal(Y[:, 0].astype(np.float64), want)
+
+
+# ---------------------------------------------------------------- mixture of experts
+def test_route_vs_stable_sort():
+    rng = np.random.default_rng(11)
+    NE, NU, T = 256, 6, 7                  # the reference's own case (tests/test_route.cpp:20)
+    lg = (rng.standard_normal((T, NE + 1)) * 2.0).astype(np.float32)
+    lg[2, 10] = lg[2, 200] = lg[2].max() + 1
+    ids, wts, sgate, counts = orc.moe_route(lg, NE, NU)
+    cnt = np.zeros(NE, np.int64)
+    for t in range(T):
+        idx = np.argsort(-lg[t, :NE], kind="stable")[:NU]
+        assert np.array_equal(ids[t], idx)
+        p = np.exp(lg[t, idx].astype(np.float64) - float(lg[t, idx[0]]))
+        assert np.abs(wts[t] - p / p.sum()).max() < 1e-6
+        assert abs(sgate[t] - 1.0 / (1.0 + np.exp(-float(lg[t, NE])))) < 1e-6
+        cnt[idx] += 1
+    assert np.array_equal(counts, cnt)
+
+
+def test_scan_scatter_invariants():
+    rng = np.random.default_rng(12)
+    NE, NU, T, TM = 16, 4, 100, 16
+    lg = rng.standard_normal((T, NE)).astype(np.float32)
+    lg[:, 3] -= 100
+    ids, wts, _, counts = orc.moe_route(lg, NE, NU)
+    offs, tiles, tstart = orc.moe_scan(counts, TM)
+    assert counts[3] == 0 and counts.sum() == T * NU
+    assert np.array_equal(offs, np.concatenate([[0], np.cumsum(counts)[:-1]]))
+    nt = tiles[0]
+    assert nt == ((counts + TM - 1) // TM).sum() == tstart[NE]
+    t3 = tiles[1:1 + 3 * nt].reshape(nt, 3)
+    for e in range(NE):
+        mine = t3[tstart[e]:tstart[e + 1]]
+        assert (mine[:, 0] == e).all() and mine[:, 2].sum() == counts[e] and (mine[:, 2] <= TM).all()
+        assert np.array_equal(mine[:, 1], offs[e] + TM * np.arange(len(mine)))
+    stok, swt, inv = orc.moe_scatter(ids, wts, offs)
+    n = T * NU
+    assert sorted(inv.tolist()) == list(range(n))
+    assert np.array_equal(stok[inv], np.arange(n) // NU) and np.array_equal(swt[inv], wts.reshape(-1))
+    assert np.array_equal(np.repeat(np.arange(NE), counts)[inv], ids.reshape(-1))
+
+
+def test_moe_quant_matches_act_quant():
+    h = make_acts(5, 256, seed=14)
+    hq, hsc = orc.moe_quant(h)
+    aq, asc, _ = orc.quantize_act(h)
+    assert np.array_equal(hq, aq) and np.array_equal(hsc, asc)
+
+
+def test_moe_layer_composition():
+    """orc_moe_layer against a float64 numpy composition of its parts."""
+    qtype, NE, NU, E, F, T = Q4_K, 4, 2, 256, 256, 6
+    Wg, Wu, Wd = (make_weights(qtype, NE * F, E, seed=1), make_weights(qtype, NE * F, E, seed=2),
+                  make_weights(qtype, NE * E, F, seed=3))
+    aq, asc, _ = orc.quantize_act(make_acts(T, E, seed=4))
+    lg = np.random.default_rng(5).standard_normal((T, NE)).astype(np.float32)
+    out, h = orc.moe_layer(qtype, Wg, Wu, Wd, NE, NU, E, F, aq, asc, lg)
+    wg = orc.dequant_rows(qtype, Wg, NE * F, E).astype(np.float64).reshape(NE, F, E)
+    wu = orc.dequant_rows(qtype, Wu, NE * F, E).astype(np.float64).reshape(NE, F, E)
+    wd = orc.dequant_rows(qtype, Wd, NE * E, F).astype(np.float64).reshape(NE, E, F)
+    x = (aq.astype(np.float32) * np.repeat(asc.T, 32, axis=1)).astype(np.float64)
+    ids, wts, _, _ = orc.moe_route(lg, NE, NU)
+    want = np.zeros((T, E))
+    for t in range(T):
+        for k in range(NU):
+            e = ids[t, k]
+            g = (wg[e] @ x[t]).astype(np.float32).astype(np.float64)
+            u = (wu[e] @ x[t]).astype(np.float32)
+            hh = (g / (1 + np.exp(-g))).astype(np.float32) * u
+            assert np.abs(hh - h[t * NU + k]).max() <= 1e-5 * np.abs(hh).max()
+            hq, hsc = orc.moe_quant(h[t * NU + k][None, :])
+            hx = (hq[0].astype(np.float32) * np.repeat(hsc[:, 0], 32)).astype(np.float64)
+            want[t] += float(wts[t, k]) * (wd[e] @ hx)
+    assert rel_err_rows(out, want).max() <= 1e-5
