@@ -79,7 +79,20 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
     const PlanesQ4K pl = planes_q4k(rows, nsb);
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < u; ++i) {
-      memcpy(dst + pl.hdr + i * 16, src + i * 144, 16);
+      // header: d, dmin, then the 6-bit scales and mins (GGUF packing, reference src/quants.h:61-69) regrouped as
+      // eight 12-bit entries sc | mn << 6
+      const uint8_t* q = src + i * 144 + 4;
+      uint8_t* h = dst + pl.hdr + i * 16;
+      memcpy(h, src + i * 144, 4);
+      uint32_t w[3] = {0, 0, 0};
+      for (int b = 0; b < 8; ++b) {
+        const uint32_t sc = b < 4 ? (q[b] & 63u) : ((q[b + 4] & 0xFu) | ((uint32_t)(q[b - 4] >> 6) << 4));
+        const uint32_t mn = b < 4 ? (q[b + 4] & 63u) : ((uint32_t)(q[b + 4] >> 4) | ((uint32_t)(q[b] >> 6) << 4));
+        const uint64_t e = (uint64_t)(sc | (mn << 6)) << ((12 * b) & 31);
+        w[(12 * b) >> 5] |= (uint32_t)e;
+        if (((12 * b) >> 5) < 2) w[((12 * b) >> 5) + 1] |= (uint32_t)(e >> 32);
+      }
+      memcpy(h + 4, w, 12);
       memcpy(dst + pl.qs + i * 128, src + i * 144 + 16, 128);
     }
     return 0;

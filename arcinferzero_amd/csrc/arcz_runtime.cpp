@@ -26,6 +26,7 @@ struct arcz_kernel {
   const KernelSpec* spec;
   std::string symbol;
   std::vector<int> hidden;  // the -D values that ride along as trailing int arguments
+  unsigned lds = 0;         // dynamic LDS bytes of every launch (-DLDS)
 };
 struct arcz_event {
   hipEvent_t start, stop;
@@ -41,7 +42,7 @@ struct Runtime {
   std::string name;
   std::set<arcz_mem*> mems;
   size_t device_bytes = 0;
-  std::map<std::string, hipModule_t> modules;
+  std::map<std::string, std::vector<hipModule_t>> modules;  // a module may be several code objects
   std::map<std::string, arcz_kernel*> kernels;
   int (*oom_hook)(void) = nullptr;
   long fake_oom = 0, allocs = 0;
@@ -77,7 +78,8 @@ bool out_of_bounds(const char* what, const arcz_mem* b, size_t off, size_t n) {
 extern "C" {
 
 // the code objects, linked in by kernel_blobs.S
-extern const unsigned char arcz_blob_ops[], arcz_blob_decode[], arcz_blob_gemm[], arcz_blob_moe[];
+extern const unsigned char arcz_blob_ops[], arcz_blob_decode[], arcz_blob_decode_q80[], arcz_blob_decode_q4k[],
+    arcz_blob_decode_q6k[], arcz_blob_gemm[], arcz_blob_moe[];
 
 int arcz_init(int device) {
   if (R.up) return ARCZ_OK;
@@ -100,7 +102,8 @@ void arcz_shutdown(void) {
   hipStreamSynchronize(R.stream);
   for (auto& kv : R.kernels) delete kv.second;
   R.kernels.clear();
-  for (auto& kv : R.modules) hipModuleUnload(kv.second);
+  for (auto& kv : R.modules)
+    for (hipModule_t m : kv.second) hipModuleUnload(m);
   R.modules.clear();
   for (arcz_mem* m : R.mems) {
     if (m->owner) hipFree(m->ptr);
@@ -221,12 +224,12 @@ int arcz_fill(arcz_mem* dst, const void* pattern, size_t ps, size_t offset, size
 
 // ---- kernels
 
-static const unsigned char* blob_of(const std::string& which) {
-  if (which == "ops") return arcz_blob_ops;
-  if (which == "decode") return arcz_blob_decode;
-  if (which == "gemm") return arcz_blob_gemm;
-  if (which == "moe") return arcz_blob_moe;
-  return nullptr;
+static std::vector<const unsigned char*> blobs_of(const std::string& which) {
+  if (which == "ops") return {arcz_blob_ops};
+  if (which == "decode") return {arcz_blob_decode, arcz_blob_decode_q80, arcz_blob_decode_q4k, arcz_blob_decode_q6k};
+  if (which == "gemm") return {arcz_blob_gemm};
+  if (which == "moe") return {arcz_blob_moe};
+  return {};
 }
 
 // "-DQT=12 -DGROWS=2 -cl-whatever" -> {QT: 12, GROWS: 2}; a -D without a value is 1
@@ -267,33 +270,45 @@ arcz_kernel* arcz_kernel_get(const char* which, const char* defs, const char* na
     symbol += (i == 0 ? "__" : "_") + std::string(spec->variant[i]) + std::to_string(f->second);
   }
   std::vector<int> hidden;
+  unsigned lds = 0;
   for (int i = 0; spec->hidden[i].name; ++i) {
     auto f = dv.find(spec->hidden[i].name);
     if (f == dv.end() && spec->hidden[i].required) {
       fail(ARCZ_E_BUILD, "%s: -D%s is required", nm.c_str(), spec->hidden[i].name);
       return nullptr;
     }
-    hidden.push_back(f == dv.end() ? spec->hidden[i].def : (int)f->second);
+    const int v = f == dv.end() ? spec->hidden[i].def : (int)f->second;
+    if (std::string(spec->hidden[i].name) == "LDS") {
+      if (v < 0 || v > 65536) { fail(ARCZ_E_BUILD, "%s: %d bytes of LDS", nm.c_str(), v); return nullptr; }
+      lds = (unsigned)v;
+    } else {
+      hidden.push_back(v);
+    }
   }
-  hipModule_t mod;
   auto mi = R.modules.find(w);
   if (mi == R.modules.end()) {
-    const unsigned char* blob = blob_of(w);
-    if (!blob) { fail(ARCZ_E_BUILD, "no module %s", w.c_str()); return nullptr; }
-    hipError_t e = hipModuleLoadData(&mod, blob);
-    if (e != hipSuccess) { fail(ARCZ_E_BUILD, "module %s does not load: %s", w.c_str(), hipGetErrorString(e)); return nullptr; }
-    R.modules[w] = mod;
-  } else {
-    mod = mi->second;
+    const std::vector<const unsigned char*> blobs = blobs_of(w);
+    if (blobs.empty()) { fail(ARCZ_E_BUILD, "no module %s", w.c_str()); return nullptr; }
+    std::vector<hipModule_t> mods;
+    for (const unsigned char* blob : blobs) {
+      hipModule_t mod;
+      hipError_t e = hipModuleLoadData(&mod, blob);
+      if (e != hipSuccess) { fail(ARCZ_E_BUILD, "module %s does not load: %s", w.c_str(), hipGetErrorString(e)); return nullptr; }
+      mods.push_back(mod);
+    }
+    mi = R.modules.emplace(w, mods).first;
   }
-  hipFunction_t fn;
-  hipError_t e = hipModuleGetFunction(&fn, mod, symbol.c_str());
-  if (e != hipSuccess) {
+  hipFunction_t fn = nullptr;
+  for (hipModule_t mod : mi->second) {
+    if (hipModuleGetFunction(&fn, mod, symbol.c_str()) == hipSuccess) break;
     (void)hipGetLastError();
+    fn = nullptr;
+  }
+  if (!fn) {
     fail(ARCZ_E_BUILD, "module %s has no variant %s (defs \"%s\")", w.c_str(), symbol.c_str(), d.c_str());
     return nullptr;
   }
-  arcz_kernel* k = new arcz_kernel{fn, spec, symbol, hidden};
+  arcz_kernel* k = new arcz_kernel{fn, spec, symbol, hidden, lds};
   R.kernels[key] = k;
   return k;
 }
@@ -359,7 +374,7 @@ int arcz_launch(arcz_kernel* k, unsigned dim, const size_t* global, const size_t
     HIP_TRY(hipEventCreate(&ev->stop));
     HIP_TRY(hipEventRecord(ev->start, R.stream));
   }
-  hipError_t e = hipModuleLaunchKernel(k->fn, gs[0] / ls[0], gs[1] / ls[1], gs[2] / ls[2], ls[0], ls[1], ls[2], 0,
+  hipError_t e = hipModuleLaunchKernel(k->fn, gs[0] / ls[0], gs[1] / ls[1], gs[2] / ls[2], ls[0], ls[1], ls[2], k->lds,
                                        R.stream, params, nullptr);
   if (e != hipSuccess) {
     if (ev) { hipEventDestroy(ev->start); hipEventDestroy(ev->stop); delete ev; }

@@ -178,26 +178,44 @@ class Engine {
       throw std::runtime_error(std::string("matmul ") + name + ": the output does not fit C");
     int a = acc;
     cl_mem tabs = nullptr;  // (the reference's codebook tables: none of the three types has one)
-    if (cur_T_ == 1) {
+    if (cur_T_ >= 1 && cur_T_ <= 8) {
       if (a > 1) throw std::logic_error(std::string("GEMV with a fused epilogue: ") + name);
-      const int grows = gemv1_rows(w);
-      int N = w.N, K = w.K, M = Mp;
-      rd_bytes += raw_bytes(w);
-      cl_kernel k = kernel("decode", "-DQT=" + std::to_string(w.type) + " -DGROWS=" + std::to_string(grows), "gemv");
-      set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
-      const size_t hws = (size_t)(N + grows - 1) / grows, l1 = 256;
-      size_t g1 = (hws * 32 + l1 - 1) / l1 * l1;
-      run(name, k, 1, &g1, &l1);
-      return;
-    }
-    if (cur_T_ > 1 && cur_T_ <= 8) {
-      if (a > 1) throw std::logic_error(std::string("GEMV with a fused epilogue: ") + name);
-      const int gr = gemv_mt_rows(w);
-      cl_kernel k = kernel("decode", "-DQT=" + std::to_string(w.type) + " -DGROWS=" + std::to_string(gr) + " -DTB=" +
-                                         std::to_string(cur_T_), "gemv_mt");
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
       rd_bytes += raw_bytes(w);
-      set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a);
+      // The main kernels stage the tokens' activations in LDS (gemv / gemv_mt); when T tokens of K values do not fit
+      // the 64 KiB a launch may ask for, the kernels that read them from global memory take over (gemv_v / gemv_mt_v).
+      const int ups = w.type == GGML_Q8_0 ? 16 : 8, units = K / 256 * ups;
+      const int tok_bytes = (w.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (w.type == GGML_Q4_K ? 8 : 4));
+      static const int force_v = getenv("ARCZ_GEMV_V") ? atoi(getenv("ARCZ_GEMV_V")) : 0;
+      // lanes per row: the fewest of 32 / 64 / 128 / 256 that leave a lane at most 6 sixteen-byte units of a row
+      static const int force_lpr = getenv("ARCZ_GEMV_LPR") ? atoi(getenv("ARCZ_GEMV_LPR")) : 0;
+      int lpr = 0;
+      for (int l : {32, 64, 128, 256})
+        if (!lpr && (units + l - 1) / l <= 6 && (!force_lpr || l == force_lpr)) lpr = l;
+      const int g = lpr ? 256 / lpr : 1, wpr = lpr > 64 ? lpr / 64 : 1;
+      const int tbl = T <= 2 ? T : T <= 4 ? 4 : 8;  // the kernel's token count (T rounded up)
+      const size_t lds = (size_t)tbl * tok_bytes + (wpr > 1 ? (size_t)2 * g * wpr * tbl * 4 : 0);
+      if (!force_v && lpr && lds <= 65536) {
+        const int pf = (units + lpr - 1) / lpr, tb = T <= 2 ? T : T <= 4 ? 4 : 8;
+        // one round of resident work-groups, rows dealt to them in turn (ARCZ_GEMV_WPC: work-groups per compute unit)
+        static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
+        const size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : 3));
+        const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
+                                 std::to_string(pf) + (T > 1 ? " -DTB=" + std::to_string(tb) : std::string()) + " -DLDS=" +
+                                 std::to_string(lds);
+        cl_kernel k = kernel("decode", defs, T == 1 ? "gemv" : "gemv_mt");
+        if (T == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
+        else set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a);
+        size_t g1 = wgs * 256, l1 = 256;
+        run(name, k, 1, &g1, &l1);
+        return;
+      }
+      const int gr = T == 1 ? gemv1_rows(w) : gemv_mt_rows(w);
+      const std::string defs = "-DQT=" + std::to_string(w.type) + " -DGROWS=" + std::to_string(gr) +
+                               (T > 1 ? " -DTB=" + std::to_string(T) : std::string());
+      cl_kernel k = kernel("decode", defs, T == 1 ? "gemv_v" : "gemv_mt_v");
+      if (T == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
+      else set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a);
       size_t g1 = ((size_t)(N + gr - 1) / gr * 32 + 255) / 256 * 256, l1 = 256;
       run(name, k, 1, &g1, &l1);
       return;

@@ -4,7 +4,7 @@
 #pragma once
 
 struct HiddenDef {
-  const char* name;  // nullptr ends the list
+  const char* name;  // nullptr ends the list; "LDS" is not an argument: it is the launch's dynamic LDS size in bytes
   int def;
   bool required;
 };
@@ -26,8 +26,10 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},
     // ---- decode
-    {"decode", "gemv", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{nullptr, 0, false}}, 256},
-    {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{nullptr, 0, false}}, 256},
+    {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
+    {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "LPR", "PF", "TB", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
+    {"decode", "gemv_v", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{nullptr, 0, false}}, 256},
+    {"decode", "gemv_mt_v", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{nullptr, 0, false}}, 256},
     // ---- gemm
     {"gemm", "gemm", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},

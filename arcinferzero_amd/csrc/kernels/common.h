@@ -21,7 +21,9 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 // consecutive lanes read consecutive 16-byte units.  The byte count equals the GGUF byte count except Q6_K's 2-byte
 // scale per superblock, which keeps its size (the plane as a whole is padded to 16 bytes).
 //   Q4_K : qs  [R][nsb][128]  (GGUF order: byte l of chunk j = element 64j+l low nibble, 64j+32+l high nibble)
-//          hdr [R][nsb][16]   (f16 d, f16 dmin, 12 bytes of packed 6-bit scales / mins, as in GGUF)
+//          hdr [R][nsb][16]   (f16 d, f16 dmin, then eight 12-bit entries sc_b | mn_b << 6 at bit 12 b: the 6-bit scale
+//                              and min of sub-block b, regrouped from GGUF's packing so that the pair of entries of a
+//                              64-element chunk is one 24-bit field)
 //   Q6_K : ql  [R][nsb][128], qh [R][nsb][64], sc [R][nsb][16] (int8), d [R][nsb] (f16)
 //   Q8_0 : qs  [R][nsb][256] (int8), d [R][nsb][8] (f16)
 // Plane offsets from the start of the buffer, in bytes (each a multiple of 256 when R * nsb is a multiple of 16;
@@ -68,21 +70,16 @@ __device__ inline float f16_bits_to_f32(uint32_t h) {
 // Per-byte (q - 32) for four 6-bit unsigned values packed in a word, without borrows between bytes.
 __device__ inline uint32_t sub32_bytes(uint32_t q) { return ((q | 0x80808080u) - 0x20202020u) ^ 0x80808080u; }
 
-// 6-bit scale and min of Q4_K sub-blocks 2j and 2j+1 from the three words of packed scale bytes (bytes 0-3, 4-7,
-// 8-11 of the 12: the GGUF packing, reference src/quants.h:61-69).
+// 6-bit scale and min of Q4_K sub-blocks 2j and 2j+1 from the three words of entries of the device header
+// (bits 24 j .. 24 j + 23 of the 96-bit string s0 | s1 << 32 | s2 << 64).  Branch-free: j differs between lanes.
 __device__ inline void q4k_scales_pair(uint32_t s0, uint32_t s1, uint32_t s2, int j, int& sc0, int& sc1, int& mn0,
                                        int& mn1) {
-  const int sh = 16 * (j & 1);
-  const uint32_t x0 = s0 >> sh, x1 = s1 >> sh, y = s2 >> sh;
-  if (j < 2) {
-    sc0 = x0 & 63; sc1 = (x0 >> 8) & 63;
-    mn0 = x1 & 63; mn1 = (x1 >> 8) & 63;
-  } else {
-    sc0 = (y & 0xF) | (((x0 >> 6) & 3) << 4);
-    sc1 = ((y >> 8) & 0xF) | (((x0 >> 14) & 3) << 4);
-    mn0 = ((y >> 4) & 0xF) | (((x1 >> 6) & 3) << 4);
-    mn1 = ((y >> 12) & 0xF) | (((x1 >> 14) & 3) << 4);
-  }
+  const uint32_t lo = j < 2 ? s0 : (j == 2 ? s1 : s2), hi = j < 2 ? s1 : s2;
+  const uint32_t g = __builtin_amdgcn_alignbit(hi, lo, (24 * j) & 31);
+  sc0 = g & 63;
+  mn0 = (g >> 6) & 63;
+  sc1 = (g >> 12) & 63;
+  mn1 = (g >> 18) & 63;
 }
 
 __device__ inline int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }

@@ -168,18 +168,19 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
     }
 }
 
-// gemv: one token.  Arguments as the reference's gemv (zero/kernels/decode.cl:913-915); `tabs` (its codebook
-// tables) is unused by these three types.  grid: ceil(N / GROWS) half waves in work-groups of 256.
+// gemv_v: one token, activations read straight from global memory (the fallback when a chunk's activations do not
+// fit LDS).  Arguments as the reference's gemv_v (zero/kernels/decode.cl:1353); `tabs` (its codebook tables) is
+// unused by these three types.  grid: ceil(N / GROWS) half waves in work-groups of 256.
 #define GEMV_INST(QT, GROWS)                                                                                         \
-  extern "C" __global__ __launch_bounds__(256) void gemv__QT##QT##_GROWS##GROWS(                                      \
+  extern "C" __global__ __launch_bounds__(256) void gemv_v__QT##QT##_GROWS##GROWS(                                      \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
       const short* absum, int M, float* C, int c_off, int accumulate) {                                               \
     gemv_body<QT, 1, GROWS>(raw, N, K, aq, asc, absum, M, 1, C, 0, c_off, accumulate, (size_t)N);                    \
   }
 
-// gemv_mt: T = TB tokens (reference zero/kernels/decode.cl:1581-1583).
+// gemv_mt_v: T = TB tokens (reference zero/kernels/decode.cl:1426).
 #define GEMV_MT_INST(QT, GROWS, TB)                                                                                  \
-  extern "C" __global__ __launch_bounds__(256) void gemv_mt__QT##QT##_GROWS##GROWS##_TB##TB(                          \
+  extern "C" __global__ __launch_bounds__(256) void gemv_mt_v__QT##QT##_GROWS##GROWS##_TB##TB(                          \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
       const short* absum, int M, int T, float* C, int ldc, int c_off, int accumulate) {                               \
     gemv_body<QT, TB, GROWS>(raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, (size_t)N);                 \

@@ -35,10 +35,10 @@ def test_buffers_views_transfers(rt):
 
 
 def test_kernel_lookup_and_launch_checks(rt):
-    k = rt.kernel("decode", "-cl-intel-256-GRF-per-thread -DQT=12 -DGROWS=2", "gemv")   # non -D options are ignored
-    assert az.lib.arcz_kernel_symbol(k) == b"gemv__QT12_GROWS2"
-    assert rt.kernel("decode", "-cl-intel-256-GRF-per-thread -DQT=12 -DGROWS=2", "gemv") == k   # cached by key
-    for bad in (("decode", "-DQT=12", "gemv"), ("decode", "-DQT=99 -DGROWS=1", "gemv"), ("nope", "", "gemv"),
+    k = rt.kernel("decode", "-cl-intel-256-GRF-per-thread -DQT=12 -DGROWS=2", "gemv_v")   # non -D options are ignored
+    assert az.lib.arcz_kernel_symbol(k) == b"gemv_v__QT12_GROWS2"
+    assert rt.kernel("decode", "-cl-intel-256-GRF-per-thread -DQT=12 -DGROWS=2", "gemv_v") == k   # cached by key
+    for bad in (("decode", "-DQT=12", "gemv_v"), ("decode", "-DQT=99 -DGROWS=1", "gemv_v"), ("nope", "", "gemv_v"),
                 ("moe", "-DNU=8", "moe_route")):
         with pytest.raises(az.ArczError) as e:
             rt.kernel(*bad)

@@ -58,7 +58,18 @@ def test_repack_planes_layout(qtype):
     if qtype == az.Q4_K:
         sb = W.reshape(u, 144)
         assert P.size == W.size
-        assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 16:]) and np.array_equal(P[u * 128:].reshape(u, 16), sb[:, :16])
+        assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 16:])
+        hdr = P[u * 128:].reshape(u, 16)
+        assert np.array_equal(hdr[:, :4], sb[:, :4])                       # d, dmin
+        bits = np.zeros(u, dtype=object)
+        for k in range(12):
+            bits = bits + (hdr[:, 4 + k].astype(object) << (8 * k))
+        for r in range(rows):                                               # entries sc | mn << 6 at bit 12 b
+            _, isc, imn, _, _ = orc.decode_row_fields(qtype, W[r * nsb * 144:(r + 1) * nsb * 144], K)
+            for s in range(nsb):
+                for b in range(8):
+                    e = (int(bits[r * nsb + s]) >> (12 * b)) & 0xFFF
+                    assert e == int(isc[s * 16 + 2 * b]) | (int(imn[s * 16 + 2 * b]) << 6)
     elif qtype == az.Q6_K:
         sb = W.reshape(u, 210)
         o = 0
