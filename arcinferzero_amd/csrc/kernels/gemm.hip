@@ -29,9 +29,9 @@
 
 #include "gemm_simple.inc"
 
-struct Gemm2Lds {
-  uint8_t act[BM][BK + LDS_PAD];
-  uint8_t wq[BN][BK + LDS_PAD];
+struct alignas(16) Gemm2Lds {
+  alignas(16) uint8_t act[BM][BK + LDS_PAD];
+  alignas(16) uint8_t wq[BN][BK + LDS_PAD];
   float sa[4][BM];   // activation scale of the step's 4 blocks
   float u[4][BM];    // sa * S (Q4_K)
   float ws[4][BN];   // weight scale d * sc (Q8_0: d)
@@ -44,7 +44,7 @@ template <int QT> struct StepRegs {
   uint4 a[4];                        // 4 x 16 int8 activation values
   uint4 w[QT == QT_Q4_K ? 2 : 4];    // packed weights
   uint4 h;                           // Q4_K header of the thread's row (Q8_0: .x = two f16 scales)
-  float sa[2];
+  float sa[4];                       // scale of the block whose first half the thread stages (even chunks only)
 };
 
 template <int QT>
@@ -58,12 +58,7 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
     const int id = t + 256 * i, row = id >> 3, c = id & 7;
     const int m = max(L.rowmap[row], 0);
     r.a[i] = *(const uint4*)(aq + (size_t)m * K + e0 + 16 * c);
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int id = t + 256 * i, b = id >> 7, row = id & 127;
-    const int m = max(L.rowmap[row], 0);
-    r.sa[i] = asc[(size_t)(s * 8 + 4 * hh + b) * M + m];
+    r.sa[i] = asc[(size_t)(s * 8 + 4 * hh + (c >> 1)) * M + m];
   }
   if constexpr (QT == QT_Q4_K) {
     const PlanesQ4K pl = planes_q4k(rows_total, nsb);
@@ -104,20 +99,13 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
       sh = dot4(r.a[i].w, 0x01010101u, sh);
       ssum[i] = sh + __shfl_xor(sh, 1, 64);  // the block's 32 values: this thread's 16 and its neighbour's
     }
-  }
-  // (the sums land in L.u as S; the caller multiplies them by the scales, which other threads hold, after a barrier)
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int id = t + 256 * i, b = id >> 7, row = id & 127;
-    const float sa = L.rowmap[row] >= 0 ? r.sa[i] : 0.0f;
-    L.sa[b][row] = sa;
+    if ((c & 1) == 0) {  // rows past the tile carry zero scales
+      const float sa = L.rowmap[row] >= 0 ? r.sa[i] : 0.0f;
+      L.sa[c >> 1][row] = sa;
+      if constexpr (QT == QT_Q4_K) L.u[c >> 1][row] = sa * (float)ssum[i];
+    }
   }
   if constexpr (QT == QT_Q4_K) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int id = t + 256 * i, row = id >> 3, c = id & 7;
-      if ((c & 1) == 0) L.u[c >> 1][row] = (float)ssum[i];  // S for now; multiplied by sa after the barrier
-    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
@@ -182,29 +170,40 @@ __device__ inline void gemm2_body(const uint8_t* __restrict__ raw, const signed 
     const int hh = st & 1;
     step_store<QT>(regs, L, hh);
     __syncthreads();
-    if constexpr (QT == QT_Q4_K) {  // U = sa * S
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int id = t + 256 * i, b = id >> 7, row = id & 127;
-        L.u[b][row] *= L.sa[b][row];
-      }
-      __syncthreads();
-    }
     if (st + 1 < steps)  // in flight during the products below
       step_load<QT>(regs, L, raw, rows_total, nsb, row_base, n0, N, aq, asc, M, K, s_begin + ((st + 1) >> 1), (st + 1) & 1);
 
+    // 16 phases (block b, tile (ms, ns)).  Each phase first issues the matrix instructions of a later phase -- the
+    // int8 product of the next tile and, every second phase, the outer product that makes the scale tiles of the next
+    // token half -- and then spends its 32 ALU instructions on the current tile, so the matrix pipe works under the
+    // ALU.  LDS operands are read one block ahead.
+    v4i a16[2], w16[2];            // [ms], [ns]: reloaded for the next block as soon as their last product is issued
+    float saop[2], wsop, uop[2], vop[2];
+    v32f P[2];                     // scale tiles of (b, ms): [ms], both ns
+    v16i I[2];                     // int sums of the current and the next tile
+    auto ld_a = [&](int b, int ms) { a16[ms] = *(const v4i*)&L.act[wm * 64 + ms * 32 + l32][32 * b + 16 * g]; };
+    auto ld_w = [&](int b, int ns) { w16[ns] = *(const v4i*)&L.wq[wn * 64 + ns * 32 + l32][32 * b + 16 * g]; };
+    auto ld_sa = [&](int b, int ms) { saop[ms] = L.sa[b][wm * 64 + ms * 32 + l32]; };
+    // lanes 0-31: columns of tile ns = 0, lanes 32-63: of ns = 1
+    auto ld_ws = [&](int b) { wsop = L.ws[b][wn * 64 + lane]; };
+    auto mfma_p = [&](int ms) {
+      v32f zf;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+      P[ms] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[ms], wsop, zf, 0, 0, 0);
+    };
+    auto mfma_i = [&](int ms, int ns, int slot) {
+      v16i z;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] = 0;
+      I[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[ms], w16[ns], z, 0, 0, 0);
+    };
+    ld_a(0, 0); ld_a(0, 1); ld_w(0, 0); ld_w(0, 1); ld_sa(0, 0); ld_sa(0, 1); ld_ws(0);
+    mfma_p(0);
+    mfma_i(0, 0, 0);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      v4i a16[2], w16[2];
-      float saop[2], uop[2], vop[2];
-#pragma unroll
-      for (int ms = 0; ms < 2; ++ms) {
-        a16[ms] = *(const v4i*)&L.act[wm * 64 + ms * 32 + l32][32 * b + 16 * g];
-        saop[ms] = L.sa[b][wm * 64 + ms * 32 + l32];
-      }
-#pragma unroll
-      for (int ns = 0; ns < 2; ++ns) w16[ns] = *(const v4i*)&L.wq[wn * 64 + ns * 32 + l32][32 * b + 16 * g];
-      const float wsop = L.ws[b][wn * 64 + lane];  // lanes 0-31: columns of tile ns = 0, lanes 32-63: of ns = 1
+      const bool more = b + 1 < 4;
       if constexpr (QT == QT_Q4_K) {
         if ((b & 1) == 0) {  // min term of blocks b and b + 1: lane half g supplies block b + g
 #pragma unroll
@@ -214,25 +213,33 @@ __device__ inline void gemm2_body(const uint8_t* __restrict__ raw, const signed 
         }
       }
 #pragma unroll
-      for (int ms = 0; ms < 2; ++ms) {
-        v32f zf;
-#pragma unroll
-        for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
-        // two outer products: P[ms][0] = sa (x) ws[tile 0], P[ms][1] = sa (x) ws[tile 1]
-        const v32f P = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[ms], wsop, zf, 0, 0, 0);
-#pragma unroll
-        for (int ns = 0; ns < 2; ++ns) {
-          v16i z;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) z[i] = 0;
-          const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[ms], w16[ns], z, 0, 0, 0);
-#pragma unroll
-          for (int i = 0; i < 16; ++i) res[ms][ns][i] = __builtin_fmaf((float)I[i], P[16 * ns + i], res[ms][ns][i]);
-          // the min term goes straight into the same accumulators on the matrix pipe; the ALU comes back to this
-          // tile only after the other three
-          if constexpr (QT == QT_Q4_K)
-            if ((b & 1) == 0) res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop[ns], res[ms][ns], 0, 0, 0);
+      for (int tile = 0; tile < 4; ++tile) {
+        const int ms = tile >> 1, ns = tile & 1, slot = tile & 1;
+        // matrix instructions of later phases, and the LDS operands of the next block into registers just freed
+        if (tile == 0) { mfma_i(0, 1, 1); }
+        if (tile == 1) {
+          mfma_p(1);
+          mfma_i(1, 0, 0);
+          if (more) { ld_a(b + 1, 0); ld_sa(b + 1, 0); }
         }
+        if (tile == 2) {
+          mfma_i(1, 1, 1);
+          if (more) { ld_w(b + 1, 0); ld_ws(b + 1); }
+        }
+        if (tile == 3 && more) {
+          mfma_p(0);
+          mfma_i(0, 0, 0);
+          ld_a(b + 1, 1); ld_w(b + 1, 1); ld_sa(b + 1, 1);
+        }
+        // the current tile on the ALU
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          res[ms][ns][i] = __builtin_fmaf((float)I[slot][i], P[ms][16 * ns + i], res[ms][ns][i]);
+        // the min term goes straight into the same accumulators on the matrix pipe; the ALU comes back to this tile
+        // only after the other three
+        if constexpr (QT == QT_Q4_K)
+          if ((b & 1) == 0) res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop[ns], res[ms][ns], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     __syncthreads();
