@@ -1,4 +1,5 @@
-/* The gfx950 code objects, one per kernel module, as read-only data of the host library. */
+/* The gfx950 code objects, one per kernel module, as read-only data of the host library
+   (found through the assembler's include path: the build directory). */
     .section .rodata
     .macro BLOB name, file
     .balign 4096
@@ -7,11 +8,11 @@
     .incbin "\file"
     .balign 8
     .endm
-    BLOB arcz_blob_ops, "build/ops.hsaco"
-    BLOB arcz_blob_decode, "build/decode.hsaco"
-    BLOB arcz_blob_decode_q80, "build/decode_q80.hsaco"
-    BLOB arcz_blob_decode_q4k, "build/decode_q4k.hsaco"
-    BLOB arcz_blob_decode_q6k, "build/decode_q6k.hsaco"
-    BLOB arcz_blob_gemm, "build/gemm.hsaco"
-    BLOB arcz_blob_moe, "build/moe.hsaco"
+    BLOB arcz_blob_ops, "ops.hsaco"
+    BLOB arcz_blob_decode, "decode.hsaco"
+    BLOB arcz_blob_decode_q80, "decode_q80.hsaco"
+    BLOB arcz_blob_decode_q4k, "decode_q4k.hsaco"
+    BLOB arcz_blob_decode_q6k, "decode_q6k.hsaco"
+    BLOB arcz_blob_gemm, "gemm.hsaco"
+    BLOB arcz_blob_moe, "moe.hsaco"
     .section .note.GNU-stack,"",@progbits

@@ -231,6 +231,7 @@ __device__ inline void gemm2_body(const uint8_t* __restrict__ raw, const signed 
           mfma_i(0, 0, 0);
           ld_a(b + 1, 1); ld_w(b + 1, 1); ld_sa(b + 1, 1);
         }
+        __builtin_amdgcn_sched_barrier(0);  // (keeps the matrix instructions above ahead of the ALU work below)
         // the current tile on the ALU
 #pragma unroll
         for (int i = 0; i < 16; ++i)
