@@ -6,5 +6,5 @@ in and out.  There is no fallback: if the library is missing, importing :mod:`ar
 """
 from .binding import (  # noqa: F401
     Q4_K, Q6_K, Q8_0, ArczError, Buffer, Engine, Runtime, Weight, MoeLayer, gen_normal, gen_weights, gguf_bytes,
-    lib, lib_path, planes_bytes, quantize_rows, repack_planes,
+    lib, lib_path, planes_bytes, quantize_rows, repack_planes, self_check,
 )

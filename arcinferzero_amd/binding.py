@@ -77,6 +77,7 @@ _sig("arcz_engine_layer_moe", _i, _p, _p, _p, _i, _p, _i, _i)
 _sig("arcz_engine_moe_route", _i, _p, _p, _p, _i, _i, _i)
 _sig("arcz_engine_moe_buffer", _p, _p, _i)
 _sig("arcz_engine_moe_slots", _i, _p)
+_sig("arcz_engine_self_check", _i)
 _sig("arcz_engine_profile", None, _p, _i)
 _sig("arcz_engine_profile_collect", _i, _p)
 _sig("arcz_engine_profile_get", _i, _p, C.c_char_p, C.POINTER(C.c_double), C.POINTER(_i))
@@ -98,6 +99,12 @@ def _check(code, engine=False):
 
 def _np_ptr(a):
     return a.ctypes.data_as(C.c_void_p)
+
+
+def self_check():
+    """Tuned GEMM against the simple GEMM and integer sums on LCG data (zero/engine_setup.h:424-520); raises on a
+    difference."""
+    _check(lib.arcz_engine_self_check(), engine=True)
 
 
 # ---------------------------------------------------------------- host helpers (no GPU)

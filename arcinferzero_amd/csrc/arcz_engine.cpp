@@ -97,6 +97,13 @@ arcz_mem* arcz_engine_moe_buffer(arcz_engine* e, int which) {
 }
 int arcz_engine_moe_slots(arcz_engine* e) { return e->e->slots_; }
 
+int arcz_engine_self_check(void) {
+  return guarded([&] {
+    const std::string r = engine_self_check();
+    if (!r.empty()) throw std::runtime_error(r);
+  });
+}
+
 void arcz_engine_profile(arcz_engine* e, int on) { e->e->profile = on != 0; }
 int arcz_engine_profile_collect(arcz_engine* e) {
   return guarded([&] { e->e->collect_profile(); });

@@ -375,3 +375,82 @@ class Engine {
   std::vector<cl_mem> mems_;
   std::vector<std::pair<std::string, cl_event>> events_;
 };
+
+// Start-up check of the tuned GEMM against the simple one (the pattern of xmx_check, zero/engine_setup.h:424-520): both
+// kernels run on the same data from the reference's LCG (1664525 / 1013904223, seed 12345), 128 tokens x 128 rows x
+// K = 1024, with unit scales (weights d = 1, sub-scales 1, mins 1; activation scales 1) so that every f32 output is an
+// integer below 2^24: the two results must be bit-equal to each other and to the integer sums counted on the host.
+// Returns an empty string, or what differed.
+inline std::string engine_self_check() {
+  const int M = 128, N = 128, K = 1024;
+  Engine e(M, K);
+  uint32_t lcg = 12345u;
+  auto next = [&]() { lcg = lcg * 1664525u + 1013904223u; return lcg >> 8; };
+  std::vector<int8_t> aq((size_t)M * K);
+  std::vector<float> asc((size_t)M * (K / 32), 1.0f);
+  std::vector<int16_t> absum((size_t)M * (K / 16));
+  for (auto& v : aq) v = (int8_t)((int)(next() % 255u) - 127);
+  for (int m = 0; m < M; ++m)
+    for (int b = 0; b < K / 16; ++b) {
+      int s = 0;
+      for (int i = 0; i < 16; ++i) s += aq[(size_t)m * K + b * 16 + i];
+      absum[(size_t)b * M + m] = (int16_t)s;
+    }
+  e.set_activations(aq.data(), asc.data(), absum.data(), K, M, M);
+  cl_mem c0 = e.buf((size_t)M * N * 4), c1 = e.buf((size_t)M * N * 4);
+  std::vector<float> y0((size_t)M * N), y1((size_t)M * N);
+  for (uint32_t type : {GGML_Q8_0, GGML_Q4_K}) {
+    const size_t rb = arcz_gguf_bytes(type, 1, K);
+    std::vector<uint8_t> w((size_t)N * rb);
+    std::vector<int> wq((size_t)N * K);  // the integer each element stands for
+    for (int n = 0; n < N; ++n)
+      for (int sb = 0; sb < K / 256; ++sb) {
+        if (type == GGML_Q8_0) {
+          for (int b = 0; b < 8; ++b) {
+            uint8_t* blk = &w[n * rb + (size_t)(sb * 8 + b) * 34];
+            blk[0] = 0x00; blk[1] = 0x3C;  // f16 1.0
+            for (int i = 0; i < 32; ++i) {
+              const int q = (int)(next() % 255u) - 127;
+              blk[2 + i] = (uint8_t)(int8_t)q;
+              wq[(size_t)n * K + sb * 256 + b * 32 + i] = q;
+            }
+          }
+        } else {
+          uint8_t* blk = &w[n * rb + (size_t)sb * 144];
+          blk[0] = 0x00; blk[1] = 0x3C; blk[2] = 0x00; blk[3] = 0x3C;  // d = dmin = 1.0
+          for (int i = 0; i < 8; ++i) blk[4 + i] = 1;                   // 6-bit scales and mins of sub-blocks 0-3: 1
+          for (int i = 0; i < 4; ++i) blk[12 + i] = 0x11;               // low nibbles of those of sub-blocks 4-7: 1
+          for (int j = 0; j < 4; ++j)
+            for (int l = 0; l < 32; ++l) {
+              const int lo = (int)(next() & 15u), hi = (int)(next() & 15u);
+              blk[16 + j * 32 + l] = (uint8_t)(lo | hi << 4);
+              wq[(size_t)n * K + sb * 256 + j * 64 + l] = lo - 1;       // value = 1 * 1 * q - 1 * 1
+              wq[(size_t)n * K + sb * 256 + j * 64 + 32 + l] = hi - 1;
+            }
+        }
+      }
+    GpuWeight gw = e.make_weight(type, w.data(), w.size(), N, K);
+    for (int which = 0; which < 2; ++which) {
+      cl_kernel k = e.kernel("gemm", "-DQTYPE=" + std::to_string(type) + " -DACT32", which ? "gemm_simple" : "gemm");
+      cl_mem unused = nullptr, C = which ? c1 : c0;
+      int MM = M, NN = N, KK = K, ldc = N, zero = 0, one = 1, s1 = K / 256;
+      set_args(k, 0, gw.raw, unused, e.aq_, e.asc_, e.absum_, C, MM, NN, KK, ldc, zero, zero, one, zero, s1);
+      size_t gws[1] = {256}, lws[1] = {256};
+      e.run("self_check", k, 1, gws, lws);
+    }
+    CL_CHECK(clEnqueueReadBuffer(e.cl_.queue, c0, CL_TRUE, 0, y0.size() * 4, y0.data(), 0, nullptr, nullptr));
+    CL_CHECK(clEnqueueReadBuffer(e.cl_.queue, c1, CL_TRUE, 0, y1.size() * 4, y1.data(), 0, nullptr, nullptr));
+    e.free_weight(gw);
+    for (int m = 0; m < M; ++m)
+      for (int n = 0; n < N; ++n) {
+        long long s = 0;
+        for (int k2 = 0; k2 < K; ++k2) s += (long long)aq[(size_t)m * K + k2] * wq[(size_t)n * K + k2];
+        const float a = y0[(size_t)m * N + n], b = y1[(size_t)m * N + n];
+        if (a != (float)s || b != (float)s)
+          return std::string("GEMM self-check ") + ggml_type_name(type) + ": token " + std::to_string(m) + " row " +
+                 std::to_string(n) + ": tuned " + std::to_string(a) + ", simple " + std::to_string(b) + ", integer sum " +
+                 std::to_string(s);
+      }
+  }
+  return std::string();
+}

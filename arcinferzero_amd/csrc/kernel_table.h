@@ -25,6 +25,7 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "mfma_probe", nullptr, "pi", {nullptr}, {{nullptr, 0, false}}, 256},
     // ---- decode
     {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "LPR", "PF", "TB", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},

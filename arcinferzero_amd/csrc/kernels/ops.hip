@@ -99,3 +99,21 @@ extern "C" __global__ void read_probe(const uint4* __restrict__ src, size_t n, u
   }
   if (acc == 0x9E3779B9u) sink[0] = acc;
 }
+
+// mfma_probe: register-resident int8 matrix instructions, four independent 32x32x32 accumulators per wave, `iters`
+// rounds: the issue-rate ceiling of the int8 matrix pipe that the GEMM figures are set against (the reference measures
+// its own in bench/gpu_bench.cpp:10-15).  2 * 32*32*32 * 4 * iters operations per wave.
+extern "C" __global__ __launch_bounds__(256) void mfma_probe(uint32_t* sink, int iters) {
+  v4i a = {(int)threadIdx.x, 1, 2, 3}, b = {4, 5, (int)blockIdx.x, 7};
+  v16i c0 = {}, c1 = {}, c2 = {}, c3 = {};
+  for (int i = 0; i < iters; ++i) {
+    c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c0, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, c1, 0, 0, 0);
+    c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, a, c2, 0, 0, 0);
+    c3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, b, c3, 0, 0, 0);
+  }
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s ^= c0[i] ^ c1[i] ^ c2[i] ^ c3[i];
+  if (s == 0x12345678) sink[0] = (uint32_t)s;
+}

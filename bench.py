@@ -20,6 +20,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
+# HBM bytes one launch of the headline GEMM moves, from two counter runs of this script (FETCH_SIZE x 2.0 KiB read,
+# WRITE_SIZE x 1.0 KiB written, the factors calibrated on the 2 GiB copy in the same runs): 1986.2 MB + 570.4 MB
+GEMM_HBM_BYTES_PER_LAUNCH = 2.557e9
 
 
 def log(*a):
@@ -128,29 +131,143 @@ def bench_decode(az, qtype, N, K, T, launches, copies):
             "distinct_weight_MB": copies * az.gguf_bytes(qtype, N, K) / 1e6}
 
 
-def cpu_baseline(az, W, qtype, N, K, budget_s=12.0):
-    """The oracle's restatement of the reference CPU matmul (dequant row -> double-accumulated dots), all host cores,
-    on a bounded sample of config 2: the first rows x tokens that fit the time budget."""
+def bench_gemm_config(az, qtype, N, K, M, launches, seed, W=None):
+    """One GEMM (or GEMV-form, M <= 8) configuration: per-launch device time from events around `launches` launches."""
+    eng = az.Engine(max(M, 16), K)
+    if W is None:
+        W = az.gen_weights(qtype, seed, N, K, 0.02)
+    w = eng.make_weight(qtype, N, K, W)
+    Mp = M if M > 8 else 16
+    xb = az.Runtime.from_numpy(az.gen_normal(seed + 1, (M, K)))
+    eng.quantize(xb, K, K, Mp, M)
+    cb = az.Runtime.alloc(max(M, 1) * N * 4)
+    eng.matmul("cfg", w, Mp, cb, N, 0, 0)
+    az.Runtime.sync()
+    e0 = az.Runtime.event()
+    for _ in range(launches):
+        eng.matmul("cfg", w, Mp, cb, N, 0, 0)
+    e1 = az.Runtime.event()
+    az.Runtime.sync()
+    ms = az.Runtime.elapsed_ms(e0, e1) / launches
+    az.Runtime.event_release(e0)
+    az.Runtime.event_release(e1)
+    ops = 2.0 * M * N * K
+    nbytes = az.gguf_bytes(qtype, N, K) + M * (K + K // 32 * 4 + K // 16 * 2) + M * N * 4
+    for b in (cb, xb):
+        b.free()
+    w.free()
+    eng.close()
+    return {"M": M, "N": N, "K": K, "ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12,
+            "frac_int8_peak": ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, "GBps": nbytes / (ms * 1e-3) / 1e9,
+            "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS}, W
+
+
+def bench_moe(az, launches):
+    """BASELINE configs[4]: 128 experts, top-8, 4096 tokens, hidden 2048, expert FFN 768, Q4_K; the whole layer
+    (route, sort, gate/up tile GEMM with SwiGLU, expert-input quantization, down tile GEMM, combine) per launch."""
+    NE, NU, T, E, F, qt = 128, 8, 4096, 2048, 768, az.Q4_K
+    eng = az.Engine(T, E)
+    Wg = az.gen_weights(qt, 21, NE * F, E, 0.02)
+    Wu = az.gen_weights(qt, 22, NE * F, E, 0.02)
+    Wd = az.gen_weights(qt, 23, NE * E, F, 0.02)
+    L = eng.make_moe_layer(qt, Wg, Wu, Wd, NE, NU, E, F)
+    del Wg, Wu, Wd
+    xb = az.Runtime.from_numpy(az.gen_normal(24, (T, E)))
+    lb = az.Runtime.from_numpy(az.gen_normal(25, (T, NE)))
+    ob = az.Runtime.alloc(T * E * 4).fill(0)
+    eng.quantize(xb, E, E, T, T)
+    eng.layer_moe(L, lb, NE, ob, T, T)
+    az.Runtime.sync()
+    eng.profile(True)
+    e0 = az.Runtime.event()
+    for _ in range(launches):
+        eng.layer_moe(L, lb, NE, ob, T, T)
+    e1 = az.Runtime.event()
+    az.Runtime.sync()
+    ms = az.Runtime.elapsed_ms(e0, e1) / launches
+    az.Runtime.event_release(e0)
+    az.Runtime.event_release(e1)
+    eng.profile_collect()
+    parts = {}
+    for name in ("moe_route", "moe_scan", "moe_scatter", "moe_gateup", "moe_quant", "moe_down", "moe_combine"):
+        t, n = eng.profile_get(name)
+        parts[name + "_ms"] = t / max(n, 1) * (2 if name == "moe_gateup" else 1)   # gate and up are two launches
+    ops = T * NU * 3 * 2.0 * F * E
+    gemm_ms = parts["moe_gateup_ms"] + parts["moe_down_ms"]
+    for b in (xb, lb, ob):
+        b.free()
+    eng.close()
+    return {"tokens": T, "experts": NE, "top": NU, "hidden": E, "ffn": F, "layer_ms": ms, "ops": ops,
+            "layer_TOPS": ops / (ms * 1e-3) / 1e12, "gemm_kernels_ms": gemm_ms,
+            "gemm_TOPS": ops / (gemm_ms * 1e-3) / 1e12, "gemm_frac_int8_peak": ops / (gemm_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS,
+            **parts}
+
+
+def bench_probes(az):
+    """What the machine itself delivers: a streaming read and a copy over 2 GiB, and the issue rate of register-resident
+    int8 matrix instructions."""
+    n = 2 << 30
+    src = az.Runtime.alloc(n).fill(0x01020304)
+    dst = az.Runtime.alloc(n)
+    sink = az.Runtime.alloc(64).fill(0)
+    cus = az.Runtime.cus()
+    out = {}
+    k = az.Runtime.kernel("ops", "", "read_probe")
+    grid = (cus * 8 * 256,)
+    best = 1e9
+    for _ in range(5):
+        best = min(best, az.Runtime.launch(k, grid, (256,), [src, ("z", n // 16), sink], timed=True))
+    out["read_GBps"] = n / (best * 1e-3) / 1e9
+    k = az.Runtime.kernel("ops", "", "copy128")
+    best = 1e9
+    for _ in range(5):
+        best = min(best, az.Runtime.launch(k, grid, (256,), [src, dst, ("z", n // 16)], timed=True))
+    out["copy_GBps_read_plus_write"] = 2 * n / (best * 1e-3) / 1e9
+    k = az.Runtime.kernel("ops", "", "mfma_probe")
+    iters, wgs = 20000, cus * 8
+    best = 1e9
+    for _ in range(3):
+        best = min(best, az.Runtime.launch(k, (wgs * 256,), (256,), [sink, iters], timed=True))
+    out["int8_mfma_issue_TOPS"] = 2.0 * 32 * 32 * 32 * 4 * iters * wgs * 4 / (best * 1e-3) / 1e12
+    for b in (src, dst, sink):
+        b.free()
+    return out
+
+
+def cpu_baseline(az, W, qtype, N, K, budget_s=15.0):
+    """The oracle's restatement of the reference CPU matmul (dequant row -> double-accumulated dots, OpenMP over rows;
+    tools/ref_forward.cpp:251-305), all host cores, on a bounded sample of config 2 (the first rows x tokens that fit
+    the time budget), and on config 1 (Q8_0 4096 x 4096, 512 tokens) in full."""
     import tests.oracle_lib as orc
     rb = az.gguf_bytes(qtype, 1, K)
-    x = az.gen_normal(2, (64, K))
-    aq, asc, _ = orc.quantize_act(x)
+    M = 8192
+    xc = az.gen_normal(2, (256, K))
+    aqc, ascc, _ = orc.quantize_act(xc)
+    orc.matmul_ref(qtype, W[:64 * rb], 64, K, aqc, ascc)          # warm the threads up
     t0 = time.perf_counter()
-    orc.matmul_ref(qtype, W[:256 * rb], 256, K, aq, asc)
-    dt = time.perf_counter() - t0
-    rate = 2.0 * 64 * 256 * K / max(dt, 1e-6)
-    toks = 256
-    rows = int(min(N, max(256, budget_s * rate / (2.0 * toks * K))))
-    rows -= rows % 16
-    x = az.gen_normal(2, (toks, K))
-    aq, asc, _ = orc.quantize_act(x)
+    orc.matmul_ref(qtype, W[:1024 * rb], 1024, K, aqc, ascc)      # calibration
+    rate = 2.0 * 256 * 1024 * K / max(time.perf_counter() - t0, 1e-3)
+    # all weight rows, and as many of the 8192 tokens as the budget allows (in steps of 256); fewer rows on a slow host
+    toks = int(min(M, max(256, budget_s * rate / (2.0 * N * K) // 256 * 256)))
+    rows = N if toks > 256 else int(min(N, max(512, budget_s * rate / (2.0 * 256 * K) // 16 * 16)))
+    x = az.gen_normal(2, (M, K))[:toks]
+    aq, asc, _ = orc.quantize_act(np.ascontiguousarray(x))
     t0 = time.perf_counter()
     orc.matmul_ref(qtype, W[:rows * rb], rows, K, aq, asc)
     dt = time.perf_counter() - t0
     ops = 2.0 * toks * rows * K
+    # config 1 in full
+    N1, K1, M1 = 4096, 4096, 512
+    W1 = az.gen_weights(az.Q8_0, 31, N1, K1, 0.02)
+    aq1, asc1, _ = orc.quantize_act(az.gen_normal(32, (M1, K1)))
+    t0 = time.perf_counter()
+    orc.matmul_ref(az.Q8_0, W1, N1, K1, aq1, asc1)
+    dt1 = time.perf_counter() - t0
     return {"value": ops / dt / 1e12, "unit": "TOP/s", "cores": orc.num_threads(), "kind": "port",
-            "sample": f"first {rows} of {N} weight rows x first {toks} of 8192 tokens, K={K}: {dt:.2f} s "
-                      f"({ops / dt / 1e9:.1f} GFLOP/s of 2*M*N*K; dequant row + double-accumulated dot, OpenMP)"}
+            "sample": f"first {rows} of {N} weight rows x first {toks} of {M} tokens, K={K}: {dt:.2f} s "
+                      f"({ops / dt / 1e9:.1f} G op/s of 2*M*N*K; dequant row + double-accumulated dot, OpenMP)",
+            "config1_full": {"workload": "Q8_0 4096x4096, 512 tokens", "seconds": dt1,
+                             "TOPS": 2.0 * M1 * N1 * K1 / dt1 / 1e12}}
 
 
 def main():
@@ -160,6 +277,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV extras")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the other configurations (Q8_0 GEMM, Q6_K output head, MoE layer) and the machine probes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -179,7 +298,8 @@ def main():
                                "quantized to int8 per 32 in the step, out 8192x17408 f32 (BASELINE configs[1])",
                    "M": M, "N": N, "K": K, "step": "quant_rows + gemm"},
         "roofline": {"bound": "mfma", "achieved": pre["kernel_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": pre["kernel_tops"] / PEAK_INT8_TOPS, "traffic": None, "kernel": "gemm__QTYPE12_ACT321",
+                     "frac": pre["kernel_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH,
+                     "kernel": "gemm__QTYPE12_ACT321",
                      "kernel_ms": pre["gemm_kernel_ms"], "ops_per_launch": pre["ops"]},
         "parity_rel_err_sampled": pre["parity_rel_err"],
         "quant_kernel_ms": pre["quant_kernel_ms"],
@@ -190,6 +310,21 @@ def main():
         d2 = bench_decode(az, az.Q4_K, 5120, 17408, 2, 200, 8)
         log(f"[bench] decode T=2: {d2}")
         out["decode"] = {"Q4_K_17408x5120_T1": d1, "Q4_K_5120x17408_T2": d2, "hbm_peak_GBps": PEAK_HBM_GBS}
+    if not args.no_extras:
+        az.self_check()
+        c1, _ = bench_gemm_config(az, az.Q8_0, 4096, 4096, 512, 50, 31)
+        log(f"[bench] Q8_0 4096x4096 M=512: {c1}")
+        out["other_configs"] = {"Q8_0_4096x4096_M512": c1}
+        W6 = None
+        for M, launches in ((1, 50), (64, 20), (2048, 3)):
+            r, W6 = bench_gemm_config(az, az.Q6_K, 151936, 5120, M, launches, 41, W6)
+            log(f"[bench] Q6_K 151936x5120 M={M}: {r}")
+            out["other_configs"][f"Q6_K_151936x5120_M{M}"] = r
+        del W6
+        out["other_configs"]["MoE_128x8_T4096_E2048_F768_Q4_K"] = bench_moe(az, 5)
+        log(f"[bench] MoE: {out['other_configs']['MoE_128x8_T4096_E2048_F768_Q4_K']}")
+        out["machine_probes"] = bench_probes(az)
+        log(f"[bench] probes: {out['machine_probes']}")
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(az, W, qtype, N, K)
     print(json.dumps(out), flush=True)

@@ -62,6 +62,11 @@ int arcz_engine_moe_route(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, i
 arcz_mem* arcz_engine_moe_buffer(arcz_engine* e, int which);
 int arcz_engine_moe_slots(arcz_engine* e);
 
+/* The start-up check of the tuned GEMM against the simple one on the reference's LCG data, both against integer sums
+ * counted on the host (the pattern of xmx_check, zero/engine_setup.h:424-520).  0, or ARCZ_E_ENGINE with the first
+ * difference in arcz_engine_error(). */
+int arcz_engine_self_check(void);
+
 /* Engine::profile / collect_profile (zero/engine.h:936-950): per-launch device time summed by name. */
 void arcz_engine_profile(arcz_engine* e, int on);
 int arcz_engine_profile_collect(arcz_engine* e);

@@ -103,3 +103,9 @@ def test_gemm_epilogues(eng):
     want = y0.astype(np.float64) * (g / (1.0 + np.exp(-g)))   # C = silu(C) * result (gemm.cl:562-565)
     assert np.abs(ys[:, c_off:c_off + N] - want).max() <= 1e-5 * np.abs(want).max()
     assert np.array_equal(ys[:, :c_off], c0[:, :c_off])
+
+
+def test_startup_self_check(rt):
+    """Tuned GEMM == simple GEMM == host integer sums, bit for bit, on the reference's LCG data with unit scales
+    (the start-up check in the pattern of xmx_check, zero/engine_setup.h:424-520)."""
+    az.self_check()
