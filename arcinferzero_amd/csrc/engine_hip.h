@@ -197,9 +197,10 @@ class Engine {
       const size_t lds = (size_t)tbl * tok_bytes + (wpr > 1 ? (size_t)2 * g * wpr * tbl * 4 : 0);
       if (!force_v && lpr && lds <= 65536) {
         const int pf = (units + lpr - 1) / lpr, tb = T <= 2 ? T : T <= 4 ? 4 : 8;
-        // one round of resident work-groups, rows dealt to them in turn (ARCZ_GEMV_WPC: work-groups per compute unit)
+        // one round of resident work-groups, passes of rows dealt to them in turn (ARCZ_GEMV_WPC: work-groups per
+        // compute unit; two measured best: more add staging work and spread the reads over more rows at a time)
         static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
-        const size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : 3));
+        const size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : 2));
         const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
                                  std::to_string(pf) + (T > 1 ? " -DTB=" + std::to_string(tb) : std::string()) + " -DLDS=" +
                                  std::to_string(lds);
