@@ -271,6 +271,251 @@ __device__ inline void gemm2_body(const uint8_t* __restrict__ raw, const signed 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Q4_K, third form: the bulk operands go from global memory straight into LDS (global_load_lds_dwordx4: a wave moves
+// 1 KB per instruction, lane l's 16 bytes land at base + 16 l, from whatever address lane l names), double-buffered,
+// so the step after the current one streams in under the products with no registers and no ALU work; the weights
+// stay packed in LDS (64 bytes per row and step) and are split into their two nibble blocks when a lane reads its
+// operand.  Rows are not padded: the 16-byte chunk c of row r sits at chunk c ^ f(r), which the loading lane realises
+// by choosing its source address, and which makes the 128-bit operand reads conflict-free.  Only the four scale vectors
+// of a step pass through registers (they need arithmetic); S, the block sums of the activations, come from absum.
+// One barrier per step.
+#define G3_STAGE 32768
+#define G3_WQ 16384
+#define G3_SA 24576
+#define G3_U (G3_SA + 2048)
+#define G3_WS (G3_SA + 4096)
+#define G3_V (G3_SA + 6144)
+
+__device__ inline void g3_dma16(const void* src, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+struct G3ScaleRegs {
+  float sa[2];
+  short bs[4];
+  uint4 h;
+};
+
+template <bool TILES>  // (only the dense form is instantiated: over expert tiles, with their short K, the register-staged
+                       //  body above measured faster)
+__device__ inline void gemm3_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+                                  const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
+                                  int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
+                                  size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
+                                  const int* __restrict__ rowmap, int use_map, const float* __restrict__ rowscale,
+                                  int use_scale) {
+  __shared__ alignas(16) uint8_t lds[2 * G3_STAGE];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8;
+  const PlanesQ4K pl = planes_q4k(rows_total, nsb);
+  auto token_row = [&](int r) {  // global token row of tile row r; rows past the tile read the tile's first row
+    const int rr = r < rows_valid ? r : 0;
+    return (TILES && use_map) ? rowmap[m0 + rr] : m0 + rr;
+  };
+
+  // ---- what this lane fetches each step.  Activations: 4 instructions a wave, 8 rows each; row R = (4 wave + i) 8 +
+  // lane / 8 lands at chunk lane % 8, so the lane names source chunk (lane % 8) ^ (R % 8).  Weights: 2 instructions a
+  // wave, 16 rows each; row R = (2 wave + i) 16 + lane / 4, source chunk (lane % 4) ^ ((R / 2) % 4).
+  // (per-lane parts as 32-bit byte offsets from bases that are the same for the whole wave and advance with the step)
+  uint32_t aoff[4], woff[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int R = (wave * 4 + i) * 8 + (lane >> 3);
+    aoff[i] = (uint32_t)token_row(R) * (uint32_t)K + 16u * ((lane & 7) ^ (lane >> 3));
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int R = (wave * 2 + i) * 16 + (lane >> 2);
+    const int n = min(n0 + R, N - 1);
+    woff[i] = (uint32_t)n * (uint32_t)nsb * 128u + 16u * ((lane & 3) ^ ((lane >> 3) & 3));
+  }
+  const signed char* abase = aq + (size_t)s_begin * 256;
+  const uint8_t* wbase = raw + pl.qs + (row_base * nsb + s_begin) * 128;
+  // scales: thread t prepares token r_s = t % 128, blocks 2 (t / 128) + {0, 1} of the step, and weight row t / 2,
+  // block pair t % 2
+  const int r_s = t & 127, bp = t >> 7;
+  const bool tok_valid = r_s < rows_valid;
+  const uint32_t m_s = (uint32_t)token_row(r_s);
+  const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
+  const uint32_t hoff = (uint32_t)n_s * (uint32_t)nsb * 16u;
+  const uint8_t* hbase = raw + pl.hdr + (row_base * nsb + s_begin) * 16;
+
+  auto dma_step = [&](int st, int stage) {  // st: half-superblock steps from s_begin
+    uint8_t* base = lds + stage * G3_STAGE;
+    const signed char* ab = abase + (size_t)st * 128;
+    const uint8_t* wb = wbase + (size_t)st * 64;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) g3_dma16(ab + aoff[i], base + (wave * 4 + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[i], base + G3_WQ + (wave * 2 + i) * 1024);
+  };
+  // (loads only: anything computed from them here would make the wave wait for the whole step's traffic)
+  auto load_scales = [&](G3ScaleRegs& r, int st) {
+    const float* ap = asc + (size_t)(s_begin * 8 + st * 4 + 2 * bp) * M;
+    const short* bp2 = absum + (size_t)(s_begin * 16 + st * 8 + 4 * bp) * M;
+    r.sa[0] = ap[m_s];
+    r.sa[1] = (ap + M)[m_s];
+    r.bs[0] = bp2[m_s];
+    r.bs[1] = (bp2 + M)[m_s];
+    r.bs[2] = (bp2 + 2 * (size_t)M)[m_s];
+    r.bs[3] = (bp2 + 3 * (size_t)M)[m_s];
+    r.h = *(const uint4*)(hbase + (size_t)(st >> 1) * 16 + hoff);
+  };
+  auto store_scales = [&](const G3ScaleRegs& r, int st, int stage) {
+    uint8_t* base = lds + stage * G3_STAGE;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const float sa = tok_valid ? r.sa[q] : 0.0f;
+      ((float*)(base + G3_SA))[(2 * bp + q) * 128 + r_s] = sa;
+      ((float*)(base + G3_U))[(2 * bp + q) * 128 + r_s] = sa * (float)((int)r.bs[2 * q] + (int)r.bs[2 * q + 1]);
+    }
+    const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
+    int sc0, sc1, mn0, mn1;
+    q4k_scales_pair(r.h.y, r.h.z, r.h.w, 2 * (st & 1) + p_s, sc0, sc1, mn0, mn1);
+    const int row = t >> 1;
+    ((float*)(base + G3_WS))[(2 * p_s) * 128 + row] = d * (float)sc0;
+    ((float*)(base + G3_WS))[(2 * p_s + 1) * 128 + row] = d * (float)sc1;
+    ((float*)(base + G3_V))[(2 * p_s) * 128 + row] = -(dmin * (float)mn0);
+    ((float*)(base + G3_V))[(2 * p_s + 1) * 128 + row] = -(dmin * (float)mn1);
+  };
+
+  // ---- operand addresses of this lane (bytes from a stage's start)
+  int oa[4], ow[2];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) oa[b] = (wm * 64 + l32) * 128 + (((2 * b + g) ^ (l32 & 7)) * 16);
+#pragma unroll
+  for (int jj = 0; jj < 2; ++jj) ow[jj] = G3_WQ + (wn * 64 + l32) * 64 + (((2 * jj + g) ^ ((l32 >> 1) & 3)) * 16);
+
+  v16f res[2][2];
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int ns = 0; ns < 2; ++ns)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) res[ms][ns][i] = 0.0f;
+
+  const int steps = 2 * (s_end - s_begin);
+  G3ScaleRegs sr;
+  if (steps > 0) {
+    dma_step(0, 0);
+    load_scales(sr, 0);
+    store_scales(sr, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the stage has landed
+  }
+  __syncthreads();
+
+  for (int st = 0; st < steps; ++st) {
+    const uint8_t* Sb = lds + (st & 1) * G3_STAGE;
+    const bool next = st + 1 < steps;
+    if (next) {  // the other stage is free: every wave has passed the barrier that ended the step reading it
+      dma_step(st + 1, (st + 1) & 1);
+      load_scales(sr, st + 1);
+    }
+
+    v4i a16[2], w16[2], wraw[2];
+    float saop[2], wsop, uop[2], vop[2];
+    v32f P[2];
+    v16i I[2];
+    auto ld_a = [&](int b, int ms) { a16[ms] = *(const v4i*)(Sb + oa[b] + ms * 32 * 128); };
+    auto ld_wraw = [&](int jj, int ns) { wraw[ns] = *(const v4i*)(Sb + ow[jj] + ns * 32 * 64); };
+    auto dec_w = [&](int b, int ns) {  // block b of the step: low nibbles of its pair's bytes if even, high if odd
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        w16[ns][i] = (b & 1) ? (int)(((uint32_t)wraw[ns][i] >> 4) & 0x0F0F0F0Fu) : (int)((uint32_t)wraw[ns][i] & 0x0F0F0F0Fu);
+    };
+    auto ld_sa = [&](int b, int ms) { saop[ms] = ((const float*)(Sb + G3_SA))[b * 128 + wm * 64 + ms * 32 + l32]; };
+    auto ld_ws = [&](int b) { wsop = ((const float*)(Sb + G3_WS))[b * 128 + wn * 64 + lane]; };
+    auto mfma_p = [&](int ms) {
+      v32f zf;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+      P[ms] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[ms], wsop, zf, 0, 0, 0);
+    };
+    auto mfma_i = [&](int ms, int ns, int slot) {
+      v16i z;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] = 0;
+      I[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[ms], w16[ns], z, 0, 0, 0);
+    };
+    ld_wraw(0, 0); ld_wraw(0, 1); ld_a(0, 0); ld_a(0, 1); ld_sa(0, 0); ld_sa(0, 1); ld_ws(0);
+    dec_w(0, 0); dec_w(0, 1);
+    mfma_p(0);
+    mfma_i(0, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const bool more = b + 1 < 4;
+      if ((b & 1) == 0) {  // min term of blocks b and b + 1: lane half g supplies block b + g
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) uop[ms] = ((const float*)(Sb + G3_U))[(b + g) * 128 + wm * 64 + ms * 32 + l32];
+#pragma unroll
+        for (int ns = 0; ns < 2; ++ns) vop[ns] = ((const float*)(Sb + G3_V))[(b + g) * 128 + wn * 64 + ns * 32 + l32];
+      }
+#pragma unroll
+      for (int tile = 0; tile < 4; ++tile) {
+        const int ms = tile >> 1, ns = tile & 1, slot = tile & 1;
+        if (tile == 0) {
+          mfma_i(0, 1, 1);
+          if (b == 1) { ld_wraw(1, 0); ld_wraw(1, 1); }  // (both nibble blocks of the first pair are in w16 by now)
+        }
+        if (tile == 1) {
+          mfma_p(1);
+          mfma_i(1, 0, 0);
+          if (more) { ld_a(b + 1, 0); ld_sa(b + 1, 0); }
+        }
+        if (tile == 2) {
+          mfma_i(1, 1, 1);
+          if (more) { dec_w(b + 1, 0); ld_ws(b + 1); }
+        }
+        if (tile == 3 && more) {
+          dec_w(b + 1, 1);
+          mfma_p(0);
+          mfma_i(0, 0, 0);
+          ld_a(b + 1, 1); ld_sa(b + 1, 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          res[ms][ns][i] = __builtin_fmaf((float)I[slot][i], P[ms][16 * ns + i], res[ms][ns][i]);
+        if ((b & 1) == 0) res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop[ns], res[ms][ns], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if (next) {
+      store_scales(sr, st + 1, (st + 1) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = weight row n, accumulator i = token row 8 * (i / 4) + 4 * g + i % 4
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int ns = 0; ns < 2; ++ns) {
+      const int n = n0 + wn * 64 + ns * 32 + l32;
+      if (n >= N) continue;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = wm * 64 + ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+        if (r >= rows_valid) continue;
+        float v = res[ms][ns][i];
+        if (TILES && use_scale) v *= rowscale[m0 + r];
+        float* cp = C + (size_t)(m0 + r) * ldc + c_off + n;
+        if (accumulate == 1) {
+          v += *cp;
+        } else if (accumulate == 2) {
+          const float gt = *cp;
+          v *= gt / (1.0f + __expf(-gt));
+        }
+        *cp = v;
+      }
+    }
+}
+
 // Tile of work-group `id` out of mt x nt tiles.  XCDs take work-groups in turn (id % 8), each running 64 at a time:
 // those 64 are made an 8 x 8 block of tiles when both tile counts are multiples of 8, token tiles fastest otherwise.
 __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
@@ -320,8 +565,18 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
   }
 
 GEMM2_INST(8)
-GEMM2_INST(12)
 GEMM2_TILES_INST(8)
+
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  gemm3_body<false>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                    min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
+}
 GEMM2_TILES_INST(12)
 
 // Q6_K (an int8 sub-scale per 16 values: two K = 16 products per block) runs the plain kernel under the main name.
