@@ -235,7 +235,8 @@ class Engine {
     static const int sk_sb = getenv("ARCZ_GEMM_SPLIT") ? std::max(0, atoi(getenv("ARCZ_GEMM_SPLIT"))) : 0;
     const int nsb = K / 256, splits = a != 2 && sk_sb > 0 ? (nsb + sk_sb - 1) / sk_sb : 1, rgroup = 1;
     cl_mem unused = nullptr;
-    const size_t tiles = (size_t)((Mp + 127) / 128) * ((N + 127) / 128);
+    const int bm = w.type == GGML_Q6_K ? 64 : 128;  // token rows of a work-group's tile
+    const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + 127) / 128);
     size_t gws[1] = {tiles * 256}, lws[1] = {256};
     for (int sp = 0; sp < splits; ++sp) {
       int s0 = nsb * sp / splits, s1 = nsb * (sp + 1) / splits, ac = sp == 0 ? a : 1;
@@ -436,7 +437,7 @@ inline std::string engine_self_check() {
       cl_mem unused = nullptr, C = which ? c1 : c0;
       int MM = M, NN = N, KK = K, ldc = N, zero = 0, one = 1, s1 = K / 256;
       set_args(k, 0, gw.raw, unused, e.aq_, e.asc_, e.absum_, C, MM, NN, KK, ldc, zero, zero, one, zero, s1);
-      size_t gws[1] = {256}, lws[1] = {256};
+      size_t gws[1] = {(size_t)(M / 128) * (N / 128) * 256}, lws[1] = {256};
       e.run("self_check", k, 1, gws, lws);
     }
     CL_CHECK(clEnqueueReadBuffer(e.cl_.queue, c0, CL_TRUE, 0, y0.size() * 4, y0.data(), 0, nullptr, nullptr));

@@ -516,6 +516,218 @@ __device__ inline void gemm3_body(const uint8_t* __restrict__ raw, const signed 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Q6_K, dense.  Same machinery as the Q4_K kernel above (operands straight into double-buffered LDS, weights kept packed
+// and rebuilt when a lane reads its operand, scale tile from an outer-product MFMA), shaped for the format's int8
+// sub-scale per 16 values: a work-group computes 64 tokens x 128 weight rows, wave w all 64 tokens (two 32-row MFMA
+// tiles) of rows [32 w, 32 w + 32), so every weight value is rebuilt by exactly one lane of the work-group.  A lane of
+// the 32x32x32 product supplies the 16 values of sub-block g = lane / 32 of a block; two products with the other
+// sub-block's lanes zeroed give the two sub-block sums I0, I1, and
+//     res += (sa[m][b] * d[n] / 4) * (float)(sc0 * I0 + sc1 * I1)
+// (four ALU instructions per product and block).  The weights enter the product as 4 (q - 32): the six bits of q with
+// bit 5 flipped are q - 32 in six-bit two's complement, and moved to the top of a byte they are that number times 4.
+#define G6_BM 64
+#define G6_STAGE 23040
+#define G6_QL 8192
+#define G6_QH 16384
+#define G6_SA 20480
+#define G6_D 21504
+#define G6_SC 22016
+
+struct G6ScaleRegs {
+  float sa;
+  uint32_t sc;
+  uint32_t d;
+};
+
+__device__ inline void gemm6_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+                                  const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
+                                  int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0) {
+  __shared__ alignas(16) uint8_t lds[2 * G6_STAGE];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8;
+  const PlanesQ6K pl = planes_q6k((size_t)N, nsb);
+  auto token_row = [&](int r) { return m0 + (r < rows_valid ? r : 0); };  // rows past the tile read its first row
+
+  // ---- what this lane fetches each step (a step = half a superblock = 128 values).  Activations: 2 instructions a
+  // wave, 8 rows each, row R = (2 wave + i) 8 + lane / 8 at chunk lane % 8 <- source chunk (lane % 8) ^ (R % 8).  Low
+  // nibbles: 2 instructions, 16 rows each, row R = (2 wave + i) 16 + lane / 4 <- source chunk (lane % 4) ^ ((R / 2) % 4).
+  // High bits: 1 instruction, 32 rows, row R = 32 wave + lane / 2 <- source chunk (lane % 2) ^ ((R / 4) % 2).
+  uint32_t aoff[2], loff[2], hoff;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int R = (wave * 2 + i) * 8 + (lane >> 3);
+    aoff[i] = (uint32_t)token_row(R) * (uint32_t)K + 16u * ((lane & 7) ^ (lane >> 3));
+    const int R2 = (wave * 2 + i) * 16 + (lane >> 2);
+    loff[i] = (uint32_t)min(n0 + R2, N - 1) * (uint32_t)nsb * 128u + 16u * ((lane & 3) ^ ((lane >> 3) & 3));
+  }
+  hoff = (uint32_t)min(n0 + wave * 32 + (lane >> 1), N - 1) * (uint32_t)nsb * 64u + 16u * ((lane & 1) ^ ((lane >> 3) & 1));
+  const signed char* abase = aq + (size_t)s_begin * 256;
+  const uint8_t* lbase = raw + pl.ql + (size_t)s_begin * 128;
+  const uint8_t* hbase = raw + pl.qh + (size_t)s_begin * 64;
+  // scales: threads 0-63 prepare token t (the step's 4 activation scales: one per thread and block -> 4 threads a
+  // token would do; here thread t takes token t % 64, block t / 64); every thread prepares weight row t / 2: the four
+  // sub-scales 4 (t % 2) .. + 3 of the step, and (t % 2 == 0) the row's d.
+  const int r_s = t & 63, b_s = t >> 6;
+  const bool tok_valid = r_s < rows_valid;
+  const uint32_t m_s = (uint32_t)token_row(r_s);
+  const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
+
+  auto dma_step = [&](int st, int stage) {
+    uint8_t* base = lds + stage * G6_STAGE;
+    const signed char* ab = abase + (size_t)st * 128;
+    const uint8_t* lb = lbase + (size_t)st * 64;
+    const uint8_t* hb = hbase + (size_t)st * 32;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) g3_dma16(ab + aoff[i], base + (wave * 2 + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) g3_dma16(lb + loff[i], base + G6_QL + (wave * 2 + i) * 1024);
+    g3_dma16(hb + hoff, base + G6_QH + wave * 1024);
+  };
+  auto load_scales = [&](G6ScaleRegs& r, int st) {
+    const int sb = s_begin + (st >> 1), hh = st & 1;
+    r.sa = (asc + (size_t)(sb * 8 + hh * 4 + b_s) * M)[m_s];
+    r.sc = *(const uint32_t*)(raw + pl.sc + ((size_t)n_s * nsb + sb) * 16 + 8 * hh + 4 * p_s);
+    r.d = *(const unsigned short*)(raw + pl.d + ((size_t)n_s * nsb + sb) * 2);
+  };
+  auto store_scales = [&](const G6ScaleRegs& r, int stage) {
+    uint8_t* base = lds + stage * G6_STAGE;
+    ((float*)(base + G6_SA))[b_s * 64 + r_s] = tok_valid ? r.sa : 0.0f;
+    ((uint32_t*)(base + G6_SC))[(t >> 1) * 2 + p_s] = r.sc;
+    if (p_s == 0) ((float*)(base + G6_D))[t >> 1] = 0.25f * f16_bits_to_f32(r.d);  // (the weights enter as 4 (q - 32))
+  };
+
+  // ---- operand addresses of this lane (bytes from a stage's start)
+  int oa[4], ol[2], oh;
+#pragma unroll
+  for (int b = 0; b < 4; ++b) oa[b] = l32 * 128 + (((2 * b + g) ^ (l32 & 7)) * 16);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) ol[j] = G6_QL + (wave * 32 + l32) * 64 + (((2 * j + g) ^ ((l32 >> 1) & 3)) * 16);
+  oh = G6_QH + (wave * 32 + l32) * 32 + ((g ^ ((l32 >> 2) & 1)) * 16);
+  const uint32_t keep0 = g == 0 ? 0xFFFFFFFFu : 0u, keep1 = ~keep0;
+
+  v16f res[2];
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) res[ms][i] = 0.0f;
+
+  const int steps = 2 * (s_end - s_begin);
+  G6ScaleRegs sr;
+  if (steps > 0) {
+    dma_step(0, 0);
+    load_scales(sr, 0);
+    store_scales(sr, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the stage has landed
+  }
+  __syncthreads();
+
+#pragma unroll 1
+  for (int st = 0; st < steps; ++st) {
+    const uint8_t* Sb = lds + (st & 1) * G6_STAGE;
+    const bool next = st + 1 < steps;
+    if (next) {
+      dma_step(st + 1, (st + 1) & 1);
+      load_scales(sr, st + 1);
+    }
+    // raw weights of the lane's row for the whole step: low nibbles of blocks (0, 2) and (1, 3), high bits of all four
+    const v4i ql0 = *(const v4i*)(Sb + ol[0]), ql1 = *(const v4i*)(Sb + ol[1]), qh = *(const v4i*)(Sb + oh);
+    const uint2 scw = *(const uint2*)(Sb + G6_SC + (wave * 32 + l32) * 8);
+    const float dop = ((const float*)(Sb + G6_D))[wave * 32 + l32];
+    v4i a16[2][2], w0[2], w1[2];  // [buffer][ms]; [buffer]
+    float saop[2];
+    v32f P[2];
+    v16i I0[2], I1[2];
+    auto ld_a = [&](int b, int buf) {
+      a16[buf][0] = *(const v4i*)(Sb + oa[b]);
+      a16[buf][1] = *(const v4i*)(Sb + oa[b] + 32 * 128);
+      saop[buf] = ((const float*)(Sb + G6_SA))[b * 64 + lane];
+    };
+    auto dec_w = [&](int b, int buf) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lw = (uint32_t)((b & 1) ? ql1[i] : ql0[i]), hw = (uint32_t)qh[i];
+        const uint32_t nib = (b >> 1) ? (lw >> 2) & 0x3C3C3C3Cu : (lw << 2) & 0x3C3C3C3Cu;
+        const uint32_t top = b == 3 ? hw & 0xC0C0C0C0u : (hw << (6 - 2 * b)) & 0xC0C0C0C0u;
+        const uint32_t w = (nib | top) ^ 0x80808080u;
+        w0[buf][i] = (int)(w & keep0);
+        w1[buf][i] = (int)(w & keep1);
+      }
+    };
+    auto mfma_p = [&](int buf) {
+      v32f zf;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+      P[buf] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[buf], dop, zf, 0, 0, 0);
+    };
+    auto mfma_i = [&](int buf, int ms, int slot) {
+      v16i z;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] = 0;
+      I0[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[buf][ms], w0[buf], z, 0, 0, 0);
+      I1[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[buf][ms], w1[buf], z, 0, 0, 0);
+    };
+    ld_a(0, 0);
+    dec_w(0, 0);
+    mfma_p(0);
+    mfma_i(0, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int buf = b & 1;
+      const bool more = b + 1 < 4;
+      // int8 sub-scales of block b: bytes 2 b and 2 b + 1 of the step's eight
+      const uint32_t scword = b < 2 ? scw.x : scw.y;
+      const int sc0 = (int)(scword << (24 - 16 * (b & 1))) >> 24, sc1 = (int)(scword << (16 - 16 * (b & 1))) >> 24;
+#pragma unroll
+      for (int ms = 0; ms < 2; ++ms) {
+        const int slot = ms;
+        if (ms == 0) {
+          mfma_i(buf, 1, 1);
+          if (more) { ld_a(b + 1, buf ^ 1); dec_w(b + 1, buf ^ 1); }
+        } else if (more) {
+          mfma_p(buf ^ 1);
+          mfma_i(buf ^ 1, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int j = __mul24(sc0, I0[slot][i]) + __mul24(sc1, I1[slot][i]);
+          res[ms][i] = __builtin_fmaf((float)j, P[buf][16 * ms + i], res[ms][i]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    asm volatile("" : "+v"(res[0]), "+v"(res[1]));  // (the sums are complete before the branches below)
+    if (next) {
+      store_scales(sr, (st + 1) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = weight row n, accumulator i = token row 8 * (i / 4) + 4 * g + i % 4
+  const int n = n0 + wave * 32 + l32;
+  if (n < N) {
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+        if (r >= rows_valid) continue;
+        float v = res[ms][i];
+        float* cp = C + (size_t)(m0 + r) * ldc + c_off + n;
+        if (accumulate == 1) {
+          v += *cp;
+        } else if (accumulate == 2) {
+          const float gt = *cp;
+          v *= gt / (1.0f + __expf(-gt));
+        }
+        *cp = v;
+      }
+  }
+}
+
 // Tile of work-group `id` out of mt x nt tiles.  XCDs take work-groups in turn (id % 8), each running 64 at a time:
 // those 64 are made an 8 x 8 block of tiles when both tile counts are multiples of 8, token tiles fastest otherwise.
 __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
@@ -579,16 +791,16 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321(
 }
 GEMM2_TILES_INST(12)
 
-// Q6_K (an int8 sub-scale per 16 values: two K = 16 products per block) runs the plain kernel under the main name.
-extern "C" __global__ __launch_bounds__(256) void gemm__QTYPE14_ACT321(
+// Q6_K: the dense form has its own body (64-token tiles: grid ceil(N / 128) * ceil(M / 64) work-groups); the form over
+// expert tiles runs the plain kernel.
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
     int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
-  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
   int tm, tn;
   tile_of(blockIdx.x, mt, nt, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  gemm_body<QT_Q6_K, false>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
-                            min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  gemm6_body(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
 }
 extern "C" __global__ __launch_bounds__(256) void gemm__QTYPE14_ACT321_MOE_TILES1(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
