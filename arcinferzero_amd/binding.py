@@ -67,6 +67,8 @@ _sig("arcz_weight_upload", _p, _p, _u32, _i, _i, _p, _z)
 _sig("arcz_weight_free", _i, _p, _p)
 _sig("arcz_weight_raw", _p, _p)
 _sig("arcz_engine_quantize", _i, _p, _p, _i, _i, _i, _i, _i)
+_sig("arcz_engine_rmsnorm_quant", _i, _p, _p, _i, _p, _i, _i, _i, _i, C.c_float, _p)
+_sig("arcz_engine_swiglu_quant", _i, _p, _p, _i, _i, _i, _i, _i, _i)
 _sig("arcz_engine_set_activations", _i, _p, _p, _p, _p, _i, _i, _i)
 _sig("arcz_engine_aq", _p, _p)
 _sig("arcz_engine_asc", _p, _p)
@@ -315,6 +317,13 @@ class Engine:
 
     def quantize(self, x, ldx, K, Mp, T, act32=1):
         _check(lib.arcz_engine_quantize(self.h, x.h, ldx, K, Mp, T, act32), engine=True)
+
+    def rmsnorm_quant(self, x, row_off, w, K, Mp, T, eps, hout=None, act32=1):
+        _check(lib.arcz_engine_rmsnorm_quant(self.h, x.h, row_off, w.h, K, Mp, T, act32, eps, hout.h if hout else None),
+               engine=True)
+
+    def swiglu_quant(self, gu, F, Mp, T, fused=0, gelu=0, act32=1):
+        _check(lib.arcz_engine_swiglu_quant(self.h, gu.h, F, Mp, T, act32, fused, gelu), engine=True)
 
     def set_activations(self, aq, asc, absum, K, Mp, T):
         aq = np.ascontiguousarray(aq, dtype=np.int8)

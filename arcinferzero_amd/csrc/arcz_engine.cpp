@@ -57,6 +57,13 @@ arcz_mem* arcz_weight_raw(const arcz_weight* w) { return w ? w->w.raw : nullptr;
 int arcz_engine_quantize(arcz_engine* e, arcz_mem* x, int ldx, int K, int Mp, int T, int act32) {
   return guarded([&] { e->e->quantize_rows(x, ldx, K, Mp, T, act32); });
 }
+int arcz_engine_rmsnorm_quant(arcz_engine* e, arcz_mem* x, int row_off, arcz_mem* w, int K, int Mp, int T, int act32,
+                              float eps, arcz_mem* hout) {
+  return guarded([&] { e->e->rmsnorm_quant(x, row_off, w, K, Mp, T, act32, eps, hout); });
+}
+int arcz_engine_swiglu_quant(arcz_engine* e, arcz_mem* gu, int F, int Mp, int T, int act32, int fused, int gelu) {
+  return guarded([&] { e->e->swiglu_quant(gu, F, Mp, T, act32, fused, gelu); });
+}
 int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp,
                                 int T) {
   return guarded([&] { e->e->set_activations(aq, asc, absum, K, Mp, T); });

@@ -138,6 +138,42 @@ class Engine {
     run("quant_rows", k, 2, gws, lws);
     cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
   }
+  // The fused producers of the reference (rmsnorm_quant, zero/engine.h:1256-1267; swiglu_quant via run_rows_quant,
+  // zero/engine.h:1404-1440): a work-group per row of the chunk, or -- a pass of 1-8 tokens -- the valid rows only,
+  // their superblocks over several work-groups (the GEMVs read nothing else).
+  static bool wide_rows(int T) { return T <= 8; }
+  void rmsnorm_quant(cl_mem x, int row_off, cl_mem w, int K, int Mp, int T, int act32, float eps, cl_mem hout = nullptr) {
+    check_chunk(K, Mp, T);
+    if (!act32) throw std::runtime_error("rmsnorm_quant: the matmul kernels take per-32 activation scales (act32)");
+    if (row_off < 0 || arcz_mem_size(x) < (size_t)(row_off + T) * K * 4 || arcz_mem_size(w) < (size_t)K * 4 ||
+        (hout && arcz_mem_size(hout) < (size_t)Mp * K * 4))
+      throw std::runtime_error("rmsnorm_quant: a buffer is too small for " + std::to_string(T) + " rows of " + std::to_string(K));
+    cl_kernel k = kernel("ops", "", "rmsnorm_quant");
+    int wh = hout ? 1 : 0;
+    set_args(k, 0, x, row_off, w, K, Mp, T, eps, aq_, asc_, absum_, hout, wh, act32);
+    size_t gws[2] = {256, (size_t)Mp}, lws[2] = {256, 1};
+    if (wide_rows(T)) {
+      gws[0] = 256 * (size_t)((K / 256 + 15) / 16);
+      gws[1] = (size_t)T;
+    }
+    run("rmsnorm_quant", k, 2, gws, lws);
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
+  }
+  // gu: rows [gate(F) | up(F)] f32, or rows of F values when the matmul before has fused the product
+  void swiglu_quant(cl_mem gu, int F, int Mp, int T, int act32, int fused, int gelu) {
+    check_chunk(F, Mp, T);
+    if (!act32) throw std::runtime_error("swiglu_quant: the matmul kernels take per-32 activation scales (act32)");
+    if (arcz_mem_size(gu) < (size_t)T * F * (fused ? 1 : 2) * 4) throw std::runtime_error("swiglu_quant: gu is too small");
+    cl_kernel k = kernel("ops", "", "swiglu_quant");
+    set_args(k, 0, gu, F, Mp, T, aq_, asc_, absum_, act32, fused, gelu);
+    size_t gws[2] = {256, (size_t)Mp}, lws[2] = {256, 1};
+    if (wide_rows(T)) {
+      gws[0] = 256 * (size_t)((F / 256 + 15) / 16);
+      gws[1] = (size_t)T;
+    }
+    run("swiglu_quant", k, 2, gws, lws);
+    cur_T_ = T; cur_K_ = F; cur_Mp_ = Mp;
+  }
   // Activations quantized elsewhere (the reference's benches quantize on the host, bench/gemv_bench.cpp:103-129).
   void set_activations(const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp, int T) {
     check_chunk(K, Mp, T);

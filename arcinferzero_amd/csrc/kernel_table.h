@@ -22,6 +22,8 @@ struct KernelSpec {
 static const KernelSpec kKernelTable[] = {
     // ---- ops
     {"ops", "quant_rows", nullptr, "piiiipppi", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},

@@ -76,6 +76,124 @@ extern "C" __global__ __launch_bounds__(256) void quant_rows(const float* __rest
   store_tile_scales(lds, s, m0, M, act32, asc, absum);
 }
 
+// ---- the two fused producers.  A work-group of 256 threads per row (or several along x, each taking a share of the
+// row's superblocks: the launch for a pass of 1-8 tokens, zero/engine.h:1404-1412); 16 threads per superblock, thread
+// = 16 consecutive values, so a wave works on 4 superblocks at a time.  Scales and sums are stored straight into the
+// token-minor layouts (one element per block and row).
+__device__ inline void store_row_quant(const float* v, int s, int lane16, int m, int M, int K, int act32,
+                                       signed char* __restrict__ aq, float* __restrict__ asc, short* __restrict__ absum) {
+  const float amax = block_amax(v, act32);
+  uint4 pk;
+  int sum;
+  quant16(v, amax, pk, sum);
+  *(uint4*)(aq + (size_t)m * K + s * 256 + 16 * lane16) = pk;
+  absum[((size_t)s * 16 + lane16) * M + m] = (short)sum;
+  if (act32) {
+    if ((lane16 & 1) == 0) asc[((size_t)s * 8 + (lane16 >> 1)) * M + m] = amax / 127.0f;
+  } else if (lane16 == 0) {
+    asc[(size_t)s * M + m] = amax / 127.0f;
+  }
+}
+
+// Sum over the work-group, the same value in every thread, in a fixed order (so every work-group that sums the same
+// row gets the same bits).
+__device__ inline float group_sum(float v, float* red) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float r = (red[0] + red[1]) + (red[2] + red[3]);
+  __syncthreads();
+  return r;
+}
+
+// rmsnorm_quant: y = x[row_off + m] * rsqrt(mean(x^2) + eps) * w, quantized for the next matmul, rows m >= M_valid as
+// zeros; with write_h also stored as f32 in hout [M][K] (reference zero/kernels/ops.cl:107-141, same arguments).
+// grid (256 * G, rows), local (256, 1).
+extern "C" __global__ __launch_bounds__(256) void rmsnorm_quant(const float* __restrict__ x, int row_off,
+                                                                const float* __restrict__ w, int K, int M, int M_valid,
+                                                                float eps, signed char* __restrict__ aq,
+                                                                float* __restrict__ asc, short* __restrict__ absum,
+                                                                float* __restrict__ hout, int write_h, int act32) {
+  __shared__ float red[4];
+  const int m = blockIdx.y;
+  const bool valid = m < M_valid;
+  const float* xr = x + (size_t)(m + row_off) * K;
+  float ss = 0.0f;
+  if (valid)
+    for (int i = threadIdx.x * 4; i < K; i += 1024) {
+      const float4 f = *(const float4*)(xr + i);
+      ss += f.x * f.x;
+      ss += f.y * f.y;
+      ss += f.z * f.z;
+      ss += f.w * f.w;
+    }
+  ss = group_sum(ss, red);
+  const float r = rsqrtf(ss / (float)K + eps);
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
+  for (int s = blockIdx.x * 16 + sub; s < K / 256; s += 16 * gridDim.x) {
+    const int base = s * 256 + 16 * lane16;
+    float v[16];
+    if (valid) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 f = *(const float4*)(xr + base + 4 * i), g = *(const float4*)(w + base + 4 * i);
+        v[4 * i] = f.x * r * g.x; v[4 * i + 1] = f.y * r * g.y; v[4 * i + 2] = f.z * r * g.z; v[4 * i + 3] = f.w * r * g.w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) v[i] = 0.0f;
+    }
+    if (write_h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        *(float4*)(hout + (size_t)m * K + base + 4 * i) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+    store_row_quant(v, s, lane16, m, M, K, act32, aq, asc, absum);
+  }
+}
+
+// swiglu_quant: y = silu(gate) * up (or the tanh form of gelu(gate) * up) from rows [gate(F) | up(F)], or the row as it
+// is when the matmul before has fused the product (`fused`), quantized with K = F (reference zero/kernels/ops.cl:
+// 271-315, same arguments; silu(x) = x / (1 + exp(-x)), ops.cl:33).  grid (256 * G, rows), local (256, 1).
+extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __restrict__ gu, int F, int M, int M_valid,
+                                                               signed char* __restrict__ aq, float* __restrict__ asc,
+                                                               short* __restrict__ absum, int act32, int fused,
+                                                               int gelu) {
+  const int m = blockIdx.y;
+  const bool valid = m < M_valid;
+  const float* gr = gu + (size_t)m * (fused ? F : 2 * F);
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
+  for (int s = blockIdx.x * 16 + sub; s < F / 256; s += 16 * gridDim.x) {
+    const int base = s * 256 + 16 * lane16;
+    float v[16];
+    if (!valid) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) v[i] = 0.0f;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 g = *(const float4*)(gr + base + 4 * i);
+        v[4 * i] = g.x; v[4 * i + 1] = g.y; v[4 * i + 2] = g.z; v[4 * i + 3] = g.w;
+      }
+      if (!fused) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float4 u = *(const float4*)(gr + F + base + 4 * i);
+          const float uv[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float g = v[4 * i + j];
+            const float a = gelu ? 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)))
+                                 : g / (1.0f + expf(-g));
+            v[4 * i + j] = a * uv[j];
+          }
+        }
+      }
+    }
+    store_row_quant(v, s, lane16, m, M, F, act32, aq, asc, absum);
+  }
+}
+
 // fill32: p[i] = v for i < n (the fill used where a captured graph must not hold a memset node).
 extern "C" __global__ void fill32(uint32_t* p, uint32_t v, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -37,6 +37,14 @@ arcz_mem* arcz_weight_raw(const arcz_weight* w);
  * zero/engine.h:1256-1267): rows [0, T) of x (f32, row stride ldx) -> the engine's aq / asc / absum laid out for
  * Mp rows; rows [T, Mp) are zero.  The next matmul takes its form from T: 1 GEMV, 2..8 multi-token GEMV, else GEMM. */
 int arcz_engine_quantize(arcz_engine* e, arcz_mem* x, int ldx, int K, int Mp, int T, int act32);
+/* The fused producers (Engine::rmsnorm_quant, zero/engine.h:1256-1267, kernel zero/kernels/ops.cl:107-141; swiglu_quant,
+ * zero/kernels/ops.cl:271-315 launched by run_rows_quant, zero/engine.h:1404-1440): rows [row_off, row_off + T) of x
+ * through RMS norm with weight w (eps), or rows [gate(F) | up(F)] of gu through silu(gate) * up (gelu: the tanh form of
+ * GELU; fused: rows of F finished values), quantized into the engine's activation buffers for Mp rows; they set the
+ * form of the next matmul like arcz_engine_quantize.  hout (may be NULL): the normalized rows as f32, [Mp][K]. */
+int arcz_engine_rmsnorm_quant(arcz_engine* e, arcz_mem* x, int row_off, arcz_mem* w, int K, int Mp, int T, int act32,
+                              float eps, arcz_mem* hout);
+int arcz_engine_swiglu_quant(arcz_engine* e, arcz_mem* gu, int F, int Mp, int T, int act32, int fused, int gelu);
 /* Activations quantized by the caller, as the reference's benches do (bench/gemv_bench.cpp:103-129). */
 int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp,
                                 int T);
