@@ -64,6 +64,22 @@ _sig("arcz_engine_error", C.c_char_p)
 _sig("arcz_engine_create", _p, _i, _i)
 _sig("arcz_engine_destroy", None, _p)
 _sig("arcz_weight_upload", _p, _p, _u32, _i, _i, _p, _z)
+_sig("arcz_weight_upload_gguf", _p, _p, _p, C.c_char_p)
+_sig("arcz_moe_layer_upload_gguf", _p, _p, _p, C.c_char_p, C.c_char_p, C.c_char_p, _i)
+_sig("arcz_gguf_open", _p, C.c_char_p)
+_sig("arcz_gguf_close", None, _p)
+_sig("arcz_gguf_error", C.c_char_p)
+_sig("arcz_gguf_version", _u32, _p)
+_sig("arcz_gguf_n_kv", _z, _p)
+_sig("arcz_gguf_n_tensors", _z, _p)
+_sig("arcz_gguf_alignment", _u64, _p)
+_sig("arcz_gguf_kv_i64", _i, _p, C.c_char_p, C.POINTER(C.c_int64))
+_sig("arcz_gguf_kv_f64", _i, _p, C.c_char_p, C.POINTER(C.c_double))
+_sig("arcz_gguf_kv_str", C.c_char_p, _p, C.c_char_p)
+_sig("arcz_gguf_tensor", _i, _p, _z, C.POINTER(C.c_char_p), C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u64 * 8),
+     C.POINTER(_p), C.POINTER(_u64))
+_sig("arcz_gguf_find", C.c_long, _p, C.c_char_p)
+_sig("arcz_ggml_block_info", _i, _u32, C.POINTER(_i), C.POINTER(_i))
 _sig("arcz_weight_free", _i, _p, _p)
 _sig("arcz_weight_raw", _p, _p)
 _sig("arcz_engine_quantize", _i, _p, _p, _i, _i, _i, _i, _i)
@@ -107,6 +123,67 @@ def self_check():
     """Tuned GEMM against the simple GEMM and integer sums on LCG data (zero/engine_setup.h:424-520); raises on a
     difference."""
     _check(lib.arcz_engine_self_check(), engine=True)
+
+
+# ---------------------------------------------------------------- GGUF files (no GPU)
+class GgufFile:
+    """A memory-mapped GGUF file: metadata scalars and strings, the tensor directory, tensor bytes as numpy views."""
+
+    def __init__(self, path):
+        self.h = lib.arcz_gguf_open(str(path).encode())
+        if not self.h:
+            raise ArczError(-100, lib.arcz_gguf_error().decode())
+
+    def close(self):
+        if self.h:
+            lib.arcz_gguf_close(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    @property
+    def version(self):
+        return lib.arcz_gguf_version(self.h)
+
+    @property
+    def n_kv(self):
+        return lib.arcz_gguf_n_kv(self.h)
+
+    @property
+    def n_tensors(self):
+        return lib.arcz_gguf_n_tensors(self.h)
+
+    @property
+    def alignment(self):
+        return lib.arcz_gguf_alignment(self.h)
+
+    def get_int(self, key, default=None):
+        v = C.c_int64()
+        return v.value if lib.arcz_gguf_kv_i64(self.h, key.encode(), C.byref(v)) else default
+
+    def get_float(self, key, default=None):
+        v = C.c_double()
+        return v.value if lib.arcz_gguf_kv_f64(self.h, key.encode(), C.byref(v)) else default
+
+    def get_str(self, key, default=None):
+        s = lib.arcz_gguf_kv_str(self.h, key.encode())
+        return s.decode() if s is not None else default
+
+    def find(self, name):
+        return lib.arcz_gguf_find(self.h, name.encode())
+
+    def tensor(self, i):
+        name, typ, nd, dims, data, nb = C.c_char_p(), _u32(), _u32(), (_u64 * 8)(), _p(), _u64()
+        if lib.arcz_gguf_tensor(self.h, i, C.byref(name), C.byref(typ), C.byref(nd), C.byref(dims), C.byref(data),
+                                C.byref(nb)) != 0:
+            raise IndexError(i)
+        buf = (C.c_uint8 * nb.value).from_address(data.value) if nb.value else None
+        return {"name": name.value.decode(), "type": typ.value, "dims": [int(dims[k]) for k in range(nd.value)],
+                "nbytes": nb.value, "data": np.frombuffer(buf, np.uint8) if buf is not None else np.zeros(0, np.uint8)}
 
 
 # ---------------------------------------------------------------- host helpers (no GPU)
@@ -314,6 +391,21 @@ class Engine:
         if not h:
             raise ArczError(-100, lib.arcz_engine_error().decode())
         return Weight(self, h, qtype, N, K)
+
+    def make_weight_gguf(self, gguf, name):
+        """A matrix of an open GgufFile, by name, as it lies in the file."""
+        h = lib.arcz_weight_upload_gguf(self.h, gguf.h, name.encode())
+        if not h:
+            raise ArczError(-100, lib.arcz_engine_error().decode())
+        t = gguf.tensor(gguf.find(name))
+        return Weight(self, h, t["type"], t["dims"][1], t["dims"][0])
+
+    def make_moe_layer_gguf(self, gguf, gate, up, down, NU):
+        h = lib.arcz_moe_layer_upload_gguf(self.h, gguf.h, gate.encode(), up.encode(), down.encode(), NU)
+        if not h:
+            raise ArczError(-100, lib.arcz_engine_error().decode())
+        t = gguf.tensor(gguf.find(gate))
+        return MoeLayer(self, h, t["dims"][2], NU, t["dims"][0], t["dims"][1])
 
     def quantize(self, x, ldx, K, Mp, T, act32=1):
         _check(lib.arcz_engine_quantize(self.h, x.h, ldx, K, Mp, T, act32), engine=True)

@@ -1,5 +1,6 @@
 // C ABI of include/arcz_engine.h over the Engine class (engine_hip.h).
 #include "../../include/arcz_engine.h"
+#include "../../include/arcz_gguf.h"
 
 #include <string>
 
@@ -46,6 +47,57 @@ arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, con
   }
   return w;
 }
+// Engine::make_weight from a tensor of a GGUF file (zero/engine_load.h:157-196): a matrix [N][K] (dims K, N) or an expert
+// tensor [NE][N][K] (dims K, N, NE), taken as it lies in the file.
+static GpuWeight weight_from_gguf(Engine& E, const arcz_gguf* g, const char* name, int* ne_out) {
+  const long i = arcz_gguf_find(g, name);
+  if (i < 0) throw std::runtime_error(std::string("missing tensor ") + name);
+  uint32_t type = 0, nd = 0;
+  uint64_t dims[8], nbytes = 0;
+  const void* data = nullptr;
+  arcz_gguf_tensor(g, (size_t)i, nullptr, &type, &nd, dims, &data, &nbytes);
+  if (nd < 2 || nd > 3 || dims[0] > (1u << 30) || dims[1] > (1u << 30) || (nd == 3 && dims[2] > 65536))
+    throw std::runtime_error(std::string("tensor ") + name + " is no matrix or expert tensor");
+  const int K = (int)dims[0], N = (int)dims[1], NE = nd == 3 ? (int)dims[2] : 1;
+  if (ne_out) *ne_out = NE;
+  return E.make_weight(type, (const uint8_t*)data, (size_t)nbytes, N, K, (size_t)NE * N);
+}
+arcz_weight* arcz_weight_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* name) {
+  arcz_weight* w = new arcz_weight();
+  if (guarded([&] { w->w = weight_from_gguf(*e->e, g, name, nullptr); }) != ARCZ_OK) {
+    delete w;
+    return nullptr;
+  }
+  return w;
+}
+arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* gate, const char* up,
+                                           const char* down, int NU) {
+  arcz_moe_layer* L = new arcz_moe_layer();
+  if (guarded([&] {
+        int ne[3];
+        Engine& E = *e->e;
+        // the geometry first (the layer's buffers are sized from it), then the three tensors
+        const long ig = arcz_gguf_find(g, gate);
+        if (ig < 0) throw std::runtime_error(std::string("missing tensor ") + gate);
+        uint32_t nd = 0;
+        uint64_t dims[8];
+        arcz_gguf_tensor(g, (size_t)ig, nullptr, nullptr, &nd, dims, nullptr, nullptr);
+        if (nd != 3) throw std::runtime_error(std::string("tensor ") + gate + " is no expert tensor");
+        const int Ed = (int)dims[0], F = (int)dims[1], NE = (int)dims[2];
+        E.moe_alloc(NE, NU, Ed, F);
+        L->L.NE = NE; L->L.NU = NU; L->L.E = Ed; L->L.F = F;
+        L->L.ex[0] = weight_from_gguf(E, g, gate, &ne[0]);
+        L->L.ex[1] = weight_from_gguf(E, g, up, &ne[1]);
+        L->L.ex[2] = weight_from_gguf(E, g, down, &ne[2]);
+        if (ne[1] != NE || ne[2] != NE || L->L.ex[1].N != F || L->L.ex[1].K != Ed || L->L.ex[2].N != Ed || L->L.ex[2].K != F)
+          throw std::runtime_error("the expert tensors' shapes do not belong to one layer");
+      }) != ARCZ_OK) {
+    delete L;
+    return nullptr;
+  }
+  return L;
+}
+
 int arcz_weight_free(arcz_engine* e, arcz_weight* w) {
   if (!w) return ARCZ_OK;
   const int r = guarded([&] { e->e->free_weight(w->w); });

@@ -10,6 +10,7 @@
 #ifndef ARCZ_ENGINE_H
 #define ARCZ_ENGINE_H
 #include "arcz_hip.h"
+#include "arcz_gguf.h"
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -30,6 +31,12 @@ void arcz_engine_destroy(arcz_engine* e);
 /* make_weight + upload_padded (zero/engine_load.h:84-130, 157-196): N rows of K values as GGUF blocks of `type`
  * (8 = Q8_0, 12 = Q4_K, 14 = Q6_K), regrouped into the device layout and uploaded. */
 arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, const void* gguf, size_t bytes);
+/* The same from a tensor of an open GGUF file (upload of zero/engine_load.h:84-196): a matrix (dims K, N) or an expert
+ * tensor (dims K, N, experts) of type Q8_0 / Q4_K / Q6_K, by name; NULL + arcz_engine_error() when it is missing, of
+ * another type or shape.  The MoE layer: its three expert tensors (gate and up [NE][F][E], down [NE][E][F]). */
+arcz_weight* arcz_weight_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* name);
+arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* gate, const char* up,
+                                           const char* down, int NU);
 int arcz_weight_free(arcz_engine* e, arcz_weight* w);
 arcz_mem* arcz_weight_raw(const arcz_weight* w);
 
