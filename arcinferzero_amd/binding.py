@@ -372,7 +372,7 @@ class MoeLayer:
 class Engine:
     """The matmul dispatch of the reference's Engine for one GPU (zero/engine.h:936-1251, zero/engine_moe.h)."""
 
-    MOE_BUFFERS = ("ids", "wts", "offs", "tiles", "tstart", "stok", "swt", "inv", "h", "hq", "hsc", "y")
+    MOE_BUFFERS = ("ids", "wts", "offs", "tiles", "tstart", "stok", "swt", "inv", "h", "hq", "hsc", "y", "hbs")
 
     def __init__(self, max_chunk, max_k):
         self.h = lib.arcz_engine_create(max_chunk, max_k)

@@ -151,8 +151,9 @@ int arcz_engine_moe_route(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, i
 }
 arcz_mem* arcz_engine_moe_buffer(arcz_engine* e, int which) {
   Engine& E = *e->e;
-  cl_mem b[12] = {E.mids_, E.mwts_, E.moffs_, E.mtiles_, E.mtstart_, E.stok_, E.swt_, E.minv_, E.mh_, E.mhq_, E.mhsc_, E.my_};
-  return which >= 0 && which < 12 ? b[which] : nullptr;
+  cl_mem b[13] = {E.mids_, E.mwts_, E.moffs_, E.mtiles_, E.mtstart_, E.stok_, E.swt_, E.minv_, E.mh_, E.mhq_, E.mhsc_, E.my_,
+                  E.mhbs_};
+  return which >= 0 && which < 13 ? b[which] : nullptr;
 }
 int arcz_engine_moe_slots(arcz_engine* e) { return e->e->slots_; }
 

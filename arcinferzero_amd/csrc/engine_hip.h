@@ -295,7 +295,7 @@ class Engine {
   // buffers of the layer (zero/engine_alloc.h:109-159): sized for max_chunk tokens
   cl_mem mids_ = nullptr, mwts_ = nullptr, sgate_ = nullptr, mcount_ = nullptr, moffs_ = nullptr, mcursor_ = nullptr,
          mtiles_ = nullptr, mtstart_ = nullptr, stok_ = nullptr, swt_ = nullptr, minv_ = nullptr, mh_ = nullptr,
-         mhq_ = nullptr, mhsc_ = nullptr, my_ = nullptr;
+         mhq_ = nullptr, mhsc_ = nullptr, mhbs_ = nullptr, my_ = nullptr;
   int slots_ = 0, moe_ne_ = 0, moe_nu_ = 0, moe_e_ = 0, moe_f_ = 0;
 
   void moe_alloc(int NE, int NU, int E, int F) {
@@ -310,7 +310,7 @@ class Engine {
     mcount_ = buf((size_t)NE * 4); moffs_ = buf((size_t)NE * 4); mcursor_ = buf((size_t)NE * 4);
     mtiles_ = buf((1 + 3 * (S + NE)) * 4); mtstart_ = buf((size_t)(NE + 1) * 4);
     stok_ = buf(S * 4); swt_ = buf(S * 4); minv_ = buf(S * 4);
-    mh_ = buf(S * F * 4); mhq_ = buf(S * F); mhsc_ = buf(S * (F / 32) * 4); my_ = buf(S * E * 4);
+    mh_ = buf(S * F * 4); mhq_ = buf(S * F); mhsc_ = buf(S * (F / 32) * 4); mhbs_ = buf(S * (F / 16) * 2); my_ = buf(S * E * 4);
     const uint32_t zero = 0;
     CL_CHECK(clEnqueueFillBuffer(cl_.queue, mcount_, &zero, 4, 0, (size_t)NE * 4, 0, nullptr, nullptr));
   }
@@ -366,7 +366,7 @@ class Engine {
       int M = i == 2 ? slots_ : Mp, NN = N, KK = K, ldc = N, acc = i == 1 ? 2 : 0, e0 = 0, e1 = NE, um = i == 2 ? 0 : 1,
           us = i == 2 ? 1 : 0;
       cl_mem unused = nullptr;
-      set_args(k, 0, L.ex[i].raw, unused, i == 2 ? mhq_ : aq_, i == 2 ? mhsc_ : asc_, absum_, i == 2 ? my_ : mh_, M, NN, KK,
+      set_args(k, 0, L.ex[i].raw, unused, i == 2 ? mhq_ : aq_, i == 2 ? mhsc_ : asc_, i == 2 ? mhbs_ : absum_, i == 2 ? my_ : mh_, M, NN, KK,
                ldc, acc, mtiles_, mtstart_, e0, e1, stok_, um, swt_, us);
       size_t gws[2] = {(size_t)(N + 127) / 128 * 256, max_tiles}, lws[2] = {256, 1};
       run(i == 2 ? "moe_down" : "moe_gateup", k, 2, gws, lws);
@@ -379,15 +379,17 @@ class Engine {
     const int E = L.E, F = L.F, NU = L.NU, n = T * NU;
     if (cur_T_ != T || cur_K_ != E || cur_Mp_ != Mp) throw std::runtime_error("layer_moe: the activations are not this chunk's");
     if (arcz_mem_size(x) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: x is too small");
-    const int tm = 128;  // slots per tile: the token rows of one work-group of the tile GEMM
+    // slots per tile = the token rows of one work-group of the tile GEMM: 64 for Q4_K experts, 128 for the others
+    const int tm = L.ex[0].type == GGML_Q4_K ? 64 : 128;
     moe_route(L, rl, ldl, T, tm);
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)
     const size_t max_tiles = (size_t)(n + tm - 1) / tm + std::min(n, L.NE);
     moe_gemm(L, 0, Mp, max_tiles);
     {
-      cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_quant");
+      // (the reference's moe_quant writes no sums; the Q4_K tile GEMM here takes them for its min term)
+      cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_quant_sums");
       int FF = F, S = slots_;
-      set_args(k, 0, mh_, FF, S, mhq_, mhsc_);
+      set_args(k, 0, mh_, FF, S, mhq_, mhsc_, mhbs_);
       size_t gws[2] = {(size_t)256 * (F / 256), (size_t)(n + 63) / 64}, lws[2] = {256, 1};
       run("moe_quant", k, 2, gws, lws);
     }

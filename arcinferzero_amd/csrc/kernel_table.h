@@ -47,5 +47,6 @@ static const KernelSpec kKernelTable[] = {
     {"moe", "moe_scan", nullptr, "ppppp", {nullptr}, {{"NE", 0, true}, {"TM", 16, false}, {nullptr, 0, false}}, 1024},
     {"moe", "moe_scatter", nullptr, "ppipppp", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},
     {"moe", "moe_quant", nullptr, "piipp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_quant_sums", nullptr, "piippp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_combine", nullptr, "pppppi", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},
 };

@@ -728,6 +728,212 @@ __device__ inline void gemm6_body(const uint8_t* __restrict__ raw, const signed 
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Q4_K over expert tiles, in the shape of the Q6_K kernel above: 64 slots x 128 weight rows per work-group (tiles of 64
+// fill better than tiles of 128 when an expert has a few hundred slots), wave w all 64 slots of rows [32 w, 32 w + 32)
+// (each packed weight is split into its nibbles by exactly one lane of the work-group), scale tile per block from one
+// outer-product MFMA (lane halves = the two slot tiles), min term of a block pair from one v_mfma_f32_32x32x2_f32 per
+// slot tile into the result accumulators, S from absum.  (For the dense matrix the 128 x 128 kernel above measured
+// faster: half the traffic from L2 per product.)
+#define G4_STAGE 22528
+#define G4_WQ 8192
+#define G4_SA 16384
+#define G4_U 17408
+#define G4_WS 18432
+#define G4_V 20480
+
+struct G4ScaleRegs {
+  float sa;
+  short bs[2];
+  uint4 h;
+};
+
+__device__ inline void gemm4_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+                                  const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
+                                  int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
+                                  size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
+                                  const int* __restrict__ rowmap, int use_map, const float* __restrict__ rowscale,
+                                  int use_scale) {
+  __shared__ alignas(16) uint8_t lds[2 * G4_STAGE];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8;
+  const PlanesQ4K pl = planes_q4k(rows_total, nsb);
+  auto token_row = [&](int r) {  // the token row slot r reads; slots past the tile read its first
+    const int rr = m0 + (r < rows_valid ? r : 0);
+    return use_map ? rowmap[rr] : rr;
+  };
+
+  uint32_t aoff[2], woff[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int R = (wave * 2 + i) * 8 + (lane >> 3);
+    aoff[i] = (uint32_t)token_row(R) * (uint32_t)K + 16u * ((lane & 7) ^ (lane >> 3));
+    const int R2 = (wave * 2 + i) * 16 + (lane >> 2);
+    woff[i] = (uint32_t)min(n0 + R2, N - 1) * (uint32_t)nsb * 128u + 16u * ((lane & 3) ^ ((lane >> 3) & 3));
+  }
+  const signed char* abase = aq + (size_t)s_begin * 256;
+  const uint8_t* wbase = raw + pl.qs + (row_base * nsb + s_begin) * 128;
+  // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t / 2, block pair t % 2
+  const int r_s = t & 63, b_s = t >> 6;
+  const bool tok_valid = r_s < rows_valid;
+  const uint32_t m_s = (uint32_t)token_row(r_s);
+  const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
+
+  auto dma_step = [&](int st, int stage) {
+    uint8_t* base = lds + stage * G4_STAGE;
+    const signed char* ab = abase + (size_t)st * 128;
+    const uint8_t* wb = wbase + (size_t)st * 64;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) g3_dma16(ab + aoff[i], base + (wave * 2 + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[i], base + G4_WQ + (wave * 2 + i) * 1024);
+  };
+  // (loads only: anything computed from them here would make the wave wait for the whole step's traffic)
+  auto load_scales = [&](G4ScaleRegs& r, int st) {
+    const int blk = s_begin * 8 + st * 4 + b_s;
+    r.sa = (asc + (size_t)blk * M)[m_s];
+    r.bs[0] = (absum + (size_t)(2 * blk) * M)[m_s];
+    r.bs[1] = (absum + (size_t)(2 * blk + 1) * M)[m_s];
+    r.h = *(const uint4*)(raw + pl.hdr + ((row_base + n_s) * nsb + s_begin + (st >> 1)) * 16);
+  };
+  auto store_scales = [&](const G4ScaleRegs& r, int st, int stage) {
+    uint8_t* base = lds + stage * G4_STAGE;
+    const float sa = tok_valid ? r.sa : 0.0f;
+    ((float*)(base + G4_SA))[b_s * 64 + r_s] = sa;
+    ((float*)(base + G4_U))[b_s * 64 + r_s] = sa * (float)((int)r.bs[0] + (int)r.bs[1]);
+    const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
+    int sc0, sc1, mn0, mn1;
+    q4k_scales_pair(r.h.y, r.h.z, r.h.w, 2 * (st & 1) + p_s, sc0, sc1, mn0, mn1);
+    const int row = t >> 1;
+    ((float*)(base + G4_WS))[(2 * p_s) * 128 + row] = d * (float)sc0;
+    ((float*)(base + G4_WS))[(2 * p_s + 1) * 128 + row] = d * (float)sc1;
+    ((float*)(base + G4_V))[(2 * p_s) * 128 + row] = -(dmin * (float)mn0);
+    ((float*)(base + G4_V))[(2 * p_s + 1) * 128 + row] = -(dmin * (float)mn1);
+  };
+
+  int oa[4], ow[2];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) oa[b] = l32 * 128 + (((2 * b + g) ^ (l32 & 7)) * 16);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) ow[j] = G4_WQ + (wave * 32 + l32) * 64 + (((2 * j + g) ^ ((l32 >> 1) & 3)) * 16);
+
+  v16f res[2];
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) res[ms][i] = 0.0f;
+
+  const int steps = 2 * (s_end - s_begin);
+  G4ScaleRegs sr;
+  if (steps > 0) {
+    dma_step(0, 0);
+    load_scales(sr, 0);
+    store_scales(sr, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the stage has landed
+  }
+  __syncthreads();
+
+#pragma unroll 1
+  for (int st = 0; st < steps; ++st) {
+    const uint8_t* Sb = lds + (st & 1) * G4_STAGE;
+    const bool next = st + 1 < steps;
+    if (next) {
+      dma_step(st + 1, (st + 1) & 1);
+      load_scales(sr, st + 1);
+    }
+    // packed weights of the lane's row for the whole step: block pairs (0, 1) and (2, 3)
+    const v4i wr0 = *(const v4i*)(Sb + ow[0]), wr1 = *(const v4i*)(Sb + ow[1]);
+    v4i a16[2][2], w16[2];  // [buffer][ms]; [buffer]
+    float saop[2], wsop[2], uop[2], vop;
+    v32f P[2];
+    v16i I[2];
+    auto ld_a = [&](int b, int buf) {
+      a16[buf][0] = *(const v4i*)(Sb + oa[b]);
+      a16[buf][1] = *(const v4i*)(Sb + oa[b] + 32 * 128);
+      saop[buf] = ((const float*)(Sb + G4_SA))[b * 64 + lane];
+      wsop[buf] = ((const float*)(Sb + G4_WS))[b * 128 + wave * 32 + l32];
+    };
+    auto dec_w = [&](int b, int buf) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t x = (uint32_t)((b >> 1) ? wr1[i] : wr0[i]);
+        w16[buf][i] = (int)((b & 1) ? (x >> 4) & 0x0F0F0F0Fu : x & 0x0F0F0F0Fu);
+      }
+    };
+    auto mfma_p = [&](int buf) {
+      v32f zf;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+      P[buf] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[buf], wsop[buf], zf, 0, 0, 0);
+    };
+    auto mfma_i = [&](int buf, int ms, int slot) {
+      v16i z;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] = 0;
+      I[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[buf][ms], w16[buf], z, 0, 0, 0);
+    };
+    ld_a(0, 0);
+    dec_w(0, 0);
+    mfma_p(0);
+    mfma_i(0, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int buf = b & 1;
+      const bool more = b + 1 < 4;
+      if ((b & 1) == 0) {  // min term of blocks b and b + 1: lane half g supplies block b + g
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) uop[ms] = ((const float*)(Sb + G4_U))[(b + g) * 64 + ms * 32 + l32];
+        vop = ((const float*)(Sb + G4_V))[(b + g) * 128 + wave * 32 + l32];
+      }
+#pragma unroll
+      for (int ms = 0; ms < 2; ++ms) {
+        const int slot = ms;
+        if (ms == 0) {
+          mfma_i(buf, 1, 1);
+          if (more) { ld_a(b + 1, buf ^ 1); dec_w(b + 1, buf ^ 1); }
+        } else if (more) {
+          mfma_p(buf ^ 1);
+          mfma_i(buf ^ 1, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) res[ms][i] = __builtin_fmaf((float)I[slot][i], P[buf][16 * ms + i], res[ms][i]);
+        if ((b & 1) == 0) res[ms] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop, res[ms], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    asm volatile("" : "+v"(res[0]), "+v"(res[1]));  // (the sums are complete before the branches below)
+    if (next) {
+      store_scales(sr, st + 1, (st + 1) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = weight row n, accumulator i = token row 8 * (i / 4) + 4 * g + i % 4
+  const int n = n0 + wave * 32 + l32;
+  if (n < N) {
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+        if (r >= rows_valid) continue;
+        float v = res[ms][i];
+        if (use_scale) v *= rowscale[m0 + r];
+        float* cp = C + (size_t)(m0 + r) * ldc + c_off + n;
+        if (accumulate == 1) {
+          v += *cp;
+        } else if (accumulate == 2) {
+          const float gt = *cp;
+          v *= gt / (1.0f + __expf(-gt));
+        }
+        *cp = v;
+      }
+  }
+}
+
 // Tile of work-group `id` out of mt x nt tiles.  XCDs take work-groups in turn (id % 8), each running 64 at a time:
 // those 64 are made an 8 x 8 block of tiles when both tile counts are multiples of 8, token tiles fastest otherwise.
 __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
@@ -789,7 +995,19 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321(
   gemm3_body<false>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
                     min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
 }
-GEMM2_TILES_INST(12)
+// (tiles of at most 64 slots: the engine builds the tile list for that size)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TILES1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
+    int use_map, const float* rowscale, int use_scale, int NE) {
+  const int t_end = tstart[e1];
+  for (int ti = tstart[e0] + blockIdx.y; ti < t_end; ti += gridDim.y) {
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+    gemm4_body(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,
+               min(nr, G6_BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
+    __syncthreads();
+  }
+}
 
 // Q6_K: the dense form has its own body (64-token tiles: grid ceil(N / 128) * ceil(M / 64) work-groups); the form over
 // expert tiles runs the plain kernel.

@@ -181,10 +181,13 @@ extern "C" __global__ __launch_bounds__(256) void moe_scatter(const int* __restr
 // moe_quant: h [S][F] f32 (S slot rows, the first n in use) -> hq [S][F] int8, hsc [F/32][S] f32 with row stride S;
 // no sums (reference zero/kernels/moe.cl:258-274; FV: columns >= FV quantize as zeros).  The grid covers the rows in
 // use in tiles of 64; rows of a tile at or past S are skipped.  grid (F/256, ceil(n/64)), local 256.
-extern "C" __global__ __launch_bounds__(256) void moe_quant(const float* __restrict__ h, int F, int S,
-                                                            signed char* __restrict__ hq, float* __restrict__ hsc,
-                                                            int FV) {
+// moe_quant_sums: the same, and the sums of each 16 quantized values, hbs [F/16][S] int16 (the layout of the dense
+// quantizer's sums), which the Q4_K tile GEMM of the down projection takes for its min term.
+template <bool SUMS>
+__device__ inline void moe_quant_body(const float* __restrict__ h, int F, int S, signed char* __restrict__ hq,
+                                      float* __restrict__ hsc, short* __restrict__ hbs, int FV) {
   __shared__ float lasc[8][64];
+  __shared__ short lsum[16][64];
   const int s = blockIdx.x, m0 = blockIdx.y * 64;
   const int lane16 = threadIdx.x & 15, rg = threadIdx.x >> 4;
 #pragma unroll 1
@@ -212,6 +215,7 @@ extern "C" __global__ __launch_bounds__(256) void moe_quant(const float* __restr
     quant16(v, amax, pk, sum);
     if (m < S) *(uint4*)(hq + (size_t)m * F + base) = pk;
     if ((lane16 & 1) == 0) lasc[lane16 >> 1][r] = amax / 127.0f;
+    if (SUMS) lsum[lane16][r] = (short)sum;
   }
   __syncthreads();
 #pragma unroll
@@ -219,6 +223,23 @@ extern "C" __global__ __launch_bounds__(256) void moe_quant(const float* __restr
     const int idx = threadIdx.x + 256 * i, b = idx >> 6, r = idx & 63;
     if (m0 + r < S) hsc[((size_t)s * 8 + b) * S + m0 + r] = lasc[b][r];
   }
+  if (SUMS) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = threadIdx.x + 256 * i, b = idx >> 6, r = idx & 63;
+      if (m0 + r < S) hbs[((size_t)s * 16 + b) * S + m0 + r] = lsum[b][r];
+    }
+  }
+}
+extern "C" __global__ __launch_bounds__(256) void moe_quant(const float* __restrict__ h, int F, int S,
+                                                            signed char* __restrict__ hq, float* __restrict__ hsc,
+                                                            int FV) {
+  moe_quant_body<false>(h, F, S, hq, hsc, nullptr, FV);
+}
+extern "C" __global__ __launch_bounds__(256) void moe_quant_sums(const float* __restrict__ h, int F, int S,
+                                                                 signed char* __restrict__ hq, float* __restrict__ hsc,
+                                                                 short* __restrict__ hbs, int FV) {
+  moe_quant_body<true>(h, F, S, hq, hsc, hbs, FV);
 }
 
 // moe_combine: x[t][c] += sum over k (in order) of y[inv[t * NU + k]][c]  (+ sgate[t] * sh[t][c] when there is a

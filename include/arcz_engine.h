@@ -72,7 +72,8 @@ arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void*
  * the T tokens whose quantized h is the current activation chunk; logits: router logits [T][ldl] f32. */
 int arcz_engine_layer_moe(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp);
 /* The routing step alone (moe_route + moe_scan + moe_scatter, zero/engine_moe.h:111-133) with tiles of tm slots, and
- * its buffers: which = 0 ids, 1 wts, 2 offs, 3 tiles, 4 tstart, 5 stok, 6 swt, 7 inv, 8 h (f32), 9 hq, 10 hsc, 11 y. */
+ * its buffers: which = 0 ids, 1 wts, 2 offs, 3 tiles, 4 tstart, 5 stok, 6 swt, 7 inv, 8 h (f32), 9 hq, 10 hsc, 11 y,
+ * 12 hbs (int16 sums of each 16 values of hq, [F/16][slots]). */
 int arcz_engine_moe_route(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, int T, int tm);
 arcz_mem* arcz_engine_moe_buffer(arcz_engine* e, int which);
 int arcz_engine_moe_slots(arcz_engine* e);

@@ -109,6 +109,8 @@ def test_moe_layer_vs_oracle(rt, qtype, NE, NU, E, F, T, Mp):
         rq, rsc = orc.moe_quant(h[used])
         assert np.array_equal(hq[used], rq)
         assert np.array_equal(hsc[:, used].view(np.uint32), rsc.view(np.uint32))
+        hbs = eng.moe_buffer("hbs").read(np.int16, (F // 16) * S).reshape(F // 16, S)
+        assert np.array_equal(hbs[:, used].T, rq.astype(np.int32).reshape(len(used), F // 16, 16).sum(axis=2))
         for b in (xb, lb, ob):
             b.free()
     finally:
