@@ -41,10 +41,10 @@ static const KernelSpec kKernelTable[] = {
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
     // ---- moe
-    {"moe", "moe_route", nullptr, "piipppp", {nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_route", nullptr, "piipppp", {nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_route1", nullptr, "pppppp", {nullptr},
      {{"NE", 0, true}, {"NU", 0, true}, {"HAS_GATE", 0, false}, {nullptr, 0, false}}, 64},
-    {"moe", "moe_scan", nullptr, "ppppp", {nullptr}, {{"NE", 0, true}, {"TM", 16, false}, {nullptr, 0, false}}, 1024},
+    {"moe", "moe_scan", nullptr, "ppppp", {nullptr}, {{"NE", 0, true}, {"TM", 16, false}, {"NPART", 1, false}, {nullptr, 0, false}}, 1024},
     {"moe", "moe_scatter", nullptr, "ppipppp", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},
     {"moe", "moe_quant", nullptr, "piipp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_quant_sums", nullptr, "piippp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},

@@ -3,57 +3,66 @@
 // compiles these with -DNE (experts), -DNU (experts per token), -DTM (slots per tile); here they are trailing
 // arguments.
 #include "quant.h"
+#include <type_traits>
 
 #define MAX_PER_LANE 8  // NE <= 512
 
 // moe_route: one wave per token.  The NU largest of NE logits (ties: the lower expert), p = exp(l - max),
-// weights p / sum of the selected p; counts[e]++ per selection; sgate[t] = sigmoid(logit NE) when the row holds one.
+// weights p / sum of the selected p; counts[copy][e]++ per selection (NPART copies [NPART][NE], 1 by default); sgate[t] = sigmoid(logit NE) when the row holds one.
 // grid: ceil(T / 4) work-groups of 256 threads.
 extern "C" __global__ __launch_bounds__(256) void moe_route(const float* __restrict__ logits, int ldl, int T,
                                                             int* __restrict__ ids, float* __restrict__ wts,
                                                             float* __restrict__ sgate, int* __restrict__ counts,
-                                                            int NE, int NU) {
+                                                            int NE, int NU, int NPART) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
   const float* lg = logits + (size_t)t * ldl;
-  float v[MAX_PER_LANE];
-  float mx = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < MAX_PER_LANE; ++i) {
-    const int e = i * 64 + lane;
-    v[i] = e < NE ? lg[e] : -INFINITY;
-    mx = fmaxf(mx, v[i]);
-  }
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
   float sum = 0.0f, myp = 0.0f;
   int mysel = 0;
-  for (int k = 0; k < NU; ++k) {
-    float bv = -INFINITY;
-    int bi = NE;
+  // (PL logits per lane: 2 serve up to 128 experts, the common case; the same steps either way)
+  auto pick = [&](auto pl_tag) {
+    constexpr int PL = decltype(pl_tag)::value;
+    float v[PL];
+    float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < MAX_PER_LANE; ++i)
-      if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
-    // wave arg-max, the lower index among equal values
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-      const float ov = __shfl_xor(bv, d, 64);
-      const int oi = __shfl_xor(bi, d, 64);
-      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    for (int i = 0; i < PL; ++i) {
+      const int e = i * 64 + lane;
+      v[i] = e < NE ? lg[e] : -INFINITY;
+      mx = fmaxf(mx, v[i]);
     }
 #pragma unroll
-    for (int i = 0; i < MAX_PER_LANE; ++i)
-      if (i * 64 + lane == bi) v[i] = -INFINITY;
-    const int sel = min(bi, NE - 1);  // (a row of NaN picks no lane: keep the index inside the tables)
-    const float p = expf(bv - mx);
-    sum += p;
-    if (lane == k) { mysel = sel; myp = p; }
-  }
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+    for (int k = 0; k < NU; ++k) {
+      float bv = -INFINITY;
+      int bi = NE;
+#pragma unroll
+      for (int i = 0; i < PL; ++i)
+        if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
+      // wave arg-max, the lower index among equal values
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) {
+        const float ov = __shfl_xor(bv, d, 64);
+        const int oi = __shfl_xor(bi, d, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+#pragma unroll
+      for (int i = 0; i < PL; ++i)
+        if (i * 64 + lane == bi) v[i] = -INFINITY;
+      const int sel = min(bi, NE - 1);  // (a row of NaN picks no lane: keep the index inside the tables)
+      const float p = expf(bv - mx);
+      sum += p;
+      if (lane == k) { mysel = sel; myp = p; }
+    }
+  };
+  if (NE <= 128) pick(std::integral_constant<int, 2>());
+  else pick(std::integral_constant<int, MAX_PER_LANE>());
   if (lane < NU) {
     ids[(size_t)t * NU + lane] = mysel;
     wts[(size_t)t * NU + lane] = myp / sum;
-    atomicAdd(&counts[mysel], 1);
+    // (NPART copies of the counters, a work-group adding to copy blockIdx % NPART: many adds to one word from all
+    //  over the chip queue up at the memory side; moe_scan sums the copies)
+    atomicAdd(&counts[(size_t)(blockIdx.x % NPART) * NE + mysel], 1);
   }
   if (lane == 0 && sgate) sgate[t] = ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
 }
@@ -110,14 +119,23 @@ extern "C" __global__ __launch_bounds__(64) void moe_route1(const float* __restr
 }
 
 // moe_scan: exclusive scan of the counts -> offs / cursor; the tile list tiles[0] = number of tiles, then (expert,
-// first slot, rows <= TM) per tile; tstart[e] = first tile of expert e, tstart[NE] = the tile count; counts reset.
+// first slot, rows <= TM) per tile; tstart[e] = first tile of expert e, tstart[NE] = the tile count; counts (all NPART copies) reset.
 // One work-group of 1024 threads (NE <= 1024).
 extern "C" __global__ __launch_bounds__(1024) void moe_scan(int* __restrict__ counts, int* __restrict__ offs,
                                                             int* __restrict__ cursor, int* __restrict__ tiles,
-                                                            int* __restrict__ tstart, int NE, int TM) {
+                                                            int* __restrict__ tstart, int NE, int TM, int NPART) {
   __shared__ int a[1024], b[1024];
   const int e = threadIdx.x;
-  const int c = e < NE ? counts[e] : 0, nt = (c + TM - 1) / TM;
+  // the copies moe_route counted into, summed (integer adds in LDS: any order gives the same sums) and reset
+  a[e] = 0;
+  __syncthreads();
+  for (int i = e; i < NPART * NE; i += 1024) {
+    atomicAdd(&a[i % NE], counts[i]);
+    counts[i] = 0;
+  }
+  __syncthreads();
+  const int c = e < NE ? a[e] : 0, nt = (c + TM - 1) / TM;
+  __syncthreads();
   a[e] = c;
   b[e] = nt;
   __syncthreads();
@@ -140,41 +158,67 @@ extern "C" __global__ __launch_bounds__(1024) void moe_scan(int* __restrict__ co
     tp[1] = off + i * TM;
     tp[2] = min(TM, c - i * TM);
   }
-  counts[e] = 0;
 }
 
 // moe_scatter: places pair i = (token i / NU, expert ids[i]) in a slot of its expert's range, in pair order: the
 // k-th pair of expert e (counting i upwards) gets slot offs[e] + k, so the layout is the same on every run (the
 // reference draws slots from an atomic counter; its results do not depend on the order, its layout does).
 // One work-group of 256 threads per expert, each scanning all n pairs.  `cursor` holds offs (as moe_scan wrote it).
+// The list is taken in pieces of 256 * SCAT_IT pairs: first every wave counts its matches in each 256-pair step of the
+// piece (no barrier between steps), then one scan over the (step, wave) counts gives every wave its first rank in
+// every step, then the steps are run again and the pairs written.
+#define SCAT_IT 32
 extern "C" __global__ __launch_bounds__(256) void moe_scatter(const int* __restrict__ ids, const float* __restrict__ wts,
                                                               int n, int* __restrict__ cursor, int* __restrict__ stok,
                                                               float* __restrict__ swt, int* __restrict__ inv, int NU) {
-  __shared__ int wsum[4];
-  __shared__ int base_s;
+  __shared__ int cnt[SCAT_IT * 4];  // matches of wave w in step j at [4 j + w], then their exclusive prefix sums
+  __shared__ int wtot[4];
   const int e = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  if (t == 0) base_s = cursor[e];
-  __syncthreads();
-  for (int i0 = 0; i0 < n; i0 += 256) {
-    const int i = i0 + t;
-    const bool mine = i < n && ids[i] == e;
-    const unsigned long long bal = __ballot(mine);
-    const int rank = __popcll(bal & ((1ull << lane) - 1));
-    if (lane == 0) wsum[wave] = __popcll(bal);
-    __syncthreads();
-    int before = 0;
-    for (int w = 0; w < wave; ++w) before += wsum[w];
-    const int total = wsum[0] + wsum[1] + wsum[2] + wsum[3];
-    const int base = base_s;
-    if (mine) {
-      const int s = base + before + rank;
-      stok[s] = i / NU;
-      swt[s] = wts[i];
-      inv[i] = s;
+  int base = cursor[e];
+  for (int p0 = 0; p0 < n; p0 += 256 * SCAT_IT) {
+    int my[SCAT_IT];  // the thread's pairs of the piece, all loads in flight together
+#pragma unroll
+    for (int j = 0; j < SCAT_IT; ++j) {
+      const int i = p0 + j * 256 + t;
+      my[j] = i < n ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < SCAT_IT; ++j) {
+      const unsigned long long bal = __ballot(my[j] == e);
+      if (lane == 0) cnt[4 * j + wave] = __popcll(bal);
     }
     __syncthreads();
-    if (t == 0) base_s = base + total;
+    // exclusive scan of cnt[0 .. 4 SCAT_IT): threads 0-63 own entries 2 t, 2 t + 1, the rest none
+    int c0 = 0, c1 = 0;
+    if (t < 2 * SCAT_IT) { c0 = cnt[2 * t]; c1 = cnt[2 * t + 1]; }
+    int incl = c0 + c1;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += o;
+    }
+    if (lane == 63) wtot[wave] = incl;
     __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += wtot[w];
+    const int total = wtot[0] + wtot[1] + wtot[2] + wtot[3];
+    const int excl = before + incl - (c0 + c1);
+    if (t < 2 * SCAT_IT) { cnt[2 * t] = excl; cnt[2 * t + 1] = excl + c0; }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < SCAT_IT; ++j) {
+      const int i = p0 + j * 256 + t;
+      const bool mine = my[j] == e;
+      const unsigned long long bal = __ballot(mine);
+      if (mine) {
+        const int s = base + cnt[4 * j + wave] + __popcll(bal & ((1ull << lane) - 1));
+        stok[s] = i / NU;
+        swt[s] = wts[i];
+        inv[i] = s;
+      }
+    }
+    base += total;
+    __syncthreads();  // (cnt and wtot are rewritten by the next piece)
   }
 }
 
