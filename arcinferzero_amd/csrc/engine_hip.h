@@ -387,7 +387,18 @@ class Engine {
     moe_route(L, rl, ldl, T, tm);
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)
     const size_t max_tiles = (size_t)(n + tm - 1) / tm + std::min(n, L.NE);
-    moe_gemm(L, 0, Mp, max_tiles);
+    if (L.ex[0].type == GGML_Q4_K && L.ex[1].type == GGML_Q4_K) {
+      // gate and up in one pass (the reference's moe_gateup_q, zero/kernels/decode_moe.cl:92-94, launched by
+      // zero/engine_moe.h:300-330): h = silu(gate) * up into mh_
+      cl_kernel k = kernel("gemm", "-DQT=12 -DNE=" + std::to_string(L.NE), "moe_gateup_q");
+      int FF = F, KK = E, MM = Mp;
+      cl_mem tabs = nullptr;
+      set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
+      size_t gws[2] = {(size_t)(F + 127) / 128 * 256, max_tiles}, lws[2] = {256, 1};
+      run("moe_gateup", k, 2, gws, lws);
+    } else {
+      moe_gemm(L, 0, Mp, max_tiles);
+    }
     {
       // (the reference's moe_quant writes no sums; the Q4_K tile GEMM here takes them for its min term)
       cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_quant_sums");

@@ -40,6 +40,7 @@ static const KernelSpec kKernelTable[] = {
     {"gemm", "gemm_simple", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     // ---- moe
     {"moe", "moe_route", nullptr, "piipppp", {nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_route1", nullptr, "pppppp", {nullptr},

@@ -934,6 +934,246 @@ __device__ inline void gemm4_body(const uint8_t* __restrict__ raw, const signed 
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Q4_K gate and up projections of a mixture-of-experts layer in one pass (the reference's moe_gateup_q,
+// zero/kernels/decode_moe.cl:92-94: h = silu(gate) * up straight from the two raw expert tensors).  The tile body above
+// with two weight streams: the 64 slots' activations are staged once for both, a wave computes its 32 rows of gate and
+// of up (16 products a step instead of 8, the same barrier and loads-issue cost), and the epilogue writes h once --
+// against two launches, the second reading the first's output back.
+#define GU_STAGE 34816
+#define GU_WQ0 8192
+#define GU_WQ1 16384
+#define GU_SA 24576
+#define GU_U 25600
+#define GU_WS0 26624
+#define GU_V0 28672
+#define GU_WS1 30720
+#define GU_V1 32768
+
+struct GuScaleRegs {
+  float sa;
+  short bs[2];
+  uint4 h;
+};
+
+__device__ inline void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
+                                    const signed char* __restrict__ aq, const float* __restrict__ asc,
+                                    const short* __restrict__ absum, float* __restrict__ H, int M, int N, int K,
+                                    size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
+                                    const int* __restrict__ rowmap) {
+  __shared__ alignas(16) uint8_t lds[2 * GU_STAGE];
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8;
+  const PlanesQ4K pl = planes_q4k(rows_total, nsb);
+  auto token_row = [&](int r) { return rowmap[m0 + (r < rows_valid ? r : 0)]; };  // slots past the tile read its first
+  const uint8_t* raws[2] = {rg, ru};
+
+  uint32_t aoff[2], woff[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int R = (wave * 2 + i) * 8 + (lane >> 3);
+    aoff[i] = (uint32_t)token_row(R) * (uint32_t)K + 16u * ((lane & 7) ^ (lane >> 3));
+    const int R2 = (wave * 2 + i) * 16 + (lane >> 2);
+    woff[i] = (uint32_t)min(n0 + R2, N - 1) * (uint32_t)nsb * 128u + 16u * ((lane & 3) ^ ((lane >> 3) & 3));
+  }
+  const size_t wrow0 = pl.qs + row_base * nsb * 128;
+  // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t % 128 of gate (t < 128) or up
+  const int r_s = t & 63, b_s = t >> 6;
+  const bool tok_valid = r_s < rows_valid;
+  const uint32_t m_s = (uint32_t)token_row(r_s);
+  const int row_s = t & 127, x_s = wave >> 1;
+  const uint8_t* hsrc = (x_s ? ru : rg) + pl.hdr + (row_base + min(n0 + row_s, N - 1)) * nsb * 16;
+
+  auto dma_step = [&](int st, int stage) {
+    uint8_t* base = lds + stage * GU_STAGE;
+    const signed char* ab = aq + (size_t)st * 128;
+    // (the offsets pass through an empty asm so that the 64-bit addresses are formed here, each step, and not kept in
+    //  twelve registers over the whole loop)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) asm volatile("" : "+v"(aoff[i]), "+v"(woff[i]));
+#pragma unroll
+    for (int i = 0; i < 2; ++i) g3_dma16(ab + aoff[i], base + (wave * 2 + i) * 1024);
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+      const uint8_t* wb = raws[x] + wrow0 + (size_t)st * 64;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[i], base + (x ? GU_WQ1 : GU_WQ0) + (wave * 2 + i) * 1024);
+    }
+  };
+  auto load_scales = [&](GuScaleRegs& r, int st) {
+    const int blk = st * 4 + b_s;
+    r.sa = (asc + (size_t)blk * M)[m_s];
+    r.bs[0] = (absum + (size_t)(2 * blk) * M)[m_s];
+    r.bs[1] = (absum + (size_t)(2 * blk + 1) * M)[m_s];
+    r.h = *(const uint4*)(hsrc + (size_t)(st >> 1) * 16);
+  };
+  auto store_scales = [&](const GuScaleRegs& r, int st, int stage) {
+    uint8_t* base = lds + stage * GU_STAGE;
+    const float sa = tok_valid ? r.sa : 0.0f;
+    ((float*)(base + GU_SA))[b_s * 64 + r_s] = sa;
+    ((float*)(base + GU_U))[b_s * 64 + r_s] = sa * (float)((int)r.bs[0] + (int)r.bs[1]);
+    const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
+    float* ws = (float*)(base + (x_s ? GU_WS1 : GU_WS0));
+    float* vv = (float*)(base + (x_s ? GU_V1 : GU_V0));
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      int sc0, sc1, mn0, mn1;
+      q4k_scales_pair(r.h.y, r.h.z, r.h.w, 2 * (st & 1) + p, sc0, sc1, mn0, mn1);
+      ws[(2 * p) * 128 + row_s] = d * (float)sc0;
+      ws[(2 * p + 1) * 128 + row_s] = d * (float)sc1;
+      vv[(2 * p) * 128 + row_s] = -(dmin * (float)mn0);
+      vv[(2 * p + 1) * 128 + row_s] = -(dmin * (float)mn1);
+    }
+  };
+
+  int oa[4], ow[2];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) oa[b] = l32 * 128 + (((2 * b + g) ^ (l32 & 7)) * 16);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) ow[j] = (wave * 32 + l32) * 64 + (((2 * j + g) ^ ((l32 >> 1) & 3)) * 16);
+
+  v16f res[2][2];  // [gate / up][slot tile]
+#pragma unroll
+  for (int x = 0; x < 2; ++x)
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) res[x][ms][i] = 0.0f;
+
+  const int steps = 2 * nsb;
+  GuScaleRegs sr;
+  dma_step(0, 0);
+  load_scales(sr, 0);
+  store_scales(sr, 0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the stage has landed
+  __syncthreads();
+
+#pragma unroll 1
+  for (int st = 0; st < steps; ++st) {
+    const uint8_t* Sb = lds + (st & 1) * GU_STAGE;
+    const bool next = st + 1 < steps;
+    if (next) {
+      dma_step(st + 1, (st + 1) & 1);
+      load_scales(sr, st + 1);
+    }
+    // packed weights of the lane's rows, [gate / up]: the block pair in use (the second pair of the step is read into
+    // the same registers once both blocks of the first are split off)
+    v4i wr[2];
+    auto ld_wr = [&](int j, int x) { wr[x] = *(const v4i*)(Sb + (x ? GU_WQ1 : GU_WQ0) + ow[j]); };
+    ld_wr(0, 0); ld_wr(0, 1);
+    v4i a16[2], w16[2];  // [slot tile], [gate / up]: reloaded for the next block as soon as their last product is issued
+    float saop, wsop[2], uop[2], vop[2];
+    v32f P[2];  // scale tiles of the block: [gate / up], both slot tiles
+    v16i I[2];
+    auto ld_a = [&](int b, int ms) { a16[ms] = *(const v4i*)(Sb + oa[b] + ms * 32 * 128); };
+    auto ld_sa = [&](int b) { saop = ((const float*)(Sb + GU_SA))[b * 64 + lane]; };
+    auto ld_ws = [&](int b, int x) { wsop[x] = ((const float*)(Sb + (x ? GU_WS1 : GU_WS0)))[b * 128 + wave * 32 + l32]; };
+    auto dec_w = [&](int b, int x) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t v = (uint32_t)wr[x][i];
+        w16[x][i] = (int)((b & 1) ? (v >> 4) & 0x0F0F0F0Fu : v & 0x0F0F0F0Fu);
+      }
+    };
+    auto mfma_p = [&](int x) {
+      v32f zf;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+      P[x] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop, wsop[x], zf, 0, 0, 0);
+    };
+    auto mfma_i = [&](int x, int ms, int slot) {
+      v16i z;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] = 0;
+      I[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[ms], w16[x], z, 0, 0, 0);
+    };
+    ld_a(0, 0); ld_a(0, 1); ld_sa(0); ld_ws(0, 0); ld_ws(0, 1);
+    dec_w(0, 0); dec_w(0, 1);
+    mfma_p(0);
+    mfma_i(0, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const bool more = b + 1 < 4;
+      if ((b & 1) == 0) {  // min term of blocks b and b + 1: lane half g supplies block b + g
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) uop[ms] = ((const float*)(Sb + GU_U))[(b + g) * 64 + ms * 32 + l32];
+#pragma unroll
+        for (int x = 0; x < 2; ++x) vop[x] = ((const float*)(Sb + (x ? GU_V1 : GU_V0)))[(b + g) * 128 + wave * 32 + l32];
+      }
+      // four phases: (gate, tile 0), (gate, tile 1), (up, tile 0), (up, tile 1); each issues the next phase's product
+#pragma unroll
+      for (int ph = 0; ph < 4; ++ph) {
+        const int x = ph >> 1, ms = ph & 1, slot = ph & 1;
+        if (ph == 0) {
+          mfma_i(0, 1, 1);                      // (gate, 1)
+          if (more) {                           // gate's operand of the next block (this block's is issued twice by now)
+            dec_w(b + 1, 0);
+            if (b == 0) ld_wr(1, 0);
+          }
+        }
+        if (ph == 1) {
+          mfma_p(1);                            // up's scale tiles of this block
+          mfma_i(1, 0, 0);                      // (up, 0)
+          if (more) { ld_a(b + 1, 0); ld_sa(b + 1); ld_ws(b + 1, 0); }
+        }
+        if (ph == 2) {
+          mfma_i(1, 1, 1);                      // (up, 1)
+          if (more) {
+            ld_a(b + 1, 1); dec_w(b + 1, 1); ld_ws(b + 1, 1);
+            if (b == 0) ld_wr(1, 1);
+          }
+        }
+        if (ph == 3 && more) {
+          mfma_p(0);                            // gate's scale tiles of the next block
+          mfma_i(0, 0, 0);                      // (gate, 0) of the next block
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          res[x][ms][i] = __builtin_fmaf((float)I[slot][i], P[x][16 * ms + i], res[x][ms][i]);
+        if ((b & 1) == 0) res[x][ms] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop[x], res[x][ms], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    asm volatile("" : "+v"(res[0][0]), "+v"(res[0][1]), "+v"(res[1][0]), "+v"(res[1][1]));
+    if (next) {
+      store_scales(sr, st + 1, (st + 1) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = row n of the expert's F, accumulator i = slot 8 * (i / 4) + 4 * g + i % 4
+  const int n = n0 + wave * 32 + l32;
+  if (n < N) {
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+        if (r >= rows_valid) continue;
+        const float gt = res[0][ms][i];
+        H[(size_t)(m0 + r) * N + n] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
+      }
+  }
+}
+
+// moe_gateup_q: arguments as the reference's (zero/kernels/decode_moe.cl:92-94) -- the two raw expert tensors
+// [NE][F][K], the tile list (tiles of at most 64 slots), stok = the token row of every slot, h [slots][F] -- and, as its
+// extra arguments, the activations' sums per 16 values.  grid (ceil(F / 128) * 256, tile work-groups): work-group y
+// takes tiles y, y + gridDim.y, ...
+extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12(
+    const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc,
+    int M, const int* tiles, const int* stok, float* h, const short* absum, int NE) {
+  const int nt = tiles[0];
+  for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+    gemm4gu_body(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), blockIdx.x * BN, stok);
+    __syncthreads();
+  }
+}
+
 // Tile of work-group `id` out of mt x nt tiles.  XCDs take work-groups in turn (id % 8), each running 64 at a time:
 // those 64 are made an 8 x 8 block of tiles when both tile counts are multiples of 8, token tiles fastest otherwise.
 __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {

@@ -191,7 +191,7 @@ def bench_moe(az, launches):
     parts = {}
     for name in ("moe_route", "moe_scan", "moe_scatter", "moe_gateup", "moe_quant", "moe_down", "moe_combine"):
         t, n = eng.profile_get(name)
-        parts[name + "_ms"] = t / max(n, 1) * (2 if name == "moe_gateup" else 1)   # gate and up are two launches
+        parts[name + "_ms"] = t / launches   # per layer, however many launches the step takes
     ops = T * NU * 3 * 2.0 * F * E
     gemm_ms = parts["moe_gateup_ms"] + parts["moe_down_ms"]
     for b in (xb, lb, ob):
