@@ -348,6 +348,12 @@ __device__ inline void gemm3_body(const uint8_t* __restrict__ raw, const signed 
     uint8_t* base = lds + stage * G3_STAGE;
     const signed char* ab = abase + (size_t)st * 128;
     const uint8_t* wb = wbase + (size_t)st * 64;
+    // (the offsets pass through an empty asm so that the 64-bit addresses are formed here, each step, and not kept in
+    //  twelve registers over the whole loop)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(aoff[i]));
+#pragma unroll
+    for (int i = 0; i < 2; ++i) asm volatile("" : "+v"(woff[i]));
 #pragma unroll
     for (int i = 0; i < 4; ++i) g3_dma16(ab + aoff[i], base + (wave * 4 + i) * 1024);
 #pragma unroll
