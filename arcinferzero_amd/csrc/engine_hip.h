@@ -45,6 +45,8 @@ class Engine {
     cl_.soft_fail = true;
     if (!cl_.init()) throw std::runtime_error(std::string("no GPU runtime: ") + arcz_last_error());
     if (max_chunk <= 0 || max_k <= 0 || max_k % 256) throw std::invalid_argument("Engine: max_k must be a positive multiple of 256");
+    // (the GEMM kernels address a chunk's int8 rows and a matrix's packed rows with 32-bit byte offsets)
+    if ((uint64_t)max_chunk * (uint64_t)max_k >= (1ull << 32)) throw std::invalid_argument("Engine: a chunk of max_chunk x max_k values must stay below 4 GiB");
     const size_t M = (size_t)max_chunk;
     aq_ = buf(M * max_k);
     asc_ = buf(M * (max_k / 32) * 4);
@@ -104,6 +106,8 @@ class Engine {
     if (type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q6_K)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
+    if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))
+      throw std::runtime_error("make_weight: a matrix of " + std::to_string(N) + " x " + std::to_string(K) + " is too large for 32-bit row offsets");
     if (nbytes != arcz_gguf_bytes(type, rows, K))
       throw std::runtime_error("make_weight: " + std::to_string(nbytes) + " bytes given, " +
                                std::to_string(arcz_gguf_bytes(type, rows, K)) + " expected");
