@@ -267,15 +267,19 @@ class Engine {
   // The prefill GEMM (zero/engine.h:1205-1250).  Token rows come in whole tiles (the reference pads a chunk to 128
   // rows from 128 tokens on, :521-522).
   void gemm_dense(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int a) {
-    cl_kernel k = gemm_kernel(w.type, false);
     int M = Mp, N = w.N, K = w.K;
+    // tiles of 128 tokens x 128 rows for Q4_K, 64 x 128 for Q6_K and Q8_0 (whose 64-token kernel measured 1.9 x the
+    // 128-token one at 17408 x 5120 x 8192 and 3 x at 4096 x 4096 x 512; ARCZ_Q8_BM=128 brings the latter back)
+    static const int q8_bm = getenv("ARCZ_Q8_BM") ? atoi(getenv("ARCZ_Q8_BM")) : 0;
+    const bool q8_small = w.type == GGML_Q8_0 && q8_bm != 128;
+    cl_kernel k = q8_small ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm") : gemm_kernel(w.type, false);
     // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
     //  registers over the whole of K.  The reference splits rows longer than 8192 into 17-superblock pieces for its
     //  cache, zero/engine.h:1236-1250; pieces after the first accumulate into C and are not bit-identical to one pass.)
     static const int sk_sb = getenv("ARCZ_GEMM_SPLIT") ? std::max(0, atoi(getenv("ARCZ_GEMM_SPLIT"))) : 0;
     const int nsb = K / 256, splits = a != 2 && sk_sb > 0 ? (nsb + sk_sb - 1) / sk_sb : 1, rgroup = 1;
     cl_mem unused = nullptr;
-    const int bm = w.type == GGML_Q6_K ? 64 : 128;  // token rows of a work-group's tile
+    const int bm = w.type == GGML_Q6_K || q8_small ? 64 : 128;  // token rows of a work-group's tile
     const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + 127) / 128);
     size_t gws[1] = {tiles * 256}, lws[1] = {256};
     for (int sp = 0; sp < splits; ++sp) {
@@ -488,11 +492,12 @@ inline std::string engine_self_check() {
         }
       }
     GpuWeight gw = e.make_weight(type, w.data(), w.size(), N, K);
-    for (int which = 0; which < 2; ++which) {
-      cl_kernel k = e.kernel("gemm", "-DQTYPE=" + std::to_string(type) + " -DACT32", which ? "gemm_simple" : "gemm");
-      cl_mem unused = nullptr, C = which ? c1 : c0;
+    e.gemm_dense("self_check", gw, M, c0, N, 0, 0);  // the kernel the engine's dispatch takes for this type
+    {
+      cl_kernel k = e.kernel("gemm", "-DQTYPE=" + std::to_string(type) + " -DACT32", "gemm_simple");
+      cl_mem unused = nullptr;
       int MM = M, NN = N, KK = K, ldc = N, zero = 0, one = 1, s1 = K / 256;
-      set_args(k, 0, gw.raw, unused, e.aq_, e.asc_, e.absum_, C, MM, NN, KK, ldc, zero, zero, one, zero, s1);
+      set_args(k, 0, gw.raw, unused, e.aq_, e.asc_, e.absum_, c1, MM, NN, KK, ldc, zero, zero, one, zero, s1);
       size_t gws[1] = {(size_t)(M / 128) * (N / 128) * 256}, lws[1] = {256};
       e.run("self_check", k, 1, gws, lws);
     }

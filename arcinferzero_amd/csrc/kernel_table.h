@@ -36,6 +36,7 @@ static const KernelSpec kKernelTable[] = {
     // ---- gemm
     {"gemm", "gemm", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "BM", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},

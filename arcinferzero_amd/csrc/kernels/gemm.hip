@@ -1180,10 +1180,174 @@ extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12(
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Q8_0, dense, 64-token tiles: the shape of the Q6_K kernel for matrices with few 128 x 128 tiles (4096 x 4096 at 512
+// tokens is 128 of them on 256 compute units; in 64-token tiles it is 256).  The int8 rows go straight into LDS and
+// into the products unchanged; res += (sa[m][b] * d[n][b]) * (float)I.
+#define G8_STAGE 27648
+#define G8_W 8192
+#define G8_SA 24576
+#define G8_WS 25600
+
+__device__ inline void gemm8_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+                                  const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
+                                  int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0) {
+  __shared__ alignas(16) uint8_t lds[2 * G8_STAGE];
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8;
+  const PlanesQ80 pl = planes_q80((size_t)N, nsb);
+  auto token_row = [&](int r) { return m0 + (r < rows_valid ? r : 0); };  // rows past the tile read its first row
+
+  // activations: 2 instructions a wave, 8 rows each; weights: 4 instructions a wave, 8 rows of 128 bytes each
+  uint32_t aoff[2], woff[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    aoff[i] = (uint32_t)token_row((wave * 2 + i) * 8 + (lane >> 3)) * (uint32_t)K + 16u * ((lane & 7) ^ (lane >> 3));
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    woff[i] = (uint32_t)min(n0 + (wave * 4 + i) * 8 + (lane >> 3), N - 1) * (uint32_t)nsb * 256u + 16u * ((lane & 7) ^ (lane >> 3));
+  const signed char* abase = aq + (size_t)s_begin * 256;
+  const uint8_t* wbase = raw + pl.qs + (size_t)s_begin * 256;
+  // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t / 2, blocks 2 (t % 2) + {0, 1}
+  const int r_s = t & 63, b_s = t >> 6;
+  const bool tok_valid = r_s < rows_valid;
+  const uint32_t m_s = (uint32_t)token_row(r_s);
+  const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
+
+  auto dma_step = [&](int st, int stage) {
+    uint8_t* base = lds + stage * G8_STAGE;
+    const signed char* ab = abase + (size_t)st * 128;
+    const uint8_t* wb = wbase + (size_t)st * 128;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) asm volatile("" : "+v"(aoff[i]));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(woff[i]));
+#pragma unroll
+    for (int i = 0; i < 2; ++i) g3_dma16(ab + aoff[i], base + (wave * 2 + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) g3_dma16(wb + woff[i], base + G8_W + (wave * 4 + i) * 1024);
+  };
+  float sa_r;
+  uint32_t d_r;
+  auto load_scales = [&](int st) {
+    sa_r = (asc + (size_t)(s_begin * 8 + st * 4 + b_s) * M)[m_s];
+    d_r = *(const uint32_t*)(raw + pl.d + (((size_t)n_s * nsb + s_begin) * 8 + st * 4 + 2 * p_s) * 2);
+  };
+  auto store_scales = [&](int stage) {
+    uint8_t* base = lds + stage * G8_STAGE;
+    ((float*)(base + G8_SA))[b_s * 64 + r_s] = tok_valid ? sa_r : 0.0f;
+    ((float*)(base + G8_WS))[(2 * p_s) * 128 + (t >> 1)] = f16_bits_to_f32(d_r);
+    ((float*)(base + G8_WS))[(2 * p_s + 1) * 128 + (t >> 1)] = f16_bits_to_f32(d_r >> 16);
+  };
+
+  int oa[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) oa[b] = l32 * 128 + (((2 * b + g) ^ (l32 & 7)) * 16);
+  const int wrow = G8_W + wave * 32 * 128;
+
+  v16f res[2];
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) res[ms][i] = 0.0f;
+
+  const int steps = 2 * (s_end - s_begin);
+  if (steps > 0) {
+    dma_step(0, 0);
+    load_scales(0);
+    store_scales(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the stage has landed
+  }
+  __syncthreads();
+
+#pragma unroll 1
+  for (int st = 0; st < steps; ++st) {
+    const uint8_t* Sb = lds + (st & 1) * G8_STAGE;
+    const bool next = st + 1 < steps;
+    if (next) {
+      dma_step(st + 1, (st + 1) & 1);
+      load_scales(st + 1);
+    }
+    v4i a16[2][2], w16[2];  // [buffer][ms]; [buffer]
+    float saop[2], wsop[2];
+    v32f P[2];
+    v16i I[2];
+    auto ld_ops = [&](int b, int buf) {
+      a16[buf][0] = *(const v4i*)(Sb + oa[b]);
+      a16[buf][1] = *(const v4i*)(Sb + oa[b] + 32 * 128);
+      w16[buf] = *(const v4i*)(Sb + wrow + oa[b]);
+      saop[buf] = ((const float*)(Sb + G8_SA))[b * 64 + lane];
+      wsop[buf] = ((const float*)(Sb + G8_WS))[b * 128 + wave * 32 + l32];
+    };
+    auto mfma_p = [&](int buf) {
+      v32f zf;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+      P[buf] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[buf], wsop[buf], zf, 0, 0, 0);
+    };
+    auto mfma_i = [&](int buf, int ms, int slot) {
+      v16i z;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) z[i] = 0;
+      I[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[buf][ms], w16[buf], z, 0, 0, 0);
+    };
+    ld_ops(0, 0);
+    mfma_p(0);
+    mfma_i(0, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int buf = b & 1;
+      const bool more = b + 1 < 4;
+#pragma unroll
+      for (int ms = 0; ms < 2; ++ms) {
+        if (ms == 0) {
+          mfma_i(buf, 1, 1);
+          if (more) ld_ops(b + 1, buf ^ 1);
+        } else if (more) {
+          mfma_p(buf ^ 1);
+          mfma_i(buf ^ 1, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) res[ms][i] = __builtin_fmaf((float)I[ms][i], P[buf][16 * ms + i], res[ms][i]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    asm volatile("" : "+v"(res[0]), "+v"(res[1]));  // (the sums are complete before the branches below)
+    if (next) {
+      store_scales((st + 1) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __syncthreads();
+  }
+
+  const int n = n0 + wave * 32 + l32;
+  if (n < N) {
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+        if (r >= rows_valid) continue;
+        float v = res[ms][i];
+        float* cp = C + (size_t)(m0 + r) * ldc + c_off + n;
+        if (accumulate == 1) {
+          v += *cp;
+        } else if (accumulate == 2) {
+          const float gt = *cp;
+          v *= gt / (1.0f + __expf(-gt));
+        }
+        *cp = v;
+      }
+  }
+}
+
 // Tile of work-group `id` out of mt x nt tiles.  XCDs take work-groups in turn (id % 8), each running 64 at a time:
-// those 64 are made an 8 x 8 block of tiles when both tile counts are multiples of 8, token tiles fastest otherwise.
+// those 64 are made an 8 x 8 block of tiles when both tile counts are multiples of 8 and the blocks share out evenly
+// over the 8 XCDs; token tiles fastest otherwise.
 __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
-  if ((mt & 7) == 0 && (nt & 7) == 0) {
+  if ((mt & 7) == 0 && (nt & 7) == 0 && (((mt >> 3) * (nt >> 3)) & 7) == 0) {  // (whole 8 x 8 blocks, 8 XCDs' worth)
     const int x = id & 7, q = id >> 3;
     const int st = (q >> 6) * 8 + x, within = q & 63;
     const int smt = mt >> 3;
@@ -1230,6 +1394,16 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
 
 GEMM2_INST(8)
 GEMM2_TILES_INST(8)
+// -DBM=64: the 64-token form (grid ceil(N / 128) * ceil(M / 64) work-groups)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE8_ACT321_BM64(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  gemm8_body(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
+}
 
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
