@@ -234,13 +234,15 @@ class Engine {
         if (!lpr && (units + l - 1) / l <= 6 && (!force_lpr || l == force_lpr)) lpr = l;
       const int g = lpr ? 256 / lpr : 1, wpr = lpr > 64 ? lpr / 64 : 1;
       const int tbl = T <= 2 ? T : T <= 4 ? 4 : 8;  // the kernel's token count (T rounded up)
-      const size_t lds = (size_t)tbl * tok_bytes + (wpr > 1 ? (size_t)2 * g * wpr * tbl * 4 : 0);
+      const size_t lds = (size_t)tbl * tok_bytes + (wpr > 1 ? (size_t)16 * g * wpr * tbl * 4 : 0);  // (16: the kernels' GEMV_FLUSH)
       if (!force_v && lpr && lds <= 65536) {
         const int pf = (units + lpr - 1) / lpr, tb = T <= 2 ? T : T <= 4 ? 4 : 8;
         // one round of resident work-groups, passes of rows dealt to them in turn (ARCZ_GEMV_WPC: work-groups per
         // compute unit; two measured best: more add staging work and spread the reads over more rows at a time)
         static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
-        const size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : 2));
+        static const int wgs_env = getenv("ARCZ_GEMV_WGS") ? atoi(getenv("ARCZ_GEMV_WGS")) : 0;
+        size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : 2));
+        if (wgs_env > 0) wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)wgs_env);
         const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
                                  std::to_string(pf) + (T > 1 ? " -DTB=" + std::to_string(tb) : std::string()) + " -DLDS=" +
                                  std::to_string(lds);
@@ -268,19 +270,26 @@ class Engine {
   // rows from 128 tokens on, :521-522).
   void gemm_dense(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int a) {
     int M = Mp, N = w.N, K = w.K;
-    // tiles of 128 tokens x 128 rows for Q4_K, 64 x 128 for Q6_K and Q8_0 (whose 64-token kernel measured 1.9 x the
+    // tiles of 128 tokens x 128 rows (or 64 x 256) for Q4_K, 64 x 128 for Q6_K and Q8_0 (whose 64-token kernel measured 1.9 x the
     // 128-token one at 17408 x 5120 x 8192 and 3 x at 4096 x 4096 x 512; ARCZ_Q8_BM=128 brings the latter back)
     static const int q8_bm = getenv("ARCZ_Q8_BM") ? atoi(getenv("ARCZ_Q8_BM")) : 0;
     const bool q8_small = w.type == GGML_Q8_0 && q8_bm != 128;
-    cl_kernel k = q8_small ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm") : gemm_kernel(w.type, false);
+    static const int q4_bm = getenv("ARCZ_Q4_BM") ? atoi(getenv("ARCZ_Q4_BM")) : 0;
+    // Q4_K: tiles of 64 tokens x 256 rows (the same work per work-group and the same rate as 128 x 128) when the last
+    // 128 token rows of a short chunk are at most half full (ARCZ_Q4_BM=64 always, =128 never)
+    const bool q4_wide = w.type == GGML_Q4_K && (q4_bm == 64 || (q4_bm == 0 && Mp <= 1024 && ((Mp - 1) & 127) < 64));
+    cl_kernel k = q8_small  ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
+                  : q4_wide ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64", "gemm")
+                            : gemm_kernel(w.type, false);
     // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
     //  registers over the whole of K.  The reference splits rows longer than 8192 into 17-superblock pieces for its
     //  cache, zero/engine.h:1236-1250; pieces after the first accumulate into C and are not bit-identical to one pass.)
     static const int sk_sb = getenv("ARCZ_GEMM_SPLIT") ? std::max(0, atoi(getenv("ARCZ_GEMM_SPLIT"))) : 0;
     const int nsb = K / 256, splits = a != 2 && sk_sb > 0 ? (nsb + sk_sb - 1) / sk_sb : 1, rgroup = 1;
     cl_mem unused = nullptr;
-    const int bm = w.type == GGML_Q6_K || q8_small ? 64 : 128;  // token rows of a work-group's tile
-    const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + 127) / 128);
+    const int bm = w.type == GGML_Q6_K || q8_small || q4_wide ? 64 : 128;  // token rows of a work-group's tile
+    const int bn = q4_wide ? 256 : 128;
+    const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + bn - 1) / bn);
     size_t gws[1] = {tiles * 256}, lws[1] = {256};
     for (int sp = 0; sp < splits; ++sp) {
       int s0 = nsb * sp / splits, s1 = nsb * (sp + 1) / splits, ac = sp == 0 ? a : 1;

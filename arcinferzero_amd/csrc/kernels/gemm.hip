@@ -962,26 +962,35 @@ struct GuScaleRegs {
   uint4 h;
 };
 
+// GU: the two streams are gate and up of an expert (rows n0.. of both tensors, h = silu(gate) * up); otherwise they are
+// rows n0.. and n0 + 128.. of one matrix and each gets the plain epilogue (a 64 x 256 tile of a dense product).
+template <bool GU>
 __device__ inline void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
                                     const signed char* __restrict__ aq, const float* __restrict__ asc,
                                     const short* __restrict__ absum, float* __restrict__ H, int M, int N, int K,
                                     size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
-                                    const int* __restrict__ rowmap) {
+                                    const int* __restrict__ rowmap, int ldc, int c_off, int accumulate) {
   __shared__ alignas(16) uint8_t lds[2 * GU_STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const PlanesQ4K pl = planes_q4k(rows_total, nsb);
-  auto token_row = [&](int r) { return rowmap[m0 + (r < rows_valid ? r : 0)]; };  // slots past the tile read its first
+  auto token_row = [&](int r) {  // slots past the tile read its first
+    const int rr = m0 + (r < rows_valid ? r : 0);
+    return GU ? rowmap[rr] : rr;
+  };
+  const int nx[2] = {n0, GU ? n0 : n0 + 128};  // first row of each stream
   const uint8_t* raws[2] = {rg, ru};
 
-  uint32_t aoff[2], woff[2];
+  uint32_t aoff[2], woff[2][2];  // woff[stream][instruction]
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int R = (wave * 2 + i) * 8 + (lane >> 3);
     aoff[i] = (uint32_t)token_row(R) * (uint32_t)K + 16u * ((lane & 7) ^ (lane >> 3));
     const int R2 = (wave * 2 + i) * 16 + (lane >> 2);
-    woff[i] = (uint32_t)min(n0 + R2, N - 1) * (uint32_t)nsb * 128u + 16u * ((lane & 3) ^ ((lane >> 3) & 3));
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+      woff[x][i] = (uint32_t)min(nx[x] + R2, N - 1) * (uint32_t)nsb * 128u + 16u * ((lane & 3) ^ ((lane >> 3) & 3));
   }
   const size_t wrow0 = pl.qs + row_base * nsb * 128;
   // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t % 128 of gate (t < 128) or up
@@ -989,7 +998,7 @@ __device__ inline void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_
   const bool tok_valid = r_s < rows_valid;
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int row_s = t & 127, x_s = wave >> 1;
-  const uint8_t* hsrc = (x_s ? ru : rg) + pl.hdr + (row_base + min(n0 + row_s, N - 1)) * nsb * 16;
+  const uint8_t* hsrc = (x_s ? ru : rg) + pl.hdr + (row_base + min(nx[x_s] + row_s, N - 1)) * nsb * 16;
 
   auto dma_step = [&](int st, int stage) {
     uint8_t* base = lds + stage * GU_STAGE;
@@ -997,14 +1006,14 @@ __device__ inline void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_
     // (the offsets pass through an empty asm so that the 64-bit addresses are formed here, each step, and not kept in
     //  twelve registers over the whole loop)
 #pragma unroll
-    for (int i = 0; i < 2; ++i) asm volatile("" : "+v"(aoff[i]), "+v"(woff[i]));
+    for (int i = 0; i < 2; ++i) asm volatile("" : "+v"(aoff[i]), "+v"(woff[0][i]), "+v"(woff[1][i]));
 #pragma unroll
     for (int i = 0; i < 2; ++i) g3_dma16(ab + aoff[i], base + (wave * 2 + i) * 1024);
 #pragma unroll
     for (int x = 0; x < 2; ++x) {
       const uint8_t* wb = raws[x] + wrow0 + (size_t)st * 64;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[i], base + (x ? GU_WQ1 : GU_WQ0) + (wave * 2 + i) * 1024);
+      for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[x][i], base + (x ? GU_WQ1 : GU_WQ0) + (wave * 2 + i) * 1024);
     }
   };
   auto load_scales = [&](GuScaleRegs& r, int st) {
@@ -1150,18 +1159,42 @@ __device__ inline void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_
     __syncthreads();
   }
 
-  // ---- epilogue: lane = row n of the expert's F, accumulator i = slot 8 * (i / 4) + 4 * g + i % 4
-  const int n = n0 + wave * 32 + l32;
-  if (n < N) {
+  // ---- epilogue: lane = row n of the stream, accumulator i = slot 8 * (i / 4) + 4 * g + i % 4
+  if constexpr (GU) {
+    const int n = n0 + wave * 32 + l32;
+    if (n < N) {
 #pragma unroll
-    for (int ms = 0; ms < 2; ++ms)
+      for (int ms = 0; ms < 2; ++ms)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-        if (r >= rows_valid) continue;
-        const float gt = res[0][ms][i];
-        H[(size_t)(m0 + r) * N + n] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
-      }
+        for (int i = 0; i < 16; ++i) {
+          const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          if (r >= rows_valid) continue;
+          const float gt = res[0][ms][i];
+          H[(size_t)(m0 + r) * N + n] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
+        }
+    }
+  } else {
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+      const int n = nx[x] + wave * 32 + l32;
+      if (n >= N) continue;
+#pragma unroll
+      for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          if (r >= rows_valid) continue;
+          float v = res[x][ms][i];
+          float* cp = H + (size_t)(m0 + r) * ldc + c_off + n;
+          if (accumulate == 1) {
+            v += *cp;
+          } else if (accumulate == 2) {
+            const float gt = *cp;
+            v *= gt / (1.0f + __expf(-gt));
+          }
+          *cp = v;
+        }
+    }
   }
 }
 
@@ -1175,7 +1208,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12(
   const int nt = tiles[0];
   for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
     const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-    gemm4gu_body(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), blockIdx.x * BN, stok);
+    gemm4gu_body<true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), blockIdx.x * BN,
+                       stok, 0, 0, 0);
     __syncthreads();
   }
 }
@@ -1394,6 +1428,17 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
 
 GEMM2_INST(8)
 GEMM2_TILES_INST(8)
+// Q4_K -DBM=64: 64 tokens x 256 rows per work-group (grid ceil(N / 256) * ceil(M / 64) work-groups), K from 0
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + 255) / 256;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * 256;
+  gemm4gu_body<false>(raw, raw, aq, asc, absum, C, M, N, K, (size_t)N, 0, m0, min(G6_BM, M - m0), n0, nullptr, ldc, c_off,
+                      accumulate);
+}
 // -DBM=64: the 64-token form (grid ceil(N / 128) * ceil(M / 64) work-groups)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE8_ACT321_BM64(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,

@@ -40,7 +40,8 @@ def run_gemm(eng, qtype, W, N, K, x, Mp, acc=0, c_init=None, ldc=None, c_off=0):
 
 
 @pytest.mark.parametrize("qtype", TYPES)
-@pytest.mark.parametrize("T,Mp,N,K", [(16, 16, 64, 256), (100, 112, 272, 512), (128, 128, 128, 1024), (300, 384, 384, 768)])
+@pytest.mark.parametrize("T,Mp,N,K", [(16, 16, 64, 256), (100, 112, 272, 512), (128, 128, 128, 1024), (300, 384, 384, 768),
+                                      (180, 192, 520, 512)])
 def test_gemm_vs_oracle(eng, qtype, T, Mp, N, K):
     print(f"gemm {TYPE_NAMES[qtype]} T={T} Mp={Mp} N={N} K={K}", flush=True)
     W = make_weights(qtype, N, K, seed=31 + qtype)
