@@ -86,12 +86,18 @@ __device__ inline int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amd
 
 // Sum over the 32 lanes of a half wave (lanes 0-31 and 32-63 separately), same value in every lane; a fixed tree,
 // so results do not depend on anything but the inputs.
+// The steps within a row of 16 lanes are data-parallel moves in the vector ALU (neighbour, other pair, other quad,
+// other eight: after each step the lanes that have met hold the same sum, so taking the mirrored lane gives the sum of
+// the other group); only the step between the two rows goes through the LDS crossbar.
+template <int CTRL> __device__ inline float dpp_from(float v) {
+  return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
 __device__ inline float half_wave_sum(float v) {
+  v += dpp_from<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_from<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_from<0x141>(v);  // row_half_mirror
+  v += dpp_from<0x140>(v);  // row_mirror
   v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 8, 64);
-  v += __shfl_xor(v, 4, 64);
-  v += __shfl_xor(v, 2, 64);
-  v += __shfl_xor(v, 1, 64);
   return v;
 }
 #endif
