@@ -100,4 +100,17 @@ __device__ inline float half_wave_sum(float v) {
   v += __shfl_xor(v, 16, 64);
   return v;
 }
+// Sum over each group of 32 (WIDE false) or all 64 lanes, valid in the LAST lane of the group only: the steps between
+// rows of 16 are row broadcasts in the vector ALU too (lane 15 of a row added into the next row, lane 31 into the
+// upper half), nothing goes through LDS.  A fixed tree as well.
+template <bool WIDE> __device__ inline float group_sum_last(float v) {
+  v += dpp_from<0xB1>(v);
+  v += dpp_from<0x4E>(v);
+  v += dpp_from<0x141>(v);
+  v += dpp_from<0x140>(v);
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));  // row_bcast15 -> rows 1, 3
+  if constexpr (WIDE)
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));  // row_bcast31 -> rows 2, 3
+  return v;
+}
 #endif
