@@ -83,6 +83,13 @@ __device__ inline void q4k_scales_pair(uint32_t s0, uint32_t s1, uint32_t s2, in
 }
 
 __device__ inline int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
+// The first product of a sum: the three-operand form with a constant 0 (the compiler picks the accumulate-in-place form
+// for sdot4 and spends a move on clearing its register first).
+__device__ inline int dot4_first(uint32_t a, uint32_t b) {
+  int r;
+  asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
 
 // Sum over the 32 lanes of a half wave (lanes 0-31 and 32-63 separately), same value in every lane; a fixed tree,
 // so results do not depend on anything but the inputs.
