@@ -84,6 +84,7 @@ _sig("arcz_weight_free", _i, _p, _p)
 _sig("arcz_weight_raw", _p, _p)
 _sig("arcz_engine_quantize", _i, _p, _p, _i, _i, _i, _i, _i)
 _sig("arcz_engine_rmsnorm_quant", _i, _p, _p, _i, _p, _i, _i, _i, _i, C.c_float, _p)
+_sig("arcz_engine_add_norm_quant", _i, _p, _p, _p, _p, _i, _i, _i, C.c_float, _p, _i, _i, C.c_float)
 _sig("arcz_engine_swiglu_quant", _i, _p, _p, _i, _i, _i, _i, _i, _i)
 _sig("arcz_engine_set_activations", _i, _p, _p, _p, _p, _i, _i, _i)
 _sig("arcz_engine_aq", _p, _p)
@@ -99,6 +100,7 @@ _sig("arcz_engine_self_check", _i)
 _sig("arcz_engine_profile", None, _p, _i)
 _sig("arcz_engine_profile_collect", _i, _p)
 _sig("arcz_engine_profile_get", _i, _p, C.c_char_p, C.POINTER(C.c_double), C.POINTER(_i))
+_sig("arcz_engine_profile_stats", _i, _p, C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_double))
 _sig("arcz_engine_profile_reset", None, _p)
 _sig("arcz_engine_rd_bytes", _u64, _p)
 _sig("arcz_gguf_bytes", _z, _u32, _z, _i)
@@ -410,6 +412,10 @@ class Engine:
     def quantize(self, x, ldx, K, Mp, T, act32=1):
         _check(lib.arcz_engine_quantize(self.h, x.h, ldx, K, Mp, T, act32), engine=True)
 
+    def add_norm_quant(self, x, t, w, K, T, Mp, s, w2, norm2, eps, act32=1):
+        _check(lib.arcz_engine_add_norm_quant(self.h, x.h, t.h, w.h, K, T, Mp, s, w2.h if w2 else None, 1 if norm2 else 0,
+                                              act32, eps), "add_norm_quant")
+
     def rmsnorm_quant(self, x, row_off, w, K, Mp, T, eps, hout=None, act32=1):
         _check(lib.arcz_engine_rmsnorm_quant(self.h, x.h, row_off, w.h, K, Mp, T, act32, eps, hout.h if hout else None),
                engine=True)
@@ -475,6 +481,13 @@ class Engine:
         if lib.arcz_engine_profile_get(self.h, name.encode(), C.byref(ms), C.byref(n)) != 0:
             return 0.0, 0
         return ms.value, n.value
+
+    def profile_stats(self, name):
+        """(minimum, median) of the per-launch times of `name`, ms."""
+        lo, med = C.c_double(), C.c_double()
+        if lib.arcz_engine_profile_stats(self.h, name.encode(), C.byref(lo), C.byref(med)) != 0:
+            return 0.0, 0.0
+        return lo.value, med.value
 
     def profile_reset(self):
         lib.arcz_engine_profile_reset(self.h)

@@ -1,4 +1,5 @@
 // C ABI of include/arcz_engine.h over the Engine class (engine_hip.h).
+#include <algorithm>
 #include "../../include/arcz_engine.h"
 #include "../../include/arcz_gguf.h"
 
@@ -113,6 +114,10 @@ int arcz_engine_rmsnorm_quant(arcz_engine* e, arcz_mem* x, int row_off, arcz_mem
                               float eps, arcz_mem* hout) {
   return guarded([&] { e->e->rmsnorm_quant(x, row_off, w, K, Mp, T, act32, eps, hout); });
 }
+int arcz_engine_add_norm_quant(arcz_engine* e, arcz_mem* x, arcz_mem* t, arcz_mem* w, int K, int T, int Mp, float s,
+                               arcz_mem* w2, int norm2, int act32, float eps) {
+  return guarded([&] { e->e->add_norm_quant(x, t, w, K, T, Mp, s, w2, norm2 != 0, act32, eps); });
+}
 int arcz_engine_swiglu_quant(arcz_engine* e, arcz_mem* gu, int F, int Mp, int T, int act32, int fused, int gelu) {
   return guarded([&] { e->e->swiglu_quant(gu, F, Mp, T, act32, fused, gelu); });
 }
@@ -175,7 +180,16 @@ int arcz_engine_profile_get(arcz_engine* e, const char* name, double* ms, int* l
   if (launches) *launches = e->e->prof_n[name];
   return ARCZ_OK;
 }
-void arcz_engine_profile_reset(arcz_engine* e) { e->e->prof_ms.clear(); e->e->prof_n.clear(); }
+int arcz_engine_profile_stats(arcz_engine* e, const char* name, double* min_ms, double* median_ms) {
+  auto it = e->e->prof_each.find(name);
+  if (it == e->e->prof_each.end() || it->second.empty()) return -1;
+  std::vector<double> v = it->second;
+  std::sort(v.begin(), v.end());
+  if (min_ms) *min_ms = v.front();
+  if (median_ms) *median_ms = v.size() % 2 ? v[v.size() / 2] : 0.5 * (v[v.size() / 2 - 1] + v[v.size() / 2]);
+  return ARCZ_OK;
+}
+void arcz_engine_profile_reset(arcz_engine* e) { e->e->prof_ms.clear(); e->e->prof_n.clear(); e->e->prof_each.clear(); }
 uint64_t arcz_engine_rd_bytes(arcz_engine* e) { return e->e->rd_bytes; }
 
 }  // extern "C"

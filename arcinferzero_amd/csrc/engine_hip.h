@@ -36,6 +36,7 @@ class Engine {
   ClRt cl_;
   bool profile = false;
   std::map<std::string, double> prof_ms;
+  std::map<std::string, std::vector<double>> prof_each;  // every launch's time (for the minimum and median)
   std::map<std::string, int> prof_n;
   uint64_t rd_bytes = 0;  // GGUF bytes of the weights the GEMVs read (zero/engine.h:150-151)
 
@@ -92,8 +93,10 @@ class Engine {
     if (!profile) return;
     clFinish(cl_.queue);
     for (auto& [n, e] : events_) {
-      prof_ms[n] += ClRt::event_ms(e);
+      const double ms = ClRt::event_ms(e);
+      prof_ms[n] += ms;
       prof_n[n]++;
+      prof_each[n].push_back(ms);
       clReleaseEvent(e);
     }
     events_.clear();
@@ -177,6 +180,24 @@ class Engine {
     }
     run("swiglu_quant", k, 2, gws, lws);
     cur_T_ = T; cur_K_ = F; cur_Mp_ = Mp;
+  }
+  // x = (x + rmsnorm(t) * w) * s over the first T rows ([T][K] f32 each), then the next matmul's input from the new x:
+  // rmsnorm(x) * w2, or x itself with norm2 = false (zero/engine.h:1393-1403 add_norm_quant, whose x_ and big_ are the
+  // residual stream and the block's output; here they are arguments).
+  void add_norm_quant(cl_mem x, cl_mem t, cl_mem w, int K, int T, int Mp, float s, cl_mem w2, bool norm2, int act32,
+                      float eps) {
+    check_chunk(K, Mp, T);
+    if (!act32) throw std::runtime_error("add_norm_quant: the matmul kernels take per-32 activation scales (act32)");
+    if (arcz_mem_size(x) < (size_t)T * K * 4 || arcz_mem_size(t) < (size_t)T * K * 4 || arcz_mem_size(w) < (size_t)K * 4 ||
+        (norm2 && (!w2 || arcz_mem_size(w2) < (size_t)K * 4)))
+      throw std::runtime_error("add_norm_quant: a buffer is too small for " + std::to_string(T) + " rows of " + std::to_string(K));
+    cl_kernel k = kernel("ops", "", "add_norm_quant");
+    int nrm = norm2 ? 1 : 0, MM = Mp, TT = T, KK = K;
+    set_args(k, 0, x, t, w, KK, eps, s, w2, nrm, MM, aq_, asc_, absum_, act32, TT);
+    // (a pass of 1-8 tokens: the valid rows only, as the reference; a longer chunk: all Mp rows, the padding as zeros)
+    size_t gws[2] = {256, (size_t)(wide_rows(T) ? T : Mp)}, lws[2] = {256, 1};
+    run("add_rmsnorm", k, 2, gws, lws);
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
   }
   // Activations quantized elsewhere (the reference's benches quantize on the host, bench/gemv_bench.cpp:103-129).
   void set_activations(const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp, int T) {

@@ -24,6 +24,7 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "quant_rows", nullptr, "piiiipppi", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "add_norm_quant", nullptr, "pppiffpiipppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},

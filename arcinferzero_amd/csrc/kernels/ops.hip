@@ -152,6 +152,77 @@ extern "C" __global__ __launch_bounds__(256) void rmsnorm_quant(const float* __r
   }
 }
 
+// add_norm_quant: x[m] = (x[m] + rmsnorm(t[m]) * w) * s in place (Gemma's post-norm residual add with the layer's
+// output scale), then the next matmul's input from the new row: rmsnorm(x[m]) * w2, or the row itself with w2_norm = 0,
+// quantized (reference zero/kernels/ops_attn_g.cl:616-667, same arguments plus M_valid: rows from M_valid on are
+// written as zeros where the reference launches the valid rows only).  Both sums of squares run in a fixed order.  A
+// thread reads back the values it has just stored to x itself, which the memory model orders.  grid (256, rows),
+// local (256, 1).
+extern "C" __global__ __launch_bounds__(256) void add_norm_quant(float* __restrict__ x, const float* __restrict__ t,
+                                                                 const float* __restrict__ w, int K, float eps, float s,
+                                                                 const float* __restrict__ w2, int w2_norm, int M,
+                                                                 signed char* __restrict__ aq, float* __restrict__ asc,
+                                                                 short* __restrict__ absum, int act32, int M_valid) {
+  __shared__ float red[4];
+  const int m = blockIdx.y;
+  const bool valid = m < M_valid;
+  const float* tr = t + (size_t)m * K;
+  float* xr = x + (size_t)m * K;
+  float ss = 0.0f;
+  if (valid)
+    for (int i = threadIdx.x * 4; i < K; i += 1024) {
+      const float4 f = *(const float4*)(tr + i);
+      ss += f.x * f.x;
+      ss += f.y * f.y;
+      ss += f.z * f.z;
+      ss += f.w * f.w;
+    }
+  ss = group_sum(ss, red);
+  const float r = rsqrtf(ss / (float)K + eps);
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
+  float s2 = 0.0f;
+  if (valid)
+    for (int sb = sub; sb < K / 256; sb += 16) {
+      const int base = sb * 256 + 16 * lane16;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 xo = *(const float4*)(xr + base + 4 * i), to = *(const float4*)(tr + base + 4 * i),
+                     wo = *(const float4*)(w + base + 4 * i);
+        float4 v;
+        v.x = (xo.x + to.x * r * wo.x) * s;
+        v.y = (xo.y + to.y * r * wo.y) * s;
+        v.z = (xo.z + to.z * r * wo.z) * s;
+        v.w = (xo.w + to.w * r * wo.w) * s;
+        s2 += v.x * v.x;
+        s2 += v.y * v.y;
+        s2 += v.z * v.z;
+        s2 += v.w * v.w;
+        *(float4*)(xr + base + 4 * i) = v;
+      }
+    }
+  s2 = group_sum(s2, red);
+  const float r2 = w2_norm ? rsqrtf(s2 / (float)K + eps) : 1.0f;
+  for (int sb = sub; sb < K / 256; sb += 16) {
+    const int base = sb * 256 + 16 * lane16;
+    float v[16];
+    if (valid) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 f = *(const float4*)(xr + base + 4 * i);
+        v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
+        if (w2_norm) {
+          const float4 g = *(const float4*)(w2 + base + 4 * i);
+          v[4 * i] = f.x * r2 * g.x; v[4 * i + 1] = f.y * r2 * g.y; v[4 * i + 2] = f.z * r2 * g.z; v[4 * i + 3] = f.w * r2 * g.w;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) v[i] = 0.0f;
+    }
+    store_row_quant(v, sb, lane16, m, M, K, act32, aq, asc, absum);
+  }
+}
+
 // swiglu_quant: y = silu(gate) * up (or the tanh form of gelu(gate) * up) from rows [gate(F) | up(F)], or the row as it
 // is when the matmul before has fused the product (`fused`), quantized with K = F (reference zero/kernels/ops.cl:
 // 271-315, same arguments; silu(x) = x / (1 + exp(-x)), ops.cl:33).  grid (256 * G, rows), local (256, 1).

@@ -52,6 +52,12 @@ int arcz_engine_quantize(arcz_engine* e, arcz_mem* x, int ldx, int K, int Mp, in
 int arcz_engine_rmsnorm_quant(arcz_engine* e, arcz_mem* x, int row_off, arcz_mem* w, int K, int Mp, int T, int act32,
                               float eps, arcz_mem* hout);
 int arcz_engine_swiglu_quant(arcz_engine* e, arcz_mem* gu, int F, int Mp, int T, int act32, int fused, int gelu);
+/* Engine::add_norm_quant (zero/engine.h:1393-1403, kernel zero/kernels/ops_attn_g.cl:616-667): rows [0, T) of x become
+ * (x + rmsnorm(t) * w) * s in place, and the next matmul's input is made from the new rows: rmsnorm(x) * w2 (norm2) or x
+ * itself, quantized into the engine's activation buffers for Mp rows.  x, t: [T][K] f32; w, w2: [K] f32 (w2 may be NULL
+ * without norm2). */
+int arcz_engine_add_norm_quant(arcz_engine* e, arcz_mem* x, arcz_mem* t, arcz_mem* w, int K, int T, int Mp, float s,
+                               arcz_mem* w2, int norm2, int act32, float eps);
 /* Activations quantized by the caller, as the reference's benches do (bench/gemv_bench.cpp:103-129). */
 int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp,
                                 int T);
@@ -87,6 +93,9 @@ int arcz_engine_self_check(void);
 void arcz_engine_profile(arcz_engine* e, int on);
 int arcz_engine_profile_collect(arcz_engine* e);
 int arcz_engine_profile_get(arcz_engine* e, const char* name, double* ms, int* launches);
+/* Minimum and median of the collected per-launch times of `name` (the reference's benches print median and minimum,
+ * bench/gemv_bench.cpp:215-229). */
+int arcz_engine_profile_stats(arcz_engine* e, const char* name, double* min_ms, double* median_ms);
 void arcz_engine_profile_reset(arcz_engine* e);
 uint64_t arcz_engine_rd_bytes(arcz_engine* e);
 

@@ -111,3 +111,56 @@ def test_producer_feeds_matmul(eng):
         assert rel_err_rows(y, ref).max() <= 1e-3
         cb.free(); xb.free()
     w.free(); nwb.free()
+
+
+@pytest.mark.parametrize("T,Mp,K,norm2,s", [(1, 16, 5120, True, 1.0), (4, 16, 2048, False, 0.5), (8, 16, 17408 // 4, True, 0.75),
+                                            (100, 128, 1024, True, 1.0), (300, 512, 768, False, 1.0)])
+def test_add_norm_quant(rt, T, Mp, K, norm2, s):
+    """x = (x + rmsnorm(t) * w) * s in place, then the next input from the new x (reference zero/kernels/ops_attn_g.cl:
+    616-667).  The new x against float64 (1e-6); with norm2 off the quantized rows are the quantizer's, bit for bit, of
+    the x the GPU stored; with norm2 on the scales agree to 1e-6 and the int8 values differ by at most one level in at
+    most 0.1 % of places (the row's second sum of squares is taken in the kernel's own order)."""
+    print(f"add_norm_quant T={T} Mp={Mp} K={K} norm2={norm2} s={s}", flush=True)
+    e = az.Engine(512, 5120)
+    try:
+        eps = 1e-6
+        x = make_acts(T, K, seed=400 + T)
+        t = (3.0 * az.gen_normal(401 + T, (T, K))).astype(np.float32)
+        w = (1.0 + 0.1 * az.gen_normal(402, (K,))).astype(np.float32)
+        w2 = (1.0 + 0.1 * az.gen_normal(403, (K,))).astype(np.float32)
+        xb, tb, wb, w2b = (az.Runtime.from_numpy(a) for a in (x, t, w, w2))
+        poison(e)
+        e.add_norm_quant(xb, tb, wb, K, T, Mp, s, w2b if norm2 else None, norm2, eps)
+        rows = T if T <= 8 else Mp
+        xn = xb.read(np.float32, T * K).reshape(T, K)
+        t64 = t.astype(np.float64)
+        ref = (x.astype(np.float64) + t64 / np.sqrt((t64 * t64).mean(axis=1, keepdims=True) + eps) * w) * s
+        assert np.abs(xn - ref).max() <= 1e-6 * np.abs(ref).max()
+        aq, asc, absum = e.read_activations(K, Mp)
+        if norm2:
+            x64 = xn.astype(np.float64)
+            v = (x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps) * w2).astype(np.float32)
+        else:
+            v = xn
+        raq, rasc, rabsum = orc.quantize_act(pad_rows(np.ascontiguousarray(v), rows))
+        if norm2:
+            assert np.abs(asc[:, :rows] - rasc).max() <= 1e-6 * np.abs(rasc).max()
+            d = np.abs(aq[:rows].astype(np.int32) - raq.astype(np.int32))
+            assert d.max() <= 1 and (d != 0).mean() <= 1e-3
+            assert np.array_equal(absum[:, :rows].T.reshape(rows, K // 16),
+                                  aq[:rows].astype(np.int32).reshape(rows, K // 16, 16).sum(axis=2))
+        else:
+            assert np.array_equal(aq[:rows], raq)
+            assert np.array_equal(asc[:, :rows].view(np.uint32), rasc.view(np.uint32))
+            assert np.array_equal(absum[:, :rows], rabsum)
+        if rows > T:
+            assert not aq[T:rows].any()
+        # the quantized rows feed the next matmul: a second call on the same inputs gives the same bits
+        xb2 = az.Runtime.from_numpy(x)
+        e.add_norm_quant(xb2, tb, wb, K, T, Mp, s, w2b if norm2 else None, norm2, eps)
+        aq2, asc2, _ = e.read_activations(K, Mp)
+        assert np.array_equal(aq2[:rows], aq[:rows]) and np.array_equal(asc2[:, :rows].view(np.uint32), asc[:, :rows].view(np.uint32))
+        for b in (xb, xb2, tb, wb, w2b):
+            b.free()
+    finally:
+        e.close()
