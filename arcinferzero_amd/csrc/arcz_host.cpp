@@ -4,12 +4,14 @@
 // tensors (weights ~ N(0, 0.02) quantized to Q4_K / Q6_K / Q8_0, activations ~ N(0, 1)) that the benchmark and the
 // tests share.  The Q4_K / Q6_K quantizers have no counterpart in the reference (it only reads those types): they
 // make valid blocks from random values and are input generators, not part of the compute path.
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
 #include <vector>
 
 #include "kernels/common.h"
+#define GGML_TYPE_Q4_0 2u  // (GGUF type id, src/gguf.h:19)
 
 namespace {
 
@@ -66,9 +68,12 @@ extern "C" {
 
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
-  return type == QT_Q4_K ? u * 144 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : 0;
+  return type == QT_Q4_K ? u * 144 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : 0;
 }
-size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) { return raw_planes_bytes((int)type, rows, K / 256); }
+// (Q4_0 rows are kept on the device as Q8_0 planes: see arcz_repack_planes)
+size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) {
+  return raw_planes_bytes(type == GGML_TYPE_Q4_0 ? QT_Q8_0 : (int)type, rows, K / 256);
+}
 
 // GGUF rows -> device planes (layout: kernels/common.h).  0 or -1 (unsupported type / K).
 int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, uint8_t* dst) {
@@ -116,6 +121,24 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
       for (int b = 0; b < 8; ++b) {
         memcpy(dst + pl.d + i * 16 + 2 * b, src + i * 272 + 34 * b, 2);
         memcpy(dst + pl.qs + i * 256 + 32 * b, src + i * 272 + 34 * b + 2, 32);
+      }
+    return 0;
+  }
+  if (type == GGML_TYPE_Q4_0) {
+    // Q4_0 is Q8_0 with q - 8 in four bits (reference src/quants.h:136-148: 18-byte blocks, f16 d, low nibbles =
+    // elements 0..15, high = 16..31): written out as Q8_0 planes, value for value, so every Q8_0 kernel serves it
+    // exactly, at 34 instead of 18 bytes per block on the device.
+    const PlanesQ80 pl = planes_q80(rows, nsb);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i)
+      for (int b = 0; b < 8; ++b) {
+        const uint8_t* blk = src + i * 144 + 18 * b;
+        memcpy(dst + pl.d + i * 16 + 2 * b, blk, 2);
+        int8_t* q = (int8_t*)(dst + pl.qs + i * 256 + 32 * b);
+        for (int e = 0; e < 16; ++e) {
+          q[e] = (int8_t)((blk[2 + e] & 0xF) - 8);
+          q[16 + e] = (int8_t)((blk[2 + e] >> 4) - 8);
+        }
       }
     return 0;
   }
@@ -247,10 +270,31 @@ void arcz_quantize_q6_k(const float* src, size_t N, int K, uint8_t* out) {
   }
 }
 
-// Quantizes f32 rows to `type` (8, 12, 14).  0 or -1.
+// f32 rows -> GGUF Q4_0 blocks the way the reference makes them (src/quants.h:444-463, llama.cpp's
+// quantize_row_q4_0_ref): d = (the value of largest magnitude) / -8, q = min(15, (int)(v / d + 8.5)).
+static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < (int64_t)(N * (size_t)(K / 32)); ++b) {
+    const float* v = src + b * 32;
+    float amax = 0.0f, mx = 0.0f;
+    for (int i = 0; i < 32; ++i)
+      if (std::fabs(v[i]) > amax) { amax = std::fabs(v[i]); mx = v[i]; }
+    const float d = mx / -8.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
+    uint8_t* blk = out + b * 18;
+    const uint16_t dh = f32_to_f16(d);
+    memcpy(blk, &dh, 2);
+    for (int i = 0; i < 16; ++i) {
+      const int q0 = std::min(15, (int)(v[i] * id + 8.5f)), q1 = std::min(15, (int)(v[i + 16] * id + 8.5f));
+      blk[2 + i] = (uint8_t)(q0 | (q1 << 4));
+    }
+  }
+}
+
+// Quantizes f32 rows to `type` (2, 8, 12, 14).  0 or -1.
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
   if (K <= 0 || K % 256) return -1;
-  if (type == QT_Q8_0) arcz_quantize_q8_0(src, N, K, out);
+  if (type == GGML_TYPE_Q4_0) arcz_quantize_q4_0(src, N, K, out);
+  else if (type == QT_Q8_0) arcz_quantize_q8_0(src, N, K, out);
   else if (type == QT_Q4_K) arcz_quantize_q4_k(src, N, K, out);
   else if (type == QT_Q6_K) arcz_quantize_q6_k(src, N, K, out);
   else return -1;

@@ -12,6 +12,7 @@
 #include "clrt_hip.h"
 #include "kernels/common.h"
 
+#define GGML_Q4_0 2u
 #define GGML_Q8_0 8u
 #define GGML_Q4_K 12u
 #define GGML_Q6_K 14u
@@ -106,7 +107,7 @@ class Engine {
   // device planes on the host, then one upload.  rows = N for a matrix, n_expert * N for an expert tensor.
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
-    if (type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q6_K)
+    if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q6_K)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
     if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))
@@ -115,11 +116,12 @@ class Engine {
       throw std::runtime_error("make_weight: " + std::to_string(nbytes) + " bytes given, " +
                                std::to_string(arcz_gguf_bytes(type, rows, K)) + " expected");
     GpuWeight w;
-    w.type = type;
+    // (Q4_0 rows become Q8_0 planes on upload, value for value -- arcz_repack_planes -- and run through the Q8_0 kernels)
+    w.type = type == GGML_Q4_0 ? GGML_Q8_0 : type;
     w.N = N;
     w.K = K;
     w.rows = rows;
-    const size_t pb = raw_planes_bytes((int)type, rows, K / 256);
+    const size_t pb = raw_planes_bytes((int)w.type, rows, K / 256);
     std::vector<uint8_t> planes(pb);
     if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
     w.raw = buf(pb, planes.data());

@@ -14,6 +14,7 @@
  *                                       golden vectors and live comparison with the compiled reference header
  *   orc_quantize_act                    closed forms (max -> +-127, zero block, ties to even); golden + compiled ref
  *   orc_quantize_rows_q8_0              golden + compiled ref; round trip bound
+ *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
  *   orc_block_sums                      brute-force integer sums in numpy (int64)
  *   orc_matmul_ref                      numpy float64 dot of dequantized rows; unit-scale known answer
  *   orc_matmul_formula                  against orc_matmul_ref within float rounding; unit-scale known answer (exact)
@@ -32,7 +33,10 @@
 #include <omp.h>
 #endif
 
+#define ORC_Q4_0 2u
 #define ORC_Q8_0 8u
+/* Q4_0 is Q8_0 with q - 8 in four bits (src/quants.h:136): everything after the decode treats the two alike */
+#define ORC_Q8LIKE(t) ((t) == ORC_Q8_0 || (t) == ORC_Q4_0)
 #define ORC_Q4_K 12u
 #define ORC_Q6_K 14u
 
@@ -91,6 +95,7 @@ uint16_t orc_f32_to_fp16(float x) {
 int orc_sb_bytes(uint32_t type) {
   switch (type) {
     case ORC_Q8_0: return 34 * 8;
+    case ORC_Q4_0: return 18 * 8;
     case ORC_Q4_K: return 144;
     case ORC_Q6_K: return 210;
     default: return 0;
@@ -161,6 +166,18 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
     }
     return 0;
   }
+  if (type == ORC_Q4_0) { /* 8 blocks of 18 bytes: f16 d, low nibbles = elements 0..15, high = 16..31, q - 8
+                             (src/quants.h:136-148) */
+    for (int b = 0; b < 8; ++b) {
+      const uint8_t* blk = p + 18 * b;
+      o->d8[b] = orc_fp16_to_f32(rd16(blk));
+      for (int i = 0; i < 16; ++i) {
+        o->q[32 * b + i] = (int16_t)((blk[2 + i] & 0xF) - 8);
+        o->q[32 * b + 16 + i] = (int16_t)((blk[2 + i] >> 4) - 8);
+      }
+    }
+    return 0;
+  }
   return -1;
 }
 
@@ -203,7 +220,7 @@ int orc_decode_row_fields(uint32_t type, const uint8_t* row, int K, int8_t* q, i
       imn[s * 16 + h] = type == ORC_Q4_K ? o.mn[h / 2] : 0;
     }
     for (int b = 0; b < 8; ++b) {
-      d[s * 8 + b] = type == ORC_Q8_0 ? o.d8[b] : o.d;
+      d[s * 8 + b] = ORC_Q8LIKE(type) ? o.d8[b] : o.d;
       dmin[s * 8 + b] = type == ORC_Q4_K ? o.dmin : 0.0f;
     }
   }
@@ -268,6 +285,28 @@ void orc_quantize_rows_q8_0(const float* src, int N, int K, uint8_t* out) {
     for (int i = 0; i < 32; ++i) {
       const float p = v[i] * inv;
       blk[2 + i] = (uint8_t)(int8_t)lrintf(p);
+    }
+  }
+}
+
+/* f32 rows [N][K] -> GGUF Q4_0 blocks as llama.cpp's quantize_row_q4_0_ref: d = (the value of largest magnitude) / -8,
+ * q = min(15, (int)(v / d + 8.5)), element i in the low nibble of byte i, element i + 16 in the high
+ * (src/quants.h:444-463). out: N * K/32 * 18 bytes. */
+void orc_quantize_rows_q4_0(const float* src, int N, int K, uint8_t* out) {
+  for (size_t b = 0; b < (size_t)N * (size_t)(K / 32); ++b) {
+    const float* v = src + b * 32;
+    float amax = 0, mx = 0;
+    for (int i = 0; i < 32; ++i)
+      if (fabsf(v[i]) > amax) { amax = fabsf(v[i]); mx = v[i]; }
+    const float d = mx / -8.0f, id = d != 0 ? 1.0f / d : 0.0f;
+    uint8_t* blk = out + b * 18;
+    const uint16_t dh = orc_f32_to_fp16(d);
+    memcpy(blk, &dh, 2);
+    for (int i = 0; i < 16; ++i) {
+      int q0 = (int)(v[i] * id + 8.5f), q1 = (int)(v[i + 16] * id + 8.5f);
+      if (q0 > 15) q0 = 15;
+      if (q1 > 15) q1 = 15;
+      blk[2 + i] = (uint8_t)(q0 | (q1 << 4));
     }
   }
 }
@@ -388,7 +427,7 @@ int orc_matmul_formula(uint32_t type, int form, const uint8_t* W, int N, int K, 
             }
           }
           if (form == 1) {
-            if (type == ORC_Q8_0) {
+            if (ORC_Q8LIKE(type)) {
               res = fmaf(sa2[0] * o.d8[2 * j], t2[0], fmaf(sa2[1] * o.d8[2 * j + 1], t2[1], res));
             } else {
               tq = fmaf(sa2[0], t2[0], fmaf(sa2[1], t2[1], tq));

@@ -35,6 +35,10 @@ void ref_quantize_rows_q8_0(const float* src, int N, int K, uint8_t* out) {
   const std::vector<uint8_t> v = quantize_rows_q8_0(src, N, K);
   memcpy(out, v.data(), v.size());
 }
+void ref_quantize_rows_q4_0(const float* src, int N, int K, uint8_t* out) {
+  const std::vector<uint8_t> v = quantize_rows_q4_0(src, N, K);
+  memcpy(out, v.data(), v.size());
+}
 // the reference's GPU raw form of one superblock (src/quants.h gpu_raw_sb), to compare layouts in tests
 int ref_raw_padded_sb_bytes(uint32_t type) { return raw_padded_sb_bytes(type); }
 void ref_gpu_raw_sb(uint32_t type, const uint8_t* src, uint8_t* dst) { gpu_raw_sb(type, src, dst); }

@@ -9,8 +9,8 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-SB_BYTES = {Q8_0: 272, Q4_K: 144, Q6_K: 210}
+Q4_0, Q8_0, Q4_K, Q6_K = 2, 8, 12, 14
+SB_BYTES = {Q4_0: 144, Q8_0: 272, Q4_K: 144, Q6_K: 210}
 
 _p, _i = C.c_void_p, C.c_int
 
@@ -99,6 +99,14 @@ def quantize_rows_q8_0(w, lib=None):
     N, K = w.shape
     out = np.empty(N * (K // 32) * 34, np.uint8)
     (orc.orc_quantize_rows_q8_0 if lib is None else lib.ref_quantize_rows_q8_0)(ptr(w), _i(N), _i(K), ptr(out))
+    return out
+
+
+def quantize_rows_q4_0(w, lib=None):
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    N, K = w.shape
+    out = np.empty(N * (K // 32) * 18, np.uint8)
+    (orc.orc_quantize_rows_q4_0 if lib is None else lib.ref_quantize_rows_q4_0)(ptr(w), _i(N), _i(K), ptr(out))
     return out
 
 

@@ -8,6 +8,7 @@ import os
 import numpy as np
 import pytest
 
+import arcinferzero_amd as az
 import oracle_lib as orc
 from common import TYPES, make_acts, make_weights, rel_err_rows, unit_scale_acts, unit_scale_weights
 
@@ -129,6 +130,58 @@ def test_q80_closed_form():
             blk[b, 2 + i] = np.int8(q).view(np.uint8)
             exp[32 * b + i] = d * q
     assert np.array_equal(orc.dequant_rows(Q8_0, blk.reshape(-1), 1, K)[0], exp)
+
+
+def test_q40_closed_form_and_quantizer():
+    """Q4_0 (src/quants.h:136-148, 444-463): blocks made by hand decode to d * (q - 8); the quantizer on values that
+    are exact multiples of a power-of-two step, with the extreme at -8 steps, returns exactly those nibbles; a zero
+    block gives d = 0 and the nibble 8 everywhere; element i sits in the low nibble of byte i, i + 16 in the high."""
+    K = 256
+    blk = np.zeros((8, 18), np.uint8)
+    exp = np.zeros(K, np.float32)
+    for b in range(8):
+        d = [0.0, 0.25, -0.5, 2.0][b % 4]
+        blk[b, 0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+        for i in range(16):
+            q0, q1 = (i * 5 + b) % 16, (i * 11 + 3 * b + 1) % 16
+            blk[b, 2 + i] = q0 | (q1 << 4)
+            exp[32 * b + i] = d * (q0 - 8)
+            exp[32 * b + 16 + i] = d * (q1 - 8)
+    assert np.array_equal(orc.dequant_rows(az.Q4_0, blk.reshape(-1), 1, K)[0], exp)
+    rng = np.random.default_rng(4)
+    q = rng.integers(1, 16, size=(4, K)).astype(np.int32)
+    q.reshape(4, 8, 32)[:, :, 7] = 0            # the extreme of every block: -8 steps
+    step = 0.125
+    w = ((q - 8) * step).astype(np.float32)
+    w[3, 32:64] = 0.0                           # a zero block
+    out = orc.quantize_rows_q4_0(w).reshape(4, 8, 18)
+    d = out[:, :, 0:2].copy().view(np.float16).astype(np.float32)[..., 0]
+    lo, hi = (out[:, :, 2:] & 0xF).astype(np.int32), (out[:, :, 2:] >> 4).astype(np.int32)
+    got = np.concatenate([lo, hi], axis=2)
+    want = q.reshape(4, 8, 32).copy()
+    want[3, 1] = 8
+    assert np.array_equal(got, want)
+    want_d = np.full((4, 8), step, np.float32)
+    want_d[3, 1] = 0.0
+    assert np.array_equal(d, want_d)
+    assert np.array_equal(orc.dequant_rows(az.Q4_0, out.reshape(-1), 4, K), w)
+
+
+@pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
+def test_q40_vs_compiled_reference():
+    w = (make_acts(16, 512, seed=8) * 0.02).astype(np.float32)
+    a, b = orc.quantize_rows_q4_0(w), orc.quantize_rows_q4_0(w, lib=orc.ref)
+    assert np.array_equal(a, b)
+    assert np.array_equal(orc.dequant_rows(az.Q4_0, a, 16, 512).view(np.uint32),
+                          orc.dequant_rows(az.Q4_0, a, 16, 512, lib=orc.ref).view(np.uint32))
+    # the product's own generator makes the same blocks as the reference's quantizer, and its device planes hold
+    # exactly the values the reference decodes
+    assert np.array_equal(az.quantize_rows(az.Q4_0, w), b)
+    planes = az.repack_planes(az.Q4_0, 16, 512, a)
+    nsb = 2
+    qs = planes[:16 * nsb * 256].view(np.int8).reshape(16, nsb * 8, 32).astype(np.float32)
+    dd = planes[16 * nsb * 256:16 * nsb * 256 + 16 * nsb * 16].view(np.float16).reshape(16, nsb * 8, 1).astype(np.float32)
+    assert np.array_equal((qs * dd).reshape(16, 512), orc.dequant_rows(az.Q4_0, a, 16, 512))
 
 
 # ---------------------------------------------------------------- quantizers
