@@ -2,7 +2,7 @@
 """Benchmark of the block-quantized matmul path on one MI355X.
 
 A step is one pass of the hot path over one prompt chunk: activation quantization (f32 -> int8 per 32) followed by the
-Q4_K prefill GEMM of BASELINE.json's config 2 (weights 17408 x 5120 Q4_K, 8192 tokens).  Inputs are resident in HBM
+Q4_K prefill GEMM of the benchmark definition's second configuration (weights 17408 x 5120 Q4_K, 8192 tokens).  Inputs are resident in HBM
 when the timed region starts.  One JSON line is printed: the GEMM throughput in int8 TOP/s (2*M*N*K per step), the
 roofline of the dominant kernel from per-launch HIP events, the decode GEMV bandwidth of config 3 as extra fields, and
 the CPU baseline (the oracle's restatement of the reference's dequant + f32 matmul) timed on this host's cores.
@@ -165,7 +165,7 @@ def bench_gemm_config(az, qtype, N, K, M, launches, seed, W=None):
 
 
 def bench_moe(az, launches):
-    """BASELINE configs[4]: 128 experts, top-8, 4096 tokens, hidden 2048, expert FFN 768, Q4_K; the whole layer
+    """The MoE configuration (configs[4] of the benchmark definition): 128 experts, top-8, 4096 tokens, hidden 2048, expert FFN 768, Q4_K; the whole layer
     (route, sort, gate/up tile GEMM with SwiGLU, expert-input quantization, down tile GEMM, combine) per launch."""
     NE, NU, T, E, F, qt = 128, 8, 4096, 2048, 768, az.Q4_K
     eng = az.Engine(T, E)
@@ -327,7 +327,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": pre["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8 x int8 -> int32 block sums, f32 scale application", "data": "synthetic",
         "config": {"workload": "Q4_K dense prefill GEMM: weights 17408x5120 Q4_K, activations 8192x5120 f32 "
-                               "quantized to int8 per 32 in the step, out 8192x17408 f32 (BASELINE configs[1])",
+                               "quantized to int8 per 32 in the step, out 8192x17408 f32 (configs[1] of the benchmark definition)",
                    "M": M, "N": N, "K": K, "step": "quant_rows + gemm"},
         "roofline": {"bound": "mfma", "achieved": pre["kernel_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": pre["kernel_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH,

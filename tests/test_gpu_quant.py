@@ -63,7 +63,7 @@ def test_quant_special_blocks(eng):
 
 
 def test_quant_full_config_sizes(eng, rt):
-    """BASELINE config 2's activation shape through size-independent properties: the row of maximum magnitude of
+    """The headline configuration's activation shape (8192 x 5120) through size-independent properties: the row of maximum magnitude of
     every block maps to +-127, sums are the sums of the int8 values, padding rows are zero; and equality with the
     oracle on a sample of rows."""
     big = az.Engine(8192, 5120)
