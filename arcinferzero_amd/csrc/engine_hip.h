@@ -453,7 +453,7 @@ class Engine {
       cl_mem sh = nullptr;
       int EE = E;
       set_args(k, 0, x, sh, sgate_, my_, minv_, EE);
-      size_t gws[2] = {((size_t)E + 255) / 256 * 256, (size_t)T}, lws[2] = {256, 1};
+      size_t gws[2] = {((size_t)E + 1023) / 1024 * 256, (size_t)T}, lws[2] = {256, 1};  // (four columns a thread)
       run("moe_combine", k, 2, gws, lws);
     }
   }
