@@ -68,7 +68,7 @@ extern "C" {
 
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
-  return type == QT_Q4_K ? u * 144 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : 0;
+  return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : 0;
 }
 // (Q4_0 rows are kept on the device as Q8_0 planes: see arcz_repack_planes)
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) {
@@ -80,15 +80,17 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
   if (K <= 0 || K % 256) return -1;
   const int nsb = K / 256;
   const int64_t u = (int64_t)rows * nsb;
-  if (type == QT_Q4_K) {
+  if (type == QT_Q4_K || type == QT_Q5_K) {
     const PlanesQ4K pl = planes_q4k(rows, nsb);
+    const bool q5 = type == QT_Q5_K;
+    const size_t sbb = q5 ? 176 : 144;
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < u; ++i) {
       // header: d, dmin, then the 6-bit scales and mins (GGUF packing, reference src/quants.h:61-69) regrouped as
       // eight 12-bit entries sc | mn << 6
-      const uint8_t* q = src + i * 144 + 4;
+      const uint8_t* q = src + i * sbb + 4;
       uint8_t* h = dst + pl.hdr + i * 16;
-      memcpy(h, src + i * 144, 4);
+      memcpy(h, src + i * sbb, 4);
       uint32_t w[3] = {0, 0, 0};
       for (int b = 0; b < 8; ++b) {
         const uint32_t sc = b < 4 ? (q[b] & 63u) : ((q[b + 4] & 0xFu) | ((uint32_t)(q[b - 4] >> 6) << 4));
@@ -98,7 +100,25 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
         if (((12 * b) >> 5) < 2) w[((12 * b) >> 5) + 1] |= (uint32_t)(e >> 32);
       }
       memcpy(h + 4, w, 12);
-      memcpy(dst + pl.qs + i * 128, src + i * 144 + 16, 128);
+      memcpy(dst + pl.qs + i * 128, src + i * sbb + (q5 ? 48 : 16), 128);
+      if (q5) {
+        // fifth bits (reference src/quants.h:101-108: bit b of byte l of qh = element 32 b + l) regrouped per 16-byte
+        // unit of nibbles: unit 2 j + half holds bytes l = 16 half .. 16 half + 15 of chunk j, low nibbles = block 2 j,
+        // high nibbles = block 2 j + 1; byte m = 4 k + c of the unit gives bits 4 + k and k of byte c of the word
+        const uint8_t* qh = src + i * sbb + 16;
+        uint32_t H[8];
+        for (int un = 0; un < 8; ++un) {
+          const int j = un >> 1, half = un & 1;
+          uint32_t word = 0;
+          for (int m = 0; m < 16; ++m) {
+            const int l = 16 * half + m, k = m >> 2, c = m & 3;
+            word |= (uint32_t)((qh[l] >> (2 * j)) & 1) << (8 * c + 4 + k);
+            word |= (uint32_t)((qh[l] >> (2 * j + 1)) & 1) << (8 * c + k);
+          }
+          H[un] = word;
+        }
+        memcpy(dst + pl.qh + i * 32, H, 32);
+      }
     }
     return 0;
   }
@@ -231,6 +251,60 @@ void arcz_quantize_q4_k(const float* src, size_t N, int K, uint8_t* out) {
   }
 }
 
+// f32 rows -> GGUF Q5_K superblocks (176 bytes per 256 values): as Q4_K with 31 steps per block; the fifth bit of
+// element 32 b + l is bit b of byte l of the 32 bytes between the scales and the nibbles (reference
+// src/quants.h:101-108).
+void arcz_quantize_q5_k(const float* src, size_t N, int K, uint8_t* out) {
+  const int64_t nsbt = (int64_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < nsbt; ++s) {
+    const float* v = src + s * 256;
+    uint8_t* p = out + s * 176;
+    float step[8], off[8], smax = 0, omax = 0;
+    for (int b = 0; b < 8; ++b) {
+      float lo = 0, hi = 0;
+      for (int i = 0; i < 32; ++i) { lo = std::fmin(lo, v[32 * b + i]); hi = std::fmax(hi, v[32 * b + i]); }
+      step[b] = (hi - lo) / 31.0f;
+      off[b] = -lo;
+      smax = std::fmax(smax, step[b]);
+      omax = std::fmax(omax, off[b]);
+    }
+    const uint16_t dh = f32_to_f16(smax / 63.0f), mh = f32_to_f16(omax / 63.0f);
+    const float d = f16_to_f32(dh), dmin = f16_to_f32(mh);
+    int sc[8], mn[8];
+    for (int b = 0; b < 8; ++b) {
+      sc[b] = d > 0 ? std::min(63, std::max(0, (int)std::lrintf(step[b] / d))) : 0;
+      mn[b] = dmin > 0 ? std::min(63, std::max(0, (int)std::lrintf(off[b] / dmin))) : 0;
+    }
+    memcpy(p, &dh, 2);
+    memcpy(p + 2, &mh, 2);
+    uint8_t* q = p + 4;
+    memset(q, 0, 12 + 32);
+    for (int j = 0; j < 8; ++j) {
+      if (j < 4) {
+        q[j] |= sc[j] & 63;
+        q[j + 4] |= mn[j] & 63;
+      } else {
+        q[j + 4] = (uint8_t)((sc[j] & 0xF) | ((mn[j] & 0xF) << 4));
+        q[j - 4] |= (uint8_t)((sc[j] >> 4) << 6);
+        q[j] |= (uint8_t)((mn[j] >> 4) << 6);
+      }
+    }
+    uint8_t *qh = p + 16, *qs = p + 48;
+    for (int j = 0; j < 4; ++j)
+      for (int l = 0; l < 32; ++l) {
+        int qq[2];
+        for (int h = 0; h < 2; ++h) {
+          const int b = 2 * j + h;
+          const float sd = d * (float)sc[b], x = v[64 * j + 32 * h + l] + dmin * (float)mn[b];
+          qq[h] = sd > 0 ? std::min(31, std::max(0, (int)std::lrintf(x / sd))) : 0;
+          qh[l] |= (uint8_t)((qq[h] >> 4) << b);
+        }
+        qs[32 * j + l] = (uint8_t)((qq[0] & 15) | ((qq[1] & 15) << 4));
+      }
+  }
+}
+
 // f32 rows -> GGUF Q6_K superblocks (210 bytes per 256 values): per 16 values a step amax / 31, rounded to int8
 // against d = max step / 127 (fp16); q = rte(v / (d * sc)) in -32..31, stored + 32 (reference src/quants.h:115-134).
 void arcz_quantize_q6_k(const float* src, size_t N, int K, uint8_t* out) {
@@ -290,12 +364,13 @@ static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) 
   }
 }
 
-// Quantizes f32 rows to `type` (2, 8, 12, 14).  0 or -1.
+// Quantizes f32 rows to `type` (2, 8, 12, 13, 14).  0 or -1.
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
   if (K <= 0 || K % 256) return -1;
   if (type == GGML_TYPE_Q4_0) arcz_quantize_q4_0(src, N, K, out);
   else if (type == QT_Q8_0) arcz_quantize_q8_0(src, N, K, out);
   else if (type == QT_Q4_K) arcz_quantize_q4_k(src, N, K, out);
+  else if (type == QT_Q5_K) arcz_quantize_q5_k(src, N, K, out);
   else if (type == QT_Q6_K) arcz_quantize_q6_k(src, N, K, out);
   else return -1;
   return 0;

@@ -15,6 +15,7 @@
 #define GGML_Q4_0 2u
 #define GGML_Q8_0 8u
 #define GGML_Q4_K 12u
+#define GGML_Q5_K 13u
 #define GGML_Q6_K 14u
 
 extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
@@ -29,7 +30,7 @@ struct GpuWeight {
 };
 
 inline const char* ggml_type_name(uint32_t t) {
-  return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q6_K ? "Q6_K" : "?";
+  return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : "?";
 }
 
 class Engine {
@@ -107,7 +108,7 @@ class Engine {
   // device planes on the host, then one upload.  rows = N for a matrix, n_expert * N for an expert tensor.
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
-    if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q6_K)
+    if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
     if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))
@@ -248,7 +249,7 @@ class Engine {
       // The main kernels stage the tokens' activations in LDS (gemv / gemv_mt); when T tokens of K values do not fit
       // the 64 KiB a launch may ask for, the kernels that read them from global memory take over (gemv_v / gemv_mt_v).
       const int ups = w.type == GGML_Q8_0 ? 16 : 8, units = K / 256 * ups;
-      const int tok_bytes = (w.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (w.type == GGML_Q4_K ? 8 : 4));
+      const int tok_bytes = (w.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (w.type == GGML_Q4_K || w.type == GGML_Q5_K ? 8 : 4));
       static const int force_v = getenv("ARCZ_GEMV_V") ? atoi(getenv("ARCZ_GEMV_V")) : 0;
       // lanes per row: the fewest of 32 / 64 / 128 / 256 that leave a lane at most 6 sixteen-byte units of a row
       static const int force_lpr = getenv("ARCZ_GEMV_LPR") ? atoi(getenv("ARCZ_GEMV_LPR")) : 0;

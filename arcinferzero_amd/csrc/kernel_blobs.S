@@ -12,6 +12,7 @@
     BLOB arcz_blob_decode, "decode.hsaco"
     BLOB arcz_blob_decode_q80, "decode_q80.hsaco"
     BLOB arcz_blob_decode_q4k, "decode_q4k.hsaco"
+    BLOB arcz_blob_decode_q5k, "decode_q5k.hsaco"
     BLOB arcz_blob_decode_q6k, "decode_q6k.hsaco"
     BLOB arcz_blob_gemm, "gemm.hsaco"
     BLOB arcz_blob_moe, "moe.hsaco"

@@ -14,6 +14,7 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 // GGUF type ids (reference src/gguf.h:18-22)
 #define QT_Q8_0 8
 #define QT_Q4_K 12
+#define QT_Q5_K 13
 #define QT_Q6_K 14
 
 // ---- device weight layout ("raw planes").  A matrix of R rows x K columns (K % 256 == 0, nsb = K / 256) is held
@@ -24,11 +25,16 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 //          hdr [R][nsb][16]   (f16 d, f16 dmin, then eight 12-bit entries sc_b | mn_b << 6 at bit 12 b: the 6-bit scale
 //                              and min of sub-block b, regrouped from GGUF's packing so that the pair of entries of a
 //                              64-element chunk is one 24-bit field)
+//   Q5_K : qs and hdr as Q4_K (the low four bits of each value), then
+//          qh  [R][nsb][8] words: word i holds the fifth bits of the 32 values of 16-byte unit i of qs, regrouped from
+//                              GGUF's 32 bytes (bit b of byte l = element 32 b + l) so that a shift and one mask put
+//                              them in place: byte c of the word, bit 4 + k = the low-nibble value of the unit's byte
+//                              4 k + c, bit k = the high-nibble value of that byte (k = 0..3)
 //   Q6_K : ql  [R][nsb][128], qh [R][nsb][64], sc [R][nsb][16] (int8), d [R][nsb] (f16)
 //   Q8_0 : qs  [R][nsb][256] (int8), d [R][nsb][8] (f16)
 // Plane offsets from the start of the buffer, in bytes (each a multiple of 256 when R * nsb is a multiple of 16;
 // always a multiple of 16 otherwise except as noted).
-struct PlanesQ4K { size_t qs, hdr; };
+struct PlanesQ4K { size_t qs, hdr, qh; };  // (qh: Q5_K only)
 struct PlanesQ6K { size_t ql, qh, sc, d; };
 struct PlanesQ80 { size_t qs, d; };
 
@@ -37,6 +43,7 @@ __host__ __device__ inline PlanesQ4K planes_q4k(size_t rows, int nsb) {
   PlanesQ4K p;
   p.qs = 0;
   p.hdr = rows * (size_t)nsb * 128;
+  p.qh = rows * (size_t)nsb * 144;
   return p;
 }
 __host__ __device__ inline PlanesQ6K planes_q6k(size_t rows, int nsb) {
@@ -57,6 +64,7 @@ __host__ __device__ inline PlanesQ80 planes_q80(size_t rows, int nsb) {
 __host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb) {
   const size_t u = rows * (size_t)nsb;
   if (qt == QT_Q4_K) return u * 144;
+  if (qt == QT_Q5_K) return u * 176;
   if (qt == QT_Q6_K) return align16(u * 208 + u * 2);
   if (qt == QT_Q8_0) return u * 272;
   return 0;
@@ -80,6 +88,13 @@ __device__ inline void q4k_scales_pair(uint32_t s0, uint32_t s1, uint32_t s2, in
   mn0 = (g >> 6) & 63;
   sc1 = (g >> 12) & 63;
   mn1 = (g >> 18) & 63;
+}
+
+// Q5_K: word k (0..3) of a 16-byte unit of nibbles with the fifth bits from the unit's word H of the qh plane: the 16
+// values of the low nibbles, and of the high nibbles, as four bytes 0..31 each.
+__device__ inline uint32_t q5k_lo(uint32_t w, uint32_t H, int k) { return (w & 0x0F0F0F0Fu) | ((H >> k) & 0x10101010u); }
+__device__ inline uint32_t q5k_hi(uint32_t w, uint32_t H, int k) {
+  return ((w >> 4) & 0x0F0F0F0Fu) | ((H << (4 - k)) & 0x10101010u);
 }
 
 __device__ inline int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }

@@ -4,6 +4,7 @@
 // Arithmetic per 16-element half block h of weight row n and token t, as the reference's gemv
 // (zero/kernels/decode.cl:992-1003):  I = sum of 16 int8 x int8 products (v_dot4_i32_i8, exact int32);
 //   Q4_K : acc += sa * (d * (float)(sc * I) - dmin * (float)(mn * bs))      sa: the token's scale of the 32-block,
+//   Q5_K : as Q4_K, the values 0..31 (the fifth bits come from their own plane)
 //   Q6_K : acc += sa * d * (float)(sc16 * I)                                bs: its int16 sum of the 16 activations
 //   Q8_0 : acc += sa * d * (float)I
 // (the reference groups the two halves of a 32-block inside the int -> float conversion; here each half is converted
@@ -32,7 +33,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
 #pragma unroll
     for (int t = 0; t < TB; ++t) acc[r][t] = 0.0f;
 
-  if constexpr (QT == QT_Q4_K) {
+  if constexpr (QT == QT_Q4_K || QT == QT_Q5_K) {
     const PlanesQ4K pl = planes_q4k(plane_rows, nsb);
     const int j = (hl >> 1) & 3, half = hl & 1;
     for (int u = hl; u < units; u += 32) {
@@ -59,9 +60,14 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
         const float d = f16_bits_to_f32(h.x), dmin = f16_bits_to_f32(h.x >> 16);
         int sc0, sc1, mn0, mn1;
         q4k_scales_pair(h.y, h.z, h.w, j, sc0, sc1, mn0, mn1);
-        const uint32_t wl[4] = {w.x & 0x0F0F0F0Fu, w.y & 0x0F0F0F0Fu, w.z & 0x0F0F0F0Fu, w.w & 0x0F0F0F0Fu};
-        const uint32_t wh[4] = {(w.x >> 4) & 0x0F0F0F0Fu, (w.y >> 4) & 0x0F0F0F0Fu, (w.z >> 4) & 0x0F0F0F0Fu,
-                                (w.w >> 4) & 0x0F0F0F0Fu};
+        uint32_t wl[4] = {w.x & 0x0F0F0F0Fu, w.y & 0x0F0F0F0Fu, w.z & 0x0F0F0F0Fu, w.w & 0x0F0F0F0Fu};
+        uint32_t wh[4] = {(w.x >> 4) & 0x0F0F0F0Fu, (w.y >> 4) & 0x0F0F0F0Fu, (w.z >> 4) & 0x0F0F0F0Fu,
+                          (w.w >> 4) & 0x0F0F0F0Fu};
+        if constexpr (QT == QT_Q5_K) {  // the fifth bits of the unit's 32 values
+          const uint32_t H = *(const uint32_t*)(raw + pl.qh + (size_t)n * nsb * 32 + (size_t)u * 4), ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) { wl[k] = q5k_lo(ww[k], H, k); wh[k] = q5k_hi(ww[k], H, k); }
+        }
 #pragma unroll
         for (int t = 0; t < TB; ++t) {
           int ilo = dot4(wl[0], alo[t].x, 0);
@@ -195,4 +201,5 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
 
 GEMV_ALL(8)
 GEMV_ALL(12)
+GEMV_ALL(13)
 GEMV_ALL(14)

@@ -5,6 +5,7 @@
 // an exact int32 sum I[m][n][b] (v_mfma_i32_32x32x32_i8, accumulator cleared per block), then in f32
 //   Q8_0 : res += (sa[m][b] * d[n][b]) * (float)I
 //   Q4_K : res += (sa[m][b] * (d[n] * sc[n][b])) * (float)I  -  (sa[m][b] * (float)S[m][b]) * (dmin[n] * mn[n][b])
+//   Q5_K : as Q4_K (values 0..31)
 // with S the sum of the block's 32 int8 activations.  Blocks are added in K order.
 //
 // The scheme needs one f32 scale per (token, weight row, block), so the vector ALU, not the matrix pipe, bounds it.
@@ -42,8 +43,9 @@ struct alignas(16) Gemm2Lds {
 // The global loads of one K step, held in registers until the step before it has been computed.
 template <int QT> struct StepRegs {
   uint4 a[4];                        // 4 x 16 int8 activation values
-  uint4 w[QT == QT_Q4_K ? 2 : 4];    // packed weights
-  uint4 h;                           // Q4_K header of the thread's row (Q8_0: .x = two f16 scales)
+  uint4 w[QT == QT_Q8_0 ? 4 : 2];    // packed weights
+  uint32_t qh[2];                    // Q5_K: the words of fifth bits of the two 16-byte units above
+  uint4 h;                           // Q4_K / Q5_K header of the thread's row (Q8_0: .x = two f16 scales)
   float sa[4];                       // scale of the block whose first half the thread stages (even chunks only)
 };
 
@@ -60,13 +62,14 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
     r.a[i] = *(const uint4*)(aq + (size_t)m * K + e0 + 16 * c);
     r.sa[i] = asc[(size_t)(s * 8 + 4 * hh + (c >> 1)) * M + m];
   }
-  if constexpr (QT == QT_Q4_K) {
+  if constexpr (QT == QT_Q4_K || QT == QT_Q5_K) {
     const PlanesQ4K pl = planes_q4k(rows_total, nsb);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
       const int n = min(n0 + row, N - 1);
       r.w[i] = *(const uint4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 128 + 64 * hh + 16 * c);
+      if constexpr (QT == QT_Q5_K) r.qh[i] = *(const uint32_t*)(raw + pl.qh + ((row_base + n) * nsb + s) * 32 + 16 * hh + 4 * c);
     }
     const int n = min(n0 + (t >> 1), N - 1);
     r.h = *(const uint4*)(raw + pl.hdr + ((row_base + n) * nsb + s) * 16);
@@ -86,13 +89,14 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
 // Registers -> LDS: int8 values, decoded weights, the four scale vectors.  Rows past the tile carry zero scales.
 template <int QT>
 __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
+  constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
   const int t = threadIdx.x;
   int ssum[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int id = t + 256 * i, row = id >> 3, c = id & 7;
     *(uint4*)&L.act[row][16 * c] = r.a[i];
-    if constexpr (QT == QT_Q4_K) {
+    if constexpr (Q45) {
       int sh = dot4(r.a[i].x, 0x01010101u, 0);
       sh = dot4(r.a[i].y, 0x01010101u, sh);
       sh = dot4(r.a[i].z, 0x01010101u, sh);
@@ -102,18 +106,24 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
     if ((c & 1) == 0) {  // rows past the tile carry zero scales
       const float sa = L.rowmap[row] >= 0 ? r.sa[i] : 0.0f;
       L.sa[c >> 1][row] = sa;
-      if constexpr (QT == QT_Q4_K) L.u[c >> 1][row] = sa * (float)ssum[i];
+      if constexpr (Q45) L.u[c >> 1][row] = sa * (float)ssum[i];
     }
   }
-  if constexpr (QT == QT_Q4_K) {
+  if constexpr (Q45) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
       const uint4 w = r.w[i];
       const int off = 64 * (c >> 1) + 16 * (c & 1);
-      *(uint4*)&L.wq[row][off] = make_uint4(w.x & 0x0F0F0F0Fu, w.y & 0x0F0F0F0Fu, w.z & 0x0F0F0F0Fu, w.w & 0x0F0F0F0Fu);
-      *(uint4*)&L.wq[row][off + 32] = make_uint4((w.x >> 4) & 0x0F0F0F0Fu, (w.y >> 4) & 0x0F0F0F0Fu,
-                                                 (w.z >> 4) & 0x0F0F0F0Fu, (w.w >> 4) & 0x0F0F0F0Fu);
+      if constexpr (QT == QT_Q5_K) {
+        const uint32_t H = r.qh[i];
+        *(uint4*)&L.wq[row][off] = make_uint4(q5k_lo(w.x, H, 0), q5k_lo(w.y, H, 1), q5k_lo(w.z, H, 2), q5k_lo(w.w, H, 3));
+        *(uint4*)&L.wq[row][off + 32] = make_uint4(q5k_hi(w.x, H, 0), q5k_hi(w.y, H, 1), q5k_hi(w.z, H, 2), q5k_hi(w.w, H, 3));
+      } else {
+        *(uint4*)&L.wq[row][off] = make_uint4(w.x & 0x0F0F0F0Fu, w.y & 0x0F0F0F0Fu, w.z & 0x0F0F0F0Fu, w.w & 0x0F0F0F0Fu);
+        *(uint4*)&L.wq[row][off + 32] = make_uint4((w.x >> 4) & 0x0F0F0F0Fu, (w.y >> 4) & 0x0F0F0F0Fu,
+                                                   (w.z >> 4) & 0x0F0F0F0Fu, (w.w >> 4) & 0x0F0F0F0Fu);
+      }
     }
     {
       const int row = t >> 1, p = t & 1;
@@ -204,7 +214,7 @@ __device__ inline void gemm2_body(const uint8_t* __restrict__ raw, const signed 
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const bool more = b + 1 < 4;
-      if constexpr (QT == QT_Q4_K) {
+      if constexpr (QT == QT_Q4_K || QT == QT_Q5_K) {
         if ((b & 1) == 0) {  // min term of blocks b and b + 1: lane half g supplies block b + g
 #pragma unroll
           for (int ms = 0; ms < 2; ++ms) uop[ms] = L.u[b + g][wm * 64 + ms * 32 + l32];
@@ -238,7 +248,7 @@ __device__ inline void gemm2_body(const uint8_t* __restrict__ raw, const signed 
           res[ms][ns][i] = __builtin_fmaf((float)I[slot][i], P[ms][16 * ns + i], res[ms][ns][i]);
         // the min term goes straight into the same accumulators on the matrix pipe; the ALU comes back to this tile
         // only after the other three
-        if constexpr (QT == QT_Q4_K)
+        if constexpr (QT == QT_Q4_K || QT == QT_Q5_K)
           if ((b & 1) == 0) res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop[ns], res[ms][ns], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -1428,6 +1438,9 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
 
 GEMM2_INST(8)
 GEMM2_TILES_INST(8)
+// Q5_K: the register-staged body (the Q4_K arithmetic on values 0..31)
+GEMM2_INST(13)
+GEMM2_TILES_INST(13)
 // Q4_K -DBM=64: 64 tokens x 256 rows per work-group (grid ceil(N / 256) * ceil(M / 64) work-groups), K from 0
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,

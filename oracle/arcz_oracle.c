@@ -15,13 +15,15 @@
  *   orc_quantize_act                    closed forms (max -> +-127, zero block, ties to even); golden + compiled ref
  *   orc_quantize_rows_q8_0              golden + compiled ref; round trip bound
  *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
+ *   Q5_K decode                         closed-form block; golden vectors (tests/golden/ref_vectors_q5k.npz) and live
+ *                                       comparison with the compiled reference header
  *   orc_block_sums                      brute-force integer sums in numpy (int64)
  *   orc_matmul_ref                      numpy float64 dot of dequantized rows; unit-scale known answer
  *   orc_matmul_formula                  against orc_matmul_ref within float rounding; unit-scale known answer (exact)
  *   orc_moe_route                       stable-sort top-k in numpy (the reference's own CPU check, tests/test_route.cpp:28-44)
  *   orc_moe_scan / orc_moe_scatter      invariants (bijection, contiguity, counts) + numpy restatement
  *   orc_moe_layer                       composition of the above, compared with a numpy float64 composition
- * The f32 -> Q4_K / Q6_K quantizers used to make synthetic weights are not part of the reference (it has none) and
+ * The f32 -> Q4_K / Q5_K / Q6_K quantizers used to make synthetic weights are not part of the reference (it has none) and
  * not part of this file: they are input generators of the product's bench/test utilities; parity unpinned by design.
  */
 #include <math.h>
@@ -38,6 +40,8 @@
 /* Q4_0 is Q8_0 with q - 8 in four bits (src/quants.h:136): everything after the decode treats the two alike */
 #define ORC_Q8LIKE(t) ((t) == ORC_Q8_0 || (t) == ORC_Q4_0)
 #define ORC_Q4_K 12u
+#define ORC_Q5_K 13u
+#define ORC_Q45(t) ((t) == ORC_Q4_K || (t) == ORC_Q5_K) /* d, dmin, 6-bit scales and mins */
 #define ORC_Q6_K 14u
 
 /* ---------------------------------------------------------------- fp16 (src/quants.h:17-52) */
@@ -97,6 +101,7 @@ int orc_sb_bytes(uint32_t type) {
     case ORC_Q8_0: return 34 * 8;
     case ORC_Q4_0: return 18 * 8;
     case ORC_Q4_K: return 144;
+    case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
     default: return 0;
   }
@@ -116,6 +121,7 @@ static void scale_min_k4(int j, const uint8_t* q, int* sc, int* mn) {
 /*
  * One decoded superblock (the fields of the reference's DecodedSB that the three types use, src/quants.h:72-84).
  *   Q4_K: q 0..15, sc[8], mn[8], d, dmin        (src/quants.h:91-113)
+ *   Q5_K: the same with q 0..31                  (src/quants.h:101-108)
  *   Q6_K: q 0..63 (offset 32 NOT removed), sc6[16], d   (src/quants.h:115-134)
  *   Q8_0: q -128..127, d8[8]                    (src/quants.h:149-157)
  */
@@ -131,15 +137,22 @@ static uint16_t rd16(const uint8_t* p) { uint16_t v; memcpy(&v, p, 2); return v;
 
 int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
   memset(o, 0, sizeof *o);
-  if (type == ORC_Q4_K) {
+  if (ORC_Q45(type)) {
     o->d = orc_fp16_to_f32(rd16(p));
     o->dmin = orc_fp16_to_f32(rd16(p + 2));
     for (int b = 0; b < 8; ++b) scale_min_k4(b, p + 4, &o->sc[b], &o->mn[b]);
-    const uint8_t* qs = p + 16;
+    /* Q5_K: 32 bytes of fifth bits between the scales and the nibbles; bit b of byte l belongs to element 32 b + l */
+    const uint8_t* qh = type == ORC_Q5_K ? p + 16 : NULL;
+    const uint8_t* qs = type == ORC_Q5_K ? p + 48 : p + 16;
     for (int j = 0; j < 4; ++j)
       for (int l = 0; l < 32; ++l) {
-        o->q[64 * j + l] = (int16_t)(qs[32 * j + l] & 0xF);
-        o->q[64 * j + 32 + l] = (int16_t)(qs[32 * j + l] >> 4);
+        int lo = qs[32 * j + l] & 0xF, hi = qs[32 * j + l] >> 4;
+        if (qh) {
+          lo += 16 * ((qh[l] >> (2 * j)) & 1);
+          hi += 16 * ((qh[l] >> (2 * j + 1)) & 1);
+        }
+        o->q[64 * j + l] = (int16_t)lo;
+        o->q[64 * j + 32 + l] = (int16_t)hi;
       }
     return 0;
   }
@@ -183,7 +196,7 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
 
 /* Value of element e of a decoded superblock, f32, evaluated left to right as written (src/quants.h:317-324). */
 static float sb_value(uint32_t type, const orc_sb* o, int e) {
-  if (type == ORC_Q4_K) return o->d * (float)o->sc[e / 32] * (float)o->q[e] - o->dmin * (float)o->mn[e / 32];
+  if (ORC_Q45(type)) return o->d * (float)o->sc[e / 32] * (float)o->q[e] - o->dmin * (float)o->mn[e / 32];
   if (type == ORC_Q6_K) return o->d * (float)o->sc6[e / 16] * (float)(o->q[e] - 32);
   return o->d8[e / 32] * (float)o->q[e];
 }
@@ -216,12 +229,12 @@ int orc_decode_row_fields(uint32_t type, const uint8_t* row, int K, int8_t* q, i
     orc_decode_sb(type, row + (size_t)s * bb, &o);
     for (int e = 0; e < 256; ++e) q[s * 256 + e] = (int8_t)sb_int(type, &o, e);
     for (int h = 0; h < 16; ++h) {
-      isc[s * 16 + h] = type == ORC_Q4_K ? o.sc[h / 2] : type == ORC_Q6_K ? o.sc6[h] : 1;
-      imn[s * 16 + h] = type == ORC_Q4_K ? o.mn[h / 2] : 0;
+      isc[s * 16 + h] = ORC_Q45(type) ? o.sc[h / 2] : type == ORC_Q6_K ? o.sc6[h] : 1;
+      imn[s * 16 + h] = ORC_Q45(type) ? o.mn[h / 2] : 0;
     }
     for (int b = 0; b < 8; ++b) {
       d[s * 8 + b] = ORC_Q8LIKE(type) ? o.d8[b] : o.d;
-      dmin[s * 8 + b] = type == ORC_Q4_K ? o.dmin : 0.0f;
+      dmin[s * 8 + b] = ORC_Q45(type) ? o.dmin : 0.0f;
     }
   }
   return 0;
@@ -412,7 +425,7 @@ int orc_matmul_formula(uint32_t type, int form, const uint8_t* W, int N, int K, 
             const int lo = h16[2 * b], hi = h16[2 * b + 1];
             const int bs0 = absum[(size_t)(s * 16 + 2 * b) * Ms + m], bs1 = absum[(size_t)(s * 16 + 2 * b + 1) * Ms + m];
             sa2[u] = sa;
-            if (type == ORC_Q4_K) {
+            if (ORC_Q45(type)) {
               t2[u] = (float)(o.sc[b] * lo + o.sc[b] * hi);
               m2[u] = (float)(o.mn[b] * bs0 + o.mn[b] * bs1);
               if (form == 0) res += sa * (o.d * t2[u] - o.dmin * m2[u]);
@@ -435,7 +448,7 @@ int orc_matmul_formula(uint32_t type, int form, const uint8_t* W, int N, int K, 
             }
           }
         }
-        if (form == 1 && type == ORC_Q4_K) res = fmaf(o.d, tq, fmaf(-o.dmin, tmn, res));
+        if (form == 1 && ORC_Q45(type)) res = fmaf(o.d, tq, fmaf(-o.dmin, tmn, res));
         if (form == 1 && type == ORC_Q6_K) res = fmaf(o.d, tq, res);
       }
       Y[(size_t)m * ldy + n] = res;

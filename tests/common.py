@@ -5,9 +5,9 @@ import numpy as np
 import arcinferzero_amd as az
 import oracle_lib as orc
 
-Q8_0, Q4_K, Q6_K = az.Q8_0, az.Q4_K, az.Q6_K
-TYPES = (Q8_0, Q4_K, Q6_K)
-TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+Q8_0, Q4_K, Q5_K, Q6_K = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K
+TYPES = (Q8_0, Q4_K, Q6_K, Q5_K)
+TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
 
 
 def make_weights(qtype, N, K, seed):
@@ -62,6 +62,17 @@ def unit_scale_weights(qtype, N, K, seed):
         blk[..., 12:16] = 1    # sc[4..7] low nibble = 1
         for j in range(4):
             blk[..., 16 + 32 * j:16 + 32 * j + 32] = (q[..., 64 * j:64 * j + 32] | (q[..., 64 * j + 32:64 * j + 64] << 4)).astype(np.uint8)
+        return blk.reshape(-1), q.reshape(N, K)
+    if qtype == Q5_K:
+        q = rng.integers(0, 32, size=(N, nsb, 256), dtype=np.int64)
+        blk = np.zeros((N, nsb, 176), np.uint8)
+        blk[..., 0:2] = one
+        blk[..., 4:8] = 1
+        blk[..., 12:16] = 1
+        for j in range(4):
+            lo, hi = q[..., 64 * j:64 * j + 32], q[..., 64 * j + 32:64 * j + 64]
+            blk[..., 48 + 32 * j:48 + 32 * j + 32] = ((lo & 15) | ((hi & 15) << 4)).astype(np.uint8)
+            blk[..., 16:48] |= (((lo >> 4) << (2 * j)) | ((hi >> 4) << (2 * j + 1))).astype(np.uint8)
         return blk.reshape(-1), q.reshape(N, K)
     if qtype == Q6_K:
         q = rng.integers(0, 64, size=(N, nsb, 256), dtype=np.int64)

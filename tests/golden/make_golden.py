@@ -4,7 +4,9 @@ from oracle/_ref/libarcz_ref.so, which oracle/Makefile compiles from the referen
 container that has the reference tree (make -C oracle ref); the fixture it writes is data only and is what travels.
 
 Functions covered: fp16_to_f32 / f32_to_fp16 (:17-52), decode_sb / dequant_row for Q8_0, Q4_K, Q6_K (:89-158,
-:519-622), quantize_act_cpu (:626-643, both scale widths), quantize_rows_q8_0 (:429-442).
+:519-622), quantize_act_cpu (:626-643, both scale widths), quantize_rows_q8_0 (:429-442).  A second file,
+ref_vectors_q5k.npz, holds the same decode vectors for Q5_K (:91-113), drawn from a generator of its own so that the
+first file's bytes stay what they were.
 """
 import ctypes as C
 import os
@@ -87,3 +89,23 @@ out["q80_rows_out"] = orc.quantize_rows_q8_0(w, lib=ref)
 
 np.savez_compressed(os.path.join(HERE, "ref_vectors.npz"), **out)
 print("wrote", os.path.join(HERE, "ref_vectors.npz"), {k: v.shape for k, v in out.items()})
+
+# ---- Q5_K blocks (176 bytes: d, dmin, 12 bytes of scales, 32 bytes of fifth bits, 128 bytes of nibbles)
+rng = np.random.default_rng(20261126)
+out5 = {}
+nblk = N * K // 256
+raw = rng.integers(0, 256, size=(nblk, 176), dtype=np.uint8)
+raw[:, 0:2] = finite_f16(nblk).reshape(-1, 1).view(np.uint8)
+raw[:, 2:4] = finite_f16(nblk).reshape(-1, 1).view(np.uint8)
+raw = raw.reshape(-1)
+out5["q5k_raw"] = raw
+out5["q5k_dequant"] = orc.dequant_rows(13, raw, N, K, lib=ref)
+q = np.zeros(256, np.int16); sc = np.zeros(8, np.int32); mn = np.zeros(8, np.int32); sc6 = np.zeros(16, np.int32)
+d8 = np.zeros(8, np.float32); d = C.c_float(); dm = C.c_float()
+first = np.ascontiguousarray(raw[:176])
+assert ref.ref_decode_sb(C.c_uint32(13), orc.ptr(first), orc.ptr(q), orc.ptr(sc), orc.ptr(mn), orc.ptr(sc6), orc.ptr(d8),
+                         C.byref(d), C.byref(dm)) == 0
+out5["q5k_sb0_q"] = q.copy(); out5["q5k_sb0_sc"] = sc.copy(); out5["q5k_sb0_mn"] = mn.copy()
+out5["q5k_sb0_d"] = np.array([d.value, dm.value], np.float32)
+np.savez_compressed(os.path.join(HERE, "ref_vectors_q5k.npz"), **out5)
+print("wrote", os.path.join(HERE, "ref_vectors_q5k.npz"), {k: v.shape for k, v in out5.items()})

@@ -1,6 +1,6 @@
 """A seeded sweep over ragged shapes, so that every launch form the engine can pick is exercised somewhere: lanes per
 row 32 / 64 / 128 / 256 and 1-6 units per lane for the GEMVs, every token count 1-8, rows that do not fill a pass,
-GEMM chunks that do not fill a tile in either direction, the short-chunk tile form, all three weight types.  Each case
+GEMM chunks that do not fill a tile in either direction, the short-chunk tile form, all four weight types.  Each case
 against the double-accumulated dequantized reference (tolerance 1e-3 as max|err| / max|ref| per token row)."""
 import numpy as np
 import pytest
@@ -17,7 +17,7 @@ def _cases(seed, n, kind):
     rng = np.random.default_rng(seed)
     out = []
     for i in range(n):
-        qt = TYPES[i % 3]
+        qt = TYPES[i % len(TYPES)]
         if kind == "gemv":
             K = 256 * int(rng.choice([1, 2, 3, 5, 8, 12, 16, 20, 24, 31, 40, 48, 68]))
             N = int(rng.integers(1, 700))

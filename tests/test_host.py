@@ -55,17 +55,35 @@ def test_repack_planes_layout(qtype):
     P = az.repack_planes(qtype, rows, K, W)
     assert P.size == az.planes_bytes(qtype, rows, K)
     u = rows * nsb
-    if qtype == az.Q4_K:
-        sb = W.reshape(u, 144)
+    if qtype in (az.Q4_K, az.Q5_K):
+        q5 = qtype == az.Q5_K
+        sbb = 176 if q5 else 144
+        sb = W.reshape(u, sbb)
         assert P.size == W.size
-        assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 16:])
-        hdr = P[u * 128:].reshape(u, 16)
+        assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, sbb - 128:])
+        hdr = P[u * 128:u * 144].reshape(u, 16)
+        if q5:
+            # the fifth bits, one word per 16-byte unit of nibbles: byte c, bit 4 + k = the low-nibble value of the
+            # unit's byte 4 k + c, bit k = its high-nibble value; put back on the nibbles they must give the oracle's q
+            H = P[u * 144:].view(np.uint32).reshape(u, 8)
+            qs = P[:u * 128].reshape(u, 8, 16)
+            q = np.zeros((u, 256), np.int64)
+            for un in range(8):
+                j, half = divmod(un, 2)
+                for m in range(16):
+                    k, c = divmod(m, 4)
+                    lo = (qs[:, un, m] & 15) | (((H[:, un] >> (8 * c + 4 + k)) & 1) << 4)
+                    hi = (qs[:, un, m] >> 4) | (((H[:, un] >> (8 * c + k)) & 1) << 4)
+                    q[:, 64 * j + 16 * half + m] = lo
+                    q[:, 64 * j + 32 + 16 * half + m] = hi
+            want = np.stack([orc.decode_row_fields(qtype, W[r * nsb * sbb:(r + 1) * nsb * sbb], K)[0] for r in range(rows)])
+            assert np.array_equal(q.reshape(rows, K), want)
         assert np.array_equal(hdr[:, :4], sb[:, :4])                       # d, dmin
         bits = np.zeros(u, dtype=object)
         for k in range(12):
             bits = bits + (hdr[:, 4 + k].astype(object) << (8 * k))
         for r in range(rows):                                               # entries sc | mn << 6 at bit 12 b
-            _, isc, imn, _, _ = orc.decode_row_fields(qtype, W[r * nsb * 144:(r + 1) * nsb * 144], K)
+            _, isc, imn, _, _ = orc.decode_row_fields(qtype, W[r * nsb * sbb:(r + 1) * nsb * sbb], K)
             for s in range(nsb):
                 for b in range(8):
                     e = (int(bits[r * nsb + s]) >> (12 * b)) & 0xFFF
@@ -88,9 +106,9 @@ def test_q8_0_quantizer_is_the_reference_one():
     assert np.array_equal(az.quantize_rows(az.Q8_0, w), orc.quantize_rows_q8_0(w))
 
 
-@pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q6_K, 0.02), (az.Q8_0, 0.006)])
+@pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q5_K, 0.04), (az.Q6_K, 0.02), (az.Q8_0, 0.006)])
 def test_block_makers_make_valid_close_blocks(qtype, rel):
-    """The Q4_K / Q6_K block makers are input generators (the reference has none): valid fields and a round-trip
+    """The Q4_K / Q5_K / Q6_K block makers are input generators (the reference has none): valid fields and a round-trip
     error of the size the bit width allows."""
     N, K = 64, 1024
     w = az.gen_normal(6, (N, K), std=0.02)
@@ -102,6 +120,8 @@ def test_block_makers_make_valid_close_blocks(qtype, rel):
     q, isc, imn, d, dmin = orc.decode_row_fields(qtype, B[:az.gguf_bytes(qtype, 1, K)], K)
     if qtype == az.Q4_K:
         assert q.min() >= 0 and q.max() <= 15 and isc.max() <= 63 and imn.max() <= 63 and len(np.unique(q)) == 16
+    elif qtype == az.Q5_K:
+        assert q.min() >= 0 and q.max() <= 31 and isc.max() <= 63 and imn.max() <= 63 and len(np.unique(q)) == 32
     elif qtype == az.Q6_K:
         assert q.min() >= -32 and q.max() <= 31 and isc.max() <= 127 and isc.min() >= 1
 

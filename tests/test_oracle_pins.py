@@ -12,9 +12,10 @@ import arcinferzero_amd as az
 import oracle_lib as orc
 from common import TYPES, make_acts, make_weights, rel_err_rows, unit_scale_acts, unit_scale_weights
 
-G = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz"))
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-NAMES = {Q4_K: "q4k", Q6_K: "q6k", Q8_0: "q80"}
+G = dict(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz")))
+G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_q5k.npz")))
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+NAMES = {Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k", Q8_0: "q80"}
 
 
 # ---------------------------------------------------------------- fp16
@@ -53,7 +54,7 @@ def test_dequant_golden(qtype):
     q, isc, imn, d, dmin = orc.decode_row_fields(qtype, G[f"{nm}_raw"][:512 // 256 * orc.SB_BYTES[qtype]], 512)
     gq = G[f"{nm}_sb0_q"].astype(np.int32) - (32 if qtype == Q6_K else 0)
     assert np.array_equal(q[:256], gq)
-    if qtype == Q4_K:
+    if qtype in (Q4_K, Q5_K):
         assert np.array_equal(isc[:16:2], G[f"{nm}_sb0_sc"]) and np.array_equal(imn[:16:2], G[f"{nm}_sb0_mn"])
         assert d[0] == G[f"{nm}_sb0_d"][0] and dmin[0] == G[f"{nm}_sb0_d"][1]
     elif qtype == Q6_K:
@@ -97,6 +98,36 @@ def test_q4k_closed_form():
             exp[256 * s + e] = d * sc[e // 32] * q - dmin * mn[e // 32]
     got = orc.dequant_rows(Q4_K, blk.reshape(-1), 1, K)[0]
     assert np.array_equal(got, exp)
+
+
+def test_q5k_closed_form():
+    """As the Q4_K case with five-bit values: bit b of byte l of the 32 bytes after the scales is the fifth bit of element
+    32 b + l (src/quants.h:101-108); expected values without the decoder."""
+    K = 256
+    blk = np.zeros(176, np.uint8)
+    d, dmin = 0.5, 0.25
+    blk[0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+    blk[2:4] = np.frombuffer(np.float16(dmin).tobytes(), np.uint8)
+    sc = [(5 * b + 9) % 64 for b in range(8)]
+    mn = [(11 * b + 2) % 64 for b in range(8)]
+    sb = blk[4:16]
+    for j in range(8):
+        if j < 4:
+            sb[j] |= sc[j]; sb[j + 4] |= mn[j]
+        else:
+            sb[j + 4] |= (sc[j] & 15) | ((mn[j] & 15) << 4)
+            sb[j - 4] |= (sc[j] >> 4) << 6
+            sb[j] |= (mn[j] >> 4) << 6
+    exp = np.zeros(K, np.float32)
+    for e in range(256):
+        q = (e * 7 + 3) % 32
+        b, l = divmod(e, 32)
+        blk[48 + 32 * (b // 2) + l] |= (q & 15) << (4 * (b % 2))
+        blk[16 + l] |= (q >> 4) << b
+        exp[e] = d * sc[b] * q - dmin * mn[b]
+    assert np.array_equal(orc.dequant_rows(Q5_K, blk, 1, K)[0], exp)
+    q, isc, imn, dd, dm = orc.decode_row_fields(Q5_K, blk, K)
+    assert np.array_equal(q, [(e * 7 + 3) % 32 for e in range(256)])
 
 
 def test_q6k_closed_form():
