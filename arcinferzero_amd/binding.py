@@ -88,6 +88,8 @@ _sig("arcz_engine_add_norm_quant", _i, _p, _p, _p, _p, _i, _i, _i, C.c_float, _p
 _sig("arcz_engine_swiglu_quant", _i, _p, _p, _i, _i, _i, _i, _i, _i)
 _sig("arcz_engine_set_activations", _i, _p, _p, _p, _p, _i, _i, _i)
 _sig("arcz_engine_aq", _p, _p)
+_sig("arcz_engine_two_pass", _i, _p, _i)
+_sig("arcz_engine_residual", _p, _p, _i)
 _sig("arcz_engine_asc", _p, _p)
 _sig("arcz_engine_absum", _p, _p)
 _sig("arcz_engine_matmul", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
@@ -441,6 +443,15 @@ class Engine:
     @property
     def absum(self):
         return Buffer(lib.arcz_engine_absum(self.h), owner=False)
+
+    def two_pass(self, on=True):
+        """Two-pass matmul inputs (the reference's q2mm_ mode): producers also quantize the residual, matmuls add its pass."""
+        _check(lib.arcz_engine_two_pass(self.h, 1 if on else 0), engine=True)
+
+    def read_residual(self, K, Mp):
+        b = [Buffer(lib.arcz_engine_residual(self.h, i), owner=False) for i in range(3)]
+        return (b[0].read(np.int8, Mp * K).reshape(Mp, K), b[1].read(np.float32, Mp * K // 32).reshape(K // 32, Mp),
+                b[2].read(np.int16, Mp * K // 16).reshape(K // 16, Mp))
 
     def read_activations(self, K, Mp):
         return (self.aq.read(np.int8, Mp * K).reshape(Mp, K), self.asc.read(np.float32, Mp * K // 32).reshape(K // 32, Mp),

@@ -125,6 +125,13 @@ int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* a
                                 int T) {
   return guarded([&] { e->e->set_activations(aq, asc, absum, K, Mp, T); });
 }
+int arcz_engine_two_pass(arcz_engine* e, int on) {
+  return guarded([&] { e->e->set_two_pass(on != 0); });
+}
+arcz_mem* arcz_engine_residual(arcz_engine* e, int which) {
+  cl_mem b[3] = {e->e->aq2_, e->e->asc2_, e->e->absum2_};
+  return which >= 0 && which < 3 ? b[which] : nullptr;
+}
 arcz_mem* arcz_engine_aq(arcz_engine* e) { return e->e->aq_; }
 arcz_mem* arcz_engine_asc(arcz_engine* e) { return e->e->asc_; }
 arcz_mem* arcz_engine_absum(arcz_engine* e) { return e->e->absum_; }

@@ -50,10 +50,51 @@ class Engine {
     if (max_chunk <= 0 || max_k <= 0 || max_k % 256) throw std::invalid_argument("Engine: max_k must be a positive multiple of 256");
     // (the GEMM kernels address a chunk's int8 rows and a matrix's packed rows with 32-bit byte offsets)
     if ((uint64_t)max_chunk * (uint64_t)max_k >= (1ull << 32)) throw std::invalid_argument("Engine: a chunk of max_chunk x max_k values must stay below 4 GiB");
+    alloc_activations();
+  }
+  // (zero/engine_alloc.h:10, 39, 41: twice the size with two-pass matmul inputs, the residual's half behind the first)
+  void alloc_activations() {
+    const size_t M = (size_t)max_chunk, f = q2mm_ ? 2 : 1;
+    aq_ = buf(M * max_k * f);
+    asc_ = buf(M * (max_k / 32) * 4 * f);
+    absum_ = buf(M * (max_k / 16) * 2 * f);
+  }
+  // Two-pass matmul inputs (zero/engine.h:1034-1075 q2_init, the mode of the reference's Gemma 4 and Qwen3 models):
+  // every producer also quantizes what its int8 values miss, v - q * scale, the same way, into the second half of the
+  // three buffers, and every matmul runs a second time over that half, accumulating (matmul below).
+  bool q2mm_ = false;
+  size_t q2_aq_ = 0, q2_sc_ = 0, q2_ab_ = 0;  // bytes
+  std::string q2_defs_;
+  cl_mem aq2_ = nullptr, asc2_ = nullptr, absum2_ = nullptr;  // views of the second halves
+  void set_two_pass(bool on) {
+    if (on == q2mm_) return;
+    for (cl_mem* v : {&aq2_, &asc2_, &absum2_})
+      if (*v) { release(*v); *v = nullptr; }
+    release(aq_); release(asc_); release(absum_);
+    q2mm_ = on;
+    cur_T_ = cur_K_ = cur_Mp_ = 0;
+    alloc_activations();
+    q2_defs_.clear();
+    q2_aq_ = q2_sc_ = q2_ab_ = 0;
+    if (!on) return;
     const size_t M = (size_t)max_chunk;
-    aq_ = buf(M * max_k);
-    asc_ = buf(M * (max_k / 32) * 4);
-    absum_ = buf(M * (max_k / 16) * 2);
+    q2_aq_ = M * max_k;
+    q2_sc_ = M * (max_k / 32) * 4;
+    q2_ab_ = M * (max_k / 16) * 2;
+    if (q2_aq_ >= (1ull << 31)) throw std::invalid_argument("two-pass mode: a chunk of max_chunk x max_k values must stay below 2 GiB");
+    q2_defs_ = " -DQ2_AQ=" + std::to_string(q2_aq_) + " -DQ2_SC=" + std::to_string(q2_sc_ / 4) + " -DQ2_AB=" +
+               std::to_string(q2_ab_ / 2);
+    aq2_ = view(aq_, q2_aq_, q2_aq_);
+    asc2_ = view(asc_, q2_sc_, q2_sc_);
+    absum2_ = view(absum_, q2_ab_, q2_ab_);
+  }
+  cl_mem view(cl_mem parent, size_t origin, size_t size) {  // (the reference's from(), zero/engine.h:251-252)
+    cl_buffer_region r{origin, size};
+    cl_int err = 0;
+    cl_mem m = clCreateSubBuffer(parent, CL_MEM_READ_WRITE, CL_BUFFER_CREATE_TYPE_REGION, &r, &err);
+    CL_CHECK(err);
+    mems_.push_back(m);
+    return m;
   }
   ~Engine() {
     for (auto& kv : kernels_) clReleaseKernel(kv.second);
@@ -142,7 +183,7 @@ class Engine {
     check_chunk(K, Mp, T);
     if (!act32) throw std::runtime_error("quantize_rows: the matmul kernels take per-32 activation scales (act32)");
     if (ldx < K || arcz_mem_size(x) < ((size_t)(T - 1) * ldx + K) * 4) throw std::runtime_error("quantize_rows: x is too small");
-    cl_kernel k = kernel("ops", "", "quant_rows");
+    cl_kernel k = kernel("ops", q2_defs_, "quant_rows");
     set_args(k, 0, x, ldx, K, Mp, T, aq_, asc_, absum_, act32);
     size_t gws[2] = {(size_t)256 * (K / 256), (size_t)(Mp + 63) / 64}, lws[2] = {256, 1};
     run("quant_rows", k, 2, gws, lws);
@@ -158,7 +199,7 @@ class Engine {
     if (row_off < 0 || arcz_mem_size(x) < (size_t)(row_off + T) * K * 4 || arcz_mem_size(w) < (size_t)K * 4 ||
         (hout && arcz_mem_size(hout) < (size_t)Mp * K * 4))
       throw std::runtime_error("rmsnorm_quant: a buffer is too small for " + std::to_string(T) + " rows of " + std::to_string(K));
-    cl_kernel k = kernel("ops", "", "rmsnorm_quant");
+    cl_kernel k = kernel("ops", q2_defs_, "rmsnorm_quant");
     int wh = hout ? 1 : 0;
     set_args(k, 0, x, row_off, w, K, Mp, T, eps, aq_, asc_, absum_, hout, wh, act32);
     size_t gws[2] = {256, (size_t)Mp}, lws[2] = {256, 1};
@@ -174,7 +215,7 @@ class Engine {
     check_chunk(F, Mp, T);
     if (!act32) throw std::runtime_error("swiglu_quant: the matmul kernels take per-32 activation scales (act32)");
     if (arcz_mem_size(gu) < (size_t)T * F * (fused ? 1 : 2) * 4) throw std::runtime_error("swiglu_quant: gu is too small");
-    cl_kernel k = kernel("ops", "", "swiglu_quant");
+    cl_kernel k = kernel("ops", q2_defs_, "swiglu_quant");
     set_args(k, 0, gu, F, Mp, T, aq_, asc_, absum_, act32, fused, gelu);
     size_t gws[2] = {256, (size_t)Mp}, lws[2] = {256, 1};
     if (wide_rows(T)) {
@@ -194,7 +235,7 @@ class Engine {
     if (arcz_mem_size(x) < (size_t)T * K * 4 || arcz_mem_size(t) < (size_t)T * K * 4 || arcz_mem_size(w) < (size_t)K * 4 ||
         (norm2 && (!w2 || arcz_mem_size(w2) < (size_t)K * 4)))
       throw std::runtime_error("add_norm_quant: a buffer is too small for " + std::to_string(T) + " rows of " + std::to_string(K));
-    cl_kernel k = kernel("ops", "", "add_norm_quant");
+    cl_kernel k = kernel("ops", q2_defs_, "add_norm_quant");
     int nrm = norm2 ? 1 : 0, MM = Mp, TT = T, KK = K;
     set_args(k, 0, x, t, w, KK, eps, s, w2, nrm, MM, aq_, asc_, absum_, act32, TT);
     // (a pass of 1-8 tokens: the valid rows only, as the reference; a longer chunk: all Mp rows, the padding as zeros)
@@ -205,16 +246,30 @@ class Engine {
   // Activations quantized elsewhere (the reference's benches quantize on the host, bench/gemv_bench.cpp:103-129).
   void set_activations(const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp, int T) {
     check_chunk(K, Mp, T);
+    if (q2mm_) throw std::runtime_error("set_activations: a two-pass engine takes its inputs from the quantizing kernels");
     CL_CHECK(clEnqueueWriteBuffer(cl_.queue, aq_, CL_TRUE, 0, (size_t)Mp * K, aq, 0, nullptr, nullptr));
     CL_CHECK(clEnqueueWriteBuffer(cl_.queue, asc_, CL_TRUE, 0, (size_t)Mp * (K / 32) * 4, asc, 0, nullptr, nullptr));
     CL_CHECK(clEnqueueWriteBuffer(cl_.queue, absum_, CL_TRUE, 0, (size_t)Mp * (K / 16) * 2, absum, 0, nullptr, nullptr));
     cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
   }
 
-  // ---- matmul (zero/engine.h:1080-1112 without the two-pass mode): C[:, c_off : c_off+N] (+)= act * W^T for the
-  // current chunk.  acc: 0 = store, 1 = accumulate into C, 2 = C = silu(C) * result (GEMM path only).
+  // ---- matmul (zero/engine.h:1080-1112): C[:, c_off : c_off+N] (+)= act * W^T for the current chunk.  acc: 0 = store,
+  // 1 = accumulate into C, 2 = C = silu(C) * result (GEMM path only).  With two-pass inputs the residual's half goes
+  // through the same kernels a second time and accumulates (the reference's fused form for 1-4 tokens, both passes over
+  // one read of the weights, is not built: here they are two launches at every token count).
   void matmul(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
     matmul1(name, w, Mp, C, ldc, c_off, acc, act32);
+    if (!q2mm_) return;
+    if (acc > 1) throw std::logic_error(std::string("two-pass activations with a fused epilogue: ") + name);
+    const cl_mem a = aq_, s = asc_, b = absum_;
+    aq_ = aq2_; asc_ = asc2_; absum_ = absum2_;
+    try {
+      matmul1(name, w, Mp, C, ldc, c_off, 1, act32);
+    } catch (...) {
+      aq_ = a; asc_ = s; absum_ = b;
+      throw;
+    }
+    aq_ = a; asc_ = s; absum_ = b;
   }
 
   // rows per half wave of the one-token GEMV (the place of the reference's gemv1_rows, zero/engine.h:1119-1123)

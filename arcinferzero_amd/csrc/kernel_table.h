@@ -20,11 +20,11 @@ struct KernelSpec {
 
 // Entries with requires_def come before the plain entry of the same name.
 static const KernelSpec kKernelTable[] = {
-    // ---- ops
-    {"ops", "quant_rows", nullptr, "piiiipppi", {nullptr}, {{nullptr, 0, false}}, 256},
-    {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{nullptr, 0, false}}, 256},
-    {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{nullptr, 0, false}}, 256},
-    {"ops", "add_norm_quant", nullptr, "pppiffpiipppii", {nullptr}, {{nullptr, 0, false}}, 256},
+    // ---- ops (Q2_AQ / Q2_SC / Q2_AB: the two-pass mode's residual offsets, the reference's -D names; 0 = one pass)
+    {"ops", "quant_rows", nullptr, "piiiipppi", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
+    {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
+    {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
+    {"ops", "add_norm_quant", nullptr, "pppiffpiipppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},

@@ -7,6 +7,11 @@
 // Layouts: aq [M][K] int8, asc [K/32][M] (or [K/256][M]) f32, absum [K/16][M] int16.  Rows m >= T are written as
 // zeros with scale 0 (the padding rows of a prompt chunk).
 //
+// Two-pass mode (reference zero/kernels/ops.cl:73-101, its -DQ2_AQ / -DQ2_SC / -DQ2_AB; here the three offsets are
+// trailing arguments, 0 = off): the residual v - q * scale of every value is quantized the same way into the same
+// layouts q2_aq bytes / q2_sc floats / q2_ab shorts further on in the three buffers, for a second matmul pass that
+// accumulates into the first one's output.
+//
 // Mapping: a work-group of 256 threads takes one superblock (256 values) of 64 token rows.  Thread t holds 16
 // consecutive values of one row (16 threads = one row's superblock, read as one contiguous KiB); the two threads of a
 // 32-block exchange their maxima with one cross-lane move.  Scales and sums go through LDS so that they leave as
@@ -41,8 +46,9 @@ __device__ inline void store_tile_scales(const QuantTile& lds, int s, int m0, in
 // quant_rows: x [T][ldx] f32 -> aq / asc / absum for M rows (rows >= T zero).  grid (K/256, ceil(M/64)), local 256.
 extern "C" __global__ __launch_bounds__(256) void quant_rows(const float* __restrict__ x, int ldx, int K, int M, int T,
                                                              signed char* __restrict__ aq, float* __restrict__ asc,
-                                                             short* __restrict__ absum, int act32) {
-  __shared__ QuantTile lds;
+                                                             short* __restrict__ absum, int act32, int q2_aq, int q2_sc,
+                                                             int q2_ab) {
+  __shared__ QuantTile lds, lds2;
   const int s = blockIdx.x, m0 = blockIdx.y * 64;
   const int lane16 = threadIdx.x & 15, rg = threadIdx.x >> 4;
 #pragma unroll 1
@@ -63,7 +69,8 @@ extern "C" __global__ __launch_bounds__(256) void quant_rows(const float* __rest
     const float amax = block_amax(v, act32);
     uint4 pk;
     int sum;
-    quant16(v, amax, pk, sum);
+    float res[16];
+    quant16(v, amax, pk, sum, q2_aq ? res : nullptr);
     if (m < M) *(uint4*)(aq + (size_t)m * K + s * 256 + 16 * lane16) = pk;
     lds.sum[lane16][r] = (short)sum;
     if (act32) {
@@ -71,27 +78,52 @@ extern "C" __global__ __launch_bounds__(256) void quant_rows(const float* __rest
     } else if (lane16 == 0) {
       lds.asc[0][r] = amax / 127.0f;
     }
+    if (q2_aq) {  // (the same for the whole launch)
+      const float rmax = block_amax(res, act32);
+      quant16(res, rmax, pk, sum);
+      if (m < M) *(uint4*)(aq + q2_aq + (size_t)m * K + s * 256 + 16 * lane16) = pk;
+      lds2.sum[lane16][r] = (short)sum;
+      if (act32) {
+        if ((lane16 & 1) == 0) lds2.asc[lane16 >> 1][r] = rmax / 127.0f;
+      } else if (lane16 == 0) {
+        lds2.asc[0][r] = rmax / 127.0f;
+      }
+    }
   }
   __syncthreads();
   store_tile_scales(lds, s, m0, M, act32, asc, absum);
+  if (q2_aq) store_tile_scales(lds2, s, m0, M, act32, asc + q2_sc, absum + q2_ab);
 }
 
 // ---- the two fused producers.  A work-group of 256 threads per row (or several along x, each taking a share of the
 // row's superblocks: the launch for a pass of 1-8 tokens, zero/engine.h:1404-1412); 16 threads per superblock, thread
 // = 16 consecutive values, so a wave works on 4 superblocks at a time.  Scales and sums are stored straight into the
 // token-minor layouts (one element per block and row).
-__device__ inline void store_row_quant(const float* v, int s, int lane16, int m, int M, int K, int act32,
-                                       signed char* __restrict__ aq, float* __restrict__ asc, short* __restrict__ absum) {
+__device__ inline void store_row_quant1(const float* v, int s, int lane16, int m, int M, int K, int act32,
+                                        signed char* __restrict__ aq, float* __restrict__ asc, short* __restrict__ absum,
+                                        float* res) {
   const float amax = block_amax(v, act32);
   uint4 pk;
   int sum;
-  quant16(v, amax, pk, sum);
+  quant16(v, amax, pk, sum, res);
   *(uint4*)(aq + (size_t)m * K + s * 256 + 16 * lane16) = pk;
   absum[((size_t)s * 16 + lane16) * M + m] = (short)sum;
   if (act32) {
     if ((lane16 & 1) == 0) asc[((size_t)s * 8 + (lane16 >> 1)) * M + m] = amax / 127.0f;
   } else if (lane16 == 0) {
     asc[(size_t)s * M + m] = amax / 127.0f;
+  }
+}
+// (q2_aq != 0: the two-pass mode's residual too, at its offsets in the same buffers)
+__device__ inline void store_row_quant(const float* v, int s, int lane16, int m, int M, int K, int act32,
+                                       signed char* __restrict__ aq, float* __restrict__ asc, short* __restrict__ absum,
+                                       int q2_aq, int q2_sc, int q2_ab) {
+  if (!q2_aq) {
+    store_row_quant1(v, s, lane16, m, M, K, act32, aq, asc, absum, nullptr);
+  } else {
+    float res[16];
+    store_row_quant1(v, s, lane16, m, M, K, act32, aq, asc, absum, res);
+    store_row_quant1(res, s, lane16, m, M, K, act32, aq + q2_aq, asc + q2_sc, absum + q2_ab, nullptr);
   }
 }
 
@@ -114,7 +146,8 @@ extern "C" __global__ __launch_bounds__(256) void rmsnorm_quant(const float* __r
                                                                 const float* __restrict__ w, int K, int M, int M_valid,
                                                                 float eps, signed char* __restrict__ aq,
                                                                 float* __restrict__ asc, short* __restrict__ absum,
-                                                                float* __restrict__ hout, int write_h, int act32) {
+                                                                float* __restrict__ hout, int write_h, int act32,
+                                                                int q2_aq, int q2_sc, int q2_ab) {
   __shared__ float red[4];
   const int m = blockIdx.y;
   const bool valid = m < M_valid;
@@ -148,7 +181,7 @@ extern "C" __global__ __launch_bounds__(256) void rmsnorm_quant(const float* __r
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         *(float4*)(hout + (size_t)m * K + base + 4 * i) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
-    store_row_quant(v, s, lane16, m, M, K, act32, aq, asc, absum);
+    store_row_quant(v, s, lane16, m, M, K, act32, aq, asc, absum, q2_aq, q2_sc, q2_ab);
   }
 }
 
@@ -162,7 +195,8 @@ extern "C" __global__ __launch_bounds__(256) void add_norm_quant(float* __restri
                                                                  const float* __restrict__ w, int K, float eps, float s,
                                                                  const float* __restrict__ w2, int w2_norm, int M,
                                                                  signed char* __restrict__ aq, float* __restrict__ asc,
-                                                                 short* __restrict__ absum, int act32, int M_valid) {
+                                                                 short* __restrict__ absum, int act32, int M_valid,
+                                                                 int q2_aq, int q2_sc, int q2_ab) {
   __shared__ float red[4];
   const int m = blockIdx.y;
   const bool valid = m < M_valid;
@@ -219,7 +253,7 @@ extern "C" __global__ __launch_bounds__(256) void add_norm_quant(float* __restri
 #pragma unroll
       for (int i = 0; i < 16; ++i) v[i] = 0.0f;
     }
-    store_row_quant(v, sb, lane16, m, M, K, act32, aq, asc, absum);
+    store_row_quant(v, sb, lane16, m, M, K, act32, aq, asc, absum, q2_aq, q2_sc, q2_ab);
   }
 }
 
@@ -229,7 +263,7 @@ extern "C" __global__ __launch_bounds__(256) void add_norm_quant(float* __restri
 extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __restrict__ gu, int F, int M, int M_valid,
                                                                signed char* __restrict__ aq, float* __restrict__ asc,
                                                                short* __restrict__ absum, int act32, int fused,
-                                                               int gelu) {
+                                                               int gelu, int q2_aq, int q2_sc, int q2_ab) {
   const int m = blockIdx.y;
   const bool valid = m < M_valid;
   const float* gr = gu + (size_t)m * (fused ? F : 2 * F);
@@ -261,7 +295,7 @@ extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __re
         }
       }
     }
-    store_row_quant(v, s, lane16, m, M, F, act32, aq, asc, absum);
+    store_row_quant(v, s, lane16, m, M, F, act32, aq, asc, absum, q2_aq, q2_sc, q2_ab);
   }
 }
 

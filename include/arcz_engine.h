@@ -58,7 +58,16 @@ int arcz_engine_swiglu_quant(arcz_engine* e, arcz_mem* gu, int F, int Mp, int T,
  * without norm2). */
 int arcz_engine_add_norm_quant(arcz_engine* e, arcz_mem* x, arcz_mem* t, arcz_mem* w, int K, int T, int Mp, float s,
                                arcz_mem* w2, int norm2, int act32, float eps);
-/* Activations quantized by the caller, as the reference's benches do (bench/gemv_bench.cpp:103-129). */
+/* Two-pass matmul inputs on or off (zero/engine.h:1034-1075 q2_init, 1080-1101 matmul; zero/kernels/ops.cl:49-59,
+ * 73-101): every quantizing call above also stores what its int8 values miss, quantized the same way, in the second
+ * half of the (re-allocated, twice as large) activation buffers, and every arcz_engine_matmul runs a second pass over
+ * that half, accumulating into the first one's output (accumulate mode 2 is refused, as in the reference).  The
+ * mixture-of-experts layer takes the first half only.  Forgets the current chunk. */
+int arcz_engine_two_pass(arcz_engine* e, int on);
+/* The second halves (0 = int8 values, 1 = scales, 2 = 16-sums) as views, NULL in one-pass mode. */
+arcz_mem* arcz_engine_residual(arcz_engine* e, int which);
+/* Activations quantized by the caller, as the reference's benches do (bench/gemv_bench.cpp:103-129).  One-pass engines
+ * only. */
 int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp,
                                 int T);
 /* The engine's activation buffers (Engine::aq_, asc_, absum_; zero/engine_sessions.h:571). */

@@ -14,6 +14,7 @@
  *                                       golden vectors and live comparison with the compiled reference header
  *   orc_quantize_act                    closed forms (max -> +-127, zero block, ties to even); golden + compiled ref
  *   orc_quantize_rows_q8_0              golden + compiled ref; round trip bound
+ *   orc_act_residual                    PARITY UNPINNED (no reference CPU twin, no vector); identities and bounds only
  *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
  *   Q5_K decode                         closed-form block; golden vectors (tests/golden/ref_vectors_q5k.npz) and live
  *                                       comparison with the compiled reference header
@@ -264,6 +265,22 @@ void orc_quantize_act(const float* x, int M, int K, int8_t* aq, float* asc, int1
       int sum = 0;
       for (int i = 0; i < 16; ++i) sum += aq[(size_t)m * K + b * 16 + i];
       absum[(size_t)b * M + m] = (int16_t)sum;
+    }
+}
+
+/* What the int8 values miss, for the two-pass matmul inputs (zero/kernels/ops.cl:49-59): res = v - (float)q * (amax / 127)
+ * per element, the product and the difference each rounded to f32 (this file is built without contraction; the
+ * reference's OpenCL text leaves that to its compiler).  res [M][K]; quantized by orc_quantize_act it gives the second
+ * pass's inputs (ops.cl:73-101).  PARITY UNPINNED against a run of the reference (its CPU twin quantize_act_cpu has no
+ * residual and no test vector holds one); pinned by what the mathematics fixes: q * scale + res == v exactly whenever
+ * the subtraction is exact (Sterbenz: always, here, for q != 0 -- see the tests), and |res| <= scale / 2 (1 + 2^-22). */
+void orc_act_residual(const float* x, int M, int K, const int8_t* aq, const float* asc, int act32, float* res) {
+  const int B = act32 ? 32 : 256;
+  for (int m = 0; m < M; ++m)
+    for (int e = 0; e < K; ++e) {
+      const float sc = asc[(size_t)(e / B) * M + m];
+      const float p = (float)aq[(size_t)m * K + e] * sc;
+      res[(size_t)m * K + e] = x[(size_t)m * K + e] - p;
     }
 }
 

@@ -84,6 +84,16 @@ def quantize_act(x, act32=True, lib=None):
     return aq, asc, absum
 
 
+def quantize_act_two_pass(x):
+    """The two-pass inputs: (aq, asc, absum) of x and of what they miss (per-32 scales)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    M, K = x.shape
+    aq, asc, absum = quantize_act(x)
+    res = np.empty((M, K), np.float32)
+    orc.orc_act_residual(ptr(x), _i(M), _i(K), ptr(aq), ptr(asc), _i(1), ptr(res))
+    return (aq, asc, absum), quantize_act(res), res
+
+
 def moe_quant(h, S=None):
     h = np.ascontiguousarray(h, dtype=np.float32)
     n, F = h.shape

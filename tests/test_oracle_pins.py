@@ -259,6 +259,25 @@ def test_quantize_rows_q8_0_golden_and_roundtrip():
     assert (np.abs(back.reshape(8, 8, 32) - w.reshape(8, 8, 32)) <= amax / 127.0 * 0.5 + amax * 2.0 ** -11 + 1e-12).all()
 
 
+def test_act_residual_identities():
+    """The two-pass residual v - q * scale: the subtraction is exact (q * scale is within a factor of two of v wherever
+    q != 0, and 0 where q == 0), so q * scale + res gives v back exactly; it is at most half a step; and quantizing it
+    leaves an error 254 times smaller than the first pass's step.  A wrong factor (127 / amax for amax / 127), a dropped
+    term or a wrong block index fails the bound."""
+    x = make_acts(6, 1024, seed=31, outliers=True)
+    x[1, 64:96] = 0.0
+    x[2, 128:160] *= 1e-30
+    (aq, asc, _), (rq, rsc, _), res = orc.quantize_act_two_pass(x)
+    sc = np.repeat(asc.T, 32, axis=1)
+    p = (aq.astype(np.float32) * sc).astype(np.float32)
+    assert np.array_equal(p.astype(np.float64) + res.astype(np.float64), x.astype(np.float64))
+    assert (np.abs(res) <= sc * 0.5 * (1 + 2.0 ** -21) + 1e-45).all()
+    assert not res[1, 64:96].any() and not rq[1, 64:96].any() and not rsc[2:3, 1].any()
+    rs = np.repeat(rsc.T, 32, axis=1)
+    left = x.astype(np.float64) - p.astype(np.float64) - rq.astype(np.float64) * rs.astype(np.float64)
+    assert (np.abs(left) <= rs * 0.5 * (1 + 2.0 ** -21) + 1e-45).all() and (rs <= sc / 253.9).all()
+
+
 # ---------------------------------------------------------------- integer sums and the f32 references
 @pytest.mark.parametrize("qtype", TYPES)
 def test_block_sums_brute_force(qtype):
