@@ -444,9 +444,10 @@ class Engine:
     def absum(self):
         return Buffer(lib.arcz_engine_absum(self.h), owner=False)
 
-    def two_pass(self, on=True):
-        """Two-pass matmul inputs (the reference's q2mm_ mode): producers also quantize the residual, matmuls add its pass."""
-        _check(lib.arcz_engine_two_pass(self.h, 1 if on else 0), engine=True)
+    def two_pass(self, on=True, fuse=True):
+        """Two-pass matmul inputs (the reference's q2mm_ mode): producers also quantize the residual, matmuls add its pass
+        (fuse: the GEMV of 1-4 tokens takes both in one launch)."""
+        _check(lib.arcz_engine_two_pass(self.h, (1 if fuse else 2) if on else 0), engine=True)
 
     def read_residual(self, K, Mp):
         b = [Buffer(lib.arcz_engine_residual(self.h, i), owner=False) for i in range(3)]

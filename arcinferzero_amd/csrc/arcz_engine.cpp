@@ -126,7 +126,10 @@ int arcz_engine_set_activations(arcz_engine* e, const int8_t* aq, const float* a
   return guarded([&] { e->e->set_activations(aq, asc, absum, K, Mp, T); });
 }
 int arcz_engine_two_pass(arcz_engine* e, int on) {
-  return guarded([&] { e->e->set_two_pass(on != 0); });
+  return guarded([&] {
+    e->e->set_two_pass(on != 0);
+    e->e->q2_nofuse_ = on == 2;
+  });
 }
 arcz_mem* arcz_engine_residual(arcz_engine* e, int which) {
   cl_mem b[3] = {e->e->aq2_, e->e->asc2_, e->e->absum2_};

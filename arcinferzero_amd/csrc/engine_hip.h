@@ -255,12 +255,23 @@ class Engine {
 
   // ---- matmul (zero/engine.h:1080-1112): C[:, c_off : c_off+N] (+)= act * W^T for the current chunk.  acc: 0 = store,
   // 1 = accumulate into C, 2 = C = silu(C) * result (GEMM path only).  With two-pass inputs the residual's half goes
-  // through the same kernels a second time and accumulates (the reference's fused form for 1-4 tokens, both passes over
-  // one read of the weights, is not built: here they are two launches at every token count).
+  // through the same kernels a second time and accumulates; for 1-4 tokens the GEMV takes both halves in one launch
+  // (as 2 T token slots, over one read of the weights: the reference's q2_fuse_, zero/engine.h:1086-1088) whenever the
+  // LDS-staged kernel can hold them, and says so in q2_fused_.  q2_nofuse_ (or ARCZ_Q2_FUSE=0): always two launches.
+  bool q2_fuse_ = false, q2_fused_ = false, q2_nofuse_ = false;
   void matmul(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
-    matmul1(name, w, Mp, C, ldc, c_off, acc, act32);
-    if (!q2mm_) return;
-    if (acc > 1) throw std::logic_error(std::string("two-pass activations with a fused epilogue: ") + name);
+    static const bool fuse_off = getenv("ARCZ_Q2_FUSE") && atoi(getenv("ARCZ_Q2_FUSE")) == 0;
+    if (q2mm_ && acc > 1) throw std::logic_error(std::string("two-pass activations with a fused epilogue: ") + name);
+    q2_fuse_ = q2mm_ && !fuse_off && !q2_nofuse_ && cur_T_ <= 4;
+    q2_fused_ = false;
+    try {
+      matmul1(name, w, Mp, C, ldc, c_off, acc, act32);
+    } catch (...) {
+      q2_fuse_ = false;
+      throw;
+    }
+    q2_fuse_ = false;
+    if (!q2mm_ || q2_fused_) return;
     const cl_mem a = aq_, s = asc_, b = absum_;
     aq_ = aq2_; asc_ = asc2_; absum_ = absum2_;
     try {
@@ -312,10 +323,14 @@ class Engine {
       for (int l : {32, 64, 128, 256})
         if (!lpr && (units + l - 1) / l <= 6 && (!force_lpr || l == force_lpr)) lpr = l;
       const int g = lpr ? 256 / lpr : 1, wpr = lpr > 64 ? lpr / 64 : 1;
-      const int tbl = T <= 2 ? T : T <= 4 ? 4 : 8;  // the kernel's token count (T rounded up)
-      const size_t lds = (size_t)tbl * tok_bytes + (wpr > 1 ? (size_t)16 * g * wpr * tbl * 4 : 0);  // (16: the kernels' GEMV_FLUSH)
+      // the kernel's token slots: T rounded up, or -- both halves of two-pass inputs in one launch -- 2 T rounded up
+      auto lds_of = [&](int slots) { return (size_t)slots * tok_bytes + (wpr > 1 ? (size_t)16 * g * wpr * slots * 4 : 0); };  // (16: the kernels' GEMV_FLUSH)
+      const int tb2 = T == 1 ? 2 : T == 2 ? 4 : 8;
+      const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= 65536;
+      const int tbl = q2f ? tb2 : T <= 2 ? T : T <= 4 ? 4 : 8;
+      const size_t lds = lds_of(tbl);
       if (!force_v && lpr && lds <= 65536) {
-        const int pf = (units + lpr - 1) / lpr, tb = T <= 2 ? T : T <= 4 ? 4 : 8;
+        const int pf = (units + lpr - 1) / lpr, tb = tbl;
         // one round of resident work-groups, passes of rows dealt to them in turn (ARCZ_GEMV_WPC: work-groups per
         // compute unit; two measured best: more add staging work and spread the reads over more rows at a time)
         static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
@@ -323,11 +338,14 @@ class Engine {
         size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : 2));
         if (wgs_env > 0) wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)wgs_env);
         const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
-                                 std::to_string(pf) + (T > 1 ? " -DTB=" + std::to_string(tb) : std::string()) + " -DLDS=" +
-                                 std::to_string(lds);
-        cl_kernel k = kernel("decode", defs, T == 1 ? "gemv" : "gemv_mt");
-        if (T == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
-        else set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a);
+                                 std::to_string(pf) + (tb > 1 ? " -DTB=" + std::to_string(tb) : std::string()) + " -DLDS=" +
+                                 std::to_string(lds) +
+                                 (q2f ? " -DQ2_AQ=" + std::to_string(q2_aq_) + " -DQ2_SC=" + std::to_string(q2_sc_ / 4) : std::string());
+        cl_kernel k = kernel("decode", defs, tb == 1 ? "gemv" : "gemv_mt");
+        int ld1 = T == 1 ? 0 : ldc;  // (one token: C is the row itself)
+        if (tb == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
+        else set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ld1, c_off, a);
+        q2_fused_ = q2f;
         size_t g1 = wgs * 256, l1 = 256;
         run(name, k, 1, &g1, &l1);
         return;

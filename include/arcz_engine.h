@@ -62,7 +62,10 @@ int arcz_engine_add_norm_quant(arcz_engine* e, arcz_mem* x, arcz_mem* t, arcz_me
  * 73-101): every quantizing call above also stores what its int8 values miss, quantized the same way, in the second
  * half of the (re-allocated, twice as large) activation buffers, and every arcz_engine_matmul runs a second pass over
  * that half, accumulating into the first one's output (accumulate mode 2 is refused, as in the reference).  The
- * mixture-of-experts layer takes the first half only.  Forgets the current chunk. */
+ * mixture-of-experts layer takes the first half only.  For 1-4 tokens the GEMV takes both halves in one launch, over
+ * one read of the weights (zero/engine.h:1086-1088), with the result two launches give bit for bit (except one token of
+ * Q4_K / Q5_K, whose one-token kernel groups a term's factors differently: equal to rounding); on = 2 keeps the two
+ * launches at every token count.  Forgets the current chunk. */
 int arcz_engine_two_pass(arcz_engine* e, int on);
 /* The second halves (0 = int8 values, 1 = scales, 2 = 16-sums) as views, NULL in one-pass mode. */
 arcz_mem* arcz_engine_residual(arcz_engine* e, int which);
