@@ -68,7 +68,7 @@ extern "C" {
 
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
-  return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : 0;
+  return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : 0;
 }
 // (Q4_0 rows are kept on the device as Q8_0 planes: see arcz_repack_planes)
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) {
@@ -131,6 +131,16 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
       memcpy(dst + pl.qh + i * 64, src + i * 210 + 128, 64);
       memcpy(dst + pl.sc + i * 16, src + i * 210 + 192, 16);
       memcpy(dst + pl.d + i * 2, src + i * 210 + 208, 2);
+    }
+    return 0;
+  }
+  if (type == QT_IQ4_XS) {
+    const PlanesIQ4XS pl = planes_iq4xs(rows, nsb);
+    memset(dst + pl.hdr + u * 8, 0, raw_planes_bytes(QT_IQ4_XS, rows, nsb) - (pl.hdr + u * 8));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i) {
+      memcpy(dst + pl.hdr + i * 8, src + i * 136, 8);
+      memcpy(dst + pl.qs + i * 128, src + i * 136 + 8, 128);
     }
     return 0;
   }
@@ -344,6 +354,51 @@ void arcz_quantize_q6_k(const float* src, size_t N, int K, uint8_t* out) {
   }
 }
 
+// f32 rows -> GGUF IQ4_XS superblocks (136 bytes per 256 values; reference src/quants.h:297-311): per 32-block a step
+// amax / 127 (the table's largest magnitude), rounded to 1..31 against d = max step / 31 (fp16) and stored + 32 in six
+// bits (low four in one nibble, high two in the 16-bit word), each value as the code of the nearest table entry.
+void arcz_quantize_iq4_xs(const float* src, size_t N, int K, uint8_t* out) {
+  static const int kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+  const int64_t nsbt = (int64_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < nsbt; ++s) {
+    const float* v = src + s * 256;
+    uint8_t* p = out + s * 136;
+    float step[8], smax = 0;
+    for (int b = 0; b < 8; ++b) {
+      float amax = 0;
+      for (int i = 0; i < 32; ++i) amax = std::fmax(amax, std::fabs(v[32 * b + i]));
+      step[b] = amax / 127.0f;
+      smax = std::fmax(smax, step[b]);
+    }
+    const uint16_t dh = f32_to_f16(smax / 31.0f);
+    const float d = f16_to_f32(dh);
+    memset(p, 0, 136);
+    memcpy(p, &dh, 2);
+    uint16_t sh = 0;
+    for (int b = 0; b < 8; ++b) {
+      const int l = d > 0 ? std::min(31, std::max(1, (int)std::lrintf(step[b] / d))) : 0;
+      const int ls = l + 32;
+      p[4 + b / 2] |= (uint8_t)((ls & 0xF) << (4 * (b % 2)));
+      sh |= (uint16_t)((ls >> 4) << (2 * b));
+      const float sd = d * (float)l;
+      for (int i = 0; i < 32; ++i) {
+        int best = 8;
+        if (sd > 0) {
+          const float x = v[32 * b + i] / sd;
+          float be = 1e30f;
+          for (int c = 0; c < 16; ++c) {
+            const float e = std::fabs(x - (float)kv[c]);
+            if (e < be) { be = e; best = c; }
+          }
+        }
+        p[8 + 16 * b + (i & 15)] |= (uint8_t)(best << (4 * (i >> 4)));
+      }
+    }
+    memcpy(p + 2, &sh, 2);
+  }
+}
+
 // f32 rows -> GGUF Q4_0 blocks the way the reference makes them (src/quants.h:444-463, llama.cpp's
 // quantize_row_q4_0_ref): d = (the value of largest magnitude) / -8, q = min(15, (int)(v / d + 8.5)).
 static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) {
@@ -364,7 +419,7 @@ static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) 
   }
 }
 
-// Quantizes f32 rows to `type` (2, 8, 12, 13, 14).  0 or -1.
+// Quantizes f32 rows to `type` (2, 8, 12, 13, 14, 23).  0 or -1.
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
   if (K <= 0 || K % 256) return -1;
   if (type == GGML_TYPE_Q4_0) arcz_quantize_q4_0(src, N, K, out);
@@ -372,6 +427,7 @@ int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t
   else if (type == QT_Q4_K) arcz_quantize_q4_k(src, N, K, out);
   else if (type == QT_Q5_K) arcz_quantize_q5_k(src, N, K, out);
   else if (type == QT_Q6_K) arcz_quantize_q6_k(src, N, K, out);
+  else if (type == QT_IQ4_XS) arcz_quantize_iq4_xs(src, N, K, out);
   else return -1;
   return 0;
 }

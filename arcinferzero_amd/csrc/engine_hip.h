@@ -17,6 +17,7 @@
 #define GGML_Q4_K 12u
 #define GGML_Q5_K 13u
 #define GGML_Q6_K 14u
+#define GGML_IQ4_XS 23u
 
 extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
 extern "C" size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
@@ -30,7 +31,7 @@ struct GpuWeight {
 };
 
 inline const char* ggml_type_name(uint32_t t) {
-  return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : "?";
+  return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : t == GGML_IQ4_XS ? "IQ4_XS" : "?";
 }
 
 class Engine {
@@ -149,7 +150,7 @@ class Engine {
   // device planes on the host, then one upload.  rows = N for a matrix, n_expert * N for an expert tensor.
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
-    if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K)
+    if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
     if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))

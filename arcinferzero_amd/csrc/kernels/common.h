@@ -16,6 +16,7 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 #define QT_Q4_K 12
 #define QT_Q5_K 13
 #define QT_Q6_K 14
+#define QT_IQ4_XS 23
 
 // ---- device weight layout ("raw planes").  A matrix of R rows x K columns (K % 256 == 0, nsb = K / 256) is held
 // as separate planes, each row-major over (row, superblock), so that every field is 16-byte aligned and a wave's
@@ -32,11 +33,15 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 //                              4 k + c, bit k = the high-nibble value of that byte (k = 0..3)
 //   Q6_K : ql  [R][nsb][128], qh [R][nsb][64], sc [R][nsb][16] (int8), d [R][nsb] (f16)
 //   Q8_0 : qs  [R][nsb][256] (int8), d [R][nsb][8] (f16)
+//   IQ4_XS: qs [R][nsb][128]  (GGUF order: byte j of block b = element 32b+j low nibble, 32b+16+j high nibble; a nibble
+//                              is a code of the 16-entry table below), hdr [R][nsb][8] (f16 d, 16 bits of the eight
+//                              6-bit block scales' high parts, 4 bytes of their low nibbles: as GGUF)
 // Plane offsets from the start of the buffer, in bytes (each a multiple of 256 when R * nsb is a multiple of 16;
 // always a multiple of 16 otherwise except as noted).
 struct PlanesQ4K { size_t qs, hdr, qh; };  // (qh: Q5_K only)
 struct PlanesQ6K { size_t ql, qh, sc, d; };
 struct PlanesQ80 { size_t qs, d; };
+struct PlanesIQ4XS { size_t qs, hdr; };
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 __host__ __device__ inline PlanesQ4K planes_q4k(size_t rows, int nsb) {
@@ -61,12 +66,19 @@ __host__ __device__ inline PlanesQ80 planes_q80(size_t rows, int nsb) {
   p.d = rows * (size_t)nsb * 256;
   return p;
 }
+__host__ __device__ inline PlanesIQ4XS planes_iq4xs(size_t rows, int nsb) {
+  PlanesIQ4XS p;
+  p.qs = 0;
+  p.hdr = rows * (size_t)nsb * 128;
+  return p;
+}
 __host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb) {
   const size_t u = rows * (size_t)nsb;
   if (qt == QT_Q4_K) return u * 144;
   if (qt == QT_Q5_K) return u * 176;
   if (qt == QT_Q6_K) return align16(u * 208 + u * 2);
   if (qt == QT_Q8_0) return u * 272;
+  if (qt == QT_IQ4_XS) return align16(u * 136);
   return 0;
 }
 
@@ -95,6 +107,17 @@ __device__ inline void q4k_scales_pair(uint32_t s0, uint32_t s1, uint32_t s2, in
 __device__ inline uint32_t q5k_lo(uint32_t w, uint32_t H, int k) { return (w & 0x0F0F0F0Fu) | ((H >> k) & 0x10101010u); }
 __device__ inline uint32_t q5k_hi(uint32_t w, uint32_t H, int k) {
   return ((w >> 4) & 0x0F0F0F0Fu) | ((H << (4 - k)) & 0x10101010u);
+}
+
+// IQ4_XS: four 4-bit codes, one in the low nibble of each byte of c, to the four int8 values of the format's table
+// (-127 -104 -83 -65 -49 -35 -22 -10 | 1 13 25 38 53 69 89 113; reference src/iq_tables.h:364-367): a byte permute per
+// table half, the code's bit 3 picks between them.
+__device__ inline uint32_t iq4_lookup(uint32_t c) {
+  const uint32_t sel = c & 0x07070707u;
+  const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, sel);  // codes 0-7: bytes 0-3 = second operand
+  const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, sel);  // codes 8-15
+  const uint32_t m = ((c >> 3) & 0x01010101u) * 0xFFu;
+  return (hi & m) | (lo & ~m);
 }
 
 __device__ inline int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }

@@ -7,6 +7,7 @@
 //   Q5_K : as Q4_K, the values 0..31 (the fifth bits come from their own plane)
 //   Q6_K : acc += sa * d * (float)(sc16 * I)                                bs: its int16 sum of the 16 activations
 //   Q8_0 : acc += sa * d * (float)I
+//   IQ4_XS: acc += sa * d * (float)(ls * I)      ls: the block's 6-bit scale - 32; values through the 16-entry table
 // (the reference groups the two halves of a 32-block inside the int -> float conversion; here each half is converted
 // alone, because a lane's 16-byte unit of Q4_K nibbles holds halves of two different blocks: the same real number,
 // rounded at another place).  Lanes add their terms in unit order; a row's 32 lanes are summed by a fixed tree.
@@ -131,6 +132,49 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
         }
       }
     }
+  } else if constexpr (QT == QT_IQ4_XS) {
+    const PlanesIQ4XS pl = planes_iq4xs(plane_rows, nsb);
+    const int ib = hl & 7;  // a unit is one 32-block: low nibbles = its elements 0..15, high = 16..31
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 3;
+      const int e1 = sb * 256 + 32 * ib;
+      uint4 a1[TB], a2[TB];
+      float sa[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) {
+        const int tt = t < T ? t : 0;
+        a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
+        a2[t] = *(const uint4*)(aq + (size_t)tt * K + e1 + 16);
+        sa[t] = asc[(size_t)(e1 >> 5) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const int n = min(r0 + r, N - 1);
+        const uint4 w = *(const uint4*)(raw + pl.qs + (size_t)n * nsb * 128 + (size_t)u * 16);
+        const uint2 h = *(const uint2*)(raw + pl.hdr + ((size_t)n * nsb + sb) * 8);
+        const int ls = (int)(((h.y >> (4 * ib)) & 0xFu) | ((((h.x >> 16) >> (2 * ib)) & 3u) << 4)) - 32;
+        const float d = f16_bits_to_f32(h.x);
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+        uint32_t w1[4], w2[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          w1[k] = iq4_lookup(ww[k]);
+          w2[k] = iq4_lookup(ww[k] >> 4);
+        }
+#pragma unroll
+        for (int t = 0; t < TB; ++t) {
+          int i1 = dot4(w1[0], a1[t].x, 0);
+          i1 = dot4(w1[1], a1[t].y, i1);
+          i1 = dot4(w1[2], a1[t].z, i1);
+          i1 = dot4(w1[3], a1[t].w, i1);
+          i1 = dot4(w2[0], a2[t].x, i1);
+          i1 = dot4(w2[1], a2[t].y, i1);
+          i1 = dot4(w2[2], a2[t].z, i1);
+          i1 = dot4(w2[3], a2[t].w, i1);
+          acc[r][t] += sa[t] * d * (float)(ls * i1);
+        }
+      }
+    }
   } else {
     const PlanesQ80 pl = planes_q80(plane_rows, nsb);
     for (int u = hl; u < units; u += 32) {
@@ -203,3 +247,4 @@ GEMV_ALL(8)
 GEMV_ALL(12)
 GEMV_ALL(13)
 GEMV_ALL(14)
+GEMV_ALL(23)

@@ -6,6 +6,7 @@
 //   Q8_0 : res += (sa[m][b] * d[n][b]) * (float)I
 //   Q4_K : res += (sa[m][b] * (d[n] * sc[n][b])) * (float)I  -  (sa[m][b] * (float)S[m][b]) * (dmin[n] * mn[n][b])
 //   Q5_K : as Q4_K (values 0..31)
+//   IQ4_XS: res += (sa[m][b] * (d[n] * ls[n][b])) * (float)I      (ls: the block's 6-bit scale - 32)
 // with S the sum of the block's 32 int8 activations.  Blocks are added in K order.
 //
 // The scheme needs one f32 scale per (token, weight row, block), so the vector ALU, not the matrix pipe, bounds it.
@@ -73,6 +74,18 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
     }
     const int n = min(n0 + (t >> 1), N - 1);
     r.h = *(const uint4*)(raw + pl.hdr + ((row_base + n) * nsb + s) * 16);
+  } else if constexpr (QT == QT_IQ4_XS) {
+    const PlanesIQ4XS pl = planes_iq4xs(rows_total, nsb);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int id = t + 256 * i, row = id >> 2, c = id & 3;
+      const int n = min(n0 + row, N - 1);
+      r.w[i] = *(const uint4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 128 + 64 * hh + 16 * c);
+    }
+    const int n = min(n0 + (t >> 1), N - 1);
+    const uint2 h = *(const uint2*)(raw + pl.hdr + ((row_base + n) * nsb + s) * 8);
+    r.h.x = h.x;
+    r.h.y = h.y;
   } else {
     const PlanesQ80 pl = planes_q80(rows_total, nsb);
 #pragma unroll
@@ -134,6 +147,22 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
       L.ws[2 * p + 1][row] = d * (float)sc1;
       L.v[2 * p][row] = -(dmin * (float)mn0);
       L.v[2 * p + 1][row] = -(dmin * (float)mn1);
+    }
+  } else if constexpr (QT == QT_IQ4_XS) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {  // block 4 hh + c of the superblock: 16 bytes -> its 32 values
+      const int id = t + 256 * i, row = id >> 2, c = id & 3;
+      const uint4 w = r.w[i];
+      *(uint4*)&L.wq[row][32 * c] = make_uint4(iq4_lookup(w.x), iq4_lookup(w.y), iq4_lookup(w.z), iq4_lookup(w.w));
+      *(uint4*)&L.wq[row][32 * c + 16] = make_uint4(iq4_lookup(w.x >> 4), iq4_lookup(w.y >> 4), iq4_lookup(w.z >> 4), iq4_lookup(w.w >> 4));
+    }
+    const int row = t >> 1, p = t & 1;
+    const float d = f16_bits_to_f32(r.h.x);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int ib = 4 * hh + 2 * p + k;
+      const int ls = (int)(((r.h.y >> (4 * ib)) & 0xFu) | ((((r.h.x >> 16) >> (2 * ib)) & 3u) << 4)) - 32;
+      L.ws[2 * p + k][row] = d * (float)ls;
     }
   } else {
 #pragma unroll
@@ -1441,6 +1470,9 @@ GEMM2_TILES_INST(8)
 // Q5_K: the register-staged body (the Q4_K arithmetic on values 0..31)
 GEMM2_INST(13)
 GEMM2_TILES_INST(13)
+// IQ4_XS: the register-staged body too (codes to values through the table as they are stored to LDS)
+GEMM2_INST(23)
+GEMM2_TILES_INST(23)
 // Q4_K -DBM=64: 64 tokens x 256 rows per work-group (grid ceil(N / 256) * ceil(M / 64) work-groups), K from 0
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,

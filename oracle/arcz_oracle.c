@@ -16,6 +16,7 @@
  *   orc_quantize_rows_q8_0              golden + compiled ref; round trip bound
  *   orc_act_residual                    PARITY UNPINNED (no reference CPU twin, no vector); identities and bounds only
  *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
+ *   IQ4_XS decode                       closed-form block; live comparison with the compiled reference header
  *   Q5_K decode                         closed-form block; golden vectors (tests/golden/ref_vectors_q5k.npz) and live
  *                                       comparison with the compiled reference header
  *   orc_block_sums                      brute-force integer sums in numpy (int64)
@@ -24,7 +25,7 @@
  *   orc_moe_route                       stable-sort top-k in numpy (the reference's own CPU check, tests/test_route.cpp:28-44)
  *   orc_moe_scan / orc_moe_scatter      invariants (bijection, contiguity, counts) + numpy restatement
  *   orc_moe_layer                       composition of the above, compared with a numpy float64 composition
- * The f32 -> Q4_K / Q5_K / Q6_K quantizers used to make synthetic weights are not part of the reference (it has none) and
+ * The f32 -> Q4_K / Q5_K / Q6_K / IQ4_XS quantizers used to make synthetic weights are not part of the reference (it has none) and
  * not part of this file: they are input generators of the product's bench/test utilities; parity unpinned by design.
  */
 #include <math.h>
@@ -44,6 +45,9 @@
 #define ORC_Q5_K 13u
 #define ORC_Q45(t) ((t) == ORC_Q4_K || (t) == ORC_Q5_K) /* d, dmin, 6-bit scales and mins */
 #define ORC_Q6_K 14u
+#define ORC_IQ4_XS 23u
+/* one int scale per 16 (Q6_K) or per 32 values (IQ4_XS: the same one for both halves), kept in sc6[], and no mins */
+#define ORC_Q6LIKE(t) ((t) == ORC_Q6_K || (t) == ORC_IQ4_XS)
 
 /* ---------------------------------------------------------------- fp16 (src/quants.h:17-52) */
 
@@ -104,6 +108,7 @@ int orc_sb_bytes(uint32_t type) {
     case ORC_Q4_K: return 144;
     case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
+    case ORC_IQ4_XS: return 136;
     default: return 0;
   }
 }
@@ -125,7 +130,11 @@ static void scale_min_k4(int j, const uint8_t* q, int* sc, int* mn) {
  *   Q5_K: the same with q 0..31                  (src/quants.h:101-108)
  *   Q6_K: q 0..63 (offset 32 NOT removed), sc6[16], d   (src/quants.h:115-134)
  *   Q8_0: q -128..127, d8[8]                    (src/quants.h:149-157)
+ *   IQ4_XS: q = the 16-entry table's value of each 4-bit code, sc6[2 b] = sc6[2 b + 1] = the block's 6-bit scale - 32,
+ *           d                                   (src/quants.h:297-311; the table: src/iq_tables.h:364-367)
  */
+static const int8_t iq4_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
 typedef struct {
   float d, dmin;
   int sc[8], mn[8];
@@ -172,6 +181,20 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
       }
     return 0;
   }
+  if (type == ORC_IQ4_XS) { /* f16 d, 16 bits of scale high parts, 4 bytes of low nibbles, 8 blocks of 16 bytes: the low
+                               nibbles are a block's elements 0..15, the high ones 16..31 */
+    o->d = orc_fp16_to_f32(rd16(p));
+    const unsigned sh = rd16(p + 2);
+    for (int ib = 0; ib < 8; ++ib) {
+      const int ls = ((p[4 + ib / 2] >> (4 * (ib % 2))) & 0xF) | (((sh >> (2 * ib)) & 3) << 4);
+      o->sc6[2 * ib] = o->sc6[2 * ib + 1] = ls - 32;
+      for (int j = 0; j < 16; ++j) {
+        o->q[32 * ib + j] = iq4_values[p[8 + 16 * ib + j] & 0xF];
+        o->q[32 * ib + 16 + j] = iq4_values[p[8 + 16 * ib + j] >> 4];
+      }
+    }
+    return 0;
+  }
   if (type == ORC_Q8_0) {
     for (int b = 0; b < 8; ++b) {
       const uint8_t* blk = p + 34 * b;
@@ -199,6 +222,7 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
 static float sb_value(uint32_t type, const orc_sb* o, int e) {
   if (ORC_Q45(type)) return o->d * (float)o->sc[e / 32] * (float)o->q[e] - o->dmin * (float)o->mn[e / 32];
   if (type == ORC_Q6_K) return o->d * (float)o->sc6[e / 16] * (float)(o->q[e] - 32);
+  if (type == ORC_IQ4_XS) return o->d * (float)o->sc6[e / 16] * (float)o->q[e]; /* (src/quants.h:321-323 generic: wd * wsc * q) */
   return o->d8[e / 32] * (float)o->q[e];
 }
 
@@ -230,7 +254,7 @@ int orc_decode_row_fields(uint32_t type, const uint8_t* row, int K, int8_t* q, i
     orc_decode_sb(type, row + (size_t)s * bb, &o);
     for (int e = 0; e < 256; ++e) q[s * 256 + e] = (int8_t)sb_int(type, &o, e);
     for (int h = 0; h < 16; ++h) {
-      isc[s * 16 + h] = ORC_Q45(type) ? o.sc[h / 2] : type == ORC_Q6_K ? o.sc6[h] : 1;
+      isc[s * 16 + h] = ORC_Q45(type) ? o.sc[h / 2] : ORC_Q6LIKE(type) ? o.sc6[h] : 1;
       imn[s * 16 + h] = ORC_Q45(type) ? o.mn[h / 2] : 0;
     }
     for (int b = 0; b < 8; ++b) {
@@ -446,7 +470,7 @@ int orc_matmul_formula(uint32_t type, int form, const uint8_t* W, int N, int K, 
               t2[u] = (float)(o.sc[b] * lo + o.sc[b] * hi);
               m2[u] = (float)(o.mn[b] * bs0 + o.mn[b] * bs1);
               if (form == 0) res += sa * (o.d * t2[u] - o.dmin * m2[u]);
-            } else if (type == ORC_Q6_K) {
+            } else if (ORC_Q6LIKE(type)) {
               t2[u] = (float)(o.sc6[2 * b] * lo + o.sc6[2 * b + 1] * hi);
               m2[u] = 0.0f;
               if (form == 0) res += sa * o.d * t2[u];
@@ -466,7 +490,7 @@ int orc_matmul_formula(uint32_t type, int form, const uint8_t* W, int N, int K, 
           }
         }
         if (form == 1 && ORC_Q45(type)) res = fmaf(o.d, tq, fmaf(-o.dmin, tmn, res));
-        if (form == 1 && type == ORC_Q6_K) res = fmaf(o.d, tq, res);
+        if (form == 1 && ORC_Q6LIKE(type)) res = fmaf(o.d, tq, res);
       }
       Y[(size_t)m * ldy + n] = res;
     }

@@ -5,9 +5,10 @@ import numpy as np
 import arcinferzero_amd as az
 import oracle_lib as orc
 
-Q8_0, Q4_K, Q5_K, Q6_K = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K
-TYPES = (Q8_0, Q4_K, Q6_K, Q5_K)
-TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K, az.IQ4_XS
+TYPES = (Q8_0, Q4_K, Q6_K, Q5_K, IQ4_XS)
+TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS"}
+IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64)
 
 
 def make_weights(qtype, N, K, seed):
@@ -74,6 +75,14 @@ def unit_scale_weights(qtype, N, K, seed):
             blk[..., 48 + 32 * j:48 + 32 * j + 32] = ((lo & 15) | ((hi & 15) << 4)).astype(np.uint8)
             blk[..., 16:48] |= (((lo >> 4) << (2 * j)) | ((hi >> 4) << (2 * j + 1))).astype(np.uint8)
         return blk.reshape(-1), q.reshape(N, K)
+    if qtype == IQ4_XS:
+        c = rng.integers(0, 16, size=(N, nsb, 8, 32), dtype=np.int64)     # codes per block
+        blk = np.zeros((N, nsb, 136), np.uint8)
+        blk[..., 0:2] = one
+        blk[..., 2:4] = [0xAA, 0xAA]    # high two bits of every 6-bit scale = 2, low nibble 1: 33 - 32 = 1
+        blk[..., 4:8] = 0x11
+        blk[..., 8:] = (c[..., :16] | (c[..., 16:] << 4)).astype(np.uint8).reshape(N, nsb, 128)
+        return blk.reshape(-1), IQ4_VALUES[c].reshape(N, K)
     if qtype == Q6_K:
         q = rng.integers(0, 64, size=(N, nsb, 256), dtype=np.int64)
         blk = np.zeros((N, nsb, 210), np.uint8)

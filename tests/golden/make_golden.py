@@ -5,8 +5,8 @@ container that has the reference tree (make -C oracle ref); the fixture it write
 
 Functions covered: fp16_to_f32 / f32_to_fp16 (:17-52), decode_sb / dequant_row for Q8_0, Q4_K, Q6_K (:89-158,
 :519-622), quantize_act_cpu (:626-643, both scale widths), quantize_rows_q8_0 (:429-442).  A second file,
-ref_vectors_q5k.npz, holds the same decode vectors for Q5_K (:91-113), drawn from a generator of its own so that the
-first file's bytes stay what they were.
+ref_vectors_types2.npz, holds the same decode vectors for Q5_K (:91-113) and IQ4_XS (:297-311), drawn from a generator
+of its own so that the first file's bytes stay what they were.
 """
 import ctypes as C
 import os
@@ -107,5 +107,11 @@ assert ref.ref_decode_sb(C.c_uint32(13), orc.ptr(first), orc.ptr(q), orc.ptr(sc)
                          C.byref(d), C.byref(dm)) == 0
 out5["q5k_sb0_q"] = q.copy(); out5["q5k_sb0_sc"] = sc.copy(); out5["q5k_sb0_mn"] = mn.copy()
 out5["q5k_sb0_d"] = np.array([d.value, dm.value], np.float32)
-np.savez_compressed(os.path.join(HERE, "ref_vectors_q5k.npz"), **out5)
-print("wrote", os.path.join(HERE, "ref_vectors_q5k.npz"), {k: v.shape for k, v in out5.items()})
+# ---- IQ4_XS blocks (136 bytes: d, 16 bits + 4 bytes of scales, 128 bytes of 4-bit codes)
+raw = rng.integers(0, 256, size=(nblk, 136), dtype=np.uint8)
+raw[:, 0:2] = finite_f16(nblk).reshape(-1, 1).view(np.uint8)
+raw = raw.reshape(-1)
+out5["iq4xs_raw"] = raw
+out5["iq4xs_dequant"] = orc.dequant_rows(23, raw, N, K, lib=ref)
+np.savez_compressed(os.path.join(HERE, "ref_vectors_types2.npz"), **out5)
+print("wrote", os.path.join(HERE, "ref_vectors_types2.npz"), {k: v.shape for k, v in out5.items()})

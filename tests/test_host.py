@@ -95,6 +95,10 @@ def test_repack_planes_layout(qtype):
             assert np.array_equal(P[o:o + u * n].reshape(u, n), sb[:, lo:lo + n])
             o += u * n
         assert not P[o:].any() and P.size % 16 == 0
+    elif qtype == az.IQ4_XS:
+        sb = W.reshape(u, 136)
+        assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 8:]) and np.array_equal(P[u * 128:u * 136].reshape(u, 8), sb[:, :8])
+        assert not P[u * 136:].any() and P.size % 16 == 0
     else:
         blk = W.reshape(u, 8, 34)
         assert np.array_equal(P[:u * 256].reshape(u, 8, 32), blk[:, :, 2:]) and np.array_equal(P[u * 256:].reshape(u, 8, 2), blk[:, :, :2])
@@ -106,7 +110,7 @@ def test_q8_0_quantizer_is_the_reference_one():
     assert np.array_equal(az.quantize_rows(az.Q8_0, w), orc.quantize_rows_q8_0(w))
 
 
-@pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q5_K, 0.04), (az.Q6_K, 0.02), (az.Q8_0, 0.006)])
+@pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q5_K, 0.04), (az.Q6_K, 0.02), (az.Q8_0, 0.006), (az.IQ4_XS, 0.09)])
 def test_block_makers_make_valid_close_blocks(qtype, rel):
     """The Q4_K / Q5_K / Q6_K block makers are input generators (the reference has none): valid fields and a round-trip
     error of the size the bit width allows."""
@@ -124,6 +128,8 @@ def test_block_makers_make_valid_close_blocks(qtype, rel):
         assert q.min() >= 0 and q.max() <= 31 and isc.max() <= 63 and imn.max() <= 63 and len(np.unique(q)) == 32
     elif qtype == az.Q6_K:
         assert q.min() >= -32 and q.max() <= 31 and isc.max() <= 127 and isc.min() >= 1
+    elif qtype == az.IQ4_XS:
+        assert isc.min() >= 1 and isc.max() <= 31 and len(np.unique(q)) == 16
 
 
 def test_generators_are_seeded_and_normal():

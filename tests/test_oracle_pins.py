@@ -13,9 +13,9 @@ import oracle_lib as orc
 from common import TYPES, make_acts, make_weights, rel_err_rows, unit_scale_acts, unit_scale_weights
 
 G = dict(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz")))
-G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_q5k.npz")))
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
-NAMES = {Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k", Q8_0: "q80"}
+G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_types2.npz")))
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = 8, 12, 13, 14, 23
+NAMES = {Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k", Q8_0: "q80", IQ4_XS: "iq4xs"}
 
 
 # ---------------------------------------------------------------- fp16
@@ -51,6 +51,8 @@ def test_dequant_golden(qtype):
     nm = NAMES[qtype]
     got = orc.dequant_rows(qtype, G[f"{nm}_raw"], 4, 512)
     assert np.array_equal(got.view(np.uint32), G[f"{nm}_dequant"].view(np.uint32))
+    if qtype == IQ4_XS:
+        return                              # (rows only: its decoded fields are pinned by the closed form below)
     q, isc, imn, d, dmin = orc.decode_row_fields(qtype, G[f"{nm}_raw"][:512 // 256 * orc.SB_BYTES[qtype]], 512)
     gq = G[f"{nm}_sb0_q"].astype(np.int32) - (32 if qtype == Q6_K else 0)
     assert np.array_equal(q[:256], gq)
@@ -128,6 +130,31 @@ def test_q5k_closed_form():
     assert np.array_equal(orc.dequant_rows(Q5_K, blk, 1, K)[0], exp)
     q, isc, imn, dd, dm = orc.decode_row_fields(Q5_K, blk, K)
     assert np.array_equal(q, [(e * 7 + 3) % 32 for e in range(256)])
+
+
+def test_iq4xs_closed_form():
+    """Every code in every position, scales across their range (the 6-bit scale's low nibble and its two high bits come
+    from different places), expected values from the table written out here (src/quants.h:297-311)."""
+    tab = [-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113]
+    K = 256
+    blk = np.zeros(136, np.uint8)
+    d = 0.0625
+    blk[0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+    ls = [0, 63, 31, 32, 17, 46, 5, 58]
+    sh = 0
+    for b in range(8):
+        blk[4 + b // 2] |= (ls[b] & 15) << (4 * (b % 2))
+        sh |= (ls[b] >> 4) << (2 * b)
+    blk[2:4] = [sh & 0xFF, sh >> 8]
+    exp = np.zeros(K, np.float32)
+    for e in range(256):
+        c = (e * 5 + e // 32) % 16
+        b, j = divmod(e, 32)
+        blk[8 + 16 * b + j % 16] |= c << (4 * (j // 16))
+        exp[e] = d * (ls[b] - 32) * tab[c]
+    assert np.array_equal(orc.dequant_rows(IQ4_XS, blk, 1, K)[0], exp)
+    q, isc, imn, dd, dm = orc.decode_row_fields(IQ4_XS, blk, K)
+    assert np.array_equal(isc, np.repeat(np.array(ls) - 32, 2)) and not imn.any() and (dd == d).all()
 
 
 def test_q6k_closed_form():
