@@ -42,11 +42,13 @@ struct alignas(16) Gemm2Lds {
 };
 
 // The global loads of one K step, held in registers until the step before it has been computed.
+// (native vector types: arrays of HIP's uint4, a struct, stay in scratch memory when they are passed around)
+typedef uint32_t g2_u4 __attribute__((ext_vector_type(4)));
 template <int QT> struct StepRegs {
-  uint4 a[4];                        // 4 x 16 int8 activation values
-  uint4 w[QT == QT_Q8_0 ? 4 : 2];    // packed weights
+  g2_u4 a[4];                        // 4 x 16 int8 activation values
+  g2_u4 w[QT == QT_Q8_0 ? 4 : 2];    // packed weights
   uint32_t qh[2];                    // Q5_K: the words of fifth bits of the two 16-byte units above
-  uint4 h;                           // Q4_K / Q5_K header of the thread's row (Q8_0: .x = two f16 scales)
+  g2_u4 h;                           // Q4_K / Q5_K header of the thread's row (Q8_0: .x = two f16 scales)
   float sa[4];                       // scale of the block whose first half the thread stages (even chunks only)
 };
 
@@ -60,7 +62,7 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
   for (int i = 0; i < 4; ++i) {
     const int id = t + 256 * i, row = id >> 3, c = id & 7;
     const int m = max(L.rowmap[row], 0);
-    r.a[i] = *(const uint4*)(aq + (size_t)m * K + e0 + 16 * c);
+    r.a[i] = *(const g2_u4*)(aq + (size_t)m * K + e0 + 16 * c);
     r.sa[i] = asc[(size_t)(s * 8 + 4 * hh + (c >> 1)) * M + m];
   }
   if constexpr (QT == QT_Q4_K || QT == QT_Q5_K) {
@@ -69,18 +71,18 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
     for (int i = 0; i < 2; ++i) {
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
       const int n = min(n0 + row, N - 1);
-      r.w[i] = *(const uint4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 128 + 64 * hh + 16 * c);
+      r.w[i] = *(const g2_u4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 128 + 64 * hh + 16 * c);
       if constexpr (QT == QT_Q5_K) r.qh[i] = *(const uint32_t*)(raw + pl.qh + ((row_base + n) * nsb + s) * 32 + 16 * hh + 4 * c);
     }
     const int n = min(n0 + (t >> 1), N - 1);
-    r.h = *(const uint4*)(raw + pl.hdr + ((row_base + n) * nsb + s) * 16);
+    r.h = *(const g2_u4*)(raw + pl.hdr + ((row_base + n) * nsb + s) * 16);
   } else if constexpr (QT == QT_IQ4_XS) {
     const PlanesIQ4XS pl = planes_iq4xs(rows_total, nsb);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
       const int n = min(n0 + row, N - 1);
-      r.w[i] = *(const uint4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 128 + 64 * hh + 16 * c);
+      r.w[i] = *(const g2_u4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 128 + 64 * hh + 16 * c);
     }
     const int n = min(n0 + (t >> 1), N - 1);
     const uint2 h = *(const uint2*)(raw + pl.hdr + ((row_base + n) * nsb + s) * 8);
@@ -92,7 +94,7 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
     for (int i = 0; i < 4; ++i) {
       const int id = t + 256 * i, row = id >> 3, c = id & 7;
       const int n = min(n0 + row, N - 1);
-      r.w[i] = *(const uint4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 256 + 128 * hh + 16 * c);
+      r.w[i] = *(const g2_u4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 256 + 128 * hh + 16 * c);
     }
     const int n = min(n0 + (t >> 1), N - 1);
     r.h.x = *(const uint32_t*)(raw + pl.d + (((row_base + n) * nsb + s) * 8 + 4 * hh + 2 * (t & 1)) * 2);
@@ -108,7 +110,7 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int id = t + 256 * i, row = id >> 3, c = id & 7;
-    *(uint4*)&L.act[row][16 * c] = r.a[i];
+    *(g2_u4*)&L.act[row][16 * c] = r.a[i];
     if constexpr (Q45) {
       int sh = dot4(r.a[i].x, 0x01010101u, 0);
       sh = dot4(r.a[i].y, 0x01010101u, sh);
@@ -126,7 +128,7 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
-      const uint4 w = r.w[i];
+      const g2_u4 w = r.w[i];
       const int off = 64 * (c >> 1) + 16 * (c & 1);
       if constexpr (QT == QT_Q5_K) {
         const uint32_t H = r.qh[i];
@@ -152,7 +154,7 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {  // block 4 hh + c of the superblock: 16 bytes -> its 32 values
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
-      const uint4 w = r.w[i];
+      const g2_u4 w = r.w[i];
       *(uint4*)&L.wq[row][32 * c] = make_uint4(iq4_lookup(w.x), iq4_lookup(w.y), iq4_lookup(w.z), iq4_lookup(w.w));
       *(uint4*)&L.wq[row][32 * c + 16] = make_uint4(iq4_lookup(w.x >> 4), iq4_lookup(w.y >> 4), iq4_lookup(w.z >> 4), iq4_lookup(w.w >> 4));
     }
@@ -168,7 +170,7 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int id = t + 256 * i, row = id >> 3, c = id & 7;
-      *(uint4*)&L.wq[row][16 * c] = r.w[i];
+      *(g2_u4*)&L.wq[row][16 * c] = r.w[i];
     }
     const int row = t >> 1, p = t & 1;
     L.ws[2 * p][row] = f16_bits_to_f32(r.h.x);
