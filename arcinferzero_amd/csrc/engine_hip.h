@@ -309,6 +309,31 @@ class Engine {
       throw std::runtime_error(std::string("matmul ") + name + ": the output does not fit C");
     int a = acc;
     cl_mem tabs = nullptr;  // (the reference's codebook tables: none of the three types has one)
+    // Q4_K and a few tokens: the matrix-vector form on the matrix pipe (gemv_mm), K in slices of at most 24 superblocks
+    // that accumulate.  It takes 9-16 tokens in chunks of 16 rows (what the reference pads them to, zero/engine.h:522;
+    // the rows from T on come out as zeros, as the GEMM writes them: 27 against 95 us at 17408 x 5120), and 3-8 tokens
+    // where it is the faster one: 7 and 8 always (26 against 30 us), 3-6 when the tokens do not fit the LDS of the
+    // dot-product kernels (5120 x 17408, 4 tokens: 50 against 88 us).  Not with two-pass inputs (their second half
+    // goes through the kernels below).  ARCZ_GEMV_MM=0: off.
+    static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
+    const bool mm_ok = !mm_off && !q2mm_ && w.type == GGML_Q4_K && a <= 1;
+    auto gemv_mm = [&] {
+      int N = w.N, K = w.K, M = Mp, T = cur_T_;
+      rd_bytes += raw_bytes(w);
+      const int nsb = K / 256, slices = (nsb + 23) / 24;
+      cl_kernel k = kernel("decode", "-DQT=12", "gemv_mm");
+      const size_t groups = (size_t)(N + 15) / 16;
+      size_t g1 = std::min<size_t>(groups, (size_t)arcz_device_cus()) * 512, l1 = 512;
+      for (int sl = 0; sl < slices; ++sl) {
+        int s0 = nsb * sl / slices, s1 = nsb * (sl + 1) / slices, ac = sl == 0 ? a : 1;
+        set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, ac, s0, s1);
+        run(name, k, 1, &g1, &l1);
+      }
+    };
+    if (mm_ok && cur_T_ >= 9 && cur_T_ <= 16 && Mp == 16) {
+      gemv_mm();
+      return;
+    }
     if (cur_T_ >= 1 && cur_T_ <= 8) {
       if (a > 1) throw std::logic_error(std::string("GEMV with a fused epilogue: ") + name);
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
@@ -330,7 +355,13 @@ class Engine {
       const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= 65536;
       const int tbl = q2f ? tb2 : T <= 2 ? T : T <= 4 ? 4 : 8;
       const size_t lds = lds_of(tbl);
-      if (!force_v && lpr && lds <= 65536) {
+      const bool fits = !force_v && lpr && lds <= 65536;
+      if (mm_ok && T >= 3 && (T >= 7 || !fits)) {
+        rd_bytes -= raw_bytes(w);  // (counted by gemv_mm)
+        gemv_mm();
+        return;
+      }
+      if (fits) {
         const int pf = (units + lpr - 1) / lpr, tb = tbl;
         // one round of resident work-groups, passes of rows dealt to them in turn (ARCZ_GEMV_WPC: work-groups per
         // compute unit; two measured best: more add staging work and spread the reads over more rows at a time)

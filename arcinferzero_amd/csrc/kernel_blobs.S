@@ -15,6 +15,7 @@
     BLOB arcz_blob_decode_q5k, "decode_q5k.hsaco"
     BLOB arcz_blob_decode_q6k, "decode_q6k.hsaco"
     BLOB arcz_blob_decode_iq4xs, "decode_iq4xs.hsaco"
+    BLOB arcz_blob_decode_mm, "decode_mm.hsaco"
     BLOB arcz_blob_gemm, "gemm.hsaco"
     BLOB arcz_blob_moe, "moe.hsaco"
     .section .note.GNU-stack,"",@progbits

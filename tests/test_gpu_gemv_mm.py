@@ -1,0 +1,71 @@
+"""gemv_mm: the Q4_K matrix-vector form for a few tokens on the matrix pipe.  The engine takes it for 9-16 tokens in a
+16-row chunk, for 7-8 tokens, and for 3-6 tokens whose activations do not fit the LDS of the dot-product kernels; every
+case here lands on it.  Against the double-accumulated dequantized reference (1e-3 as max|err| / max|ref| per token
+row), with unit scales against the exact integer sums, with K in one slice and in several (later slices accumulate),
+storing and accumulating, rows that do not fill a group of 16."""
+import numpy as np
+import pytest
+
+import arcinferzero_amd as az
+import oracle_lib as orc
+from common import make_acts, make_weights, pad_rows, quantize_padded, rel_err_rows, unit_scale_acts, unit_scale_weights
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def eng(rt):
+    e = az.Engine(16, 17408)
+    yield e
+    e.close()
+
+
+CASES = [(7, 100, 256), (8, 1000, 5120), (9, 333, 2048), (13, 4097, 1024), (16, 64, 6144), (16, 250, 6400),
+         (3, 77, 17408), (6, 300, 17408), (12, 129, 17408)]
+
+
+@pytest.mark.parametrize("T,N,K", CASES)
+def test_gemv_mm_parity(eng, T, N, K):
+    print(f"gemv_mm T={T} N={N} K={K}", flush=True)
+    W = make_weights(az.Q4_K, N, K, seed=800 + T)
+    x = make_acts(T, K, seed=801 + T, outliers=True)
+    w = eng.make_weight(az.Q4_K, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, 16, T)
+    rows = T if T <= 8 else 16
+    cb = az.Runtime.alloc(rows * N * 4).fill(0xFFFFFFFF)
+    eng.matmul("mm", w, 16, cb, N, 0, 0)
+    y = cb.read(np.float32, rows * N).reshape(rows, N)
+    aq, asc, _ = quantize_padded(x, 16)
+    ref = orc.matmul_ref(az.Q4_K, W, N, K, aq[:T], asc)
+    assert np.isfinite(y).all()
+    assert rel_err_rows(y[:T], ref).max() <= 1e-3
+    if rows > T:
+        assert not y[T:].any()                       # the chunk's padding rows: zeros, as the GEMM writes them
+    eng.matmul("mm", w, 16, cb, N, 0, 1)             # accumulate: C + the same product
+    y2 = cb.read(np.float32, rows * N).reshape(rows, N)
+    assert rel_err_rows(y2[:T], 2.0 * ref).max() <= 1e-3
+    # the same bits on every run
+    eng.matmul("mm", w, 16, cb, N, 0, 0)
+    assert np.array_equal(cb.read(np.float32, rows * N).reshape(rows, N), y)
+    for b in (cb, xb):
+        b.free()
+    w.free()
+
+
+@pytest.mark.parametrize("T,N,K", [(8, 48, 512), (16, 37, 7168)])
+def test_gemv_mm_unit_scales_exact(eng, T, N, K):
+    """All scales 1: the f32 output is the exact integer sum (partial sums stay below 2^24)."""
+    W, wi = unit_scale_weights(az.Q4_K, N, K, seed=820)
+    x = unit_scale_acts(T, K, seed=821)
+    w = eng.make_weight(az.Q4_K, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, 16, T)
+    rows = T if T <= 8 else 16
+    cb = az.Runtime.alloc(rows * N * 4)
+    eng.matmul("mm", w, 16, cb, N, 0, 0)
+    y = cb.read(np.float32, rows * N).reshape(rows, N)[:T]
+    assert np.array_equal(y, (x.astype(np.int64) @ wi.T).astype(np.float32))
+    for b in (cb, xb):
+        b.free()
+    w.free()
