@@ -64,25 +64,47 @@ extern "C" __global__ __launch_bounds__(512, 1) void gemv_mm__QT12(
   const int gd = (int)gridDim.x;
   mm_load(ra, raw, pl, nsb, min(min(grp, groups - 1) * 16 + n16, N - 1), g, wave, s_begin, sbs);
 
-  // ---- staging: 16-byte chunks of the 16 token rows (tokens from T on: zeros), the blocks' scales and scaled sums
-  const int cpr = Ks >> 4;  // chunks per row (even)
-  for (int c = tid; c < 16 * cpr; c += 512) {
-    const int t = c / cpr, k16 = c - t * cpr;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    float sa = 0.0f;
-    if (t < T) {
-      v = *(const uint4*)(aq + (size_t)t * K + (size_t)s_begin * 256 + k16 * 16);
-      sa = asc[(size_t)(s_begin * 8 + (k16 >> 1)) * M + t];
+  // ---- staging: wave w takes token rows 2 w and 2 w + 1 (tokens from T on: zeros), a lane their 16-byte chunks lane,
+  // lane + 64, ...; all loads first (an index past the row's end is clamped: the lanes that get the same chunk store
+  // the same bytes), so the staging costs one memory latency.  Per block the tokens' scale and scaled sum of the 32
+  // values (the two lanes of a block add their halves' sums).
+  {
+    constexpr int NCH = MM_WAVES * MM_SPW * 16 / 64;  // chunks per lane and row at most
+    const int cpr = Ks >> 4;                          // chunks per row (even)
+    mm_u4 va[2][NCH];
+    float vs[2][NCH];
+#pragma unroll
+    for (int r2 = 0; r2 < 2; ++r2) {
+      const int t = 2 * wave + r2, tt = t < T ? t : 0;
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int k16 = min(lane + 64 * i, cpr - 1);
+        va[r2][i] = *(const mm_u4*)(aq + (size_t)tt * K + (size_t)s_begin * 256 + k16 * 16);
+        vs[r2][i] = asc[(size_t)(s_begin * 8 + (k16 >> 1)) * M + tt];
+      }
     }
-    *(uint4*)(A + t * astride + k16 * 16) = v;
-    int s = dot4(v.x, 0x01010101u, 0);
-    s = dot4(v.y, 0x01010101u, s);
-    s = dot4(v.z, 0x01010101u, s);
-    s = dot4(v.w, 0x01010101u, s);
-    s += __shfl_xor(s, 1, 64);  // (the block's other half: the neighbouring lane's chunk; 512 and cpr are even)
-    if ((k16 & 1) == 0) {
-      SA[(k16 >> 1) * 16 + t] = sa;
-      U[(k16 >> 1) * 16 + t] = sa * (float)s;
+#pragma unroll
+    for (int r2 = 0; r2 < 2; ++r2) {
+      const int t = 2 * wave + r2;
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int k16 = min(lane + 64 * i, cpr - 1);
+        mm_u4 v = va[r2][i];
+        float sa = vs[r2][i];
+        if (t >= T) { v = mm_u4{0, 0, 0, 0}; sa = 0.0f; }
+        *(mm_u4*)(A + t * astride + k16 * 16) = v;
+        int sm = dot4(v.x, 0x01010101u, 0);
+        sm = dot4(v.y, 0x01010101u, sm);
+        sm = dot4(v.z, 0x01010101u, sm);
+        sm = dot4(v.w, 0x01010101u, sm);
+        // (the block's other half is the neighbouring lane's chunk; for the clamped lanes of the last chunk, an odd
+        //  one, the neighbour holds the same chunk and they are not the ones that store)
+        sm += __shfl_xor(sm, 1, 64);
+        if ((k16 & 1) == 0) {
+          SA[(k16 >> 1) * 16 + t] = sa;
+          U[(k16 >> 1) * 16 + t] = sa * (float)sm;
+        }
+      }
     }
   }
   __syncthreads();
@@ -149,8 +171,8 @@ extern "C" __global__ __launch_bounds__(512, 1) void gemv_mm__QT12(
 #pragma unroll
     for (int i = 0; i < 4; ++i) red[(wave * 16 + 4 * g + i) * 16 + n16] = acc[i];
     __syncthreads();
-    if (tid < 256) {
-      const int t = tid >> 4, n = grp * 16 + (tid & 15);
+    if (tid >= 256) {  // (the upper four waves: the ones with fewer superblocks when these do not divide by 8)
+      const int t = (tid - 256) >> 4, n = grp * 16 + (tid & 15);
       float v = 0.0f;
 #pragma unroll
       for (int w = 0; w < MM_WAVES; ++w) v += red[(w * 16 + t) * 16 + (tid & 15)];
