@@ -56,13 +56,11 @@ extern "C" __global__ __launch_bounds__(512, 1) void gemv_mm__QT12(
   const PlanesQ4K pl = planes_q4k((size_t)N, nsb);
   const int groups = (N + 15) >> 4;
 
-  // the first group's loads go out ahead of the staging
   // (two buffers with fixed names -- one chosen by a run-time index would live in memory: the next group is in flight
   //  while a group is computed)
   MmSb ra[MM_SPW], rb[MM_SPW];
   int grp = blockIdx.x;
   const int gd = (int)gridDim.x;
-  mm_load(ra, raw, pl, nsb, min(min(grp, groups - 1) * 16 + n16, N - 1), g, wave, s_begin, sbs);
 
   // ---- staging: wave w takes token rows 2 w and 2 w + 1 (tokens from T on: zeros), a lane their 16-byte chunks lane,
   // lane + 64, ...; all loads first (an index past the row's end is clamped: the lanes that get the same chunk store
@@ -83,6 +81,11 @@ extern "C" __global__ __launch_bounds__(512, 1) void gemv_mm__QT12(
         vs[r2][i] = asc[(size_t)(s_begin * 8 + (k16 >> 1)) * M + tt];
       }
     }
+    // the first group's rows right behind the staging loads: loads come back in order, so the stores below wait for
+    // the tokens alone while the rows are on their way (the other way round the tokens queued behind 12 MB of rows)
+    __builtin_amdgcn_sched_barrier(0);
+    mm_load(ra, raw, pl, nsb, min(min(grp, groups - 1) * 16 + n16, N - 1), g, wave, s_begin, sbs);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int r2 = 0; r2 < 2; ++r2) {
       const int t = 2 * wave + r2;
