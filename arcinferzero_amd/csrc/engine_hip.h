@@ -397,8 +397,49 @@ class Engine {
 
   // The prefill GEMM (zero/engine.h:1205-1250).  Token rows come in whole tiles (the reference pads a chunk to 128
   // rows from 128 tokens on, :521-522).
+  // Workspace of the short-chunk GEMM's partial tiles, [slices][Mp][N] f32: grown on demand, kept.
+  cl_mem sk_ws_ = nullptr;
+  size_t sk_ws_bytes_ = 0;
   void gemm_dense(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int a) {
     int M = Mp, N = w.N, K = w.K;
+    // Q4_K and Q8_0, a chunk so short that its tiles are fewer than two per compute unit: K is shared out over `ny`
+    // work-groups per tile, which store partial tiles in a workspace, and splitk_reduce adds the slices in order (the
+    // same bits on every run) and applies c_off and the accumulate mode.  One work-group needs 75 us for K = 5120, so
+    // 64 tokens x 17408 rows took 100 us whatever the tile; now 136 tiles x 3 pieces, 52 us (128 tokens: 101 -> 88 us;
+    // Q8_0 4096 x 4096: 64 tokens 41 -> 19 us, 256 tokens 44 -> 35 us).  ARCZ_Q4_SPLITK=0: off, =n: n pieces.
+    static const bool sk_off = getenv("ARCZ_Q4_SPLITK") && atoi(getenv("ARCZ_Q4_SPLITK")) == 0;
+    if (!sk_off && (w.type == GGML_Q4_K || w.type == GGML_Q8_0)) {
+      // (tiles of 64 tokens up to 64 tokens, else of 128: the pieces of all tiles together must fit the resident slots,
+      //  two work-groups per compute unit: one more piece than fits costs a whole second round)
+      const int tm = Mp <= 64 || w.type == GGML_Q8_0 ? 64 : 128;
+      const size_t tiles64 = (size_t)((Mp + tm - 1) / tm) * ((N + 127) / 128), slots = 2 * (size_t)arcz_device_cus();
+      const int nsb = K / 256;
+      static const int sk_force = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : 0;
+      int ny = (int)std::min<size_t>({(size_t)8, (size_t)nsb / 2, slots / std::max<size_t>(tiles64, 1)});
+      if (sk_force >= 2) ny = std::min(sk_force, nsb);
+      // (from three pieces on: with two, 256 tiles of Q8_0 4096 x 4096 x 512 went from 50 to 54 us, the reduce included)
+      if (ny >= 3 || (sk_force >= 2 && ny >= 2)) {
+        const size_t need = (size_t)ny * Mp * N * 4;
+        if (need > sk_ws_bytes_) {
+          if (sk_ws_) release(sk_ws_);
+          sk_ws_ = buf(need);
+          sk_ws_bytes_ = need;
+        }
+        cl_kernel k = kernel("gemm", std::string("-DQTYPE=") + std::to_string(w.type) + " -DACT32 -DBM=" + std::to_string(tm) +
+                                         " -DBN=128 -DSPLITK", "gemm");
+        cl_mem unused = nullptr;
+        int zero = 0, one = 1, ldw = N, s1 = nsb;
+        set_args(k, 0, w.raw, unused, aq_, asc_, absum_, sk_ws_, M, N, K, ldw, zero, zero, one, zero, s1);
+        size_t gws[2] = {tiles64 * 256, (size_t)ny}, lws[2] = {256, 1};
+        run(name, k, 2, gws, lws);
+        cl_kernel r = kernel("gemm", "", "splitk_reduce");
+        int nyy = ny;
+        set_args(r, 0, sk_ws_, nyy, C, M, N, ldc, c_off, a);
+        size_t g1 = ((size_t)M * N + 255) / 256 * 256, l1 = 256;
+        run(name, r, 1, &g1, &l1);
+        return;
+      }
+    }
     // tiles of 128 tokens x 128 rows (or 64 x 256) for Q4_K, 64 x 128 for Q6_K and Q8_0 (whose 64-token kernel measured 1.9 x the
     // 128-token one at 17408 x 5120 x 8192 and 3 x at 4096 x 4096 x 512; ARCZ_Q8_BM=128 brings the latter back)
     static const int q8_bm = getenv("ARCZ_Q8_BM") ? atoi(getenv("ARCZ_Q8_BM")) : 0;
@@ -407,7 +448,12 @@ class Engine {
     // Q4_K: tiles of 64 tokens x 256 rows (the same work per work-group and the same rate as 128 x 128) when the last
     // 128 token rows of a short chunk are at most half full (ARCZ_Q4_BM=64 always, =128 never)
     const bool q4_wide = w.type == GGML_Q4_K && (q4_bm == 64 || (q4_bm == 0 && Mp <= 1024 && ((Mp - 1) & 127) < 64));
+    // Q4_K, few tokens: 64 x 128 tiles when the larger ones would leave compute units idle (ARCZ_Q4_BN=128 always)
+    static const int q4_bn = getenv("ARCZ_Q4_BN") ? atoi(getenv("ARCZ_Q4_BN")) : 0;
+    static const int q4_small_max = getenv("ARCZ_Q4_SMALL") ? atoi(getenv("ARCZ_Q4_SMALL")) : 0;
+    const bool q4_small = w.type == GGML_Q4_K && (q4_bn == 128 || (q4_bn == 0 && Mp <= q4_small_max));
     cl_kernel k = q8_small  ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
+                  : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")
                   : q4_wide ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64", "gemm")
                             : gemm_kernel(w.type, false);
     // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
@@ -416,8 +462,8 @@ class Engine {
     static const int sk_sb = getenv("ARCZ_GEMM_SPLIT") ? std::max(0, atoi(getenv("ARCZ_GEMM_SPLIT"))) : 0;
     const int nsb = K / 256, splits = a != 2 && sk_sb > 0 ? (nsb + sk_sb - 1) / sk_sb : 1, rgroup = 1;
     cl_mem unused = nullptr;
-    const int bm = w.type == GGML_Q6_K || q8_small || q4_wide ? 64 : 128;  // token rows of a work-group's tile
-    const int bn = q4_wide ? 256 : 128;
+    const int bm = w.type == GGML_Q6_K || q8_small || q4_wide || q4_small ? 64 : 128;  // token rows of a work-group's tile
+    const int bn = q4_wide && !q4_small ? 256 : 128;
     const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + bn - 1) / bn);
     size_t gws[1] = {tiles * 256}, lws[1] = {256};
     for (int sp = 0; sp < splits; ++sp) {

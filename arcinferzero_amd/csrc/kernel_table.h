@@ -13,7 +13,7 @@ struct KernelSpec {
   const char* name;
   const char* requires_def;  // this entry is taken only when the -D string holds this name (nullptr: always)
   const char* args;
-  const char* variant[5];  // nullptr-terminated
+  const char* variant[6];  // nullptr-terminated
   HiddenDef hidden[6];     // {nullptr} terminated
   int local_x;             // threads per work-group the kernel is written for (0 = any)
 };
@@ -39,11 +39,14 @@ static const KernelSpec kKernelTable[] = {
     // ---- gemm
     {"gemm", "gemm", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "SPLITK", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "BN", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", "BM", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "splitk_reduce", nullptr, "pipiiiii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     // ---- moe
     {"moe", "moe_route", nullptr, "piipppp", {nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},

@@ -1486,6 +1486,75 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64(
   gemm4gu_body<false>(raw, raw, aq, asc, absum, C, M, N, K, (size_t)N, 0, m0, min(G6_BM, M - m0), n0, nullptr, ldc, c_off,
                       accumulate);
 }
+// Q4_K -DBM=64 -DBN=128: 64 tokens x 128 rows per work-group (grid ceil(N / 128) * ceil(M / 64)): the expert-tile body on
+// the dense matrix, for chunks so short that the larger tiles leave most compute units without a work-group
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64_BN128(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  gemm4_body(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0, min(G6_BM, M - m0),
+             n0, nullptr, 0, nullptr, 0);
+}
+// The same with K shared out over gridDim.y work-groups per tile (-DSPLITK): work-group (x, y) takes the y-th of
+// gridDim.y even pieces of superblocks [s_begin, s_end) and stores its partial tile in slice y of C, here a workspace
+// [gridDim.y][M][ldc] (c_off and accumulate apply in splitk_reduce, which adds the slices in order).  A chunk of 64
+// tokens gives 136 tiles for 256 compute units, and a tile's work-group needs 75 us to walk through K = 5120 alone.
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64_BN128_SPLITK1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm4_body(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+             s_begin + ns * (y + 1) / ny, (size_t)N, 0, m0, min(G6_BM, M - m0), n0, nullptr, 0, nullptr, 0);
+}
+// (-DBM=128 -DBN=128 -DSPLITK: the same over the 128 x 128 tiles of the dense kernel, for 65-128 tokens)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM128_BN128_SPLITK1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm3_body<false>(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+                    s_begin + ns * (y + 1) / ny, (size_t)N, 0, m0, min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
+}
+// (Q8_0 -DBM=64 -DBN=128 -DSPLITK: the 64-token form's tiles)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE8_ACT321_BM64_BN128_SPLITK1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm8_body(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny, s_begin + ns * (y + 1) / ny,
+             m0, min(G6_BM, M - m0), n0);
+}
+// splitk_reduce: C[m][c_off + n] (=, +=, silu(C) *) sum over the ny slices of ws [ny][M][N], slice 0 first.
+// grid: ceil(M * N / 256) work-groups of 256.
+extern "C" __global__ __launch_bounds__(256) void splitk_reduce(const float* __restrict__ ws, int ny, float* C, int M, int N,
+                                                                int ldc, int c_off, int accumulate) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, total = (size_t)M * N;
+  if (i >= total) return;
+  float v = ws[i];
+  for (int y = 1; y < ny; ++y) v += ws[(size_t)y * total + i];
+  const size_t m = i / (size_t)N, n = i - m * (size_t)N;
+  float* cp = C + m * ldc + c_off + n;
+  if (accumulate == 1) {
+    v += *cp;
+  } else if (accumulate == 2) {
+    const float gt = *cp;
+    v *= gt / (1.0f + __expf(-gt));
+  }
+  *cp = v;
+}
 // -DBM=64: the 64-token form (grid ceil(N / 128) * ceil(M / 64) work-groups)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE8_ACT321_BM64(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,

@@ -106,6 +106,41 @@ def test_gemm_epilogues(eng):
     assert np.array_equal(ys[:, :c_off], c0[:, :c_off])
 
 
+@pytest.mark.parametrize("T,Mp,N,K", [(64, 64, 130, 4096), (40, 48, 300, 5120), (100, 112, 260, 2560), (128, 128, 128, 4096)])
+def test_gemm_split_k(eng, T, Mp, N, K):
+    """Short Q4_K chunks whose tiles are few: K shared out over several work-groups per tile, partial tiles added in a
+    fixed order by a second kernel that also applies c_off and the accumulate mode (tiles of 64 tokens up to 64 tokens,
+    of 128 above).  Parity with the oracle, the three epilogues, the same bits on every run."""
+    qtype = az.Q4_K
+    print(f"gemm split-K T={T} Mp={Mp} N={N} K={K}", flush=True)
+    W = make_weights(qtype, N, K, seed=71)
+    x = make_acts(T, K, seed=72 + T, outliers=True)
+    y0 = run_gemm(eng, qtype, W, N, K, x, Mp)
+    aq, asc, absum = quantize_padded(x, Mp)
+    ref = orc.matmul_ref(qtype, W, N, K, aq[:T], asc)
+    assert rel_err_rows(y0[:T], ref).max() <= TOL and not y0[T:].any()
+    assert np.array_equal(run_gemm(eng, qtype, W, N, K, x, Mp).view(np.uint32), y0.view(np.uint32))
+    ldc, c_off = N + 70, 33
+    c0 = az.gen_normal(73, (Mp, ldc))
+    ya = run_gemm(eng, qtype, W, N, K, x, Mp, acc=1, c_init=c0, ldc=ldc, c_off=c_off)
+    assert np.array_equal(ya[:, :c_off], c0[:, :c_off]) and np.array_equal(ya[:, c_off + N:], c0[:, c_off + N:])
+    assert np.array_equal(ya[:, c_off:c_off + N], y0 + c0[:, c_off:c_off + N])
+    ys = run_gemm(eng, qtype, W, N, K, x, Mp, acc=2, c_init=c0, ldc=ldc, c_off=c_off)
+    g = c0[:, c_off:c_off + N].astype(np.float64)
+    want = y0.astype(np.float64) * (g / (1.0 + np.exp(-g)))
+    assert np.abs(ys[:, c_off:c_off + N] - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.array_equal(ys[:, :c_off], c0[:, :c_off])
+
+
+def test_gemm_split_k_unit_scales_exact(eng):
+    """Unit scales: the sum of the partial tiles is the exact integer sum (every partial sum below 2^24)."""
+    T, N, K = 64, 96, 4096
+    W, wi = unit_scale_weights(az.Q4_K, N, K, seed=75)
+    x = unit_scale_acts(T, K, seed=76)
+    y = run_gemm(eng, az.Q4_K, W, N, K, x, 64)
+    assert np.array_equal(y, (x.astype(np.int64) @ wi.T).astype(np.float32))
+
+
 def test_startup_self_check(rt):
     """Tuned GEMM == simple GEMM == host integer sums, bit for bit, on the reference's LCG data with unit scales
     (the start-up check in the pattern of xmx_check, zero/engine_setup.h:424-520)."""
