@@ -402,16 +402,17 @@ class Engine {
   size_t sk_ws_bytes_ = 0;
   void gemm_dense(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int a) {
     int M = Mp, N = w.N, K = w.K;
-    // Q4_K, Q6_K and Q8_0, a chunk so short that its tiles are fewer than two per compute unit: K is shared out over `ny`
+    // Any type, a chunk so short that its tiles are fewer than two per compute unit: K is shared out over `ny`
     // work-groups per tile, which store partial tiles in a workspace, and splitk_reduce adds the slices in order (the
     // same bits on every run) and applies c_off and the accumulate mode.  One work-group needs 75 us for K = 5120, so
     // 64 tokens x 17408 rows took 100 us whatever the tile; now 136 tiles x 3 pieces, 52 us (128 tokens: 101 -> 88 us;
     // Q8_0 4096 x 4096: 64 tokens 41 -> 19 us, 256 tokens 44 -> 35 us).  ARCZ_Q4_SPLITK=0: off, =n: n pieces.
     static const bool sk_off = getenv("ARCZ_Q4_SPLITK") && atoi(getenv("ARCZ_Q4_SPLITK")) == 0;
-    if (!sk_off && (w.type == GGML_Q4_K || w.type == GGML_Q8_0 || w.type == GGML_Q6_K)) {
+    if (!sk_off) {
       // (tiles of 64 tokens up to 64 tokens, else of 128: the pieces of all tiles together must fit the resident slots,
       //  two work-groups per compute unit: one more piece than fits costs a whole second round)
-      const int tm = Mp <= 64 || w.type != GGML_Q4_K ? 64 : 128;
+      // (Q8_0, Q6_K: their dense kernels' 64-token tiles; Q5_K, IQ4_XS: the register-staged body's 128-token tiles)
+      const int tm = w.type == GGML_Q8_0 || w.type == GGML_Q6_K ? 64 : w.type == GGML_Q4_K ? (Mp <= 64 ? 64 : 128) : 128;
       const size_t tiles64 = (size_t)((Mp + tm - 1) / tm) * ((N + 127) / 128), slots = 2 * (size_t)arcz_device_cus();
       const int nsb = K / 256;
       static const int sk_force = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : 0;
