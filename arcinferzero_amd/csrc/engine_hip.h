@@ -413,6 +413,7 @@ class Engine {
       //  two work-groups per compute unit: one more piece than fits costs a whole second round)
       // (Q8_0, Q6_K: their dense kernels' 64-token tiles; Q5_K, IQ4_XS: the register-staged body's 128-token tiles)
       const int tm = w.type == GGML_Q8_0 || w.type == GGML_Q6_K ? 64 : w.type == GGML_Q4_K ? (Mp <= 64 ? 64 : 128) : 128;
+      const int bm = tm == 64 && w.type == GGML_Q4_K && Mp <= 32 ? 32 : tm;  // (Q4_K, at most 32 rows: the one-slot-tile kernel)
       const size_t tiles64 = (size_t)((Mp + tm - 1) / tm) * ((N + 127) / 128), slots = 2 * (size_t)arcz_device_cus();
       const int nsb = K / 256;
       static const int sk_force = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : 0;
@@ -426,7 +427,7 @@ class Engine {
           sk_ws_ = buf(need);
           sk_ws_bytes_ = need;
         }
-        cl_kernel k = kernel("gemm", std::string("-DQTYPE=") + std::to_string(w.type) + " -DACT32 -DBM=" + std::to_string(tm) +
+        cl_kernel k = kernel("gemm", std::string("-DQTYPE=") + std::to_string(w.type) + " -DACT32 -DBM=" + std::to_string(bm) +
                                          " -DBN=128 -DSPLITK", "gemm");
         cl_mem unused = nullptr;
         int zero = 0, one = 1, ldw = N, s1 = nsb;

@@ -53,7 +53,7 @@ template <int QT> struct StepRegs {
 };
 
 template <int QT>
-__device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8_t* __restrict__ raw, size_t rows_total,
+__device__ __forceinline__ void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8_t* __restrict__ raw, size_t rows_total,
                                  int nsb, size_t row_base, int n0, int N, const signed char* __restrict__ aq,
                                  const float* __restrict__ asc, int M, int K, int s, int hh) {
   const int t = threadIdx.x;
@@ -103,7 +103,7 @@ __device__ inline void step_load(StepRegs<QT>& r, const Gemm2Lds& L, const uint8
 
 // Registers -> LDS: int8 values, decoded weights, the four scale vectors.  Rows past the tile carry zero scales.
 template <int QT>
-__device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
+__device__ __forceinline__ void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
   constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
   const int t = threadIdx.x;
   int ssum[4];
@@ -179,7 +179,7 @@ __device__ inline void step_store(const StepRegs<QT>& r, Gemm2Lds& L, int hh) {
 }
 
 template <int QT, bool TILES>
-__device__ inline void gemm2_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+__device__ __forceinline__ void gemm2_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
                                   int c_off, int accumulate, int s_begin, int s_end, size_t rows_total, size_t row_base,
                                   int m0, int rows_valid, int n0, const int* __restrict__ rowmap, int use_map,
@@ -341,7 +341,7 @@ struct G3ScaleRegs {
 
 template <bool TILES>  // (only the dense form is instantiated: over expert tiles, with their short K, the register-staged
                        //  body above measured faster)
-__device__ inline void gemm3_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+__device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
                                   int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
                                   size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
@@ -587,7 +587,7 @@ struct G6ScaleRegs {
   uint32_t d;
 };
 
-__device__ inline void gemm6_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+__device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
                                   int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0) {
   __shared__ alignas(16) uint8_t lds[2 * G6_STAGE];
@@ -795,7 +795,10 @@ struct G4ScaleRegs {
   uint4 h;
 };
 
-__device__ inline void gemm4_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+// TWO = false: tiles of at most 32 slots; the second slot tile, whose scales would all be zero, is left out (half
+// the matrix and vector instructions of a step).
+template <bool TWO = true>
+__device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
                                   int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
                                   size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
@@ -897,7 +900,7 @@ __device__ inline void gemm4_body(const uint8_t* __restrict__ raw, const signed 
     v16i I[2];
     auto ld_a = [&](int b, int buf) {
       a16[buf][0] = *(const v4i*)(Sb + oa[b]);
-      a16[buf][1] = *(const v4i*)(Sb + oa[b] + 32 * 128);
+      if constexpr (TWO) a16[buf][1] = *(const v4i*)(Sb + oa[b] + 32 * 128);
       saop[buf] = ((const float*)(Sb + G4_SA))[b * 64 + lane];
       wsop[buf] = ((const float*)(Sb + G4_WS))[b * 128 + wave * 32 + l32];
     };
@@ -930,23 +933,38 @@ __device__ inline void gemm4_body(const uint8_t* __restrict__ raw, const signed 
       const bool more = b + 1 < 4;
       if ((b & 1) == 0) {  // min term of blocks b and b + 1: lane half g supplies block b + g
 #pragma unroll
-        for (int ms = 0; ms < 2; ++ms) uop[ms] = ((const float*)(Sb + G4_U))[(b + g) * 64 + ms * 32 + l32];
+        for (int ms = 0; ms < (TWO ? 2 : 1); ++ms) uop[ms] = ((const float*)(Sb + G4_U))[(b + g) * 64 + ms * 32 + l32];
         vop = ((const float*)(Sb + G4_V))[(b + g) * 128 + wave * 32 + l32];
       }
+      if constexpr (TWO) {
 #pragma unroll
-      for (int ms = 0; ms < 2; ++ms) {
-        const int slot = ms;
-        if (ms == 0) {
-          mfma_i(buf, 1, 1);
-          if (more) { ld_a(b + 1, buf ^ 1); dec_w(b + 1, buf ^ 1); }
-        } else if (more) {
+        for (int ms = 0; ms < 2; ++ms) {
+          const int slot = ms;
+          if (ms == 0) {
+            mfma_i(buf, 1, 1);
+            if (more) { ld_a(b + 1, buf ^ 1); dec_w(b + 1, buf ^ 1); }
+          } else if (more) {
+            mfma_p(buf ^ 1);
+            mfma_i(buf ^ 1, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 0; i < 16; ++i) res[ms][i] = __builtin_fmaf((float)I[slot][i], P[buf][16 * ms + i], res[ms][i]);
+          if ((b & 1) == 0) res[ms] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop, res[ms], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        // one slot tile: the next block's matrix instructions go out, then this block's products (slots alternate)
+        if (more) {
+          ld_a(b + 1, buf ^ 1);
+          dec_w(b + 1, buf ^ 1);
           mfma_p(buf ^ 1);
-          mfma_i(buf ^ 1, 0, 0);
+          mfma_i(buf ^ 1, 0, buf ^ 1);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) res[ms][i] = __builtin_fmaf((float)I[slot][i], P[buf][16 * ms + i], res[ms][i]);
-        if ((b & 1) == 0) res[ms] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop, res[ms], 0, 0, 0);
+        for (int i = 0; i < 16; ++i) res[0][i] = __builtin_fmaf((float)I[buf][i], P[buf][i], res[0][i]);
+        if ((b & 1) == 0) res[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[0], vop, res[0], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -962,7 +980,7 @@ __device__ inline void gemm4_body(const uint8_t* __restrict__ raw, const signed 
   const int n = n0 + wave * 32 + l32;
   if (n < N) {
 #pragma unroll
-    for (int ms = 0; ms < 2; ++ms)
+    for (int ms = 0; ms < (TWO ? 2 : 1); ++ms)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
@@ -1006,7 +1024,7 @@ struct GuScaleRegs {
 // GU: the two streams are gate and up of an expert (rows n0.. of both tensors, h = silu(gate) * up); otherwise they are
 // rows n0.. and n0 + 128.. of one matrix and each gets the plain epilogue (a 64 x 256 tile of a dense product).
 template <bool GU>
-__device__ inline void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
+__device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
                                     const signed char* __restrict__ aq, const float* __restrict__ asc,
                                     const short* __restrict__ absum, float* __restrict__ H, int M, int N, int K,
                                     size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
@@ -1264,7 +1282,7 @@ extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12(
 #define G8_SA 24576
 #define G8_WS 25600
 
-__device__ inline void gemm8_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
+__device__ __forceinline__ void gemm8_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
                                   int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0) {
   __shared__ alignas(16) uint8_t lds[2 * G8_STAGE];
@@ -1510,8 +1528,18 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64_B
   tile_of(blockIdx.x, mt, nt, tm, tn);
   const int m0 = tm * G6_BM, n0 = tn * BN;
   const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
-  gemm4_body(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
-             s_begin + ns * (y + 1) / ny, (size_t)N, 0, m0, min(G6_BM, M - m0), n0, nullptr, 0, nullptr, 0);
+  gemm4_body<true>(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+                   s_begin + ns * (y + 1) / ny, (size_t)N, 0, m0, min(G6_BM, M - m0), n0, nullptr, 0, nullptr, 0);
+}
+// (-DBM=32: chunks of at most 32 rows, M <= 32: one slot tile.  A kernel of its own: the body's LDS is a static array
+//  per instantiation, and two in one kernel would halve the work-groups a compute unit holds)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM32_BN128_SPLITK1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int n0 = blockIdx.x * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm4_body<false>(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+                    s_begin + ns * (y + 1) / ny, (size_t)N, 0, 0, min(32, M), n0, nullptr, 0, nullptr, 0);
 }
 // (-DBM=128 -DBN=128 -DSPLITK: the same over the 128 x 128 tiles of the dense kernel, for 65-128 tokens)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM128_BN128_SPLITK1(
@@ -1611,8 +1639,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TI
   const int t_end = tstart[e1];
   for (int ti = tstart[e0] + blockIdx.y; ti < t_end; ti += gridDim.y) {
     const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-    gemm4_body(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,
-               min(nr, G6_BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
+    gemm4_body<true>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,
+                     min(nr, G6_BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
     __syncthreads();
   }
 }
