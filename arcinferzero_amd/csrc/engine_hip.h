@@ -405,7 +405,7 @@ class Engine {
     // Any type, a chunk so short that its tiles are fewer than two per compute unit: K is shared out over `ny`
     // work-groups per tile, which store partial tiles in a workspace, and splitk_reduce adds the slices in order (the
     // same bits on every run) and applies c_off and the accumulate mode.  One work-group needs 75 us for K = 5120, so
-    // 64 tokens x 17408 rows took 100 us whatever the tile; now 136 tiles x 3 pieces, 52 us (128 tokens: 101 -> 88 us;
+    // 64 tokens x 17408 rows took 100 us whatever the tile; now 136 tiles x 3 pieces, 42 us (128 tokens: 101 -> 71 us;
     // Q8_0 4096 x 4096: 64 tokens 41 -> 19 us, 256 tokens 44 -> 35 us).  ARCZ_Q4_SPLITK=0: off, =n: n pieces.
     static const bool sk_off = getenv("ARCZ_Q4_SPLITK") && atoi(getenv("ARCZ_Q4_SPLITK")) == 0;
     if (!sk_off) {
