@@ -3,7 +3,9 @@
 // Same entry points, argument meaning and error behaviour; launch shapes and tuning rules are gfx950's own.
 #pragma once
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
+#include <cstring>
 #include <map>
 #include <stdexcept>
 #include <string>
@@ -623,83 +625,128 @@ class Engine {
   std::vector<cl_mem> mems_;
   std::vector<std::pair<std::string, cl_event>> events_;
 };
-
-// Start-up check of the tuned GEMM against the simple one (the pattern of xmx_check, zero/engine_setup.h:424-520): both
-// kernels run on the same data from the reference's LCG (1664525 / 1013904223, seed 12345), 128 tokens x 128 rows x
-// K = 1024, with unit scales (weights d = 1, sub-scales 1, mins 1; activation scales 1) so that every f32 output is an
-// integer below 2^24: the two results must be bit-equal to each other and to the integer sums counted on the host.
-// Returns an empty string, or what differed.
+// Start-up check in the pattern of the reference's xmx_check (zero/engine_setup.h:424-520): every tuned GEMM the
+// dispatch can take -- for each weight type, storing, accumulating and with the fused SwiGLU epilogue, in one piece
+// and with K shared out over several work-groups per tile -- against the plain kernel of the same type on the
+// reference's LCG data, with unit scales (weights d = 1, sub-scales 1, Q4_K / Q5_K mins 1; activation scales 1) so that
+// every f32 sum is an integer below 2^24: the two results must be bit-equal to each other and, for store and add, to
+// the integer sums counted on the host.  Returns an empty string, or what differed.
 inline std::string engine_self_check() {
-  const int M = 128, N = 128, K = 1024;
-  Engine e(M, K);
+  const int M = 128, N = 128;
   uint32_t lcg = 12345u;
   auto next = [&]() { lcg = lcg * 1664525u + 1013904223u; return lcg >> 8; };
-  std::vector<int8_t> aq((size_t)M * K);
-  std::vector<float> asc((size_t)M * (K / 32), 1.0f);
-  std::vector<int16_t> absum((size_t)M * (K / 16));
-  for (auto& v : aq) v = (int8_t)((int)(next() % 255u) - 127);
-  for (int m = 0; m < M; ++m)
-    for (int b = 0; b < K / 16; ++b) {
-      int s = 0;
-      for (int i = 0; i < 16; ++i) s += aq[(size_t)m * K + b * 16 + i];
-      absum[(size_t)b * M + m] = (int16_t)s;
-    }
-  e.set_activations(aq.data(), asc.data(), absum.data(), K, M, M);
-  cl_mem c0 = e.buf((size_t)M * N * 4), c1 = e.buf((size_t)M * N * 4);
-  std::vector<float> y0((size_t)M * N), y1((size_t)M * N);
-  for (uint32_t type : {GGML_Q8_0, GGML_Q4_K}) {
-    const size_t rb = arcz_gguf_bytes(type, 1, K);
-    std::vector<uint8_t> w((size_t)N * rb);
-    std::vector<int> wq((size_t)N * K);  // the integer each element stands for
-    for (int n = 0; n < N; ++n)
-      for (int sb = 0; sb < K / 256; ++sb) {
-        if (type == GGML_Q8_0) {
-          for (int b = 0; b < 8; ++b) {
-            uint8_t* blk = &w[n * rb + (size_t)(sb * 8 + b) * 34];
-            blk[0] = 0x00; blk[1] = 0x3C;  // f16 1.0
-            for (int i = 0; i < 32; ++i) {
-              const int q = (int)(next() % 255u) - 127;
-              blk[2 + i] = (uint8_t)(int8_t)q;
-              wq[(size_t)n * K + sb * 256 + b * 32 + i] = q;
-            }
-          }
-        } else {
-          uint8_t* blk = &w[n * rb + (size_t)sb * 144];
-          blk[0] = 0x00; blk[1] = 0x3C; blk[2] = 0x00; blk[3] = 0x3C;  // d = dmin = 1.0
-          for (int i = 0; i < 8; ++i) blk[4 + i] = 1;                   // 6-bit scales and mins of sub-blocks 0-3: 1
-          for (int i = 0; i < 4; ++i) blk[12 + i] = 0x11;               // low nibbles of those of sub-blocks 4-7: 1
-          for (int j = 0; j < 4; ++j)
-            for (int l = 0; l < 32; ++l) {
-              const int lo = (int)(next() & 15u), hi = (int)(next() & 15u);
-              blk[16 + j * 32 + l] = (uint8_t)(lo | hi << 4);
-              wq[(size_t)n * K + sb * 256 + j * 64 + l] = lo - 1;       // value = 1 * 1 * q - 1 * 1
-              wq[(size_t)n * K + sb * 256 + j * 64 + 32 + l] = hi - 1;
-            }
+  static const int iq4[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+  // one superblock with unit scales and random quants; wq: the integer each element stands for
+  auto make_sb = [&](uint32_t type, uint8_t* blk, int* wq) {
+    if (type == GGML_Q8_0) {
+      for (int b = 0; b < 8; ++b) {
+        uint8_t* p = blk + 34 * b;
+        p[0] = 0x00; p[1] = 0x3C;  // f16 1.0
+        for (int i = 0; i < 32; ++i) {
+          const int q = (int)(next() % 255u) - 127;
+          p[2 + i] = (uint8_t)(int8_t)q;
+          wq[b * 32 + i] = q;
         }
       }
-    GpuWeight gw = e.make_weight(type, w.data(), w.size(), N, K);
-    e.gemm_dense("self_check", gw, M, c0, N, 0, 0);  // the kernel the engine's dispatch takes for this type
-    {
-      cl_kernel k = e.kernel("gemm", "-DQTYPE=" + std::to_string(type) + " -DACT32", "gemm_simple");
-      cl_mem unused = nullptr;
-      int MM = M, NN = N, KK = K, ldc = N, zero = 0, one = 1, s1 = K / 256;
-      set_args(k, 0, gw.raw, unused, e.aq_, e.asc_, e.absum_, c1, MM, NN, KK, ldc, zero, zero, one, zero, s1);
-      size_t gws[1] = {(size_t)(M / 128) * (N / 128) * 256}, lws[1] = {256};
-      e.run("self_check", k, 1, gws, lws);
+    } else if (type == GGML_Q4_K || type == GGML_Q5_K) {
+      const bool q5 = type == GGML_Q5_K;
+      memset(blk, 0, q5 ? 176 : 144);
+      blk[0] = 0x00; blk[1] = 0x3C; blk[2] = 0x00; blk[3] = 0x3C;  // d = dmin = 1.0
+      for (int i = 0; i < 8; ++i) blk[4 + i] = 1;                   // 6-bit scales and mins of sub-blocks 0-3: 1
+      for (int i = 0; i < 4; ++i) blk[12 + i] = 0x11;               // low nibbles of those of sub-blocks 4-7: 1
+      uint8_t *qh = blk + 16, *qs = blk + (q5 ? 48 : 16);
+      for (int j = 0; j < 4; ++j)
+        for (int l = 0; l < 32; ++l) {
+          const int lim = q5 ? 31 : 15;
+          const int lo = (int)(next() & lim), hi = (int)(next() & lim);
+          qs[j * 32 + l] = (uint8_t)((lo & 15) | (hi & 15) << 4);
+          if (q5) qh[l] |= (uint8_t)(((lo >> 4) << (2 * j)) | ((hi >> 4) << (2 * j + 1)));
+          wq[j * 64 + l] = lo - 1;  // value = 1 * 1 * q - 1 * 1
+          wq[j * 64 + 32 + l] = hi - 1;
+        }
+    } else if (type == GGML_Q6_K) {
+      memset(blk, 0, 210);
+      for (int i = 0; i < 16; ++i) blk[192 + i] = 1;  // int8 scales
+      blk[208] = 0x00; blk[209] = 0x3C;
+      for (int n2 = 0; n2 < 2; ++n2)
+        for (int l = 0; l < 32; ++l) {
+          int q[4];
+          for (int k = 0; k < 4; ++k) { q[k] = (int)(next() & 63u); wq[128 * n2 + 32 * k + l] = q[k] - 32; }
+          blk[64 * n2 + l] = (uint8_t)((q[0] & 15) | (q[2] & 15) << 4);
+          blk[64 * n2 + 32 + l] = (uint8_t)((q[1] & 15) | (q[3] & 15) << 4);
+          blk[128 + 32 * n2 + l] = (uint8_t)((q[0] >> 4) | (q[1] >> 4) << 2 | (q[2] >> 4) << 4 | (q[3] >> 4) << 6);
+        }
+    } else {  // IQ4_XS: 6-bit scales 33 (- 32 = 1): low nibble 1, high two bits 2
+      memset(blk, 0, 136);
+      blk[0] = 0x00; blk[1] = 0x3C; blk[2] = 0xAA; blk[3] = 0xAA;
+      for (int i = 0; i < 4; ++i) blk[4 + i] = 0x11;
+      for (int b = 0; b < 8; ++b)
+        for (int j = 0; j < 16; ++j) {
+          const int lo = (int)(next() & 15u), hi = (int)(next() & 15u);
+          blk[8 + 16 * b + j] = (uint8_t)(lo | hi << 4);
+          wq[32 * b + j] = iq4[lo];
+          wq[32 * b + 16 + j] = iq4[hi];
+        }
     }
-    CL_CHECK(clEnqueueReadBuffer(e.cl_.queue, c0, CL_TRUE, 0, y0.size() * 4, y0.data(), 0, nullptr, nullptr));
-    CL_CHECK(clEnqueueReadBuffer(e.cl_.queue, c1, CL_TRUE, 0, y1.size() * 4, y1.data(), 0, nullptr, nullptr));
-    e.free_weight(gw);
+  };
+  // K = 1024: one piece (few superblocks); K = 2048 with smaller activations: the tile's K in four pieces
+  for (int K : {1024, 2048}) {
+    Engine e(M, K);
+    const int amax = K == 1024 ? 127 : 63;
+    std::vector<int8_t> aq((size_t)M * K);
+    std::vector<float> asc((size_t)M * (K / 32), 1.0f);
+    std::vector<int16_t> absum((size_t)M * (K / 16));
+    for (auto& v : aq) v = (int8_t)((int)(next() % (unsigned)(2 * amax + 1)) - amax);
     for (int m = 0; m < M; ++m)
-      for (int n = 0; n < N; ++n) {
-        long long s = 0;
-        for (int k2 = 0; k2 < K; ++k2) s += (long long)aq[(size_t)m * K + k2] * wq[(size_t)n * K + k2];
-        const float a = y0[(size_t)m * N + n], b = y1[(size_t)m * N + n];
-        if (a != (float)s || b != (float)s)
-          return std::string("GEMM self-check ") + ggml_type_name(type) + ": token " + std::to_string(m) + " row " +
-                 std::to_string(n) + ": tuned " + std::to_string(a) + ", simple " + std::to_string(b) + ", integer sum " +
-                 std::to_string(s);
+      for (int b = 0; b < K / 16; ++b) {
+        int sm = 0;
+        for (int i = 0; i < 16; ++i) sm += aq[(size_t)m * K + b * 16 + i];
+        absum[(size_t)b * M + m] = (int16_t)sm;
       }
+    e.set_activations(aq.data(), asc.data(), absum.data(), K, M, M);
+    cl_mem c0 = e.buf((size_t)M * N * 4), c1 = e.buf((size_t)M * N * 4);
+    std::vector<float> y0((size_t)M * N), y1((size_t)M * N), cinit((size_t)M * N);
+    for (auto& v : cinit) v = (float)((int)(next() % 9u) - 4);  // small integers: sums with them stay exact
+    for (uint32_t type : {GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ4_XS}) {
+      const size_t rb = arcz_gguf_bytes(type, 1, K), sbb = rb / (size_t)(K / 256);
+      std::vector<uint8_t> w((size_t)N * rb);
+      std::vector<int> wq((size_t)N * K);
+      for (int n = 0; n < N; ++n)
+        for (int sb = 0; sb < K / 256; ++sb) make_sb(type, &w[n * rb + sb * sbb], &wq[(size_t)n * K + sb * 256]);
+      GpuWeight gw = e.make_weight(type, w.data(), w.size(), N, K);
+      for (int mode = 0; mode < 3; ++mode) {
+        CL_CHECK(clEnqueueWriteBuffer(e.cl_.queue, c0, CL_TRUE, 0, cinit.size() * 4, cinit.data(), 0, nullptr, nullptr));
+        CL_CHECK(clEnqueueWriteBuffer(e.cl_.queue, c1, CL_TRUE, 0, cinit.size() * 4, cinit.data(), 0, nullptr, nullptr));
+        e.gemm_dense("self_check", gw, M, c0, N, 0, mode);  // the kernel(s) the engine's dispatch takes for this type
+        {
+          cl_kernel k = e.kernel("gemm", "-DQTYPE=" + std::to_string(type) + " -DACT32", "gemm_simple");
+          cl_mem unused = nullptr;
+          int MM = M, NN = N, KK = K, ldc = N, zero = 0, one = 1, s1 = K / 256, md = mode;
+          set_args(k, 0, gw.raw, unused, e.aq_, e.asc_, e.absum_, c1, MM, NN, KK, ldc, zero, md, one, zero, s1);
+          size_t gws[1] = {(size_t)(M / 128) * (N / 128) * 256}, lws[1] = {256};
+          e.run("self_check", k, 1, gws, lws);
+        }
+        CL_CHECK(clEnqueueReadBuffer(e.cl_.queue, c0, CL_TRUE, 0, y0.size() * 4, y0.data(), 0, nullptr, nullptr));
+        CL_CHECK(clEnqueueReadBuffer(e.cl_.queue, c1, CL_TRUE, 0, y1.size() * 4, y1.data(), 0, nullptr, nullptr));
+        for (int m = 0; m < M; ++m)
+          for (int n = 0; n < N; ++n) {
+            long long sm = 0;
+            for (int k2 = 0; k2 < K; ++k2) sm += (long long)aq[(size_t)m * K + k2] * wq[(size_t)n * K + k2];
+            const float a = y0[(size_t)m * N + n], b = y1[(size_t)m * N + n];
+            const float want = mode == 0 ? (float)sm : mode == 1 ? (float)sm + cinit[(size_t)m * N + n] : a;
+            uint32_t ab, bb;
+            memcpy(&ab, &a, 4);
+            memcpy(&bb, &b, 4);
+            if (ab != bb || a != want || !std::isfinite(a)) {
+              e.free_weight(gw);
+              return std::string("GEMM self-check ") + ggml_type_name(type) + " K=" + std::to_string(K) + " mode " +
+                     std::to_string(mode) + ": token " + std::to_string(m) + " row " + std::to_string(n) + ": tuned " +
+                     std::to_string(a) + ", simple " + std::to_string(b) + ", integer sum " + std::to_string(sm);
+            }
+          }
+      }
+      e.free_weight(gw);
+    }
   }
   return std::string();
 }

@@ -96,8 +96,9 @@ int arcz_engine_moe_route(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, i
 arcz_mem* arcz_engine_moe_buffer(arcz_engine* e, int which);
 int arcz_engine_moe_slots(arcz_engine* e);
 
-/* The start-up check of the tuned GEMM against the simple one on the reference's LCG data, both against integer sums
- * counted on the host (the pattern of xmx_check, zero/engine_setup.h:424-520).  0, or ARCZ_E_ENGINE with the first
+/* The start-up check of the tuned GEMMs against the simple one on the reference's LCG data, both against integer sums
+ * counted on the host (the pattern of xmx_check, zero/engine_setup.h:424-520): every weight type, the three accumulate
+ * modes, K in one piece and in several.  0, or ARCZ_E_ENGINE with the first
  * difference in arcz_engine_error(). */
 int arcz_engine_self_check(void);
 
