@@ -578,6 +578,61 @@ class Engine {
     const int E = L.E, F = L.F, NU = L.NU, n = T * NU;
     if (cur_T_ != T || cur_K_ != E || cur_Mp_ != Mp) throw std::runtime_error("layer_moe: the activations are not this chunk's");
     if (arcz_mem_size(x) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: x is too small");
+    // A pass of 1-8 tokens (zero/engine_moe.h:86-262): tiles of 1, 2, 4 or 8 slots through the matrix-vector kernels
+    // moe_gateup_q / moe_down_q -- one token's NU experts are the tiles straight from moe_route1, no counts, scan or
+    // scatter -- instead of the 64-slot tile GEMMs, which for one token walked K alone in 8 x 6 work-groups (128 us a
+    // layer at 128 experts x 768 x 2048; ARCZ_MOE_DECODE=0 brings that back).
+    static const bool dec_off = getenv("ARCZ_MOE_DECODE") && atoi(getenv("ARCZ_MOE_DECODE")) == 0;
+    if (!dec_off && T <= 8) {
+      const int NE = L.NE;
+      const int tmd = T == 1 ? 1 : T <= 2 ? 2 : T <= 4 ? 4 : 8;
+      size_t tiles_max;
+      if (T == 1) {
+        if (ldl < NE || arcz_mem_size(rl) < (size_t)NE * 4) throw std::runtime_error("layer_moe: router logits do not fit");
+        cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DHAS_GATE=" +
+                                        std::to_string(ldl > NE ? 1 : 0), "moe_route1");
+        set_args(k, 0, rl, sgate_, mtiles_, stok_, swt_, minv_);
+        size_t g1 = 64, l1 = 64;
+        run("moe_route", k, 1, &g1, &l1);
+        tiles_max = (size_t)NU;
+      } else {
+        moe_route(L, rl, ldl, T, tmd);
+        tiles_max = (size_t)(n + tmd - 1) / tmd + std::min(n, NE);
+      }
+      cl_mem tabs = nullptr;
+      const std::string dd = " -DGROWS=2 -DTM=" + std::to_string(tmd) + " -DNE=" + std::to_string(NE);
+      {
+        if (L.ex[0].type != L.ex[1].type) throw std::runtime_error("layer_moe: gate and up experts of different types");
+        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + dd, "moe_gateup_q");
+        int FF = F, KK = E, MM = Mp;
+        set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
+        size_t gws[2] = {((size_t)(F + 1) / 2 * 32 + 255) / 256 * 256, tiles_max}, lws[2] = {256, 1};
+        run("moe_gateup", k, 2, gws, lws);
+      }
+      {
+        cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU), "moe_quant_sums");
+        int FF = F, S = slots_;
+        set_args(k, 0, mh_, FF, S, mhq_, mhsc_, mhbs_);
+        size_t gws[2] = {(size_t)256 * (F / 256), (size_t)(n + 63) / 64}, lws[2] = {256, 1};
+        run("moe_quant", k, 2, gws, lws);
+      }
+      {
+        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + dd, "moe_down_q");
+        int NN = E, KK = F, S = slots_;
+        set_args(k, 0, L.ex[2].raw, NN, KK, tabs, mhq_, mhsc_, S, mtiles_, swt_, my_, mhbs_);
+        size_t gws[2] = {((size_t)(E + 1) / 2 * 32 + 255) / 256 * 256, tiles_max}, lws[2] = {256, 1};
+        run("moe_down", k, 2, gws, lws);
+      }
+      {
+        cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU), "moe_combine");
+        cl_mem sh = nullptr;
+        int EE = E;
+        set_args(k, 0, x, sh, sgate_, my_, minv_, EE);
+        size_t gws[2] = {((size_t)E + 1023) / 1024 * 256, (size_t)T}, lws[2] = {256, 1};
+        run("moe_combine", k, 2, gws, lws);
+      }
+      return;
+    }
     // slots per tile = the token rows of one work-group of the tile GEMM: 64 for Q4_K experts, 128 for the others
     const int tm = L.ex[0].type == GGML_Q4_K ? 64 : 128;
     moe_route(L, rl, ldl, T, tm);

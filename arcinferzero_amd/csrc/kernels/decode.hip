@@ -19,21 +19,14 @@
 
 template <int QT> struct UnitsPerSb { static constexpr int v = QT == QT_Q8_0 ? 16 : 8; };
 
+// acc[r][t] += the products of plane rows rows[r] (absolute rows of planes that hold `plane_rows` rows) with the token
+// rows tok[t] of aq / asc / absum, this half wave's share (lane hl takes the 16-byte units hl, hl + 32, ...).
 template <int QT, int TB, int GROWS>
-__device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ aq,
-                                 const float* __restrict__ asc, const short* __restrict__ absum, int M, int T,
-                                 float* __restrict__ C, int ldc, int c_off, int accumulate, size_t plane_rows) {
+__device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t plane_rows, const size_t (&rows)[GROWS], int K,
+                                         const int (&tok)[TB], const signed char* __restrict__ aq,
+                                         const float* __restrict__ asc, const short* __restrict__ absum, int M, int hl,
+                                         float (&acc)[GROWS][TB], int nt = TB) {
   const int nsb = K >> 8, units = nsb * UnitsPerSb<QT>::v;
-  const int hl = threadIdx.x & 31;
-  const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
-  const int r0 = hw * GROWS;
-  if (r0 >= N) return;
-  float acc[GROWS][TB];
-#pragma unroll
-  for (int r = 0; r < GROWS; ++r)
-#pragma unroll
-    for (int t = 0; t < TB; ++t) acc[r][t] = 0.0f;
-
   if constexpr (QT == QT_Q4_K || QT == QT_Q5_K) {
     const PlanesQ4K pl = planes_q4k(plane_rows, nsb);
     const int j = (hl >> 1) & 3, half = hl & 1;
@@ -44,8 +37,8 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
       float salo[TB], sahi[TB];
       int bslo[TB], bshi[TB];
 #pragma unroll
-      for (int t = 0; t < TB; ++t) {
-        const int tt = t < T ? t : 0;
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
         alo[t] = *(const uint4*)(aq + (size_t)tt * K + e_lo);
         ahi[t] = *(const uint4*)(aq + (size_t)tt * K + e_lo + 32);
         salo[t] = asc[(size_t)(sb * 8 + 2 * j) * M + tt];
@@ -55,9 +48,9 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
       }
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
-        const int n = min(r0 + r, N - 1);
-        const uint4 w = *(const uint4*)(raw + pl.qs + (size_t)n * nsb * 128 + (size_t)u * 16);
-        const uint4 h = *(const uint4*)(raw + pl.hdr + ((size_t)n * nsb + sb) * 16);
+        const size_t n = rows[r];
+        const uint4 w = *(const uint4*)(raw + pl.qs + n * nsb * 128 + (size_t)u * 16);
+        const uint4 h = *(const uint4*)(raw + pl.hdr + (n * nsb + sb) * 16);
         const float d = f16_bits_to_f32(h.x), dmin = f16_bits_to_f32(h.x >> 16);
         int sc0, sc1, mn0, mn1;
         q4k_scales_pair(h.y, h.z, h.w, j, sc0, sc1, mn0, mn1);
@@ -65,12 +58,12 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
         uint32_t wh[4] = {(w.x >> 4) & 0x0F0F0F0Fu, (w.y >> 4) & 0x0F0F0F0Fu, (w.z >> 4) & 0x0F0F0F0Fu,
                           (w.w >> 4) & 0x0F0F0F0Fu};
         if constexpr (QT == QT_Q5_K) {  // the fifth bits of the unit's 32 values
-          const uint32_t H = *(const uint32_t*)(raw + pl.qh + (size_t)n * nsb * 32 + (size_t)u * 4), ww[4] = {w.x, w.y, w.z, w.w};
+          const uint32_t H = *(const uint32_t*)(raw + pl.qh + n * nsb * 32 + (size_t)u * 4), ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
           for (int k = 0; k < 4; ++k) { wl[k] = q5k_lo(ww[k], H, k); wh[k] = q5k_hi(ww[k], H, k); }
         }
 #pragma unroll
-        for (int t = 0; t < TB; ++t) {
+        for (int t = 0; t < TB; ++t) if (t < nt) {
           int ilo = dot4(wl[0], alo[t].x, 0);
           ilo = dot4(wl[1], alo[t].y, ilo);
           ilo = dot4(wl[2], alo[t].z, ilo);
@@ -94,8 +87,8 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
       uint4 a1[TB], a2[TB];
       float sa1[TB], sa2[TB];
 #pragma unroll
-      for (int t = 0; t < TB; ++t) {
-        const int tt = t < T ? t : 0;
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
         a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
         a2[t] = *(const uint4*)(aq + (size_t)tt * K + e2);
         sa1[t] = asc[(size_t)(e1 >> 5) * M + tt];
@@ -103,9 +96,9 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
       }
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
-        const int n = min(r0 + r, N - 1);
-        const size_t rs = (size_t)n * nsb + sb;
-        const uint4 L = *(const uint4*)(raw + pl.ql + (size_t)n * nsb * 128 + (size_t)u * 16);
+        const size_t n = rows[r];
+        const size_t rs = n * nsb + sb;
+        const uint4 L = *(const uint4*)(raw + pl.ql + n * nsb * 128 + (size_t)u * 16);
         const uint4 H = *(const uint4*)(raw + pl.qh + rs * 64 + 32 * n2 + (l0 & 31));
         const signed char* scp = (const signed char*)(raw + pl.sc + rs * 16 + 8 * n2 + (idx & 3));
         const int sc1 = scp[0], sc2 = scp[4];
@@ -118,7 +111,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
           w2[k] = sub32_bytes(((Lw[k] >> 4) & 0x0F0F0F0Fu) | (((Hw[k] >> hsh2) & 0x03030303u) << 4));
         }
 #pragma unroll
-        for (int t = 0; t < TB; ++t) {
+        for (int t = 0; t < TB; ++t) if (t < nt) {
           int i1 = dot4(w1[0], a1[t].x, 0);
           i1 = dot4(w1[1], a1[t].y, i1);
           i1 = dot4(w1[2], a1[t].z, i1);
@@ -141,17 +134,17 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
       uint4 a1[TB], a2[TB];
       float sa[TB];
 #pragma unroll
-      for (int t = 0; t < TB; ++t) {
-        const int tt = t < T ? t : 0;
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
         a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
         a2[t] = *(const uint4*)(aq + (size_t)tt * K + e1 + 16);
         sa[t] = asc[(size_t)(e1 >> 5) * M + tt];
       }
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
-        const int n = min(r0 + r, N - 1);
-        const uint4 w = *(const uint4*)(raw + pl.qs + (size_t)n * nsb * 128 + (size_t)u * 16);
-        const uint2 h = *(const uint2*)(raw + pl.hdr + ((size_t)n * nsb + sb) * 8);
+        const size_t n = rows[r];
+        const uint4 w = *(const uint4*)(raw + pl.qs + n * nsb * 128 + (size_t)u * 16);
+        const uint2 h = *(const uint2*)(raw + pl.hdr + (n * nsb + sb) * 8);
         const int ls = (int)(((h.y >> (4 * ib)) & 0xFu) | ((((h.x >> 16) >> (2 * ib)) & 3u) << 4)) - 32;
         const float d = f16_bits_to_f32(h.x);
         const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
@@ -162,7 +155,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
           w2[k] = iq4_lookup(ww[k] >> 4);
         }
 #pragma unroll
-        for (int t = 0; t < TB; ++t) {
+        for (int t = 0; t < TB; ++t) if (t < nt) {
           int i1 = dot4(w1[0], a1[t].x, 0);
           i1 = dot4(w1[1], a1[t].y, i1);
           i1 = dot4(w1[2], a1[t].z, i1);
@@ -183,18 +176,18 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
       uint4 a[TB];
       float sa[TB];
 #pragma unroll
-      for (int t = 0; t < TB; ++t) {
-        const int tt = t < T ? t : 0;
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
         a[t] = *(const uint4*)(aq + (size_t)tt * K + e);
         sa[t] = asc[(size_t)(e >> 5) * M + tt];
       }
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
-        const int n = min(r0 + r, N - 1);
-        const uint4 w = *(const uint4*)(raw + pl.qs + (size_t)n * nsb * 256 + (size_t)u * 16);
-        const float d = f16_bits_to_f32(*(const unsigned short*)(raw + pl.d + (((size_t)n * nsb + sb) * 8 + b) * 2));
+        const size_t n = rows[r];
+        const uint4 w = *(const uint4*)(raw + pl.qs + n * nsb * 256 + (size_t)u * 16);
+        const float d = f16_bits_to_f32(*(const unsigned short*)(raw + pl.d + ((n * nsb + sb) * 8 + b) * 2));
 #pragma unroll
-        for (int t = 0; t < TB; ++t) {
+        for (int t = 0; t < TB; ++t) if (t < nt) {
           int i = dot4(w.x, a[t].x, 0);
           i = dot4(w.y, a[t].y, i);
           i = dot4(w.z, a[t].z, i);
@@ -204,6 +197,28 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
       }
     }
   }
+}
+
+template <int QT, int TB, int GROWS>
+__device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ aq,
+                                 const float* __restrict__ asc, const short* __restrict__ absum, int M, int T,
+                                 float* __restrict__ C, int ldc, int c_off, int accumulate, size_t plane_rows) {
+  const int hl = threadIdx.x & 31;
+  const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
+  const int r0 = hw * GROWS;
+  if (r0 >= N) return;
+  float acc[GROWS][TB];
+  size_t rows[GROWS];
+  int tok[TB];
+#pragma unroll
+  for (int r = 0; r < GROWS; ++r) {
+    rows[r] = (size_t)min(r0 + r, N - 1);
+#pragma unroll
+    for (int t = 0; t < TB; ++t) acc[r][t] = 0.0f;
+  }
+#pragma unroll
+  for (int t = 0; t < TB; ++t) tok[t] = t < T ? t : 0;
+  gemv_acc<QT, TB, GROWS>(raw, plane_rows, rows, K, tok, aq, asc, absum, M, hl, acc);
 
 #pragma unroll
   for (int r = 0; r < GROWS; ++r)
@@ -248,3 +263,104 @@ GEMV_ALL(12)
 GEMV_ALL(13)
 GEMV_ALL(14)
 GEMV_ALL(23)
+
+// ---- the experts of a pass of 1-8 tokens (the reference's per-tile kernels moe_gateup_q / moe_down_q,
+// zero/kernels/decode.cl, launched by zero/engine_moe.h:196-262 with tiles of TM = 1, 2, 4 or 8 slots): the
+// matrix-vector form above on the rows of one expert.  A tile of the list = (expert, first slot, slots <= TM); with one
+// token moe_route1 makes its NU experts the tiles, otherwise moe_scan cuts the experts' slot ranges into tiles of TM.
+// grid (ceil(rows / GROWS) half waves in work-groups of 256, tile work-groups: y, y + gridDim.y, ...).
+
+// moe_gateup_q: h[slot][f] = silu(gate) * up for the tile's slots, gate and up from the two expert tensors' rows
+// [NE][F][K]; slot r reads token row stok[r].  Arguments as the reference's (rg, ru, F, K, tabs, aq, asc, M, tiles, stok,
+// h) plus absum (the 16-value sums the Q4_K / Q5_K min term takes) and NE.
+template <int QT, int TM, int GROWS>
+__device__ inline void moe_gateup_rows(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru, int F, int K,
+                                       const signed char* __restrict__ aq, const float* __restrict__ asc,
+                                       const short* __restrict__ absum, int M, const int* __restrict__ tiles,
+                                       const int* __restrict__ stok, float* __restrict__ h, int NE) {
+  const int hl = threadIdx.x & 31;
+  const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
+  const int f0 = hw * GROWS;
+  if (f0 >= F) return;
+  const int nt = tiles[0];
+  for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = min(tiles[3 + 3 * ti], TM);
+    float ag[GROWS][TM], au[GROWS][TM];
+    size_t rows[GROWS];
+    int tok[TM];
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r) {
+      rows[r] = (size_t)e * F + min(f0 + r, F - 1);
+#pragma unroll
+      for (int t = 0; t < TM; ++t) ag[r][t] = au[r][t] = 0.0f;
+    }
+#pragma unroll
+    for (int t = 0; t < TM; ++t) tok[t] = stok[r0 + min(t, nr - 1)];
+    gemv_acc<QT, TM, GROWS>(rg, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, ag, nr);
+    gemv_acc<QT, TM, GROWS>(ru, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, au, nr);
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r)
+#pragma unroll
+      for (int t = 0; t < TM; ++t) {
+        if (t >= nr) continue;  // (the same for the whole wave)
+        const float g = half_wave_sum(ag[r][t]), u = half_wave_sum(au[r][t]);
+        if (hl == 0 && f0 + r < F) h[(size_t)(r0 + t) * F + f0 + r] = g / (1.0f + __expf(-g)) * u;
+      }
+  }
+}
+
+// moe_down_q: y[slot][n] = swt[slot] * (Wd[expert][n] . hq[slot]) for the tile's slots; the expert tensor's rows
+// [NE][N][K], hq / hsc / hbs the expert inputs as moe_quant_sums leaves them (row stride S slots).  Arguments as the
+// reference's (raw, N, K, tabs, hq, hsc, S, tiles, swt, y) plus hbs and NE.
+template <int QT, int TM, int GROWS>
+__device__ inline void moe_down_rows(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ hq,
+                                     const float* __restrict__ hsc, const short* __restrict__ hbs, int S,
+                                     const int* __restrict__ tiles, const float* __restrict__ swt, float* __restrict__ y,
+                                     int NE) {
+  const int hl = threadIdx.x & 31;
+  const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
+  const int n0 = hw * GROWS;
+  if (n0 >= N) return;
+  const int nt = tiles[0];
+  for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = min(tiles[3 + 3 * ti], TM);
+    float acc[GROWS][TM];
+    size_t rows[GROWS];
+    int tok[TM];
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r) {
+      rows[r] = (size_t)e * N + min(n0 + r, N - 1);
+#pragma unroll
+      for (int t = 0; t < TM; ++t) acc[r][t] = 0.0f;
+    }
+#pragma unroll
+    for (int t = 0; t < TM; ++t) tok[t] = r0 + min(t, nr - 1);
+    gemv_acc<QT, TM, GROWS>(raw, (size_t)NE * N, rows, K, tok, hq, hsc, hbs, S, hl, acc, nr);
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r)
+#pragma unroll
+      for (int t = 0; t < TM; ++t) {
+        if (t >= nr) continue;
+        const float v = half_wave_sum(acc[r][t]);
+        if (hl == 0 && n0 + r < N) y[(size_t)(r0 + t) * N + n0 + r] = swt[r0 + t] * v;
+      }
+  }
+}
+
+#define MOE_DECODE_INST(QT, TM)                                                                                      \
+  extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS2_TM##TM(                             \
+      const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
+      int M, const int* tiles, const int* stok, float* h, const short* absum, int NE) {                              \
+    moe_gateup_rows<QT, TM, 2>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE);                                 \
+  }                                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void moe_down_q__QT##QT##_GROWS2_TM##TM(                               \
+      const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
+      const int* tiles, const float* swt, float* y, const short* hbs, int NE) {                                      \
+    moe_down_rows<QT, TM, 2>(raw, N, K, hq, hsc, hbs, S, tiles, swt, y, NE);                                         \
+  }
+#define MOE_DECODE_ALL(QT) MOE_DECODE_INST(QT, 1) MOE_DECODE_INST(QT, 2) MOE_DECODE_INST(QT, 4) MOE_DECODE_INST(QT, 8)
+MOE_DECODE_ALL(8)
+MOE_DECODE_ALL(12)
+MOE_DECODE_ALL(13)
+MOE_DECODE_ALL(14)
+MOE_DECODE_ALL(23)

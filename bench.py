@@ -205,6 +205,35 @@ def bench_moe(az, launches):
             **parts}
 
 
+def bench_moe_decode(az, launches):
+    """The same layer for passes of 1, 2, 4 and 8 tokens (the matrix-vector expert kernels): microseconds per layer,
+    launches back to back."""
+    NE, NU, E, F, qt = 128, 8, 2048, 768, az.Q4_K
+    eng = az.Engine(16, E)
+    L = eng.make_moe_layer(qt, az.gen_weights(qt, 21, NE * F, E, 0.02), az.gen_weights(qt, 22, NE * F, E, 0.02),
+                           az.gen_weights(qt, 23, NE * E, F, 0.02), NE, NU, E, F)
+    out = {}
+    for T in (1, 2, 4, 8):
+        xb = az.Runtime.from_numpy(az.gen_normal(24, (T, E)))
+        lb = az.Runtime.from_numpy(az.gen_normal(25 + T, (T, NE)))
+        ob = az.Runtime.alloc(T * E * 4).fill(0)
+        eng.quantize(xb, E, E, 16, T)
+        eng.layer_moe(L, lb, NE, ob, T, 16)
+        az.Runtime.sync()
+        e0 = az.Runtime.event()
+        for _ in range(launches):
+            eng.layer_moe(L, lb, NE, ob, T, 16)
+        e1 = az.Runtime.event()
+        az.Runtime.sync()
+        out[f"T{T}_layer_us"] = az.Runtime.elapsed_ms(e0, e1) / launches * 1e3
+        az.Runtime.event_release(e0)
+        az.Runtime.event_release(e1)
+        for b in (xb, lb, ob):
+            b.free()
+    eng.close()
+    return out
+
+
 def bench_producers(az, M, K):
     """The fused producers at the headline chunk's shape: RMS norm + quantization of M rows of K, SwiGLU + quantization
     of M rows of [gate(K) | up(K)]; HBM bytes = f32 rows read once + int8 rows, scales and sums written."""
@@ -361,6 +390,8 @@ def main():
         log(f"[bench] Q5_K 17408x5120: {out['other_configs']['Q5_K_17408x5120_T1']} {r5}")
         out["other_configs"]["MoE_128x8_T4096_E2048_F768_Q4_K"] = bench_moe(az, 5)
         log(f"[bench] MoE: {out['other_configs']['MoE_128x8_T4096_E2048_F768_Q4_K']}")
+        out["other_configs"]["MoE_128x8_E2048_F768_Q4_K_decode"] = bench_moe_decode(az, 50)
+        log(f"[bench] MoE decode: {out['other_configs']['MoE_128x8_E2048_F768_Q4_K_decode']}")
         out["producers_8192x5120"] = bench_producers(az, M, K)
         log(f"[bench] producers: {out['producers_8192x5120']}")
         out["machine_probes"] = bench_probes(az)

@@ -74,7 +74,13 @@ def test_routing_and_sort(rt, NE, NU, T, tm):
 @pytest.mark.parametrize("qtype,NE,NU,E,F,T,Mp", [(az.Q4_K, 8, 2, 256, 256, 40, 48), (az.Q8_0, 4, 2, 256, 512, 20, 32),
                                                    (az.Q6_K, 6, 3, 512, 256, 33, 48), (az.Q4_K, 16, 4, 512, 768, 300, 384),
                                                    (az.Q5_K, 8, 2, 512, 256, 70, 80),
-                                                   (az.IQ4_XS, 4, 2, 256, 512, 150, 160)])
+                                                   (az.IQ4_XS, 4, 2, 256, 512, 150, 160),
+                                                   # passes of 1-8 tokens: the matrix-vector expert kernels on tiles of
+                                                   # 1, 2, 4 and 8 slots (one token: its experts straight from moe_route1)
+                                                   (az.Q4_K, 128, 8, 512, 768, 1, 16), (az.Q4_K, 16, 4, 512, 256, 2, 16),
+                                                   (az.Q4_K, 8, 2, 256, 768, 3, 16), (az.Q4_K, 128, 8, 2048, 768, 8, 16),
+                                                   (az.Q8_0, 4, 2, 256, 512, 1, 16), (az.Q6_K, 6, 3, 512, 256, 5, 16),
+                                                   (az.Q5_K, 8, 2, 512, 256, 7, 16), (az.IQ4_XS, 4, 2, 256, 512, 4, 16)])
 def test_moe_layer_vs_oracle(rt, qtype, NE, NU, E, F, T, Mp):
     print(f"moe layer {TYPE_NAMES[qtype]} NE={NE} NU={NU} E={E} F={F} T={T}", flush=True)
     eng = az.Engine(Mp, max(E, F))
