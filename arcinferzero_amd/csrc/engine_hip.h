@@ -601,35 +601,58 @@ class Engine {
       }
       cl_mem tabs = nullptr;
       const std::string dd = " -DGROWS=2 -DTM=" + std::to_string(tmd) + " -DNE=" + std::to_string(NE);
-      {
-        if (L.ex[0].type != L.ex[1].type) throw std::runtime_error("layer_moe: gate and up experts of different types");
-        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + dd, "moe_gateup_q");
-        int FF = F, KK = E, MM = Mp;
-        set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
-        size_t gws[2] = {((size_t)(F + 1) / 2 * 32 + 255) / 256 * 256, tiles_max}, lws[2] = {256, 1};
+      if (L.ex[0].type != L.ex[1].type) throw std::runtime_error("layer_moe: gate and up experts of different types");
+      // One or two tokens: the gate/up kernel quantizes its own output (32 rows a work-group: one block per slot), and
+      // one token's down kernel sums its experts into x itself: 3 launches instead of 5 (ARCZ_MOE_FUSE=0: the 5).
+      static const bool fuse_off = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
+      const bool fq = !fuse_off && T <= 2 && F % 32 == 0, fc = !fuse_off && T == 1;
+      if (fq) {
+        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + " -DGROWS=4 -DTM=" + std::to_string(tmd) +
+                                           " -DQUANT=1 -DNE=" + std::to_string(NE), "moe_gateup_q");
+        int FF = F, KK = E, MM = Mp, S = slots_;
+        set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_, S, mhq_, mhsc_,
+                 mhbs_);
+        size_t gws[2] = {(size_t)(F / 32) * 256, tiles_max}, lws[2] = {256, 1};
         run("moe_gateup", k, 2, gws, lws);
+      } else {
+        {
+          cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + dd, "moe_gateup_q");
+          int FF = F, KK = E, MM = Mp;
+          set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
+          size_t gws[2] = {((size_t)(F + 1) / 2 * 32 + 255) / 256 * 256, tiles_max}, lws[2] = {256, 1};
+          run("moe_gateup", k, 2, gws, lws);
+        }
+        {
+          cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU), "moe_quant_sums");
+          int FF = F, S = slots_;
+          set_args(k, 0, mh_, FF, S, mhq_, mhsc_, mhbs_);
+          size_t gws[2] = {(size_t)256 * (F / 256), (size_t)(n + 63) / 64}, lws[2] = {256, 1};
+          run("moe_quant", k, 2, gws, lws);
+        }
       }
-      {
-        cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU), "moe_quant_sums");
-        int FF = F, S = slots_;
-        set_args(k, 0, mh_, FF, S, mhq_, mhsc_, mhbs_);
-        size_t gws[2] = {(size_t)256 * (F / 256), (size_t)(n + 63) / 64}, lws[2] = {256, 1};
-        run("moe_quant", k, 2, gws, lws);
-      }
-      {
-        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + dd, "moe_down_q");
+      if (fc) {
+        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + " -DGROWS=2 -DNE=" + std::to_string(NE),
+                             "moe_down1_q");
         int NN = E, KK = F, S = slots_;
-        set_args(k, 0, L.ex[2].raw, NN, KK, tabs, mhq_, mhsc_, S, mtiles_, swt_, my_, mhbs_);
-        size_t gws[2] = {((size_t)(E + 1) / 2 * 32 + 255) / 256 * 256, tiles_max}, lws[2] = {256, 1};
-        run("moe_down", k, 2, gws, lws);
-      }
-      {
-        cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU), "moe_combine");
-        cl_mem sh = nullptr;
-        int EE = E;
-        set_args(k, 0, x, sh, sgate_, my_, minv_, EE);
-        size_t gws[2] = {((size_t)E + 1023) / 1024 * 256, (size_t)T}, lws[2] = {256, 1};
-        run("moe_combine", k, 2, gws, lws);
+        set_args(k, 0, L.ex[2].raw, NN, KK, tabs, mhq_, mhsc_, S, mtiles_, swt_, x, mhbs_);
+        size_t gws = ((size_t)(E + 1) / 2 * 32 + 255) / 256 * 256, lws = 256;
+        run("moe_down", k, 1, &gws, &lws);
+      } else {
+        {
+          cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + dd, "moe_down_q");
+          int NN = E, KK = F, S = slots_;
+          set_args(k, 0, L.ex[2].raw, NN, KK, tabs, mhq_, mhsc_, S, mtiles_, swt_, my_, mhbs_);
+          size_t gws[2] = {((size_t)(E + 1) / 2 * 32 + 255) / 256 * 256, tiles_max}, lws[2] = {256, 1};
+          run("moe_down", k, 2, gws, lws);
+        }
+        {
+          cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU), "moe_combine");
+          cl_mem sh = nullptr;
+          int EE = E;
+          set_args(k, 0, x, sh, sgate_, my_, minv_, EE);
+          size_t gws[2] = {((size_t)E + 1023) / 1024 * 256, (size_t)T}, lws[2] = {256, 1};
+          run("moe_combine", k, 2, gws, lws);
+        }
       }
       return;
     }

@@ -347,6 +347,130 @@ __device__ inline void moe_down_rows(const uint8_t* __restrict__ raw, int N, int
   }
 }
 
+// moe_gateup_q -DQUANT: the same with the expert inputs' quantization (moe_quant_sums) done on the way out: a
+// work-group's 8 half waves take 4 rows each, one 32-block of h per slot, which the first half wave quantizes as
+// quant_store16 does -- amax over the block, q = rte(v * (127 / amax)), scale amax / 127, the sums of 16 -- and stores
+// next to the f32 values: hq [S][F], hsc [F/32][S], hbs [F/16][S].  One launch less in a pass of one or two tokens.
+template <int QT, int TM>
+__device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru, int F, int K,
+                                             const signed char* __restrict__ aq, const float* __restrict__ asc,
+                                             const short* __restrict__ absum, int M, const int* __restrict__ tiles,
+                                             const int* __restrict__ stok, float* __restrict__ h, int NE, int S,
+                                             signed char* __restrict__ hq, float* __restrict__ hsc,
+                                             short* __restrict__ hbs) {
+  constexpr int GROWS = 4;
+  __shared__ float hs[TM][32];
+  const int hl = threadIdx.x & 31, w = threadIdx.x >> 5;
+  const int fb = blockIdx.x * 32, f0 = fb + w * GROWS;  // (F is a multiple of 32: every row of the block exists)
+  const int nt = tiles[0];
+  for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = min(tiles[3 + 3 * ti], TM);
+    float ag[GROWS][TM], au[GROWS][TM];
+    size_t rows[GROWS];
+    int tok[TM];
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r) {
+      rows[r] = (size_t)e * F + f0 + r;
+#pragma unroll
+      for (int t = 0; t < TM; ++t) ag[r][t] = au[r][t] = 0.0f;
+    }
+#pragma unroll
+    for (int t = 0; t < TM; ++t) tok[t] = stok[r0 + min(t, nr - 1)];
+    gemv_acc<QT, TM, GROWS>(rg, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, ag, nr);
+    gemv_acc<QT, TM, GROWS>(ru, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, au, nr);
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r)
+#pragma unroll
+      for (int t = 0; t < TM; ++t) {
+        if (t >= nr) continue;  // (the same for the whole work-group)
+        const float g = half_wave_sum(ag[r][t]), u = half_wave_sum(au[r][t]);
+        if (hl == 0) hs[t][w * GROWS + r] = g / (1.0f + __expf(-g)) * u;
+      }
+    __syncthreads();
+    if (w == 0) {
+#pragma unroll
+      for (int t = 0; t < TM; ++t) {
+        if (t >= nr) continue;
+        const float v = hs[t][hl];
+        float amax = fabsf(v);
+#pragma unroll
+        for (int o = 16; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+        const int q = __float2int_rn(__fmul_rn(v, inv));
+        int sm = q;
+#pragma unroll
+        for (int o = 8; o >= 1; o >>= 1) sm += __shfl_xor(sm, o, 64);  // the 16 lanes of a half block
+        const size_t slot = (size_t)(r0 + t);
+        h[slot * F + fb + hl] = v;
+        hq[slot * F + fb + hl] = (signed char)q;
+        if (hl == 0) hsc[(size_t)(fb >> 5) * S + slot] = amax / 127.0f;
+        if ((hl & 15) == 0) hbs[(size_t)((fb >> 4) + (hl >> 4)) * S + slot] = (short)sm;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// moe_down1_q: one token's down projections and their sum in one kernel: x[n] += sum over the tiles (the token's NU
+// experts, one slot each, in order) of swt[slot] * (Wd[expert][n] . hq[slot]) -- moe_down_q and moe_combine without
+// the y rows in between; the same sums in the same order.
+template <int QT, int GROWS>
+__device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ hq,
+                                      const float* __restrict__ hsc, const short* __restrict__ hbs, int S,
+                                      const int* __restrict__ tiles, const float* __restrict__ swt, float* __restrict__ x,
+                                      int NE) {
+  const int hl = threadIdx.x & 31;
+  const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
+  const int n0 = hw * GROWS;
+  if (n0 >= N) return;
+  const int nt = tiles[0];
+  float v[GROWS];
+#pragma unroll
+  for (int r = 0; r < GROWS; ++r) v[r] = 0.0f;
+  for (int ti = 0; ti < nt; ++ti) {
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti];
+    float acc[GROWS][1];
+    size_t rows[GROWS];
+    const int tok[1] = {r0};
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r) {
+      rows[r] = (size_t)e * N + min(n0 + r, N - 1);
+      acc[r][0] = 0.0f;
+    }
+    gemv_acc<QT, 1, GROWS>(raw, (size_t)NE * N, rows, K, tok, hq, hsc, hbs, S, hl, acc);
+    const float wt = swt[r0];
+#pragma unroll
+    for (int r = 0; r < GROWS; ++r) v[r] += wt * half_wave_sum(acc[r][0]);
+  }
+#pragma unroll
+  for (int r = 0; r < GROWS; ++r)
+    if (hl == 0 && n0 + r < N) x[n0 + r] += v[r];
+}
+
+#define MOE_DECODE_FUSED_INST(QT)                                                                                    \
+  extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS4_TM1_QUANT1(                         \
+      const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
+      int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
+      short* hbs, int NE) {                                                                                           \
+    moe_gateup_quant_rows<QT, 1>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
+  }                                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS4_TM2_QUANT1(                         \
+      const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
+      int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
+      short* hbs, int NE) {                                                                                           \
+    moe_gateup_quant_rows<QT, 2>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
+  }                                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void moe_down1_q__QT##QT##_GROWS2(                                     \
+      const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
+      const int* tiles, const float* swt, float* x, const short* hbs, int NE) {                                      \
+    moe_down1_rows<QT, 2>(raw, N, K, hq, hsc, hbs, S, tiles, swt, x, NE);                                            \
+  }
+MOE_DECODE_FUSED_INST(8)
+MOE_DECODE_FUSED_INST(12)
+MOE_DECODE_FUSED_INST(13)
+MOE_DECODE_FUSED_INST(14)
+MOE_DECODE_FUSED_INST(23)
+
 #define MOE_DECODE_INST(QT, TM)                                                                                      \
   extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS2_TM##TM(                             \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
