@@ -170,6 +170,7 @@ int arcz_ggml_block_info(uint32_t type, int* blk, int* bytes) {
     case 13: b = 256; n = 176; break;               // Q5_K
     case 14: b = 256; n = 210; break;               // Q6_K
     case 20: b = 32; n = 18; break;                 // IQ4_NL
+    case 21: b = 256; n = 110; break;               // IQ3_S
     case 23: b = 256; n = 136; break;               // IQ4_XS
     default: return 0;
   }

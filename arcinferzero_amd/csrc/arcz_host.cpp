@@ -12,8 +12,71 @@
 
 #include "kernels/common.h"
 #define GGML_TYPE_Q4_0 2u  // (GGUF type id, src/gguf.h:19)
+#define GGML_TYPE_IQ3_S 21u  // (src/gguf.h:22)
 
 namespace {
+
+// The IQ3_S codebook (ggml's iq3s_grid, a constant of the GGUF format; the reference carries it as src/iq_tables.h:297):
+// 512 groups of four magnitudes, each one of 1, 3, ..., 15, here as three hex digits per entry: magnitude j of an entry
+// = 2 * ((code >> 3 j) & 7) + 1.
+const char kIq3sCodes[] =
+"00000100200500700800900a00c00e01001101501b02002202502702902b03003203903c03f04004104204404804904d"
+"05005305705905d06407107507a08008108508708808b08e09109509809c0a20a50a70a90ab0b80bb0c30c90cd0d00d2"
+"0d90db0de0e40e80ea0f70f90fd10010b10f11111411a12012312913814214415015215615b16116516717617b186189"
+"18b1991aa1b91c01c21c41d01d21d61db1e81ec20020120220420820920b20d20f21021221921c21e22c22e23123a240"
+"24124324624824c25125825b26126826a27827e28028a28d28f29029429a2a02a32ad2b02ba2c12c42c72c82cb2d12d7"
+"2d82dc2e12f22f830330530a30c31931b32232632832c34134834b35135835a3693903943973a43a63c13c33c83ca3d1"
+"3dd3e13f23f840040140340540740840a40c40e41141341741841a42142342542842a43743843b43d44044244844b44f"
+"45245545945c46246948148448749149349849f4a14ab4af4b94bc4c04c24c54c94d24d44d94db4e24e84f6501507510"
+"51351a51d52153a53d54454955255f56056b5785805825875915ad5b15c55c95d65d85e35e860260960b60d60f612619"
+"61b61d62262462762963363964164364564c65165366067067a67e68068a69069a69c6a86c16c86cc6d16d36d76d86e1"
+"6e36e76ed6fb70370970e71271972a73073474174874a75575a76476e77b78e7a17c17c37d07d27dd80080480a810814"
+"81781a82182883884284784984b85285885d86386986d88188388888d89189b8a08af8b28b88c48c98cb8d08d28d98dd"
+"90090291491f92093994594795197298b99c9b09c89cd9d89e39e9a02a08a0ca12a20a24a27a2aa36a3ca41a43a45a4a"
+"a51a5aa7aa80a89a93a98a9eaabac2ac7ac8ad7ae4ae9af5afbb01b04b10b1ab26b4ab56b69b6bba2bc2bc4bd2c09c0b"
+"c0dc19c1bc30c40c50c57c74c8ac9cca2cadcb2cb8cc0ccccd1ce0d15d23d32d40d43d5cd70d85da0dc9dcbe00e04e07"
+"e10e12e1ee20e2ce32e42e49e54e63e65e81e84e88e8ee91e98ea9ec2edaeddeebf01f05f0bf10f28f52f62f82f99fc0";
+struct Iq3sGrid {
+  uint8_t m[512][4];
+  Iq3sGrid() {
+    for (int i = 0; i < 512; ++i) {
+      int c = 0;
+      for (int k = 0; k < 3; ++k) {
+        const char ch = kIq3sCodes[3 * i + k];
+        c = c * 16 + (ch <= '9' ? ch - '0' : ch - 'a' + 10);
+      }
+      for (int j = 0; j < 4; ++j) m[i][j] = (uint8_t)(2 * ((c >> (3 * j)) & 7) + 1);
+    }
+  }
+};
+const Iq3sGrid kIq3s;
+
+// The 256 values of one IQ3_S superblock (110 bytes: f16 d, 64 index bytes, 8 bytes of ninth index bits, 32 sign bytes,
+// 4 bytes of scale nibbles; reference src/quants.h:240-262) as signed integers -15..15, and the 8 sub-scales 1 + 2 s.
+void iq3s_values(const uint8_t* p, int8_t* q, int* sc) {
+  const uint8_t *qs = p + 2, *qh = p + 66, *sg = p + 74, *scl = p + 106;
+  for (int ib = 0; ib < 8; ++ib) {
+    sc[ib] = 1 + 2 * ((scl[ib / 2] >> (4 * (ib % 2))) & 0xF);
+    for (int g = 0; g < 8; ++g) {
+      const uint8_t* m = kIq3s.m[qs[8 * ib + g] | (((qh[ib] >> g) & 1) << 8)];
+      for (int j = 0; j < 4; ++j) {
+        const int e = 4 * g + j;
+        q[32 * ib + e] = (int8_t)(((sg[4 * ib + e / 8] >> (e % 8)) & 1) ? -(int)m[j] : (int)m[j]);
+      }
+    }
+  }
+}
+
+// 256 six-bit values (0..63) into the ql / qh bytes of a Q6_K superblock (reference src/quants.h:115-134 read backwards)
+void q6k_pack(const int* q, uint8_t* ql, uint8_t* qh) {
+  for (int n = 0; n < 2; ++n)
+    for (int l = 0; l < 32; ++l) {
+      const int q0 = q[128 * n + l], q1 = q[128 * n + l + 32], q2 = q[128 * n + l + 64], q3 = q[128 * n + l + 96];
+      ql[64 * n + l] = (uint8_t)((q0 & 0xF) | ((q2 & 0xF) << 4));
+      ql[64 * n + l + 32] = (uint8_t)((q1 & 0xF) | ((q3 & 0xF) << 4));
+      qh[32 * n + l] = (uint8_t)((q0 >> 4) | ((q1 >> 4) << 2) | ((q2 >> 4) << 4) | ((q3 >> 4) << 6));
+    }
+}
 
 // IEEE binary16 conversions, round to nearest even, subnormals kept (the reference's own are src/quants.h:17-52)
 float f16_to_f32(uint16_t h) {
@@ -68,11 +131,11 @@ extern "C" {
 
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
-  return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : 0;
+  return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : type == GGML_TYPE_IQ3_S ? u * 110 : 0;
 }
-// (Q4_0 rows are kept on the device as Q8_0 planes: see arcz_repack_planes)
+// (Q4_0 rows are kept on the device as Q8_0 planes, IQ3_S rows as Q6_K planes: see arcz_repack_planes)
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) {
-  return raw_planes_bytes(type == GGML_TYPE_Q4_0 ? QT_Q8_0 : (int)type, rows, K / 256);
+  return raw_planes_bytes(type == GGML_TYPE_Q4_0 ? QT_Q8_0 : type == GGML_TYPE_IQ3_S ? QT_Q6_K : (int)type, rows, K / 256);
 }
 
 // GGUF rows -> device planes (layout: kernels/common.h).  0 or -1 (unsupported type / K).
@@ -131,6 +194,25 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
       memcpy(dst + pl.qh + i * 64, src + i * 210 + 128, 64);
       memcpy(dst + pl.sc + i * 16, src + i * 210 + 192, 16);
       memcpy(dst + pl.d + i * 2, src + i * 210 + 208, 2);
+    }
+    return 0;
+  }
+  if (type == GGML_TYPE_IQ3_S) {
+    // An IQ3_S superblock is d * (1 + 2 s) * (+-1, 3, ..., 15) with one s per 32 values (reference src/quants.h:240-262):
+    // exactly a Q6_K superblock with the same d, sub-scale 1 + 2 s for both 16-value halves and q = value + 32.
+    // Written out as Q6_K planes, value for value, so every Q6_K kernel serves it exactly, at 210 instead of 110 bytes
+    // per superblock on the device.
+    const PlanesQ6K pl = planes_q6k(rows, nsb);
+    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_Q6_K, rows, nsb) - (pl.d + u * 2));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i) {
+      int8_t v[256];
+      int sc[8], q[256];
+      iq3s_values(src + i * 110, v, sc);
+      for (int e = 0; e < 256; ++e) q[e] = v[e] + 32;
+      q6k_pack(q, dst + pl.ql + i * 128, dst + pl.qh + i * 64);
+      for (int b = 0; b < 16; ++b) dst[pl.sc + i * 16 + b] = (uint8_t)sc[b / 2];
+      memcpy(dst + pl.d + i * 2, src + i * 110, 2);
     }
     return 0;
   }
@@ -340,15 +422,7 @@ void arcz_quantize_q6_k(const float* src, size_t N, int K, uint8_t* out) {
       for (int i = 0; i < 16; ++i)
         q[16 * b + i] = 32 + (sd > 0 ? std::min(31, std::max(-32, (int)std::lrintf(v[16 * b + i] / sd))) : 0);
     }
-    uint8_t *ql = p, *qh = p + 128;
-    memset(p, 0, 192);
-    for (int n = 0; n < 2; ++n)
-      for (int l = 0; l < 32; ++l) {
-        const int q0 = q[128 * n + l], q1 = q[128 * n + l + 32], q2 = q[128 * n + l + 64], q3 = q[128 * n + l + 96];
-        ql[64 * n + l] = (uint8_t)((q0 & 0xF) | ((q2 & 0xF) << 4));
-        ql[64 * n + l + 32] = (uint8_t)((q1 & 0xF) | ((q3 & 0xF) << 4));
-        qh[32 * n + l] = (uint8_t)((q0 >> 4) | ((q1 >> 4) << 2) | ((q2 >> 4) << 4) | ((q3 >> 4) << 6));
-      }
+    q6k_pack(q, p, p + 128);
     memcpy(p + 192, sc, 16);
     memcpy(p + 208, &dh, 2);
   }
@@ -399,6 +473,52 @@ void arcz_quantize_iq4_xs(const float* src, size_t N, int K, uint8_t* out) {
   }
 }
 
+// f32 rows -> GGUF IQ3_S superblocks (110 bytes per 256 values; reference src/quants.h:240-262): per 32-block a step
+// amax / 15 (the codebook's largest magnitude), d = max step / 31 (fp16), sub-scale 1 + 2 s with s = the nearest of
+// 0..15; each 4 values take the codebook entry nearest to their magnitudes (all 512 tried), signs apart.  An input
+// generator for tests: no search over scales as a real quantizer would make.
+void arcz_quantize_iq3_s(const float* src, size_t N, int K, uint8_t* out) {
+  const int64_t nsbt = (int64_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < nsbt; ++s) {
+    const float* v = src + s * 256;
+    uint8_t* p = out + s * 110;
+    memset(p, 0, 110);
+    float step[8], smax = 0;
+    for (int b = 0; b < 8; ++b) {
+      float amax = 0;
+      for (int i = 0; i < 32; ++i) amax = std::fmax(amax, std::fabs(v[32 * b + i]));
+      step[b] = amax / 15.0f;
+      smax = std::fmax(smax, step[b]);
+    }
+    const uint16_t dh = f32_to_f16(smax / 31.0f);
+    const float d = f16_to_f32(dh);
+    memcpy(p, &dh, 2);
+    for (int b = 0; b < 8; ++b) {
+      const int sn = d > 0 ? std::min(15, std::max(0, (int)std::lrintf((step[b] / d - 1.0f) * 0.5f))) : 0;
+      p[106 + b / 2] |= (uint8_t)(sn << (4 * (b % 2)));
+      const float sd = d * (float)(1 + 2 * sn), inv = sd > 0 ? 1.0f / sd : 0.0f;
+      for (int g = 0; g < 8; ++g) {
+        float a[4];
+        for (int j = 0; j < 4; ++j) {
+          const float x = v[32 * b + 4 * g + j];
+          a[j] = std::fabs(x) * inv;
+          if (x < 0) p[74 + 4 * b + (4 * g + j) / 8] |= (uint8_t)(1u << ((4 * g + j) % 8));
+        }
+        int best = 0;
+        float bd = 1e30f;
+        for (int i = 0; i < 512; ++i) {
+          float e = 0;
+          for (int j = 0; j < 4; ++j) e += (a[j] - (float)kIq3s.m[i][j]) * (a[j] - (float)kIq3s.m[i][j]);
+          if (e < bd) { bd = e; best = i; }
+        }
+        p[2 + 8 * b + g] = (uint8_t)(best & 255);
+        p[66 + b] |= (uint8_t)((best >> 8) << g);
+      }
+    }
+  }
+}
+
 // f32 rows -> GGUF Q4_0 blocks the way the reference makes them (src/quants.h:444-463, llama.cpp's
 // quantize_row_q4_0_ref): d = (the value of largest magnitude) / -8, q = min(15, (int)(v / d + 8.5)).
 static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) {
@@ -419,7 +539,7 @@ static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) 
   }
 }
 
-// Quantizes f32 rows to `type` (2, 8, 12, 13, 14, 23).  0 or -1.
+// Quantizes f32 rows to `type` (2, 8, 12, 13, 14, 21, 23).  0 or -1.
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
   if (K <= 0 || K % 256) return -1;
   if (type == GGML_TYPE_Q4_0) arcz_quantize_q4_0(src, N, K, out);
@@ -428,6 +548,7 @@ int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t
   else if (type == QT_Q5_K) arcz_quantize_q5_k(src, N, K, out);
   else if (type == QT_Q6_K) arcz_quantize_q6_k(src, N, K, out);
   else if (type == QT_IQ4_XS) arcz_quantize_iq4_xs(src, N, K, out);
+  else if (type == GGML_TYPE_IQ3_S) arcz_quantize_iq3_s(src, N, K, out);
   else return -1;
   return 0;
 }

@@ -15,6 +15,7 @@
 #include "kernels/common.h"
 
 #define GGML_Q4_0 2u
+#define GGML_IQ3_S 21u
 #define GGML_Q8_0 8u
 #define GGML_Q4_K 12u
 #define GGML_Q5_K 13u
@@ -152,7 +153,8 @@ class Engine {
   // device planes on the host, then one upload.  rows = N for a matrix, n_expert * N for an expert tensor.
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
-    if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS)
+    if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS &&
+        type != GGML_IQ3_S)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
     if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))
@@ -161,8 +163,9 @@ class Engine {
       throw std::runtime_error("make_weight: " + std::to_string(nbytes) + " bytes given, " +
                                std::to_string(arcz_gguf_bytes(type, rows, K)) + " expected");
     GpuWeight w;
-    // (Q4_0 rows become Q8_0 planes on upload, value for value -- arcz_repack_planes -- and run through the Q8_0 kernels)
-    w.type = type == GGML_Q4_0 ? GGML_Q8_0 : type;
+    // (Q4_0 rows become Q8_0 planes on upload, IQ3_S rows Q6_K planes, value for value -- arcz_repack_planes -- and run
+    //  through those kernels)
+    w.type = type == GGML_Q4_0 ? GGML_Q8_0 : type == GGML_IQ3_S ? GGML_Q6_K : type;
     w.N = N;
     w.K = K;
     w.rows = rows;

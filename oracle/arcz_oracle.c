@@ -17,6 +17,8 @@
  *   orc_act_residual                    PARITY UNPINNED (no reference CPU twin, no vector); identities and bounds only
  *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
  *   IQ4_XS decode                       closed-form block; live comparison with the compiled reference header
+ *   IQ3_S decode (and its grid table)   closed-form block; golden vectors (tests/golden/ref_vectors_types2.npz) and live
+ *                                       comparison with the compiled reference header over every grid index
  *   Q5_K decode                         closed-form block; golden vectors (tests/golden/ref_vectors_q5k.npz) and live
  *                                       comparison with the compiled reference header
  *   orc_block_sums                      brute-force integer sums in numpy (int64)
@@ -47,7 +49,9 @@
 #define ORC_Q6_K 14u
 #define ORC_IQ4_XS 23u
 /* one int scale per 16 (Q6_K) or per 32 values (IQ4_XS: the same one for both halves), kept in sc6[], and no mins */
-#define ORC_Q6LIKE(t) ((t) == ORC_Q6_K || (t) == ORC_IQ4_XS)
+#define ORC_IQ3_S 21u
+#define ORC_IQLIKE(t) ((t) == ORC_IQ4_XS || (t) == ORC_IQ3_S) /* q[] holds the signed value itself */
+#define ORC_Q6LIKE(t) ((t) == ORC_Q6_K || ORC_IQLIKE(t))
 
 /* ---------------------------------------------------------------- fp16 (src/quants.h:17-52) */
 
@@ -109,6 +113,7 @@ int orc_sb_bytes(uint32_t type) {
     case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
     case ORC_IQ4_XS: return 136;
+    case ORC_IQ3_S: return 110;
     default: return 0;
   }
 }
@@ -134,6 +139,35 @@ static void scale_min_k4(int j, const uint8_t* q, int* sc, int* mn) {
  *           d                                   (src/quants.h:297-311; the table: src/iq_tables.h:364-367)
  */
 static const int8_t iq4_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+/* The IQ3_S codebook (ggml's iq3s_grid, a constant of the GGUF format; the reference carries it as
+ * src/iq_tables.h:297): 512 groups of four magnitudes, each one of 1, 3, ..., 15.  Kept as three hex digits per entry,
+ * magnitude j = 2 * ((code >> 3 j) & 7) + 1. */
+static const char iq3s_codes[] =
+"00000100200500700800900a00c00e01001101501b02002202502702902b03003203903c03f04004104204404804904d"
+"05005305705905d06407107507a08008108508708808b08e09109509809c0a20a50a70a90ab0b80bb0c30c90cd0d00d2"
+"0d90db0de0e40e80ea0f70f90fd10010b10f11111411a12012312913814214415015215615b16116516717617b186189"
+"18b1991aa1b91c01c21c41d01d21d61db1e81ec20020120220420820920b20d20f21021221921c21e22c22e23123a240"
+"24124324624824c25125825b26126826a27827e28028a28d28f29029429a2a02a32ad2b02ba2c12c42c72c82cb2d12d7"
+"2d82dc2e12f22f830330530a30c31931b32232632832c34134834b35135835a3693903943973a43a63c13c33c83ca3d1"
+"3dd3e13f23f840040140340540740840a40c40e41141341741841a42142342542842a43743843b43d44044244844b44f"
+"45245545945c46246948148448749149349849f4a14ab4af4b94bc4c04c24c54c94d24d44d94db4e24e84f6501507510"
+"51351a51d52153a53d54454955255f56056b5785805825875915ad5b15c55c95d65d85e35e860260960b60d60f612619"
+"61b61d62262462762963363964164364564c65165366067067a67e68068a69069a69c6a86c16c86cc6d16d36d76d86e1"
+"6e36e76ed6fb70370970e71271972a73073474174874a75575a76476e77b78e7a17c17c37d07d27dd80080480a810814"
+"81781a82182883884284784984b85285885d86386986d88188388888d89189b8a08af8b28b88c48c98cb8d08d28d98dd"
+"90090291491f92093994594795197298b99c9b09c89cd9d89e39e9a02a08a0ca12a20a24a27a2aa36a3ca41a43a45a4a"
+"a51a5aa7aa80a89a93a98a9eaabac2ac7ac8ad7ae4ae9af5afbb01b04b10b1ab26b4ab56b69b6bba2bc2bc4bd2c09c0b"
+"c0dc19c1bc30c40c50c57c74c8ac9cca2cadcb2cb8cc0ccccd1ce0d15d23d32d40d43d5cd70d85da0dc9dcbe00e04e07"
+"e10e12e1ee20e2ce32e42e49e54e63e65e81e84e88e8ee91e98ea9ec2edaeddeebf01f05f0bf10f28f52f62f82f99fc0";
+static void iq3s_entry(int idx, int out[4]) {
+  int c = 0;
+  for (int k = 0; k < 3; ++k) {
+    const char ch = iq3s_codes[3 * idx + k];
+    c = c * 16 + (ch <= '9' ? ch - '0' : ch - 'a' + 10);
+  }
+  for (int j = 0; j < 4; ++j) out[j] = 2 * ((c >> (3 * j)) & 7) + 1;
+}
 
 typedef struct {
   float d, dmin;
@@ -195,6 +229,25 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
     }
     return 0;
   }
+  if (type == ORC_IQ3_S) { /* 110 bytes: f16 d, qs[64] (the low 8 bits of a grid index per 4 values), qh[8] (the ninth
+                              bits of a 32-block's 8 indices), signs[32] (one bit per value), scales[4] (a nibble per
+                              32-block: sub-scale 1 + 2 s); src/quants.h:240-262 */
+    o->d = orc_fp16_to_f32(rd16(p));
+    const uint8_t *qs = p + 2, *qh = p + 66, *sg = p + 74, *scl = p + 106;
+    for (int ib = 0; ib < 8; ++ib) {
+      o->sc6[2 * ib] = o->sc6[2 * ib + 1] = 1 + 2 * ((scl[ib / 2] >> (4 * (ib % 2))) & 0xF);
+      for (int g = 0; g < 8; ++g) { /* group g of the block: values 4 g .. 4 g + 3 */
+        const int idx = qs[8 * ib + g] | (((qh[ib] >> g) & 1) << 8);
+        int m[4];
+        iq3s_entry(idx, m);
+        for (int j = 0; j < 4; ++j) {
+          const int e = 4 * g + j; /* sign bit e % 8 of the block's byte e / 8 */
+          o->q[32 * ib + e] = (int16_t)(((sg[4 * ib + e / 8] >> (e % 8)) & 1) ? -m[j] : m[j]);
+        }
+      }
+    }
+    return 0;
+  }
   if (type == ORC_Q8_0) {
     for (int b = 0; b < 8; ++b) {
       const uint8_t* blk = p + 34 * b;
@@ -222,7 +275,7 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
 static float sb_value(uint32_t type, const orc_sb* o, int e) {
   if (ORC_Q45(type)) return o->d * (float)o->sc[e / 32] * (float)o->q[e] - o->dmin * (float)o->mn[e / 32];
   if (type == ORC_Q6_K) return o->d * (float)o->sc6[e / 16] * (float)(o->q[e] - 32);
-  if (type == ORC_IQ4_XS) return o->d * (float)o->sc6[e / 16] * (float)o->q[e]; /* (src/quants.h:321-323 generic: wd * wsc * q) */
+  if (ORC_IQLIKE(type)) return o->d * (float)o->sc6[e / 16] * (float)o->q[e]; /* (src/quants.h:321-323 generic: wd * wsc * q) */
   return o->d8[e / 32] * (float)o->q[e];
 }
 

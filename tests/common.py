@@ -7,7 +7,7 @@ import oracle_lib as orc
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K, az.IQ4_XS
 TYPES = (Q8_0, Q4_K, Q6_K, Q5_K, IQ4_XS)
-TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS"}
+TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS", az.IQ3_S: "IQ3_S", az.Q4_0: "Q4_0"}
 IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64)
 
 

@@ -5,8 +5,8 @@ container that has the reference tree (make -C oracle ref); the fixture it write
 
 Functions covered: fp16_to_f32 / f32_to_fp16 (:17-52), decode_sb / dequant_row for Q8_0, Q4_K, Q6_K (:89-158,
 :519-622), quantize_act_cpu (:626-643, both scale widths), quantize_rows_q8_0 (:429-442).  A second file,
-ref_vectors_types2.npz, holds the same decode vectors for Q5_K (:91-113) and IQ4_XS (:297-311), drawn from a generator
-of its own so that the first file's bytes stay what they were.
+ref_vectors_types2.npz, holds the same decode vectors for Q5_K (:91-113), IQ4_XS (:297-311) and IQ3_S (:240-262, with
+the whole codebook), drawn from a generator of its own so that the first file's bytes stay what they were.
 """
 import ctypes as C
 import os
@@ -113,5 +113,23 @@ raw[:, 0:2] = finite_f16(nblk).reshape(-1, 1).view(np.uint8)
 raw = raw.reshape(-1)
 out5["iq4xs_raw"] = raw
 out5["iq4xs_dequant"] = orc.dequant_rows(23, raw, N, K, lib=ref)
+# ---- IQ3_S blocks (110 bytes: d, 64 index bytes, 8 bytes of ninth index bits, 32 sign bytes, 4 bytes of scale nibbles;
+# src/quants.h:240-262): random ones, and 8 superblocks whose 512 groups of four name the codebook's entries 0..511 in
+# order with d = 1, sub-scale 1 and no signs: their decoded row is the codebook itself as the reference holds it
+raw = rng.integers(0, 256, size=(nblk, 110), dtype=np.uint8)
+raw[:, 0:2] = finite_f16(nblk).reshape(-1, 1).view(np.uint8)
+raw = raw.reshape(-1)
+out5["iq3s_raw"] = raw
+out5["iq3s_dequant"] = orc.dequant_rows(21, raw, N, K, lib=ref)
+grid = np.zeros((8, 110), np.uint8)
+grid[:, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+for sb in range(8):
+    for b in range(8):
+        for g in range(8):
+            idx = 64 * sb + 8 * b + g
+            grid[sb, 2 + 8 * b + g] = idx & 255
+            grid[sb, 66 + b] |= (idx >> 8) << g
+out5["iq3s_grid_raw"] = grid.reshape(-1)
+out5["iq3s_grid_dequant"] = orc.dequant_rows(21, grid.reshape(-1), 1, 2048, lib=ref)
 np.savez_compressed(os.path.join(HERE, "ref_vectors_types2.npz"), **out5)
 print("wrote", os.path.join(HERE, "ref_vectors_types2.npz"), {k: v.shape for k, v in out5.items()})

@@ -15,7 +15,8 @@ def test_matrices_from_gguf(rt, tmp_path):
     K, N = 1024, 384
     Ws = {az.Q8_0: make_weights(az.Q8_0, N, K, seed=401), az.Q4_K: make_weights(az.Q4_K, N, K, seed=402),
           az.Q6_K: make_weights(az.Q6_K, N, K, seed=403), az.Q4_0: make_weights(az.Q4_0, N, K, seed=404),
-          az.Q5_K: make_weights(az.Q5_K, N, K, seed=405), az.IQ4_XS: make_weights(az.IQ4_XS, N, K, seed=406)}
+          az.Q5_K: make_weights(az.Q5_K, N, K, seed=405), az.IQ4_XS: make_weights(az.IQ4_XS, N, K, seed=406),
+          az.IQ3_S: make_weights(az.IQ3_S, N, K, seed=407)}
     tensors = [(f"blk.{t}.weight", t, [K, N], W) for t, W in Ws.items()]
     tensors.insert(1, ("pad.me", 0, [3], np.zeros(12, np.uint8)))      # makes the next tensor's offset matter
     p = tmp_path / "w.gguf"

@@ -157,6 +157,87 @@ def test_iq4xs_closed_form():
     assert np.array_equal(isc, np.repeat(np.array(ls) - 32, 2)) and not imn.any() and (dd == d).all()
 
 
+def test_iq3s_closed_form():
+    """IQ3_S (src/quants.h:240-262): groups of four magnitudes by 9-bit codebook index (the ninth bit of group g of a
+    block is bit g of the block's qh byte), one sign bit per value, sub-scale 1 + 2 s from a nibble.  Expected values
+    from codebook entries written out here (entry i as a little-endian word: its low byte is the first magnitude)."""
+    known = {0: (1, 1, 1, 1), 1: (3, 1, 1, 1), 4: (15, 1, 1, 1), 100: (1, 1, 15, 1), 255: (1, 5, 9, 5),
+             256: (7, 5, 9, 5), 300: (3, 5, 3, 7), 511: (1, 1, 15, 15)}
+    idxs = list(known)
+    K = 256
+    blk = np.zeros(110, np.uint8)
+    d = 0.125
+    blk[0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+    sn = [0, 15, 7, 8, 1, 14, 3, 12]
+    exp = np.zeros(K, np.float32)
+    for b in range(8):
+        blk[106 + b // 2] |= sn[b] << (4 * (b % 2))
+        for g in range(8):
+            idx = idxs[(3 * b + 5 * g) % len(idxs)]
+            blk[2 + 8 * b + g] = idx & 255
+            blk[66 + b] |= (idx >> 8) << g
+            for j in range(4):
+                e = 4 * g + j
+                neg = (e * 7 + b) % 3 == 0
+                if neg:
+                    blk[74 + 4 * b + e // 8] |= 1 << (e % 8)
+                exp[32 * b + e] = d * (1 + 2 * sn[b]) * (-known[idx][j] if neg else known[idx][j])
+    assert np.array_equal(orc.dequant_rows(orc.IQ3_S, blk, 1, K)[0], exp)
+    q, isc, imn, dd, dm = orc.decode_row_fields(orc.IQ3_S, blk, K)
+    assert np.array_equal(isc, np.repeat(1 + 2 * np.array(sn), 2)) and not imn.any() and (dd == d).all()
+
+
+def test_iq3s_golden_with_whole_codebook():
+    """The reference's decode of random IQ3_S blocks, and of blocks that name codebook entries 0..511 in order with
+    d = 1, sub-scale 1 and no signs: the second pins every entry of the codebook (odd magnitudes 1..15, 2048 values)."""
+    got = orc.dequant_rows(orc.IQ3_S, G["iq3s_raw"], 4, 512)
+    assert np.array_equal(got.view(np.uint32), G["iq3s_dequant"].view(np.uint32))
+    got = orc.dequant_rows(orc.IQ3_S, G["iq3s_grid_raw"], 1, 2048)
+    assert np.array_equal(got, G["iq3s_grid_dequant"])
+    v = got.reshape(512, 4)
+    assert set(np.unique(v)) == {1.0, 3.0, 5.0, 7.0, 9.0, 11.0, 13.0, 15.0}
+    assert len({tuple(r) for r in v}) == 512          # (all entries differ)
+    # the product's own copy of the codebook: the device planes of the same blocks are Q6_K planes holding value + 32
+    planes = az.repack_planes(az.IQ3_S, 1, 2048, G["iq3s_grid_raw"])
+    assert np.array_equal(planes, az.repack_planes(az.Q6_K, 1, 2048, _iq3s_as_q6k(G["iq3s_grid_raw"], 1, 2048)))
+
+
+def _iq3s_as_q6k(W3, N, K):
+    """The same values as GGUF Q6_K superblocks: d kept, sub-scale 1 + 2 s for both halves of a block, q = value + 32."""
+    nsb = N * K // 256
+    out = np.zeros((nsb, 210), np.uint8)
+    src = W3.reshape(nsb, 110)
+    for s in range(nsb):
+        qq, sc, _, _, _ = orc.decode_row_fields(orc.IQ3_S, src[s], 256)
+        b = (qq + 32).astype(np.int64)
+        for n in range(2):
+            q0, q1, q2, q3 = (b[128 * n + 32 * i:128 * n + 32 * i + 32] for i in range(4))
+            out[s, 64 * n:64 * n + 32] = (q0 & 15) | ((q2 & 15) << 4)
+            out[s, 64 * n + 32:64 * n + 64] = (q1 & 15) | ((q3 & 15) << 4)
+            out[s, 128 + 32 * n:128 + 32 * n + 32] = (q0 >> 4) | ((q1 >> 4) << 2) | ((q2 >> 4) << 4) | ((q3 >> 4) << 6)
+        out[s, 192:208] = sc.astype(np.int8).view(np.uint8)
+        out[s, 208:210] = src[s, 0:2]
+    return out.reshape(-1)
+
+
+@pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
+def test_iq3s_vs_compiled_reference():
+    W = az.quantize_rows(az.IQ3_S, (make_acts(16, 1024, seed=9) * 0.02).astype(np.float32))
+    a = orc.dequant_rows(orc.IQ3_S, W, 16, 1024)
+    assert np.array_equal(a.view(np.uint32), orc.dequant_rows(orc.IQ3_S, W, 16, 1024, lib=orc.ref).view(np.uint32))
+    rng = np.random.default_rng(12)
+    R = rng.integers(0, 256, size=(64, 110), dtype=np.uint8)          # every field random: all indices, signs, scales
+    R[:, 0:2] = np.frombuffer(np.float16(rng.normal(0, 0.01, size=64)).tobytes(), np.uint8).reshape(64, 2)
+    R = R.reshape(-1)
+    assert np.array_equal(orc.dequant_rows(orc.IQ3_S, R, 16, 1024).view(np.uint32),
+                          orc.dequant_rows(orc.IQ3_S, R, 16, 1024, lib=orc.ref).view(np.uint32))
+    # the Q6_K superblocks the device planes stand for decode to the same f32 values, bit for bit
+    assert np.array_equal(orc.dequant_rows(Q6_K, _iq3s_as_q6k(R, 16, 1024), 16, 1024).view(np.uint32),
+                          orc.dequant_rows(orc.IQ3_S, R, 16, 1024).view(np.uint32))
+    assert np.array_equal(az.repack_planes(az.IQ3_S, 16, 1024, R),
+                          az.repack_planes(az.Q6_K, 16, 1024, _iq3s_as_q6k(R, 16, 1024)))
+
+
 def test_q6k_closed_form():
     K = 256
     blk = np.zeros(210, np.uint8)
