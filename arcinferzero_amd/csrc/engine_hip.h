@@ -581,14 +581,20 @@ class Engine {
     const int E = L.E, F = L.F, NU = L.NU, n = T * NU;
     if (cur_T_ != T || cur_K_ != E || cur_Mp_ != Mp) throw std::runtime_error("layer_moe: the activations are not this chunk's");
     if (arcz_mem_size(x) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: x is too small");
-    // A pass of 1-8 tokens (zero/engine_moe.h:86-262): tiles of 1, 2, 4 or 8 slots through the matrix-vector kernels
-    // moe_gateup_q / moe_down_q -- one token's NU experts are the tiles straight from moe_route1, no counts, scan or
-    // scatter -- instead of the 64-slot tile GEMMs, which for one token walked K alone in 8 x 6 work-groups (128 us a
-    // layer at 128 experts x 768 x 2048; ARCZ_MOE_DECODE=0 brings that back).
+    // A pass of 1-16 tokens (zero/engine_moe.h:86-262 has this form for 1-8): small tiles through the matrix-vector
+    // kernels moe_gateup_q / moe_down_q, routed by one launch (moe_route1 for one token, whose NU experts are the tiles;
+    // moe_route_small for more) instead of the 64-slot tile GEMMs, which for one token walked K alone in 8 x 6
+    // work-groups (128 us a layer at 128 experts x 768 x 2048; ARCZ_MOE_DECODE=0 brings that back).  At 128 x 8 experts
+    // the two forms meet at 24 tokens (170 us); 16 tokens take 112 against 137 us (ARCZ_MOE_DECODE_MAX moves the limit).
     static const bool dec_off = getenv("ARCZ_MOE_DECODE") && atoi(getenv("ARCZ_MOE_DECODE")) == 0;
-    if (!dec_off && T <= 8) {
+    static const int dec_max = getenv("ARCZ_MOE_DECODE_MAX") ? atoi(getenv("ARCZ_MOE_DECODE_MAX")) : 16;
+    if (!dec_off && T <= dec_max && T * NU <= 512) {
       const int NE = L.NE;
-      const int tmd = T == 1 ? 1 : T <= 2 ? 2 : T <= 4 ? 4 : 8;
+      // (one-slot tiles at every count: eight tokens' 64 pairs hit about 50 experts, so a tile of 8 slots holds 1.3 on
+      //  average, and the one-slot kernels are the light ones: 71 us a layer against 113 with 8-slot tiles, 45 against
+      //  60 for four tokens; ARCZ_MOE_TMD=2|4|8 sets larger tiles)
+      static const int tmd_env = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
+      const int tmd = T > 1 && (tmd_env == 2 || tmd_env == 4 || tmd_env == 8) ? tmd_env : 1;
       size_t tiles_max;
       if (T == 1) {
         if (ldl < NE || arcz_mem_size(rl) < (size_t)NE * 4) throw std::runtime_error("layer_moe: router logits do not fit");
@@ -598,6 +604,16 @@ class Engine {
         size_t g1 = 64, l1 = 64;
         run("moe_route", k, 1, &g1, &l1);
         tiles_max = (size_t)NU;
+      } else if (n <= 512 && NE <= 512) {
+        // routing, scan and scatter of the few pairs in one work-group (the three launches took 19 us)
+        if (ldl < NE || arcz_mem_size(rl) < ((size_t)(T - 1) * ldl + NE) * 4) throw std::runtime_error("layer_moe: router logits do not fit");
+        cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DTM=" + std::to_string(tmd),
+                             "moe_route_small");
+        int NR = ldl, TT = T;
+        set_args(k, 0, rl, NR, TT, mids_, mwts_, sgate_, mtiles_, stok_, swt_, minv_);
+        size_t g1 = 512, l1 = 512;
+        run("moe_route", k, 1, &g1, &l1);
+        tiles_max = (size_t)(n + tmd - 1) / tmd + std::min(n, NE);
       } else {
         moe_route(L, rl, ldl, T, tmd);
         tiles_max = (size_t)(n + tmd - 1) / tmd + std::min(n, NE);
@@ -605,10 +621,11 @@ class Engine {
       cl_mem tabs = nullptr;
       const std::string dd = " -DGROWS=2 -DTM=" + std::to_string(tmd) + " -DNE=" + std::to_string(NE);
       if (L.ex[0].type != L.ex[1].type) throw std::runtime_error("layer_moe: gate and up experts of different types");
-      // One or two tokens: the gate/up kernel quantizes its own output (32 rows a work-group: one block per slot), and
-      // one token's down kernel sums its experts into x itself: 3 launches instead of 5 (ARCZ_MOE_FUSE=0: the 5).
+      // Tiles of one or two slots: the gate/up kernel quantizes its own output (32 rows a work-group: one block per
+      // slot); one-slot tiles: the down kernel sums a token's experts into x itself.  3 launches instead of 5
+      // (ARCZ_MOE_FUSE=0: the 5).
       static const bool fuse_off = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
-      const bool fq = !fuse_off && T <= 2 && F % 32 == 0, fc = !fuse_off && T == 1;
+      const bool fq = !fuse_off && tmd <= 2 && F % 32 == 0, fc = !fuse_off && tmd == 1;
       if (fq) {
         cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + " -DGROWS=4 -DTM=" + std::to_string(tmd) +
                                            " -DQUANT=1 -DNE=" + std::to_string(NE), "moe_gateup_q");
@@ -637,9 +654,10 @@ class Engine {
         cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + " -DGROWS=2 -DNE=" + std::to_string(NE),
                              "moe_down1_q");
         int NN = E, KK = F, S = slots_;
-        set_args(k, 0, L.ex[2].raw, NN, KK, tabs, mhq_, mhsc_, S, mtiles_, swt_, x, mhbs_);
-        size_t gws = ((size_t)(E + 1) / 2 * 32 + 255) / 256 * 256, lws = 256;
-        run("moe_down", k, 1, &gws, &lws);
+        int NUU = NU;
+        set_args(k, 0, L.ex[2].raw, NN, KK, tabs, mhq_, mhsc_, S, mtiles_, swt_, x, mhbs_, minv_, NUU);
+        size_t gws[2] = {((size_t)(E + 1) / 2 * 32 + 255) / 256 * 256, (size_t)T}, lws[2] = {256, 1};
+        run("moe_down", k, 2, gws, lws);
       } else {
         {
           cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + dd, "moe_down_q");

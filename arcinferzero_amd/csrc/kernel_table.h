@@ -35,7 +35,7 @@ static const KernelSpec kKernelTable[] = {
      {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mm", nullptr, "piippppiipiiiii", {"QT", nullptr}, {{nullptr, 0, false}}, 512},
     {"decode", "moe_gateup_q", "QUANT", "ppiipppippppippp", {"QT", "GROWS", "TM", "QUANT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
-    {"decode", "moe_down1_q", nullptr, "piipppipppp", {"QT", "GROWS", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
+    {"decode", "moe_down1_q", nullptr, "piipppipppppi", {"QT", "GROWS", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", "GROWS", "TM", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "moe_down_q", nullptr, "piipppipppp", {"QT", "GROWS", "TM", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_v", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{nullptr, 0, false}}, 256},
@@ -56,6 +56,8 @@ static const KernelSpec kKernelTable[] = {
     {"moe", "moe_route", nullptr, "piipppp", {nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_route1", nullptr, "pppppp", {nullptr},
      {{"NE", 0, true}, {"NU", 0, true}, {"HAS_GATE", 0, false}, {nullptr, 0, false}}, 64},
+    {"moe", "moe_route_small", nullptr, "piippppppp", {nullptr},
+     {{"NE", 0, true}, {"NU", 0, true}, {"TM", 16, false}, {nullptr, 0, false}}, 512},
     {"moe", "moe_scan", nullptr, "ppppp", {nullptr}, {{"NE", 0, true}, {"TM", 16, false}, {"NPART", 1, false}, {nullptr, 0, false}}, 1024},
     {"moe", "moe_scatter", nullptr, "ppipppp", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},
     {"moe", "moe_quant", nullptr, "piipp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},

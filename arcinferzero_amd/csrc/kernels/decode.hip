@@ -411,40 +411,39 @@ __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, con
   }
 }
 
-// moe_down1_q: one token's down projections and their sum in one kernel: x[n] += sum over the tiles (the token's NU
-// experts, one slot each, in order) of swt[slot] * (Wd[expert][n] . hq[slot]) -- moe_down_q and moe_combine without
-// the y rows in between; the same sums in the same order.
+// moe_down1_q: the down projections of a pass whose tiles hold one slot each (slot s is tile s) and their sum in one
+// kernel: x[t][n] += sum over k (in order) of swt[s] * (Wd[expert of s][n] . hq[s]), s = inv[t * NU + k] -- moe_down_q
+// and moe_combine without the y rows in between; the same sums in the same order.  grid.y = tokens.
 template <int QT, int GROWS>
 __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ hq,
                                       const float* __restrict__ hsc, const short* __restrict__ hbs, int S,
                                       const int* __restrict__ tiles, const float* __restrict__ swt, float* __restrict__ x,
-                                      int NE) {
+                                      const int* __restrict__ inv, int NU, int NE) {
   const int hl = threadIdx.x & 31;
   const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
-  const int n0 = hw * GROWS;
+  const int n0 = hw * GROWS, t = blockIdx.y;
   if (n0 >= N) return;
-  const int nt = tiles[0];
   float v[GROWS];
 #pragma unroll
   for (int r = 0; r < GROWS; ++r) v[r] = 0.0f;
-  for (int ti = 0; ti < nt; ++ti) {
-    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti];
+  for (int k = 0; k < NU; ++k) {
+    const int sl = inv[t * NU + k], e = tiles[1 + 3 * sl];
     float acc[GROWS][1];
     size_t rows[GROWS];
-    const int tok[1] = {r0};
+    const int tok[1] = {sl};
 #pragma unroll
     for (int r = 0; r < GROWS; ++r) {
       rows[r] = (size_t)e * N + min(n0 + r, N - 1);
       acc[r][0] = 0.0f;
     }
     gemv_acc<QT, 1, GROWS>(raw, (size_t)NE * N, rows, K, tok, hq, hsc, hbs, S, hl, acc);
-    const float wt = swt[r0];
+    const float wt = swt[sl];
 #pragma unroll
     for (int r = 0; r < GROWS; ++r) v[r] += wt * half_wave_sum(acc[r][0]);
   }
 #pragma unroll
   for (int r = 0; r < GROWS; ++r)
-    if (hl == 0 && n0 + r < N) x[n0 + r] += v[r];
+    if (hl == 0 && n0 + r < N) x[(size_t)t * N + n0 + r] += v[r];
 }
 
 #define MOE_DECODE_FUSED_INST(QT)                                                                                    \
@@ -462,8 +461,8 @@ __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, in
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(256) void moe_down1_q__QT##QT##_GROWS2(                                     \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
-      const int* tiles, const float* swt, float* x, const short* hbs, int NE) {                                      \
-    moe_down1_rows<QT, 2>(raw, N, K, hq, hsc, hbs, S, tiles, swt, x, NE);                                            \
+      const int* tiles, const float* swt, float* x, const short* hbs, const int* inv, int NU, int NE) {              \
+    moe_down1_rows<QT, 2>(raw, N, K, hq, hsc, hbs, S, tiles, swt, x, inv, NU, NE);                                   \
   }
 MOE_DECODE_FUSED_INST(8)
 MOE_DECODE_FUSED_INST(12)

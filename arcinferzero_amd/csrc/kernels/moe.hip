@@ -118,6 +118,95 @@ extern "C" __global__ __launch_bounds__(64) void moe_route1(const float* __restr
   }
 }
 
+// moe_route_small: the routing of a pass of a few tokens in one work-group of 512 threads -- moe_route, moe_scan and
+// moe_scatter in one launch, with the same results: wave w routes tokens w, w + 8, ... (as moe_route), then thread i places pair
+// i = (token i / NU, expert sid[i]) in slot (pairs of lower experts) + (earlier pairs of the same expert), which is
+// the scan's offset plus the scatter's rank in pair order, and the first pair of every expert writes the expert's
+// tiles of up to TM slots after those of the lower experts.  n = T * NU <= 512.
+extern "C" __global__ __launch_bounds__(512) void moe_route_small(const float* __restrict__ logits, int ldl, int T,
+                                                                  int* __restrict__ ids, float* __restrict__ wts,
+                                                                  float* __restrict__ sgate, int* __restrict__ tiles,
+                                                                  int* __restrict__ stok, float* __restrict__ swt,
+                                                                  int* __restrict__ inv, int NE, int NU, int TM) {
+  __shared__ int sid[512], ntile[512];
+  __shared__ float sw[512];
+  const int lane = threadIdx.x & 63, n = T * NU;
+  for (int t = threadIdx.x >> 6; t < T; t += 8) {
+    const float* lg = logits + (size_t)t * ldl;
+    float v[MAX_PER_LANE];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < MAX_PER_LANE; ++i) {
+      const int e = i * 64 + lane;
+      v[i] = e < NE ? lg[e] : -INFINITY;
+      mx = fmaxf(mx, v[i]);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+    float sum = 0.0f, myp = 0.0f;
+    int mysel = 0;
+    for (int k = 0; k < NU; ++k) {
+      float bv = -INFINITY;
+      int bi = NE;
+#pragma unroll
+      for (int i = 0; i < MAX_PER_LANE; ++i)
+        if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) {
+        const float ov = __shfl_xor(bv, d, 64);
+        const int oi = __shfl_xor(bi, d, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+#pragma unroll
+      for (int i = 0; i < MAX_PER_LANE; ++i)
+        if (i * 64 + lane == bi) v[i] = -INFINITY;
+      const float p = expf(bv - mx);
+      sum += p;
+      if (lane == k) { mysel = min(bi, NE - 1); myp = p; }
+    }
+    if (lane < NU) {
+      sid[t * NU + lane] = mysel;
+      sw[t * NU + lane] = myp / sum;
+      ids[(size_t)t * NU + lane] = mysel;
+      wts[(size_t)t * NU + lane] = myp / sum;
+    }
+    if (lane == 0 && sgate) sgate[t] = ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
+  }
+  __syncthreads();
+  const int i = threadIdx.x;
+  int e = -1, slot = 0, rank = 0, cnt = 0;
+  if (i < n) {
+    e = sid[i];
+    for (int j = 0; j < n; ++j) {
+      const int ej = sid[j];
+      slot += ej < e ? 1 : 0;
+      cnt += ej == e ? 1 : 0;
+      rank += (ej == e && j < i) ? 1 : 0;
+    }
+    slot += rank;
+    stok[slot] = i / NU;
+    swt[slot] = sw[i];
+    inv[i] = slot;
+  }
+  ntile[i] = (i < n && rank == 0) ? (cnt + TM - 1) / TM : 0;
+  __syncthreads();
+  if (i < n && rank == 0) {
+    int tb = 0;
+    for (int j = 0; j < n; ++j) tb += sid[j] < e ? ntile[j] : 0;
+    for (int q = 0; q < ntile[i]; ++q) {
+      int* tp = tiles + 1 + 3 * (tb + q);
+      tp[0] = e;
+      tp[1] = slot + q * TM;
+      tp[2] = min(TM, cnt - q * TM);
+    }
+  }
+  if (i == 0) {
+    int tot = 0;
+    for (int j = 0; j < n; ++j) tot += ntile[j];
+    tiles[0] = tot;
+  }
+}
+
 // moe_scan: exclusive scan of the counts -> offs / cursor; the tile list tiles[0] = number of tiles, then (expert,
 // first slot, rows <= TM) per tile; tstart[e] = first tile of expert e, tstart[NE] = the tile count; counts (all NPART copies) reset.
 // One work-group of 1024 threads (NE <= 1024).

@@ -206,14 +206,14 @@ def bench_moe(az, launches):
 
 
 def bench_moe_decode(az, launches):
-    """The same layer for passes of 1, 2, 4 and 8 tokens (the matrix-vector expert kernels): microseconds per layer,
+    """The same layer for passes of 1 to 16 tokens (the matrix-vector expert kernels): microseconds per layer,
     launches back to back."""
     NE, NU, E, F, qt = 128, 8, 2048, 768, az.Q4_K
     eng = az.Engine(16, E)
     L = eng.make_moe_layer(qt, az.gen_weights(qt, 21, NE * F, E, 0.02), az.gen_weights(qt, 22, NE * F, E, 0.02),
                            az.gen_weights(qt, 23, NE * E, F, 0.02), NE, NU, E, F)
     out = {}
-    for T in (1, 2, 4, 8):
+    for T in (1, 2, 4, 8, 16):
         xb = az.Runtime.from_numpy(az.gen_normal(24, (T, E)))
         lb = az.Runtime.from_numpy(az.gen_normal(25 + T, (T, NE)))
         ob = az.Runtime.alloc(T * E * 4).fill(0)

@@ -82,7 +82,11 @@ def test_routing_and_sort(rt, NE, NU, T, tm):
                                                    (az.Q8_0, 4, 2, 256, 512, 1, 16), (az.Q6_K, 6, 3, 512, 256, 5, 16),
                                                    (az.Q5_K, 8, 2, 512, 256, 7, 16), (az.IQ4_XS, 4, 2, 256, 512, 4, 16),
                                                    # IQ3_S experts (uploaded as Q6_K planes): one token and a tile pass
-                                                   (az.IQ3_S, 4, 2, 256, 512, 1, 16), (az.IQ3_S, 6, 2, 512, 256, 40, 48)])
+                                                   (az.IQ3_S, 4, 2, 256, 512, 1, 16), (az.IQ3_S, 6, 2, 512, 256, 40, 48),
+                                                   # 9-16 tokens: still the matrix-vector form, the routing kernel's waves
+                                                   # take two tokens each; 17: the tile GEMMs
+                                                   (az.Q4_K, 128, 8, 512, 256, 16, 16), (az.Q6_K, 8, 3, 256, 256, 11, 16),
+                                                   (az.Q4_K, 16, 4, 512, 256, 17, 32)])
 def test_moe_layer_vs_oracle(rt, qtype, NE, NU, E, F, T, Mp):
     print(f"moe layer {TYPE_NAMES[qtype]} NE={NE} NU={NU} E={E} F={F} T={T}", flush=True)
     eng = az.Engine(Mp, max(E, F))
