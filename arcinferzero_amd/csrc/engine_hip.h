@@ -596,7 +596,13 @@ class Engine {
       static const int tmd_env = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
       const int tmd = T > 1 && (tmd_env == 2 || tmd_env == 4 || tmd_env == 8) ? tmd_env : 1;
       size_t tiles_max;
-      if (T == 1) {
+      static const bool fuse_off = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
+      // one token, everything fused: the gate/up kernel routes the token itself (no routing launch: 2 launches a layer)
+      const bool froute = T == 1 && !fuse_off && F % 32 == 0 && NE <= 512 && NU <= 64;
+      if (froute) {
+        if (ldl < NE || arcz_mem_size(rl) < (size_t)NE * 4) throw std::runtime_error("layer_moe: router logits do not fit");
+        tiles_max = (size_t)NU;
+      } else if (T == 1) {
         if (ldl < NE || arcz_mem_size(rl) < (size_t)NE * 4) throw std::runtime_error("layer_moe: router logits do not fit");
         cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DHAS_GATE=" +
                                         std::to_string(ldl > NE ? 1 : 0), "moe_route1");
@@ -624,15 +630,22 @@ class Engine {
       // Tiles of one or two slots: the gate/up kernel quantizes its own output (32 rows a work-group: one block per
       // slot); one-slot tiles: the down kernel sums a token's experts into x itself.  3 launches instead of 5
       // (ARCZ_MOE_FUSE=0: the 5).
-      static const bool fuse_off = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
-      const bool fq = !fuse_off && tmd <= 2 && F % 32 == 0, fc = !fuse_off && tmd == 1;
-      if (fq) {
+      const bool fq = !fuse_off && tmd <= 2 && F % 32 == 0, fc = !fuse_off && tmd == 1 && NU <= 64;
+      if (froute) {
+        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + " -DGROWS=4 -DTM=1 -DQUANT=1 -DROUTE=1 -DNE=" +
+                                           std::to_string(NE), "moe_gateup_q");
+        int FF = F, KK = E, MM = Mp, S = slots_, NUU = NU, hg = ldl > NE ? 1 : 0;
+        set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_, S, mhq_, mhsc_,
+                 mhbs_, rl, sgate_, swt_, minv_, NUU, hg);
+        size_t gws[2] = {(size_t)(F / 32) * 512, tiles_max}, lws[2] = {512, 1};
+        run("moe_gateup", k, 2, gws, lws);
+      } else if (fq) {
         cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + " -DGROWS=4 -DTM=" + std::to_string(tmd) +
                                            " -DQUANT=1 -DNE=" + std::to_string(NE), "moe_gateup_q");
         int FF = F, KK = E, MM = Mp, S = slots_;
         set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_, S, mhq_, mhsc_,
                  mhbs_);
-        size_t gws[2] = {(size_t)(F / 32) * 256, tiles_max}, lws[2] = {256, 1};
+        size_t gws[2] = {(size_t)(F / 32) * 512, tiles_max}, lws[2] = {512, 1};
         run("moe_gateup", k, 2, gws, lws);
       } else {
         {
@@ -651,12 +664,12 @@ class Engine {
         }
       }
       if (fc) {
-        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + " -DGROWS=2 -DNE=" + std::to_string(NE),
+        cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[2].type) + " -DGROWS=4 -DNE=" + std::to_string(NE),
                              "moe_down1_q");
         int NN = E, KK = F, S = slots_;
         int NUU = NU;
         set_args(k, 0, L.ex[2].raw, NN, KK, tabs, mhq_, mhsc_, S, mtiles_, swt_, x, mhbs_, minv_, NUU);
-        size_t gws[2] = {((size_t)(E + 1) / 2 * 32 + 255) / 256 * 256, (size_t)T}, lws[2] = {256, 1};
+        size_t gws[2] = {((size_t)E + 3) / 4 * 256, (size_t)T}, lws[2] = {256, 1};
         run("moe_down", k, 2, gws, lws);
       } else {
         {

@@ -16,16 +16,19 @@
 // row's quant plane, so a wave's load instruction covers two contiguous 512-byte runs.  The token's int8 values,
 // scales and sums of a unit are loaded once and used for all GROWS rows.
 #include "common.h"
+#include "route1.h"
 
 template <int QT> struct UnitsPerSb { static constexpr int v = QT == QT_Q8_0 ? 16 : 8; };
 
 // acc[r][t] += the products of plane rows rows[r] (absolute rows of planes that hold `plane_rows` rows) with the token
 // rows tok[t] of aq / asc / absum, this half wave's share (lane hl takes the 16-byte units hl, hl + 32, ...).
-template <int QT, int TB, int GROWS>
+// SPLIT < GROWS: rows[SPLIT..GROWS) are rows of a second set of planes of the same shape, raw2 (the gate and the up
+// experts in one pass: the token's values are loaded once for both, and both matrices' loads are in flight together).
+template <int QT, int TB, int GROWS, int SPLIT = GROWS>
 __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t plane_rows, const size_t (&rows)[GROWS], int K,
                                          const int (&tok)[TB], const signed char* __restrict__ aq,
                                          const float* __restrict__ asc, const short* __restrict__ absum, int M, int hl,
-                                         float (&acc)[GROWS][TB], int nt = TB) {
+                                         float (&acc)[GROWS][TB], int nt = TB, const uint8_t* __restrict__ raw2 = nullptr) {
   const int nsb = K >> 8, units = nsb * UnitsPerSb<QT>::v;
   if constexpr (QT == QT_Q4_K || QT == QT_Q5_K) {
     const PlanesQ4K pl = planes_q4k(plane_rows, nsb);
@@ -49,8 +52,9 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
         const size_t n = rows[r];
-        const uint4 w = *(const uint4*)(raw + pl.qs + n * nsb * 128 + (size_t)u * 16);
-        const uint4 h = *(const uint4*)(raw + pl.hdr + (n * nsb + sb) * 16);
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
+        const uint4 w = *(const uint4*)(rb + pl.qs + n * nsb * 128 + (size_t)u * 16);
+        const uint4 h = *(const uint4*)(rb + pl.hdr + (n * nsb + sb) * 16);
         const float d = f16_bits_to_f32(h.x), dmin = f16_bits_to_f32(h.x >> 16);
         int sc0, sc1, mn0, mn1;
         q4k_scales_pair(h.y, h.z, h.w, j, sc0, sc1, mn0, mn1);
@@ -58,7 +62,7 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
         uint32_t wh[4] = {(w.x >> 4) & 0x0F0F0F0Fu, (w.y >> 4) & 0x0F0F0F0Fu, (w.z >> 4) & 0x0F0F0F0Fu,
                           (w.w >> 4) & 0x0F0F0F0Fu};
         if constexpr (QT == QT_Q5_K) {  // the fifth bits of the unit's 32 values
-          const uint32_t H = *(const uint32_t*)(raw + pl.qh + n * nsb * 32 + (size_t)u * 4), ww[4] = {w.x, w.y, w.z, w.w};
+          const uint32_t H = *(const uint32_t*)(rb + pl.qh + n * nsb * 32 + (size_t)u * 4), ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
           for (int k = 0; k < 4; ++k) { wl[k] = q5k_lo(ww[k], H, k); wh[k] = q5k_hi(ww[k], H, k); }
         }
@@ -97,12 +101,13 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
         const size_t n = rows[r];
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
         const size_t rs = n * nsb + sb;
-        const uint4 L = *(const uint4*)(raw + pl.ql + n * nsb * 128 + (size_t)u * 16);
-        const uint4 H = *(const uint4*)(raw + pl.qh + rs * 64 + 32 * n2 + (l0 & 31));
-        const signed char* scp = (const signed char*)(raw + pl.sc + rs * 16 + 8 * n2 + (idx & 3));
+        const uint4 L = *(const uint4*)(rb + pl.ql + n * nsb * 128 + (size_t)u * 16);
+        const uint4 H = *(const uint4*)(rb + pl.qh + rs * 64 + 32 * n2 + (l0 & 31));
+        const signed char* scp = (const signed char*)(rb + pl.sc + rs * 16 + 8 * n2 + (idx & 3));
         const int sc1 = scp[0], sc2 = scp[4];
-        const float d = f16_bits_to_f32(*(const unsigned short*)(raw + pl.d + rs * 2));
+        const float d = f16_bits_to_f32(*(const unsigned short*)(rb + pl.d + rs * 2));
         const uint32_t Lw[4] = {L.x, L.y, L.z, L.w}, Hw[4] = {H.x, H.y, H.z, H.w};
         uint32_t w1[4], w2[4];
 #pragma unroll
@@ -143,8 +148,9 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
         const size_t n = rows[r];
-        const uint4 w = *(const uint4*)(raw + pl.qs + n * nsb * 128 + (size_t)u * 16);
-        const uint2 h = *(const uint2*)(raw + pl.hdr + (n * nsb + sb) * 8);
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
+        const uint4 w = *(const uint4*)(rb + pl.qs + n * nsb * 128 + (size_t)u * 16);
+        const uint2 h = *(const uint2*)(rb + pl.hdr + (n * nsb + sb) * 8);
         const int ls = (int)(((h.y >> (4 * ib)) & 0xFu) | ((((h.x >> 16) >> (2 * ib)) & 3u) << 4)) - 32;
         const float d = f16_bits_to_f32(h.x);
         const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
@@ -184,8 +190,9 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
 #pragma unroll
       for (int r = 0; r < GROWS; ++r) {
         const size_t n = rows[r];
-        const uint4 w = *(const uint4*)(raw + pl.qs + n * nsb * 256 + (size_t)u * 16);
-        const float d = f16_bits_to_f32(*(const unsigned short*)(raw + pl.d + ((n * nsb + sb) * 8 + b) * 2));
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
+        const uint4 w = *(const uint4*)(rb + pl.qs + n * nsb * 256 + (size_t)u * 16);
+        const float d = f16_bits_to_f32(*(const unsigned short*)(rb + pl.d + ((n * nsb + sb) * 8 + b) * 2));
 #pragma unroll
         for (int t = 0; t < TB; ++t) if (t < nt) {
           int i = dot4(w.x, a[t].x, 0);
@@ -351,40 +358,74 @@ __device__ inline void moe_down_rows(const uint8_t* __restrict__ raw, int N, int
 // work-group's 8 half waves take 4 rows each, one 32-block of h per slot, which the first half wave quantizes as
 // quant_store16 does -- amax over the block, q = rte(v * (127 / amax)), scale amax / 127, the sums of 16 -- and stores
 // next to the f32 values: hq [S][F], hsc [F/32][S], hbs [F/16][S].  One launch less in a pass of one or two tokens.
-template <int QT, int TM>
+// ROUTE (one token): the work-group routes the token itself (wave 0, as moe_route1; every work-group gets the same
+// list) instead of reading a tile list, and the first work-group writes the list out for the down kernel: no routing
+// launch at all.
+struct MoeRouteArgs {
+  const float* logits;
+  float *sgate, *swt;
+  int *tiles_out, *stok_out, *inv;
+  int NU, has_gate;
+};
+template <int QT, int TM, bool ROUTE = false>
 __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru, int F, int K,
                                              const signed char* __restrict__ aq, const float* __restrict__ asc,
-                                             const short* __restrict__ absum, int M, const int* __restrict__ tiles,
-                                             const int* __restrict__ stok, float* __restrict__ h, int NE, int S,
-                                             signed char* __restrict__ hq, float* __restrict__ hsc,
-                                             short* __restrict__ hbs) {
-  constexpr int GROWS = 4;
+                                             const short* __restrict__ absum, int M, const int* tiles, const int* stok,
+                                             float* __restrict__ h, int NE, int S, signed char* __restrict__ hq,
+                                             float* __restrict__ hsc, short* __restrict__ hbs,
+                                             MoeRouteArgs ra = MoeRouteArgs()) {
+  constexpr int GR = 2;  // rows of each matrix per half wave: 16 half waves (512 threads) make the 32 rows
   __shared__ float hs[TM][32];
+  __shared__ int s_e[ROUTE ? 64 : 1];
+  if constexpr (ROUTE) {
+    if (threadIdx.x < 64) {
+      const int lane = threadIdx.x;
+      int sel;
+      float wt;
+      route_one_token(ra.logits, NE, ra.NU, lane, sel, wt);
+      s_e[lane] = sel;
+      if (blockIdx.x == 0 && blockIdx.y == 0) {
+        if (lane < ra.NU) {
+          ra.tiles_out[1 + 3 * lane] = sel;
+          ra.tiles_out[2 + 3 * lane] = lane;
+          ra.tiles_out[3 + 3 * lane] = 1;
+          ra.stok_out[lane] = 0;
+          ra.swt[lane] = wt;
+          ra.inv[lane] = lane;
+        }
+        if (lane == 0) {
+          ra.tiles_out[0] = ra.NU;
+          if (ra.sgate) ra.sgate[0] = ra.has_gate ? 1.0f / (1.0f + expf(-ra.logits[NE])) : 0.0f;
+        }
+      }
+    }
+    __syncthreads();
+  }
   const int hl = threadIdx.x & 31, w = threadIdx.x >> 5;
-  const int fb = blockIdx.x * 32, f0 = fb + w * GROWS;  // (F is a multiple of 32: every row of the block exists)
-  const int nt = tiles[0];
+  const int fb = blockIdx.x * 32, f0 = fb + w * GR;  // (F is a multiple of 32: every row of the block exists)
+  const int nt = ROUTE ? ra.NU : tiles[0];
   for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
-    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = min(tiles[3 + 3 * ti], TM);
-    float ag[GROWS][TM], au[GROWS][TM];
-    size_t rows[GROWS];
+    const int e = ROUTE ? s_e[ti] : tiles[1 + 3 * ti], r0 = ROUTE ? ti : tiles[2 + 3 * ti],
+              nr = ROUTE ? 1 : min(tiles[3 + 3 * ti], TM);
+    float a[2 * GR][TM];  // [0, GR): gate rows, [GR, 2 GR): the same rows of up
+    size_t rows[2 * GR];
     int tok[TM];
 #pragma unroll
-    for (int r = 0; r < GROWS; ++r) {
-      rows[r] = (size_t)e * F + f0 + r;
+    for (int r = 0; r < 2 * GR; ++r) {
+      rows[r] = (size_t)e * F + f0 + (r % GR);
 #pragma unroll
-      for (int t = 0; t < TM; ++t) ag[r][t] = au[r][t] = 0.0f;
+      for (int t = 0; t < TM; ++t) a[r][t] = 0.0f;
     }
 #pragma unroll
-    for (int t = 0; t < TM; ++t) tok[t] = stok[r0 + min(t, nr - 1)];
-    gemv_acc<QT, TM, GROWS>(rg, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, ag, nr);
-    gemv_acc<QT, TM, GROWS>(ru, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, au, nr);
+    for (int t = 0; t < TM; ++t) tok[t] = ROUTE ? 0 : stok[r0 + min(t, nr - 1)];
+    gemv_acc<QT, TM, 2 * GR, GR>(rg, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, a, nr, ru);
 #pragma unroll
-    for (int r = 0; r < GROWS; ++r)
+    for (int r = 0; r < GR; ++r)
 #pragma unroll
       for (int t = 0; t < TM; ++t) {
         if (t >= nr) continue;  // (the same for the whole work-group)
-        const float g = half_wave_sum(ag[r][t]), u = half_wave_sum(au[r][t]);
-        if (hl == 0) hs[t][w * GROWS + r] = g / (1.0f + __expf(-g)) * u;
+        const float g = half_wave_sum(a[r][t]), u = half_wave_sum(a[GR + r][t]);
+        if (hl == 0) hs[t][w * GR + r] = g / (1.0f + __expf(-g)) * u;
       }
     __syncthreads();
     if (w == 0) {
@@ -413,20 +454,19 @@ __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, con
 
 // moe_down1_q: the down projections of a pass whose tiles hold one slot each (slot s is tile s) and their sum in one
 // kernel: x[t][n] += sum over k (in order) of swt[s] * (Wd[expert of s][n] . hq[s]), s = inv[t * NU + k] -- moe_down_q
-// and moe_combine without the y rows in between; the same sums in the same order.  grid.y = tokens.
+// and moe_combine without the y rows in between; the same sums in the same order.  grid (ceil(N / GROWS) work-groups
+// of 256, tokens); NU <= 64.
 template <int QT, int GROWS>
 __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ hq,
                                       const float* __restrict__ hsc, const short* __restrict__ hbs, int S,
                                       const int* __restrict__ tiles, const float* __restrict__ swt, float* __restrict__ x,
                                       const int* __restrict__ inv, int NU, int NE) {
-  const int hl = threadIdx.x & 31;
-  const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
-  const int n0 = hw * GROWS, t = blockIdx.y;
-  if (n0 >= N) return;
-  float v[GROWS];
-#pragma unroll
-  for (int r = 0; r < GROWS; ++r) v[r] = 0.0f;
-  for (int k = 0; k < NU; ++k) {
+  // a work-group takes GROWS rows of x[t]; its 8 half waves take the token's experts k = w, w + 8, ... side by side
+  // (one after the other a token's 8 short rows were 8 memory latencies), and the weighted products meet in LDS
+  __shared__ float part[64][GROWS];
+  const int hl = threadIdx.x & 31, w = threadIdx.x >> 5;
+  const int n0 = blockIdx.x * GROWS, t = blockIdx.y;
+  for (int k = w; k < NU; k += 8) {
     const int sl = inv[t * NU + k], e = tiles[1 + 3 * sl];
     float acc[GROWS][1];
     size_t rows[GROWS];
@@ -439,30 +479,45 @@ __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, in
     gemv_acc<QT, 1, GROWS>(raw, (size_t)NE * N, rows, K, tok, hq, hsc, hbs, S, hl, acc);
     const float wt = swt[sl];
 #pragma unroll
-    for (int r = 0; r < GROWS; ++r) v[r] += wt * half_wave_sum(acc[r][0]);
+    for (int r = 0; r < GROWS; ++r) {
+      const float v = half_wave_sum(acc[r][0]);
+      if (hl == 0) part[k][r] = wt * v;
+    }
   }
-#pragma unroll
-  for (int r = 0; r < GROWS; ++r)
-    if (hl == 0 && n0 + r < N) x[(size_t)t * N + n0 + r] += v[r];
+  __syncthreads();
+  if (threadIdx.x < GROWS && n0 + (int)threadIdx.x < N) {
+    float v = 0.0f;
+    for (int k = 0; k < NU; ++k) v += part[k][threadIdx.x];
+    x[(size_t)t * N + n0 + threadIdx.x] += v;
+  }
 }
 
 #define MOE_DECODE_FUSED_INST(QT)                                                                                    \
-  extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS4_TM1_QUANT1(                         \
+  extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM1_QUANT1(                         \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
       short* hbs, int NE) {                                                                                           \
     moe_gateup_quant_rows<QT, 1>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
   }                                                                                                                   \
-  extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS4_TM2_QUANT1(                         \
+  extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM2_QUANT1(                         \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
       short* hbs, int NE) {                                                                                           \
     moe_gateup_quant_rows<QT, 2>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
   }                                                                                                                   \
-  extern "C" __global__ __launch_bounds__(256) void moe_down1_q__QT##QT##_GROWS2(                                     \
+  extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM1_QUANT1_ROUTE1(                  \
+      const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
+      int M, int* tiles, int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc, short* hbs,     \
+      const float* logits, float* sgate, float* swt, int* inv, int NU, int has_gate, int NE) {                        \
+    MoeRouteArgs ra;                                                                                                  \
+    ra.logits = logits; ra.sgate = sgate; ra.swt = swt; ra.tiles_out = tiles; ra.stok_out = stok; ra.inv = inv;       \
+    ra.NU = NU; ra.has_gate = has_gate;                                                                               \
+    moe_gateup_quant_rows<QT, 1, true>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs, ra);     \
+  }                                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void moe_down1_q__QT##QT##_GROWS4(                                     \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
       const int* tiles, const float* swt, float* x, const short* hbs, const int* inv, int NU, int NE) {              \
-    moe_down1_rows<QT, 2>(raw, N, K, hq, hsc, hbs, S, tiles, swt, x, inv, NU, NE);                                   \
+    moe_down1_rows<QT, 4>(raw, N, K, hq, hsc, hbs, S, tiles, swt, x, inv, NU, NE);                                   \
   }
 MOE_DECODE_FUSED_INST(8)
 MOE_DECODE_FUSED_INST(12)

@@ -3,6 +3,7 @@
 // compiles these with -DNE (experts), -DNU (experts per token), -DTM (slots per tile); here they are trailing
 // arguments.
 #include "quant.h"
+#include "route1.h"
 #include <type_traits>
 
 #define MAX_PER_LANE 8  // NE <= 512
@@ -73,43 +74,15 @@ extern "C" __global__ __launch_bounds__(64) void moe_route1(const float* __restr
                                                             float* __restrict__ swt, int* __restrict__ inv, int NE,
                                                             int NU, int has_gate) {
   const int lane = threadIdx.x & 63;
-  float v[MAX_PER_LANE];
-  float mx = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < MAX_PER_LANE; ++i) {
-    const int e = i * 64 + lane;
-    v[i] = e < NE ? logits[e] : -INFINITY;
-    mx = fmaxf(mx, v[i]);
-  }
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
-  float sum = 0.0f, myp = 0.0f;
-  int mysel = 0;
-  for (int k = 0; k < NU; ++k) {
-    float bv = -INFINITY;
-    int bi = NE;
-#pragma unroll
-    for (int i = 0; i < MAX_PER_LANE; ++i)
-      if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-      const float ov = __shfl_xor(bv, d, 64);
-      const int oi = __shfl_xor(bi, d, 64);
-      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
-#pragma unroll
-    for (int i = 0; i < MAX_PER_LANE; ++i)
-      if (i * 64 + lane == bi) v[i] = -INFINITY;
-    const float p = expf(bv - mx);
-    sum += p;
-    if (lane == k) { mysel = min(bi, NE - 1); myp = p; }
-  }
+  int mysel;
+  float mywt;
+  route_one_token(logits, NE, NU, lane, mysel, mywt);
   if (lane < NU) {
     tiles[1 + 3 * lane] = mysel;
     tiles[2 + 3 * lane] = lane;
     tiles[3 + 3 * lane] = 1;
     stok[lane] = 0;
-    swt[lane] = myp / sum;
+    swt[lane] = mywt;
     inv[lane] = lane;
   }
   if (lane == 0) {
@@ -128,60 +101,38 @@ extern "C" __global__ __launch_bounds__(512) void moe_route_small(const float* _
                                                                   float* __restrict__ sgate, int* __restrict__ tiles,
                                                                   int* __restrict__ stok, float* __restrict__ swt,
                                                                   int* __restrict__ inv, int NE, int NU, int TM) {
-  __shared__ int sid[512], ntile[512];
+  __shared__ __attribute__((aligned(16))) int sid[512], ntile[512];
   __shared__ float sw[512];
   const int lane = threadIdx.x & 63, n = T * NU;
   for (int t = threadIdx.x >> 6; t < T; t += 8) {
     const float* lg = logits + (size_t)t * ldl;
-    float v[MAX_PER_LANE];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < MAX_PER_LANE; ++i) {
-      const int e = i * 64 + lane;
-      v[i] = e < NE ? lg[e] : -INFINITY;
-      mx = fmaxf(mx, v[i]);
-    }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
-    float sum = 0.0f, myp = 0.0f;
-    int mysel = 0;
-    for (int k = 0; k < NU; ++k) {
-      float bv = -INFINITY;
-      int bi = NE;
-#pragma unroll
-      for (int i = 0; i < MAX_PER_LANE; ++i)
-        if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
-#pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) {
-        const float ov = __shfl_xor(bv, d, 64);
-        const int oi = __shfl_xor(bi, d, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-      }
-#pragma unroll
-      for (int i = 0; i < MAX_PER_LANE; ++i)
-        if (i * 64 + lane == bi) v[i] = -INFINITY;
-      const float p = expf(bv - mx);
-      sum += p;
-      if (lane == k) { mysel = min(bi, NE - 1); myp = p; }
-    }
+    int mysel;
+    float mywt;
+    route_one_token(lg, NE, NU, lane, mysel, mywt);
     if (lane < NU) {
       sid[t * NU + lane] = mysel;
-      sw[t * NU + lane] = myp / sum;
+      sw[t * NU + lane] = mywt;
       ids[(size_t)t * NU + lane] = mysel;
-      wts[(size_t)t * NU + lane] = myp / sum;
+      wts[(size_t)t * NU + lane] = mywt;
     }
     if (lane == 0 && sgate) sgate[t] = ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
   }
+  if ((int)threadIdx.x >= n) sid[threadIdx.x] = 0x7FFFFFFF;  // (past the pairs: an expert no pair has, so that the
+                                                             //  loops below can take the list four entries at a time)
   __syncthreads();
-  const int i = threadIdx.x;
+  const int i = threadIdx.x, n4 = (n + 3) & ~3;
   int e = -1, slot = 0, rank = 0, cnt = 0;
   if (i < n) {
     e = sid[i];
-    for (int j = 0; j < n; ++j) {
-      const int ej = sid[j];
-      slot += ej < e ? 1 : 0;
-      cnt += ej == e ? 1 : 0;
-      rank += (ej == e && j < i) ? 1 : 0;
+    for (int j = 0; j < n4; j += 4) {
+      const int4 q = *(const int4*)&sid[j];
+      const int ej[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        slot += ej[c] < e ? 1 : 0;
+        cnt += ej[c] == e ? 1 : 0;
+        rank += (ej[c] == e && j + c < i) ? 1 : 0;
+      }
     }
     slot += rank;
     stok[slot] = i / NU;
@@ -192,7 +143,11 @@ extern "C" __global__ __launch_bounds__(512) void moe_route_small(const float* _
   __syncthreads();
   if (i < n && rank == 0) {
     int tb = 0;
-    for (int j = 0; j < n; ++j) tb += sid[j] < e ? ntile[j] : 0;
+    for (int j = 0; j < n4; j += 4) {
+      const int4 q = *(const int4*)&sid[j];
+      const int4 nt4 = *(const int4*)&ntile[j];
+      tb += (q.x < e ? nt4.x : 0) + (q.y < e ? nt4.y : 0) + (q.z < e ? nt4.z : 0) + (q.w < e ? nt4.w : 0);
+    }
     for (int q = 0; q < ntile[i]; ++q) {
       int* tp = tiles + 1 + 3 * (tb + q);
       tp[0] = e;
@@ -200,9 +155,12 @@ extern "C" __global__ __launch_bounds__(512) void moe_route_small(const float* _
       tp[2] = min(TM, cnt - q * TM);
     }
   }
-  if (i == 0) {
+  if (i == (n < 512 ? 511 : 0)) {  // (a thread without a pair, when there is one)
     int tot = 0;
-    for (int j = 0; j < n; ++j) tot += ntile[j];
+    for (int j = 0; j < n4; j += 4) {
+      const int4 nt4 = *(const int4*)&ntile[j];
+      tot += nt4.x + nt4.y + nt4.z + nt4.w;
+    }
     tiles[0] = tot;
   }
 }
