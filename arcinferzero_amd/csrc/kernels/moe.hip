@@ -4,9 +4,7 @@
 // arguments.
 #include "quant.h"
 #include "route1.h"
-#include <type_traits>
 
-#define MAX_PER_LANE 8  // NE <= 512
 
 // moe_route: one wave per token.  The NU largest of NE logits (ties: the lower expert), p = exp(l - max),
 // weights p / sum of the selected p; counts[copy][e]++ per selection (NPART copies [NPART][NE], 1 by default); sgate[t] = sigmoid(logit NE) when the row holds one.
@@ -19,48 +17,12 @@ extern "C" __global__ __launch_bounds__(256) void moe_route(const float* __restr
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
   const float* lg = logits + (size_t)t * ldl;
-  float sum = 0.0f, myp = 0.0f;
-  int mysel = 0;
-  // (PL logits per lane: 2 serve up to 128 experts, the common case; the same steps either way)
-  auto pick = [&](auto pl_tag) {
-    constexpr int PL = decltype(pl_tag)::value;
-    float v[PL];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < PL; ++i) {
-      const int e = i * 64 + lane;
-      v[i] = e < NE ? lg[e] : -INFINITY;
-      mx = fmaxf(mx, v[i]);
-    }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) mx = fmaxf(mx, __shfl_xor(mx, d, 64));
-    for (int k = 0; k < NU; ++k) {
-      float bv = -INFINITY;
-      int bi = NE;
-#pragma unroll
-      for (int i = 0; i < PL; ++i)
-        if (v[i] > bv) { bv = v[i]; bi = i * 64 + lane; }
-      // wave arg-max, the lower index among equal values
-#pragma unroll
-      for (int d = 32; d >= 1; d >>= 1) {
-        const float ov = __shfl_xor(bv, d, 64);
-        const int oi = __shfl_xor(bi, d, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-      }
-#pragma unroll
-      for (int i = 0; i < PL; ++i)
-        if (i * 64 + lane == bi) v[i] = -INFINITY;
-      const int sel = min(bi, NE - 1);  // (a row of NaN picks no lane: keep the index inside the tables)
-      const float p = expf(bv - mx);
-      sum += p;
-      if (lane == k) { mysel = sel; myp = p; }
-    }
-  };
-  if (NE <= 128) pick(std::integral_constant<int, 2>());
-  else pick(std::integral_constant<int, MAX_PER_LANE>());
+  int mysel;
+  float mywt;
+  route_one_token(lg, NE, NU, lane, mysel, mywt);
   if (lane < NU) {
     ids[(size_t)t * NU + lane] = mysel;
-    wts[(size_t)t * NU + lane] = myp / sum;
+    wts[(size_t)t * NU + lane] = mywt;
     // (NPART copies of the counters, a work-group adding to copy blockIdx % NPART: many adds to one word from all
     //  over the chip queue up at the memory side; moe_scan sums the copies)
     atomicAdd(&counts[(size_t)(blockIdx.x % NPART) * NE + mysel], 1);
