@@ -358,14 +358,14 @@ __device__ inline void moe_down_rows(const uint8_t* __restrict__ raw, int N, int
 // work-group's 8 half waves take 4 rows each, one 32-block of h per slot, which the first half wave quantizes as
 // quant_store16 does -- amax over the block, q = rte(v * (127 / amax)), scale amax / 127, the sums of 16 -- and stores
 // next to the f32 values: hq [S][F], hsc [F/32][S], hbs [F/16][S].  One launch less in a pass of one or two tokens.
-// ROUTE (one token): the work-group routes the token itself (wave 0, as moe_route1; every work-group gets the same
-// list) instead of reading a tile list, and the first work-group writes the list out for the down kernel: no routing
-// launch at all.
+// ROUTE (up to 8 tokens, one-slot tiles, grid.y = T * NU): the work-group routes the tokens itself -- wave w token w, as
+// moe_route_small does, every work-group the same list -- and takes the pair whose slot is its blockIdx.y; the first
+// work-group writes the lists out for the down kernel.  No routing launch at all.
 struct MoeRouteArgs {
   const float* logits;
-  float *sgate, *swt;
-  int *tiles_out, *stok_out, *inv;
-  int NU, has_gate;
+  float *sgate, *swt, *wts;
+  int *tiles_out, *stok_out, *inv, *ids;
+  int NU, ldl, T;
 };
 template <int QT, int TM, bool ROUTE = false>
 __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru, int F, int K,
@@ -376,36 +376,54 @@ __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, con
                                              MoeRouteArgs ra = MoeRouteArgs()) {
   constexpr int GR = 2;  // rows of each matrix per half wave: 16 half waves (512 threads) make the 32 rows
   __shared__ float hs[TM][32];
-  __shared__ int s_e[ROUTE ? 64 : 1];
+  __shared__ __attribute__((aligned(16))) int sid[ROUTE ? 512 : 4];
+  __shared__ float sw[ROUTE ? 512 : 1];
+  __shared__ int s_et[2];  // this work-group's pair: expert, token
   if constexpr (ROUTE) {
-    if (threadIdx.x < 64) {
-      const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63, tw = threadIdx.x >> 6, NU = ra.NU, n = ra.T * NU;
+    const bool first = blockIdx.x == 0 && blockIdx.y == 0;
+    if (tw < ra.T) {
+      const float* lg = ra.logits + (size_t)tw * ra.ldl;
       int sel;
       float wt;
-      route_one_token(ra.logits, NE, ra.NU, lane, sel, wt);
-      s_e[lane] = sel;
-      if (blockIdx.x == 0 && blockIdx.y == 0) {
-        if (lane < ra.NU) {
-          ra.tiles_out[1 + 3 * lane] = sel;
-          ra.tiles_out[2 + 3 * lane] = lane;
-          ra.tiles_out[3 + 3 * lane] = 1;
-          ra.stok_out[lane] = 0;
-          ra.swt[lane] = wt;
-          ra.inv[lane] = lane;
-        }
-        if (lane == 0) {
-          ra.tiles_out[0] = ra.NU;
-          if (ra.sgate) ra.sgate[0] = ra.has_gate ? 1.0f / (1.0f + expf(-ra.logits[NE])) : 0.0f;
-        }
+      route_one_token(lg, NE, NU, lane, sel, wt);
+      if (lane < NU) {
+        sid[tw * NU + lane] = sel;
+        sw[tw * NU + lane] = wt;
+        if (first) { ra.ids[tw * NU + lane] = sel; ra.wts[tw * NU + lane] = wt; }
+      }
+      if (first && lane == 0 && ra.sgate) ra.sgate[tw] = ra.ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
+    }
+    if ((int)threadIdx.x >= n) sid[threadIdx.x] = 0x7FFFFFFF;  // (an expert no pair has: the list is read in fours)
+    __syncthreads();
+    const int i = threadIdx.x;
+    if (i < n) {  // slot of pair i = pairs of lower experts + earlier pairs of its own (moe_route_small's layout)
+      const int e = sid[i];
+      int slot = 0;
+      for (int j = 0; j < ((n + 3) & ~3); j += 4) {
+        const int4 q = *(const int4*)&sid[j];
+        const int ej[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) slot += (ej[c] < e || (ej[c] == e && j + c < i)) ? 1 : 0;
+      }
+      if (slot == (int)blockIdx.y) { s_et[0] = e; s_et[1] = i / NU; }
+      if (first) {
+        ra.tiles_out[1 + 3 * slot] = e;
+        ra.tiles_out[2 + 3 * slot] = slot;
+        ra.tiles_out[3 + 3 * slot] = 1;
+        ra.stok_out[slot] = i / NU;
+        ra.swt[slot] = sw[i];
+        ra.inv[i] = slot;
+        if (i == 0) ra.tiles_out[0] = n;
       }
     }
     __syncthreads();
   }
   const int hl = threadIdx.x & 31, w = threadIdx.x >> 5;
   const int fb = blockIdx.x * 32, f0 = fb + w * GR;  // (F is a multiple of 32: every row of the block exists)
-  const int nt = ROUTE ? ra.NU : tiles[0];
+  const int nt = ROUTE ? (int)blockIdx.y + 1 : tiles[0];  // (ROUTE: exactly the one tile)
   for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
-    const int e = ROUTE ? s_e[ti] : tiles[1 + 3 * ti], r0 = ROUTE ? ti : tiles[2 + 3 * ti],
+    const int e = ROUTE ? s_et[0] : tiles[1 + 3 * ti], r0 = ROUTE ? ti : tiles[2 + 3 * ti],
               nr = ROUTE ? 1 : min(tiles[3 + 3 * ti], TM);
     float a[2 * GR][TM];  // [0, GR): gate rows, [GR, 2 GR): the same rows of up
     size_t rows[2 * GR];
@@ -417,7 +435,7 @@ __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, con
       for (int t = 0; t < TM; ++t) a[r][t] = 0.0f;
     }
 #pragma unroll
-    for (int t = 0; t < TM; ++t) tok[t] = ROUTE ? 0 : stok[r0 + min(t, nr - 1)];
+    for (int t = 0; t < TM; ++t) tok[t] = ROUTE ? s_et[1] : stok[r0 + min(t, nr - 1)];
     gemv_acc<QT, TM, 2 * GR, GR>(rg, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, a, nr, ru);
 #pragma unroll
     for (int r = 0; r < GR; ++r)
@@ -508,10 +526,10 @@ __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, in
   extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM1_QUANT1_ROUTE1(                  \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, int* tiles, int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc, short* hbs,     \
-      const float* logits, float* sgate, float* swt, int* inv, int NU, int has_gate, int NE) {                        \
+      const float* logits, float* sgate, float* swt, int* inv, int NU, int ldl, int T, int* ids, float* wts, int NE) { \
     MoeRouteArgs ra;                                                                                                  \
     ra.logits = logits; ra.sgate = sgate; ra.swt = swt; ra.tiles_out = tiles; ra.stok_out = stok; ra.inv = inv;       \
-    ra.NU = NU; ra.has_gate = has_gate;                                                                               \
+    ra.NU = NU; ra.ldl = ldl; ra.T = T; ra.ids = ids; ra.wts = wts;                                                   \
     moe_gateup_quant_rows<QT, 1, true>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs, ra);     \
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(256) void moe_down1_q__QT##QT##_GROWS4(                                     \
