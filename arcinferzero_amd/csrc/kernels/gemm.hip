@@ -1476,13 +1476,13 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
       const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum,      \
       float* C, int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1,    \
       const int* rowmap, int use_map, const float* rowscale, int use_scale, int NE) {                                 \
-    const int t_end = tstart[e1];                                                                                     \
-    for (int ti = tstart[e0] + blockIdx.y; ti < t_end; ti += gridDim.y) {                                             \
-      const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];                                \
-      gemm2_body<QT, true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N,    \
-                           r0, min(nr, BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);                   \
-      __syncthreads();                                                                                                \
-    }                                                                                                                 \
+    /* one tile a work-group (grid.y covers the most tiles there can be, as the reference launches it,              \
+       zero/engine_moe.h:153): as a loop over tiles the body spilled 15-45 registers */                              \
+    const int ti = tstart[e0] + blockIdx.y;                                                                           \
+    if (ti >= tstart[e1]) return;                                                                                     \
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];                                  \
+    gemm2_body<QT, true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,  \
+                         min(nr, BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);                         \
   }
 
 GEMM2_INST(8)
