@@ -586,17 +586,18 @@ class Engine {
     // moe_route_small for more) instead of the 64-slot tile GEMMs, which for one token walked K alone in 8 x 6
     // work-groups (128 us a layer at 128 experts x 768 x 2048; ARCZ_MOE_DECODE=0 brings that back).  At 128 x 8 experts
     // the two forms meet at 24 tokens (170 us); 16 tokens take 112 against 137 us (ARCZ_MOE_DECODE_MAX moves the limit).
-    static const bool dec_off = getenv("ARCZ_MOE_DECODE") && atoi(getenv("ARCZ_MOE_DECODE")) == 0;
-    static const int dec_max = getenv("ARCZ_MOE_DECODE_MAX") ? atoi(getenv("ARCZ_MOE_DECODE_MAX")) : 16;
+    // (the four switches of this function are read at every call, so that a test can set them)
+    const bool dec_off = getenv("ARCZ_MOE_DECODE") && atoi(getenv("ARCZ_MOE_DECODE")) == 0;
+    const int dec_max = getenv("ARCZ_MOE_DECODE_MAX") ? atoi(getenv("ARCZ_MOE_DECODE_MAX")) : 16;
     if (!dec_off && T <= dec_max && T * NU <= 512) {
       const int NE = L.NE;
       // (one-slot tiles at every count: eight tokens' 64 pairs hit about 50 experts, so a tile of 8 slots holds 1.3 on
       //  average, and the one-slot kernels are the light ones: 71 us a layer against 113 with 8-slot tiles, 45 against
       //  60 for four tokens; ARCZ_MOE_TMD=2|4|8 sets larger tiles)
-      static const int tmd_env = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
+      const int tmd_env = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
       const int tmd = T > 1 && (tmd_env == 2 || tmd_env == 4 || tmd_env == 8) ? tmd_env : 1;
       size_t tiles_max;
-      static const bool fuse_off = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
+      const bool fuse_off = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
       // one or two tokens, everything fused: the gate/up kernel routes the tokens itself (no routing launch: 2 launches
       // a layer; the kernel takes up to 8 tokens, but every work-group routes all of them, and from 4 tokens on the
       // routing launch is the cheaper way: 36.6 against 35.7 us at 4, 65.5 against 56.4 at 8)

@@ -271,10 +271,10 @@ GEMV_ALL(13)
 GEMV_ALL(14)
 GEMV_ALL(23)
 
-// ---- the experts of a pass of 1-8 tokens (the reference's per-tile kernels moe_gateup_q / moe_down_q,
-// zero/kernels/decode.cl, launched by zero/engine_moe.h:196-262 with tiles of TM = 1, 2, 4 or 8 slots): the
-// matrix-vector form above on the rows of one expert.  A tile of the list = (expert, first slot, slots <= TM); with one
-// token moe_route1 makes its NU experts the tiles, otherwise moe_scan cuts the experts' slot ranges into tiles of TM.
+// ---- the experts of a pass of a few tokens (the reference's per-tile kernels moe_gateup_q / moe_down_q,
+// zero/kernels/decode.cl, launched by zero/engine_moe.h:196-262 with tiles of TM = 1, 2, 4 or 8 slots for 1-8 tokens):
+// the matrix-vector form above on the rows of one expert.  A tile of the list = (expert, first slot, slots <= TM), made
+// by moe_route1 (one token: its NU experts are the tiles), moe_route_small or moe_scan.
 // grid (ceil(rows / GROWS) half waves in work-groups of 256, tile work-groups: y, y + gridDim.y, ...).
 
 // moe_gateup_q: h[slot][f] = silu(gate) * up for the tile's slots, gate and up from the two expert tensors' rows

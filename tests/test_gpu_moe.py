@@ -75,8 +75,8 @@ def test_routing_and_sort(rt, NE, NU, T, tm):
                                                    (az.Q6_K, 6, 3, 512, 256, 33, 48), (az.Q4_K, 16, 4, 512, 768, 300, 384),
                                                    (az.Q5_K, 8, 2, 512, 256, 70, 80),
                                                    (az.IQ4_XS, 4, 2, 256, 512, 150, 160),
-                                                   # passes of 1-8 tokens: the matrix-vector expert kernels on tiles of
-                                                   # 1, 2, 4 and 8 slots (one token: its experts straight from moe_route1)
+                                                   # passes of 1-16 tokens: the matrix-vector expert kernels on one-slot
+                                                   # tiles (one or two tokens: routed inside the gate/up kernel)
                                                    (az.Q4_K, 128, 8, 512, 768, 1, 16), (az.Q4_K, 16, 4, 512, 256, 2, 16),
                                                    (az.Q4_K, 8, 2, 256, 768, 3, 16), (az.Q4_K, 128, 8, 2048, 768, 8, 16),
                                                    (az.Q8_0, 4, 2, 256, 512, 1, 16), (az.Q6_K, 6, 3, 512, 256, 5, 16),
@@ -88,6 +88,23 @@ def test_routing_and_sort(rt, NE, NU, T, tm):
                                                    (az.Q4_K, 128, 8, 512, 256, 16, 16), (az.Q6_K, 8, 3, 256, 256, 11, 16),
                                                    (az.Q4_K, 16, 4, 512, 256, 17, 32)])
 def test_moe_layer_vs_oracle(rt, qtype, NE, NU, E, F, T, Mp):
+    _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp)
+
+
+@pytest.mark.parametrize("env", [{"ARCZ_MOE_TMD": "2"}, {"ARCZ_MOE_TMD": "4"}, {"ARCZ_MOE_TMD": "8"},
+                                 {"ARCZ_MOE_FUSE": "0"}, {"ARCZ_MOE_FUSE": "0", "ARCZ_MOE_TMD": "4"},
+                                 {"ARCZ_MOE_DECODE": "0"}, {"ARCZ_MOE_DECODE_MAX": "4"}])
+@pytest.mark.parametrize("qtype,NE,NU,E,F,T", [(az.Q4_K, 16, 4, 512, 256, 7), (az.Q6_K, 8, 3, 256, 256, 2),
+                                               (az.Q5_K, 128, 8, 512, 256, 1)])
+def test_moe_small_pass_other_forms(rt, monkeypatch, env, qtype, NE, NU, E, F, T):
+    """The earlier forms of a small pass, which the launch-rule switches bring back (the engine reads them at every
+    call): larger tiles, the five-launch form, the tile GEMMs.  Same checks as the default form."""
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, 16)
+
+
+def _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp):
     print(f"moe layer {TYPE_NAMES[qtype]} NE={NE} NU={NU} E={E} F={F} T={T}", flush=True)
     eng = az.Engine(Mp, max(E, F))
     try:
