@@ -422,9 +422,14 @@ __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, con
   const int hl = threadIdx.x & 31, w = threadIdx.x >> 5;
   const int fb = blockIdx.x * 32, f0 = fb + w * GR;  // (F is a multiple of 32: every row of the block exists)
   const int nt = ROUTE ? (int)blockIdx.y + 1 : tiles[0];  // (ROUTE: exactly the one tile)
-  for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
-    const int e = ROUTE ? s_et[0] : tiles[1 + 3 * ti], r0 = ROUTE ? ti : tiles[2 + 3 * ti],
-              nr = ROUTE ? 1 : min(tiles[3 + 3 * ti], TM);
+  for (int ti = blockIdx.y; ROUTE || TM == 1 || ti < nt; ti += gridDim.y) {
+    // (one-slot tiles: tile ti is slot ti, so the tile's expert and the slot's token are read beside the tile count,
+    //  one memory latency instead of three in a row; an index past the lists' used part reads what lies there and is
+    //  dropped by the test below)
+    const int e = ROUTE ? s_et[0] : tiles[1 + 3 * ti], r0 = ROUTE || TM == 1 ? ti : tiles[2 + 3 * ti],
+              nr = ROUTE || TM == 1 ? 1 : min(tiles[3 + 3 * ti], TM);
+    const int tok1 = ROUTE ? s_et[1] : TM == 1 ? stok[min(ti, S - 1)] : 0;
+    if (ti >= nt) break;
     float a[2 * GR][TM];  // [0, GR): gate rows, [GR, 2 GR): the same rows of up
     size_t rows[2 * GR];
     int tok[TM];
@@ -435,7 +440,7 @@ __device__ inline void moe_gateup_quant_rows(const uint8_t* __restrict__ rg, con
       for (int t = 0; t < TM; ++t) a[r][t] = 0.0f;
     }
 #pragma unroll
-    for (int t = 0; t < TM; ++t) tok[t] = ROUTE ? s_et[1] : stok[r0 + min(t, nr - 1)];
+    for (int t = 0; t < TM; ++t) tok[t] = ROUTE || TM == 1 ? tok1 : stok[r0 + min(t, nr - 1)];
     gemv_acc<QT, TM, 2 * GR, GR>(rg, (size_t)NE * F, rows, K, tok, aq, asc, absum, M, hl, a, nr, ru);
 #pragma unroll
     for (int r = 0; r < GR; ++r)
