@@ -339,15 +339,19 @@ struct G3ScaleRegs {
   uint4 h;
 };
 
-template <bool TILES>  // (only the dense form is instantiated: over expert tiles, with their short K, the register-staged
-                       //  body above measured faster)
+// QT = Q5_K: the same with the fifth bits of a step's 128 values per row (16 bytes of the qh plane) brought into LDS by
+// one more DMA instruction of the first two waves, and merged into the nibbles when a lane reads its operand.
+template <bool TILES, int QT = QT_Q4_K>  // (only the dense form is instantiated: over expert tiles, with their short K,
+                                         //  the register-staged body above measured faster)
 __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
                                   int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
                                   size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
                                   const int* __restrict__ rowmap, int use_map, const float* __restrict__ rowscale,
                                   int use_scale) {
-  __shared__ alignas(16) uint8_t lds[2 * G3_STAGE];
+  constexpr bool Q5 = QT == QT_Q5_K;
+  constexpr int STAGE = Q5 ? G3_STAGE + 2048 : G3_STAGE, QH = G3_STAGE;  // (the fifth bits behind the scale vectors)
+  __shared__ alignas(16) uint8_t lds[2 * STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, g = lane >> 5;
@@ -376,6 +380,9 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   }
   const signed char* abase = aq + (size_t)s_begin * 256;
   const uint8_t* wbase = raw + pl.qs + (row_base * nsb + s_begin) * 128;
+  // Q5_K: row R = 64 wave + lane (waves 0 and 1) brings the 16 bytes of its step's fifth bits to QH + 16 R
+  const uint8_t* qbase = raw + pl.qh + (row_base * nsb + s_begin) * 32;
+  uint32_t qoff = (uint32_t)min(n0 + (wave & 1) * 64 + lane, N - 1) * (uint32_t)nsb * 32u;
   // scales: thread t prepares token r_s = t % 128, blocks 2 (t / 128) + {0, 1} of the step, and weight row t / 2,
   // block pair t % 2
   const int r_s = t & 127, bp = t >> 7;
@@ -386,7 +393,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   const uint8_t* hbase = raw + pl.hdr + (row_base * nsb + s_begin) * 16;
 
   auto dma_step = [&](int st, int stage) {  // st: half-superblock steps from s_begin
-    uint8_t* base = lds + stage * G3_STAGE;
+    uint8_t* base = lds + stage * STAGE;
     const signed char* ab = abase + (size_t)st * 128;
     const uint8_t* wb = wbase + (size_t)st * 64;
     // (the offsets pass through an empty asm so that the 64-bit addresses are formed here, each step, and not kept in
@@ -399,6 +406,10 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
     for (int i = 0; i < 4; ++i) g3_dma16(ab + aoff[i], base + (wave * 4 + i) * 1024);
 #pragma unroll
     for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[i], base + G3_WQ + (wave * 2 + i) * 1024);
+    if constexpr (Q5) {
+      asm volatile("" : "+v"(qoff));
+      if (wave < 2) g3_dma16(qbase + (size_t)st * 16 + qoff, base + QH + wave * 1024);
+    }
   };
   // (loads only: anything computed from them here would make the wave wait for the whole step's traffic)
   auto load_scales = [&](G3ScaleRegs& r, int st) {
@@ -413,7 +424,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
     r.h = *(const uint4*)(hbase + (size_t)(st >> 1) * 16 + hoff);
   };
   auto store_scales = [&](const G3ScaleRegs& r, int st, int stage) {
-    uint8_t* base = lds + stage * G3_STAGE;
+    uint8_t* base = lds + stage * STAGE;
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
       const float sa = tok_valid ? r.sa[q] : 0.0f;
@@ -456,7 +467,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   __syncthreads();
 
   for (int st = 0; st < steps; ++st) {
-    const uint8_t* Sb = lds + (st & 1) * G3_STAGE;
+    const uint8_t* Sb = lds + (st & 1) * STAGE;
     const bool next = st + 1 < steps;
     if (next) {  // the other stage is free: every wave has passed the barrier that ended the step reading it
       dma_step(st + 1, (st + 1) & 1);
@@ -464,15 +475,23 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
     }
 
     v4i a16[2], w16[2], wraw[2];
+    uint32_t h5[2];  // Q5_K: the fifth bits of the unit in wraw
     float saop[2], wsop, uop[2], vop[2];
     v32f P[2];
     v16i I[2];
     auto ld_a = [&](int b, int ms) { a16[ms] = *(const v4i*)(Sb + oa[b] + ms * 32 * 128); };
-    auto ld_wraw = [&](int jj, int ns) { wraw[ns] = *(const v4i*)(Sb + ow[jj] + ns * 32 * 64); };
+    auto ld_wraw = [&](int jj, int ns) {
+      wraw[ns] = *(const v4i*)(Sb + ow[jj] + ns * 32 * 64);
+      if constexpr (Q5) h5[ns] = *(const uint32_t*)(Sb + QH + (wn * 64 + ns * 32 + l32) * 16 + 4 * (2 * jj + g));
+    };
     auto dec_w = [&](int b, int ns) {  // block b of the step: low nibbles of its pair's bytes if even, high if odd
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        w16[ns][i] = (b & 1) ? (int)(((uint32_t)wraw[ns][i] >> 4) & 0x0F0F0F0Fu) : (int)((uint32_t)wraw[ns][i] & 0x0F0F0F0Fu);
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (Q5)
+          w16[ns][i] = (b & 1) ? (int)q5k_hi((uint32_t)wraw[ns][i], h5[ns], i) : (int)q5k_lo((uint32_t)wraw[ns][i], h5[ns], i);
+        else
+          w16[ns][i] = (b & 1) ? (int)(((uint32_t)wraw[ns][i] >> 4) & 0x0F0F0F0Fu) : (int)((uint32_t)wraw[ns][i] & 0x0F0F0F0Fu);
+      }
     };
     auto ld_sa = [&](int b, int ms) { saop[ms] = ((const float*)(Sb + G3_SA))[b * 128 + wm * 64 + ms * 32 + l32]; };
     auto ld_ws = [&](int b) { wsop = ((const float*)(Sb + G3_WS))[b * 128 + wn * 64 + lane]; };
@@ -1487,8 +1506,7 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
 
 GEMM2_INST(8)
 GEMM2_TILES_INST(8)
-// Q5_K: the register-staged body (the Q4_K arithmetic on values 0..31)
-GEMM2_INST(13)
+// Q5_K over expert tiles: the register-staged body (the Q4_K arithmetic on values 0..31); dense: the DMA-staged body below
 GEMM2_TILES_INST(13)
 // IQ4_XS: the register-staged body too (codes to values through the table as they are stored to LDS)
 GEMM2_INST(23)
@@ -1630,6 +1648,16 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321(
   const int m0 = tm * BM, n0 = tn * BN;
   gemm3_body<false>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
                     min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  gemm3_body<false, QT_Q5_K>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                             min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
 }
 // (tiles of at most 64 slots: the engine builds the tile list for that size)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TILES1(
