@@ -1608,8 +1608,19 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_B
     gemm2_body<QT, false>(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,           \
                           s_begin + ns * (y + 1) / ny, (size_t)N, 0, m0, min(BM, M - m0), n0, nullptr, 0, nullptr, 0); \
   }
-GEMM2_SPLITK_INST(13)
 GEMM2_SPLITK_INST(23)
+// (Q5_K: the DMA-staged body, as Q4_K)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_BM128_BN128_SPLITK1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm3_body<false, QT_Q5_K>(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+                             s_begin + ns * (y + 1) / ny, (size_t)N, 0, m0, min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
+}
 // splitk_reduce: C[m][c_off + n] (=, +=, silu(C) *) sum over the ny slices of ws [ny][M][N], slice 0 first.
 // grid: ceil(M * N / 256) work-groups of 256.
 extern "C" __global__ __launch_bounds__(256) void splitk_reduce(const float* __restrict__ ws, int ny, float* C, int M, int N,
