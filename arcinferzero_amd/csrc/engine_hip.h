@@ -416,9 +416,10 @@ class Engine {
     if (!sk_off) {
       // (tiles of 64 tokens up to 64 tokens, else of 128: the pieces of all tiles together must fit the resident slots,
       //  two work-groups per compute unit: one more piece than fits costs a whole second round)
-      // (Q8_0, Q6_K: their dense kernels' 64-token tiles; Q5_K, IQ4_XS: the register-staged body's 128-token tiles)
-      const int tm = w.type == GGML_Q8_0 || w.type == GGML_Q6_K ? 64 : w.type == GGML_Q4_K ? (Mp <= 64 ? 64 : 128) : 128;
-      const int bm = tm == 64 && w.type == GGML_Q4_K && Mp <= 32 ? 32 : tm;  // (Q4_K, at most 32 rows: the one-slot-tile kernel)
+      // (Q8_0, Q6_K: their dense kernels' 64-token tiles; IQ4_XS: the register-staged body's 128-token tiles)
+      const bool q45 = w.type == GGML_Q4_K || w.type == GGML_Q5_K;
+      const int tm = w.type == GGML_Q8_0 || w.type == GGML_Q6_K ? 64 : q45 ? (Mp <= 64 ? 64 : 128) : 128;
+      const int bm = tm == 64 && q45 && Mp <= 32 ? 32 : tm;  // (Q4_K / Q5_K, at most 32 rows: the one-slot-tile kernel)
       const size_t tiles64 = (size_t)((Mp + tm - 1) / tm) * ((N + 127) / 128), slots = 2 * (size_t)arcz_device_cus();
       const int nsb = K / 256;
       static const int sk_force = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : 0;
@@ -693,8 +694,11 @@ class Engine {
       }
       return;
     }
-    // slots per tile = the token rows of one work-group of the tile GEMM: 64 for Q4_K experts, 128 for the others
-    const int tm = L.ex[0].type == GGML_Q4_K ? 64 : 128;
+    // slots per tile = the token rows of one work-group of the tile GEMM: 64 when any of the three tensors is Q4_K or
+    // Q5_K (their tile kernel takes at most 64; the others' take up to 128 and run 64-slot tiles as well), else 128
+    bool t64 = false;
+    for (int i = 0; i < 3; ++i) t64 = t64 || L.ex[i].type == GGML_Q4_K || L.ex[i].type == GGML_Q5_K;
+    const int tm = t64 ? 64 : 128;
     moe_route(L, rl, ldl, T, tm);
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)
     const size_t max_tiles = (size_t)(n + tm - 1) / tm + std::min(n, L.NE);

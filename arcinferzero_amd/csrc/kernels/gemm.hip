@@ -816,14 +816,17 @@ struct G4ScaleRegs {
 
 // TWO = false: tiles of at most 32 slots; the second slot tile, whose scales would all be zero, is left out (half
 // the matrix and vector instructions of a step).
-template <bool TWO = true>
+// QT = Q5_K: as in the 128 x 128 body, a step's fifth bits (16 bytes a row) by one more DMA of the first two waves.
+template <bool TWO = true, int QT = QT_Q4_K>
 __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
                                   int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
                                   size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
                                   const int* __restrict__ rowmap, int use_map, const float* __restrict__ rowscale,
                                   int use_scale) {
-  __shared__ alignas(16) uint8_t lds[2 * G4_STAGE];
+  constexpr bool Q5 = QT == QT_Q5_K;
+  constexpr int STAGE = Q5 ? G4_STAGE + 2048 : G4_STAGE, QH = G4_STAGE;
+  __shared__ alignas(16) uint8_t lds[2 * STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int l32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
@@ -843,6 +846,8 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
   }
   const signed char* abase = aq + (size_t)s_begin * 256;
   const uint8_t* wbase = raw + pl.qs + (row_base * nsb + s_begin) * 128;
+  const uint8_t* qbase = raw + pl.qh + (row_base * nsb + s_begin) * 32;  // Q5_K: row 64 wave + lane, waves 0 and 1
+  uint32_t qoff = (uint32_t)min(n0 + (wave & 1) * 64 + lane, N - 1) * (uint32_t)nsb * 32u;
   // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t / 2, block pair t % 2
   const int r_s = t & 63, b_s = t >> 6;
   const bool tok_valid = r_s < rows_valid;
@@ -850,13 +855,17 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
 
   auto dma_step = [&](int st, int stage) {
-    uint8_t* base = lds + stage * G4_STAGE;
+    uint8_t* base = lds + stage * STAGE;
     const signed char* ab = abase + (size_t)st * 128;
     const uint8_t* wb = wbase + (size_t)st * 64;
 #pragma unroll
     for (int i = 0; i < 2; ++i) g3_dma16(ab + aoff[i], base + (wave * 2 + i) * 1024);
 #pragma unroll
     for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[i], base + G4_WQ + (wave * 2 + i) * 1024);
+    if constexpr (Q5) {
+      asm volatile("" : "+v"(qoff));
+      if (wave < 2) g3_dma16(qbase + (size_t)st * 16 + qoff, base + QH + wave * 1024);
+    }
   };
   // (loads only: anything computed from them here would make the wave wait for the whole step's traffic)
   auto load_scales = [&](G4ScaleRegs& r, int st) {
@@ -867,7 +876,7 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
     r.h = *(const uint4*)(raw + pl.hdr + ((row_base + n_s) * nsb + s_begin + (st >> 1)) * 16);
   };
   auto store_scales = [&](const G4ScaleRegs& r, int st, int stage) {
-    uint8_t* base = lds + stage * G4_STAGE;
+    uint8_t* base = lds + stage * STAGE;
     const float sa = tok_valid ? r.sa : 0.0f;
     ((float*)(base + G4_SA))[b_s * 64 + r_s] = sa;
     ((float*)(base + G4_U))[b_s * 64 + r_s] = sa * (float)((int)r.bs[0] + (int)r.bs[1]);
@@ -905,7 +914,7 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
 
 #pragma unroll 1
   for (int st = 0; st < steps; ++st) {
-    const uint8_t* Sb = lds + (st & 1) * G4_STAGE;
+    const uint8_t* Sb = lds + (st & 1) * STAGE;
     const bool next = st + 1 < steps;
     if (next) {
       dma_step(st + 1, (st + 1) & 1);
@@ -913,6 +922,11 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
     }
     // packed weights of the lane's row for the whole step: block pairs (0, 1) and (2, 3)
     const v4i wr0 = *(const v4i*)(Sb + ow[0]), wr1 = *(const v4i*)(Sb + ow[1]);
+    uint32_t h50 = 0, h51 = 0;  // Q5_K: the fifth bits of the units in wr0, wr1
+    if constexpr (Q5) {
+      h50 = *(const uint32_t*)(Sb + QH + (wave * 32 + l32) * 16 + 4 * g);
+      h51 = *(const uint32_t*)(Sb + QH + (wave * 32 + l32) * 16 + 4 * (2 + g));
+    }
     v4i a16[2][2], w16[2];  // [buffer][ms]; [buffer]
     float saop[2], wsop[2], uop[2], vop;
     v32f P[2];
@@ -927,7 +941,12 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const uint32_t x = (uint32_t)((b >> 1) ? wr1[i] : wr0[i]);
-        w16[buf][i] = (int)((b & 1) ? (x >> 4) & 0x0F0F0F0Fu : x & 0x0F0F0F0Fu);
+        if constexpr (Q5) {
+          const uint32_t H = (b >> 1) ? h51 : h50;
+          w16[buf][i] = (int)((b & 1) ? q5k_hi(x, H, i) : q5k_lo(x, H, i));
+        } else {
+          w16[buf][i] = (int)((b & 1) ? (x >> 4) & 0x0F0F0F0Fu : x & 0x0F0F0F0Fu);
+        }
       }
     };
     auto mfma_p = [&](int buf) {
@@ -1506,8 +1525,7 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
 
 GEMM2_INST(8)
 GEMM2_TILES_INST(8)
-// Q5_K over expert tiles: the register-staged body (the Q4_K arithmetic on values 0..31); dense: the DMA-staged body below
-GEMM2_TILES_INST(13)
+// Q5_K: the DMA-staged bodies below (the Q4_K arithmetic on values 0..31)
 // IQ4_XS: the register-staged body too (codes to values through the table as they are stored to LDS)
 GEMM2_INST(23)
 GEMM2_TILES_INST(23)
@@ -1558,6 +1576,26 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM32_B
   const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
   gemm4_body<false>(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
                     s_begin + ns * (y + 1) / ny, (size_t)N, 0, 0, min(32, M), n0, nullptr, 0, nullptr, 0);
+}
+// (the same two for Q5_K)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_BM64_BN128_SPLITK1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm4_body<true, QT_Q5_K>(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+                            s_begin + ns * (y + 1) / ny, (size_t)N, 0, m0, min(G6_BM, M - m0), n0, nullptr, 0, nullptr, 0);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_BM32_BN128_SPLITK1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int n0 = blockIdx.x * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm4_body<false, QT_Q5_K>(raw, aq, asc, absum, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+                             s_begin + ns * (y + 1) / ny, (size_t)N, 0, 0, min(32, M), n0, nullptr, 0, nullptr, 0);
 }
 // (-DBM=128 -DBN=128 -DSPLITK: the same over the 128 x 128 tiles of the dense kernel, for 65-128 tokens)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM128_BN128_SPLITK1(
@@ -1682,6 +1720,18 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TI
                      min(nr, G6_BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
     __syncthreads();
   }
+}
+
+// (Q5_K experts: the same body, one tile of at most 64 slots per work-group)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_MOE_TILES1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
+    int use_map, const float* rowscale, int use_scale, int NE) {
+  const int ti = tstart[e0] + blockIdx.y;
+  if (ti >= tstart[e1]) return;
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm4_body<true, QT_Q5_K>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N,
+                            r0, min(nr, G6_BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
 }
 
 // Q6_K: the dense form has its own body (64-token tiles: grid ceil(N / 128) * ceil(M / 64) work-groups); the form over
