@@ -106,13 +106,14 @@ def test_gemm_epilogues(eng):
     assert np.array_equal(ys[:, :c_off], c0[:, :c_off])
 
 
-@pytest.mark.parametrize("T,Mp,N,K", [(64, 64, 130, 4096), (40, 48, 300, 5120), (100, 112, 260, 2560), (128, 128, 128, 4096)])
-def test_gemm_split_k(eng, T, Mp, N, K):
-    """Short Q4_K chunks whose tiles are few: K shared out over several work-groups per tile, partial tiles added in a
-    fixed order by a second kernel that also applies c_off and the accumulate mode (tiles of 64 tokens up to 64 tokens,
-    of 128 above).  Parity with the oracle, the three epilogues, the same bits on every run."""
-    qtype = az.Q4_K
-    print(f"gemm split-K T={T} Mp={Mp} N={N} K={K}", flush=True)
+@pytest.mark.parametrize("qtype", [az.Q4_K, az.Q5_K])
+@pytest.mark.parametrize("T,Mp,N,K", [(64, 64, 130, 4096), (40, 48, 300, 5120), (100, 112, 260, 2560), (128, 128, 128, 4096),
+                                      (20, 32, 200, 4096), (17, 32, 129, 2560)])
+def test_gemm_split_k(eng, qtype, T, Mp, N, K):
+    """Short Q4_K / Q5_K chunks whose tiles are few: K shared out over several work-groups per tile, partial tiles added
+    in a fixed order by a second kernel that also applies c_off and the accumulate mode (tiles of 32 tokens up to 32
+    tokens, of 64 up to 64, of 128 above).  Parity with the oracle, the three epilogues, the same bits on every run."""
+    print(f"gemm split-K {TYPE_NAMES[qtype]} T={T} Mp={Mp} N={N} K={K}", flush=True)
     W = make_weights(qtype, N, K, seed=71)
     x = make_acts(T, K, seed=72 + T, outliers=True)
     y0 = run_gemm(eng, qtype, W, N, K, x, Mp)
@@ -132,12 +133,14 @@ def test_gemm_split_k(eng, T, Mp, N, K):
     assert np.array_equal(ys[:, :c_off], c0[:, :c_off])
 
 
-def test_gemm_split_k_unit_scales_exact(eng):
+@pytest.mark.parametrize("qtype", [az.Q4_K, az.Q5_K])
+@pytest.mark.parametrize("T", [64, 32])
+def test_gemm_split_k_unit_scales_exact(eng, qtype, T):
     """Unit scales: the sum of the partial tiles is the exact integer sum (every partial sum below 2^24)."""
-    T, N, K = 64, 96, 4096
-    W, wi = unit_scale_weights(az.Q4_K, N, K, seed=75)
+    N, K = 96, 4096
+    W, wi = unit_scale_weights(qtype, N, K, seed=75)
     x = unit_scale_acts(T, K, seed=76)
-    y = run_gemm(eng, az.Q4_K, W, N, K, x, 64)
+    y = run_gemm(eng, qtype, W, N, K, x, T)
     assert np.array_equal(y, (x.astype(np.int64) @ wi.T).astype(np.float32))
 
 

@@ -74,6 +74,8 @@ def test_routing_and_sort(rt, NE, NU, T, tm):
 @pytest.mark.parametrize("qtype,NE,NU,E,F,T,Mp", [(az.Q4_K, 8, 2, 256, 256, 40, 48), (az.Q8_0, 4, 2, 256, 512, 20, 32),
                                                    (az.Q6_K, 6, 3, 512, 256, 33, 48), (az.Q4_K, 16, 4, 512, 768, 300, 384),
                                                    (az.Q5_K, 8, 2, 512, 256, 70, 80),
+                                                   # Q5_K experts with several tiles each, full ones among them
+                                                   (az.Q5_K, 4, 2, 256, 512, 300, 320),
                                                    (az.IQ4_XS, 4, 2, 256, 512, 150, 160),
                                                    # passes of 1-16 tokens: the matrix-vector expert kernels on one-slot
                                                    # tiles (one or two tokens: routed inside the gate/up kernel)
@@ -127,7 +129,7 @@ def _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp):
         ref, href = orc.moe_layer(qtype, Wg, Wu, Wd, NE, NU, E, F, aq[:T], asc, logits)
         err = rel_err_rows(out - x0, ref)
         print(f"  layer rel err {err.max():.2e}")
-        assert np.isfinite(out).all() and err.max() <= 1e-3
+        assert np.isfinite(out).all()
         # h on the GPU (slot order) against the oracle's (pair order), then the second quantization bit for bit
         n = T * NU
         S = eng.moe_slots
@@ -136,6 +138,29 @@ def _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp):
         assert rel_err_rows(h[inv], href).max() <= 1e-3
         hq = eng.moe_buffer("hq").read(np.int8, S * F).reshape(S, F)
         hsc = eng.moe_buffer("hsc").read(np.float32, (F // 32) * S).reshape(F // 32, S)
+        # The whole layer against the oracle's: 1e-3 for every token whose int8 h equals the quantized h of the oracle.
+        # The two h differ in their last bits (summation order), so a value on a rounding boundary may come out one
+        # step apart; such a token's row carries that step (about 1 / 127 of one block maximum) and is held to 1e-2
+        # here and, through the GPU's own int8 h, to 1e-3 by the check of the down projection below.
+        flipped = np.zeros(T, bool)
+        flipped[np.nonzero((hq[inv] != orc.moe_quant(href)[0]).any(axis=1))[0] // NU] = True
+        print(f"  tokens with an int8 h one step from the oracle's: {int(flipped.sum())}")
+        assert flipped.sum() <= max(1, T // 20)
+        assert err[~flipped].max(initial=0.0) <= 1e-3 and err.max() <= 1e-2
+        if T >= 17:
+            # the tile passes keep the down projection's weighted rows in y [S][E]: each expert's slots against the
+            # oracle's matmul on the GPU's own int8 h
+            y = eng.moe_buffer("y").read(np.float32, S * E).reshape(S, E)
+            ids = eng.moe_buffer("ids").read(np.int32, n)
+            swt = eng.moe_buffer("swt").read(np.float32, n)
+            e_of_slot = np.full(S, -1)
+            e_of_slot[inv] = ids
+            rb = az.gguf_bytes(qtype, E, F)
+            for e in range(NE):
+                sl = np.nonzero(e_of_slot == e)[0]
+                if sl.size:
+                    yr = orc.matmul_ref(qtype, Wd[e * rb:(e + 1) * rb], E, F, hq[sl], np.ascontiguousarray(hsc[:, sl]))
+                    assert rel_err_rows(y[sl], yr * swt[sl, None]).max() <= 1e-3
         used = np.sort(inv)
         rq, rsc = orc.moe_quant(h[used])
         assert np.array_equal(hq[used], rq)
