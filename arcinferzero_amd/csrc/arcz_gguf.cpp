@@ -22,7 +22,7 @@ struct Tensor {
   uint64_t offset = 0, nbytes = 0;
 };
 struct Value {
-  enum Kind { INT, FLOAT, STRING, OTHER } kind = OTHER;
+  enum Kind { INT, BOOL, FLOAT, STRING, OTHER } kind = OTHER;  // (BOOL: an integer to get_int, nothing to get_float, as src/gguf.h:151-166)
   int64_t i = 0;
   double f = 0.0;
   std::string s;
@@ -79,7 +79,7 @@ struct arcz_gguf {
       case 4: v.kind = Value::INT; v.i = rd<uint32_t>(); break;
       case 5: v.kind = Value::INT; v.i = rd<int32_t>(); break;
       case 6: v.kind = Value::FLOAT; v.f = rd<float>(); break;
-      case 7: v.kind = Value::INT; v.i = rd<uint8_t>() != 0; break;
+      case 7: v.kind = Value::BOOL; v.i = rd<uint8_t>() != 0; break;
       case 8: v.kind = Value::STRING; v.s = rd_str(); break;
       case 10: v.kind = Value::INT; v.i = (int64_t)rd<uint64_t>(); break;
       case 11: v.kind = Value::INT; v.i = rd<int64_t>(); break;
@@ -129,7 +129,7 @@ struct arcz_gguf {
       index[t.name] = i;
     }
     auto it = kv.find("general.alignment");
-    const int64_t a = it != kv.end() && it->second.kind == Value::INT ? it->second.i : 32;
+    const int64_t a = it != kv.end() && (it->second.kind == Value::INT || it->second.kind == Value::BOOL) ? it->second.i : 32;
     if (a <= 0 || a > (1 << 20) || (a & (a - 1))) throw std::runtime_error("bad alignment " + std::to_string(a));
     align = (uint64_t)a;
     data_start = (pos + align - 1) / align * align;
@@ -172,6 +172,18 @@ int arcz_ggml_block_info(uint32_t type, int* blk, int* bytes) {
     case 20: b = 32; n = 18; break;                 // IQ4_NL
     case 21: b = 256; n = 110; break;               // IQ3_S
     case 23: b = 256; n = 136; break;               // IQ4_XS
+    // types the matmul path does not take (make_weight refuses them) but a model file may hold: sized, so that the
+    // directory of such a file still parses
+    case 16: b = 256; n = 66; break;                // IQ2_XXS
+    case 17: b = 256; n = 74; break;                // IQ2_XS
+    case 22: b = 256; n = 82; break;                // IQ2_S
+    case 18: b = 256; n = 98; break;                // IQ3_XXS
+    case 19: b = 256; n = 50; break;                // IQ1_S
+    case 29: b = 256; n = 56; break;                // IQ1_M
+    case 39: b = 32; n = 17; break;                 // MXFP4
+    case 43: b = 32; n = 33; break;                 // MXFP8
+    case 42: b = 64; n = 18; break;                 // Q2_0
+    case 0x41523447u: b = 128; n = 66; break;       // AR4_128
     default: return 0;
   }
   if (blk) *blk = b;
@@ -209,7 +221,7 @@ uint64_t arcz_gguf_alignment(const arcz_gguf* g) { return g->align; }
 
 int arcz_gguf_kv_i64(const arcz_gguf* g, const char* key, int64_t* out) {
   auto it = g->kv.find(key);
-  if (it == g->kv.end() || it->second.kind != Value::INT) return 0;
+  if (it == g->kv.end() || (it->second.kind != Value::INT && it->second.kind != Value::BOOL)) return 0;
   if (out) *out = it->second.i;
   return 1;
 }

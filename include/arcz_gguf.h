@@ -28,7 +28,7 @@ size_t arcz_gguf_n_tensors(const arcz_gguf* g);
 uint64_t arcz_gguf_alignment(const arcz_gguf* g); /* "general.alignment", 32 when absent (src/gguf.h:344-346) */
 
 /* Metadata (GgufFile::get_int / get_float / get_str, src/gguf.h:150-190): 1 and *out set when the key holds an integer
- * or bool (i64), any number (f64); 0 otherwise.  Strings: NULL when absent or not a string; valid until close. */
+ * or bool (i64), an integer or a float but no bool (f64); 0 otherwise.  Strings: NULL when absent or not a string; valid until close. */
 int arcz_gguf_kv_i64(const arcz_gguf* g, const char* key, int64_t* out);
 int arcz_gguf_kv_f64(const arcz_gguf* g, const char* key, double* out);
 const char* arcz_gguf_kv_str(const arcz_gguf* g, const char* key);

@@ -9,7 +9,7 @@ import gguf_writer as gw
 from common import make_weights
 
 
-def sample(tmp_path, alignment=32, version=3):
+def sample(tmp_path, alignment=32, version=3, nested=True):
     rng = np.random.default_rng(5)
     W8 = make_weights(az.Q8_0, 8, 256, seed=1)
     W4 = make_weights(az.Q4_K, 4, 512, seed=2)
@@ -21,6 +21,8 @@ def sample(tmp_path, alignment=32, version=3):
           ("a.u64", gw.T_U64, 1 << 40), ("a.i64", gw.T_I64, -(1 << 40)), ("a.f64", gw.T_F64, 2.25),
           ("tok.list", gw.T_ARR, (gw.T_STR, ["<s>", "</s>", "hello"])), ("tok.scores", gw.T_ARR, (gw.T_F32, [0.0, 1.0, 2.0])),
           ("nested", gw.T_ARR, (gw.T_ARR, [(gw.T_I32, [1, 2]), (gw.T_I32, [3])])), ("after.arrays", gw.T_I32, 77)]
+    if not nested:  # (arrays of arrays: this reader skips them, the reference's refuses the file)
+        kv = [e for e in kv if e[0] != "nested"]
     tensors = [("blk.0.ffn_up.weight", az.Q4_K, [512, 4], W4), ("output.weight", az.Q6_K, [256, 6], W6),
                ("blk.0.attn_q.weight", az.Q8_0, [256, 8], W8), ("blk.0.norm.weight", 0, [7], f32.view(np.uint8))]
     p = tmp_path / "m.gguf"

@@ -30,6 +30,8 @@ def spread(n, k):
 
 @pytest.mark.parametrize("qtype,N,K,M,T", [(az.Q4_K, 17408, 5120, 8192, 8192), (az.Q4_K, 17408, 5120, 8192, 8000),
                                            (az.Q6_K, 151936, 5120, 64, 64), (az.Q8_0, 4096, 4096, 512, 512),
+                                           # the output head as a prefill GEMM: 2048 tokens, 1.24 GB of output
+                                           (az.Q6_K, 151936, 5120, 2048, 2048),
                                            # the other weight types and launch forms at the headline matrix's size:
                                            # Q5_K and IQ4_XS, a 64- and a 128-token chunk (K shared out over several
                                            # work-groups per tile), 16 and 7 tokens (the matrix-pipe GEMV)
