@@ -147,6 +147,14 @@ int arcz_engine_matmul(arcz_engine* e, const char* name, arcz_weight* w, int Mp,
   });
 }
 
+int arcz_engine_matmul_noalloc(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off,
+                               int acc, int act32) {
+  return guarded([&] {
+    if (!w) throw std::runtime_error("matmul_noalloc: no weight");
+    e->e->matmul_noalloc(name ? name : "matmul", w->w, Mp, C, ldc, c_off, acc, act32 != 0);
+  });
+}
+
 arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, const void* up, const void* down,
                                       int NE, int NU, int E, int F) {
   arcz_moe_layer* L = new arcz_moe_layer;

@@ -14,6 +14,7 @@
 #include <string>
 #include <vector>
 
+#include "arcz_scratch.h"
 #include "kernel_table.h"
 
 struct arcz_mem {
@@ -48,6 +49,7 @@ struct Runtime {
   long fake_oom = 0, allocs = 0;
   uint64_t launches = 0;
   std::string err;
+  arcz_mem* scratch = nullptr;  // non-owning handle onto the device's static scratch array (arcz_scratch.hip)
 };
 Runtime R;
 
@@ -81,6 +83,8 @@ extern "C" {
 extern const unsigned char arcz_blob_ops[], arcz_blob_decode[], arcz_blob_decode_q80[], arcz_blob_decode_q4k[],
     arcz_blob_decode_q5k[], arcz_blob_decode_q6k[], arcz_blob_decode_iq4xs[], arcz_blob_decode_mm[], arcz_blob_gemm[], arcz_blob_moe[];
 
+static std::vector<const unsigned char*> blobs_of(const std::string& which);
+
 int arcz_init(int device) {
   if (R.up) return ARCZ_OK;
   int n = 0;
@@ -93,9 +97,45 @@ int arcz_init(int device) {
     return fail(ARCZ_E_DEVICE, "device %d is %s: the kernels are built for gfx950 only", device, R.name.c_str());
   HIP_TRY(hipStreamCreate(&R.stream));
   R.device = device;
+  // Everything a later call could otherwise make the HIP runtime allocate for is done here, so that the entry point
+  // that must not allocate (arcz_engine_matmul_noalloc) finds it in place: the address of the static scratch array on
+  // this device (asked for once, with the device current) behind a non-owning handle, and the code objects loaded.
+  void* sp = nullptr;
+  size_t sb = 0;
+  const char* serr = "";
+  if (arcz_scratch_setup(device, &sp, &sb, &serr) != 0) {
+    hipStreamDestroy(R.stream);
+    R.stream = nullptr;
+    return fail(ARCZ_E_DEVICE, "the static device scratch has no address on device %d: %s", device, serr);
+  }
+  R.scratch = new arcz_mem{(char*)sp, sb, false};
+  R.mems.insert(R.scratch);
+  for (const char* w : {"ops", "decode", "gemm", "moe"}) {
+    std::vector<hipModule_t> mods;
+    for (const unsigned char* blob : blobs_of(w)) {
+      hipModule_t mod;
+      hipError_t e = hipModuleLoadData(&mod, blob);
+      if (e != hipSuccess) {
+        for (hipModule_t m : mods) hipModuleUnload(m);
+        for (auto& kv : R.modules)
+          for (hipModule_t m : kv.second) hipModuleUnload(m);
+        R.modules.clear();
+        R.mems.erase(R.scratch);
+        delete R.scratch;
+        R.scratch = nullptr;
+        hipStreamDestroy(R.stream);
+        R.stream = nullptr;
+        return fail(ARCZ_E_BUILD, "module %s does not load: %s", w, hipGetErrorString(e));
+      }
+      mods.push_back(mod);
+    }
+    R.modules.emplace(w, mods);
+  }
   R.up = true;
   return ARCZ_OK;
 }
+
+arcz_mem* arcz_scratch_mem(void) { return R.up ? R.scratch : nullptr; }
 
 void arcz_shutdown(void) {
   if (!R.up) return;
@@ -110,6 +150,7 @@ void arcz_shutdown(void) {
     delete m;
   }
   R.mems.clear();
+  R.scratch = nullptr;  // (its handle went with the others; the array itself stays with the device)
   R.device_bytes = 0;
   hipStreamDestroy(R.stream);
   R.stream = nullptr;
@@ -158,6 +199,7 @@ arcz_mem* arcz_view(arcz_mem* parent, size_t offset, size_t bytes) {
 
 int arcz_free(arcz_mem* m) {
   if (!m) return ARCZ_OK;
+  if (m == R.scratch) return fail(ARCZ_E_ARG_VALUE, "arcz_free of the library's static scratch");
   if (!R.mems.count(m)) return fail(ARCZ_E_ARG_VALUE, "arcz_free of a handle that is not live");
   if (m->owner) {
     HIP_TRY(hipStreamSynchronize(R.stream));

@@ -11,6 +11,7 @@
 #include <string>
 #include <vector>
 
+#include "arcz_scratch.h"
 #include "clrt_hip.h"
 #include "kernels/common.h"
 
@@ -55,6 +56,11 @@ class Engine {
     // (the GEMM kernels address a chunk's int8 rows and a matrix's packed rows with 32-bit byte offsets)
     if ((uint64_t)max_chunk * (uint64_t)max_k >= (1ull << 32)) throw std::invalid_argument("Engine: a chunk of max_chunk x max_k values must stay below 4 GiB");
     alloc_activations();
+    // the short-chunk GEMM's workspace, sized once for the most its launch rule can ask for (below: pieces x tiles
+    // within two work-groups per compute unit, tiles of at most 128 x 128 f32), so that no matmul allocates or frees
+    sk_force_ = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : -1;
+    sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
+    sk_ws_ = buf(sk_ws_bytes_);
   }
   // (zero/engine_alloc.h:10, 39, 41: twice the size with two-pass matmul inputs, the residual's half behind the first)
   void alloc_activations() {
@@ -133,8 +139,9 @@ class Engine {
   // (zero/engine.h:936-950)
   void run(const char* name, cl_kernel k, int dims, const size_t* gws, const size_t* lws) {
     cl_event e = nullptr;
-    CL_CHECK(clEnqueueNDRangeKernel(cl_.queue, k, dims, nullptr, gws, lws, 0, nullptr, profile ? &e : nullptr));
-    if (profile && e) events_.push_back({name, e});
+    const bool timed = profile && !noalloc_;  // (a timed launch creates its events)
+    CL_CHECK(clEnqueueNDRangeKernel(cl_.queue, k, dims, nullptr, gws, lws, 0, nullptr, timed ? &e : nullptr));
+    if (timed && e) events_.push_back({name, e});
   }
   void collect_profile() {
     if (!profile) return;
@@ -289,6 +296,26 @@ class Engine {
     aq_ = a; asc_ = s; absum_ = b;
   }
 
+  // The same matmul for callers that must not allocate device memory (code under HIP graph capture, serving loops,
+  // harnesses that forbid it): no counterpart in the reference.  The only device memory a matmul uses beyond its inputs
+  // and outputs is the short-chunk GEMM's workspace of partial tiles; here it is the library's static scratch array
+  // (arcz_scratch.hip, ARCZ_SCRATCH_BYTES, its address taken once at arcz_init) instead of the engine's buffer, the same
+  // kernels with the same arguments otherwise, so the result is the ordinary entry point's bit for bit.  A launch that
+  // would need more than the array holds is refused.  Launches are not timed (events are allocations).  Every call on
+  // a GPU shares that GPU's array: calls that overlap on one GPU race (the library has one stream, so its own do not).
+  bool noalloc_ = false;
+  void matmul_noalloc(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
+    if (!arcz_scratch_mem()) throw std::runtime_error("matmul_noalloc: the static device scratch was not set up");
+    noalloc_ = true;
+    try {
+      matmul(name, w, Mp, C, ldc, c_off, acc, act32);
+    } catch (...) {
+      noalloc_ = false;
+      throw;
+    }
+    noalloc_ = false;
+  }
+
   // rows per half wave of the one-token GEMV (the place of the reference's gemv1_rows, zero/engine.h:1119-1123)
   static int gemv1_rows(const GpuWeight& w) {
     static const int force = getenv("ARCZ_GROWS") ? atoi(getenv("ARCZ_GROWS")) : 0;
@@ -402,9 +429,11 @@ class Engine {
 
   // The prefill GEMM (zero/engine.h:1205-1250).  Token rows come in whole tiles (the reference pads a chunk to 128
   // rows from 128 tokens on, :521-522).
-  // Workspace of the short-chunk GEMM's partial tiles, [slices][Mp][N] f32: grown on demand, kept.
+  // Workspace of the short-chunk GEMM's partial tiles, [slices][Mp][N] f32: allocated with the engine (only a forced
+  // piece count, ARCZ_Q4_SPLITK=n read when the engine is made, can outgrow it; then it is replaced by a larger one).
   cl_mem sk_ws_ = nullptr;
   size_t sk_ws_bytes_ = 0;
+  int sk_force_ = -1;  // ARCZ_Q4_SPLITK: 0 = never share K out, n >= 2: n pieces, -1 = the rule below
   void gemm_dense(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int a) {
     int M = Mp, N = w.N, K = w.K;
     // Any type, a chunk so short that its tiles are fewer than two per compute unit: K is shared out over `ny`
@@ -412,8 +441,7 @@ class Engine {
     // same bits on every run) and applies c_off and the accumulate mode.  One work-group needs 75 us for K = 5120, so
     // 64 tokens x 17408 rows took 100 us whatever the tile; now 136 tiles x 3 pieces, 42 us (128 tokens: 101 -> 71 us;
     // Q8_0 4096 x 4096: 64 tokens 41 -> 19 us, 256 tokens 44 -> 35 us).  ARCZ_Q4_SPLITK=0: off, =n: n pieces.
-    static const bool sk_off = getenv("ARCZ_Q4_SPLITK") && atoi(getenv("ARCZ_Q4_SPLITK")) == 0;
-    if (!sk_off) {
+    if (sk_force_ != 0) {
       // (tiles of 64 tokens up to 64 tokens, else of 128: the pieces of all tiles together must fit the resident slots,
       //  two work-groups per compute unit: one more piece than fits costs a whole second round)
       // (Q8_0, Q6_K: their dense kernels' 64-token tiles; IQ4_XS: the register-staged body's 128-token tiles)
@@ -422,27 +450,37 @@ class Engine {
       const int bm = tm == 64 && q45 && Mp <= 32 ? 32 : tm;  // (Q4_K / Q5_K, at most 32 rows: the one-slot-tile kernel)
       const size_t tiles64 = (size_t)((Mp + tm - 1) / tm) * ((N + 127) / 128), slots = 2 * (size_t)arcz_device_cus();
       const int nsb = K / 256;
-      static const int sk_force = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : 0;
+      const int sk_force = sk_force_;
       int ny = (int)std::min<size_t>({(size_t)8, (size_t)nsb / 2, slots / std::max<size_t>(tiles64, 1)});
       if (sk_force >= 2) ny = std::min(sk_force, nsb);
       // (from three pieces on: with two, 256 tiles of Q8_0 4096 x 4096 x 512 went from 50 to 54 us, the reduce included)
       if (ny >= 3 || (sk_force >= 2 && ny >= 2)) {
         const size_t need = (size_t)ny * Mp * N * 4;
-        if (need > sk_ws_bytes_) {
+        cl_mem ws = sk_ws_;
+        if (noalloc_) {
+          ws = arcz_scratch_mem();
+          if (need > arcz_mem_size(ws))
+            throw std::runtime_error(std::string("matmul_noalloc ") + name + ": " + std::to_string(ny) + " partial tiles of " +
+                                     std::to_string(Mp) + " x " + std::to_string(N) + " need " + std::to_string(need) +
+                                     " bytes of workspace, the static scratch holds " + std::to_string(arcz_mem_size(ws)));
+        } else if (need > sk_ws_bytes_) {
           if (sk_ws_) release(sk_ws_);
+          sk_ws_ = nullptr;
+          sk_ws_bytes_ = 0;
           sk_ws_ = buf(need);
           sk_ws_bytes_ = need;
+          ws = sk_ws_;
         }
         cl_kernel k = kernel("gemm", std::string("-DQTYPE=") + std::to_string(w.type) + " -DACT32 -DBM=" + std::to_string(bm) +
                                          " -DBN=128 -DSPLITK", "gemm");
         cl_mem unused = nullptr;
         int zero = 0, one = 1, ldw = N, s1 = nsb;
-        set_args(k, 0, w.raw, unused, aq_, asc_, absum_, sk_ws_, M, N, K, ldw, zero, zero, one, zero, s1);
+        set_args(k, 0, w.raw, unused, aq_, asc_, absum_, ws, M, N, K, ldw, zero, zero, one, zero, s1);
         size_t gws[2] = {tiles64 * 256, (size_t)ny}, lws[2] = {256, 1};
         run(name, k, 2, gws, lws);
         cl_kernel r = kernel("gemm", "", "splitk_reduce");
         int nyy = ny;
-        set_args(r, 0, sk_ws_, nyy, C, M, N, ldc, c_off, a);
+        set_args(r, 0, ws, nyy, C, M, N, ldc, c_off, a);
         size_t g1 = ((size_t)M * N + 255) / 256 * 256, l1 = 256;
         run(name, r, 1, &g1, &l1);
         return;

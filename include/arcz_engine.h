@@ -83,6 +83,19 @@ arcz_mem* arcz_engine_absum(arcz_engine* e);
 int arcz_engine_matmul(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off, int acc,
                        int act32);
 
+/* arcz_engine_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels, the same
+ * result bit for bit; the one buffer a matmul uses beyond its inputs and outputs -- the workspace of partial tiles of
+ * the short-chunk GEMM -- is the library's static device array (ARCZ_NOALLOC_SCRATCH_BYTES per GPU, held until the
+ * process ends, its address taken once in arcz_init) instead of the engine's own buffer.  The call makes no hipMalloc,
+ * hipFree or event; a launch whose partial tiles would not fit the array is refused with ARCZ_E_ENGINE and a message
+ * that names both sizes; launches are not timed by the engine's profile.  Every call on a GPU shares that GPU's array
+ * and finds the last call's contents in it (the kernels write every partial tile before reading it: nothing needs
+ * clearing): calls that overlap in time on one GPU race. */
+#define ARCZ_NOALLOC_SCRATCH_BYTES (32u << 20)
+int arcz_engine_matmul_noalloc(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off,
+                               int acc, int act32);
+
 /* Expert tensors of one MoE layer: gate, up [NE][F][E] and down [NE][E][F] as GGUF blocks of `type`. */
 arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, const void* up, const void* down,
                                       int NE, int NU, int E, int F);

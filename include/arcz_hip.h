@@ -34,7 +34,7 @@ typedef struct arcz_kernel arcz_kernel; /* the reference's cl_kernel = ZKernel (
 typedef struct arcz_event arcz_event;   /* the reference's cl_event of a launch (clrt.h:982-983) */
 
 /* Starts the runtime on GPU `device` (once per process; again = no-op): device, one stream, the embedded code
- * objects are loaded on first use.  Replaces ClRt::init (clrt.h:1064-1103).  0 or ARCZ_E_DEVICE. */
+ * objects loaded, the address of the library's static device scratch taken.  Replaces ClRt::init (clrt.h:1064-1103).  0 or ARCZ_E_DEVICE. */
 int arcz_init(int device);
 /* Frees every live buffer, module and the stream (the reference's ClRt destructor path). */
 void arcz_shutdown(void);
