@@ -29,10 +29,12 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def time_steps(az, fn, steps, warmup):
+def time_steps(az, fn, steps, warmup, after_warmup=None):
     for _ in range(warmup):
         fn()
     az.Runtime.sync()
+    if after_warmup is not None:
+        after_warmup()
     e0 = az.Runtime.event()
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -60,7 +62,11 @@ def bench_prefill(az, steps, warmup, M, N, K, qtype):
         eng.quantize(xb, K, K, M, M)
         eng.matmul("gemm", w, M, cb, N, 0, 0)
 
-    ms_dev, ms_wall = time_steps(az, step, steps, warmup)
+    def forget_warmup():   # the per-kernel statistics cover the timed launches only
+        eng.profile_collect()
+        eng.profile_reset()
+
+    ms_dev, ms_wall = time_steps(az, step, steps, warmup, forget_warmup)
     eng.profile_collect()
     gemm_ms, gemm_n = eng.profile_get("gemm")
     quant_ms, quant_n = eng.profile_get("quant_rows")
@@ -234,22 +240,27 @@ def bench_moe_decode(az, launches):
     return out
 
 
-def bench_producers(az, M, K):
+def bench_producers(az, M, K, copies=4):
     """The fused producers at the headline chunk's shape: RMS norm + quantization of M rows of K, SwiGLU + quantization
-    of M rows of [gate(K) | up(K)]; HBM bytes = f32 rows read once + int8 rows, scales and sums written."""
+    of M rows of [gate(K) | up(K)]; HBM bytes = f32 rows read once + int8 rows, scales and sums written.  The launches
+    go round `copies` distinct inputs (4 x 168 MB, 4 x 336 MB for SwiGLU: more than the 256 MB last-level cache holds),
+    so the rates are HBM rates."""
     eng = az.Engine(M, K)
-    xb = az.Runtime.from_numpy(az.gen_normal(51, (M, K)))
+    xs = [az.Runtime.from_numpy(az.gen_normal(51 + i, (M, K))) for i in range(copies)]
     wb = az.Runtime.from_numpy(np.ones(K, np.float32))
-    gb = az.Runtime.from_numpy(az.gen_normal(52, (M, 2 * K)))
+    g0 = az.gen_normal(52, (M, 2 * K))
+    gs = [az.Runtime.from_numpy(g0) for _ in range(copies)]
+    del g0
     out = {}
-    for name, fn, rd in (("rmsnorm_quant", lambda: eng.rmsnorm_quant(xb, 0, wb, K, M, M, 1e-6), 4.0 * M * K),
-                         ("swiglu_quant", lambda: eng.swiglu_quant(gb, K, M, M), 8.0 * M * K),
-                         ("quant_rows", lambda: eng.quantize(xb, K, K, M, M), 4.0 * M * K)):
-        fn()
+    for name, fn, rd in (("rmsnorm_quant", lambda i: eng.rmsnorm_quant(xs[i], 0, wb, K, M, M, 1e-6), 4.0 * M * K),
+                         ("swiglu_quant", lambda i: eng.swiglu_quant(gs[i], K, M, M), 8.0 * M * K),
+                         ("quant_rows", lambda i: eng.quantize(xs[i], K, K, M, M), 4.0 * M * K)):
+        for i in range(copies):
+            fn(i)
         az.Runtime.sync()
         e0 = az.Runtime.event()
-        for _ in range(20):
-            fn()
+        for it in range(20):
+            fn(it % copies)
         e1 = az.Runtime.event()
         az.Runtime.sync()
         us = az.Runtime.elapsed_ms(e0, e1) / 20 * 1e3
@@ -257,8 +268,9 @@ def bench_producers(az, M, K):
         az.Runtime.event_release(e1)
         nbytes = rd + M * K * (1 + 4 / 32 + 2 / 16)
         out[name] = {"us": us, "GBps": nbytes / us / 1e3, "frac_hbm_peak": nbytes / us / 1e3 / PEAK_HBM_GBS}
-    out["note"] = "back-to-back launches on inputs that fit the 256 MB last-level cache: the rates are not HBM rates"
-    for b in (xb, wb, gb):
+    out["shape"] = [M, K]
+    out["note"] = f"back-to-back launches cycling through {copies} distinct inputs (more than the last-level cache holds)"
+    for b in xs + gs + [wb]:
         b.free()
     eng.close()
     return out
@@ -360,6 +372,8 @@ def main():
                    "M": M, "N": N, "K": K, "step": "quant_rows + gemm"},
         "roofline": {"bound": "mfma", "achieved": pre["kernel_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": pre["kernel_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH,
+                     "traffic_source": "profiles/bench_hbm_traffic_fetch_write.txt (counter runs of this script; "
+                                       "a constant here, not read in this run)",
                      "kernel": "gemm__QTYPE12_ACT321",
                      "kernel_ms": pre["gemm_kernel_ms"], "kernel_ms_median": pre["gemm_kernel_ms_median"],
                      "kernel_ms_min": pre["gemm_kernel_ms_min"], "ops_per_launch": pre["ops"]},
@@ -378,10 +392,10 @@ def main():
         log(f"[bench] Q8_0 4096x4096 M=512: {c1}")
         out["other_configs"] = {"Q8_0_4096x4096_M512": c1}
         W6 = None
-        for M, launches in ((1, 50), (64, 20), (2048, 3)):
-            r, W6 = bench_gemm_config(az, az.Q6_K, 151936, 5120, M, launches, 41, W6)
-            log(f"[bench] Q6_K 151936x5120 M={M}: {r}")
-            out["other_configs"][f"Q6_K_151936x5120_M{M}"] = r
+        for M6, launches in ((1, 50), (64, 20), (2048, 3)):
+            r, W6 = bench_gemm_config(az, az.Q6_K, 151936, 5120, M6, launches, 41, W6)
+            log(f"[bench] Q6_K 151936x5120 M={M6}: {r}")
+            out["other_configs"][f"Q6_K_151936x5120_M{M6}"] = r
         del W6
         # Q5_K (one of the further weight types): the same matrix as the headline, one token and 8192
         out["other_configs"]["Q5_K_17408x5120_T1"] = bench_decode(az, az.Q5_K, 17408, 5120, 1, 200, 8)
