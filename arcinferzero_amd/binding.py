@@ -93,6 +93,7 @@ _sig("arcz_engine_residual", _p, _p, _i)
 _sig("arcz_engine_asc", _p, _p)
 _sig("arcz_engine_absum", _p, _p)
 _sig("arcz_engine_matmul", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
+_sig("arcz_engine_gemv_gu", _i, _p, _p, _p, _i, _p)
 _sig("arcz_engine_matmul_noalloc", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
 _sig("arcz_moe_layer_upload", _p, _p, _u32, _p, _p, _p, _i, _i, _i, _i)
 _sig("arcz_engine_layer_moe", _i, _p, _p, _p, _i, _p, _i, _i)
@@ -461,6 +462,13 @@ class Engine:
 
     def matmul(self, name, w, Mp, Cbuf, ldc, c_off=0, acc=0, act32=True):
         _check(lib.arcz_engine_matmul(self.h, name.encode(), w.h, Mp, Cbuf.h, ldc, c_off, acc, 1 if act32 else 0), engine=True)
+
+    def gemv_gu(self, g, u, Mp, Cbuf):
+        """Gate and up of one token in one launch: True if taken, False if the caller must run the two matmuls."""
+        r = lib.arcz_engine_gemv_gu(self.h, g.h, u.h, Mp, Cbuf.h)
+        if r < 0:
+            _check(r, engine=True)
+        return r == 1
 
     def matmul_noalloc(self, name, w, Mp, Cbuf, ldc, c_off=0, acc=0, act32=True):
         """The same matmul on the library's static device scratch: no device allocation, event or free in the call."""

@@ -147,6 +147,15 @@ int arcz_engine_matmul(arcz_engine* e, const char* name, arcz_weight* w, int Mp,
   });
 }
 
+int arcz_engine_gemv_gu(arcz_engine* e, arcz_weight* g, arcz_weight* u, int Mp, arcz_mem* C) {
+  int taken = 0;
+  const int r = guarded([&] {
+    if (!g || !u) throw std::runtime_error("gemv_gu: no weight");
+    taken = e->e->gemv_gu(g->w, u->w, Mp, C) ? 1 : 0;
+  });
+  return r != ARCZ_OK ? r : taken;
+}
+
 int arcz_engine_matmul_noalloc(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off,
                                int acc, int act32) {
   return guarded([&] {

@@ -427,6 +427,43 @@ class Engine {
     gemm_dense(name, w, Mp, C, ldc, c_off, a);
   }
 
+  // One token: the FFN's gate and up GEMVs in one launch (zero/engine.h:1124-1146, the kernel's -DGU2 form): rows
+  // [0, F) of gate at C and [0, F) of up at C + F, every row by the lanes and arithmetic of its own launch, bit for bit.
+  // On this machine a launch of 50 MB spends about 4 of its 10 us filling and draining the chip; one launch of twice
+  // the bytes pays that once.  false: not taken (the caller runs the two launches): more than one token, two-pass
+  // inputs, matrices that differ in type or shape, rows too long for the LDS-staged kernel, or F not a multiple of the
+  // rows of a pass.  ARCZ_GEMV_GU=0: never taken.
+  bool gemv_gu(const GpuWeight& g, const GpuWeight& u, int Mp, cl_mem C) {
+    static const bool off = getenv("ARCZ_GEMV_GU") && atoi(getenv("ARCZ_GEMV_GU")) == 0;
+    if (off || cur_T_ != 1 || q2mm_ || !g.raw || !u.raw || g.type != u.type || g.N != u.N || g.K != u.K) return false;
+    if (g.K != cur_K_ || Mp != cur_Mp_)
+      throw std::runtime_error("gemv_gu: the activations hold " + std::to_string(cur_Mp_) + " x " + std::to_string(cur_K_) +
+                               ", the matrices take " + std::to_string(Mp) + " x " + std::to_string(g.K));
+    const int N = g.N, K = g.K;
+    const int ups = g.type == GGML_Q8_0 ? 16 : 8, units = K / 256 * ups;
+    const int tok_bytes = (g.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (g.type == GGML_Q4_K || g.type == GGML_Q5_K ? 8 : 4));
+    int lpr = 0;
+    for (int l : {32, 64, 128, 256})
+      if (!lpr && (units + l - 1) / l <= 6) lpr = l;
+    if (!lpr) return false;
+    const int gr = 256 / lpr, wpr = lpr > 64 ? lpr / 64 : 1;
+    const size_t lds = (size_t)tok_bytes + (wpr > 1 ? (size_t)16 * gr * wpr * 4 : 0);
+    if (lds > 65536 || N % gr) return false;
+    if (arcz_mem_size(C) < (size_t)2 * N * 4) throw std::runtime_error("gemv_gu: the output does not fit C");
+    rd_bytes += raw_bytes(g) + raw_bytes(u);
+    const int pf = (units + lpr - 1) / lpr;
+    const std::string defs = "-DQT=" + std::to_string(g.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" + std::to_string(pf) +
+                             " -DLDS=" + std::to_string(lds) + " -DGU2";
+    cl_kernel k = kernel("decode", defs, "gemv");
+    cl_mem tabs = nullptr;
+    int NN = N, KK = K, M = Mp, c_off = 0, a = 0;
+    set_args(k, 0, g.raw, NN, KK, tabs, aq_, asc_, absum_, M, C, c_off, a, u.raw);
+    const size_t wgs = std::min<size_t>((size_t)2 * N / gr, (size_t)arcz_device_cus() * 2);
+    size_t g1 = wgs * 256, l1 = 256;
+    run("gemm_gate_up", k, 1, &g1, &l1);
+    return true;
+  }
+
   // The prefill GEMM (zero/engine.h:1205-1250).  Token rows come in whole tiles (the reference pads a chunk to 128
   // rows from 128 tokens on, :521-522).
   // Workspace of the short-chunk GEMM's partial tiles, [slices][Mp][N] f32: allocated with the engine (only a forced

@@ -30,6 +30,7 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "mfma_probe", nullptr, "pi", {nullptr}, {{nullptr, 0, false}}, 256},
     // ---- decode
+    {"decode", "gemv", "GU2", "piippppipiip", {"QT", "LPR", "PF", "GU2", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "LPR", "PF", "TB", nullptr},
      {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {nullptr, 0, false}}, 256},

@@ -139,6 +139,36 @@ def bench_decode(az, qtype, N, K, T, launches, copies):
             "distinct_weight_MB": copies * az.gguf_bytes(qtype, N, K) / 1e6}
 
 
+def bench_gemv_gu(az, qtype, F, K, launches, copies):
+    """Gate and up of one token in one launch (Engine::gemv_gu), over `copies` distinct pairs of matrices in turn."""
+    eng = az.Engine(16, K)
+    Wg, Wu = az.gen_weights(qtype, 5, F, K, 0.02), az.gen_weights(qtype, 6, F, K, 0.02)
+    ws = [(eng.make_weight(qtype, F, K, Wg), eng.make_weight(qtype, F, K, Wu)) for _ in range(copies)]
+    xb = az.Runtime.from_numpy(az.gen_normal(4, (1, K)))
+    eng.quantize(xb, K, K, 16, 1)
+    cb = az.Runtime.alloc(2 * F * 4)
+    for g, u in ws:
+        assert eng.gemv_gu(g, u, 16, cb)
+    az.Runtime.sync()
+    e0 = az.Runtime.event()
+    for i in range(launches):
+        eng.gemv_gu(ws[i % copies][0], ws[i % copies][1], 16, cb)
+    e1 = az.Runtime.event()
+    az.Runtime.sync()
+    us = az.Runtime.elapsed_ms(e0, e1) / launches * 1e3
+    az.Runtime.event_release(e0)
+    az.Runtime.event_release(e1)
+    nbytes = 2 * az.gguf_bytes(qtype, F, K) + (K + K // 32 * 4 + K // 16 * 2) + 2 * F * 4
+    for g, u in ws:
+        g.free()
+        u.free()
+    cb.free()
+    xb.free()
+    eng.close()
+    return {"kernel_us": us, "bytes": nbytes, "GBps": nbytes / us / 1e3, "frac_hbm_peak": nbytes / us / 1e3 / PEAK_HBM_GBS,
+            "launches": launches, "distinct_weight_MB": 2 * copies * az.gguf_bytes(qtype, F, K) / 1e6}
+
+
 def bench_gemm_config(az, qtype, N, K, M, launches, seed, W=None):
     """One GEMM (or GEMV-form, M <= 8) configuration: per-launch device time from events around `launches` launches."""
     eng = az.Engine(max(M, 16), K)
@@ -385,7 +415,10 @@ def main():
         log(f"[bench] decode T=1: {d1}")
         d2 = bench_decode(az, az.Q4_K, 5120, 17408, 2, 200, 8)
         log(f"[bench] decode T=2: {d2}")
-        out["decode"] = {"Q4_K_17408x5120_T1": d1, "Q4_K_5120x17408_T2": d2, "hbm_peak_GBps": PEAK_HBM_GBS}
+        dgu = bench_gemv_gu(az, az.Q4_K, 17408, 5120, 200, 4)
+        log(f"[bench] decode gate + up in one launch: {dgu}")
+        out["decode"] = {"Q4_K_17408x5120_T1": d1, "Q4_K_5120x17408_T2": d2, "Q4_K_gate_up_2x17408x5120_T1": dgu,
+                         "hbm_peak_GBps": PEAK_HBM_GBS}
     if not args.no_extras:
         az.self_check()
         c1, _ = bench_gemm_config(az, az.Q8_0, 4096, 4096, 512, 50, 31)

@@ -83,6 +83,13 @@ arcz_mem* arcz_engine_absum(arcz_engine* e);
 int arcz_engine_matmul(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off, int acc,
                        int act32);
 
+/* Engine::gemv_gu(g, u, Mp, C) (zero/engine.h:1124-1146): one token, the FFN's gate and up matrices (same type, N = F
+ * rows, K) in one launch -- rows [0, F) of gate at C[0, F), rows [0, F) of up at C[F, 2 F), each bit for bit what its
+ * own arcz_engine_matmul gives.  1 = done; 0 = not taken, nothing was launched and the caller runs the two matmuls
+ * (more than one token in the chunk, two-pass inputs, matrices of different type or shape, rows the LDS-staged GEMV
+ * does not take); negative: an error. */
+int arcz_engine_gemv_gu(arcz_engine* e, arcz_weight* g, arcz_weight* u, int Mp, arcz_mem* C);
+
 /* arcz_engine_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels, the same
  * result bit for bit; the one buffer a matmul uses beyond its inputs and outputs -- the workspace of partial tiles of

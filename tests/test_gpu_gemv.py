@@ -105,3 +105,41 @@ def test_gemv_accumulate_and_offset(eng):
     y = run_gemv(eng, az.Q4_K, W, N, K, x, Mp, acc=1, c_init=c0, ldc=ldc, c_off=c_off)
     assert np.array_equal(y[:, :c_off], c0[:, :c_off]) and np.array_equal(y[:, c_off + N:], c0[:, c_off + N:])
     assert np.array_equal(y[:, c_off:c_off + N], c0[:, c_off:c_off + N] + y0)
+
+
+@pytest.mark.parametrize("qtype,F,K", [(az.Q4_K, 17408, 5120), (az.Q4_K, 264, 512), (az.Q6_K, 1024, 2048), (az.Q8_0, 512, 1024),
+                                       (az.Q5_K, 776, 2560), (az.IQ4_XS, 128, 17408)])
+def test_gemv_gu_equals_two_launches(eng, qtype, F, K):
+    """Gate and up of one token in one launch (zero/engine.h:1124-1146): rows [0, F) of gate, then of up at C + F, bit
+    for bit what the two launches give; and the cases that are not taken."""
+    print(f"gemv_gu {TYPE_NAMES[qtype]} F={F} K={K}", flush=True)
+    Wg, Wu = make_weights(qtype, F, K, seed=61), make_weights(qtype, F, K, seed=62)
+    g, u = eng.make_weight(qtype, F, K, Wg), eng.make_weight(qtype, F, K, Wu)
+    x = make_acts(1, K, seed=63, outliers=True)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, 16, 1)
+    c2 = az.Runtime.alloc(2 * F * 4).fill(0xFFFFFFFF)
+    eng.matmul("gate", g, 16, c2, 2 * F, 0, 0)
+    eng.matmul("up", u, 16, c2, 2 * F, F, 0)
+    want = c2.read(np.uint32, 2 * F)
+    c1 = az.Runtime.alloc(2 * F * 4).fill(0xFFFFFFFF)
+    assert eng.gemv_gu(g, u, 16, c1)
+    got = c1.read(np.uint32, 2 * F)
+    assert np.array_equal(got, want) and np.isfinite(got.view(np.float32)).all()
+    aq, asc, _ = quantize_padded(x, 16)
+    rows = np.arange(0, F, max(1, F // 256))
+    rb = az.gguf_bytes(qtype, 1, K)
+    for W, y in ((Wg, got[:F]), (Wu, got[F:])):
+        ref = orc.matmul_ref(qtype, np.concatenate([W[r * rb:(r + 1) * rb] for r in rows]), len(rows), K, aq[:1], asc)
+        assert rel_err_rows(y.view(np.float32)[rows][None], ref).max() <= TOL
+    # not taken: two tokens in the chunk; matrices of different shapes
+    eng.quantize(az.Runtime.from_numpy(make_acts(2, K, seed=64)), K, K, 16, 2)
+    assert not eng.gemv_gu(g, u, 16, c1)
+    eng.quantize(xb, K, K, 16, 1)
+    if F > 8:
+        w3 = eng.make_weight(qtype, F - 8, K, make_weights(qtype, F - 8, K, seed=65))
+        assert not eng.gemv_gu(g, w3, 16, c1)
+        w3.free()
+    for b in (c1, c2, xb):
+        b.free()
+    g.free(); u.free()
