@@ -93,11 +93,16 @@ _sig("arcz_engine_residual", _p, _p, _i)
 _sig("arcz_engine_asc", _p, _p)
 _sig("arcz_engine_absum", _p, _p)
 _sig("arcz_engine_matmul", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
+_sig("arcz_weight_set_softcap", _i, _p, C.c_float)
 _sig("arcz_engine_gemv_gu", _i, _p, _p, _p, _i, _p)
 _sig("arcz_engine_matmul_noalloc", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
 _sig("arcz_moe_layer_upload", _p, _p, _u32, _p, _p, _p, _i, _i, _i, _i)
 _sig("arcz_engine_layer_moe", _i, _p, _p, _p, _i, _p, _i, _i)
 _sig("arcz_engine_moe_route", _i, _p, _p, _p, _i, _i, _i)
+_sig("arcz_engine_layer_moe_sh", _i, _p, _p, _p, _i, _p, _i, _i, _p)
+_sig("arcz_moe_layer_set_routing", _i, _p, _p, _p, _p, C.c_float)
+_sig("arcz_moe_layer_free", _i, _p, _p)
+_sig("arcz_engine_moe_sgate", _p, _p)
 _sig("arcz_engine_moe_buffer", _p, _p, _i)
 _sig("arcz_engine_moe_slots", _i, _p)
 _sig("arcz_engine_self_check", _i)
@@ -361,6 +366,10 @@ class Runtime:
 
 # ---------------------------------------------------------------- engine (include/arcz_engine.h)
 class Weight:
+    def set_softcap(self, cap):
+        """This matrix is an output head with final-logit soft-capping c: GEMVs over 1-8 tokens write c * tanh(v / c)."""
+        _check(lib.arcz_weight_set_softcap(self.h, float(cap)), engine=True)
+
     def __init__(self, eng, h, qtype, N, K):
         self.eng, self.h, self.type, self.N, self.K = eng, h, qtype, N, K
 
@@ -483,8 +492,21 @@ class Engine:
             raise ArczError(-100, lib.arcz_engine_error().decode())
         return MoeLayer(self, h, NE, NU, E, F)
 
-    def layer_moe(self, L, logits, ldl, x, T, Mp):
-        _check(lib.arcz_engine_layer_moe(self.h, L.h, logits.h, ldl, x.h, T, Mp), engine=True)
+    def layer_moe(self, L, logits, ldl, x, T, Mp, sh=None):
+        if sh is None:
+            _check(lib.arcz_engine_layer_moe(self.h, L.h, logits.h, ldl, x.h, T, Mp), engine=True)
+        else:
+            _check(lib.arcz_engine_layer_moe_sh(self.h, L.h, logits.h, ldl, x.h, T, Mp, sh.h), engine=True)
+
+    def set_moe_routing(self, L, escale=None, ebias=None, rscale=1.0):
+        es = None if escale is None else np.ascontiguousarray(escale, dtype=np.float32)
+        eb = None if ebias is None else np.ascontiguousarray(ebias, dtype=np.float32)
+        _check(lib.arcz_moe_layer_set_routing(self.h, L.h, _np_ptr(es) if es is not None else None,
+                                              _np_ptr(eb) if eb is not None else None, float(rscale)), engine=True)
+
+    @property
+    def moe_sgate(self):
+        return Buffer(lib.arcz_engine_moe_sgate(self.h), owner=False)
 
     def moe_route(self, L, logits, ldl, T, tm):
         _check(lib.arcz_engine_moe_route(self.h, L.h, logits.h, ldl, T, tm), engine=True)

@@ -106,6 +106,11 @@ int arcz_weight_free(arcz_engine* e, arcz_weight* w) {
   return r;
 }
 arcz_mem* arcz_weight_raw(const arcz_weight* w) { return w ? w->w.raw : nullptr; }
+int arcz_weight_set_softcap(arcz_weight* w, float cap) {
+  if (!w || !(cap >= 0.0f)) return ARCZ_E_ENGINE;
+  w->w.softcap = cap;
+  return ARCZ_OK;
+}
 
 int arcz_engine_quantize(arcz_engine* e, arcz_mem* x, int ldx, int K, int Mp, int T, int act32) {
   return guarded([&] { e->e->quantize_rows(x, ldx, K, Mp, T, act32); });
@@ -178,6 +183,23 @@ arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void*
 int arcz_engine_layer_moe(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp) {
   return guarded([&] { e->e->layer_moe(L->L, logits, ldl, x, T, Mp); });
 }
+int arcz_engine_layer_moe_sh(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp,
+                             arcz_mem* sh) {
+  return guarded([&] { e->e->layer_moe(L->L, logits, ldl, x, T, Mp, sh); });
+}
+int arcz_moe_layer_set_routing(arcz_engine* e, arcz_moe_layer* L, const float* escale, const float* ebias, float rscale) {
+  return guarded([&] { e->e->set_moe_routing(L->L, escale, ebias, rscale); });
+}
+int arcz_moe_layer_free(arcz_engine* e, arcz_moe_layer* L) {
+  if (!L) return ARCZ_OK;
+  const int r = guarded([&] {
+    for (int i = 0; i < 3; ++i) e->e->free_weight(L->L.ex[i]);
+    e->e->set_moe_routing(L->L, nullptr, nullptr, 1.0f);
+  });
+  delete L;
+  return r;
+}
+arcz_mem* arcz_engine_moe_sgate(arcz_engine* e) { return e->e->sgate_; }
 int arcz_engine_moe_route(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, int T, int tm) {
   return guarded([&] { e->e->moe_route(L->L, logits, ldl, T, tm); });
 }

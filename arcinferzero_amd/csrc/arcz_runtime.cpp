@@ -236,6 +236,25 @@ int arcz_d2d(arcz_mem* dst, size_t dst_offset, const arcz_mem* src, size_t src_o
   return ARCZ_OK;
 }
 
+// zrt::host_alloc / mem_free of a host pointer (clrt.h:445-452, 160): pinned host memory the device can copy to and from at
+// full rate; allocated, never registered over existing memory.
+void* arcz_host_alloc(size_t bytes) {
+  if (!R.up) { fail(ARCZ_E_DEVICE, "arcz_host_alloc before arcz_init"); return nullptr; }
+  void* p = nullptr;
+  const hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault);
+  if (e != hipSuccess || !p) {
+    (void)hipGetLastError();
+    fail(ARCZ_E_OOM, "pinned host allocation of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+    return nullptr;
+  }
+  return p;
+}
+int arcz_host_free(void* p) {
+  if (!p) return ARCZ_OK;
+  HIP_TRY(hipHostFree(p));
+  return ARCZ_OK;
+}
+
 static arcz_kernel* fill_kernel();
 
 int arcz_fill(arcz_mem* dst, const void* pattern, size_t ps, size_t offset, size_t bytes) {
@@ -276,7 +295,7 @@ static std::vector<const unsigned char*> blobs_of(const std::string& which) {
 
 // "-DQT=12 -DGROWS=2 -cl-whatever" -> {QT: 12, GROWS: 2}; a -D without a value is 1
 static std::map<std::string, long> parse_defs(const char* defs) {
-  std::map<std::string, long> out;
+  std::map<std::string, long> out;  // (SOFTCAP, RSCALE: the bit pattern of the float value)
   const std::string s = defs ? defs : "";
   size_t i = 0;
   while (i < s.size()) {
@@ -287,7 +306,14 @@ static std::map<std::string, long> parse_defs(const char* defs) {
     if (tok.size() > 2 && tok[0] == '-' && tok[1] == 'D') {
       const size_t eq = tok.find('=');
       const std::string name = tok.substr(2, eq == std::string::npos ? std::string::npos : eq - 2);
-      out[name] = eq == std::string::npos ? 1 : strtol(tok.c_str() + eq + 1, nullptr, 0);
+      if ((name == "SOFTCAP" || name == "RSCALE") && eq != std::string::npos) {
+        const float f = strtof(tok.c_str() + eq + 1, nullptr);
+        uint32_t bits;
+        memcpy(&bits, &f, 4);
+        out[name] = (long)bits;
+      } else {
+        out[name] = eq == std::string::npos ? 1 : strtol(tok.c_str() + eq + 1, nullptr, 0);
+      }
     }
     i = j;
   }

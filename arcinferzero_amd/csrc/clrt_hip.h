@@ -43,6 +43,17 @@ typedef ArczKernelArgs* cl_kernel;
 #define CL_MEM_READ_ONLY (1 << 2)
 #define CL_MEM_COPY_HOST_PTR (1 << 5)
 #define CL_BUFFER_CREATE_TYPE_REGION 0x1220
+#define CL_MAP_READ (1 << 0)
+#define CL_MAP_WRITE (1 << 1)
+#define CL_MAP_WRITE_INVALIDATE_REGION (1 << 2)
+
+// cl_program: what ClRt::build returns.  The reference compiles OpenCL C with an option string at run time
+// (zero/clrt.h:1189-1281); here the kernels are compiled ahead of time, so a "program" is the module's name and the
+// option string, and ClRt::kernel looks the variant up.
+struct ArczProgram {
+  std::string which, opts;
+};
+typedef ArczProgram* cl_program;
 
 // Any failure ends the process with a message, unless the owner asked for exceptions (the reference's CL_CHECK,
 // zero/clrt.h:85-93, and soft_fail, :1050).
@@ -96,6 +107,51 @@ inline cl_int clEnqueueFillBuffer(cl_command_queue, cl_mem b, const void* patter
   if (ev) *ev = nullptr;
   return arcz_fill(b, pattern, ps, off, n);
 }
+// clEnqueueMapBuffer / clEnqueueUnmapMemObject (zero/clrt.h:711-743): a pinned host copy of [off, off + n) of b -- read
+// from the device when mapped for reading, written back when a map for writing is released.
+namespace arcz {
+struct Map { cl_mem m; size_t off, n; void* host; cl_map_flags flags; };
+inline std::vector<Map>& maps() { static std::vector<Map> v; return v; }
+}  // namespace arcz
+inline void* clEnqueueMapBuffer(cl_command_queue, cl_mem b, cl_bool, cl_map_flags flags, size_t off, size_t n, cl_uint,
+                                const cl_event*, cl_event* ev, cl_int* err) {
+  if (ev) *ev = nullptr;
+  if (!b || off > arcz_mem_size(b) || n > arcz_mem_size(b) - off) {  // (refused as the transfers refuse it)
+    if (err) *err = ARCZ_E_BOUNDS;
+    return nullptr;
+  }
+  void* h = arcz_host_alloc(n);
+  if (!h) {
+    if (err) *err = ARCZ_E_OOM;
+    return nullptr;
+  }
+  if (flags & CL_MAP_READ) {
+    const cl_int e = arcz_d2h(h, b, off, n);
+    if (e != CL_SUCCESS) {
+      arcz_host_free(h);
+      if (err) *err = e;
+      return nullptr;
+    }
+  }
+  arcz::maps().push_back({b, off, n, h, flags});
+  if (err) *err = CL_SUCCESS;
+  return h;
+}
+inline cl_int clEnqueueUnmapMemObject(cl_command_queue, cl_mem b, void* p, cl_uint, const cl_event*, cl_event* ev) {
+  if (ev) *ev = nullptr;
+  auto& mp = arcz::maps();
+  for (size_t i = 0; i < mp.size(); ++i)
+    if (mp[i].host == p && mp[i].m == b) {
+      cl_int e = CL_SUCCESS;
+      if (mp[i].flags & (CL_MAP_WRITE | CL_MAP_WRITE_INVALIDATE_REGION)) e = arcz_h2d(b, mp[i].off, p, mp[i].n);
+      arcz_host_free(p);
+      mp.erase(mp.begin() + (long)i);
+      return e;
+    }
+  return ARCZ_E_BOUNDS;  // (not a live map of b)
+}
+inline cl_int clReleaseProgram(cl_program p) { delete p; return CL_SUCCESS; }
+
 inline cl_int clSetKernelArg(cl_kernel k, cl_uint i, size_t sz, const void* v) {
   if (!k || sz > 8 || !v) return ARCZ_E_ARG_SIZE;
   if (k->args.size() <= i) k->args.resize(i + 1);
@@ -136,6 +192,11 @@ struct ClRt {
     device_id = arcz_device_name();
     return true;
   }
+  // build(src, opts) + kernel(prog, name) (zero/clrt.h:1189, 1282).  `src` is the module's name ("ops", "decode",
+  // "gemm", "moe") where the reference passes the text of its .cl file; options that are not -D are ignored.  An
+  // unknown module is reported by kernel(), as a failed build is in the reference.
+  cl_program build(const std::string& src, const std::string& opts) { return new ArczProgram{src, opts}; }
+  cl_kernel kernel(cl_program prog, const char* name) { return kernel(prog->which, prog->opts, name); }
   cl_kernel kernel(const std::string& which, const std::string& defs, const std::string& name) {
     arcz_kernel* h = arcz_kernel_get(which.c_str(), defs.c_str(), name.c_str());
     if (!h) {

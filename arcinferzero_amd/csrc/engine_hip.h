@@ -32,6 +32,9 @@ struct GpuWeight {
   int N = 0, K = 0;
   cl_mem raw = nullptr;
   size_t rows = 0;
+  // > 0: this matrix is the output head of a model with final-logit soft-capping (the reference's lm_head_ with
+  // hp.softcap, zero/engine.h:984-990): the GEMVs (1-8 tokens) write c * tanh(v / c)
+  float softcap = 0.0f;
 };
 
 inline const char* ggml_type_name(uint32_t t) {
@@ -108,6 +111,7 @@ class Engine {
   }
   ~Engine() {
     for (auto& kv : kernels_) clReleaseKernel(kv.second);
+    for (cl_program p : progs_) clReleaseProgram(p);
     for (auto it = mems_.rbegin(); it != mems_.rend(); ++it) clReleaseMemObject(*it);  // views before parents
   }
   Engine(const Engine&) = delete;
@@ -132,7 +136,9 @@ class Engine {
     const std::string key = which + defs + "|" + name;
     auto it = kernels_.find(key);
     if (it != kernels_.end()) return it->second;
-    cl_kernel k = cl_.kernel(which, defs, name);
+    cl_program p = cl_.build(which, defs);  // (the module's name stands where the reference passes its source text)
+    progs_.push_back(p);
+    cl_kernel k = cl_.kernel(p, name.c_str());
     kernels_[key] = k;
     return k;
   }
@@ -272,28 +278,54 @@ class Engine {
   // (as 2 T token slots, over one read of the weights: the reference's q2_fuse_, zero/engine.h:1086-1088) whenever the
   // LDS-staged kernel can hold them, and says so in q2_fused_.  q2_nofuse_ (or ARCZ_Q2_FUSE=0): always two launches.
   bool q2_fuse_ = false, q2_fused_ = false, q2_nofuse_ = false;
+  bool q2_nocap_ = false;  // (a two-pass output head: both passes run without the cap, softcap_rows caps their sum)
+  // (zero/engine.h:984-990 head_defs) the GEMVs' -DSOFTCAP for an output head with a cap
+  std::string head_defs(const GpuWeight& w) const {
+    if (w.softcap <= 0.0f || q2_nocap_) return "";
+    char b[48];
+    snprintf(b, sizeof b, " -DSOFTCAP=%.9ef", w.softcap);
+    return b;
+  }
   void matmul(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
     static const bool fuse_off = getenv("ARCZ_Q2_FUSE") && atoi(getenv("ARCZ_Q2_FUSE")) == 0;
     if (q2mm_ && acc > 1) throw std::logic_error(std::string("two-pass activations with a fused epilogue: ") + name);
+    // (the output head with a logit soft cap and two-pass inputs: the cap applies to the sum of both passes, so both
+    //  run without it and softcap_rows caps the sum; zero/engine.h:1081-1110)
+    const bool cap = q2mm_ && w.softcap > 0.0f;
+    if (cap && cur_T_ > 8) throw std::logic_error("two-pass output head over more than 8 rows (no softcap there)");
+    q2_nocap_ = cap;
     q2_fuse_ = q2mm_ && !fuse_off && !q2_nofuse_ && cur_T_ <= 4;
     q2_fused_ = false;
     try {
       matmul1(name, w, Mp, C, ldc, c_off, acc, act32);
     } catch (...) {
       q2_fuse_ = false;
+      q2_nocap_ = false;
       throw;
     }
     q2_fuse_ = false;
-    if (!q2mm_ || q2_fused_) return;
-    const cl_mem a = aq_, s = asc_, b = absum_;
-    aq_ = aq2_; asc_ = asc2_; absum_ = absum2_;
-    try {
-      matmul1(name, w, Mp, C, ldc, c_off, 1, act32);
-    } catch (...) {
+    if (!q2mm_) return;
+    if (!q2_fused_) {
+      const cl_mem a = aq_, s = asc_, b = absum_;
+      aq_ = aq2_; asc_ = asc2_; absum_ = absum2_;
+      try {
+        matmul1(name, w, Mp, C, ldc, c_off, 1, act32);
+      } catch (...) {
+        aq_ = a; asc_ = s; absum_ = b;
+        q2_nocap_ = false;
+        throw;
+      }
       aq_ = a; asc_ = s; absum_ = b;
-      throw;
     }
-    aq_ = a; asc_ = s; absum_ = b;
+    q2_nocap_ = false;
+    if (cap) {
+      cl_kernel k = kernel("ops", "", "softcap_rows");
+      int ld = cur_T_ == 1 ? 0 : ldc, off = c_off, N = w.N;
+      float cp = w.softcap;
+      set_args(k, 0, C, ld, off, N, cp);
+      size_t gws[2] = {((size_t)N + 255) / 256 * 256, (size_t)cur_T_}, lws[2] = {256, 1};
+      run(name, k, 2, gws, lws);
+    }
   }
 
   // The same matmul for callers that must not allocate device memory (code under HIP graph capture, serving loops,
@@ -348,7 +380,7 @@ class Engine {
     // dot-product kernels (5120 x 17408, 4 tokens: 50 against 88 us).  Not with two-pass inputs (their second half
     // goes through the kernels below).  ARCZ_GEMV_MM=0: off.
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
-    const bool mm_ok = !mm_off && !q2mm_ && w.type == GGML_Q4_K && a <= 1;
+    const bool mm_ok = !mm_off && !q2mm_ && w.type == GGML_Q4_K && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
       rd_bytes += raw_bytes(w);
@@ -404,7 +436,8 @@ class Engine {
         const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
                                  std::to_string(pf) + (tb > 1 ? " -DTB=" + std::to_string(tb) : std::string()) + " -DLDS=" +
                                  std::to_string(lds) +
-                                 (q2f ? " -DQ2_AQ=" + std::to_string(q2_aq_) + " -DQ2_SC=" + std::to_string(q2_sc_ / 4) : std::string());
+                                 (q2f ? " -DQ2_AQ=" + std::to_string(q2_aq_) + " -DQ2_SC=" + std::to_string(q2_sc_ / 4) : std::string()) +
+                                 head_defs(w);
         cl_kernel k = kernel("decode", defs, tb == 1 ? "gemv" : "gemv_mt");
         int ld1 = T == 1 ? 0 : ldc;  // (one token: C is the row itself)
         if (tb == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
@@ -416,7 +449,7 @@ class Engine {
       }
       const int gr = T == 1 ? gemv1_rows(w) : gemv_mt_rows(w);
       const std::string defs = "-DQT=" + std::to_string(w.type) + " -DGROWS=" + std::to_string(gr) +
-                               (T > 1 ? " -DTB=" + std::to_string(T) : std::string());
+                               (T > 1 ? " -DTB=" + std::to_string(T) : std::string()) + head_defs(w);
       cl_kernel k = kernel("decode", defs, T == 1 ? "gemv_v" : "gemv_mt_v");
       if (T == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
       else set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a);
@@ -566,7 +599,29 @@ class Engine {
   struct MoeLayer {
     GpuWeight ex[3];  // gate, up [NE][F][E]; down [NE][E][F]
     int NE = 0, NU = 0, E = 0, F = 0;
+    // the reference's routing variants (zero/engine_moe.h:99-101, zero/kernels/moe.cl:17-46): escale [NE] f32 -- each
+    // chosen expert's weight times its scale (-DESCALE); ebias [NE] f32 + rscale -- the sqrt(softplus) scores chosen with
+    // a bias (-DROUTE_DS -DRSCALE)
+    cl_mem escale = nullptr, ebias = nullptr;
+    float rscale = 1.0f;
+    bool variant() const { return escale || ebias; }
+    std::string route_defs() const {
+      if (ebias) {
+        char b[64];
+        snprintf(b, sizeof b, " -DROUTE_DS -DRSCALE=%.9ef", rscale);
+        return b;
+      }
+      return escale ? " -DESCALE" : "";
+    }
   };
+  void set_moe_routing(MoeLayer& L, const float* escale, const float* ebias, float rscale) {
+    if (escale && ebias) throw std::runtime_error("set_moe_routing: expert scales and the biased routing do not combine");
+    for (cl_mem* m : {&L.escale, &L.ebias})
+      if (*m) { release(*m); *m = nullptr; }
+    if (escale) L.escale = buf((size_t)L.NE * 4, escale);
+    if (ebias) L.ebias = buf((size_t)L.NE * 4, ebias);
+    L.rscale = rscale;
+  }
   // buffers of the layer (zero/engine_alloc.h:109-159): sized for max_chunk tokens
   cl_mem mids_ = nullptr, mwts_ = nullptr, sgate_ = nullptr, mcount_ = nullptr, moffs_ = nullptr, mcursor_ = nullptr,
          mtiles_ = nullptr, mtstart_ = nullptr, stok_ = nullptr, swt_ = nullptr, minv_ = nullptr, mh_ = nullptr,
@@ -612,9 +667,11 @@ class Engine {
     const std::string defs = "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DTM=" + std::to_string(tm) +
                              " -DNPART=" + std::to_string(kCountCopies);
     {
-      cl_kernel k = kernel("moe", defs, "moe_route");
+      cl_kernel k = kernel("moe", defs + L.route_defs(), "moe_route");
       int NR = ldl, TT = T;
       set_args(k, 0, rl, NR, TT, mids_, mwts_, sgate_, mcount_);
+      if (L.escale) set_args(k, 7, L.escale);  // (zero/engine_moe.h:114-115)
+      if (L.ebias) set_args(k, 7, L.ebias);
       size_t g1 = (size_t)(T + 3) / 4 * 256, l1 = 256;
       run("moe_route", k, 1, &g1, &l1);
     }
@@ -653,8 +710,11 @@ class Engine {
 
   // x[t] += sum_k w_k * expert_k(h[t]) for the T tokens whose quantized h is the current activation chunk
   // (zero/engine_moe.h:8-361 layer_moe: standard experts, no shared expert).  x: [T][E] f32.
-  void layer_moe(const MoeLayer& L, cl_mem rl, int ldl, cl_mem x, int T, int Mp) {
+  // sh (may be null): the shared expert's output rows [T][E] f32, added as sgate[t] * sh[t] (zero/kernels/moe.cl:344-352;
+  // sgate = sigmoid of the router row's logit past the experts', column NE of a row of ldl > NE values).
+  void layer_moe(const MoeLayer& L, cl_mem rl, int ldl, cl_mem x, int T, int Mp, cl_mem sh = nullptr) {
     const int E = L.E, F = L.F, NU = L.NU, n = T * NU;
+    if (sh && arcz_mem_size(sh) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: sh is too small");
     if (cur_T_ != T || cur_K_ != E || cur_Mp_ != Mp) throw std::runtime_error("layer_moe: the activations are not this chunk's");
     if (arcz_mem_size(x) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: x is too small");
     // A pass of 1-16 tokens (zero/engine_moe.h:86-262 has this form for 1-8): small tiles through the matrix-vector
@@ -677,19 +737,21 @@ class Engine {
       // one or two tokens, everything fused: the gate/up kernel routes the tokens itself (no routing launch: 2 launches
       // a layer; the kernel takes up to 8 tokens, but every work-group routes all of them, and from 4 tokens on the
       // routing launch is the cheaper way: 36.6 against 35.7 us at 4, 65.5 against 56.4 at 8)
-      const bool froute = T <= 2 && tmd == 1 && !fuse_off && F % 32 == 0 && NE <= 512 && NU <= 64;
+      const bool froute = T <= 2 && tmd == 1 && !fuse_off && F % 32 == 0 && NE <= 512 && NU <= 64 && !L.variant();
       if (froute) {
         if (ldl < NE || arcz_mem_size(rl) < ((size_t)(T - 1) * ldl + NE) * 4) throw std::runtime_error("layer_moe: router logits do not fit");
         tiles_max = (size_t)n;
       } else if (T == 1) {
         if (ldl < NE || arcz_mem_size(rl) < (size_t)NE * 4) throw std::runtime_error("layer_moe: router logits do not fit");
         cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DHAS_GATE=" +
-                                        std::to_string(ldl > NE ? 1 : 0), "moe_route1");
+                                        std::to_string(ldl > NE ? 1 : 0) + L.route_defs(), "moe_route1");
         set_args(k, 0, rl, sgate_, mtiles_, stok_, swt_, minv_);
+        if (L.escale) set_args(k, 6, L.escale);  // (zero/engine_moe.h:103-104)
+        if (L.ebias) set_args(k, 6, L.ebias);
         size_t g1 = 64, l1 = 64;
         run("moe_route", k, 1, &g1, &l1);
         tiles_max = (size_t)NU;
-      } else if (n <= 512 && NE <= 512) {
+      } else if (n <= 512 && NE <= 512 && !L.variant()) {
         // routing, scan and scatter of the few pairs in one work-group (the three launches took 19 us)
         if (ldl < NE || arcz_mem_size(rl) < ((size_t)(T - 1) * ldl + NE) * 4) throw std::runtime_error("layer_moe: router logits do not fit");
         cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DTM=" + std::to_string(tmd),
@@ -709,7 +771,7 @@ class Engine {
       // Tiles of one or two slots: the gate/up kernel quantizes its own output (32 rows a work-group: one block per
       // slot); one-slot tiles: the down kernel sums a token's experts into x itself.  3 launches instead of 5
       // (ARCZ_MOE_FUSE=0: the 5).
-      const bool fq = !fuse_off && tmd <= 2 && F % 32 == 0, fc = !fuse_off && tmd == 1 && NU <= 64;
+      const bool fq = !fuse_off && tmd <= 2 && F % 32 == 0, fc = !fuse_off && tmd == 1 && NU <= 64 && !sh;
       if (froute) {
         cl_kernel k = kernel("decode", "-DQT=" + std::to_string(L.ex[0].type) + " -DGROWS=4 -DTM=1 -DQUANT=1 -DROUTE=1 -DNE=" +
                                            std::to_string(NE), "moe_gateup_q");
@@ -760,7 +822,6 @@ class Engine {
         }
         {
           cl_kernel k = kernel("moe", "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU), "moe_combine");
-          cl_mem sh = nullptr;
           int EE = E;
           set_args(k, 0, x, sh, sgate_, my_, minv_, EE);
           size_t gws[2] = {((size_t)E + 1023) / 1024 * 256, (size_t)T}, lws[2] = {256, 1};
@@ -800,7 +861,6 @@ class Engine {
     moe_gemm(L, 2, Mp, max_tiles);
     {
       cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_combine");
-      cl_mem sh = nullptr;
       int EE = E;
       set_args(k, 0, x, sh, sgate_, my_, minv_, EE);
       size_t gws[2] = {((size_t)E + 1023) / 1024 * 256, (size_t)T}, lws[2] = {256, 1};  // (four columns a thread)
@@ -816,6 +876,7 @@ class Engine {
                                std::to_string(max_k) + ")");
   }
   std::map<std::string, cl_kernel> kernels_;
+  std::vector<cl_program> progs_;
   std::vector<cl_mem> mems_;
   std::vector<std::pair<std::string, cl_event>> events_;
 };

@@ -4,7 +4,8 @@
 #pragma once
 
 struct HiddenDef {
-  const char* name;  // nullptr ends the list; "LDS" is not an argument: it is the launch's dynamic LDS size in bytes
+  const char* name;  // nullptr ends the list; "LDS" is not an argument: it is the launch's dynamic LDS size in bytes;
+                     // "SOFTCAP" and "RSCALE" are read as floats ("-DSOFTCAP=30.0f") and ride along as their bit patterns
   int def;
   bool required;
 };
@@ -25,23 +26,24 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "add_norm_quant", nullptr, "pppiffpiipppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
+    {"ops", "softcap_rows", nullptr, "piiif", {nullptr}, {{nullptr, 0, false}}, 0},
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "mfma_probe", nullptr, "pi", {nullptr}, {{nullptr, 0, false}}, 256},
     // ---- decode
     {"decode", "gemv", "GU2", "piippppipiip", {"QT", "LPR", "PF", "GU2", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
-    {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
+    {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "LPR", "PF", "TB", nullptr},
-     {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {nullptr, 0, false}}, 256},
+     {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mm", nullptr, "piippppiipiiiii", {"QT", nullptr}, {{nullptr, 0, false}}, 512},
     {"decode", "moe_gateup_q", "ROUTE", "ppiipppippppipppppppiiipp", {"QT", "GROWS", "TM", "QUANT", "ROUTE", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 512},
     {"decode", "moe_gateup_q", "QUANT", "ppiipppippppippp", {"QT", "GROWS", "TM", "QUANT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 512},
     {"decode", "moe_down1_q", nullptr, "piipppipppppi", {"QT", "GROWS", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", "GROWS", "TM", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "moe_down_q", nullptr, "piipppipppp", {"QT", "GROWS", "TM", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
-    {"decode", "gemv_v", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{nullptr, 0, false}}, 256},
-    {"decode", "gemv_mt_v", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{nullptr, 0, false}}, 256},
+    {"decode", "gemv_v", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
+    {"decode", "gemv_mt_v", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     // ---- gemm
     {"gemm", "gemm", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
@@ -55,6 +57,13 @@ static const KernelSpec kKernelTable[] = {
     {"gemm", "splitk_reduce", nullptr, "pipiiiii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     // ---- moe
+    {"moe", "moe_route", "ESCALE", "piippppp", {"ESCALE", nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_route", "ROUTE_DS", "piippppp", {"ROUTE_DS", nullptr},
+     {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {"RSCALE", 0x3F800000, false}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_route1", "ESCALE", "ppppppp", {"ESCALE", nullptr},
+     {{"NE", 0, true}, {"NU", 0, true}, {"HAS_GATE", 0, false}, {nullptr, 0, false}}, 64},
+    {"moe", "moe_route1", "ROUTE_DS", "ppppppp", {"ROUTE_DS", nullptr},
+     {{"NE", 0, true}, {"NU", 0, true}, {"HAS_GATE", 0, false}, {"RSCALE", 0x3F800000, false}, {nullptr, 0, false}}, 64},
     {"moe", "moe_route", nullptr, "piipppp", {nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_route1", nullptr, "pppppp", {nullptr},
      {{"NE", 0, true}, {"NU", 0, true}, {"HAS_GATE", 0, false}, {nullptr, 0, false}}, 64},

@@ -158,4 +158,7 @@ template <bool WIDE> __device__ inline float group_sum_last(float v) {
     v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));  // row_bcast31 -> rows 2, 3
   return v;
 }
+// The output head's soft cap (the reference's -DSOFTCAP=c, zero/kernels/decode.cl:882-886): c * tanh(v / c) for c > 0,
+// v itself for c = 0 (no cap).  c is the same for the whole launch.
+__device__ inline float head_out(float v, float cap) { return cap > 0.0f ? cap * tanhf(v * (1.0f / cap)) : v; }
 #endif

@@ -209,7 +209,8 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
 template <int QT, int TB, int GROWS>
 __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, const signed char* __restrict__ aq,
                                  const float* __restrict__ asc, const short* __restrict__ absum, int M, int T,
-                                 float* __restrict__ C, int ldc, int c_off, int accumulate, size_t plane_rows) {
+                                 float* __restrict__ C, int ldc, int c_off, int accumulate, size_t plane_rows,
+                                 float softcap = 0.0f) {
   const int hl = threadIdx.x & 31;
   const int hw = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 5);
   const int r0 = hw * GROWS;
@@ -231,7 +232,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
   for (int r = 0; r < GROWS; ++r)
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
-      const float v = half_wave_sum(acc[r][t]);
+      const float v = head_out(half_wave_sum(acc[r][t]), softcap);
       const int n = r0 + r;
       if (hl == 0 && n < N && t < T) {
         float* cp = C + (size_t)t * ldc + c_off + n;
@@ -246,16 +247,16 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
 #define GEMV_INST(QT, GROWS)                                                                                         \
   extern "C" __global__ __launch_bounds__(256) void gemv_v__QT##QT##_GROWS##GROWS(                                      \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
-      const short* absum, int M, float* C, int c_off, int accumulate) {                                               \
-    gemv_body<QT, 1, GROWS>(raw, N, K, aq, asc, absum, M, 1, C, 0, c_off, accumulate, (size_t)N);                    \
+      const short* absum, int M, float* C, int c_off, int accumulate, float softcap) {                                \
+    gemv_body<QT, 1, GROWS>(raw, N, K, aq, asc, absum, M, 1, C, 0, c_off, accumulate, (size_t)N, softcap);           \
   }
 
 // gemv_mt_v: T = TB tokens (reference zero/kernels/decode.cl:1426).
 #define GEMV_MT_INST(QT, GROWS, TB)                                                                                  \
   extern "C" __global__ __launch_bounds__(256) void gemv_mt_v__QT##QT##_GROWS##GROWS##_TB##TB(                          \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
-      const short* absum, int M, int T, float* C, int ldc, int c_off, int accumulate) {                               \
-    gemv_body<QT, TB, GROWS>(raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, (size_t)N);                 \
+      const short* absum, int M, int T, float* C, int ldc, int c_off, int accumulate, float softcap) {                \
+    gemv_body<QT, TB, GROWS>(raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, (size_t)N, softcap);        \
   }
 
 #define GEMV_ALL(QT)                                                                                                 \

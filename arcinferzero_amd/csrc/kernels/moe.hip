@@ -9,17 +9,16 @@
 // moe_route: one wave per token.  The NU largest of NE logits (ties: the lower expert), p = exp(l - max),
 // weights p / sum of the selected p; counts[copy][e]++ per selection (NPART copies [NPART][NE], 1 by default); sgate[t] = sigmoid(logit NE) when the row holds one.
 // grid: ceil(T / 4) work-groups of 256 threads.
-extern "C" __global__ __launch_bounds__(256) void moe_route(const float* __restrict__ logits, int ldl, int T,
-                                                            int* __restrict__ ids, float* __restrict__ wts,
-                                                            float* __restrict__ sgate, int* __restrict__ counts,
-                                                            int NE, int NU, int NPART) {
+__device__ inline void moe_route_body(const float* __restrict__ logits, int ldl, int T, int* __restrict__ ids,
+                                      float* __restrict__ wts, float* __restrict__ sgate, int* __restrict__ counts,
+                                      int NE, int NU, int NPART, const RouteVariant rv) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;
   const float* lg = logits + (size_t)t * ldl;
   int mysel;
   float mywt;
-  route_one_token(lg, NE, NU, lane, mysel, mywt);
+  route_one_token(lg, NE, NU, lane, mysel, mywt, rv);
   if (lane < NU) {
     ids[(size_t)t * NU + lane] = mysel;
     wts[(size_t)t * NU + lane] = mywt;
@@ -27,18 +26,43 @@ extern "C" __global__ __launch_bounds__(256) void moe_route(const float* __restr
     //  over the chip queue up at the memory side; moe_scan sums the copies)
     atomicAdd(&counts[(size_t)(blockIdx.x % NPART) * NE + mysel], 1);
   }
-  if (lane == 0 && sgate) sgate[t] = ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
+  if (lane == 0 && sgate) sgate[t] = route_sgate(lg, NE, ldl > NE, rv);
+}
+extern "C" __global__ __launch_bounds__(256) void moe_route(const float* __restrict__ logits, int ldl, int T,
+                                                            int* __restrict__ ids, float* __restrict__ wts,
+                                                            float* __restrict__ sgate, int* __restrict__ counts,
+                                                            int NE, int NU, int NPART) {
+  moe_route_body(logits, ldl, T, ids, wts, sgate, counts, NE, NU, NPART, RouteVariant());
+}
+// (-DESCALE: argument 7 is escale [NE]; -DROUTE_DS -DRSCALE=s: argument 7 is ebias [NE]; zero/engine_moe.h:113-116)
+extern "C" __global__ __launch_bounds__(256) void moe_route__ESCALE1(const float* __restrict__ logits, int ldl, int T,
+                                                                     int* __restrict__ ids, float* __restrict__ wts,
+                                                                     float* __restrict__ sgate, int* __restrict__ counts,
+                                                                     const float* __restrict__ escale, int NE, int NU,
+                                                                     int NPART) {
+  RouteVariant rv;
+  rv.escale = escale;
+  moe_route_body(logits, ldl, T, ids, wts, sgate, counts, NE, NU, NPART, rv);
+}
+extern "C" __global__ __launch_bounds__(256) void moe_route__ROUTE_DS1(const float* __restrict__ logits, int ldl, int T,
+                                                                       int* __restrict__ ids, float* __restrict__ wts,
+                                                                       float* __restrict__ sgate, int* __restrict__ counts,
+                                                                       const float* __restrict__ ebias, int NE, int NU,
+                                                                       int NPART, float rscale) {
+  RouteVariant rv;
+  rv.ebias = ebias;
+  rv.rscale = rscale;
+  moe_route_body(logits, ldl, T, ids, wts, sgate, counts, NE, NU, NPART, rv);
 }
 
 // moe_route1: a single token straight into NU one-slot tiles (no counts, scan or scatter).  One wave.
-extern "C" __global__ __launch_bounds__(64) void moe_route1(const float* __restrict__ logits, float* __restrict__ sgate,
-                                                            int* __restrict__ tiles, int* __restrict__ stok,
-                                                            float* __restrict__ swt, int* __restrict__ inv, int NE,
-                                                            int NU, int has_gate) {
+__device__ inline void moe_route1_body(const float* __restrict__ logits, float* __restrict__ sgate, int* __restrict__ tiles,
+                                       int* __restrict__ stok, float* __restrict__ swt, int* __restrict__ inv, int NE,
+                                       int NU, int has_gate, const RouteVariant rv) {
   const int lane = threadIdx.x & 63;
   int mysel;
   float mywt;
-  route_one_token(logits, NE, NU, lane, mysel, mywt);
+  route_one_token(logits, NE, NU, lane, mysel, mywt, rv);
   if (lane < NU) {
     tiles[1 + 3 * lane] = mysel;
     tiles[2 + 3 * lane] = lane;
@@ -49,8 +73,33 @@ extern "C" __global__ __launch_bounds__(64) void moe_route1(const float* __restr
   }
   if (lane == 0) {
     tiles[0] = NU;
-    if (sgate) sgate[0] = has_gate ? 1.0f / (1.0f + expf(-logits[NE])) : 0.0f;
+    if (sgate) sgate[0] = route_sgate(logits, NE, has_gate != 0, rv);
   }
+}
+extern "C" __global__ __launch_bounds__(64) void moe_route1(const float* __restrict__ logits, float* __restrict__ sgate,
+                                                            int* __restrict__ tiles, int* __restrict__ stok,
+                                                            float* __restrict__ swt, int* __restrict__ inv, int NE,
+                                                            int NU, int has_gate) {
+  moe_route1_body(logits, sgate, tiles, stok, swt, inv, NE, NU, has_gate, RouteVariant());
+}
+extern "C" __global__ __launch_bounds__(64) void moe_route1__ESCALE1(const float* __restrict__ logits, float* __restrict__ sgate,
+                                                                     int* __restrict__ tiles, int* __restrict__ stok,
+                                                                     float* __restrict__ swt, int* __restrict__ inv,
+                                                                     const float* __restrict__ escale, int NE, int NU,
+                                                                     int has_gate) {
+  RouteVariant rv;
+  rv.escale = escale;
+  moe_route1_body(logits, sgate, tiles, stok, swt, inv, NE, NU, has_gate, rv);
+}
+extern "C" __global__ __launch_bounds__(64) void moe_route1__ROUTE_DS1(const float* __restrict__ logits, float* __restrict__ sgate,
+                                                                       int* __restrict__ tiles, int* __restrict__ stok,
+                                                                       float* __restrict__ swt, int* __restrict__ inv,
+                                                                       const float* __restrict__ ebias, int NE, int NU,
+                                                                       int has_gate, float rscale) {
+  RouteVariant rv;
+  rv.ebias = ebias;
+  rv.rscale = rscale;
+  moe_route1_body(logits, sgate, tiles, stok, swt, inv, NE, NU, has_gate, rv);
 }
 
 // moe_route_small: the routing of a pass of a few tokens in one work-group of 512 threads -- moe_route, moe_scan and

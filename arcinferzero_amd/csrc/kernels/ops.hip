@@ -299,6 +299,16 @@ extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __re
   }
 }
 
+// softcap_rows: C[t][off + n] = cap * tanh(C[t][off + n] / cap) over N columns of the launch's rows (the output head of
+// a two-pass engine: the cap applies to the sum of both passes; reference zero/engine.h:1103-1110).
+// grid (ceil(N / 256) * 256, T).
+extern "C" __global__ void softcap_rows(float* C, int ld, int off, int N, float cap) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+  if (n >= N) return;
+  float* p = C + (size_t)t * ld + off + n;
+  *p = head_out(*p, cap);
+}
+
 // fill32: p[i] = v for i < n (the fill used where a captured graph must not hold a memset node).
 extern "C" __global__ void fill32(uint32_t* p, uint32_t v, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -33,14 +33,26 @@ __device__ inline void route_wave_best(float& bv, int& bi) {
   for (int r = 1; r < 4; ++r) route_better(bv, bi, rv[r], ri[r]);
 }
 
+// The reference's routing variants (zero/kernels/moe.cl:17-46), chosen per launch: escale (its -DESCALE, Gemma 4) -- each
+// chosen expert's weight times escale[e] after the normalization; ebias (its -DROUTE_DS, DeepSeek-V4.1) -- the score is
+// s = sqrt(softplus(logit)), experts are chosen by s + ebias[e], and the weights are s / (sum of the chosen s + 1e-20) *
+// rscale.  Both null: the softmax routing.
+struct RouteVariant {
+  const float* escale = nullptr;
+  const float* ebias = nullptr;
+  float rscale = 1.0f;
+};
+__device__ inline float route_ds_sp(float g) { return sqrtf(g > 20.0f ? g + log1pf(expf(-g)) : log1pf(expf(g))); }
+
 template <int PL>
-__device__ inline void route_one_token_pl(const float* __restrict__ lg, int NE, int NU, int lane, int& sel, float& wt) {
+__device__ inline void route_one_token_pl(const float* __restrict__ lg, int NE, int NU, int lane, int& sel, float& wt,
+                                          const RouteVariant rv = RouteVariant()) {
   float v[PL];
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < PL; ++i) {
     const int e = i * 64 + lane;
-    v[i] = e < NE ? lg[e] : -INFINITY;
+    v[i] = e < NE ? (rv.ebias ? route_ds_sp(lg[e]) + rv.ebias[e] : lg[e]) : -INFINITY;
     mx = fmaxf(mx, v[i]);
   }
 #pragma unroll
@@ -57,16 +69,24 @@ __device__ inline void route_one_token_pl(const float* __restrict__ lg, int NE, 
 #pragma unroll
     for (int i = 0; i < PL; ++i)
       if (i * 64 + lane == bi) v[i] = -INFINITY;
-    const float p = expf(bv - mx);
+    const int sk = min(bi, NE - 1);  // (a row of NaN picks no lane: keep the index inside the tables)
+    const float p = rv.ebias ? route_ds_sp(lg[sk]) : expf(bv - mx);
     sum += p;
-    if (lane == k) { mysel = min(bi, NE - 1); myp = p; }  // (a row of NaN picks no lane: keep the index inside the tables)
+    if (lane == k) { mysel = sk; myp = p; }
   }
   sel = mysel;
-  wt = myp / sum;
+  wt = rv.ebias ? myp / (sum + 1e-20f) * rv.rscale : myp / sum;
+  if (rv.escale) wt *= rv.escale[mysel];
 }
 
 // (two logits a lane serve up to 128 experts, the common case; the same steps either way)
-__device__ inline void route_one_token(const float* __restrict__ lg, int NE, int NU, int lane, int& sel, float& wt) {
-  if (NE <= 128) route_one_token_pl<2>(lg, NE, NU, lane, sel, wt);
-  else route_one_token_pl<ROUTE_PER_LANE>(lg, NE, NU, lane, sel, wt);
+__device__ inline void route_one_token(const float* __restrict__ lg, int NE, int NU, int lane, int& sel, float& wt,
+                                       const RouteVariant rv = RouteVariant()) {
+  if (NE <= 128) route_one_token_pl<2>(lg, NE, NU, lane, sel, wt, rv);
+  else route_one_token_pl<ROUTE_PER_LANE>(lg, NE, NU, lane, sel, wt, rv);
+}
+// The shared expert's gate of a token (moe.cl:40, 46): sigmoid of the logit past the experts' when the row holds one;
+// 1 with the -DROUTE_DS routing.
+__device__ inline float route_sgate(const float* __restrict__ lg, int NE, bool has_gate, const RouteVariant rv) {
+  return rv.ebias ? 1.0f : has_gate ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
 }

@@ -39,6 +39,12 @@ arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, c
                                            const char* down, int NU);
 int arcz_weight_free(arcz_engine* e, arcz_weight* w);
 arcz_mem* arcz_weight_raw(const arcz_weight* w);
+/* Marks w as the output head of a model with final-logit soft-capping (the reference's lm_head_ with hp.softcap,
+ * zero/engine.h:984-990; kernel epilogue -DSOFTCAP=c, zero/kernels/decode.cl:882-886): arcz_engine_matmul over 1-8
+ * tokens writes c * tanh(v / c) (then adds C when accumulating); with two-pass inputs both passes run without the cap
+ * and the sum is capped (zero/engine.h:1081-1110).  Chunks of more than 8 tokens are not capped (the reference's heads
+ * never see them).  cap = 0: no cap. */
+int arcz_weight_set_softcap(arcz_weight* w, float cap);
 
 /* The activation quantizer as a step of its own (quant_store16 of zero/kernels/ops.cl:38-72 inside the launch of
  * zero/engine.h:1256-1267): rows [0, T) of x (f32, row stride ldx) -> the engine's aq / asc / absum laid out for
@@ -109,6 +115,20 @@ arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void*
 /* Engine::layer_moe (zero/engine_moe.h:8-361, standard experts, no shared expert): x[t] += sum_k w_k expert_k(h[t]) for
  * the T tokens whose quantized h is the current activation chunk; logits: router logits [T][ldl] f32. */
 int arcz_engine_layer_moe(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp);
+/* The same with the shared expert's term (moe_combine's sgate * sh, zero/kernels/moe.cl:344-352): sh [T][E] f32 is the
+ * shared expert's output for the chunk (computed by the caller with arcz_engine_matmul, as zero/engine_moe.h:66-84
+ * does); x[t] += sgate[t] * sh[t] + the experts' sum, sgate[t] = sigmoid(logits[t][NE]) for rows of ldl > NE values. */
+int arcz_engine_layer_moe_sh(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp,
+                             arcz_mem* sh);
+/* The reference's routing variants (zero/kernels/moe.cl:17-46, set by zero/engine_moe.h:99-116): escale [NE] (host f32,
+ * its -DESCALE: each chosen expert's weight times its scale, after the normalization) or ebias [NE] + rscale (its
+ * -DROUTE_DS -DRSCALE: scores sqrt(softplus(logit)), experts chosen by score + bias, weights score / (sum + 1e-20) *
+ * rscale, shared-expert gate 1).  Both NULL: the softmax routing again.  Not both at once. */
+int arcz_moe_layer_set_routing(arcz_engine* e, arcz_moe_layer* L, const float* escale, const float* ebias, float rscale);
+/* Frees a layer's expert tensors and routing tables. */
+int arcz_moe_layer_free(arcz_engine* e, arcz_moe_layer* L);
+/* sgate [max_chunk] f32: the shared expert's gate per token, as the last routing wrote it. */
+arcz_mem* arcz_engine_moe_sgate(arcz_engine* e);
 /* The routing step alone (moe_route + moe_scan + moe_scatter, zero/engine_moe.h:111-133) with tiles of tm slots, and
  * its buffers: which = 0 ids, 1 wts, 2 offs, 3 tiles, 4 tstart, 5 stok, 6 swt, 7 inv, 8 h (f32), 9 hq, 10 hsc, 11 y,
  * 12 hbs (int16 sums of each 16 values of hq, [F/16][slots]). */

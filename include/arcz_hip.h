@@ -65,6 +65,11 @@ int arcz_d2h(void* dst, const arcz_mem* src, size_t offset, size_t bytes);
 int arcz_d2d(arcz_mem* dst, size_t dst_offset, const arcz_mem* src, size_t src_offset, size_t bytes);
 int arcz_fill(arcz_mem* dst, const void* pattern, size_t pattern_bytes, size_t offset, size_t bytes);
 
+/* zrt::host_alloc and zrt::mem_free of such a pointer (clrt.h:445-452, 160): pinned host memory, the staging behind
+ * clEnqueueMapBuffer / clEnqueueUnmapMemObject (clrt.h:711-743).  NULL + error text on failure. */
+void* arcz_host_alloc(size_t bytes);
+int arcz_host_free(void* p);
+
 /* Engine::kernel(which, defs, name) (zero/engine_setup.h:317-362) over ClRt::build + ClRt::kernel
  * (clrt.h:1189-1307): `which` names the module ("ops", "decode", "gemm", "moe"), `defs` is the reference's -D string
  * and `name` the kernel.  The reference compiles one program per -D string at run time; here every variant is

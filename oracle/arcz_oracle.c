@@ -559,6 +559,43 @@ float orc_silu(float x) { return x < -80.0f ? 0.0f : x / (1.0f + expf(-x)); }
 /* Routing of T tokens (zero/kernels/moe.cl:50-89): the NU largest of NE logits (ties: the lower expert id),
  * p_k = exp(l_k - max l), weights p_k / sum of the selected p; per-expert counts; sgate = sigmoid(l[NE]) when the
  * row has a shared-expert logit at column NE (ldl > NE), else 0.5 is NOT written: sgate may be NULL. */
+/* The routing variants of zero/kernels/moe.cl:17-46 (parity unpinned: none of the reference's tests or files holds a
+ * vector of them; held by a float64 numpy restatement of the same formulas in tests/test_gpu_moe.py): escale (-DESCALE):
+ * the weight times escale[e] after the normalization; ebias + rscale (-DROUTE_DS -DRSCALE): score s = sqrt(softplus(l)),
+ * chosen by s + ebias[e], weight s / (sum + 1e-20) * rscale, shared-expert gate 1. */
+static float orc_ds_sp(float g) { return sqrtf(g > 20.0f ? g + log1pf(expf(-g)) : log1pf(expf(g))); }
+void orc_moe_route_v(const float* logits, int ldl, int T, int NE, int NU, int32_t* ids, float* wts, float* sgate,
+                     int32_t* counts, const float* escale, const float* ebias, float rscale) {
+  for (int e = 0; e < NE; ++e) counts[e] = 0;
+  float* v = (float*)malloc((size_t)NE * sizeof(float));
+  for (int t = 0; t < T; ++t) {
+    const float* lg = logits + (size_t)t * ldl;
+    float mx = -INFINITY;
+    for (int e = 0; e < NE; ++e) { v[e] = ebias ? orc_ds_sp(lg[e]) + ebias[e] : lg[e]; mx = fmaxf(mx, v[e]); }
+    float p[64], sum = 0.0f;
+    int sel[64];
+    for (int k = 0; k < NU; ++k) {
+      float bv = -INFINITY;
+      int bi = NE;
+      for (int e = 0; e < NE; ++e)
+        if (v[e] > bv) { bv = v[e]; bi = e; }
+      if (bi < NE) v[bi] = -INFINITY;
+      sel[k] = bi < NE - 1 ? bi : NE - 1;
+      p[k] = ebias ? orc_ds_sp(lg[sel[k]]) : expf(bv - mx);
+      sum += p[k];
+    }
+    for (int k = 0; k < NU; ++k) {
+      float w = ebias ? p[k] / (sum + 1e-20f) * rscale : p[k] / sum;
+      if (escale) w *= escale[sel[k]];
+      ids[(size_t)t * NU + k] = sel[k];
+      wts[(size_t)t * NU + k] = w;
+      counts[sel[k]]++;
+    }
+    if (sgate) sgate[t] = ebias ? 1.0f : ldl > NE ? 1.0f / (1.0f + expf(-lg[NE])) : 0.0f;
+  }
+  free(v);
+}
+
 void orc_moe_route(const float* logits, int ldl, int T, int NE, int NU, int32_t* ids, float* wts, float* sgate,
                    int32_t* counts) {
   for (int e = 0; e < NE; ++e) counts[e] = 0;

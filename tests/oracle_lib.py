@@ -163,6 +163,21 @@ def moe_route(logits, NE, NU):
     return ids, wts, sgate, counts
 
 
+def moe_route_v(logits, NE, NU, escale=None, ebias=None, rscale=1.0):
+    """The routing with the reference's variants (moe.cl:17-46): expert scales, or the biased sqrt(softplus) scores."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    T, ldl = logits.shape
+    ids = np.empty((T, NU), np.int32)
+    wts = np.empty((T, NU), np.float32)
+    sgate = np.empty(T, np.float32)
+    counts = np.empty(NE, np.int32)
+    es = None if escale is None else np.ascontiguousarray(escale, dtype=np.float32)
+    eb = None if ebias is None else np.ascontiguousarray(ebias, dtype=np.float32)
+    orc.orc_moe_route_v(ptr(logits), _i(ldl), _i(T), _i(NE), _i(NU), ptr(ids), ptr(wts), ptr(sgate), ptr(counts),
+                        ptr(es) if es is not None else None, ptr(eb) if eb is not None else None, C.c_float(rscale))
+    return ids, wts, sgate, counts
+
+
 def moe_scan(counts, TM):
     counts = np.ascontiguousarray(counts, dtype=np.int32)
     NE = counts.size

@@ -143,3 +143,38 @@ def test_gemv_gu_equals_two_launches(eng, qtype, F, K):
     for b in (c1, c2, xb):
         b.free()
     g.free(); u.free()
+
+
+@pytest.mark.parametrize("qtype,N,K,T", [(az.Q6_K, 1000, 512, 1), (az.Q4_K, 264, 512, 3), (az.Q8_0, 300, 17408, 2),
+                                         (az.Q6_K, 520, 17408, 5), (az.Q4_K, 264, 1024, 8)])
+def test_gemv_softcap_output_head(eng, qtype, N, K, T):
+    """The output head's soft cap (the reference's -DSOFTCAP=c, zero/kernels/decode.cl:882-886, 1029-1031): the GEMVs
+    write c * tanh(v / c), then add C when accumulating.  LDS-staged and global-memory kernels, 1-8 tokens."""
+    cap = 30.0
+    print(f"softcap {TYPE_NAMES[qtype]} N={N} K={K} T={T}", flush=True)
+    W = make_weights(qtype, N, K, seed=81)
+    # (values large enough for the cap to bend them)
+    x = make_acts(T, K, seed=82) * np.float32(40.0)
+    w = eng.make_weight(qtype, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, 16, T)
+    plain = az.Runtime.alloc(T * N * 4)
+    eng.matmul("head", w, 16, plain, N, 0, 0)
+    y = plain.read(np.float32, T * N).reshape(T, N)
+    w.set_softcap(cap)
+    c0 = az.gen_normal(83, (T, N))
+    capped, capped_acc = az.Runtime.alloc(T * N * 4).fill(0xFFFFFFFF), az.Runtime.from_numpy(c0)
+    eng.matmul("head", w, 16, capped, N, 0, 0)
+    eng.matmul("head", w, 16, capped_acc, N, 0, 1)
+    yc = capped.read(np.float32, T * N).reshape(T, N)
+    ya = capped_acc.read(np.float32, T * N).reshape(T, N)
+    want = cap * np.tanh(y.astype(np.float64) / cap)
+    assert np.abs(y).max() > cap / 2                               # the cap matters here
+    assert np.abs(yc - want).max() <= 2e-6 * cap
+    assert np.abs(ya - (c0 + yc)).max() <= 1e-6 * cap
+    w.set_softcap(0.0)
+    eng.matmul("head", w, 16, capped, N, 0, 0)
+    assert np.array_equal(capped.read(np.uint32, T * N), y.view(np.uint32).ravel())
+    for b in (plain, capped, capped_acc, xb):
+        b.free()
+    w.free()

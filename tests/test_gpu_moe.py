@@ -183,3 +183,104 @@ def _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp):
             b.free()
     finally:
         eng.close()
+
+
+@pytest.mark.parametrize("T", [1, 7, 40, 300])
+@pytest.mark.parametrize("variant", ["escale", "route_ds"])
+def test_routing_variants(rt, variant, T):
+    """The reference's routing variants (zero/kernels/moe.cl:17-46): expert scales applied after the normalization; the
+    sqrt(softplus) scores chosen with a bias.  Against the oracle and against the same formulas in float64."""
+    NE, NU = 64, 6
+    print(f"routing variant {variant} T={T}", flush=True)
+    eng = az.Engine(512, 256)
+    try:
+        dummy = np.zeros(az.gguf_bytes(az.Q8_0, NE * 256, 256), np.uint8)
+        L = eng.make_moe_layer(az.Q8_0, dummy, dummy, dummy, NE, NU, 256, 256)
+        rng = np.random.default_rng(31 + T)
+        logits = (rng.standard_normal((T, NE + 1)) * 2.0).astype(np.float32)
+        escale = (0.5 + rng.random(NE)).astype(np.float32)
+        ebias = (rng.standard_normal(NE) * 0.3).astype(np.float32)
+        rscale = 2.5
+        if variant == "escale":
+            eng.set_moe_routing(L, escale=escale)
+            ids, wts, sgate, counts = orc.moe_route_v(logits, NE, NU, escale=escale)
+        else:
+            eng.set_moe_routing(L, ebias=ebias, rscale=rscale)
+            ids, wts, sgate, counts = orc.moe_route_v(logits, NE, NU, ebias=ebias, rscale=rscale)
+        lb = az.Runtime.from_numpy(logits)
+        x = az.Runtime.from_numpy(az.gen_normal(1, (T, 256)))
+        eng.quantize(x, 256, 256, 512 if T > 16 else 16, T)
+        out = az.Runtime.alloc(T * 256 * 4).fill(0)
+        eng.layer_moe(L, lb, NE + 1, out, T, 512 if T > 16 else 16)       # (zero weights: only the routing matters)
+        n = T * NU
+        gi = eng.moe_buffer("ids").read(np.int32, n).reshape(T, NU) if T > 1 else None
+        inv = eng.moe_buffer("inv").read(np.int32, n)
+        gw = eng.moe_buffer("swt").read(np.float32, n)[inv].reshape(T, NU)
+        gs = eng.moe_sgate.read(np.float32, T)
+        if gi is not None:
+            assert np.array_equal(gi, ids)
+        else:   # one token: the chosen experts are the tiles' experts
+            tiles = eng.moe_buffer("tiles").read(np.int32, 1 + 3 * NU)
+            assert tiles[0] == NU and np.array_equal(tiles[1::3], ids[0])
+        assert np.abs(gw - wts).max() < 1e-6 * max(1.0, np.abs(wts).max())
+        assert np.abs(gs - sgate).max() < 1e-6
+        # the formulas in float64
+        l64 = logits[:, :NE].astype(np.float64)
+        if variant == "escale":
+            for t in range(T):
+                idx = np.argsort(-l64[t], kind="stable")[:NU]
+                p = np.exp(l64[t, idx] - l64[t, idx[0]])
+                assert np.array_equal(ids[t], idx) and np.abs(wts[t] - p / p.sum() * escale[idx]).max() < 1e-5
+            assert np.abs(sgate - 1.0 / (1.0 + np.exp(-logits[:, NE].astype(np.float64)))).max() < 1e-6
+        else:
+            sp = np.sqrt(np.where(l64 > 20, l64 + np.log1p(np.exp(-l64)), np.log1p(np.exp(l64))))
+            for t in range(T):
+                idx = np.argsort(-(sp[t].astype(np.float32) + ebias), kind="stable")[:NU]
+                assert np.array_equal(ids[t], idx)
+                assert np.abs(wts[t] - sp[t, idx] / (sp[t, idx].sum() + 1e-20) * rscale).max() < 1e-5
+            assert (sgate == 1.0).all()
+        eng.set_moe_routing(L)                                           # back to the softmax routing
+        eng.layer_moe(L, lb, NE + 1, out, T, 512 if T > 16 else 16)
+        inv = eng.moe_buffer("inv").read(np.int32, n)
+        gw = eng.moe_buffer("swt").read(np.float32, n)[inv].reshape(T, NU)
+        assert np.abs(gw - orc.moe_route(logits, NE, NU)[1]).max() < 1e-6
+        for b in (lb, x, out):
+            b.free()
+    finally:
+        eng.close()
+
+
+@pytest.mark.parametrize("qtype,T,Mp", [(az.Q4_K, 1, 16), (az.Q4_K, 2, 16), (az.Q6_K, 6, 16), (az.Q4_K, 70, 80), (az.Q8_0, 33, 48)])
+def test_moe_layer_with_shared_expert_term(rt, qtype, T, Mp):
+    """moe_combine's shared-expert term (zero/kernels/moe.cl:344-352): router rows of NE + 1 logits, the last the shared
+    expert's gate; x += sigmoid(gate) * sh + the experts' sum.  Against the same layer without the term."""
+    NE, NU, E, F = 8, 2, 256, 256
+    print(f"moe layer with sh, type {qtype} T={T}", flush=True)
+    eng = az.Engine(Mp, 256)
+    try:
+        L = eng.make_moe_layer(qtype, make_weights(qtype, NE * F, E, seed=1), make_weights(qtype, NE * F, E, seed=2),
+                               make_weights(qtype, NE * E, F, seed=3), NE, NU, E, F)
+        rng = np.random.default_rng(7)
+        logits = rng.standard_normal((T, NE + 1)).astype(np.float32)
+        x0 = az.gen_normal(9, (T, E))
+        sh = az.gen_normal(10, (T, E))
+        xb = az.Runtime.from_numpy(make_acts(T, E, seed=4))
+        eng.quantize(xb, E, E, Mp, T)
+        lb, shb = az.Runtime.from_numpy(logits), az.Runtime.from_numpy(sh)
+        o0, o1 = az.Runtime.from_numpy(x0), az.Runtime.from_numpy(x0)
+        eng.layer_moe(L, lb, NE + 1, o0, T, Mp)
+        eng.layer_moe(L, lb, NE + 1, o1, T, Mp, sh=shb)
+        plain = o0.read(np.float32, T * E).reshape(T, E)
+        with_sh = o1.read(np.float32, T * E).reshape(T, E)
+        gate = 1.0 / (1.0 + np.exp(-logits[:, NE].astype(np.float64)))
+        assert np.abs(eng.moe_sgate.read(np.float32, T) - gate).max() < 1e-6
+        want = plain.astype(np.float64) + gate[:, None] * sh
+        assert np.abs(with_sh - want).max() <= 2e-6 * np.abs(want).max()
+        # and the routing ignored the extra column
+        ids, _, _, _ = orc.moe_route(logits, NE, NU)
+        if T > 1:
+            assert np.array_equal(eng.moe_buffer("ids").read(np.int32, T * NU).reshape(T, NU), ids)
+        for b in (xb, lb, shb, o0, o1):
+            b.free()
+    finally:
+        eng.close()

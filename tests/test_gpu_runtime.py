@@ -106,3 +106,16 @@ def test_fake_oom_and_hook(rt):
         a.free()
     finally:
         az.lib.arcz_set_fake_oom(0)
+
+
+def test_reference_style_snippet_against_the_shim(rt):
+    """tests/clrt_snippet.cpp -- clCreateBuffer, cl.build, cl.kernel, set_args, clEnqueueNDRangeKernel, CL_CHECK,
+    clEnqueueMapBuffer / clEnqueueUnmapMemObject written as the reference's engine code writes them (zero/clrt.h:711-743,
+    1189-1307) -- compiled against clrt_hip.h by the library's Makefile, run here as a process of its own."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "clrt_snippet")
+    assert os.path.exists(exe), "tests/clrt_snippet is not built (make -C arcinferzero_amd/csrc)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr)
+    assert r.returncode == 0 and "clrt_snippet ok" in r.stdout

@@ -135,3 +135,26 @@ def test_mode_switch(rt):
                 e.set_activations(aq, asc, absum, K, 16, 1)
     assert np.array_equal(outs[0], outs[2]) and not np.array_equal(outs[0], outs[1])
     e.close()
+
+
+@pytest.mark.parametrize("qtype,T", [(az.Q6_K, 1), (az.Q4_K, 3), (az.Q8_0, 7)])
+def test_two_pass_output_head_softcap(eng, qtype, T):
+    """An output head with a soft cap under two-pass inputs (zero/engine.h:1081-1110): both passes run without the cap and
+    the cap is applied to their sum -- c * tanh((v1 + v2) / c), not the sum of two capped values."""
+    N, K, cap = 264, 1024, 30.0
+    W = make_weights(qtype, N, K, seed=91)
+    w = eng.make_weight(qtype, N, K, W)
+    xb = az.Runtime.from_numpy(make_acts(T, K, seed=92) * np.float32(40.0))
+    eng.quantize(xb, K, K, 16, T)
+    plain = az.Runtime.alloc(T * N * 4)
+    eng.matmul("head", w, 16, plain, N, 0, 0)
+    y = plain.read(np.float32, T * N).reshape(T, N)
+    w.set_softcap(cap)
+    capped = az.Runtime.alloc(T * N * 4).fill(0xFFFFFFFF)
+    eng.matmul("head", w, 16, capped, N, 0, 0)
+    yc = capped.read(np.float32, T * N).reshape(T, N)
+    assert np.abs(y).max() > cap / 2
+    assert np.abs(yc - cap * np.tanh(y.astype(np.float64) / cap)).max() <= 2e-6 * cap
+    for b in (plain, capped, xb):
+        b.free()
+    w.free()
