@@ -9,7 +9,7 @@ import os
 
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, IQ3_S, IQ4_XS = 2, 8, 12, 13, 14, 21, 23  # GGUF type ids (Q4_0 is uploaded as Q8_0 planes, IQ3_S as Q6_K planes, value for value)
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, IQ3_S, IQ4_XS = 2, 8, 12, 13, 14, 21, 23  # GGUF type ids
 
 lib_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libarcz_hip.so")
 if not os.path.exists(lib_path):
@@ -93,6 +93,7 @@ _sig("arcz_engine_residual", _p, _p, _i)
 _sig("arcz_engine_asc", _p, _p)
 _sig("arcz_engine_absum", _p, _p)
 _sig("arcz_engine_matmul", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
+_sig("arcz_iq3s_grid", None, _p)
 _sig("arcz_weight_set_softcap", _i, _p, C.c_float)
 _sig("arcz_engine_gemv_gu", _i, _p, _p, _p, _i, _p)
 _sig("arcz_engine_matmul_noalloc", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)

@@ -51,22 +51,6 @@ struct Iq3sGrid {
 };
 const Iq3sGrid kIq3s;
 
-// The 256 values of one IQ3_S superblock (110 bytes: f16 d, 64 index bytes, 8 bytes of ninth index bits, 32 sign bytes,
-// 4 bytes of scale nibbles; reference src/quants.h:240-262) as signed integers -15..15, and the 8 sub-scales 1 + 2 s.
-void iq3s_values(const uint8_t* p, int8_t* q, int* sc) {
-  const uint8_t *qs = p + 2, *qh = p + 66, *sg = p + 74, *scl = p + 106;
-  for (int ib = 0; ib < 8; ++ib) {
-    sc[ib] = 1 + 2 * ((scl[ib / 2] >> (4 * (ib % 2))) & 0xF);
-    for (int g = 0; g < 8; ++g) {
-      const uint8_t* m = kIq3s.m[qs[8 * ib + g] | (((qh[ib] >> g) & 1) << 8)];
-      for (int j = 0; j < 4; ++j) {
-        const int e = 4 * g + j;
-        q[32 * ib + e] = (int8_t)(((sg[4 * ib + e / 8] >> (e % 8)) & 1) ? -(int)m[j] : (int)m[j]);
-      }
-    }
-  }
-}
-
 // 256 six-bit values (0..63) into the ql / qh bytes of a Q6_K superblock (reference src/quants.h:115-134 read backwards)
 void q6k_pack(const int* q, uint8_t* ql, uint8_t* qh) {
   for (int n = 0; n < 2; ++n)
@@ -133,9 +117,11 @@ size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
   return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : type == GGML_TYPE_IQ3_S ? u * 110 : 0;
 }
-// (Q4_0 rows are kept on the device as Q8_0 planes, IQ3_S rows as Q6_K planes: see arcz_repack_planes)
-size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) {
-  return raw_planes_bytes(type == GGML_TYPE_Q4_0 ? QT_Q8_0 : type == GGML_TYPE_IQ3_S ? QT_Q6_K : (int)type, rows, K / 256);
+size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) { return raw_planes_bytes((int)type, rows, K / 256); }
+// The IQ3_S codebook as the kernels take it: 512 words, byte j of a word = magnitude j of the entry (1, 3, ..., 15).
+void arcz_iq3s_grid(uint32_t* out) {
+  for (int i = 0; i < 512; ++i)
+    out[i] = (uint32_t)kIq3s.m[i][0] | ((uint32_t)kIq3s.m[i][1] << 8) | ((uint32_t)kIq3s.m[i][2] << 16) | ((uint32_t)kIq3s.m[i][3] << 24);
 }
 
 // GGUF rows -> device planes (layout: kernels/common.h).  0 or -1 (unsupported type / K).
@@ -198,21 +184,18 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
     return 0;
   }
   if (type == GGML_TYPE_IQ3_S) {
-    // An IQ3_S superblock is d * (1 + 2 s) * (+-1, 3, ..., 15) with one s per 32 values (reference src/quants.h:240-262):
-    // exactly a Q6_K superblock with the same d, sub-scale 1 + 2 s for both 16-value halves and q = value + 32.
-    // Written out as Q6_K planes, value for value, so every Q6_K kernel serves it exactly, at 210 instead of 110 bytes
-    // per superblock on the device.
-    const PlanesQ6K pl = planes_q6k(rows, nsb);
-    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_Q6_K, rows, nsb) - (pl.d + u * 2));
+    // 110-byte superblocks (f16 d, 64 index bytes, 8 bytes of ninth bits, 32 sign bytes, 4 bytes of scale nibbles;
+    // reference src/quants.h:240-262) regrouped into planes, byte for byte
+    const PlanesIQ3S pl = planes_iq3s(rows, nsb);
+    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_IQ3_S, rows, nsb) - (pl.d + u * 2));
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < u; ++i) {
-      int8_t v[256];
-      int sc[8], q[256];
-      iq3s_values(src + i * 110, v, sc);
-      for (int e = 0; e < 256; ++e) q[e] = v[e] + 32;
-      q6k_pack(q, dst + pl.ql + i * 128, dst + pl.qh + i * 64);
-      for (int b = 0; b < 16; ++b) dst[pl.sc + i * 16 + b] = (uint8_t)sc[b / 2];
-      memcpy(dst + pl.d + i * 2, src + i * 110, 2);
+      const uint8_t* p = src + i * 110;
+      memcpy(dst + pl.d + i * 2, p, 2);
+      memcpy(dst + pl.qs + i * 64, p + 2, 64);
+      memcpy(dst + pl.hd + i * 12, p + 66, 8);
+      memcpy(dst + pl.sg + i * 32, p + 74, 32);
+      memcpy(dst + pl.hd + i * 12 + 8, p + 106, 4);
     }
     return 0;
   }
@@ -237,20 +220,15 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
     return 0;
   }
   if (type == GGML_TYPE_Q4_0) {
-    // Q4_0 is Q8_0 with q - 8 in four bits (reference src/quants.h:136-148: 18-byte blocks, f16 d, low nibbles =
-    // elements 0..15, high = 16..31): written out as Q8_0 planes, value for value, so every Q8_0 kernel serves it
-    // exactly, at 34 instead of 18 bytes per block on the device.
-    const PlanesQ80 pl = planes_q80(rows, nsb);
+    // eight 18-byte blocks (f16 d, 16 bytes of nibbles: low = elements 0..15, high = 16..31, value = nibble - 8;
+    // reference src/quants.h:136-148) -> 128 bytes of nibbles and 8 scales per superblock
+    const PlanesQ40 pl = planes_q40(rows, nsb);
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < u; ++i)
       for (int b = 0; b < 8; ++b) {
         const uint8_t* blk = src + i * 144 + 18 * b;
         memcpy(dst + pl.d + i * 16 + 2 * b, blk, 2);
-        int8_t* q = (int8_t*)(dst + pl.qs + i * 256 + 32 * b);
-        for (int e = 0; e < 16; ++e) {
-          q[e] = (int8_t)((blk[2 + e] & 0xF) - 8);
-          q[16 + e] = (int8_t)((blk[2 + e] >> 4) - 8);
-        }
+        memcpy(dst + pl.qs + i * 128 + 16 * b, blk + 2, 16);
       }
     return 0;
   }

@@ -25,6 +25,7 @@
 
 extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
 extern "C" size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
+extern "C" void arcz_iq3s_grid(uint32_t* out);
 
 // (zero/engine.h:27-34) raw = the device planes of all `rows` rows (an expert tensor holds n_expert * N rows)
 struct GpuWeight {
@@ -38,7 +39,8 @@ struct GpuWeight {
 };
 
 inline const char* ggml_type_name(uint32_t t) {
-  return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : t == GGML_IQ4_XS ? "IQ4_XS" : "?";
+  return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : t == GGML_IQ4_XS ? "IQ4_XS"
+         : t == GGML_Q4_0 ? "Q4_0" : t == GGML_IQ3_S ? "IQ3_S" : "?";
 }
 
 class Engine {
@@ -64,6 +66,30 @@ class Engine {
     sk_force_ = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : -1;
     sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
     sk_ws_ = buf(sk_ws_bytes_);
+    // the codebook tables the kernels take as `tabs` (the reference's tabs_, zero/engine_setup.h): IQ3_S's 512 entries
+    uint32_t grid[512];
+    arcz_iq3s_grid(grid);
+    tabs_ = buf(sizeof grid, grid);
+  }
+  cl_mem tabs_ = nullptr;
+  // IQ3_S in the GEMM forms (prefill chunks, expert tiles): the matrix is first written out as Q6_K planes, value for
+  // value, into xw_ -- the place of the reference's decode pass in front of its GEMM (zero/engine.h:1205-1250) -- and
+  // the Q6_K kernels run on that.  xw_ is sized when such a weight is uploaded (the largest one), never in a matmul.
+  cl_mem xw_ = nullptr;
+  size_t xw_bytes_ = 0;
+  GpuWeight gemm_form(const char* name, const GpuWeight& w) {
+    if (w.type != GGML_IQ3_S) return w;
+    const size_t need = raw_planes_bytes(QT_Q6_K, w.rows, w.K / 256);
+    if (need > xw_bytes_) throw std::logic_error("gemm_form: the expansion buffer is smaller than the weight");
+    cl_kernel k = kernel("decode", "", "expand_iq3s");
+    int rows = (int)w.rows, nsb = w.K / 256;
+    set_args(k, 0, w.raw, xw_, tabs_, rows, nsb);
+    size_t g1 = ((size_t)rows * nsb + 3) / 4 * 256, l1 = 256;
+    run(name, k, 1, &g1, &l1);
+    GpuWeight x = w;
+    x.type = GGML_Q6_K;
+    x.raw = xw_;
+    return x;
   }
   // (zero/engine_alloc.h:10, 39, 41: twice the size with two-pass matmul inputs, the residual's half behind the first)
   void alloc_activations() {
@@ -175,10 +201,9 @@ class Engine {
     if (nbytes != arcz_gguf_bytes(type, rows, K))
       throw std::runtime_error("make_weight: " + std::to_string(nbytes) + " bytes given, " +
                                std::to_string(arcz_gguf_bytes(type, rows, K)) + " expected");
+    if (rows * (size_t)(K / 256) >= (1ull << 31)) throw std::runtime_error("make_weight: too many superblocks for one tensor");
     GpuWeight w;
-    // (Q4_0 rows become Q8_0 planes on upload, IQ3_S rows Q6_K planes, value for value -- arcz_repack_planes -- and run
-    //  through those kernels)
-    w.type = type == GGML_Q4_0 ? GGML_Q8_0 : type == GGML_IQ3_S ? GGML_Q6_K : type;
+    w.type = type;
     w.N = N;
     w.K = K;
     w.rows = rows;
@@ -186,6 +211,16 @@ class Engine {
     std::vector<uint8_t> planes(pb);
     if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
     w.raw = buf(pb, planes.data());
+    if (type == GGML_IQ3_S) {  // (room for its GEMM form)
+      const size_t need = raw_planes_bytes(QT_Q6_K, rows, K / 256);
+      if (need > xw_bytes_) {
+        if (xw_) release(xw_);
+        xw_ = nullptr;
+        xw_bytes_ = 0;
+        xw_ = buf(need);
+        xw_bytes_ = need;
+      }
+    }
     return w;
   }
   void free_weight(GpuWeight& w) {
@@ -372,7 +407,7 @@ class Engine {
         arcz_mem_size(C) < ((size_t)(rows_out - 1) * (cur_T_ == 1 ? 0 : ldc) + c_off + w.N) * 4)
       throw std::runtime_error(std::string("matmul ") + name + ": the output does not fit C");
     int a = acc;
-    cl_mem tabs = nullptr;  // (the reference's codebook tables: none of the three types has one)
+    cl_mem tabs = tabs_;  // (the reference's codebook tables; IQ3_S's kernels read theirs from it)
     // Q4_K and a few tokens: the matrix-vector form on the matrix pipe (gemv_mm), K in slices of at most 24 superblocks
     // that accumulate.  It takes 9-16 tokens in chunks of 16 rows (what the reference pads them to, zero/engine.h:522;
     // the rows from T on come out as zeros, as the GEMM writes them: 27 against 95 us at 17408 x 5120), and 3-8 tokens
@@ -419,7 +454,8 @@ class Engine {
       const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= 65536;
       const int tbl = q2f ? tb2 : T <= 2 ? T : T <= 4 ? 4 : 8;
       const size_t lds = lds_of(tbl);
-      const bool fits = !force_v && lpr && lds <= 65536;
+      // (IQ3_S: its GEMV reads the weights straight into registers, the reference's gemv_v form)
+      const bool fits = !force_v && lpr && lds <= 65536 && w.type != GGML_IQ3_S;
       if (mm_ok && T >= 3 && (T >= 7 || !fits)) {
         rd_bytes -= raw_bytes(w);  // (counted by gemv_mm)
         gemv_mm();
@@ -468,7 +504,8 @@ class Engine {
   // rows of a pass.  ARCZ_GEMV_GU=0: never taken.
   bool gemv_gu(const GpuWeight& g, const GpuWeight& u, int Mp, cl_mem C) {
     static const bool off = getenv("ARCZ_GEMV_GU") && atoi(getenv("ARCZ_GEMV_GU")) == 0;
-    if (off || cur_T_ != 1 || q2mm_ || !g.raw || !u.raw || g.type != u.type || g.N != u.N || g.K != u.K) return false;
+    if (off || cur_T_ != 1 || q2mm_ || !g.raw || !u.raw || g.type != u.type || g.N != u.N || g.K != u.K || g.type == GGML_IQ3_S)
+      return false;
     if (g.K != cur_K_ || Mp != cur_Mp_)
       throw std::runtime_error("gemv_gu: the activations hold " + std::to_string(cur_Mp_) + " x " + std::to_string(cur_K_) +
                                ", the matrices take " + std::to_string(Mp) + " x " + std::to_string(g.K));
@@ -488,7 +525,7 @@ class Engine {
     const std::string defs = "-DQT=" + std::to_string(g.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" + std::to_string(pf) +
                              " -DLDS=" + std::to_string(lds) + " -DGU2";
     cl_kernel k = kernel("decode", defs, "gemv");
-    cl_mem tabs = nullptr;
+    cl_mem tabs = tabs_;
     int NN = N, KK = K, M = Mp, c_off = 0, a = 0;
     set_args(k, 0, g.raw, NN, KK, tabs, aq_, asc_, absum_, M, C, c_off, a, u.raw);
     const size_t wgs = std::min<size_t>((size_t)2 * N / gr, (size_t)arcz_device_cus() * 2);
@@ -504,7 +541,8 @@ class Engine {
   cl_mem sk_ws_ = nullptr;
   size_t sk_ws_bytes_ = 0;
   int sk_force_ = -1;  // ARCZ_Q4_SPLITK: 0 = never share K out, n >= 2: n pieces, -1 = the rule below
-  void gemm_dense(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int a) {
+  void gemm_dense(const char* name, const GpuWeight& w0, int Mp, cl_mem C, int ldc, int c_off, int a) {
+    const GpuWeight w = gemm_form(name, w0);
     int M = Mp, N = w.N, K = w.K;
     // Any type, a chunk so short that its tiles are fewer than two per compute unit: K is shared out over `ny`
     // work-groups per tile, which store partial tiles in a workspace, and splitk_reduce adds the slices in order (the
@@ -697,11 +735,12 @@ class Engine {
     const int E = L.E, F = L.F, NE = L.NE;
     for (int i = part; i < (part == 0 ? 2 : 3); ++i) {
       const int N = i == 2 ? E : F, K = i == 2 ? F : E;
-      cl_kernel k = gemm_kernel(L.ex[i].type, true, NE);
+      const GpuWeight wx = gemm_form(i == 2 ? "moe_down" : "moe_gateup", L.ex[i]);
+      cl_kernel k = gemm_kernel(wx.type, true, NE);
       int M = i == 2 ? slots_ : Mp, NN = N, KK = K, ldc = N, acc = i == 1 ? 2 : 0, e0 = 0, e1 = NE, um = i == 2 ? 0 : 1,
           us = i == 2 ? 1 : 0;
       cl_mem unused = nullptr;
-      set_args(k, 0, L.ex[i].raw, unused, i == 2 ? mhq_ : aq_, i == 2 ? mhsc_ : asc_, i == 2 ? mhbs_ : absum_, i == 2 ? my_ : mh_, M, NN, KK,
+      set_args(k, 0, wx.raw, unused, i == 2 ? mhq_ : aq_, i == 2 ? mhsc_ : asc_, i == 2 ? mhbs_ : absum_, i == 2 ? my_ : mh_, M, NN, KK,
                ldc, acc, mtiles_, mtstart_, e0, e1, stok_, um, swt_, us);
       size_t gws[2] = {(size_t)(N + 127) / 128 * 256, max_tiles}, lws[2] = {256, 1};
       run(i == 2 ? "moe_down" : "moe_gateup", k, 2, gws, lws);
@@ -765,7 +804,7 @@ class Engine {
         moe_route(L, rl, ldl, T, tmd);
         tiles_max = (size_t)(n + tmd - 1) / tmd + std::min(n, NE);
       }
-      cl_mem tabs = nullptr;
+      cl_mem tabs = tabs_;
       const std::string dd = " -DGROWS=2 -DTM=" + std::to_string(tmd) + " -DNE=" + std::to_string(NE);
       if (L.ex[0].type != L.ex[1].type) throw std::runtime_error("layer_moe: gate and up experts of different types");
       // Tiles of one or two slots: the gate/up kernel quantizes its own output (32 rows a work-group: one block per
@@ -903,6 +942,17 @@ inline std::string engine_self_check() {
           wq[b * 32 + i] = q;
         }
       }
+    } else if (type == GGML_Q4_0) {
+      for (int b = 0; b < 8; ++b) {
+        uint8_t* p = blk + 18 * b;
+        p[0] = 0x00; p[1] = 0x3C;  // f16 1.0
+        for (int i = 0; i < 16; ++i) {
+          const int lo = (int)(next() & 15u), hi = (int)(next() & 15u);
+          p[2 + i] = (uint8_t)(lo | hi << 4);
+          wq[b * 32 + i] = lo - 8;
+          wq[b * 32 + 16 + i] = hi - 8;
+        }
+      }
     } else if (type == GGML_Q4_K || type == GGML_Q5_K) {
       const bool q5 = type == GGML_Q5_K;
       memset(blk, 0, q5 ? 176 : 144);
@@ -962,7 +1012,7 @@ inline std::string engine_self_check() {
     cl_mem c0 = e.buf((size_t)M * N * 4), c1 = e.buf((size_t)M * N * 4);
     std::vector<float> y0((size_t)M * N), y1((size_t)M * N), cinit((size_t)M * N);
     for (auto& v : cinit) v = (float)((int)(next() % 9u) - 4);  // small integers: sums with them stay exact
-    for (uint32_t type : {GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ4_XS}) {
+    for (uint32_t type : {GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ4_XS, GGML_Q4_0}) {
       const size_t rb = arcz_gguf_bytes(type, 1, K), sbb = rb / (size_t)(K / 256);
       std::vector<uint8_t> w((size_t)N * rb);
       std::vector<int> wq((size_t)N * K);

@@ -11,6 +11,7 @@
     BLOB arcz_blob_ops, "ops.hsaco"
     BLOB arcz_blob_decode, "decode.hsaco"
     BLOB arcz_blob_decode_q80, "decode_q80.hsaco"
+    BLOB arcz_blob_decode_q40, "decode_q40.hsaco"
     BLOB arcz_blob_decode_q4k, "decode_q4k.hsaco"
     BLOB arcz_blob_decode_q5k, "decode_q5k.hsaco"
     BLOB arcz_blob_decode_q6k, "decode_q6k.hsaco"

@@ -12,10 +12,12 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 #endif
 
 // GGUF type ids (reference src/gguf.h:18-22)
+#define QT_Q4_0 2
 #define QT_Q8_0 8
 #define QT_Q4_K 12
 #define QT_Q5_K 13
 #define QT_Q6_K 14
+#define QT_IQ3_S 21
 #define QT_IQ4_XS 23
 
 // ---- device weight layout ("raw planes").  A matrix of R rows x K columns (K % 256 == 0, nsb = K / 256) is held
@@ -36,12 +38,22 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 //   IQ4_XS: qs [R][nsb][128]  (GGUF order: byte j of block b = element 32b+j low nibble, 32b+16+j high nibble; a nibble
 //                              is a code of the 16-entry table below), hdr [R][nsb][8] (f16 d, 16 bits of the eight
 //                              6-bit block scales' high parts, 4 bytes of their low nibbles: as GGUF)
+//   Q4_0 : qs  [R][nsb][128]  (the sixteen nibble bytes of each of the superblock's eight 32-value blocks, as GGUF: byte
+//                              j of block b = element 32b+j low nibble, 32b+16+j high nibble; value = nibble - 8),
+//          d   [R][nsb][8] (f16: the eight blocks' scales).  144 bytes per 256 values, as GGUF's eight 18-byte blocks.
+//   IQ3_S: qs  [R][nsb][64]   (the low bytes of the 64 codebook indices: 8 per 32-value block, each naming 4 magnitudes),
+//          sg  [R][nsb][32]   (sign bits: 4 bytes per block, bit e of the block's 32 = element e is negative),
+//          hd  [R][nsb][12]   (8 bytes of ninth index bits, bit g of byte b = index g of block b; 4 bytes of scale nibbles,
+//                              nibble b = s of block b, sub-scale 1 + 2 s),
+//          d   [R][nsb]       (f16).  110 bytes per 256 values, as GGUF (src/quants.h:240-262).
 // Plane offsets from the start of the buffer, in bytes (each a multiple of 256 when R * nsb is a multiple of 16;
 // always a multiple of 16 otherwise except as noted).
 struct PlanesQ4K { size_t qs, hdr, qh; };  // (qh: Q5_K only)
 struct PlanesQ6K { size_t ql, qh, sc, d; };
 struct PlanesQ80 { size_t qs, d; };
 struct PlanesIQ4XS { size_t qs, hdr; };
+struct PlanesQ40 { size_t qs, d; };
+struct PlanesIQ3S { size_t qs, sg, hd, d; };
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 __host__ __device__ inline PlanesQ4K planes_q4k(size_t rows, int nsb) {
@@ -72,8 +84,25 @@ __host__ __device__ inline PlanesIQ4XS planes_iq4xs(size_t rows, int nsb) {
   p.hdr = rows * (size_t)nsb * 128;
   return p;
 }
+__host__ __device__ inline PlanesQ40 planes_q40(size_t rows, int nsb) {
+  PlanesQ40 p;
+  p.qs = 0;
+  p.d = rows * (size_t)nsb * 128;
+  return p;
+}
+__host__ __device__ inline PlanesIQ3S planes_iq3s(size_t rows, int nsb) {
+  PlanesIQ3S p;
+  const size_t u = rows * (size_t)nsb;
+  p.qs = 0;
+  p.sg = u * 64;
+  p.hd = u * 96;
+  p.d = u * 108;
+  return p;
+}
 __host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb) {
   const size_t u = rows * (size_t)nsb;
+  if (qt == QT_IQ3_S) return align16(u * 110);
+  if (qt == QT_Q4_0) return u * 144;
   if (qt == QT_Q4_K) return u * 144;
   if (qt == QT_Q5_K) return u * 176;
   if (qt == QT_Q6_K) return align16(u * 208 + u * 2);
@@ -118,6 +147,18 @@ __device__ inline uint32_t iq4_lookup(uint32_t c) {
   const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, sel);  // codes 8-15
   const uint32_t m = ((c >> 3) & 0x01010101u) * 0xFFu;
   return (hi & m) | (lo & ~m);
+}
+
+// Q4_0: four nibbles, one in the low nibble of each byte of c (the other bits ignored), to the four int8 values
+// nibble - 8, without borrows between bytes.
+__device__ inline uint32_t q40_vals(uint32_t c) { return (((c & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
+
+// IQ3_S: four magnitudes (bytes of a codebook entry g) with the four sign bits s4 (bit j: byte j is negative) applied:
+// the bits are spread to the bytes' low bits by one multiply, and a byte is negated as (x ^ 0xFF) + 1 -- no carry
+// leaves a byte, the magnitudes being 1..15.
+__device__ inline uint32_t iq3s_signed4(uint32_t g, uint32_t s4) {
+  const uint32_t m = (s4 * 0x00204081u) & 0x01010101u;
+  return (g ^ (m * 0xFFu)) + m;
 }
 
 __device__ inline int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }

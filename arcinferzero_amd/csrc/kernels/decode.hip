@@ -20,6 +20,14 @@
 
 template <int QT> struct UnitsPerSb { static constexpr int v = QT == QT_Q8_0 ? 16 : 8; };
 
+// IQ3_S: the codebook (512 entries of four magnitudes 1, 3, ..., 15, one per byte; ggml's iq3s_grid) in LDS, copied from
+// the kernels' `tabs` argument once per work-group, before anything else (every thread of the work-group calls this).
+__shared__ uint32_t iq3s_grid_lds[512];
+__device__ inline void iq3s_grid_init(const uint32_t* __restrict__ tabs) {
+  for (int i = threadIdx.x; i < 512; i += blockDim.x) iq3s_grid_lds[i] = tabs[i];
+  __syncthreads();
+}
+
 // acc[r][t] += the products of plane rows rows[r] (absolute rows of planes that hold `plane_rows` rows) with the token
 // rows tok[t] of aq / asc / absum, this half wave's share (lane hl takes the 16-byte units hl, hl + 32, ...).
 // SPLIT < GROWS: rows[SPLIT..GROWS) are rows of a second set of planes of the same shape, raw2 (the gate and the up
@@ -127,6 +135,90 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
           i2 = dot4(w2[3], a2[t].w, i2);
           acc[r][t] += sa1[t] * d * (float)(sc1 * i1);
           acc[r][t] += sa2[t] * d * (float)(sc2 * i2);
+        }
+      }
+    }
+  } else if constexpr (QT == QT_IQ3_S) {
+    // a unit is one 32-value block: 8 codebook indices (9 bits: a byte and a bit of the block's ninth-bit byte), 32
+    // sign bits, one 4-bit scale s; value = +-(1, 3, ..., 15), sub-scale 1 + 2 s (zero/kernels/decode.cl:400-414)
+    const PlanesIQ3S pl = planes_iq3s(plane_rows, nsb);
+    const int ib = hl & 7;
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 3;
+      const int e1 = sb * 256 + 32 * ib;
+      uint4 a1[TB], a2[TB];
+      float sa[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
+        a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
+        a2[t] = *(const uint4*)(aq + (size_t)tt * K + e1 + 16);
+        sa[t] = asc[(size_t)(e1 >> 5) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const size_t n = rows[r];
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
+        const size_t rs = n * nsb + sb;
+        const uint2 q = *(const uint2*)(rb + pl.qs + rs * 64 + ib * 8);
+        const uint32_t sg = *(const uint32_t*)(rb + pl.sg + rs * 32 + ib * 4);
+        const uint32_t h9 = rb[pl.hd + rs * 12 + ib];
+        const uint32_t scb = rb[pl.hd + rs * 12 + 8 + (ib >> 1)];
+        const int sc = 1 + 2 * (int)((scb >> (4 * (ib & 1))) & 0xFu);
+        const float d = f16_bits_to_f32(*(const unsigned short*)(rb + pl.d + rs * 2));
+        uint32_t w[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const uint32_t idx = (((k < 4 ? q.x : q.y) >> (8 * (k & 3))) & 0xFFu) | (((h9 >> k) & 1u) << 8);
+          w[k] = iq3s_signed4(iq3s_grid_lds[idx], (sg >> (4 * k)) & 0xFu);
+        }
+#pragma unroll
+        for (int t = 0; t < TB; ++t) if (t < nt) {
+          int i1 = dot4(w[0], a1[t].x, 0);
+          i1 = dot4(w[1], a1[t].y, i1);
+          i1 = dot4(w[2], a1[t].z, i1);
+          i1 = dot4(w[3], a1[t].w, i1);
+          i1 = dot4(w[4], a2[t].x, i1);
+          i1 = dot4(w[5], a2[t].y, i1);
+          i1 = dot4(w[6], a2[t].z, i1);
+          i1 = dot4(w[7], a2[t].w, i1);
+          acc[r][t] += sa[t] * d * (float)(sc * i1);
+        }
+      }
+    }
+  } else if constexpr (QT == QT_Q4_0) {
+    const PlanesQ40 pl = planes_q40(plane_rows, nsb);
+    const int ib = hl & 7;  // a unit is one 32-block: low nibbles = its elements 0..15, high = 16..31, value = nibble - 8
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 3;
+      const int e1 = sb * 256 + 32 * ib;
+      uint4 a1[TB], a2[TB];
+      float sa[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
+        a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
+        a2[t] = *(const uint4*)(aq + (size_t)tt * K + e1 + 16);
+        sa[t] = asc[(size_t)(e1 >> 5) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const size_t n = rows[r];
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
+        const uint4 w = *(const uint4*)(rb + pl.qs + n * nsb * 128 + (size_t)u * 16);
+        const float d = f16_bits_to_f32(*(const unsigned short*)(rb + pl.d + (n * nsb * 8 + u) * 2));
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int t = 0; t < TB; ++t) if (t < nt) {
+          int i1 = dot4(q40_vals(ww[0]), a1[t].x, 0);
+          i1 = dot4(q40_vals(ww[1]), a1[t].y, i1);
+          i1 = dot4(q40_vals(ww[2]), a1[t].z, i1);
+          i1 = dot4(q40_vals(ww[3]), a1[t].w, i1);
+          i1 = dot4(q40_vals(ww[0] >> 4), a2[t].x, i1);
+          i1 = dot4(q40_vals(ww[1] >> 4), a2[t].y, i1);
+          i1 = dot4(q40_vals(ww[2] >> 4), a2[t].z, i1);
+          i1 = dot4(q40_vals(ww[3] >> 4), a2[t].w, i1);
+          acc[r][t] += sa[t] * d * (float)i1;   // (the 32-block in one conversion, as the reference's gemv: decode.cl:1003)
         }
       }
     }
@@ -248,6 +340,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
   extern "C" __global__ __launch_bounds__(256) void gemv_v__QT##QT##_GROWS##GROWS(                                      \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
       const short* absum, int M, float* C, int c_off, int accumulate, float softcap) {                                \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     gemv_body<QT, 1, GROWS>(raw, N, K, aq, asc, absum, M, 1, C, 0, c_off, accumulate, (size_t)N, softcap);           \
   }
 
@@ -256,6 +349,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
   extern "C" __global__ __launch_bounds__(256) void gemv_mt_v__QT##QT##_GROWS##GROWS##_TB##TB(                          \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
       const short* absum, int M, int T, float* C, int ldc, int c_off, int accumulate, float softcap) {                \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     gemv_body<QT, TB, GROWS>(raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, (size_t)N, softcap);        \
   }
 
@@ -271,6 +365,8 @@ GEMV_ALL(12)
 GEMV_ALL(13)
 GEMV_ALL(14)
 GEMV_ALL(23)
+GEMV_ALL(2)
+GEMV_ALL(21)
 
 // ---- the experts of a pass of a few tokens (the reference's per-tile kernels moe_gateup_q / moe_down_q,
 // zero/kernels/decode.cl, launched by zero/engine_moe.h:196-262 with tiles of TM = 1, 2, 4 or 8 slots for 1-8 tokens):
@@ -521,18 +617,21 @@ __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, in
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
       short* hbs, int NE) {                                                                                           \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     moe_gateup_quant_rows<QT, 1>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM2_QUANT1(                         \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
       short* hbs, int NE) {                                                                                           \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     moe_gateup_quant_rows<QT, 2>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM1_QUANT1_ROUTE1(                  \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, int* tiles, int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc, short* hbs,     \
       const float* logits, float* sgate, float* swt, int* inv, int NU, int ldl, int T, int* ids, float* wts, int NE) { \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     MoeRouteArgs ra;                                                                                                  \
     ra.logits = logits; ra.sgate = sgate; ra.swt = swt; ra.tiles_out = tiles; ra.stok_out = stok; ra.inv = inv;       \
     ra.NU = NU; ra.ldl = ldl; ra.T = T; ra.ids = ids; ra.wts = wts;                                                   \
@@ -541,6 +640,7 @@ __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, in
   extern "C" __global__ __launch_bounds__(256) void moe_down1_q__QT##QT##_GROWS4(                                     \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
       const int* tiles, const float* swt, float* x, const short* hbs, const int* inv, int NU, int NE) {              \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     moe_down1_rows<QT, 4>(raw, N, K, hq, hsc, hbs, S, tiles, swt, x, inv, NU, NE);                                   \
   }
 MOE_DECODE_FUSED_INST(8)
@@ -548,16 +648,20 @@ MOE_DECODE_FUSED_INST(12)
 MOE_DECODE_FUSED_INST(13)
 MOE_DECODE_FUSED_INST(14)
 MOE_DECODE_FUSED_INST(23)
+MOE_DECODE_FUSED_INST(2)
+MOE_DECODE_FUSED_INST(21)
 
 #define MOE_DECODE_INST(QT, TM)                                                                                      \
   extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS2_TM##TM(                             \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int NE) {                              \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     moe_gateup_rows<QT, TM, 2>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE);                                 \
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(256) void moe_down_q__QT##QT##_GROWS2_TM##TM(                               \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
       const int* tiles, const float* swt, float* y, const short* hbs, int NE) {                                      \
+    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
     moe_down_rows<QT, TM, 2>(raw, N, K, hq, hsc, hbs, S, tiles, swt, y, NE);                                         \
   }
 #define MOE_DECODE_ALL(QT) MOE_DECODE_INST(QT, 1) MOE_DECODE_INST(QT, 2) MOE_DECODE_INST(QT, 4) MOE_DECODE_INST(QT, 8)
@@ -566,3 +670,39 @@ MOE_DECODE_ALL(12)
 MOE_DECODE_ALL(13)
 MOE_DECODE_ALL(14)
 MOE_DECODE_ALL(23)
+MOE_DECODE_ALL(2)
+MOE_DECODE_ALL(21)
+
+// expand_iq3s: the IQ3_S planes of `rows` rows to Q6_K planes of the same rows, value for value -- the same f16 d, the
+// int8 sub-scale 1 + 2 s for both 16-value halves of a block, q = value + 32 in six bits -- for the prefill GEMM and
+// the expert-tile GEMM, which run their Q6_K kernels on the result (the place of the reference's decode pass in front
+// of its GEMM, zero/engine.h:1205-1250 with zero/kernels/decode.cl:183-478).  Thread (superblock, n, l) makes the bytes
+// ql[64 n + l], ql[64 n + 32 + l] and qh[32 n + l]: the values l of blocks 4 n .. 4 n + 3.
+// grid: ceil(rows * nsb / 4) work-groups of 256 (64 threads a superblock).
+extern "C" __global__ __launch_bounds__(256) void expand_iq3s(const uint8_t* __restrict__ raw, uint8_t* __restrict__ out,
+                                                              const uint32_t* __restrict__ tabs, int rows, int nsb) {
+  iq3s_grid_init(tabs);
+  const size_t total = (size_t)rows * nsb;
+  const size_t rs = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (rs >= total) return;
+  const PlanesIQ3S pi = planes_iq3s((size_t)rows, nsb);
+  const PlanesQ6K po = planes_q6k((size_t)rows, nsb);
+  const int n = (threadIdx.x >> 5) & 1, l = threadIdx.x & 31, gi = l >> 2, j = l & 3;
+  int q[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int ib = 4 * n + k;
+    const uint32_t idx = raw[pi.qs + rs * 64 + ib * 8 + gi] | ((((uint32_t)raw[pi.hd + rs * 12 + ib] >> gi) & 1u) << 8);
+    const int mag = (int)((iq3s_grid_lds[idx] >> (8 * j)) & 0xFFu);
+    const int neg = (raw[pi.sg + rs * 32 + ib * 4 + (l >> 3)] >> (l & 7)) & 1;
+    q[k] = (neg ? -mag : mag) + 32;
+  }
+  out[po.ql + rs * 128 + 64 * n + l] = (uint8_t)((q[0] & 15) | ((q[2] & 15) << 4));
+  out[po.ql + rs * 128 + 64 * n + 32 + l] = (uint8_t)((q[1] & 15) | ((q[3] & 15) << 4));
+  out[po.qh + rs * 64 + 32 * n + l] = (uint8_t)((q[0] >> 4) | ((q[1] >> 4) << 2) | ((q[2] >> 4) << 4) | ((q[3] >> 4) << 6));
+  if (n == 0 && l < 16) {
+    const int ib = l >> 1;
+    out[po.sc + rs * 16 + l] = (uint8_t)(1 + 2 * ((raw[pi.hd + rs * 12 + 8 + (ib >> 1)] >> (4 * (ib & 1))) & 0xF));
+  }
+  if (n == 1 && l < 2) out[po.d + rs * 2 + l] = raw[pi.d + rs * 2 + l];
+}

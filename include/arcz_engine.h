@@ -29,7 +29,8 @@ arcz_engine* arcz_engine_create(int max_chunk, int max_k);
 void arcz_engine_destroy(arcz_engine* e);
 
 /* make_weight + upload_padded (zero/engine_load.h:84-130, 157-196): N rows of K values as GGUF blocks of `type`
- * (2 = Q4_0, 8 = Q8_0, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K, 21 = IQ3_S, 23 = IQ4_XS), regrouped into the device layout and uploaded. */
+ * (2 = Q4_0, 8 = Q8_0, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K, 21 = IQ3_S, 23 = IQ4_XS), regrouped into the device layout -- every
+ * type in its own form, the GGUF byte count -- and uploaded. */
 arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, const void* gguf, size_t bytes);
 /* The same from a tensor of an open GGUF file (upload of zero/engine_load.h:84-196): a matrix (dims K, N) or an expert
  * tensor (dims K, N, experts) of type Q4_0 / Q8_0 / Q4_K / Q5_K / Q6_K / IQ3_S / IQ4_XS, by name; NULL + arcz_engine_error() when it is missing, of
@@ -156,6 +157,9 @@ uint64_t arcz_engine_rd_bytes(arcz_engine* e);
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K);
 int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* planes);
+/* The IQ3_S codebook (ggml's iq3s_grid, src/iq_tables.h:297) as the kernels take it in their `tabs` argument: 512 words,
+ * byte j of a word = magnitude j of the entry (1, 3, ..., 15). */
+void arcz_iq3s_grid(uint32_t* out512);
 /* quantize_rows_q8_0 (src/quants.h:429-442) and this library's own Q4_K / Q5_K / Q6_K / IQ4_XS / IQ3_S block makers (input generators). */
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out);
 void arcz_gen_normal(uint64_t seed, size_t n, float mean, float std, float* out);

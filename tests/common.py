@@ -5,8 +5,14 @@ import numpy as np
 import arcinferzero_amd as az
 import oracle_lib as orc
 
-Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K, az.IQ4_XS
+import os
+
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS, Q4_0, IQ3_S = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K, az.IQ4_XS, az.Q4_0, az.IQ3_S
 TYPES = (Q8_0, Q4_K, Q6_K, Q5_K, IQ4_XS)
+ALL_TYPES = TYPES + (Q4_0, IQ3_S)     # with the two types the golden files of the first five do not cover
+# the IQ3_S codebook as the compiled reference decodes it (a golden vector): 512 entries of four magnitudes
+IQ3S_GRID = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors_types2.npz"))[
+    "iq3s_grid_dequant"].reshape(512, 4).astype(np.int64)
 TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS", az.IQ3_S: "IQ3_S", az.Q4_0: "Q4_0"}
 IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64)
 
@@ -83,6 +89,23 @@ def unit_scale_weights(qtype, N, K, seed):
         blk[..., 4:8] = 0x11
         blk[..., 8:] = (c[..., :16] | (c[..., 16:] << 4)).astype(np.uint8).reshape(N, nsb, 128)
         return blk.reshape(-1), IQ4_VALUES[c].reshape(N, K)
+    if qtype == Q4_0:
+        q = rng.integers(0, 16, size=(N, nsb * 8, 32), dtype=np.int64)
+        blk = np.zeros((N, nsb * 8, 18), np.uint8)
+        blk[..., 0:2] = one
+        blk[..., 2:] = (q[..., :16] | (q[..., 16:] << 4)).astype(np.uint8)
+        return blk.reshape(-1), (q - 8).reshape(N, K)
+    if qtype == IQ3_S:
+        # d = 1, every 4-bit scale 0 (sub-scale 1): values = the codebook's magnitudes with random signs
+        idx = rng.integers(0, 512, size=(N, nsb, 8, 8), dtype=np.int64)            # [block][group of 4]
+        sg = rng.integers(0, 2, size=(N, nsb, 8, 32), dtype=np.int64)              # sign bit per value
+        blk = np.zeros((N, nsb, 110), np.uint8)
+        blk[..., 0:2] = one
+        blk[..., 2:66] = (idx & 255).astype(np.uint8).reshape(N, nsb, 64)
+        blk[..., 66:74] = ((idx >> 8) << np.arange(8)).sum(axis=-1).astype(np.uint8)
+        blk[..., 74:106] = (sg.reshape(N, nsb, 8, 4, 8) << np.arange(8)).sum(axis=-1).astype(np.uint8).reshape(N, nsb, 32)
+        vals = IQ3S_GRID[idx].reshape(N, nsb, 8, 32) * (1 - 2 * sg)
+        return blk.reshape(-1), vals.reshape(N, K)
     if qtype == Q6_K:
         q = rng.integers(0, 64, size=(N, nsb, 256), dtype=np.int64)
         blk = np.zeros((N, nsb, 210), np.uint8)

@@ -5,7 +5,7 @@ import pytest
 
 import arcinferzero_amd as az
 import oracle_lib as orc
-from common import (TYPES, TYPE_NAMES, make_acts, make_weights, mixed_err, quantize_padded, rel_err_rows,
+from common import (ALL_TYPES, TYPES, TYPE_NAMES, make_acts, make_weights, mixed_err, quantize_padded, rel_err_rows,
                     unit_scale_acts, unit_scale_weights)
 
 pytestmark = pytest.mark.gpu
@@ -39,7 +39,7 @@ def run_gemm(eng, qtype, W, N, K, x, Mp, acc=0, c_init=None, ldc=None, c_off=0):
     return y
 
 
-@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("qtype", ALL_TYPES)
 @pytest.mark.parametrize("T,Mp,N,K", [(16, 16, 64, 256), (100, 112, 272, 512), (128, 128, 128, 1024), (300, 384, 384, 768),
                                       (180, 192, 520, 512)])
 def test_gemm_vs_oracle(eng, qtype, T, Mp, N, K):
@@ -60,7 +60,7 @@ def test_gemm_vs_oracle(eng, qtype, T, Mp, N, K):
     assert np.array_equal(y.view(np.uint32), y2.view(np.uint32))   # bit-identical run to run
 
 
-@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_gemm_block_sums_exact(eng, qtype):
     T, N, K = 160, 160, 512
     W, wi = unit_scale_weights(qtype, N, K, seed=15)
@@ -71,7 +71,7 @@ def test_gemm_block_sums_exact(eng, qtype):
     assert np.array_equal(y, exact.astype(np.float32))
 
 
-@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_gemm_matches_gemv(eng, qtype):
     """Rows 0..7 of a 16-row GEMM against the 8-token GEMV on the same inputs: both within tolerance of the same
     reference and of each other."""

@@ -10,7 +10,7 @@ import pytest
 
 import arcinferzero_amd as az
 import oracle_lib as orc
-from common import (TYPES, TYPE_NAMES, make_acts, make_weights, mixed_err, quantize_padded, rel_err_rows,
+from common import (ALL_TYPES, TYPES, TYPE_NAMES, make_acts, make_weights, mixed_err, quantize_padded, rel_err_rows,
                     unit_scale_acts, unit_scale_weights)
 
 pytestmark = pytest.mark.gpu
@@ -44,7 +44,7 @@ def run_gemv(eng, qtype, W, N, K, x, Mp, acc=0, c_init=None, ldc=None, c_off=0):
     return y
 
 
-@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("qtype", ALL_TYPES)
 @pytest.mark.parametrize("T", [1, 2, 3, 5, 8])
 def test_gemv_small_vs_oracle(eng, qtype, T):
     N, K, Mp = 264, 512, 16   # N not a multiple of the rows per work-group
@@ -61,7 +61,7 @@ def test_gemv_small_vs_oracle(eng, qtype, T):
     print(f"  rel {rel_err_rows(y, ref).max():.2e} mixed {mixed_err(y, ref):.2e} vs formula {rel_err_rows(y, form).max():.2e}")
 
 
-@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("qtype", ALL_TYPES)
 @pytest.mark.parametrize("T", [1, 2, 7])
 def test_gemv_block_sums_exact(eng, qtype, T):
     """Unit scales: the f32 output must be the exact integer dot product (all partial sums stay below 2^24)."""

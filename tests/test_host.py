@@ -10,7 +10,7 @@ import pytest
 
 import arcinferzero_amd as az
 import oracle_lib as orc
-from common import TYPES, make_weights
+from common import ALL_TYPES, TYPES, make_weights
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -47,7 +47,7 @@ def test_no_device_fails_loudly():
     assert "engine refused" in r.stdout
 
 
-@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_repack_planes_layout(qtype):
     rows, K = 6, 768
     nsb = K // 256
@@ -99,6 +99,17 @@ def test_repack_planes_layout(qtype):
         sb = W.reshape(u, 136)
         assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 8:]) and np.array_equal(P[u * 128:u * 136].reshape(u, 8), sb[:, :8])
         assert not P[u * 136:].any() and P.size % 16 == 0
+    elif qtype == az.Q4_0:
+        blk = W.reshape(u, 8, 18)                                            # eight 18-byte blocks: f16 d, 16 nibble bytes
+        assert P.size == W.size == u * 144
+        assert np.array_equal(P[:u * 128].reshape(u, 8, 16), blk[:, :, 2:]) and np.array_equal(P[u * 128:].reshape(u, 8, 2), blk[:, :, :2])
+    elif qtype == az.IQ3_S:
+        sb = W.reshape(u, 110)                                               # d, 64 index bytes, 8 ninth-bit bytes, 32 sign bytes, 4 scale bytes
+        assert P.size == (W.size + 15) // 16 * 16
+        assert np.array_equal(P[:u * 64].reshape(u, 64), sb[:, 2:66]) and np.array_equal(P[u * 64:u * 96].reshape(u, 32), sb[:, 74:106])
+        hd = P[u * 96:u * 108].reshape(u, 12)
+        assert np.array_equal(hd[:, :8], sb[:, 66:74]) and np.array_equal(hd[:, 8:], sb[:, 106:110])
+        assert np.array_equal(P[u * 108:u * 110].reshape(u, 2), sb[:, :2]) and not P[u * 110:].any()
     else:
         blk = W.reshape(u, 8, 34)
         assert np.array_equal(P[:u * 256].reshape(u, 8, 32), blk[:, :, 2:]) and np.array_equal(P[u * 256:].reshape(u, 8, 2), blk[:, :, :2])

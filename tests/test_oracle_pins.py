@@ -197,9 +197,10 @@ def test_iq3s_golden_with_whole_codebook():
     v = got.reshape(512, 4)
     assert set(np.unique(v)) == {1.0, 3.0, 5.0, 7.0, 9.0, 11.0, 13.0, 15.0}
     assert len({tuple(r) for r in v}) == 512          # (all entries differ)
-    # the product's own copy of the codebook: the device planes of the same blocks are Q6_K planes holding value + 32
-    planes = az.repack_planes(az.IQ3_S, 1, 2048, G["iq3s_grid_raw"])
-    assert np.array_equal(planes, az.repack_planes(az.Q6_K, 1, 2048, _iq3s_as_q6k(G["iq3s_grid_raw"], 1, 2048)))
+    # the product's own copy of the codebook, as its kernels take it (512 words, magnitude j of an entry in byte j)
+    grid = np.zeros(512, np.uint32)
+    az.lib.arcz_iq3s_grid(grid.ctypes.data_as(C.c_void_p))
+    assert np.array_equal(grid.view(np.uint8).reshape(512, 4), v.astype(np.uint8))
 
 
 def _iq3s_as_q6k(W3, N, K):
@@ -231,11 +232,9 @@ def test_iq3s_vs_compiled_reference():
     R = R.reshape(-1)
     assert np.array_equal(orc.dequant_rows(orc.IQ3_S, R, 16, 1024).view(np.uint32),
                           orc.dequant_rows(orc.IQ3_S, R, 16, 1024, lib=orc.ref).view(np.uint32))
-    # the Q6_K superblocks the device planes stand for decode to the same f32 values, bit for bit
+    # the Q6_K superblocks the GEMM forms expand the matrix to decode to the same f32 values, bit for bit
     assert np.array_equal(orc.dequant_rows(Q6_K, _iq3s_as_q6k(R, 16, 1024), 16, 1024).view(np.uint32),
                           orc.dequant_rows(orc.IQ3_S, R, 16, 1024).view(np.uint32))
-    assert np.array_equal(az.repack_planes(az.IQ3_S, 16, 1024, R),
-                          az.repack_planes(az.Q6_K, 16, 1024, _iq3s_as_q6k(R, 16, 1024)))
 
 
 def test_q6k_closed_form():
@@ -318,8 +317,9 @@ def test_q40_vs_compiled_reference():
     assert np.array_equal(az.quantize_rows(az.Q4_0, w), b)
     planes = az.repack_planes(az.Q4_0, 16, 512, a)
     nsb = 2
-    qs = planes[:16 * nsb * 256].view(np.int8).reshape(16, nsb * 8, 32).astype(np.float32)
-    dd = planes[16 * nsb * 256:16 * nsb * 256 + 16 * nsb * 16].view(np.float16).reshape(16, nsb * 8, 1).astype(np.float32)
+    nib = planes[:16 * nsb * 128].reshape(16, nsb * 8, 16)                      # a block's 16 nibble bytes
+    qs = np.concatenate([nib & 0xF, nib >> 4], axis=2).astype(np.float32) - 8.0   # low nibbles: values 0..15, high: 16..31
+    dd = planes[16 * nsb * 128:].view(np.float16).reshape(16, nsb * 8, 1).astype(np.float32)
     assert np.array_equal((qs * dd).reshape(16, 512), orc.dequant_rows(az.Q4_0, a, 16, 512))
 
 
