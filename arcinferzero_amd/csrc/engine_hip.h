@@ -664,8 +664,9 @@ class Engine {
   cl_mem mids_ = nullptr, mwts_ = nullptr, sgate_ = nullptr, mcount_ = nullptr, moffs_ = nullptr, mcursor_ = nullptr,
          mtiles_ = nullptr, mtstart_ = nullptr, stok_ = nullptr, swt_ = nullptr, minv_ = nullptr, mh_ = nullptr,
          mhq_ = nullptr, mhsc_ = nullptr, mhbs_ = nullptr, my_ = nullptr;
-  // copies of the per-expert counters that moe_route spreads its atomic adds over (moe_scan sums them)
-  static constexpr int kCountCopies = 64;
+  // The pair list is sorted in chunks of moe_tpc_ tokens (at most 512 pairs): counters [chunks][NE]
+  int moe_tpc_ = 0;
+  int moe_chunks(int T) const { return (T + moe_tpc_ - 1) / moe_tpc_; }
   int slots_ = 0, moe_ne_ = 0, moe_nu_ = 0, moe_e_ = 0, moe_f_ = 0;
 
   void moe_alloc(int NE, int NU, int E, int F) {
@@ -677,12 +678,15 @@ class Engine {
     slots_ = max_chunk * NU;
     const size_t S = (size_t)slots_;
     mids_ = buf(S * 4); mwts_ = buf(S * 4); sgate_ = buf((size_t)max_chunk * 4);
-    mcount_ = buf((size_t)kCountCopies * NE * 4); moffs_ = buf((size_t)NE * 4); mcursor_ = buf((size_t)NE * 4);
+    moe_tpc_ = std::max(4, (512 / NU) & ~3);  // (a multiple of the 4 tokens of a routing work-group)
+    if (moe_tpc_ * NU > 512) throw std::runtime_error("moe_alloc: more than 128 experts per token");
+    const size_t nchunks = (size_t)moe_chunks(max_chunk);
+    mcount_ = buf(nchunks * NE * 4); moffs_ = buf((size_t)NE * 4); mcursor_ = buf((size_t)NE * 4);
     mtiles_ = buf((1 + 3 * (S + NE)) * 4); mtstart_ = buf((size_t)(NE + 1) * 4);
     stok_ = buf(S * 4); swt_ = buf(S * 4); minv_ = buf(S * 4);
     mh_ = buf(S * F * 4); mhq_ = buf(S * F); mhsc_ = buf(S * (F / 32) * 4); mhbs_ = buf(S * (F / 16) * 2); my_ = buf(S * E * 4);
     const uint32_t zero = 0;
-    CL_CHECK(clEnqueueFillBuffer(cl_.queue, mcount_, &zero, 4, 0, (size_t)kCountCopies * NE * 4, 0, nullptr, nullptr));
+    CL_CHECK(clEnqueueFillBuffer(cl_.queue, mcount_, &zero, 4, 0, nchunks * NE * 4, 0, nullptr, nullptr));
   }
 
   MoeLayer make_moe_layer(uint32_t type, const uint8_t* gate, const uint8_t* up, const uint8_t* down, int NE, int NU,
@@ -703,7 +707,7 @@ class Engine {
     if (T <= 0 || T > max_chunk || ldl < NE || arcz_mem_size(rl) < ((size_t)(T - 1) * ldl + NE) * 4)
       throw std::runtime_error("moe_route: router logits do not fit");
     const std::string defs = "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DTM=" + std::to_string(tm) +
-                             " -DNPART=" + std::to_string(kCountCopies);
+                             " -DNPART=" + std::to_string(moe_tpc_) + " -DNCH=" + std::to_string(moe_chunks(T));
     {
       cl_kernel k = kernel("moe", defs + L.route_defs(), "moe_route");
       int NR = ldl, TT = T;
@@ -722,8 +726,8 @@ class Engine {
     {
       cl_kernel k = kernel("moe", defs, "moe_scatter");
       int nn = n;
-      set_args(k, 0, mids_, mwts_, nn, mcursor_, stok_, swt_, minv_);
-      size_t g1 = (size_t)NE * 256, l1 = 256;
+      set_args(k, 0, mids_, mwts_, nn, mcount_, stok_, swt_, minv_);  // (the cursor: the chunks' first slots per expert)
+      size_t g1 = (size_t)moe_chunks(T) * 512, l1 = 512;
       run("moe_scatter", k, 1, &g1, &l1);
     }
   }

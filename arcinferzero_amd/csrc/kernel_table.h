@@ -70,8 +70,8 @@ static const KernelSpec kKernelTable[] = {
      {{"NE", 0, true}, {"NU", 0, true}, {"HAS_GATE", 0, false}, {nullptr, 0, false}}, 64},
     {"moe", "moe_route_small", nullptr, "piippppppp", {nullptr},
      {{"NE", 0, true}, {"NU", 0, true}, {"TM", 16, false}, {nullptr, 0, false}}, 512},
-    {"moe", "moe_scan", nullptr, "ppppp", {nullptr}, {{"NE", 0, true}, {"TM", 16, false}, {"NPART", 1, false}, {nullptr, 0, false}}, 1024},
-    {"moe", "moe_scatter", nullptr, "ppipppp", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},
+    {"moe", "moe_scan", nullptr, "ppppp", {nullptr}, {{"NE", 0, true}, {"TM", 16, false}, {"NCH", 1, false}, {nullptr, 0, false}}, 1024},
+    {"moe", "moe_scatter", nullptr, "ppipppp", {nullptr}, {{"NU", 0, true}, {"NE", 0, true}, {"NPART", 0, true}, {nullptr, 0, false}}, 512},
     {"moe", "moe_quant", nullptr, "piipp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_quant_sums", nullptr, "piippp", {nullptr}, {{"FV", 1 << 30, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_combine", nullptr, "pppppi", {nullptr}, {{"NU", 0, true}, {nullptr, 0, false}}, 256},

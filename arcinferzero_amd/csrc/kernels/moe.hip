@@ -7,7 +7,8 @@
 
 
 // moe_route: one wave per token.  The NU largest of NE logits (ties: the lower expert), p = exp(l - max),
-// weights p / sum of the selected p; counts[copy][e]++ per selection (NPART copies [NPART][NE], 1 by default); sgate[t] = sigmoid(logit NE) when the row holds one.
+// weights p / sum of the selected p; counts[t / NPART][e]++ per selection (NPART: the tokens of a chunk of the pair
+// list, see moe_scan); sgate[t] = sigmoid(logit NE) when the row holds one.
 // grid: ceil(T / 4) work-groups of 256 threads.
 __device__ inline void moe_route_body(const float* __restrict__ logits, int ldl, int T, int* __restrict__ ids,
                                       float* __restrict__ wts, float* __restrict__ sgate, int* __restrict__ counts,
@@ -22,9 +23,8 @@ __device__ inline void moe_route_body(const float* __restrict__ logits, int ldl,
   if (lane < NU) {
     ids[(size_t)t * NU + lane] = mysel;
     wts[(size_t)t * NU + lane] = mywt;
-    // (NPART copies of the counters, a work-group adding to copy blockIdx % NPART: many adds to one word from all
-    //  over the chip queue up at the memory side; moe_scan sums the copies)
-    atomicAdd(&counts[(size_t)(blockIdx.x % NPART) * NE + mysel], 1);
+    // (the counters of the token's chunk: many adds to one word from all over the chip queue up at the memory side)
+    atomicAdd(&counts[(size_t)(t / NPART) * NE + mysel], 1);
   }
   if (lane == 0 && sgate) sgate[t] = route_sgate(lg, NE, ldl > NE, rv);
 }
@@ -176,108 +176,121 @@ extern "C" __global__ __launch_bounds__(512) void moe_route_small(const float* _
   }
 }
 
-// moe_scan: exclusive scan of the counts -> offs / cursor; the tile list tiles[0] = number of tiles, then (expert,
-// first slot, rows <= TM) per tile; tstart[e] = first tile of expert e, tstart[NE] = the tile count; counts (all NPART copies) reset.
-// One work-group of 1024 threads (NE <= 1024).
+// The grouping of the (token, expert) pairs by expert is a counting sort over chunks of the pair list.  moe_route counts
+// the pairs of each expert per chunk of TPC tokens (counts [chunks][NE]: the adds of a chunk go to words of its own, so
+// the many adds of a long prompt do not queue up on NE words); moe_scan turns the counts into each chunk's first slot
+// per expert; moe_scatter places a chunk's pairs.  Pair i of expert e lands at offs[e] + (pairs of e before i), so the
+// layout is the pair order within each expert: the same on every run (the reference draws slots from an atomic
+// counter, zero/kernels/moe.cl:171-179; its results do not depend on the order, its layout does).
+
+// moe_scan: counts [NCH][NE] (NCH = the chunks of this call, from n pairs of NU per token and TPC tokens a chunk) ->
+// offs[e] / cursor[e] (first slot of expert e), the tile list tiles[0] = number of tiles then (expert, first slot,
+// rows <= TM) per tile, tstart[e] = first tile of expert e, tstart[NE] = the tile count; and in place of each count the
+// chunk's first slot for that expert, counts[c][e] = offs[e] + pairs of e in chunks before c.
+// One work-group of 1024 threads, NE <= 512: thread (p, e) = (tid / NE, tid % NE) sums the chunks c = p, p + P, ...
+// (P = 1024 / NE), the experts' totals are scanned by waves (shuffles, one meeting), then every thread walks its chunks
+// again.  The two walks are dependent chains of at most ceil(NCH / P) loads.
 extern "C" __global__ __launch_bounds__(1024) void moe_scan(int* __restrict__ counts, int* __restrict__ offs,
                                                             int* __restrict__ cursor, int* __restrict__ tiles,
-                                                            int* __restrict__ tstart, int NE, int TM, int NPART) {
-  __shared__ int a[1024], b[1024];
-  const int e = threadIdx.x;
-  // the copies moe_route counted into, summed (integer adds in LDS: any order gives the same sums) and reset
-  a[e] = 0;
+                                                            int* __restrict__ tstart, int NE, int TM, int NCH) {
+  __shared__ int part[1024];      // [p][e]: pairs of expert e in the chunks of part p
+  __shared__ int wsum[2][16];     // per wave: experts' pair and tile totals
+  __shared__ int eoff[512];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int P = 1024 / NE, p = tid / NE, e = tid - p * NE;
+  const bool live = p < P;
+  // chunks are dealt to the parts in runs: part p takes chunks [p * cpp, min(NCH, (p + 1) * cpp))
+  const int cpp = (NCH + P - 1) / P, c0 = p * cpp, c1 = min(NCH, c0 + cpp);
+  // (the first eight chunks' counts are read together, one memory latency, and kept for the second walk)
+  int v8[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v8[k] = live && c0 + k < c1 ? counts[(size_t)(c0 + k) * NE + e] : 0;
+  int tot = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) tot += v8[k];
+  if (live)
+    for (int c = c0 + 8; c < c1; ++c) tot += counts[(size_t)c * NE + e];
+  part[tid] = live ? tot : 0;
   __syncthreads();
-  for (int i = e; i < NPART * NE; i += 1024) {
-    atomicAdd(&a[i % NE], counts[i]);
-    counts[i] = 0;
+  // experts' totals and tile counts, scanned: thread e < NE
+  int c = 0, nt = 0;
+  if (tid < NE) {
+    for (int q = 0; q < P; ++q) c += part[q * NE + tid];
+    nt = (c + TM - 1) / TM;
+  }
+  int ic = c, it = nt;  // inclusive scans within the wave
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int oc = __shfl_up(ic, d, 64), ot = __shfl_up(it, d, 64);
+    if (lane >= d) { ic += oc; it += ot; }
+  }
+  if (lane == 63) { wsum[0][wave] = ic; wsum[1][wave] = it; }
+  __syncthreads();
+  if (tid < NE) {
+    int bc = 0, bt = 0;
+    for (int w = 0; w < wave; ++w) { bc += wsum[0][w]; bt += wsum[1][w]; }
+    const int off = bc + ic - c, toff = bt + it - nt;
+    offs[tid] = off;
+    cursor[tid] = off;
+    tstart[tid] = toff;
+    eoff[tid] = off;
+    if (tid == NE - 1) tiles[0] = tstart[NE] = toff + nt;
+    for (int i = 0; i < nt; ++i) {
+      int* tp = tiles + 1 + 3 * (toff + i);
+      tp[0] = tid;
+      tp[1] = off + i * TM;
+      tp[2] = min(TM, c - i * TM);
+    }
   }
   __syncthreads();
-  const int c = e < NE ? a[e] : 0, nt = (c + TM - 1) / TM;
-  __syncthreads();
-  a[e] = c;
-  b[e] = nt;
-  __syncthreads();
-  for (int d = 1; d < 1024; d <<= 1) {
-    const int x = e >= d ? a[e - d] : 0, y = e >= d ? b[e - d] : 0;
-    __syncthreads();
-    a[e] += x;
-    b[e] += y;
-    __syncthreads();
-  }
-  if (e >= NE) return;
-  const int off = a[e] - c, toff = b[e] - nt;
-  offs[e] = off;
-  cursor[e] = off;
-  tstart[e] = toff;
-  if (e == NE - 1) tiles[0] = tstart[NE] = b[e];
-  for (int i = 0; i < nt; ++i) {
-    int* tp = tiles + 1 + 3 * (toff + i);
-    tp[0] = e;
-    tp[1] = off + i * TM;
-    tp[2] = min(TM, c - i * TM);
+  if (live) {
+    int base = eoff[e];
+    for (int q = 0; q < p; ++q) base += part[q * NE + e];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (c0 + k < c1) {
+        counts[(size_t)(c0 + k) * NE + e] = base;
+        base += v8[k];
+      }
+    for (int cc = c0 + 8; cc < c1; ++cc) {
+      const int v = counts[(size_t)cc * NE + e];
+      counts[(size_t)cc * NE + e] = base;
+      base += v;
+    }
   }
 }
 
-// moe_scatter: places pair i = (token i / NU, expert ids[i]) in a slot of its expert's range, in pair order: the
-// k-th pair of expert e (counting i upwards) gets slot offs[e] + k, so the layout is the same on every run (the
-// reference draws slots from an atomic counter; its results do not depend on the order, its layout does).
-// One work-group of 256 threads per expert, each scanning all n pairs.  `cursor` holds offs (as moe_scan wrote it).
-// The list is taken in pieces of 256 * SCAT_IT pairs: first every wave counts its matches in each 256-pair step of the
-// piece (no barrier between steps), then one scan over the (step, wave) counts gives every wave its first rank in
-// every step, then the steps are run again and the pairs written.
-#define SCAT_IT 32
-extern "C" __global__ __launch_bounds__(256) void moe_scatter(const int* __restrict__ ids, const float* __restrict__ wts,
+// moe_scatter: work-group c places the pairs of chunk c (at most 512: TPC tokens of NU pairs).  Thread i takes pair
+// i0 + i = (token, expert e): its slot is the chunk's first slot for e (cursor [chunks][NE], as moe_scan left it) plus
+// the number of earlier pairs of e in the chunk, counted from the chunk's expert list in LDS four entries a read.  The
+// chunk's row of `cursor` is cleared for the next layer's counts.  grid: chunks x 512 threads.
+extern "C" __global__ __launch_bounds__(512) void moe_scatter(const int* __restrict__ ids, const float* __restrict__ wts,
                                                               int n, int* __restrict__ cursor, int* __restrict__ stok,
-                                                              float* __restrict__ swt, int* __restrict__ inv, int NU) {
-  __shared__ int cnt[SCAT_IT * 4];  // matches of wave w in step j at [4 j + w], then their exclusive prefix sums
-  __shared__ int wtot[4];
-  const int e = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  int base = cursor[e];
-  for (int p0 = 0; p0 < n; p0 += 256 * SCAT_IT) {
-    int my[SCAT_IT];  // the thread's pairs of the piece, all loads in flight together
-#pragma unroll
-    for (int j = 0; j < SCAT_IT; ++j) {
-      const int i = p0 + j * 256 + t;
-      my[j] = i < n ? ids[i] : -1;
+                                                              float* __restrict__ swt, int* __restrict__ inv, int NU,
+                                                              int NE, int TPC) {
+  __shared__ __attribute__((aligned(16))) int sid[512];
+  const int i = threadIdx.x, i0 = blockIdx.x * TPC * NU, m = min(n - i0, TPC * NU);
+  int e = 0x7FFFFFFF;  // (past the chunk's pairs: an expert no pair has)
+  if (i < m) e = ids[i0 + i];
+  sid[i] = e;
+  int base = 0;
+  if (i < m) base = cursor[(size_t)blockIdx.x * NE + e];
+  __syncthreads();
+  if (i < m) {
+    int rank = 0;
+    const int full = i & ~3;
+    for (int j = 0; j < full; j += 4) {
+      const int4 q = *(const int4*)&sid[j];
+      rank += (q.x == e) + (q.y == e) + (q.z == e) + (q.w == e);
     }
-#pragma unroll
-    for (int j = 0; j < SCAT_IT; ++j) {
-      const unsigned long long bal = __ballot(my[j] == e);
-      if (lane == 0) cnt[4 * j + wave] = __popcll(bal);
-    }
-    __syncthreads();
-    // exclusive scan of cnt[0 .. 4 SCAT_IT): threads 0-63 own entries 2 t, 2 t + 1, the rest none
-    int c0 = 0, c1 = 0;
-    if (t < 2 * SCAT_IT) { c0 = cnt[2 * t]; c1 = cnt[2 * t + 1]; }
-    int incl = c0 + c1;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int o = __shfl_up(incl, d, 64);
-      if (lane >= d) incl += o;
-    }
-    if (lane == 63) wtot[wave] = incl;
-    __syncthreads();
-    int before = 0;
-    for (int w = 0; w < wave; ++w) before += wtot[w];
-    const int total = wtot[0] + wtot[1] + wtot[2] + wtot[3];
-    const int excl = before + incl - (c0 + c1);
-    if (t < 2 * SCAT_IT) { cnt[2 * t] = excl; cnt[2 * t + 1] = excl + c0; }
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < SCAT_IT; ++j) {
-      const int i = p0 + j * 256 + t;
-      const bool mine = my[j] == e;
-      const unsigned long long bal = __ballot(mine);
-      if (mine) {
-        const int s = base + cnt[4 * j + wave] + __popcll(bal & ((1ull << lane) - 1));
-        stok[s] = i / NU;
-        swt[s] = wts[i];
-        inv[i] = s;
-      }
-    }
-    base += total;
-    __syncthreads();  // (cnt and wtot are rewritten by the next piece)
+    for (int j = full; j < i; ++j) rank += sid[j] == e;
+    const int s = base + rank;
+    stok[s] = (i0 + i) / NU;
+    swt[s] = wts[i0 + i];
+    inv[i0 + i] = s;
   }
+  __syncthreads();  // (every base has been read)
+  for (int k = i; k < NE; k += 512) cursor[(size_t)blockIdx.x * NE + k] = 0;
 }
 
 // moe_quant: h [S][F] f32 (S slot rows, the first n in use) -> hq [S][F] int8, hsc [F/32][S] f32 with row stride S;
