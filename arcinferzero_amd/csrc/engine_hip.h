@@ -447,7 +447,12 @@ class Engine {
       int lpr = 0;
       for (int l : {32, 64, 128, 256})
         if (!lpr && (units + l - 1) / l <= 6 && (!force_lpr || l == force_lpr)) lpr = l;
-      const int g = lpr ? 256 / lpr : 1, wpr = lpr > 64 ? lpr / 64 : 1;
+      // Rows of 128 or 256 lanes, two tokens: work-groups of 512 threads, one a compute unit, stage the tokens once per
+      // compute unit instead of twice (5120 x 17408 Q4_K: 15.0 -> 14.4 us; one token: 11.9 -> 12.2, so not taken there;
+      // ARCZ_GEMV_BT=256: never, =512: for one token too)
+      static const int bt_env = getenv("ARCZ_GEMV_BT") ? atoi(getenv("ARCZ_GEMV_BT")) : 0;
+      const int bt = lpr >= 128 && (T == 2 || (T == 1 && bt_env == 512)) && !q2_fuse_ && bt_env != 256 ? 512 : 256;
+      const int g = lpr ? bt / lpr : 1, wpr = lpr > 64 ? lpr / 64 : 1;
       // the kernel's token slots: T rounded up, or -- both halves of two-pass inputs in one launch -- 2 T rounded up
       auto lds_of = [&](int slots) { return (size_t)slots * tok_bytes + (wpr > 1 ? (size_t)16 * g * wpr * slots * 4 : 0); };  // (16: the kernels' GEMV_FLUSH)
       const int tb2 = T == 1 ? 2 : T == 2 ? 4 : 8;
@@ -467,10 +472,11 @@ class Engine {
         // compute unit; two measured best: more add staging work and spread the reads over more rows at a time)
         static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
         static const int wgs_env = getenv("ARCZ_GEMV_WGS") ? atoi(getenv("ARCZ_GEMV_WGS")) : 0;
-        size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : 2));
+        size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : bt == 512 ? 1 : 2));
         if (wgs_env > 0) wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)wgs_env);
         const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
-                                 std::to_string(pf) + (tb > 1 ? " -DTB=" + std::to_string(tb) : std::string()) + " -DLDS=" +
+                                 std::to_string(pf) + (tb > 1 ? " -DTB=" + std::to_string(tb) : std::string()) +
+                                 (bt == 512 ? " -DBT=512" : "") + " -DLDS=" +
                                  std::to_string(lds) +
                                  (q2f ? " -DQ2_AQ=" + std::to_string(q2_aq_) + " -DQ2_SC=" + std::to_string(q2_sc_ / 4) : std::string()) +
                                  head_defs(w);
@@ -479,7 +485,7 @@ class Engine {
         if (tb == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
         else set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ld1, c_off, a);
         q2_fused_ = q2f;
-        size_t g1 = wgs * 256, l1 = 256;
+        size_t g1 = wgs * (size_t)bt, l1 = (size_t)bt;
         run(name, k, 1, &g1, &l1);
         return;
       }

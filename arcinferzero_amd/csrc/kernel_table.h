@@ -33,6 +33,9 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "mfma_probe", nullptr, "pi", {nullptr}, {{nullptr, 0, false}}, 256},
     // ---- decode
     {"decode", "gemv", "GU2", "piippppipiip", {"QT", "LPR", "PF", "GU2", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
+    {"decode", "gemv", "BT", "piippppipii", {"QT", "LPR", "PF", "BT", nullptr}, {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 512},
+    {"decode", "gemv_mt", "BT", "piippppiipiii", {"QT", "LPR", "PF", "TB", "BT", nullptr},
+     {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 512},
     {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "LPR", "PF", "TB", nullptr},
      {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
