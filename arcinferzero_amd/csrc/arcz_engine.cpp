@@ -84,6 +84,8 @@ arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, c
         uint64_t dims[8];
         arcz_gguf_tensor(g, (size_t)ig, nullptr, nullptr, &nd, dims, nullptr, nullptr);
         if (nd != 3) throw std::runtime_error(std::string("tensor ") + gate + " is no expert tensor");
+        if (dims[0] > (1u << 30) || dims[1] > (1u << 30) || dims[2] > 65536)  // (before they become ints)
+          throw std::runtime_error(std::string("tensor ") + gate + ": dimensions out of range");
         const int Ed = (int)dims[0], F = (int)dims[1], NE = (int)dims[2];
         E.moe_alloc(NE, NU, Ed, F);
         L->L.NE = NE; L->L.NU = NU; L->L.E = Ed; L->L.F = F;

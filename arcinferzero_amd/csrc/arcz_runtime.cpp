@@ -21,6 +21,7 @@ struct arcz_mem {
   char* ptr;
   size_t size;
   bool owner;
+  arcz_mem* parent = nullptr;  // a view's owner (the root of a chain of views)
 };
 struct arcz_kernel {
   hipFunction_t fn;
@@ -192,7 +193,7 @@ arcz_mem* arcz_view(arcz_mem* parent, size_t offset, size_t bytes) {
     fail(ARCZ_E_SUBBUFFER, "view of %zu bytes at %zu past its parent's end", bytes, offset);
     return nullptr;
   }
-  arcz_mem* m = new arcz_mem{parent->ptr + offset, bytes, false};
+  arcz_mem* m = new arcz_mem{parent->ptr + offset, bytes, false, parent->owner ? parent : parent->parent};
   R.mems.insert(m);
   return m;
 }
@@ -202,6 +203,10 @@ int arcz_free(arcz_mem* m) {
   if (m == R.scratch) return fail(ARCZ_E_ARG_VALUE, "arcz_free of the library's static scratch");
   if (!R.mems.count(m)) return fail(ARCZ_E_ARG_VALUE, "arcz_free of a handle that is not live");
   if (m->owner) {
+    // (the caller frees views before their parents, zero/engine.h:251-252; a view that is still live would name freed
+    //  memory: refused, nothing is freed)
+    for (const arcz_mem* v : R.mems)
+      if (v->parent == m) return fail(ARCZ_E_ARG_VALUE, "arcz_free of a buffer that still has live views");
     HIP_TRY(hipStreamSynchronize(R.stream));
     HIP_TRY(hipFree(m->ptr));
     R.device_bytes -= m->size;
@@ -267,7 +272,8 @@ int arcz_fill(arcz_mem* dst, const void* pattern, size_t ps, size_t offset, size
   if (ps == 1) v |= v << 8;
   if (ps <= 2) v |= v << 16;
   if (bytes % 4 == 0 && offset % 4 == 0) {
-    // a small kernel rather than a memset node: callers may be under stream capture
+    // a small kernel rather than a memset node (the call still waits for the stream, as the reference's fill does,
+    // clrt.h:703-710: the pattern is the caller's; it is not a call for a stream that is being captured)
     arcz_kernel* k = fill_kernel();
     if (!k) return ARCZ_E_BUILD;
     void* p = dst->ptr + offset;

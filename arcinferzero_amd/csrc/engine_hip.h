@@ -107,6 +107,9 @@ class Engine {
   cl_mem aq2_ = nullptr, asc2_ = nullptr, absum2_ = nullptr;  // views of the second halves
   void set_two_pass(bool on) {
     if (on == q2mm_) return;
+    // (checked before anything is changed: a refusal leaves the engine as it was)
+    if (on && (size_t)max_chunk * max_k >= (1ull << 31))
+      throw std::invalid_argument("two-pass mode: a chunk of max_chunk x max_k values must stay below 2 GiB");
     for (cl_mem* v : {&aq2_, &asc2_, &absum2_})
       if (*v) { release(*v); *v = nullptr; }
     release(aq_); release(asc_); release(absum_);
@@ -120,7 +123,6 @@ class Engine {
     q2_aq_ = M * max_k;
     q2_sc_ = M * (max_k / 32) * 4;
     q2_ab_ = M * (max_k / 16) * 2;
-    if (q2_aq_ >= (1ull << 31)) throw std::invalid_argument("two-pass mode: a chunk of max_chunk x max_k values must stay below 2 GiB");
     q2_defs_ = " -DQ2_AQ=" + std::to_string(q2_aq_) + " -DQ2_SC=" + std::to_string(q2_sc_ / 4) + " -DQ2_AB=" +
                std::to_string(q2_ab_ / 2);
     aq2_ = view(aq_, q2_aq_, q2_aq_);

@@ -152,6 +152,51 @@ extern "C" __global__ __launch_bounds__(256) void rmsnorm_quant(const float* __r
   const int m = blockIdx.y;
   const bool valid = m < M_valid;
   const float* xr = x + (size_t)(m + row_off) * K;
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
+  constexpr int MAXU = 5;  // superblocks a thread can hold: rows of up to 16 * 5 * 256 = 20480 values
+  if (gridDim.x == 1 && K <= 16 * MAXU * 256) {
+    // One work-group per row: the row stays in registers between the sum of squares and the quantization (a thread
+    // holds its 16 values of superblocks sub, sub + 16, ...), so x is read once, every load of the row in flight at once.
+    const int nsb = K >> 8;
+    float4 xv[MAXU][4];
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+      const int sb = sub + 16 * u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        xv[u][i] = valid && sb < nsb ? *(const float4*)(xr + sb * 256 + 16 * lane16 + 4 * i) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ss += xv[u][i].x * xv[u][i].x;
+        ss += xv[u][i].y * xv[u][i].y;
+        ss += xv[u][i].z * xv[u][i].z;
+        ss += xv[u][i].w * xv[u][i].w;
+      }
+    ss = group_sum(ss, red);
+    const float r = rsqrtf(ss / (float)K + eps);
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+      const int sb = sub + 16 * u;
+      if (sb >= nsb) break;  // (the same for the 16 threads of a superblock)
+      const int base = sb * 256 + 16 * lane16;
+      float v[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 f = xv[u][i], g = *(const float4*)(w + base + 4 * i);
+        v[4 * i] = f.x * r * g.x; v[4 * i + 1] = f.y * r * g.y; v[4 * i + 2] = f.z * r * g.z; v[4 * i + 3] = f.w * r * g.w;
+      }
+      if (write_h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          *(float4*)(hout + (size_t)m * K + base + 4 * i) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+      store_row_quant(v, sb, lane16, m, M, K, act32, aq, asc, absum, q2_aq, q2_sc, q2_ab);
+    }
+    return;
+  }
   float ss = 0.0f;
   if (valid)
     for (int i = threadIdx.x * 4; i < K; i += 1024) {
@@ -163,7 +208,6 @@ extern "C" __global__ __launch_bounds__(256) void rmsnorm_quant(const float* __r
     }
   ss = group_sum(ss, red);
   const float r = rsqrtf(ss / (float)K + eps);
-  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
   for (int s = blockIdx.x * 16 + sub; s < K / 256; s += 16 * gridDim.x) {
     const int base = s * 256 + 16 * lane16;
     float v[16];
@@ -268,23 +312,34 @@ extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __re
   const bool valid = m < M_valid;
   const float* gr = gu + (size_t)m * (fused ? F : 2 * F);
   const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
-  for (int s = blockIdx.x * 16 + sub; s < F / 256; s += 16 * gridDim.x) {
-    const int base = s * 256 + 16 * lane16;
-    float v[16];
-    if (!valid) {
+  const int nsb = F >> 8, stride = 16 * gridDim.x;
+  // (a thread's superblocks two at a time: the loads of both are issued before the first is worked on)
+  for (int s0 = blockIdx.x * 16 + sub; s0 < nsb; s0 += 2 * stride) {
+    float4 gv[2][4], uv4[2][4];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) v[i] = 0.0f;
-    } else {
+    for (int h = 0; h < 2; ++h) {
+      const int s = s0 + h * stride;
+      const bool in = valid && s < nsb;
+      const int base = (in ? s : 0) * 256 + 16 * lane16;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float4 g = *(const float4*)(gr + base + 4 * i);
-        v[4 * i] = g.x; v[4 * i + 1] = g.y; v[4 * i + 2] = g.z; v[4 * i + 3] = g.w;
+        gv[h][i] = in ? *(const float4*)(gr + base + 4 * i) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        uv4[h][i] = in && !fused ? *(const float4*)(gr + F + base + 4 * i) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
       }
-      if (!fused) {
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int s = s0 + h * stride;
+      if (s >= nsb) break;
+      float v[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[4 * i] = gv[h][i].x; v[4 * i + 1] = gv[h][i].y; v[4 * i + 2] = gv[h][i].z; v[4 * i + 3] = gv[h][i].w;
+      }
+      if (valid && !fused) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float4 u = *(const float4*)(gr + F + base + 4 * i);
-          const float uv[4] = {u.x, u.y, u.z, u.w};
+          const float uv[4] = {uv4[h][i].x, uv4[h][i].y, uv4[h][i].z, uv4[h][i].w};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const float g = v[4 * i + j];
@@ -294,8 +349,8 @@ extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __re
           }
         }
       }
+      store_row_quant(v, s, lane16, m, M, F, act32, aq, asc, absum, q2_aq, q2_sc, q2_ab);
     }
-    store_row_quant(v, s, lane16, m, M, F, act32, aq, asc, absum, q2_aq, q2_sc, q2_ab);
   }
 }
 

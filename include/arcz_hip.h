@@ -50,7 +50,8 @@ arcz_mem* arcz_alloc(size_t bytes);
 /* clCreateSubBuffer (clrt.h:752-762): a non-owning view; NULL if it would pass the parent's end. */
 arcz_mem* arcz_view(arcz_mem* parent, size_t offset, size_t bytes);
 /* clReleaseMemObject (clrt.h:763-769): waits for the stream, then frees (an owner) or forgets (a view).  The
- * caller frees views before their parents (zero/engine.h:251-252). */
+ * caller frees views before their parents (zero/engine.h:251-252): an owner that still has live views is refused
+ * (ARCZ_E_ARG_VALUE, nothing freed). */
 int arcz_free(arcz_mem* m);
 size_t arcz_mem_size(const arcz_mem* m);
 /* The device address of a buffer (for interop with another runtime on the same device; not used by the engine). */

@@ -28,6 +28,9 @@ def test_buffers_views_transfers(rt):
     with pytest.raises(az.ArczError) as e:
         b.view(4000, 200)
     assert e.value.code == -13
+    with pytest.raises(az.ArczError) as e:                 # a parent with a live view is not freed
+        b.free()
+    assert e.value.code == -50 and np.array_equal(v.read(np.uint32, 4), np.full(4, 7, np.uint32))
     small = rt.alloc(1)                                    # at least 64 bytes are there
     small.write(np.zeros(1, np.uint8))
     for x in (v, small, b):
