@@ -84,7 +84,7 @@ class Engine {
     cl_kernel k = kernel("decode", "", "expand_iq3s");
     int rows = (int)w.rows, nsb = w.K / 256;
     set_args(k, 0, w.raw, xw_, tabs_, rows, nsb);
-    size_t g1 = ((size_t)rows * nsb + 3) / 4 * 256, l1 = 256;
+    size_t g1 = ((size_t)rows * nsb + 15) / 16 * 256, l1 = 256;
     run(name, k, 1, &g1, &l1);
     GpuWeight x = w;
     x.type = GGML_Q6_K;
@@ -881,10 +881,12 @@ class Engine {
       }
       return;
     }
-    // slots per tile = the token rows of one work-group of the tile GEMM: 64 when any of the three tensors is Q4_K or
-    // Q5_K (their tile kernel takes at most 64; the others' take up to 128 and run 64-slot tiles as well), else 128
+    // slots per tile = the token rows of one work-group of the tile GEMM: 64 when any of the three tensors is Q4_K,
+    // Q5_K or Q6_K (IQ3_S runs as Q6_K) -- their tile kernels take at most 64; the others' take up to 128 and run
+    // 64-slot tiles as well -- else 128
     bool t64 = false;
-    for (int i = 0; i < 3; ++i) t64 = t64 || L.ex[i].type == GGML_Q4_K || L.ex[i].type == GGML_Q5_K;
+    for (int i = 0; i < 3; ++i)
+      t64 = t64 || L.ex[i].type == GGML_Q4_K || L.ex[i].type == GGML_Q5_K || L.ex[i].type == GGML_Q6_K || L.ex[i].type == GGML_IQ3_S;
     const int tm = t64 ? 64 : 128;
     moe_route(L, rl, ldl, T, tm);
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)

@@ -676,33 +676,37 @@ MOE_DECODE_ALL(21)
 // expand_iq3s: the IQ3_S planes of `rows` rows to Q6_K planes of the same rows, value for value -- the same f16 d, the
 // int8 sub-scale 1 + 2 s for both 16-value halves of a block, q = value + 32 in six bits -- for the prefill GEMM and
 // the expert-tile GEMM, which run their Q6_K kernels on the result (the place of the reference's decode pass in front
-// of its GEMM, zero/engine.h:1205-1250 with zero/kernels/decode.cl:183-478).  Thread (superblock, n, l) makes the bytes
-// ql[64 n + l], ql[64 n + 32 + l] and qh[32 n + l]: the values l of blocks 4 n .. 4 n + 3.
-// grid: ceil(rows * nsb / 4) work-groups of 256 (64 threads a superblock).
+// of its GEMM, zero/engine.h:1205-1250 with zero/kernels/decode.cl:183-478).  Thread (superblock, n, j) makes the words
+// ql[64 n + 4 j ..], ql[64 n + 32 + 4 j ..] and qh[32 n + 4 j ..]: the values 4 j .. 4 j + 3 of blocks 4 n .. 4 n + 3,
+// one codebook entry per block.  grid: ceil(rows * nsb / 16) work-groups of 256 (16 threads a superblock).
 extern "C" __global__ __launch_bounds__(256) void expand_iq3s(const uint8_t* __restrict__ raw, uint8_t* __restrict__ out,
                                                               const uint32_t* __restrict__ tabs, int rows, int nsb) {
   iq3s_grid_init(tabs);
   const size_t total = (size_t)rows * nsb;
-  const size_t rs = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const size_t rs = (size_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   if (rs >= total) return;
   const PlanesIQ3S pi = planes_iq3s((size_t)rows, nsb);
   const PlanesQ6K po = planes_q6k((size_t)rows, nsb);
-  const int n = (threadIdx.x >> 5) & 1, l = threadIdx.x & 31, gi = l >> 2, j = l & 3;
-  int q[4];
+  const int n = (threadIdx.x >> 3) & 1, j = threadIdx.x & 7;
+  const uint32_t h9 = *(const uint32_t*)(raw + pi.hd + rs * 12 + 4 * n);  // the ninth bits of blocks 4 n .. 4 n + 3
+  uint32_t q[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const int ib = 4 * n + k;
-    const uint32_t idx = raw[pi.qs + rs * 64 + ib * 8 + gi] | ((((uint32_t)raw[pi.hd + rs * 12 + ib] >> gi) & 1u) << 8);
-    const int mag = (int)((iq3s_grid_lds[idx] >> (8 * j)) & 0xFFu);
-    const int neg = (raw[pi.sg + rs * 32 + ib * 4 + (l >> 3)] >> (l & 7)) & 1;
-    q[k] = (neg ? -mag : mag) + 32;
+    const uint32_t idx = raw[pi.qs + rs * 64 + ib * 8 + j] | ((((h9 >> (8 * k)) >> j) & 1u) << 8);
+    const uint32_t s4 = ((uint32_t)raw[pi.sg + rs * 32 + ib * 4 + (j >> 1)] >> (4 * (j & 1))) & 0xFu;
+    const uint32_t v = iq3s_signed4(iq3s_grid_lds[idx], s4);
+    q[k] = ((v & 0x7F7F7F7Fu) + 0x20202020u) ^ (v & 0x80808080u);  // value + 32 in every byte, no carry between bytes
   }
-  out[po.ql + rs * 128 + 64 * n + l] = (uint8_t)((q[0] & 15) | ((q[2] & 15) << 4));
-  out[po.ql + rs * 128 + 64 * n + 32 + l] = (uint8_t)((q[1] & 15) | ((q[3] & 15) << 4));
-  out[po.qh + rs * 64 + 32 * n + l] = (uint8_t)((q[0] >> 4) | ((q[1] >> 4) << 2) | ((q[2] >> 4) << 4) | ((q[3] >> 4) << 6));
-  if (n == 0 && l < 16) {
-    const int ib = l >> 1;
-    out[po.sc + rs * 16 + l] = (uint8_t)(1 + 2 * ((raw[pi.hd + rs * 12 + 8 + (ib >> 1)] >> (4 * (ib & 1))) & 0xF));
+  const uint32_t lo = 0x0F0F0F0Fu, two = 0x03030303u;
+  *(uint32_t*)(out + po.ql + rs * 128 + 64 * n + 4 * j) = (q[0] & lo) | ((q[2] & lo) << 4);
+  *(uint32_t*)(out + po.ql + rs * 128 + 64 * n + 32 + 4 * j) = (q[1] & lo) | ((q[3] & lo) << 4);
+  *(uint32_t*)(out + po.qh + rs * 64 + 32 * n + 4 * j) =
+      ((q[0] >> 4) & two) | (((q[1] >> 4) & two) << 2) | (((q[2] >> 4) & two) << 4) | (((q[3] >> 4) & two) << 6);
+  if (n == 0 && j < 4) {  // sub-scales 4 j .. 4 j + 3: blocks 2 j and 2 j + 1, each for both of its halves
+    const uint32_t sb = raw[pi.hd + rs * 12 + 8 + j];
+    const uint32_t s0 = 1 + 2 * (sb & 0xFu), s1 = 1 + 2 * (sb >> 4);
+    *(uint32_t*)(out + po.sc + rs * 16 + 4 * j) = s0 | (s0 << 8) | (s1 << 16) | (s1 << 24);
   }
-  if (n == 1 && l < 2) out[po.d + rs * 2 + l] = raw[pi.d + rs * 2 + l];
+  if (n == 1 && j == 0) *(unsigned short*)(out + po.d + rs * 2) = *(const unsigned short*)(raw + pi.d + rs * 2);
 }

@@ -628,15 +628,23 @@ struct G6ScaleRegs {
   uint32_t d;
 };
 
+// TILES: one expert tile -- the planes hold rows_total rows, the expert's N rows start at row_base, slot r of the tile
+// reads token row rowmap[m0 + r] (use_map) and its results are scaled by rowscale[m0 + r] (use_scale).
+template <bool TILES = false>
 __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
-                                  int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0) {
+                                  int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0,
+                                  size_t rows_total = 0, size_t row_base = 0, const int* __restrict__ rowmap = nullptr,
+                                  int use_map = 0, const float* __restrict__ rowscale = nullptr, int use_scale = 0) {
   __shared__ alignas(16) uint8_t lds[2 * G6_STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int l32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
-  const PlanesQ6K pl = planes_q6k((size_t)N, nsb);
-  auto token_row = [&](int r) { return m0 + (r < rows_valid ? r : 0); };  // rows past the tile read its first row
+  const PlanesQ6K pl = planes_q6k(TILES ? rows_total : (size_t)N, nsb);
+  auto token_row = [&](int r) {  // rows past the tile read its first row
+    const int rr = r < rows_valid ? r : 0;
+    return (TILES && use_map) ? rowmap[m0 + rr] : m0 + rr;
+  };
 
   // ---- what this lane fetches each step (a step = half a superblock = 128 values).  Activations: 2 instructions a
   // wave, 8 rows each, row R = (2 wave + i) 8 + lane / 8 at chunk lane % 8 <- source chunk (lane % 8) ^ (R % 8).  Low
@@ -652,8 +660,8 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
   }
   hoff = (uint32_t)min(n0 + wave * 32 + (lane >> 1), N - 1) * (uint32_t)nsb * 64u + 16u * ((lane & 1) ^ ((lane >> 3) & 1));
   const signed char* abase = aq + (size_t)s_begin * 256;
-  const uint8_t* lbase = raw + pl.ql + (size_t)s_begin * 128;
-  const uint8_t* hbase = raw + pl.qh + (size_t)s_begin * 64;
+  const uint8_t* lbase = raw + pl.ql + (row_base * nsb + s_begin) * 128;
+  const uint8_t* hbase = raw + pl.qh + (row_base * nsb + s_begin) * 64;
   // scales: threads 0-63 prepare token t (the step's 4 activation scales: one per thread and block -> 4 threads a
   // token would do; here thread t takes token t % 64, block t / 64); every thread prepares weight row t / 2: the four
   // sub-scales 4 (t % 2) .. + 3 of the step, and (t % 2 == 0) the row's d.
@@ -676,8 +684,8 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
   auto load_scales = [&](G6ScaleRegs& r, int st) {
     const int sb = s_begin + (st >> 1), hh = st & 1;
     r.sa = (asc + (size_t)(sb * 8 + hh * 4 + b_s) * M)[m_s];
-    r.sc = *(const uint32_t*)(raw + pl.sc + ((size_t)n_s * nsb + sb) * 16 + 8 * hh + 4 * p_s);
-    r.d = *(const unsigned short*)(raw + pl.d + ((size_t)n_s * nsb + sb) * 2);
+    r.sc = *(const uint32_t*)(raw + pl.sc + ((row_base + n_s) * nsb + sb) * 16 + 8 * hh + 4 * p_s);
+    r.d = *(const unsigned short*)(raw + pl.d + ((row_base + n_s) * nsb + sb) * 2);
   };
   auto store_scales = [&](const G6ScaleRegs& r, int stage) {
     uint8_t* base = lds + stage * G6_STAGE;
@@ -804,6 +812,7 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
         const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
         if (r >= rows_valid) continue;
         float v = res[ms][i];
+        if (TILES && use_scale) v *= rowscale[m0 + r];
         float* cp = C + (size_t)(m0 + r) * ldc + c_off + n;
         if (accumulate == 1) {
           v += *cp;
@@ -1655,7 +1664,7 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_B
   tile_of(blockIdx.x, mt, nt, tm, tn);
   const int m0 = tm * G6_BM, n0 = tn * BN;
   const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
-  gemm6_body(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny, s_begin + ns * (y + 1) / ny,
+  gemm6_body<false>(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny, s_begin + ns * (y + 1) / ny,
              m0, min(G6_BM, M - m0), n0);
 }
 // (Q5_K, IQ4_XS -DBM=128 -DBN=128 -DSPLITK: the register-staged body's tiles)
@@ -1769,17 +1778,18 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321(
   int tm, tn;
   tile_of(blockIdx.x, mt, nt, tm, tn);
   const int m0 = tm * G6_BM, n0 = tn * BN;
-  gemm6_body(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
+  gemm6_body<false>(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
 }
-extern "C" __global__ __launch_bounds__(256) void gemm__QTYPE14_ACT321_MOE_TILES1(
+// (Q6_K experts: the dense kernel's body over tiles of at most 64 slots -- the engine builds the list for that size)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_MOE_TILES1(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
     int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
     int use_map, const float* rowscale, int use_scale, int NE) {
   const int t_end = tstart[e1];
   for (int ti = tstart[e0] + blockIdx.y; ti < t_end; ti += gridDim.y) {
     const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-    gemm_body<QT_Q6_K, true>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N,
-                             (size_t)e * N, r0, min(nr, BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
+    gemm6_body<true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, r0, min(nr, G6_BM), blockIdx.x * BN,
+                     (size_t)NE * N, (size_t)e * N, rowmap, use_map, rowscale, use_scale);
     __syncthreads();
   }
 }
