@@ -458,11 +458,12 @@ class Engine {
       // the kernel's token slots: T rounded up, or -- both halves of two-pass inputs in one launch -- 2 T rounded up
       auto lds_of = [&](int slots) { return (size_t)slots * tok_bytes + (wpr > 1 ? (size_t)16 * g * wpr * slots * 4 : 0); };  // (16: the kernels' GEMV_FLUSH)
       const int tb2 = T == 1 ? 2 : T == 2 ? 4 : 8;
-      const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= 65536;
+      const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= (w.type == GGML_IQ3_S ? 65536 - 2048 : 65536);
       const int tbl = q2f ? tb2 : T <= 2 ? T : T <= 4 ? 4 : 8;
       const size_t lds = lds_of(tbl);
-      // (IQ3_S: its GEMV reads the weights straight into registers, the reference's gemv_v form)
-      const bool fits = !force_v && lpr && lds <= 65536 && w.type != GGML_IQ3_S;
+      // (IQ3_S: 2 KiB of the work-group's LDS hold the codebook)
+      const size_t lds_max = w.type == GGML_IQ3_S ? 65536 - 2048 : 65536;
+      const bool fits = !force_v && lpr && lds <= lds_max;
       if (mm_ok && T >= 3 && (T >= 7 || !fits)) {
         rd_bytes -= raw_bytes(w);  // (counted by gemv_mm)
         gemv_mm();
@@ -512,7 +513,7 @@ class Engine {
   // rows of a pass.  ARCZ_GEMV_GU=0: never taken.
   bool gemv_gu(const GpuWeight& g, const GpuWeight& u, int Mp, cl_mem C) {
     static const bool off = getenv("ARCZ_GEMV_GU") && atoi(getenv("ARCZ_GEMV_GU")) == 0;
-    if (off || cur_T_ != 1 || q2mm_ || !g.raw || !u.raw || g.type != u.type || g.N != u.N || g.K != u.K || g.type == GGML_IQ3_S)
+    if (off || cur_T_ != 1 || q2mm_ || !g.raw || !u.raw || g.type != u.type || g.N != u.N || g.K != u.K)
       return false;
     if (g.K != cur_K_ || Mp != cur_Mp_)
       throw std::runtime_error("gemv_gu: the activations hold " + std::to_string(cur_Mp_) + " x " + std::to_string(cur_K_) +
@@ -526,7 +527,7 @@ class Engine {
     if (!lpr) return false;
     const int gr = 256 / lpr, wpr = lpr > 64 ? lpr / 64 : 1;
     const size_t lds = (size_t)tok_bytes + (wpr > 1 ? (size_t)16 * gr * wpr * 4 : 0);
-    if (lds > 65536 || N % gr) return false;
+    if (lds > (g.type == GGML_IQ3_S ? 65536u - 2048u : 65536u) || N % gr) return false;
     if (arcz_mem_size(C) < (size_t)2 * N * 4) throw std::runtime_error("gemv_gu: the output does not fit C");
     rd_bytes += raw_bytes(g) + raw_bytes(u);
     const int pf = (units + lpr - 1) / lpr;
