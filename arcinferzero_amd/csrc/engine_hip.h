@@ -97,7 +97,13 @@ class Engine {
     aq_ = buf(M * max_k * f);
     asc_ = buf(M * (max_k / 32) * 4 * f);
     absum_ = buf(M * (max_k / 16) * 2 * f);
+    if (!asc_rep_) asc_rep_ = buf(M * (max_k / 32) * 4);
   }
+  // Per-256 activation scales (act32 = 0: the reference's choice for insensitive inputs when its act32_all is off,
+  // zero/engine.h:1254): the quantizers store one scale per superblock, asc [K/256][M]; the matmul kernels here take
+  // per-32 scales, so a matmul of such a chunk first writes each scale out eight times into asc_rep_ and reads that.
+  cl_mem asc_rep_ = nullptr;
+  int cur_act32_ = 1;
   // Two-pass matmul inputs (zero/engine.h:1034-1075 q2_init, the mode of the reference's Gemma 4 and Qwen3 models):
   // every producer also quantizes what its int8 values miss, v - q * scale, the same way, into the second half of the
   // three buffers, and every matmul runs a second time over that half, accumulating (matmul below).
@@ -237,13 +243,13 @@ class Engine {
   // matmul takes (cur_T_).
   void quantize_rows(cl_mem x, int ldx, int K, int Mp, int T, int act32) {
     check_chunk(K, Mp, T);
-    if (!act32) throw std::runtime_error("quantize_rows: the matmul kernels take per-32 activation scales (act32)");
+    if (!act32 && q2mm_) throw std::runtime_error("quantize_rows: two-pass inputs take per-32 activation scales (act32)");
     if (ldx < K || arcz_mem_size(x) < ((size_t)(T - 1) * ldx + K) * 4) throw std::runtime_error("quantize_rows: x is too small");
     cl_kernel k = kernel("ops", q2_defs_, "quant_rows");
     set_args(k, 0, x, ldx, K, Mp, T, aq_, asc_, absum_, act32);
     size_t gws[2] = {(size_t)256 * (K / 256), (size_t)(Mp + 63) / 64}, lws[2] = {256, 1};
     run("quant_rows", k, 2, gws, lws);
-    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp; cur_act32_ = act32 ? 1 : 0;
   }
   // The fused producers of the reference (rmsnorm_quant, zero/engine.h:1256-1267; swiglu_quant via run_rows_quant,
   // zero/engine.h:1404-1440): a work-group per row of the chunk, or -- a pass of 1-8 tokens -- the valid rows only,
@@ -251,7 +257,7 @@ class Engine {
   static bool wide_rows(int T) { return T <= 8; }
   void rmsnorm_quant(cl_mem x, int row_off, cl_mem w, int K, int Mp, int T, int act32, float eps, cl_mem hout = nullptr) {
     check_chunk(K, Mp, T);
-    if (!act32) throw std::runtime_error("rmsnorm_quant: the matmul kernels take per-32 activation scales (act32)");
+    if (!act32 && q2mm_) throw std::runtime_error("rmsnorm_quant: two-pass inputs take per-32 activation scales (act32)");
     if (row_off < 0 || arcz_mem_size(x) < (size_t)(row_off + T) * K * 4 || arcz_mem_size(w) < (size_t)K * 4 ||
         (hout && arcz_mem_size(hout) < (size_t)Mp * K * 4))
       throw std::runtime_error("rmsnorm_quant: a buffer is too small for " + std::to_string(T) + " rows of " + std::to_string(K));
@@ -264,12 +270,12 @@ class Engine {
       gws[1] = (size_t)T;
     }
     run("rmsnorm_quant", k, 2, gws, lws);
-    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp; cur_act32_ = act32 ? 1 : 0;
   }
   // gu: rows [gate(F) | up(F)] f32, or rows of F values when the matmul before has fused the product
   void swiglu_quant(cl_mem gu, int F, int Mp, int T, int act32, int fused, int gelu) {
     check_chunk(F, Mp, T);
-    if (!act32) throw std::runtime_error("swiglu_quant: the matmul kernels take per-32 activation scales (act32)");
+    if (!act32 && q2mm_) throw std::runtime_error("swiglu_quant: two-pass inputs take per-32 activation scales (act32)");
     if (arcz_mem_size(gu) < (size_t)T * F * (fused ? 1 : 2) * 4) throw std::runtime_error("swiglu_quant: gu is too small");
     cl_kernel k = kernel("ops", q2_defs_, "swiglu_quant");
     set_args(k, 0, gu, F, Mp, T, aq_, asc_, absum_, act32, fused, gelu);
@@ -279,7 +285,7 @@ class Engine {
       gws[1] = (size_t)T;
     }
     run("swiglu_quant", k, 2, gws, lws);
-    cur_T_ = T; cur_K_ = F; cur_Mp_ = Mp;
+    cur_T_ = T; cur_K_ = F; cur_Mp_ = Mp; cur_act32_ = act32 ? 1 : 0;
   }
   // x = (x + rmsnorm(t) * w) * s over the first T rows ([T][K] f32 each), then the next matmul's input from the new x:
   // rmsnorm(x) * w2, or x itself with norm2 = false (zero/engine.h:1393-1403 add_norm_quant, whose x_ and big_ are the
@@ -287,7 +293,7 @@ class Engine {
   void add_norm_quant(cl_mem x, cl_mem t, cl_mem w, int K, int T, int Mp, float s, cl_mem w2, bool norm2, int act32,
                       float eps) {
     check_chunk(K, Mp, T);
-    if (!act32) throw std::runtime_error("add_norm_quant: the matmul kernels take per-32 activation scales (act32)");
+    if (!act32 && q2mm_) throw std::runtime_error("add_norm_quant: two-pass inputs take per-32 activation scales (act32)");
     if (arcz_mem_size(x) < (size_t)T * K * 4 || arcz_mem_size(t) < (size_t)T * K * 4 || arcz_mem_size(w) < (size_t)K * 4 ||
         (norm2 && (!w2 || arcz_mem_size(w2) < (size_t)K * 4)))
       throw std::runtime_error("add_norm_quant: a buffer is too small for " + std::to_string(T) + " rows of " + std::to_string(K));
@@ -297,7 +303,7 @@ class Engine {
     // (a pass of 1-8 tokens: the valid rows only, as the reference; a longer chunk: all Mp rows, the padding as zeros)
     size_t gws[2] = {256, (size_t)(wide_rows(T) ? T : Mp)}, lws[2] = {256, 1};
     run("add_rmsnorm", k, 2, gws, lws);
-    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp; cur_act32_ = act32 ? 1 : 0;
   }
   // Activations quantized elsewhere (the reference's benches quantize on the host, bench/gemv_bench.cpp:103-129).
   void set_activations(const int8_t* aq, const float* asc, const int16_t* absum, int K, int Mp, int T) {
@@ -306,7 +312,7 @@ class Engine {
     CL_CHECK(clEnqueueWriteBuffer(cl_.queue, aq_, CL_TRUE, 0, (size_t)Mp * K, aq, 0, nullptr, nullptr));
     CL_CHECK(clEnqueueWriteBuffer(cl_.queue, asc_, CL_TRUE, 0, (size_t)Mp * (K / 32) * 4, asc, 0, nullptr, nullptr));
     CL_CHECK(clEnqueueWriteBuffer(cl_.queue, absum_, CL_TRUE, 0, (size_t)Mp * (K / 16) * 2, absum, 0, nullptr, nullptr));
-    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp;
+    cur_T_ = T; cur_K_ = K; cur_Mp_ = Mp; cur_act32_ = 1;
   }
 
   // ---- matmul (zero/engine.h:1080-1112): C[:, c_off : c_off+N] (+)= act * W^T for the current chunk.  acc: 0 = store,
@@ -326,6 +332,26 @@ class Engine {
   void matmul(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
     static const bool fuse_off = getenv("ARCZ_Q2_FUSE") && atoi(getenv("ARCZ_Q2_FUSE")) == 0;
     if (q2mm_ && acc > 1) throw std::logic_error(std::string("two-pass activations with a fused epilogue: ") + name);
+    if ((act32 ? 1 : 0) != cur_act32_)
+      throw std::runtime_error(std::string("matmul ") + name + ": the chunk was quantized with " + (cur_act32_ ? "per-32" : "per-256") +
+                               " scales, the call says " + (act32 ? "per-32" : "per-256"));
+    if (!act32) {  // (one-pass engines only: the quantizers refuse it otherwise)
+      cl_kernel k = kernel("ops", "", "asc_expand");
+      int MM = cur_Mp_, nsb = cur_K_ / 256;
+      set_args(k, 0, asc_, asc_rep_, MM, nsb);
+      size_t g1 = ((size_t)nsb * 8 * MM + 255) / 256 * 256, l1 = 256;
+      run("asc_expand", k, 1, &g1, &l1);
+      const cl_mem s0 = asc_;
+      asc_ = asc_rep_;
+      try {
+        matmul1(name, w, Mp, C, ldc, c_off, acc, true);
+      } catch (...) {
+        asc_ = s0;
+        throw;
+      }
+      asc_ = s0;
+      return;
+    }
     // (the output head with a logit soft cap and two-pass inputs: the cap applies to the sum of both passes, so both
     //  run without it and softcap_rows caps the sum; zero/engine.h:1081-1110)
     const bool cap = q2mm_ && w.softcap > 0.0f;
@@ -399,7 +425,6 @@ class Engine {
 
   void matmul1(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
     if (!w.raw) throw std::runtime_error(std::string("matmul ") + name + ": the weight is not loaded");
-    if (!act32) throw std::runtime_error(std::string("matmul ") + name + ": per-256 activation scales are not built");
     if (cur_T_ <= 0 || w.K != cur_K_ || Mp != cur_Mp_)
       throw std::runtime_error(std::string("matmul ") + name + ": the activations hold " + std::to_string(cur_Mp_) + " x " +
                                std::to_string(cur_K_) + ", the matrix takes " + std::to_string(Mp) + " x " + std::to_string(w.K));
@@ -513,7 +538,7 @@ class Engine {
   // rows of a pass.  ARCZ_GEMV_GU=0: never taken.
   bool gemv_gu(const GpuWeight& g, const GpuWeight& u, int Mp, cl_mem C) {
     static const bool off = getenv("ARCZ_GEMV_GU") && atoi(getenv("ARCZ_GEMV_GU")) == 0;
-    if (off || cur_T_ != 1 || q2mm_ || !g.raw || !u.raw || g.type != u.type || g.N != u.N || g.K != u.K)
+    if (off || cur_T_ != 1 || q2mm_ || !cur_act32_ || !g.raw || !u.raw || g.type != u.type || g.N != u.N || g.K != u.K)
       return false;
     if (g.K != cur_K_ || Mp != cur_Mp_)
       throw std::runtime_error("gemv_gu: the activations hold " + std::to_string(cur_Mp_) + " x " + std::to_string(cur_K_) +
@@ -768,6 +793,7 @@ class Engine {
     const int E = L.E, F = L.F, NU = L.NU, n = T * NU;
     if (sh && arcz_mem_size(sh) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: sh is too small");
     if (cur_T_ != T || cur_K_ != E || cur_Mp_ != Mp) throw std::runtime_error("layer_moe: the activations are not this chunk's");
+    if (!cur_act32_) throw std::runtime_error("layer_moe: the expert kernels take per-32 activation scales (as the reference's, zero/kernels/gemm.cl:140-142)");
     if (arcz_mem_size(x) < (size_t)T * E * 4) throw std::runtime_error("layer_moe: x is too small");
     // A pass of 1-16 tokens (zero/engine_moe.h:86-262 has this form for 1-8): small tiles through the matrix-vector
     // kernels moe_gateup_q / moe_down_q, routed by one launch (moe_route1 for one token, whose NU experts are the tiles;

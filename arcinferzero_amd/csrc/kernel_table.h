@@ -26,6 +26,7 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "add_norm_quant", nullptr, "pppiffpiipppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
+    {"ops", "asc_expand", nullptr, "ppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "softcap_rows", nullptr, "piiif", {nullptr}, {{nullptr, 0, false}}, 0},
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "copy128", nullptr, "ppz", {nullptr}, {{nullptr, 0, false}}, 256},

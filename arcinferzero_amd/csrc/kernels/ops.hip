@@ -364,6 +364,17 @@ extern "C" __global__ void softcap_rows(float* C, int ld, int off, int N, float 
   *p = head_out(*p, cap);
 }
 
+// asc_expand: per-256 activation scales a256 [nsb][M] written out per 32-block, a32 [nsb * 8][M] (each scale eight
+// times): the matmul kernels take per-32 scales, and a chunk quantized with one scale per superblock (the reference's
+// act32 = 0, zero/kernels/ops.cl:38-72 and the non-ACT32 GEMM, zero/kernels/gemm.cl:489-520) runs through them with the
+// same integer sums and the same scale on each of a superblock's blocks.  grid: ceil(nsb * 8 * M / 256) x 256.
+extern "C" __global__ void asc_expand(const float* __restrict__ a256, float* __restrict__ a32, int M, int nsb) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (size_t)nsb * 8 * M) return;
+  const size_t row = i / M, m = i - row * M;
+  a32[i] = a256[(row >> 3) * M + m];
+}
+
 // fill32: p[i] = v for i < n (the fill used where a captured graph must not hold a memset node).
 extern "C" __global__ void fill32(uint32_t* p, uint32_t v, size_t n) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

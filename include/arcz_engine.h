@@ -49,7 +49,9 @@ int arcz_weight_set_softcap(arcz_weight* w, float cap);
 
 /* The activation quantizer as a step of its own (quant_store16 of zero/kernels/ops.cl:38-72 inside the launch of
  * zero/engine.h:1256-1267): rows [0, T) of x (f32, row stride ldx) -> the engine's aq / asc / absum laid out for
- * Mp rows; rows [T, Mp) are zero.  The next matmul takes its form from T: 1 GEMV, 2..8 multi-token GEMV, else GEMM. */
+ * Mp rows; rows [T, Mp) are zero.  The next matmul takes its form from T: 1 GEMV, 2..8 multi-token GEMV, else GEMM.
+ * act32 = 1: one scale per 32 values, asc [K/32][Mp]; act32 = 0: one per 256 (the maximum over the superblock), asc
+ * [K/256][Mp] (one-pass engines only).  The matmuls of that chunk take the same act32. */
 int arcz_engine_quantize(arcz_engine* e, arcz_mem* x, int ldx, int K, int Mp, int T, int act32);
 /* The fused producers (Engine::rmsnorm_quant, zero/engine.h:1256-1267, kernel zero/kernels/ops.cl:107-141; swiglu_quant,
  * zero/kernels/ops.cl:271-315 launched by run_rows_quant, zero/engine.h:1404-1440): rows [row_off, row_off + T) of x
@@ -86,7 +88,11 @@ arcz_mem* arcz_engine_asc(arcz_engine* e);
 arcz_mem* arcz_engine_absum(arcz_engine* e);
 
 /* Engine::matmul(name, w, Mp, C, ldc, c_off, acc, act32) (zero/engine.h:1080): C[:, c_off : c_off + N] (+)= act W^T
- * for the current chunk.  acc 0 = store, 1 = add to C, 2 = C = silu(C) * result (GEMM form only). */
+ * for the current chunk.  acc 0 = store, 1 = add to C, 2 = C = silu(C) * result (GEMM form only).  act32 must be what
+ * the chunk was quantized with (an error otherwise); with act32 = 0 the superblock's scale stands for each of its
+ * eight blocks (the reference's non-ACT32 kernels, zero/kernels/gemm.cl:489-520): the engine spreads it over a
+ * per-32 scale array of its own in one small launch and runs the same kernels.  The fused gate + up GEMV and the
+ * mixture-of-experts layer take per-32 chunks only. */
 int arcz_engine_matmul(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off, int acc,
                        int act32);
 

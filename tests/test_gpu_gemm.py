@@ -148,3 +148,33 @@ def test_startup_self_check(rt):
     """Tuned GEMM == simple GEMM == host integer sums, bit for bit, on the reference's LCG data with unit scales
     (the start-up check in the pattern of xmx_check, zero/engine_setup.h:424-520)."""
     az.self_check()
+
+
+@pytest.mark.parametrize("qtype", [az.Q4_K, az.Q6_K, az.Q8_0, az.Q4_0])
+@pytest.mark.parametrize("T,Mp,N,K", [(1, 16, 264, 1024), (5, 16, 136, 512), (100, 112, 272, 768), (64, 64, 130, 4096)])
+def test_per_256_activation_scales(eng, qtype, T, Mp, N, K):
+    """act32 = 0: one activation scale per superblock (the reference's quant_store16 with act32 = 0, zero/kernels/ops.cl:
+    38-72, and its non-ACT32 GEMM, gemm.cl:489-520).  The quantizer's output bit for bit against the oracle's, the
+    matmul against the double-accumulated reference with that one scale on each of a superblock's eight blocks."""
+    print(f"act32=0 {TYPE_NAMES[qtype]} T={T} Mp={Mp} N={N} K={K}", flush=True)
+    W = make_weights(qtype, N, K, seed=91)
+    x = make_acts(T, K, seed=92 + T, outliers=True)
+    w = eng.make_weight(qtype, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, Mp, T, act32=0)
+    xp = np.zeros((Mp, K), np.float32)
+    xp[:T] = x
+    raq, rasc, rabsum = orc.quantize_act(xp, act32=False)
+    assert np.array_equal(eng.aq.read(np.int8, Mp * K).reshape(Mp, K), raq)
+    assert np.array_equal(eng.asc.read(np.uint32, Mp * K // 256).reshape(K // 256, Mp), rasc.view(np.uint32))
+    rows = Mp if T > 8 else T
+    cb = az.Runtime.alloc(rows * N * 4).fill(0xFFFFFFFF)
+    with pytest.raises(az.ArczError):
+        eng.matmul("m", w, Mp, cb, N, 0, 0, act32=True)          # the chunk has per-256 scales
+    eng.matmul("m", w, Mp, cb, N, 0, 0, act32=False)
+    y = cb.read(np.float32, rows * N).reshape(rows, N)[:T]
+    ref = orc.matmul_ref(qtype, W, N, K, raq[:T], np.ascontiguousarray(np.repeat(rasc, 8, axis=0)))
+    assert np.isfinite(y).all() and rel_err_rows(y, ref).max() <= TOL
+    for b in (cb, xb):
+        b.free()
+    w.free()
