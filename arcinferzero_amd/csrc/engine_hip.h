@@ -925,7 +925,7 @@ class Engine {
       int FF = F, KK = E, MM = Mp;
       cl_mem tabs = nullptr;
       set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
-      size_t gws[2] = {(size_t)(F + 127) / 128 * 256, max_tiles}, lws[2] = {256, 1};
+      size_t gws[2] = {(size_t)(F + 127) / 128 * 256, (max_tiles + 7) / 8 * 8}, lws[2] = {256, 1};  // (a multiple of 8: moe_tile_of)
       run("moe_gateup", k, 2, gws, lws);
     } else {
       moe_gemm(L, 0, Mp, max_tiles);

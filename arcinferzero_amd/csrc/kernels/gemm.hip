@@ -309,27 +309,39 @@ __device__ __forceinline__ void gemm2_body(const uint8_t* __restrict__ raw, cons
     __syncthreads();
   }
 
-  // ---- epilogue: lane = weight row n, accumulator i = token row 8 * (i / 4) + 4 * g + i % 4
+  // ---- epilogue: lane = weight row n, accumulator i = token row 8 * (i / 4) + 4 * g + i % 4.  The slots' scales come
+  // from LDS (read from global memory between the stores, each load would wait for the stores before it: one counter
+  // orders both), and what the accumulate modes read of C is loaded for a whole tile before its first store.
+  if (TILES && use_scale) {
+    if (t < BM) L.sa[0][t] = t < rows_valid ? rowscale[m0 + t] : 0.0f;
+    __syncthreads();
+  }
 #pragma unroll
   for (int ms = 0; ms < 2; ++ms)
 #pragma unroll
     for (int ns = 0; ns < 2; ++ns) {
       const int n = n0 + wn * 64 + ns * 32 + l32;
       if (n >= N) continue;
+      float cv[16];
+      if (accumulate != 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int r = wm * 64 + ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+          cv[i] = r < rows_valid ? C[(size_t)(m0 + r) * ldc + c_off + n] : 0.0f;
+        }
+      }
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int r = wm * 64 + ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
         if (r >= rows_valid) continue;
         float v = res[ms][ns][i];
-        if (TILES && use_scale) v *= rowscale[m0 + r];
-        float* cp = C + (size_t)(m0 + r) * ldc + c_off + n;
+        if (TILES && use_scale) v *= L.sa[0][r];
         if (accumulate == 1) {
-          v += *cp;
+          v += cv[i];
         } else if (accumulate == 2) {  // fused SwiGLU: C holds the gate projection, v the up projection
-          const float gt = *cp;
-          v *= gt / (1.0f + __expf(-gt));
+          v *= cv[i] / (1.0f + __expf(-cv[i]));
         }
-        *cp = v;
+        C[(size_t)(m0 + r) * ldc + c_off + n] = v;
       }
     }
 }
@@ -628,6 +640,58 @@ struct G6ScaleRegs {
   uint32_t d;
 };
 
+// Epilogue of the 64-slot bodies (a wave holds all 64 slots of its 32 weight rows: lane = row, accumulator i of tile ms
+// = slot 32 ms + 8 (i / 4) + 4 g + i % 4) for a whole tile of 128 rows whose output rows are 16-byte aligned: the sums
+// go through LDS (the stages are free: every wave is past the last step's barrier), slot r at 528 r bytes behind the
+// slots' scales -- 16 bytes of padding keep the two lane halves, four slots apart, on different banks -- so that a
+// thread writes 16 bytes and a wave two whole 512-byte rows of the tile: 8 store instructions a lane instead of 32,
+// each over half as many lines.  What the accumulate modes read of C is loaded for all 8 before the first store, and
+// the slots' scales come from LDS: loads between the stores would each wait for the stores before them (one counter
+// orders both), 32 round trips to memory in a row.  false: not such a tile, nothing done (the caller's scalar path).
+__device__ __forceinline__ bool store_tile64(uint8_t* lds, const v16f (&res)[2], float* __restrict__ C, int ldc, int c_off,
+                                             int accumulate, int m0, int rows_valid, int n0, int N,
+                                             const float* __restrict__ rowscale, int use_scale) {
+  if (n0 + BN > N || ((ldc | c_off) & 3) != 0 || ((uintptr_t)C & 15) != 0) return false;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l32 = lane & 31, g = lane >> 5;
+  float* rs = (float*)lds;
+  uint8_t* tl = lds + 256;
+  if (use_scale && t < G6_BM) rs[t] = t < rows_valid ? rowscale[m0 + t] : 0.0f;
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      *(float*)(tl + (ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3)) * 528 + (wave * 32 + l32) * 4) = res[ms][i];
+  const int c4 = t & 31, rr = t >> 5;
+  float* cp = C + (size_t)(m0 + rr) * ldc + c_off + n0 + 4 * c4;
+  float4 cv[8];
+  if (accumulate != 0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      cv[i] = rr + 8 * i < rows_valid ? *(const float4*)(cp + (size_t)8 * i * ldc) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = rr + 8 * i;
+    if (r >= rows_valid) continue;
+    float4 v = *(const float4*)(tl + r * 528 + c4 * 16);
+    if (use_scale) {
+      const float sc = rs[r];
+      v.x *= sc; v.y *= sc; v.z *= sc; v.w *= sc;
+    }
+    if (accumulate == 1) {
+      v.x += cv[i].x; v.y += cv[i].y; v.z += cv[i].z; v.w += cv[i].w;
+    } else if (accumulate == 2) {  // fused SwiGLU: C holds the gate projection, v the up projection
+      v.x *= cv[i].x / (1.0f + __expf(-cv[i].x));
+      v.y *= cv[i].y / (1.0f + __expf(-cv[i].y));
+      v.z *= cv[i].z / (1.0f + __expf(-cv[i].z));
+      v.w *= cv[i].w / (1.0f + __expf(-cv[i].w));
+    }
+    *(float4*)(cp + (size_t)8 * i * ldc) = v;
+  }
+  return true;
+}
+
 // TILES: one expert tile -- the planes hold rows_total rows, the expert's N rows start at row_base, slot r of the tile
 // reads token row rowmap[m0 + r] (use_map) and its results are scaled by rowscale[m0 + r] (use_scale).
 template <bool TILES = false>
@@ -803,6 +867,7 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
   }
 
   // ---- epilogue: lane = weight row n, accumulator i = token row 8 * (i / 4) + 4 * g + i % 4
+  if (store_tile64(lds, res, C, ldc, c_off, accumulate, m0, rows_valid, n0, N, rowscale, TILES && use_scale)) return;
   const int n = n0 + wave * 32 + l32;
   if (n < N) {
 #pragma unroll
@@ -1046,6 +1111,9 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
   }
 
   // ---- epilogue: lane = weight row n, accumulator i = token row 8 * (i / 4) + 4 * g + i % 4
+  if constexpr (TWO) {
+    if (store_tile64(lds, res, C, ldc, c_off, accumulate, m0, rows_valid, n0, N, rowscale, use_scale)) return;
+  }
   const int n = n0 + wave * 32 + l32;
   if (n < N) {
 #pragma unroll
@@ -1289,6 +1357,15 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
 
   // ---- epilogue: lane = row n of the stream, accumulator i = slot 8 * (i / 4) + 4 * g + i % 4
   if constexpr (GU) {
+    v16f hv[2];
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float gt = res[0][ms][i];
+        hv[ms][i] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
+      }
+    if (store_tile64(lds, hv, H, N, 0, 0, m0, rows_valid, n0, N, nullptr, 0)) return;
     const int n = n0 + wave * 32 + l32;
     if (n < N) {
 #pragma unroll
@@ -1297,8 +1374,7 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
         for (int i = 0; i < 16; ++i) {
           const int r = ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
           if (r >= rows_valid) continue;
-          const float gt = res[0][ms][i];
-          H[(size_t)(m0 + r) * N + n] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
+          H[(size_t)(m0 + r) * N + n] = hv[ms][i];
         }
     }
   } else {
@@ -1326,20 +1402,35 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
   }
 }
 
+// The (tile, row chunk) a work-group of a tile kernel takes, nc row chunks a tile, grid (nc, tile work-groups) with the
+// tile work-groups a multiple of 8.  The XCDs take work-groups in turn (linear id % 8) and each has its own L2, so the
+// tile list, which is sorted by expert, is cut into 8 runs, one per XCD, and the work-groups of an XCD walk their run
+// in groups of 4 tiles, row chunk by row chunk: four neighbours read the same rows of an expert (mostly: an expert of
+// 256 slots has 4 or 5 tiles), and the 4 nc work-groups of a group the same slots' activations, out of one L2.  Every
+// tile and chunk is taken exactly once; work-groups beyond their XCD's run do nothing (false).
+__device__ inline bool moe_tile_of(int nt, int nc, int& ti, int& chunk) {
+  const int id = blockIdx.x + gridDim.x * blockIdx.y, x = id & 7, j = id >> 3;
+  const int t0 = (int)(((long long)nt * x) >> 3), t1 = (int)(((long long)nt * (x + 1)) >> 3);  // this XCD's tiles
+  if (j >= (t1 - t0) * nc) return false;
+  const int grp = j / (4 * nc), first = t0 + 4 * grp, in_grp = min(4, t1 - first);  // (the run's last group may be short)
+  const int r = j - grp * 4 * nc;
+  chunk = r / in_grp;
+  ti = first + r - chunk * in_grp;
+  return true;
+}
+
 // moe_gateup_q: arguments as the reference's (zero/kernels/decode_moe.cl:92-94) -- the two raw expert tensors
 // [NE][F][K], the tile list (tiles of at most 64 slots), stok = the token row of every slot, h [slots][F] -- and, as its
-// extra arguments, the activations' sums per 16 values.  grid (ceil(F / 128) * 256, tile work-groups): work-group y
-// takes tiles y, y + gridDim.y, ...
+// extra arguments, the activations' sums per 16 values.  grid (ceil(F / 128) * 256, tile work-groups: the most tiles
+// there can be, rounded up to a multiple of 8): one tile and row chunk a work-group, dealt by moe_tile_of.
 extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12(
     const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc,
     int M, const int* tiles, const int* stok, float* h, const short* absum, int NE) {
-  const int nt = tiles[0];
-  for (int ti = blockIdx.y; ti < nt; ti += gridDim.y) {
-    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-    gemm4gu_body<true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), blockIdx.x * BN,
-                       stok, 0, 0, 0);
-    __syncthreads();
-  }
+  int ti, chunk;
+  if (!moe_tile_of(tiles[0], gridDim.x, ti, chunk)) return;
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm4gu_body<true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), chunk * BN, stok,
+                     0, 0, 0);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
