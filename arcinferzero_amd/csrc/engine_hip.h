@@ -780,7 +780,8 @@ class Engine {
       cl_mem unused = nullptr;
       set_args(k, 0, wx.raw, unused, i == 2 ? mhq_ : aq_, i == 2 ? mhsc_ : asc_, i == 2 ? mhbs_ : absum_, i == 2 ? my_ : mh_, M, NN, KK,
                ldc, acc, mtiles_, mtstart_, e0, e1, stok_, um, swt_, us);
-      size_t gws[2] = {(size_t)(N + 127) / 128 * 256, max_tiles}, lws[2] = {256, 1};
+      // (tile work-groups in a multiple of 8: the kernels deal tiles to the XCDs in runs of the expert-sorted list)
+      size_t gws[2] = {(size_t)(N + 127) / 128 * 256, (max_tiles + 7) / 8 * 8}, lws[2] = {256, 1};
       run(i == 2 ? "moe_down" : "moe_gateup", k, 2, gws, lws);
     }
   }

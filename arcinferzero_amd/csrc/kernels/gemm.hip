@@ -41,6 +41,28 @@ struct alignas(16) Gemm2Lds {
   int rowmap[BM];
 };
 
+// The (tile, row chunk) a work-group of a tile kernel takes, nc row chunks a tile, grid (nc, tile work-groups) with the
+// tile work-groups at least the tiles there are, and a multiple of 8.  The XCDs take work-groups in turn (linear id % 8) and each has its own L2, so the
+// tile list, which is sorted by expert, is cut into 8 runs, one per XCD, and the work-groups of an XCD walk their run
+// in groups of 4 tiles, row chunk by row chunk: four neighbours read the same rows of an expert (mostly: an expert of
+// 256 slots has 4 or 5 tiles), and the 4 nc work-groups of a group the same slots' activations, out of one L2.  Every
+// tile and chunk is taken exactly once; work-groups beyond their XCD's run do nothing (false).
+__device__ inline bool moe_tile_of(int nt, int nc, int& ti, int& chunk) {
+  if (gridDim.y & 7) {  // (a launch of another shape: work-group (x, y) takes chunk x of tile y)
+    ti = blockIdx.y;
+    chunk = blockIdx.x;
+    return ti < nt;
+  }
+  const int id = blockIdx.x + gridDim.x * blockIdx.y, x = id & 7, j = id >> 3;
+  const int t0 = (int)(((long long)nt * x) >> 3), t1 = (int)(((long long)nt * (x + 1)) >> 3);  // this XCD's tiles
+  if (j >= (t1 - t0) * nc) return false;
+  const int grp = j / (4 * nc), first = t0 + 4 * grp, in_grp = min(4, t1 - first);  // (the run's last group may be short)
+  const int r = j - grp * 4 * nc;
+  chunk = r / in_grp;
+  ti = first + r - chunk * in_grp;
+  return true;
+}
+
 // The global loads of one K step, held in registers until the step before it has been computed.
 // (native vector types: arrays of HIP's uint4, a struct, stay in scratch memory when they are passed around)
 typedef uint32_t g2_u4 __attribute__((ext_vector_type(4)));
@@ -1402,23 +1424,6 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
   }
 }
 
-// The (tile, row chunk) a work-group of a tile kernel takes, nc row chunks a tile, grid (nc, tile work-groups) with the
-// tile work-groups a multiple of 8.  The XCDs take work-groups in turn (linear id % 8) and each has its own L2, so the
-// tile list, which is sorted by expert, is cut into 8 runs, one per XCD, and the work-groups of an XCD walk their run
-// in groups of 4 tiles, row chunk by row chunk: four neighbours read the same rows of an expert (mostly: an expert of
-// 256 slots has 4 or 5 tiles), and the 4 nc work-groups of a group the same slots' activations, out of one L2.  Every
-// tile and chunk is taken exactly once; work-groups beyond their XCD's run do nothing (false).
-__device__ inline bool moe_tile_of(int nt, int nc, int& ti, int& chunk) {
-  const int id = blockIdx.x + gridDim.x * blockIdx.y, x = id & 7, j = id >> 3;
-  const int t0 = (int)(((long long)nt * x) >> 3), t1 = (int)(((long long)nt * (x + 1)) >> 3);  // this XCD's tiles
-  if (j >= (t1 - t0) * nc) return false;
-  const int grp = j / (4 * nc), first = t0 + 4 * grp, in_grp = min(4, t1 - first);  // (the run's last group may be short)
-  const int r = j - grp * 4 * nc;
-  chunk = r / in_grp;
-  ti = first + r - chunk * in_grp;
-  return true;
-}
-
 // moe_gateup_q: arguments as the reference's (zero/kernels/decode_moe.cl:92-94) -- the two raw expert tensors
 // [NE][F][K], the tile list (tiles of at most 64 slots), stok = the token row of every slot, h [slots][F] -- and, as its
 // extra arguments, the activations' sums per 16 values.  grid (ceil(F / 128) * 256, tile work-groups: the most tiles
@@ -1629,8 +1634,8 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
 
 // gemm over expert tiles (reference zero/kernels/gemm.cl:146-161, -DMOE_TILES): W holds all experts' rows (N each);
 // tile t of the list = (expert, first slot, rows <= 128) from moe_scan; slot r reads token row rowmap[r] (use_map) or
-// r, writes C row r, times rowscale[r] (use_scale).  Experts [e0, e1).  grid (ceil(N / 128), tile work-groups):
-// work-group y loops over tiles y, y + gridDim.y, ...
+// r, writes C row r, times rowscale[r] (use_scale).  Experts [e0, e1).  grid (ceil(N / 128), tile work-groups >= the
+// tiles of those experts): one tile and row chunk a work-group, dealt by moe_tile_of.
 #define GEMM2_TILES_INST(QT)                                                                                         \
   extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE##QT##_ACT321_MOE_TILES1(                           \
       const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum,      \
@@ -1638,11 +1643,12 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
       const int* rowmap, int use_map, const float* rowscale, int use_scale, int NE) {                                 \
     /* one tile a work-group (grid.y covers the most tiles there can be, as the reference launches it,              \
        zero/engine_moe.h:153): as a loop over tiles the body spilled 15-45 registers */                              \
-    const int ti = tstart[e0] + blockIdx.y;                                                                           \
-    if (ti >= tstart[e1]) return;                                                                                     \
+    int ti, chunk;                                                                                                    \
+    if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;                                          \
+    ti += tstart[e0];                                                                                                 \
     const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];                                  \
     gemm2_body<QT, true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,  \
-                         min(nr, BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);                         \
+                         min(nr, BM), chunk * BN, rowmap, use_map, rowscale, use_scale);                              \
   }
 
 GEMM2_INST(8)
@@ -1839,13 +1845,12 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TI
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
     int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
     int use_map, const float* rowscale, int use_scale, int NE) {
-  const int t_end = tstart[e1];
-  for (int ti = tstart[e0] + blockIdx.y; ti < t_end; ti += gridDim.y) {
-    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-    gemm4_body<true>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,
-                     min(nr, G6_BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
-    __syncthreads();
-  }
+  int ti, chunk;  // one tile and row chunk a work-group (as a loop over tiles the body spilled registers)
+  if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;
+  ti += tstart[e0];
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm4_body<true>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,
+                   min(nr, G6_BM), chunk * BN, rowmap, use_map, rowscale, use_scale);
 }
 
 // (Q5_K experts: the same body, one tile of at most 64 slots per work-group)
@@ -1853,11 +1858,12 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_MOE_TI
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
     int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
     int use_map, const float* rowscale, int use_scale, int NE) {
-  const int ti = tstart[e0] + blockIdx.y;
-  if (ti >= tstart[e1]) return;
+  int ti, chunk;
+  if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;
+  ti += tstart[e0];
   const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
   gemm4_body<true, QT_Q5_K>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N,
-                            r0, min(nr, G6_BM), blockIdx.x * BN, rowmap, use_map, rowscale, use_scale);
+                            r0, min(nr, G6_BM), chunk * BN, rowmap, use_map, rowscale, use_scale);
 }
 
 // Q6_K: the dense form has its own body (64-token tiles: grid ceil(N / 128) * ceil(M / 64) work-groups); the form over
@@ -1876,11 +1882,10 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_MOE_TI
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
     int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
     int use_map, const float* rowscale, int use_scale, int NE) {
-  const int t_end = tstart[e1];
-  for (int ti = tstart[e0] + blockIdx.y; ti < t_end; ti += gridDim.y) {
-    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-    gemm6_body<true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, r0, min(nr, G6_BM), blockIdx.x * BN,
-                     (size_t)NE * N, (size_t)e * N, rowmap, use_map, rowscale, use_scale);
-    __syncthreads();
-  }
+  int ti, chunk;
+  if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;
+  ti += tstart[e0];
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm6_body<true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, r0, min(nr, G6_BM), chunk * BN,
+                   (size_t)NE * N, (size_t)e * N, rowmap, use_map, rowscale, use_scale);
 }
