@@ -95,14 +95,22 @@ class Engine {
   void alloc_activations() {
     const size_t M = (size_t)max_chunk, f = q2mm_ ? 2 : 1;
     aq_ = buf(M * max_k * f);
-    asc_ = buf(M * (max_k / 32) * 4 * f);
+    // (+ 512 bytes: the prefill GEMM's last token tile reads its scale vectors in whole 128-token rows)
+    asc_ = buf(M * (max_k / 32) * 4 * f + 512);
     absum_ = buf(M * (max_k / 16) * 2 * f);
-    if (!asc_rep_) asc_rep_ = buf(M * (max_k / 32) * 4);
+    if (!asc_rep_) asc_rep_ = buf(M * (max_k / 32) * 4 + 512);
+    if (!au_) au_ = buf(M * (max_k / 32) * 4 + 512);
   }
   // Per-256 activation scales (act32 = 0: the reference's choice for insensitive inputs when its act32_all is off,
   // zero/engine.h:1254): the quantizers store one scale per superblock, asc [K/256][M]; the matmul kernels here take
   // per-32 scales, so a matmul of such a chunk first writes each scale out eight times into asc_rep_ and reads that.
   cl_mem asc_rep_ = nullptr;
+  // sa * S per 32-block and token of the current matmul's input (act_usum), for the Q4_K / Q5_K prefill GEMM
+  cl_mem au_ = nullptr;
+  // d * sc and -(dmin * mn) per 32-block and row of the current matmul's Q4_K / Q5_K matrix (q4k_wscales), written in
+  // front of a GEMM of many tokens; sized when such a matrix is uploaded (the largest one), never in a matmul
+  cl_mem wsv_ = nullptr;
+  size_t wsv_bytes_ = 0;
   int cur_act32_ = 1;
   // Two-pass matmul inputs (zero/engine.h:1034-1075 q2_init, the mode of the reference's Gemma 4 and Qwen3 models):
   // every producer also quantizes what its int8 values miss, v - q * scale, the same way, into the second half of the
@@ -219,6 +227,16 @@ class Engine {
     std::vector<uint8_t> planes(pb);
     if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
     w.raw = buf(pb, planes.data());
+    if ((type == GGML_Q4_K || type == GGML_Q5_K) && rows == (size_t)N) {  // (room for its rows' scale vectors, gemm_dense)
+      const size_t need = (size_t)2 * N * (K / 32) * 4 + 1024;
+      if (need > wsv_bytes_) {
+        if (wsv_) release(wsv_);
+        wsv_ = nullptr;
+        wsv_bytes_ = 0;
+        wsv_ = buf(need);
+        wsv_bytes_ = need;
+      }
+    }
     if (type == GGML_IQ3_S) {  // (room for its GEMM form)
       const size_t need = raw_planes_bytes(QT_Q6_K, rows, K / 256);
       if (need > xw_bytes_) {
@@ -640,9 +658,17 @@ class Engine {
     static const int q4_bn = getenv("ARCZ_Q4_BN") ? atoi(getenv("ARCZ_Q4_BN")) : 0;
     static const int q4_small_max = getenv("ARCZ_Q4_SMALL") ? atoi(getenv("ARCZ_Q4_SMALL")) : 0;
     const bool q4_small = w.type == GGML_Q4_K && (q4_bn == 128 || (q4_bn == 0 && Mp <= q4_small_max));
+    // Q4_K / Q5_K in 128 x 128 tiles: the token side's scale vectors ready-made (-DAU; ARCZ_Q4_AU=0: formed in the kernel)
+    static const int q4_au = getenv("ARCZ_Q4_AU") ? atoi(getenv("ARCZ_Q4_AU")) : 2;
+    const bool au = q4_au && (w.type == GGML_Q4_K || w.type == GGML_Q5_K) && !q4_wide && !q4_small && M % 4 == 0;
+    // ... and the row side's too (-DAU=2) when the chunk is long enough to pay for writing them (8 bytes per 32
+    // weights: 22 MB, about 8 us, for 17408 x 5120): ARCZ_Q4_AU=1 never, ARCZ_Q4_AU2_MIN=n from n token rows on
+    static const int au2_min = getenv("ARCZ_Q4_AU2_MIN") ? atoi(getenv("ARCZ_Q4_AU2_MIN")) : 1024;
+    const bool au2 = au && q4_au >= 2 && Mp >= au2_min && N % 4 == 0 && (size_t)2 * N * (K / 32) * 4 + 1024 <= wsv_bytes_;
     cl_kernel k = q8_small  ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
                   : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")
                   : q4_wide ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64", "gemm")
+                  : au      ? kernel("gemm", "-DQTYPE=" + std::to_string(w.type) + (au2 ? " -DACT32 -DAU=2" : " -DACT32 -DAU"), "gemm")
                             : gemm_kernel(w.type, false);
     // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
     //  registers over the whole of K.  The reference splits rows longer than 8192 into 17-superblock pieces for its
@@ -654,9 +680,26 @@ class Engine {
     const int bn = q4_wide && !q4_small ? 256 : 128;
     const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + bn - 1) / bn);
     size_t gws[1] = {tiles * 256}, lws[1] = {256};
+    if (au) {
+      cl_kernel ku = kernel("ops", "", "act_usum");
+      set_args(ku, 0, asc_, absum_, M, au_);
+      size_t g2[2] = {(size_t)(M + 255) / 256 * 256, (size_t)(K / 32)}, l2[2] = {256, 1};
+      run("act_usum", ku, 2, g2, l2);
+      unused = au_;
+    }
+    cl_mem sums = absum_;
+    if (au2) {
+      cl_kernel kw = kernel("ops", "", "q4k_wscales");
+      size_t hdr = planes_q4k((size_t)N, K / 256).hdr;
+      int NN = N, nsb2 = K / 256;
+      set_args(kw, 0, w.raw, hdr, NN, nsb2, wsv_);
+      size_t g2[2] = {(size_t)(N + 255) / 256 * 256, (size_t)(K / 256)}, l2[2] = {256, 1};
+      run("q4k_wscales", kw, 2, g2, l2);
+      sums = wsv_;
+    }
     for (int sp = 0; sp < splits; ++sp) {
       int s0 = nsb * sp / splits, s1 = nsb * (sp + 1) / splits, ac = sp == 0 ? a : 1;
-      set_args(k, 0, w.raw, unused, aq_, asc_, absum_, C, M, N, K, ldc, c_off, ac, rgroup, s0, s1);
+      set_args(k, 0, w.raw, unused, aq_, asc_, sums, C, M, N, K, ldc, c_off, ac, rgroup, s0, s1);
       run(name, k, 1, gws, lws);
     }
   }

@@ -26,6 +26,8 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "add_norm_quant", nullptr, "pppiffpiipppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
+    {"ops", "act_usum", nullptr, "ppip", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "q4k_wscales", nullptr, "pziip", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "asc_expand", nullptr, "ppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "softcap_rows", nullptr, "piiif", {nullptr}, {{nullptr, 0, false}}, 0},
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},
@@ -54,6 +56,7 @@ static const KernelSpec kKernelTable[] = {
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm", "SPLITK", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", "BN", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "AU", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "AU", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", "BM", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},

@@ -397,14 +397,25 @@ struct G3ScaleRegs {
 
 // QT = Q5_K: the same with the fifth bits of a step's 128 values per row (16 bytes of the qh plane) brought into LDS by
 // one more DMA instruction of the first two waves, and merged into the nibbles when a lane reads its operand.
-template <bool TILES, int QT = QT_Q4_K>  // (only the dense form is instantiated: over expert tiles, with their short K,
-                                         //  the register-staged body above measured faster)
+// AU: the token side's two scale vectors come ready-made and go into LDS by DMA like the int8 rows -- asc itself and
+// au[K / 32][M] = sa * S (act_usum in ops.hip makes it once per matmul) -- one more DMA instruction a wave and step in
+// the place of six loads, the products and four LDS stores per thread; M must be a multiple of 4, the tile's first
+// row of 128, and 512 bytes past the end of both arrays readable (rows past the chunk's last take what lies there:
+// their results are not stored).
+// PRE = 2: the row side's vectors too -- wsv = ws[K / 32][N] (d * sc) followed by v[K / 32][N] (-(dmin * mn)), made by
+// q4k_wscales in front of a matmul of many tokens -- N a multiple of 4, 512 readable bytes past each: no scale
+// arithmetic, no loads into registers and no LDS stores are left in the loop.
+template <bool TILES, int QT = QT_Q4_K, int PRE = 0>  // (only the dense form is instantiated: over expert tiles,
+                                                     //  with their short K, the register-staged body measured faster)
 __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
                                   int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
                                   size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
                                   const int* __restrict__ rowmap, int use_map, const float* __restrict__ rowscale,
-                                  int use_scale) {
+                                  int use_scale, const float* __restrict__ au = nullptr,
+                                  const float* __restrict__ wsv = nullptr) {
+  constexpr bool AU = PRE >= 1, WS = PRE >= 2;
+  static_assert(!(AU && TILES), "the ready-made scale vectors are rows of the dense chunk");
   constexpr bool Q5 = QT == QT_Q5_K;
   constexpr int STAGE = Q5 ? G3_STAGE + 2048 : G3_STAGE, QH = G3_STAGE;  // (the fifth bits behind the scale vectors)
   __shared__ alignas(16) uint8_t lds[2 * STAGE];
@@ -447,11 +458,26 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
   const uint32_t hoff = (uint32_t)n_s * (uint32_t)nsb * 16u;
   const uint8_t* hbase = raw + pl.hdr + (row_base * nsb + s_begin) * 16;
+  // AU: waves 0 and 1 bring sa of blocks (0, 1) and (2, 3) of the step, waves 2 and 3 sa * S of the same: lane l the
+  // four tokens 4 (l % 32) .. + 3 of block 2 (wave % 2) + l / 32
+  const uint8_t* sbase = (const uint8_t*)(wave < 2 ? asc : au) + (size_t)s_begin * 8 * M * 4;
+  uint32_t soff = ((uint32_t)(2 * (wave & 1) + (lane >> 5)) * (uint32_t)M + (uint32_t)m0 + 4u * (lane & 31)) * 4u;
+  // WS: the same split for the row side: waves 0 and 1 d * sc, waves 2 and 3 -(dmin * mn), rows n0 + 4 (l % 32) .. + 3
+  const uint8_t* rbase = (const uint8_t*)wsv + ((wave < 2 ? (size_t)0 : (size_t)(K >> 5) * N) + (size_t)s_begin * 8 * N) * 4;
+  uint32_t roff = ((uint32_t)(2 * (wave & 1) + (lane >> 5)) * (uint32_t)N + (uint32_t)n0 + 4u * (lane & 31)) * 4u;
 
   auto dma_step = [&](int st, int stage) {  // st: half-superblock steps from s_begin
     uint8_t* base = lds + stage * STAGE;
     const signed char* ab = abase + (size_t)st * 128;
     const uint8_t* wb = wbase + (size_t)st * 64;
+    if constexpr (AU) {
+      asm volatile("" : "+v"(soff));
+      g3_dma16(sbase + (size_t)st * 4 * M * 4 + soff, base + (wave < 2 ? G3_SA : G3_U) + (wave & 1) * 1024);
+    }
+    if constexpr (WS) {
+      asm volatile("" : "+v"(roff));
+      g3_dma16(rbase + (size_t)st * 4 * N * 4 + roff, base + (wave < 2 ? G3_WS : G3_V) + (wave & 1) * 1024);
+    }
     // (the offsets pass through an empty asm so that the 64-bit addresses are formed here, each step, and not kept in
     //  twelve registers over the whole loop)
 #pragma unroll
@@ -469,23 +495,28 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   };
   // (loads only: anything computed from them here would make the wave wait for the whole step's traffic)
   auto load_scales = [&](G3ScaleRegs& r, int st) {
-    const float* ap = asc + (size_t)(s_begin * 8 + st * 4 + 2 * bp) * M;
-    const short* bp2 = absum + (size_t)(s_begin * 16 + st * 8 + 4 * bp) * M;
-    r.sa[0] = ap[m_s];
-    r.sa[1] = (ap + M)[m_s];
-    r.bs[0] = bp2[m_s];
-    r.bs[1] = (bp2 + M)[m_s];
-    r.bs[2] = (bp2 + 2 * (size_t)M)[m_s];
-    r.bs[3] = (bp2 + 3 * (size_t)M)[m_s];
-    r.h = *(const uint4*)(hbase + (size_t)(st >> 1) * 16 + hoff);
+    if constexpr (!AU) {
+      const float* ap = asc + (size_t)(s_begin * 8 + st * 4 + 2 * bp) * M;
+      const short* bp2 = absum + (size_t)(s_begin * 16 + st * 8 + 4 * bp) * M;
+      r.sa[0] = ap[m_s];
+      r.sa[1] = (ap + M)[m_s];
+      r.bs[0] = bp2[m_s];
+      r.bs[1] = (bp2 + M)[m_s];
+      r.bs[2] = (bp2 + 2 * (size_t)M)[m_s];
+      r.bs[3] = (bp2 + 3 * (size_t)M)[m_s];
+    }
+    if constexpr (!WS) r.h = *(const uint4*)(hbase + (size_t)(st >> 1) * 16 + hoff);
   };
   auto store_scales = [&](const G3ScaleRegs& r, int st, int stage) {
     uint8_t* base = lds + stage * STAGE;
+    if constexpr (WS) return;
+    if constexpr (!AU) {
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const float sa = tok_valid ? r.sa[q] : 0.0f;
-      ((float*)(base + G3_SA))[(2 * bp + q) * 128 + r_s] = sa;
-      ((float*)(base + G3_U))[(2 * bp + q) * 128 + r_s] = sa * (float)((int)r.bs[2 * q] + (int)r.bs[2 * q + 1]);
+      for (int q = 0; q < 2; ++q) {
+        const float sa = tok_valid ? r.sa[q] : 0.0f;
+        ((float*)(base + G3_SA))[(2 * bp + q) * 128 + r_s] = sa;
+        ((float*)(base + G3_U))[(2 * bp + q) * 128 + r_s] = sa * (float)((int)r.bs[2 * q] + (int)r.bs[2 * q + 1]);
+      }
     }
     const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
     int sc0, sc1, mn0, mn1;
@@ -1840,6 +1871,43 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321(
   gemm3_body<false, QT_Q5_K>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
                              min(BM, M - m0), n0, nullptr, 0, nullptr, 0);
 }
+// -DAU: the same two kernels with the token side's scale vectors ready-made (gemm3_body<..., AU>): the second argument,
+// unused otherwise, is au[K / 32][M] = sa * S; M a multiple of 4.  No counterpart in the reference.
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_AU1(
+    const uint8_t* raw, const uint8_t* au, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  gemm3_body<false, QT_Q4_K, 1>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                                min(BM, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_AU1(
+    const uint8_t* raw, const uint8_t* au, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  gemm3_body<false, QT_Q5_K, 1>(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                                min(BM, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au);
+}
+// -DAU=2: the row side's scale vectors ready-made as well: wsv (q4k_wscales) stands in absum's place, which the kernel
+// no longer reads.  N a multiple of 4.
+#define GEMM3_AU2_INST(QT)                                                                                           \
+  extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE##QT##_ACT321_AU2(                                  \
+      const uint8_t* raw, const uint8_t* au, const signed char* aq, const float* asc, const short* wsv, float* C,     \
+      int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {                  \
+    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;                                                         \
+    int tm, tn;                                                                                                       \
+    tile_of(blockIdx.x, mt, nt, tm, tn);                                                                              \
+    const int m0 = tm * BM, n0 = tn * BN;                                                                             \
+    gemm3_body<false, QT, 2>(raw, aq, asc, nullptr, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, \
+                             m0, min(BM, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au, (const float*)wsv);   \
+  }
+GEMM3_AU2_INST(12)
+GEMM3_AU2_INST(13)
 // (tiles of at most 64 slots: the engine builds the tile list for that size)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TILES1(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,

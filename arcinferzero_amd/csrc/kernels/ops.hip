@@ -301,6 +301,42 @@ extern "C" __global__ __launch_bounds__(256) void add_norm_quant(float* __restri
   }
 }
 
+// act_usum: au[b][m] = sa * S for every 32-block b and token m of a chunk, S the sum of the block's int8 values
+// (absum's two halves): the min term's token-side factor, which the prefill GEMM otherwise forms per work-group and
+// step, made once per matmul so that it can go into LDS by DMA.  The same expression as in the kernel: the same bits.
+// No counterpart in the reference.  grid (ceil(M / 256) * 256, K / 32), local (256, 1).
+extern "C" __global__ __launch_bounds__(256) void act_usum(const float* __restrict__ asc, const short* __restrict__ absum,
+                                                           int M, float* __restrict__ au) {
+  const int m = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+  if (m >= M) return;
+  const float sa = asc[(size_t)b * M + m];
+  au[(size_t)b * M + m] = sa * (float)((int)absum[(size_t)(2 * b) * M + m] + (int)absum[(size_t)(2 * b + 1) * M + m]);
+}
+
+// q4k_wscales: the row side's scale vectors of a Q4_K / Q5_K matrix (the two share the header plane at hdr_off bytes
+// into the raw planes) for the prefill GEMM: ws[b][n] = d * sc_b and, N * K / 32 floats further on, v[b][n] =
+// -(dmin * mn_b), the expressions of the kernel's own scale preparation (the same bits), written once in front of a
+// matmul of many tokens instead of once per 128-token tile and step.  No counterpart in the reference.
+// grid (ceil(N / 256) * 256, K / 256), local (256, 1).
+extern "C" __global__ __launch_bounds__(256) void q4k_wscales(const uint8_t* __restrict__ raw, size_t hdr_off, int N, int nsb,
+                                                              float* __restrict__ wsv) {
+  const int n = blockIdx.x * 256 + threadIdx.x, sb = blockIdx.y;
+  if (n >= N) return;
+  const uint4 h = *(const uint4*)(raw + hdr_off + ((size_t)n * nsb + sb) * 16);
+  const float d = f16_bits_to_f32(h.x), dmin = f16_bits_to_f32(h.x >> 16);
+  float* ws = wsv + (size_t)sb * 8 * N + n;
+  float* v = ws + (size_t)nsb * 8 * N;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int sc0, sc1, mn0, mn1;
+    q4k_scales_pair(h.y, h.z, h.w, j, sc0, sc1, mn0, mn1);
+    ws[(size_t)(2 * j) * N] = d * (float)sc0;
+    ws[(size_t)(2 * j + 1) * N] = d * (float)sc1;
+    v[(size_t)(2 * j) * N] = -(dmin * (float)mn0);
+    v[(size_t)(2 * j + 1) * N] = -(dmin * (float)mn1);
+  }
+}
+
 // swiglu_quant: y = silu(gate) * up (or the tanh form of gelu(gate) * up) from rows [gate(F) | up(F)], or the row as it
 // is when the matmul before has fused the product (`fused`), quantized with K = F (reference zero/kernels/ops.cl:
 // 271-315, same arguments; silu(x) = x / (1 + exp(-x)), ops.cl:33).  grid (256 * G, rows), local (256, 1).

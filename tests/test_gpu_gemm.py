@@ -178,3 +178,30 @@ def test_per_256_activation_scales(eng, qtype, T, Mp, N, K):
     for b in (cb, xb):
         b.free()
     w.free()
+
+
+@pytest.mark.parametrize("qtype", [az.Q4_K, az.Q5_K])
+@pytest.mark.parametrize("T,Mp,N,K,acc", [(1100, 1104, 392, 512, 0), (1100, 1104, 390, 512, 0), (1030, 1040, 640, 768, 1),
+                                          (760, 768, 520, 1024, 2), (1200, 1216, 132, 256, 0)])
+def test_gemm_ready_made_scale_vectors(rt, qtype, T, Mp, N, K, acc):
+    """The 128 x 128 Q4_K / Q5_K kernel whose scale vectors are written by small kernels in front of it (token side: sa and
+    sa * S; row side, from 1024 token rows on when N is a multiple of 4: d * sc and -(dmin * mn)) and go into LDS by DMA:
+    chunks whose last token tile and last row tile are partly empty, so that the whole-row reads run into the next
+    block's entries and past the arrays' ends; the three epilogues.  Against the oracle, and run to run."""
+    print(f"ready-made scales {TYPE_NAMES[qtype]} T={T} Mp={Mp} N={N} K={K} acc={acc}", flush=True)
+    eng = az.Engine(Mp, K)            # (an engine of exactly this chunk: the arrays end where the chunk ends)
+    W = make_weights(qtype, N, K, seed=71)
+    x = make_acts(T, K, seed=72, outliers=True)
+    c0 = np.random.default_rng(73).standard_normal((Mp, N)).astype(np.float32)
+    y = run_gemm(eng, qtype, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
+    y2 = run_gemm(eng, qtype, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
+    eng.close()
+    assert np.array_equal(y.view(np.uint32), y2.view(np.uint32))
+    aq, asc, _ = quantize_padded(x, Mp)
+    ref = orc.matmul_ref(qtype, W, N, K, aq[:T], np.ascontiguousarray(asc[:, :T]))
+    if acc == 1:
+        ref = ref + c0[:T]
+    elif acc == 2:
+        g = c0[:T].astype(np.float64)
+        ref = ref * (g / (1.0 + np.exp(-g)))
+    assert np.isfinite(y).all() and mixed_err(y, ref) <= TOL
