@@ -493,6 +493,31 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
       if (wave < 2) g3_dma16(qbase + (size_t)st * 16 + qoff, base + QH + wave * 1024);
     }
   };
+  // the same instructions one at a time (piece 0..7; Q5_K: 8 as well), for the forms that issue them between the
+  // products instead of all at the head of the step: the memory pipe takes a wave's instruction every ~16 cycles and
+  // eight waves of the compute unit ask at once, so a wave that issues all of its loads first stands in that queue
+  // before its first product
+  auto dma_piece = [&](int st, int stage, int piece) {
+    uint8_t* base = lds + stage * STAGE;
+    if (piece < 4) {
+      asm volatile("" : "+v"(aoff[piece]));
+      g3_dma16(abase + (size_t)st * 128 + aoff[piece], base + (wave * 4 + piece) * 1024);
+    } else if (piece < 6) {
+      asm volatile("" : "+v"(woff[piece - 4]));
+      g3_dma16(wbase + (size_t)st * 64 + woff[piece - 4], base + G3_WQ + (wave * 2 + piece - 4) * 1024);
+    } else if (piece == 6) {
+      asm volatile("" : "+v"(soff));
+      g3_dma16(sbase + (size_t)st * 4 * M * 4 + soff, base + (wave < 2 ? G3_SA : G3_U) + (wave & 1) * 1024);
+    } else if (piece == 7) {
+      if constexpr (WS) {
+        asm volatile("" : "+v"(roff));
+        g3_dma16(rbase + (size_t)st * 4 * N * 4 + roff, base + (wave < 2 ? G3_WS : G3_V) + (wave & 1) * 1024);
+      }
+    } else if constexpr (Q5) {  // (no branch: waves 2 and 3 bring what waves 0 and 1 bring, to the same place)
+      asm volatile("" : "+v"(qoff));
+      g3_dma16(qbase + (size_t)st * 16 + qoff, base + QH + (wave & 1) * 1024);
+    }
+  };
   // (loads only: anything computed from them here would make the wave wait for the whole step's traffic)
   auto load_scales = [&](G3ScaleRegs& r, int st) {
     if constexpr (!AU) {
@@ -557,7 +582,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
     const uint8_t* Sb = lds + (st & 1) * STAGE;
     const bool next = st + 1 < steps;
     if (next) {  // the other stage is free: every wave has passed the barrier that ended the step reading it
-      dma_step(st + 1, (st + 1) & 1);
+      if constexpr (!AU) dma_step(st + 1, (st + 1) & 1);  // (AU: one piece per product phase, below)
       load_scales(sr, st + 1);
     }
 
@@ -628,6 +653,10 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
           mfma_p(0);
           mfma_i(0, 0, 0);
           ld_a(b + 1, 1); ld_sa(b + 1, 1);
+        }
+        if constexpr (AU) {  // the next step's loads, one instruction per phase over the first nine (no branch: the
+                             //  last step brings its own stage once more, into the stage nobody reads)
+          if (4 * b + tile < 9) dma_piece(next ? st + 1 : st, (st + 1) & 1, 4 * b + tile);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
