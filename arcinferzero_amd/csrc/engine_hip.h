@@ -962,19 +962,26 @@ class Engine {
     moe_route(L, rl, ldl, T, tm);
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)
     const size_t max_tiles = (size_t)(n + tm - 1) / tm + std::min(n, L.NE);
+    bool quant_fused = false;
     if (L.ex[0].type == GGML_Q4_K && L.ex[1].type == GGML_Q4_K) {
       // gate and up in one pass (the reference's moe_gateup_q, zero/kernels/decode_moe.cl:92-94, launched by
       // zero/engine_moe.h:300-330): h = silu(gate) * up into mh_
-      cl_kernel k = kernel("gemm", "-DQT=12 -DNE=" + std::to_string(L.NE), "moe_gateup_q");
-      int FF = F, KK = E, MM = Mp;
+      // ... and, when F is whole tiles of 128 rows, the expert inputs' quantization in the same kernel's epilogue
+      // (-DQUANT=1: hq / hsc / hbs as moe_quant_sums makes them, bit for bit; ARCZ_MOE_QFUSE=0: the separate launch)
+      quant_fused = F % 128 == 0 && !(getenv("ARCZ_MOE_QFUSE") && atoi(getenv("ARCZ_MOE_QFUSE")) == 0);
+      cl_kernel k = kernel("gemm", std::string(quant_fused ? "-DQT=12 -DQUANT=1 -DNE=" : "-DQT=12 -DNE=") + std::to_string(L.NE), "moe_gateup_q");
+      int FF = F, KK = E, MM = Mp, S = slots_;
       cl_mem tabs = nullptr;
-      set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
+      if (quant_fused)
+        set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_, S, mhq_, mhsc_, mhbs_);
+      else
+        set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
       size_t gws[2] = {(size_t)(F + 127) / 128 * 256, (max_tiles + 7) / 8 * 8}, lws[2] = {256, 1};  // (a multiple of 8: moe_tile_of)
       run("moe_gateup", k, 2, gws, lws);
     } else {
       moe_gemm(L, 0, Mp, max_tiles);
     }
-    {
+    if (!quant_fused) {
       // (the reference's moe_quant writes no sums; the Q4_K tile GEMM here takes them for its min term)
       cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_quant_sums");
       int FF = F, S = slots_;

@@ -63,6 +63,7 @@ static const KernelSpec kKernelTable[] = {
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "splitk_reduce", nullptr, "pipiiiii", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "moe_gateup_q", "QUANT", "ppiipppippppippp", {"QT", "QUANT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     // ---- moe
     {"moe", "moe_route", "ESCALE", "piippppp", {"ESCALE", nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},

@@ -23,6 +23,7 @@
 // and B the weight tile, so a lane owns one weight row n and writes 128-byte runs of C.  Work-groups are numbered so
 // that the 64 that run together on one XCD form an 8 x 8 block of tiles and share their operands in that XCD's L2.
 #include "common.h"
+#include "quant.h"
 
 #define BM 128
 #define BN 128
@@ -774,6 +775,60 @@ __device__ __forceinline__ bool store_tile64(uint8_t* lds, const v16f (&res)[2],
   return true;
 }
 
+// The gate/up tile's h = silu(gate) * up, stored as store_tile64 stores it, and quantized on the way out as the expert
+// inputs' quantizer does (moe_quant_sums in moe.hip: per 32 values amax, q = rte(v * (127 / amax)), scale amax / 127,
+// the sums of 16 -- the same helper, the same bits): the tile lies in LDS slot-major for the stores, a thread takes
+// two half blocks of 16 values (neighbouring lanes the two halves of a block), writes their int8 values, and the
+// scales and sums leave through LDS in rows of 64 slots.  hq [S][F], hsc [F/32][S], hbs [F/16][S].  Whole tiles of 128
+// rows only (F a multiple of 128).
+__device__ __forceinline__ void store_tile64_quant(uint8_t* lds, const v16f (&hv)[2], float* __restrict__ H, int F, int m0,
+                                                   int rows_valid, int n0, int S, signed char* __restrict__ hq,
+                                                   float* __restrict__ hsc, short* __restrict__ hbs) {
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l32 = lane & 31, g = lane >> 5;
+  uint8_t* tl = lds + 256;
+  float* lasc = (float*)(lds + 256 + 64 * 528);       // [4][64]
+  short* lsum = (short*)(lds + 256 + 64 * 528 + 1024);  // [8][64]
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      *(float*)(tl + (ms * 32 + 8 * (i >> 2) + 4 * g + (i & 3)) * 528 + (wave * 32 + l32) * 4) = hv[ms][i];
+  __syncthreads();
+  const int c4 = t & 31, rr = t >> 5;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = rr + 8 * i;
+    if (r < rows_valid) *(float4*)(H + (size_t)(m0 + r) * F + n0 + 4 * c4) = *(const float4*)(tl + r * 528 + c4 * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = t + 256 * i, hb = idx & 7, r = idx >> 3;
+    float v[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 f = *(const float4*)(tl + r * 528 + hb * 64 + q * 16);
+      v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+    }
+    const float amax = block_amax(v, 1);
+    uint4 pk;
+    int sum;
+    quant16(v, amax, pk, sum);
+    if (r < rows_valid) *(uint4*)(hq + (size_t)(m0 + r) * F + n0 + hb * 16) = pk;
+    if ((hb & 1) == 0) lasc[(hb >> 1) * 64 + r] = amax / 127.0f;
+    lsum[hb * 64 + r] = (short)sum;
+  }
+  __syncthreads();
+  {
+    const int b = t >> 6, r = t & 63;
+    if (r < rows_valid) hsc[((size_t)(n0 >> 5) + b) * S + m0 + r] = lasc[b * 64 + r];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int hb = b + 4 * i;
+      if (r < rows_valid) hbs[((size_t)(n0 >> 4) + hb) * S + m0 + r] = lsum[hb * 64 + r];
+    }
+  }
+}
+
 // TILES: one expert tile -- the planes hold rows_total rows, the expert's N rows start at row_base, slot r of the tile
 // reads token row rowmap[m0 + r] (use_map) and its results are scaled by rowscale[m0 + r] (use_scale).
 template <bool TILES = false>
@@ -1242,12 +1297,14 @@ struct GuScaleRegs {
 
 // GU: the two streams are gate and up of an expert (rows n0.. of both tensors, h = silu(gate) * up); otherwise they are
 // rows n0.. and n0 + 128.. of one matrix and each gets the plain epilogue (a 64 x 256 tile of a dense product).
-template <bool GU>
+template <bool GU, bool QUANT = false>
 __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
                                     const signed char* __restrict__ aq, const float* __restrict__ asc,
                                     const short* __restrict__ absum, float* __restrict__ H, int M, int N, int K,
                                     size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
-                                    const int* __restrict__ rowmap, int ldc, int c_off, int accumulate) {
+                                    const int* __restrict__ rowmap, int ldc, int c_off, int accumulate, int S = 0,
+                                    signed char* __restrict__ hq = nullptr, float* __restrict__ hsc = nullptr,
+                                    short* __restrict__ hbs = nullptr) {
   __shared__ alignas(16) uint8_t lds[2 * GU_STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
@@ -1447,6 +1504,10 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
         const float gt = res[0][ms][i];
         hv[ms][i] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
       }
+    if constexpr (QUANT) {
+      store_tile64_quant(lds, hv, H, N, m0, rows_valid, n0, S, hq, hsc, hbs);
+      return;
+    }
     if (store_tile64(lds, hv, H, N, 0, 0, m0, rows_valid, n0, N, nullptr, 0)) return;
     const int n = n0 + wave * 32 + l32;
     if (n < N) {
@@ -1496,6 +1557,18 @@ extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12(
   const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
   gemm4gu_body<true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), chunk * BN, stok,
                      0, 0, 0);
+}
+// -DQUANT=1: with the expert inputs' quantization done on the way out (store_tile64_quant): h as before and
+// hq [S][F], hsc [F/32][S], hbs [F/16][S], what moe_quant_sums would make of h, bit for bit.  F a multiple of 128.
+extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12_QUANT1(
+    const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc,
+    int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,
+    short* hbs, int NE) {
+  int ti, chunk;
+  if (!moe_tile_of(tiles[0], gridDim.x, ti, chunk)) return;
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm4gu_body<true, true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), chunk * BN,
+                           stok, 0, 0, 0, S, hq, hsc, hbs);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

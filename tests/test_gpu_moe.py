@@ -106,6 +106,17 @@ def test_moe_small_pass_other_forms(rt, monkeypatch, env, qtype, NE, NU, E, F, T
     _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, 16)
 
 
+@pytest.mark.parametrize("env", [{}, {"ARCZ_MOE_QFUSE": "0"}])
+@pytest.mark.parametrize("NE,NU,E,F,T,Mp", [(16, 4, 512, 256, 300, 304), (8, 2, 256, 512, 70, 80), (8, 3, 256, 768, 90, 96)])
+def test_moe_tile_pass_quantization_forms(rt, monkeypatch, env, NE, NU, E, F, T, Mp):
+    """Q4_K experts, a tile pass: the expert inputs quantized in the gate/up kernel's epilogue (F a multiple of 128, the
+    default) and by the separate launch (ARCZ_MOE_QFUSE=0): the layer checks hold
+    for both, among them hq / hsc / hbs bit for bit what the quantizer makes of the GPU's own h."""
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    _moe_layer_vs_oracle(az.Q4_K, NE, NU, E, F, T, Mp)
+
+
 def _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp):
     print(f"moe layer {TYPE_NAMES[qtype]} NE={NE} NU={NU} E={E} F={F} T={T}", flush=True)
     eng = az.Engine(Mp, max(E, F))
