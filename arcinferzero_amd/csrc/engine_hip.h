@@ -515,10 +515,16 @@ class Engine {
       if (fits) {
         const int pf = (units + lpr - 1) / lpr, tb = tbl;
         // one round of resident work-groups, passes of rows dealt to them in turn (ARCZ_GEMV_WPC: work-groups per
-        // compute unit; two measured best: more add staging work and spread the reads over more rows at a time)
+        // compute unit).  One token: one work-group a compute unit -- measured at the settled clock against two, us per
+        // launch: Q4_K 17408 x 5120 10.56 / 10.66, 5120 x 17408 10.93 / 11.84, 4096 x 4096 4.25 / 4.69, 1024 x 5120
+        // 5.13 / 5.74, Q6_K 151936 x 5120 107.7 / 111.5, Q5_K 13.11 / 13.42 -- except for the codebook types, whose
+        // decode wants the second work-group's waves (IQ4_XS 13.24 / 12.95).  More tokens: two (four tokens at
+        // 17408 x 5120: 20.2 against 25.7 with one; three or four per unit are slower everywhere).
         static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
         static const int wgs_env = getenv("ARCZ_GEMV_WGS") ? atoi(getenv("ARCZ_GEMV_WGS")) : 0;
-        size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * (wpc_env > 0 ? wpc_env : bt == 512 ? 1 : 2));
+        const bool codebook = w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S;
+        const int wpc = wpc_env > 0 ? wpc_env : bt == 512 || (tb == 1 && !codebook) ? 1 : 2;
+        size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * wpc);
         if (wgs_env > 0) wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)wgs_env);
         const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
                                  std::to_string(pf) + (tb > 1 ? " -DTB=" + std::to_string(tb) : std::string()) +
@@ -580,7 +586,8 @@ class Engine {
     cl_mem tabs = tabs_;
     int NN = N, KK = K, M = Mp, c_off = 0, a = 0;
     set_args(k, 0, g.raw, NN, KK, tabs, aq_, asc_, absum_, M, C, c_off, a, u.raw);
-    const size_t wgs = std::min<size_t>((size_t)2 * N / gr, (size_t)arcz_device_cus() * 2);
+    static const int gu_wpc = getenv("ARCZ_GEMV_GU_WPC") ? atoi(getenv("ARCZ_GEMV_GU_WPC")) : 1;  // (17.6 against 18.2 us with two)
+    const size_t wgs = std::min<size_t>((size_t)2 * N / gr, (size_t)arcz_device_cus() * gu_wpc);
     size_t g1 = wgs * 256, l1 = 256;
     run("gemm_gate_up", k, 1, &g1, &l1);
     return true;
