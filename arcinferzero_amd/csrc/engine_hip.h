@@ -99,7 +99,7 @@ class Engine {
     asc_ = buf(M * (max_k / 32) * 4 * f + 512);
     absum_ = buf(M * (max_k / 16) * 2 * f);
     if (!asc_rep_) asc_rep_ = buf(M * (max_k / 32) * 4 + 512);
-    if (!au_) au_ = buf(M * (max_k / 32) * 4 + 512);
+    if (!au_) au_ = buf(M * (max_k / 32) * 8 + 1024);  // (entries of 4 bytes, or 8: the bf16 pieces)
   }
   // Per-256 activation scales (act32 = 0: the reference's choice for insensitive inputs when its act32_all is off,
   // zero/engine.h:1254): the quantizers store one scale per superblock, asc [K/256][M]; the matmul kernels here take
@@ -228,7 +228,7 @@ class Engine {
     if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
     w.raw = buf(pb, planes.data());
     if ((type == GGML_Q4_K || type == GGML_Q5_K) && rows == (size_t)N) {  // (room for its rows' scale vectors, gemm_dense)
-      const size_t need = (size_t)2 * N * (K / 32) * 4 + 1024;
+      const size_t need = (size_t)N * (K / 32) * 20 + 4096;  // (4 + 4 bytes a block and row, or 4 + 16: the bf16 pieces)
       if (need > wsv_bytes_) {
         if (wsv_) release(wsv_);
         wsv_ = nullptr;
@@ -666,16 +666,20 @@ class Engine {
     static const int q4_small_max = getenv("ARCZ_Q4_SMALL") ? atoi(getenv("ARCZ_Q4_SMALL")) : 0;
     const bool q4_small = w.type == GGML_Q4_K && (q4_bn == 128 || (q4_bn == 0 && Mp <= q4_small_max));
     // Q4_K / Q5_K in 128 x 128 tiles: the token side's scale vectors ready-made (-DAU; ARCZ_Q4_AU=0: formed in the kernel)
-    static const int q4_au = getenv("ARCZ_Q4_AU") ? atoi(getenv("ARCZ_Q4_AU")) : 2;
+    static const int q4_au = getenv("ARCZ_Q4_AU") ? atoi(getenv("ARCZ_Q4_AU")) : 3;
     const bool au = q4_au && (w.type == GGML_Q4_K || w.type == GGML_Q5_K) && !q4_wide && !q4_small && M % 4 == 0;
     // ... and the row side's too (-DAU=2) when the chunk is long enough to pay for writing them (8 bytes per 32
     // weights: 22 MB, about 8 us, for 17408 x 5120): ARCZ_Q4_AU=1 never, ARCZ_Q4_AU2_MIN=n from n token rows on
     static const int au2_min = getenv("ARCZ_Q4_AU2_MIN") ? atoi(getenv("ARCZ_Q4_AU2_MIN")) : 1024;
-    const bool au2 = au && q4_au >= 2 && Mp >= au2_min && N % 4 == 0 && (size_t)2 * N * (K / 32) * 4 + 1024 <= wsv_bytes_;
+    const bool au2 = au && q4_au >= 2 && Mp >= au2_min && N % 4 == 0 && (size_t)N * (K / 32) * 20 + 4096 <= wsv_bytes_;
+    // ... and, Q4_K from 2048 token rows on, the min term's operands as bf16 pieces (-DAU=3: 20 bytes per block and
+    // row to write, 56 MB for 17408 x 5120; ARCZ_Q4_AU=2 never, ARCZ_Q4_AU3_MIN=n from n token rows on)
+    static const int au3_min = getenv("ARCZ_Q4_AU3_MIN") ? atoi(getenv("ARCZ_Q4_AU3_MIN")) : 2048;
+    const bool au3 = au2 && q4_au >= 3 && w.type == GGML_Q4_K && Mp >= au3_min;
     cl_kernel k = q8_small  ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
                   : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")
                   : q4_wide ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64", "gemm")
-                  : au      ? kernel("gemm", "-DQTYPE=" + std::to_string(w.type) + (au2 ? " -DACT32 -DAU=2" : " -DACT32 -DAU"), "gemm")
+                  : au      ? kernel("gemm", "-DQTYPE=" + std::to_string(w.type) + (au3 ? " -DACT32 -DAU=3" : au2 ? " -DACT32 -DAU=2" : " -DACT32 -DAU"), "gemm")
                             : gemm_kernel(w.type, false);
     // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
     //  registers over the whole of K.  The reference splits rows longer than 8192 into 17-superblock pieces for its
@@ -688,7 +692,7 @@ class Engine {
     const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + bn - 1) / bn);
     size_t gws[1] = {tiles * 256}, lws[1] = {256};
     if (au) {
-      cl_kernel ku = kernel("ops", "", "act_usum");
+      cl_kernel ku = kernel("ops", "", au3 ? "act_usum_bf16" : "act_usum");
       set_args(ku, 0, asc_, absum_, M, au_);
       size_t g2[2] = {(size_t)(M + 255) / 256 * 256, (size_t)(K / 32)}, l2[2] = {256, 1};
       run("act_usum", ku, 2, g2, l2);
@@ -696,7 +700,7 @@ class Engine {
     }
     cl_mem sums = absum_;
     if (au2) {
-      cl_kernel kw = kernel("ops", "", "q4k_wscales");
+      cl_kernel kw = kernel("ops", "", au3 ? "q4k_wscales_bf16" : "q4k_wscales");
       size_t hdr = planes_q4k((size_t)N, K / 256).hdr;
       int NN = N, nsb2 = K / 256;
       set_args(kw, 0, w.raw, hdr, NN, nsb2, wsv_);

@@ -170,6 +170,17 @@ __device__ inline int dot4_first(uint32_t a, uint32_t b) {
   return r;
 }
 
+// x = x1 + x2 + x3 exactly, each piece a bf16 (x1 the top 8 significant bits by truncation, x2 the next 8, x3 the
+// rest); w0 = x1 | x2 << 16, w1 = x3 (as bf16 bit patterns).
+__device__ inline void split3(float x, uint32_t& w0, uint32_t& w1) {
+  const uint32_t p1 = __float_as_uint(x) & 0xFFFF0000u;
+  const float r1 = x - __uint_as_float(p1);
+  const uint32_t p2 = __float_as_uint(r1) & 0xFFFF0000u;
+  const float r2 = r1 - __uint_as_float(p2);
+  w0 = (p1 >> 16) | p2;
+  w1 = __float_as_uint(r2) >> 16;
+}
+
 // Sum over the 32 lanes of a half wave (lanes 0-31 and 32-63 separately), same value in every lane; a fixed tree,
 // so results do not depend on anything but the inputs.
 // The steps within a row of 16 lanes are data-parallel moves in the vector ALU (neighbour, other pair, other quad,

@@ -378,6 +378,9 @@ __device__ __forceinline__ void gemm2_body(const uint8_t* __restrict__ raw, cons
 // by choosing its source address, and which makes the 128-bit operand reads conflict-free.  Only the four scale vectors
 // of a step pass through registers (they need arithmetic); S, the block sums of the activations, come from absum.
 // One barrier per step.
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+__device__ inline v8bf as_bf16x8(v4u v) { return __builtin_bit_cast(v8bf, v); }
 #define G3_STAGE 32768
 #define G3_WQ 16384
 #define G3_SA 24576
@@ -406,6 +409,14 @@ struct G3ScaleRegs {
 // PRE = 2: the row side's vectors too -- wsv = ws[K / 32][N] (d * sc) followed by v[K / 32][N] (-(dmin * mn)), made by
 // q4k_wscales in front of a matmul of many tokens -- N a multiple of 4, 512 readable bytes past each: no scale
 // arithmetic, no loads into registers and no LDS stores are left in the loop.
+// PRE = 3 (Q4_K): the min term on the bf16 matrix instruction, which runs beside the vector ALU's work where the f32
+// one does not (measured in this kernel: without the min term a launch takes 13 % less, with it on the bf16
+// instruction 8 % less).  A float x is x1 + x2 + x3 exactly, three bf16 pieces by truncation; of the nine products of
+// two such splits the eight without x3 y3 carry everything above 2^-32 of the product and fill the eight k-slots a
+// lane half has in v_mfma_f32_32x32x16_bf16 (bf16 products are exact in f32, the sum is f32).  The pieces come
+// ready-made: au[K / 32][M] entries (u1 | u2 << 16, u3 | u3 << 16), and behind ws in wsv v[K / 32][N] entries
+// (v1 v1, v2 v2, v3 v3, v1 v2); a lane's token-side operand is the words (x, x, x, y) of its entry, its row-side
+// operand the entry as it lies.  M even, 1 KB and 2 KB past the arrays' ends readable.  A stage is 40 KB.
 template <bool TILES, int QT = QT_Q4_K, int PRE = 0>  // (only the dense form is instantiated: over expert tiles,
                                                      //  with their short K, the register-staged body measured faster)
 __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
@@ -418,7 +429,12 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   constexpr bool AU = PRE >= 1, WS = PRE >= 2;
   static_assert(!(AU && TILES), "the ready-made scale vectors are rows of the dense chunk");
   constexpr bool Q5 = QT == QT_Q5_K;
-  constexpr int STAGE = Q5 ? G3_STAGE + 2048 : G3_STAGE, QH = G3_STAGE;  // (the fifth bits behind the scale vectors)
+  constexpr bool BF = PRE >= 3;
+  static_assert(!(BF && Q5), "the bf16 min-term form is built for Q4_K");
+  // the scale vectors of a stage: f32 per block and token / row (2 KB each), or, BF: sa, ws as before, then the min
+  // term's operands, 8 bytes per block and token (4 KB) and 16 per block and row (8 KB): a stage of 40 KB
+  constexpr int oSA = G3_SA, oWS = BF ? G3_SA + 2048 : G3_WS, oU = BF ? G3_SA + 4096 : G3_U, oV = BF ? G3_SA + 8192 : G3_V;
+  constexpr int STAGE = BF ? G3_SA + 16384 : Q5 ? G3_STAGE + 2048 : G3_STAGE, QH = G3_STAGE;  // (Q5_K: the fifth bits behind the scale vectors)
   __shared__ alignas(16) uint8_t lds[2 * STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -466,19 +482,21 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   // WS: the same split for the row side: waves 0 and 1 d * sc, waves 2 and 3 -(dmin * mn), rows n0 + 4 (l % 32) .. + 3
   const uint8_t* rbase = (const uint8_t*)wsv + ((wave < 2 ? (size_t)0 : (size_t)(K >> 5) * N) + (size_t)s_begin * 8 * N) * 4;
   uint32_t roff = ((uint32_t)(2 * (wave & 1) + (lane >> 5)) * (uint32_t)N + (uint32_t)n0 + 4u * (lane & 31)) * 4u;
+  // BF: waves 0 and 1 bring sa (asc), waves 2 and 3 d * sc (the f32 half of wsv), two blocks each as above; then wave w
+  // the min term's operands of block w of the step: 128 token entries of 8 bytes (au: one instruction, lane l tokens
+  // 2 l, 2 l + 1) and 128 row entries of 16 bytes (behind the f32 half of wsv: two instructions, lane l row 64 i + l)
+  const uint8_t* fbase = wave < 2 ? (const uint8_t*)asc + (size_t)s_begin * 8 * M * 4 : (const uint8_t*)wsv + (size_t)s_begin * 8 * N * 4;
+  const uint32_t fstep = 16u * (uint32_t)(wave < 2 ? M : N);  // (bytes of four blocks' f32 entries)
+  uint32_t foff = wave < 2 ? soff : roff;
+  const uint8_t* ubase = (const uint8_t*)au + ((size_t)s_begin * 8 + wave) * M * 8;
+  uint32_t uoff = ((uint32_t)m0 + 2u * lane) * 8u;
+  const uint8_t* vbase = (const uint8_t*)wsv + (size_t)(K >> 5) * N * 4 + ((size_t)s_begin * 8 + wave) * N * 16;
+  uint32_t voff = ((uint32_t)n0 + lane) * 16u;
 
   auto dma_step = [&](int st, int stage) {  // st: half-superblock steps from s_begin
     uint8_t* base = lds + stage * STAGE;
     const signed char* ab = abase + (size_t)st * 128;
     const uint8_t* wb = wbase + (size_t)st * 64;
-    if constexpr (AU) {
-      asm volatile("" : "+v"(soff));
-      g3_dma16(sbase + (size_t)st * 4 * M * 4 + soff, base + (wave < 2 ? G3_SA : G3_U) + (wave & 1) * 1024);
-    }
-    if constexpr (WS) {
-      asm volatile("" : "+v"(roff));
-      g3_dma16(rbase + (size_t)st * 4 * N * 4 + roff, base + (wave < 2 ? G3_WS : G3_V) + (wave & 1) * 1024);
-    }
     // (the offsets pass through an empty asm so that the 64-bit addresses are formed here, each step, and not kept in
     //  twelve registers over the whole loop)
 #pragma unroll
@@ -506,13 +524,24 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
     } else if (piece < 6) {
       asm volatile("" : "+v"(woff[piece - 4]));
       g3_dma16(wbase + (size_t)st * 64 + woff[piece - 4], base + G3_WQ + (wave * 2 + piece - 4) * 1024);
+    } else if constexpr (BF) {
+      if (piece == 6) {
+        asm volatile("" : "+v"(foff));
+        g3_dma16(fbase + (size_t)st * fstep + foff, base + (wave < 2 ? oSA : oWS) + (wave & 1) * 1024);
+      } else if (piece == 7) {
+        asm volatile("" : "+v"(uoff));
+        g3_dma16(ubase + (size_t)st * 4 * M * 8 + uoff, base + oU + wave * 1024);
+      } else if (piece < 10) {
+        asm volatile("" : "+v"(voff));
+        g3_dma16(vbase + (size_t)st * 4 * N * 16 + voff + (piece - 8) * 1024, base + oV + wave * 2048 + (piece - 8) * 1024);
+      }
     } else if (piece == 6) {
       asm volatile("" : "+v"(soff));
-      g3_dma16(sbase + (size_t)st * 4 * M * 4 + soff, base + (wave < 2 ? G3_SA : G3_U) + (wave & 1) * 1024);
+      g3_dma16(sbase + (size_t)st * 4 * M * 4 + soff, base + (wave < 2 ? oSA : oU) + (wave & 1) * 1024);
     } else if (piece == 7) {
       if constexpr (WS) {
         asm volatile("" : "+v"(roff));
-        g3_dma16(rbase + (size_t)st * 4 * N * 4 + roff, base + (wave < 2 ? G3_WS : G3_V) + (wave & 1) * 1024);
+        g3_dma16(rbase + (size_t)st * 4 * N * 4 + roff, base + (wave < 2 ? oWS : oV) + (wave & 1) * 1024);
       }
     } else if constexpr (Q5) {  // (no branch: waves 2 and 3 bring what waves 0 and 1 bring, to the same place)
       asm volatile("" : "+v"(qoff));
@@ -540,18 +569,18 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const float sa = tok_valid ? r.sa[q] : 0.0f;
-        ((float*)(base + G3_SA))[(2 * bp + q) * 128 + r_s] = sa;
-        ((float*)(base + G3_U))[(2 * bp + q) * 128 + r_s] = sa * (float)((int)r.bs[2 * q] + (int)r.bs[2 * q + 1]);
+        ((float*)(base + oSA))[(2 * bp + q) * 128 + r_s] = sa;
+        ((float*)(base + oU))[(2 * bp + q) * 128 + r_s] = sa * (float)((int)r.bs[2 * q] + (int)r.bs[2 * q + 1]);
       }
     }
     const float d = f16_bits_to_f32(r.h.x), dmin = f16_bits_to_f32(r.h.x >> 16);
     int sc0, sc1, mn0, mn1;
     q4k_scales_pair(r.h.y, r.h.z, r.h.w, 2 * (st & 1) + p_s, sc0, sc1, mn0, mn1);
     const int row = t >> 1;
-    ((float*)(base + G3_WS))[(2 * p_s) * 128 + row] = d * (float)sc0;
-    ((float*)(base + G3_WS))[(2 * p_s + 1) * 128 + row] = d * (float)sc1;
-    ((float*)(base + G3_V))[(2 * p_s) * 128 + row] = -(dmin * (float)mn0);
-    ((float*)(base + G3_V))[(2 * p_s + 1) * 128 + row] = -(dmin * (float)mn1);
+    ((float*)(base + oWS))[(2 * p_s) * 128 + row] = d * (float)sc0;
+    ((float*)(base + oWS))[(2 * p_s + 1) * 128 + row] = d * (float)sc1;
+    ((float*)(base + oV))[(2 * p_s) * 128 + row] = -(dmin * (float)mn0);
+    ((float*)(base + oV))[(2 * p_s + 1) * 128 + row] = -(dmin * (float)mn1);
   };
 
   // ---- operand addresses of this lane (bytes from a stage's start)
@@ -572,7 +601,12 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   const int steps = 2 * (s_end - s_begin);
   G3ScaleRegs sr;
   if (steps > 0) {
-    dma_step(0, 0);
+    if constexpr (AU) {
+#pragma unroll
+      for (int p = 0; p < 10; ++p) dma_piece(0, 0, p);
+    } else {
+      dma_step(0, 0);
+    }
     load_scales(sr, 0);
     store_scales(sr, 0, 0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the stage has landed
@@ -590,6 +624,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
     v4i a16[2], w16[2], wraw[2];
     uint32_t h5[2];  // Q5_K: the fifth bits of the unit in wraw
     float saop[2], wsop, uop[2], vop[2];
+    v4u uopb[2], vopb[2];  // BF: the min term's bf16 operands
     v32f P[2];
     v16i I[2];
     auto ld_a = [&](int b, int ms) { a16[ms] = *(const v4i*)(Sb + oa[b] + ms * 32 * 128); };
@@ -606,8 +641,8 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
           w16[ns][i] = (b & 1) ? (int)(((uint32_t)wraw[ns][i] >> 4) & 0x0F0F0F0Fu) : (int)((uint32_t)wraw[ns][i] & 0x0F0F0F0Fu);
       }
     };
-    auto ld_sa = [&](int b, int ms) { saop[ms] = ((const float*)(Sb + G3_SA))[b * 128 + wm * 64 + ms * 32 + l32]; };
-    auto ld_ws = [&](int b) { wsop = ((const float*)(Sb + G3_WS))[b * 128 + wn * 64 + lane]; };
+    auto ld_sa = [&](int b, int ms) { saop[ms] = ((const float*)(Sb + oSA))[b * 128 + wm * 64 + ms * 32 + l32]; };
+    auto ld_ws = [&](int b) { wsop = ((const float*)(Sb + oWS))[b * 128 + wn * 64 + lane]; };
     auto mfma_p = [&](int ms) {
       v32f zf;
 #pragma unroll
@@ -629,9 +664,21 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
       const bool more = b + 1 < 4;
       if ((b & 1) == 0) {  // min term of blocks b and b + 1: lane half g supplies block b + g
 #pragma unroll
-        for (int ms = 0; ms < 2; ++ms) uop[ms] = ((const float*)(Sb + G3_U))[(b + g) * 128 + wm * 64 + ms * 32 + l32];
+        for (int ms = 0; ms < 2; ++ms) {
+          if constexpr (BF) {  // slots (u1 u2 | u1 u2 | u1 u2 | u3 u3) against the row side's (v1 v1 | v2 v2 | v3 v3 | v1 v2)
+            const uint2 e = ((const uint2*)(Sb + oU))[(b + g) * 128 + wm * 64 + ms * 32 + l32];
+            uopb[ms] = v4u{e.x, e.x, e.x, e.y};
+          } else {
+            uop[ms] = ((const float*)(Sb + oU))[(b + g) * 128 + wm * 64 + ms * 32 + l32];
+          }
+        }
 #pragma unroll
-        for (int ns = 0; ns < 2; ++ns) vop[ns] = ((const float*)(Sb + G3_V))[(b + g) * 128 + wn * 64 + ns * 32 + l32];
+        for (int ns = 0; ns < 2; ++ns) {
+          if constexpr (BF)
+            vopb[ns] = *(const v4u*)(Sb + oV + ((b + g) * 128 + wn * 64 + ns * 32 + l32) * 16);
+          else
+            vop[ns] = ((const float*)(Sb + oV))[(b + g) * 128 + wn * 64 + ns * 32 + l32];
+        }
       }
 #pragma unroll
       for (int tile = 0; tile < 4; ++tile) {
@@ -657,13 +704,18 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
         }
         if constexpr (AU) {  // the next step's loads, one instruction per phase over the first nine (no branch: the
                              //  last step brings its own stage once more, into the stage nobody reads)
-          if (4 * b + tile < 9) dma_piece(next ? st + 1 : st, (st + 1) & 1, 4 * b + tile);
+          if (4 * b + tile < (BF ? 10 : 9)) dma_piece(next ? st + 1 : st, (st + 1) & 1, 4 * b + tile);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 16; ++i)
           res[ms][ns][i] = __builtin_fmaf((float)I[slot][i], P[ms][16 * ns + i], res[ms][ns][i]);
-        if ((b & 1) == 0) res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop[ns], res[ms][ns], 0, 0, 0);
+        if ((b & 1) == 0) {
+          if constexpr (BF)
+            res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(uopb[ms]), as_bf16x8(vopb[ns]), res[ms][ns], 0, 0, 0);
+          else
+            res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop[ms], vop[ns], res[ms][ns], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -2010,6 +2062,18 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_AU1(
   }
 GEMM3_AU2_INST(12)
 GEMM3_AU2_INST(13)
+// -DAU=3: Q4_K with the min term on the bf16 matrix instruction: au and wsv hold the operands' pieces (act_usum_bf16,
+// q4k_wscales_bf16).  M even, N a multiple of 4.
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_AU3(
+    const uint8_t* raw, const uint8_t* au, const signed char* aq, const float* asc, const short* wsv, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  gemm3_body<false, QT_Q4_K, 3>(raw, aq, asc, nullptr, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                                min(BM, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au, (const float*)wsv);
+}
 // (tiles of at most 64 slots: the engine builds the tile list for that size)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TILES1(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,

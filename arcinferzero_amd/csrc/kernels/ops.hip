@@ -337,6 +337,43 @@ extern "C" __global__ __launch_bounds__(256) void q4k_wscales(const uint8_t* __r
   }
 }
 
+// The same two vectors as operands of the bf16 matrix instruction (the prefill GEMM's min term, its -DAU=3 form):
+// x = x1 + x2 + x3 exactly, each piece a bf16 by truncation (split3).  act_usum_bf16: au[b][m] = (u1 | u2 << 16,
+// u3 | u3 << 16) of u = sa * S.  q4k_wscales_bf16: ws[b][n] = d * sc as f32, then v[b][n] = (v1 v1, v2 v2, v3 v3, v1 v2)
+// of v = -(dmin * mn), 16 bytes an entry.  Grids as act_usum and q4k_wscales.
+extern "C" __global__ __launch_bounds__(256) void act_usum_bf16(const float* __restrict__ asc, const short* __restrict__ absum,
+                                                                int M, uint2* __restrict__ au) {
+  const int m = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+  if (m >= M) return;
+  const float sa = asc[(size_t)b * M + m];
+  const float u = sa * (float)((int)absum[(size_t)(2 * b) * M + m] + (int)absum[(size_t)(2 * b + 1) * M + m]);
+  uint32_t w0, w1;
+  split3(u, w0, w1);
+  au[(size_t)b * M + m] = make_uint2(w0, w1 | w1 << 16);
+}
+extern "C" __global__ __launch_bounds__(256) void q4k_wscales_bf16(const uint8_t* __restrict__ raw, size_t hdr_off, int N, int nsb,
+                                                                   float* __restrict__ wsv) {
+  const int n = blockIdx.x * 256 + threadIdx.x, sb = blockIdx.y;
+  if (n >= N) return;
+  const uint4 h = *(const uint4*)(raw + hdr_off + ((size_t)n * nsb + sb) * 16);
+  const float d = f16_bits_to_f32(h.x), dmin = f16_bits_to_f32(h.x >> 16);
+  float* ws = wsv + (size_t)sb * 8 * N + n;
+  uint4* v = (uint4*)(wsv + (size_t)nsb * 8 * N) + (size_t)sb * 8 * N + n;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int sc[2], mn[2];
+    q4k_scales_pair(h.y, h.z, h.w, j, sc[0], sc[1], mn[0], mn[1]);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      ws[(size_t)(2 * j + q) * N] = d * (float)sc[q];
+      uint32_t w0, w1;
+      split3(-(dmin * (float)mn[q]), w0, w1);
+      const uint32_t v1 = w0 & 0xFFFFu, v2 = w0 >> 16, v3 = w1;
+      v[(size_t)(2 * j + q) * N] = make_uint4(v1 | v1 << 16, v2 | v2 << 16, v3 | v3 << 16, w0);
+    }
+  }
+}
+
 // swiglu_quant: y = silu(gate) * up (or the tanh form of gelu(gate) * up) from rows [gate(F) | up(F)], or the row as it
 // is when the matmul before has fused the product (`fused`), quantized with K = F (reference zero/kernels/ops.cl:
 // 271-315, same arguments; silu(x) = x / (1 + exp(-x)), ops.cl:33).  grid (256 * G, rows), local (256, 1).
