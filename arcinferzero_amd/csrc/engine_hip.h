@@ -668,13 +668,16 @@ class Engine {
     // Q4_K / Q5_K in 128 x 128 tiles: the token side's scale vectors ready-made (-DAU; ARCZ_Q4_AU=0: formed in the kernel)
     static const int q4_au = getenv("ARCZ_Q4_AU") ? atoi(getenv("ARCZ_Q4_AU")) : 3;
     const bool au = q4_au && (w.type == GGML_Q4_K || w.type == GGML_Q5_K) && !q4_wide && !q4_small && M % 4 == 0;
-    // ... and the row side's too (-DAU=2) when the chunk is long enough to pay for writing them (8 bytes per 32
-    // weights: 22 MB, about 8 us, for 17408 x 5120): ARCZ_Q4_AU=1 never, ARCZ_Q4_AU2_MIN=n from n token rows on
-    static const int au2_min = getenv("ARCZ_Q4_AU2_MIN") ? atoi(getenv("ARCZ_Q4_AU2_MIN")) : 1024;
+    // ... and the row side's too (-DAU=2), written in front of the launch (8 bytes per 32 weights: 22 MB, about 8 us,
+    // for 17408 x 5120; pays from the shortest chunks this path takes: ARCZ_Q4_AU=1 never, ARCZ_Q4_AU2_MIN=n from n
+    // token rows on)
+    static const int au2_min = getenv("ARCZ_Q4_AU2_MIN") ? atoi(getenv("ARCZ_Q4_AU2_MIN")) : 256;
     const bool au2 = au && q4_au >= 2 && Mp >= au2_min && N % 4 == 0 && (size_t)N * (K / 32) * 20 + 4096 <= wsv_bytes_;
-    // ... and, Q4_K from 2048 token rows on, the min term's operands as bf16 pieces (-DAU=3: 20 bytes per block and
-    // row to write, 56 MB for 17408 x 5120; ARCZ_Q4_AU=2 never, ARCZ_Q4_AU3_MIN=n from n token rows on)
-    static const int au3_min = getenv("ARCZ_Q4_AU3_MIN") ? atoi(getenv("ARCZ_Q4_AU3_MIN")) : 2048;
+    // ... and, Q4_K, the min term's operands as bf16 pieces (-DAU=3: 20 bytes per block and row to write, 56 MB,
+    // about 15 us, for 17408 x 5120; us per launch at that shape against the -DAU=2 form, both with their pre-passes:
+    // 512 tokens 199 / 210, 1024 313 / 331, 2048 545 / 577, 8192 2062 / 2121; ARCZ_Q4_AU=2 never, ARCZ_Q4_AU3_MIN=n
+    // from n token rows on)
+    static const int au3_min = getenv("ARCZ_Q4_AU3_MIN") ? atoi(getenv("ARCZ_Q4_AU3_MIN")) : 256;
     const bool au3 = au2 && q4_au >= 3 && w.type == GGML_Q4_K && Mp >= au3_min;
     cl_kernel k = q8_small  ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
                   : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")

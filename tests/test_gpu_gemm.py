@@ -183,11 +183,10 @@ def test_per_256_activation_scales(eng, qtype, T, Mp, N, K):
 @pytest.mark.parametrize("qtype", [az.Q4_K, az.Q5_K])
 @pytest.mark.parametrize("T,Mp,N,K,acc", [(1100, 1104, 392, 512, 0), (1100, 1104, 390, 512, 0), (1030, 1040, 640, 768, 1),
                                           (760, 768, 520, 1024, 2), (1200, 1216, 132, 256, 0),
-                                          # from 2048 token rows on, Q4_K: the min term on the bf16 matrix instruction
                                           (2100, 2112, 392, 512, 0), (2050, 2064, 136, 256, 1), (2048, 2048, 256, 768, 2)])
 def test_gemm_ready_made_scale_vectors(rt, qtype, T, Mp, N, K, acc):
     """The 128 x 128 Q4_K / Q5_K kernel whose scale vectors are written by small kernels in front of it (token side: sa and
-    sa * S; row side, from 1024 token rows on when N is a multiple of 4: d * sc and -(dmin * mn); from 2048 on the min
+    sa * S; row side, from 256 token rows on when N is a multiple of 4: d * sc and -(dmin * mn), for Q4_K with the min
     term's factors as bf16 pieces for the matrix instruction) and go into LDS by DMA:
     chunks whose last token tile and last row tile are partly empty, so that the whole-row reads run into the next
     block's entries and past the arrays' ends; the three epilogues.  Against the oracle, and run to run."""
