@@ -21,8 +21,8 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
 # HBM bytes one launch of the headline GEMM moves, from two counter runs of this script (FETCH_SIZE x 2.0 KiB read,
-# WRITE_SIZE x 1.0 KiB written, the factors calibrated on the 2 GiB copy in the same runs): 2173.6 MB + 570.4 MB
-GEMM_HBM_BYTES_PER_LAUNCH = 2.743e9
+# WRITE_SIZE x 1.0 KiB written, the factors calibrated on the 2 GiB copy in the same runs): 2745.3 MB + 570.4 MB
+GEMM_HBM_BYTES_PER_LAUNCH = 3.316e9
 
 
 def log(*a):
@@ -431,7 +431,7 @@ def main():
                      "frac": pre["kernel_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH,
                      "traffic_source": "profiles/bench_hbm_traffic_fetch_write.txt (counter runs of this script; "
                                        "a constant here, not read in this run)",
-                     "kernel": "gemm__QTYPE12_ACT321",
+                     "kernel": "gemm__QTYPE12_ACT321_AU3",
                      "kernel_ms": pre["gemm_kernel_ms"], "kernel_ms_median": pre["gemm_kernel_ms_median"],
                      "kernel_ms_min": pre["gemm_kernel_ms_min"], "ops_per_launch": pre["ops"]},
         "parity_rel_err_sampled": pre["parity_rel_err"],
