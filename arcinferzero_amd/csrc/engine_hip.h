@@ -615,7 +615,9 @@ class Engine {
       const bool q45 = w.type == GGML_Q4_K || w.type == GGML_Q5_K;
       const int tm = w.type == GGML_Q8_0 || w.type == GGML_Q6_K ? 64 : q45 ? (Mp <= 64 ? 64 : 128) : 128;
       const int bm = tm == 64 && q45 && Mp <= 32 ? 32 : tm;  // (Q4_K / Q5_K, at most 32 rows: the one-slot-tile kernel)
-      const size_t tiles64 = (size_t)((Mp + tm - 1) / tm) * ((N + 127) / 128), slots = 2 * (size_t)arcz_device_cus();
+      // (the one-slot-tile kernel is light enough for three work-groups a compute unit: 17408 x 5120, 32 tokens, 3 pieces
+      //  of K 30.0 us, 5 pieces 28.3)
+      const size_t tiles64 = (size_t)((Mp + tm - 1) / tm) * ((N + 127) / 128), slots = (bm == 32 ? 3 : 2) * (size_t)arcz_device_cus();
       const int nsb = K / 256;
       const int sk_force = sk_force_;
       int ny = (int)std::min<size_t>({(size_t)8, (size_t)nsb / 2, slots / std::max<size_t>(tiles64, 1)});
