@@ -453,26 +453,24 @@ class Engine {
       throw std::runtime_error(std::string("matmul ") + name + ": the output does not fit C");
     int a = acc;
     cl_mem tabs = tabs_;  // (the reference's codebook tables; IQ3_S's kernels read theirs from it)
-    // Q4_K and a few tokens: the matrix-vector form on the matrix pipe (gemv_mm), K in slices of at most 24 superblocks
-    // that accumulate.  It takes 9-16 tokens in chunks of 16 rows (what the reference pads them to, zero/engine.h:522;
-    // the rows from T on come out as zeros, as the GEMM writes them: 27 against 95 us at 17408 x 5120), and 3-8 tokens
-    // where it is the faster one: 7 and 8 always (26 against 30 us), 3-6 when the tokens do not fit the LDS of the
-    // dot-product kernels (5120 x 17408, 4 tokens: 50 against 88 us).  Not with two-pass inputs (their second half
+    // Q4_K and a few tokens: the matrix-vector form on the matrix pipe (gemv_mm; it takes K in slices of at most 24
+    // superblocks of the tokens in LDS).  It takes 9-16 tokens in chunks of 16 rows (what the reference pads them to, zero/engine.h:522;
+    // the rows from T on come out as zeros, as the GEMM writes them: 22 against 95 us at 17408 x 5120), and 3-8 tokens
+    // where it is the faster one: from 5 on always (us at the settled clock, against the dot-product kernels: 17408 x
+    // 5120 21.9 / 27.6, 5120 x 5120 12.1 / 13.7, 1024 x 5120 9.8 / 9.2; with 3 and 4 tokens 21.3 / 19.0, 11.6 / 8.5,
+    // 9.2 / 6.9: not taken; ARCZ_GEMV_MM_MIN: the first count it takes), 3 and 4 when the tokens do not fit the LDS of
+    // the dot-product kernels (5120 x 17408, 4 tokens: 41 against 88 us).  Not with two-pass inputs (their second half
     // goes through the kernels below).  ARCZ_GEMV_MM=0: off.
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
     const bool mm_ok = !mm_off && !q2mm_ && w.type == GGML_Q4_K && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
       rd_bytes += raw_bytes(w);
-      const int nsb = K / 256, slices = (nsb + 23) / 24;
       cl_kernel k = kernel("decode", "-DQT=12", "gemv_mm");
       const size_t groups = (size_t)(N + 15) / 16;
       size_t g1 = std::min<size_t>(groups, (size_t)arcz_device_cus()) * 512, l1 = 512;
-      for (int sl = 0; sl < slices; ++sl) {
-        int s0 = nsb * sl / slices, s1 = nsb * (sl + 1) / slices, ac = sl == 0 ? a : 1;
-        set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, ac, s0, s1);
-        run(name, k, 1, &g1, &l1);
-      }
+      set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a, 0, K / 256);
+      run(name, k, 1, &g1, &l1);
     };
     if (mm_ok && cur_T_ >= 9 && cur_T_ <= 16 && Mp == 16) {
       gemv_mm();
@@ -507,7 +505,8 @@ class Engine {
       // (IQ3_S: 2 KiB of the work-group's LDS hold the codebook)
       const size_t lds_max = w.type == GGML_IQ3_S ? 65536 - 2048 : 65536;
       const bool fits = !force_v && lpr && lds <= lds_max;
-      if (mm_ok && T >= 3 && (T >= 7 || !fits)) {
+      static const int mm_min = getenv("ARCZ_GEMV_MM_MIN") ? atoi(getenv("ARCZ_GEMV_MM_MIN")) : 5;
+      if (mm_ok && T >= 3 && (T >= mm_min || !fits)) {
         rd_bytes -= raw_bytes(w);  // (counted by gemv_mm)
         gemv_mm();
         return;

@@ -1,5 +1,5 @@
 """gemv_mm: the Q4_K matrix-vector form for a few tokens on the matrix pipe.  The engine takes it for 9-16 tokens in a
-16-row chunk, for 7-8 tokens, and for 3-6 tokens whose activations do not fit the LDS of the dot-product kernels; every
+16-row chunk, for 5-8 tokens, and for 3-4 tokens whose activations do not fit the LDS of the dot-product kernels; every
 case here lands on it.  Against the double-accumulated dequantized reference (1e-3 as max|err| / max|ref| per token
 row), with unit scales against the exact integer sums, with K in one slice and in several (later slices accumulate),
 storing and accumulating, rows that do not fill a group of 16."""
@@ -21,7 +21,9 @@ def eng(rt):
 
 
 CASES = [(7, 100, 256), (8, 1000, 5120), (9, 333, 2048), (13, 4097, 1024), (16, 64, 6144), (16, 250, 6400),
-         (3, 77, 17408), (6, 300, 17408), (12, 129, 17408)]
+         (3, 77, 17408), (6, 300, 17408), (12, 129, 17408), (5, 200, 5120), (4, 5120, 17408),
+         # rounds of one, two and four waves a group, then the rest spread wider
+         (7, 33000, 256), (16, 20000, 1024), (8, 17408, 512), (11, 17408, 5120)]
 
 
 @pytest.mark.parametrize("T,N,K", CASES)
