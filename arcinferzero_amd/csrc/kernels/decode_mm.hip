@@ -47,7 +47,7 @@ struct MmQ { mm_u4 a, b; };  // the lane's 16 bytes of a superblock of rows 0-7 
 __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, int N, int K,
                                 const signed char* __restrict__ aq, const float* __restrict__ asc,
                                 const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off, int accumulate,
-                                int s_begin, int s_end) {
+                                int s_begin, int s_end, float* GA, bool first, bool last) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n16 = lane & 15, g = lane >> 4;
   const int nsb = K >> 8, sbs = s_end - s_begin, Ks = sbs * 256, nb = sbs * 8;
   uint8_t* A = lds;                            // [16][Ks] int8; 16-byte piece k of token t sits at piece k ^ t of its row
@@ -194,8 +194,19 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
 
   // lane (n16, g) holds tokens 4 g .. 4 g + 3 of row n16 of a group
   const int tmax = T > 8 ? 16 : T;  // (9-16 tokens: the chunk has 16 rows, those from T on come out as zeros)
-  auto store = [&](const v4f& v, int gl) {
+  // GA: the work-group's groups' sums over the slices so far, in LDS ([group][16 tokens][16 rows]; a load from C at
+  // every group's end would wait for all the weights in flight behind it): C is written by the last slice alone
+  auto store = [&](v4f v, int gl) {
     const int n = (gb0 + gl) * 16 + n16;
+    if (GA) {
+      float* ga = GA + gl * 256 + 64 * g + n16;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (!first) v[i] += ga[16 * i];
+        if (!last) ga[16 * i] = v[i];
+      }
+      if (!last) return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int t = 4 * g + i;
@@ -268,19 +279,25 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   }
 }
 
-// Superblocks [s_begin, s_end) of K, in slices of at most 24 that the work-group takes one after the other: a later
-// slice adds to what the work-group itself has stored (other waves of it, as the stretches fall: the meetings between
-// the slices order those stores and loads within the work-group).
+// Superblocks [s_begin, s_end) of K, in slices of at most 24 that the work-group takes one after the other.  With more
+// than one slice the sums of a work-group's groups wait in LDS for the last slice (up to MM_GA groups a work-group);
+// with more groups than that a later slice adds to what the work-group itself has stored in C (other waves of it, as
+// the stretches fall: the meetings between the slices order those stores and loads within the work-group).
+#define MM_GA 12
+
 extern "C" __global__ __launch_bounds__(512, 1) void gemv_mm__QT12(
     const uint8_t* __restrict__ raw, int N, int K, const uint32_t* tabs, const signed char* __restrict__ aq,
     const float* __restrict__ asc, const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off,
     int accumulate, int s_begin, int s_end) {
-  // tokens 24 x (4096 + 1024) bytes at most, then 3 KiB per wave
-  __shared__ __attribute__((aligned(16))) uint8_t lds[MM_WAVES * MM_SPW * 5120 + MM_WAVES * 3072];
+  // tokens 24 x (4096 + 1024) bytes at most, 3 KiB per wave, 1 KiB per group of sums
+  __shared__ __attribute__((aligned(16))) uint8_t lds[MM_WAVES * MM_SPW * 5120 + MM_WAVES * 3072 + MM_GA * 1024];
   const int all = s_end - s_begin, slices = (all + MM_WAVES * MM_SPW - 1) / (MM_WAVES * MM_SPW);
+  const int groups = (N + 15) >> 4, gd = (int)gridDim.x;
+  const int ng = (int)((long)(blockIdx.x + 1) * groups / gd) - (int)((long)blockIdx.x * groups / gd);
+  float* GA = slices > 1 && ng <= MM_GA ? (float*)(lds + MM_WAVES * MM_SPW * 5120 + MM_WAVES * 3072) : nullptr;
   for (int sl = 0; sl < slices; ++sl) {
     if (sl) __syncthreads();  // (the tokens and partial sums of the slice before have been read)
-    mm_slice(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate || sl, s_begin + all * sl / slices,
-             s_begin + all * (sl + 1) / slices);
+    mm_slice(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, GA ? accumulate : (accumulate || sl),
+             s_begin + all * sl / slices, s_begin + all * (sl + 1) / slices, GA, sl == 0, sl == slices - 1);
   }
 }

@@ -23,7 +23,9 @@ def eng(rt):
 CASES = [(7, 100, 256), (8, 1000, 5120), (9, 333, 2048), (13, 4097, 1024), (16, 64, 6144), (16, 250, 6400),
          (3, 77, 17408), (6, 300, 17408), (12, 129, 17408), (5, 200, 5120), (4, 5120, 17408),
          # rounds of one, two and four waves a group, then the rest spread wider
-         (7, 33000, 256), (16, 20000, 1024), (8, 17408, 512), (11, 17408, 5120)]
+         (7, 33000, 256), (16, 20000, 1024), (8, 17408, 512), (11, 17408, 5120),
+         # several slices of K: the sums wait in LDS, or (13 groups to a work-group) are added to C slice by slice
+         (8, 53000, 6400)]
 
 
 @pytest.mark.parametrize("T,N,K", CASES)
