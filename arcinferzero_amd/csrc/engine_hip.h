@@ -462,11 +462,12 @@ class Engine {
     // the dot-product kernels (5120 x 17408, 4 tokens: 41 against 88 us).  Not with two-pass inputs (their second half
     // goes through the kernels below).  ARCZ_GEMV_MM=0: off.
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
-    const bool mm_ok = !mm_off && !q2mm_ && w.type == GGML_Q4_K && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
+    const bool mm_type = w.type == GGML_Q4_K || w.type == GGML_Q5_K || w.type == GGML_Q6_K || w.type == GGML_Q8_0;
+    const bool mm_ok = !mm_off && !q2mm_ && mm_type && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
       rd_bytes += raw_bytes(w);
-      cl_kernel k = kernel("decode", "-DQT=12", "gemv_mm");
+      cl_kernel k = kernel("decode", "-DQT=" + std::to_string(w.type), "gemv_mm");
       const size_t groups = (size_t)(N + 15) / 16;
       size_t g1 = std::min<size_t>(groups, (size_t)arcz_device_cus()) * 512, l1 = 512;
       set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a, 0, K / 256);

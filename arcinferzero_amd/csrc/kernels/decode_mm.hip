@@ -1,29 +1,36 @@
-// "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K).
+// "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0).
 //
 // From a handful of tokens on, the dot-product GEMVs are bound by their vector ALU work (eight v_dot4 per token and
 // 16-byte unit), not by memory, and past eight tokens the engine had only the prefill GEMM with its 64-token tiles.
 // Here the int32 block sums come from v_mfma_i32_16x16x32_i8: a wave multiplies the 32 values of one block of 16
 // weight rows with up to 16 tokens in one instruction, and the vector ALU is left with the f32 scale step of the
-// prefill GEMM (reference zero/kernels/gemm.cl:454-469, 483):
+// prefill GEMM (reference zero/kernels/gemm.cl:439-488), for Q4_K and Q5_K
 //   res += (sa[t][b] * (d[n] * sc[n][b])) * (float)I[t][n][b]  -  (sa[t][b] * (float)S[t][b]) * (dmin[n] * mn[n][b])
-// with S the sum of the block's 32 int8 activations.  The weights are read once, as in the GEMVs.
+// with S the sum of the block's 32 int8 activations, for Q6_K (two int8 sub-scales per block, :457-464, 485)
+//   res += d[n] * sa[t][b] * (float)(sc0[n][b] * I0[t][n][b] + sc1[n][b] * I1[t][n][b])
+// and for Q8_0 (:445-447)  res += (sa[t][b] * d[n][b]) * (float)I[t][n][b].  The weights are read once, as in the GEMVs.
 //
 // Tokens.  A work-group of 8 waves stages superblocks [s_begin, s_end) of the tokens in LDS -- int8 rows, and per block
-// the 16 tokens' sa and sa * S -- and keeps them for all its weight rows.  K in slices (s_begin, s_end) that fit LDS;
-// later slices accumulate into C.
+// the 16 tokens' sa and (where the type has a min term) sa * S -- and keeps them for all its weight rows.  K in slices
+// that fit LDS, one after the other inside the launch.
 //
 // Products.  Lane (n, g) = (lane % 16, lane / 16) is weight row n of a group of 16 rows as the instruction's column
-// and supplies the 8 values 8 g .. 8 g + 7 of a block: bytes 8 g .. 8 g + 7 of a 32-byte chunk of Q4_K nibbles hold
-// exactly those of the chunk's two blocks (low and high nibbles).  The instruction leaves the lane the sums of tokens
-// 4 g .. 4 g + 3 with its row, whose scales it has decoded itself.  The min term of four blocks is one f32 matrix
-// instruction (16 x 16 x 4) straight into the sums.
+// and supplies the 8 values 8 g .. 8 g + 7 of a block.  Q4_K / Q5_K: bytes 8 g .. 8 g + 7 of a 32-byte chunk of
+// nibbles hold exactly those of the chunk's two blocks (low and high nibbles); Q5_K's fifth bits come from the word of
+// the 16-byte unit those bytes lie in.  Q6_K: a block is the low or the high nibbles of 32 consecutive bytes of ql
+// with two bits of 32 bytes of qh, and its two halves of 16 values have different scales: two instructions a block,
+// the weights of the other half's lanes (g < 2, g >= 2) zeroed; the values enter as 4 (q - 32) (bit 5 flipped, the six
+// bits at the top of the byte), the 4 goes into d.  Q8_0: the int8 values as they lie.  The instruction leaves the
+// lane the sums of tokens 4 g .. 4 g + 3 with its row, whose scales it has decoded itself.  The min term of four
+// blocks is one f32 matrix instruction (16 x 16 x 4) straight into the sums.
 //
-// Weights.  Were a lane to load the 8 bytes of a chunk that the matrix instruction wants from it, an instruction would
-// touch 16 rows' lines for 32 bytes each: that form ran at 2 TB/s with or without its arithmetic.  Instead a lane
-// loads 16 bytes such that eight lanes cover one row's superblock (a wave's instruction: 8 rows x 128 bytes), eight
-// superblocks ahead in registers, and the wave turns a superblock's 2 KiB round through a piece of LDS of its own into
-// the matrix instruction's layout (LDS operations of one wave complete in order: no barrier).  Headers come four
-// superblocks at a time (lane (n, j): row n, superblock j of the four) through LDS in the same way.
+// Weights.  Were a lane to load the 8 bytes that the matrix instruction wants from it, an instruction would touch 16
+// rows' lines for 32 bytes each: that form ran at 2 TB/s with or without its arithmetic.  Instead a lane loads 16
+// bytes such that eight lanes (Q8_0: sixteen) cover one row's superblock in the type's main plane, several
+// superblocks ahead in registers, and the wave turns a superblock's rows through a piece of LDS of its own into the
+// matrix instruction's layout (LDS operations of one wave complete in order: no barrier).  Headers (Q6_K: the 16
+// scales, Q8_0: the 8 block scales) come four superblocks at a time (lane (n, j): row n, superblock j of the four)
+// through LDS in the same way, and so do the smaller planes (Q5_K's qh, Q6_K's qh and d), in whole lines.
 //
 // Work.  A work-group takes a contiguous run of 16-row groups (groups / gridDim.x of them, or one more); the run's
 // (group, superblock) units, group-major, are cut into eight equal stretches, one per wave, so every wave streams the
@@ -33,32 +40,73 @@
 #include "common.h"
 
 #define MM_WAVES 8
-#define MM_SPW 3  // slices of up to MM_WAVES * MM_SPW = 24 superblocks
+#define MM_LDS_MAX (160 * 1024 - 1024)
 
 typedef uint32_t mm_u2 __attribute__((ext_vector_type(2)));
 typedef uint32_t mm_u4 __attribute__((ext_vector_type(4)));
-struct MmSb { mm_u2 c[4]; mm_u4 h; };  // a lane's 8 bytes of each of a superblock's four chunks, the superblock's header
 
-#define MM2_D 8  // superblocks in flight per wave
+// Per type: SB, the superblocks of a slice at most; QB, the bytes of a row's superblock in the main plane; D, the
+// superblocks a wave has in flight; XB, the bytes per row and superblock of the second plane that goes through LDS in
+// batches of four; MIN, whether the type has a min term; DPL, whether d is a plane of its own (2 bytes).
+template <int QT> struct MmT;
+template <> struct MmT<QT_Q4_K> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 1, DPL = 0 }; };
+template <> struct MmT<QT_Q5_K> { enum { SB = 22, QB = 128, D = 4, XB = 32, MIN = 1, DPL = 0 }; };
+template <> struct MmT<QT_Q6_K> { enum { SB = 20, QB = 128, D = 4, XB = 64, MIN = 0, DPL = 1 }; };
+template <> struct MmT<QT_Q8_0> { enum { SB = 24, QB = 256, D = 4, XB = 0, MIN = 0, DPL = 0 }; };
+// LDS: per superblock of a slice 4096 bytes of tokens and 512 of sa (512 more of sa * S); per wave the main plane's rows
+// of one superblock, 1 KiB of headers, the second plane's four superblocks, 256 bytes of d; then 1 KiB per group whose
+// sums wait for the last slice (as many as fit, 12 at most)
+template <int QT> struct MmL {
+  static constexpr int TOK = 4096 + 512 + (MmT<QT>::MIN ? 512 : 0);
+  static constexpr int WQ = MmT<QT>::QB * 16, WH = 1024, WX = MmT<QT>::XB * 64, WD = MmT<QT>::DPL ? 256 : 0;
+  static constexpr int WSZ = WQ + WH + WX + WD;
+  static constexpr int FREE = (MM_LDS_MAX - MmT<QT>::SB * TOK - MM_WAVES * WSZ) / 1024;
+  static constexpr int GA = FREE < 12 ? FREE : 12;
+  static constexpr int LDS = MmT<QT>::SB * TOK + MM_WAVES * WSZ + GA * 1024;
+  static_assert(GA >= 1, "no room for the groups' sums");
+};
 
-struct MmQ { mm_u4 a, b; };  // the lane's 16 bytes of a superblock of rows 0-7 and of rows 8-15 of the group
+template <int QT> struct MmQ { mm_u4 r[MmT<QT>::QB / 64]; };  // the lane's 16-byte pieces of a superblock of 16 rows
+template <int QT> struct MmX { mm_u4 r[MmT<QT>::XB / 16 > 0 ? MmT<QT>::XB / 16 : 1]; uint32_t d; };  // of four superblocks' second plane
+// a superblock as the products take it: the lane's 8 bytes of each 32-byte chunk of the main plane, the header
+template <int QT> struct MmSb { mm_u2 c[MmT<QT>::QB / 32]; mm_u4 h; mm_u2 x[2]; uint32_t d; };
 
-// one slice of K, superblocks [s_begin, s_end): at most MM_WAVES * MM_SPW of them
+// one slice of K, superblocks [s_begin, s_end): at most MmT<QT>::SB of them
+template <int QT>
 __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, int N, int K,
                                 const signed char* __restrict__ aq, const float* __restrict__ asc,
                                 const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off, int accumulate,
                                 int s_begin, int s_end, float* GA, bool first, bool last) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n16 = lane & 15, g = lane >> 4;
+  using TT = MmT<QT>;
+  using LL = MmL<QT>;
+  constexpr int QB = TT::QB, NQ = QB / 64, D = TT::D, LPRW = QB / 16, RPI = 64 / LPRW;
+  constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
+  const int tid = threadIdx.x, lane = tid & 63, n16 = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (a scalar: what follows from it is scalar arithmetic)
   const int nsb = K >> 8, sbs = s_end - s_begin, Ks = sbs * 256, nb = sbs * 8;
   uint8_t* A = lds;                            // [16][Ks] int8; 16-byte piece k of token t sits at piece k ^ t of its row
   float* SA = (float*)(lds + 16 * Ks);         // [nb][16] sa
-  float* U = SA + nb * 16;                     // [nb][16] sa * S
-  uint8_t* WB = (uint8_t*)(U + nb * 16);       // per wave: 2 KiB of nibbles, 1 KiB of headers
-  uint8_t* WQ = WB + wave * 3072;
-  uint8_t* WH = WQ + 2048;
-  const PlanesQ4K pl = planes_q4k((size_t)N, nsb);
-  const uint8_t* qs = raw + pl.qs;
-  const uint8_t* hd = raw + pl.hdr;
+  float* U = SA + nb * 16;                     // [nb][16] sa * S (types with a min term)
+  uint8_t* WB = (uint8_t*)(SA + (TT::MIN ? 2 : 1) * nb * 16);  // per wave: WQ, WH, WX, WD
+  uint8_t* WQ = WB + wave * LL::WSZ;
+  uint8_t* WH = WQ + LL::WQ;
+  uint8_t* WX = WH + LL::WH;
+  uint8_t* WD = WX + LL::WX;
+  // the planes (all have the main plane first, a row's superblocks together)
+  size_t o_hdr, o_x = 0, o_d = 0;
+  if constexpr (Q45) {
+    const PlanesQ4K pl = planes_q4k((size_t)N, nsb);
+    o_hdr = pl.hdr; o_x = pl.qh;
+  } else if constexpr (QT == QT_Q6_K) {
+    const PlanesQ6K pl = planes_q6k((size_t)N, nsb);
+    o_hdr = pl.sc; o_x = pl.qh; o_d = pl.d;
+  } else {
+    o_hdr = planes_q80((size_t)N, nsb).d;
+  }
+  const uint8_t* qs = raw;
+  const uint8_t* hd = raw + o_hdr;
+  const uint8_t* xp = raw + o_x;
+  const uint8_t* dp = raw + o_d;
   const int groups = (N + 15) >> 4, gd = (int)gridDim.x;
   const int gb0 = (int)((long)blockIdx.x * groups / gd), gb1 = (int)((long)(blockIdx.x + 1) * groups / gd);
   const int units = (gb1 - gb0) * sbs;         // >= 1: the grid has at most `groups` work-groups
@@ -68,12 +116,18 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   const uint32_t magic = 0xFFFFFFFFu / (uint32_t)sbs + 1u;
   auto group_of = [&](int u) { return sbs == 1 ? u : (int)__umulhi((uint32_t)u, magic); };
 
-  auto qload = [&](MmQ& q, int u) {  // u: the same in the whole wave, within the run
+  // (the unit's base is a scalar; a lane adds its row of the group -- rows past the matrix: the last -- times the row
+  //  stride, below 2^24, and its piece)
+  const uint32_t row_stride = (uint32_t)nsb * QB, piece_off = (uint32_t)(lane % LPRW) * 16;
+  auto qload = [&](MmQ<QT>& q, int u) {  // u: the same in the whole wave, within the run
     const int gl = group_of(u), sb = u - gl * sbs;
-    const int r0 = (gb0 + gl) * 16 + (lane >> 3);
-    const size_t o = (size_t)(s_begin + sb) * 128 + (lane & 7) * 16;
-    q.a = *(const mm_u4*)(qs + (size_t)min(r0, N - 1) * nsb * 128 + o);
-    q.b = *(const mm_u4*)(qs + (size_t)min(r0 + 8, N - 1) * nsb * 128 + o);
+    const int g0 = (gb0 + gl) * 16;
+    const uint8_t* base = qs + ((size_t)g0 * nsb + (s_begin + sb)) * QB;
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      const uint32_t rel = (uint32_t)min(i * RPI + lane / LPRW, N - 1 - g0);
+      q.r[i] = *(const mm_u4*)(base + (__umul24(rel, row_stride) + piece_off));
+    }
   };
   auto hload = [&](mm_u4& h, int ub) {  // the headers of units ub .. ub + 3 (past the stretch: its last)
     const int u = min(ub + g, ulast);
@@ -81,12 +135,33 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     const int r = min((gb0 + gl) * 16 + n16, N - 1);
     h = *(const mm_u4*)(hd + ((size_t)r * nsb + s_begin + sb) * 16);
   };
+  // the second plane of units ub .. ub + 3: a row's XB bytes of a unit are XB / 16 lanes' pieces, whole lines where the
+  // four units are superblocks of one group; Q6_K's d with the header's lanes
+  auto xload = [&](MmX<QT>& x, int ub) {
+    if constexpr (TT::XB > 0) {
+      constexpr int PU = TT::XB / 16, RX = 64 / (4 * PU);  // pieces per unit and row; rows per instruction
+#pragma unroll
+      for (int i = 0; i < PU; ++i) {
+        const int row = i * RX + lane / (4 * PU), j = (lane % (4 * PU)) / PU, p = lane % PU;
+        const int u = min(ub + j, ulast);
+        const int gl = group_of(u), sb = u - gl * sbs;
+        const int r = min((gb0 + gl) * 16 + row, N - 1);
+        x.r[i] = *(const mm_u4*)(xp + ((size_t)r * nsb + s_begin + sb) * TT::XB + p * 16);
+      }
+    }
+    if constexpr (TT::DPL) {
+      const int u = min(ub + g, ulast);
+      const int gl = group_of(u), sb = u - gl * sbs;
+      const int r = min((gb0 + gl) * 16 + n16, N - 1);
+      x.d = *(const unsigned short*)(dp + ((size_t)r * nsb + s_begin + sb) * 2);
+    }
+  };
 
   // ---- staging.  Loads first: the tokens' int8 rows (wave w: rows 2 w and 2 w + 1, 16-byte pieces lane, lane + 64, ..),
   // their scales and sums (asc [K / 32][M], absum [K / 16][M]), then the wave's first superblocks right behind them:
   // loads come back in order, so the stores below wait for the tokens alone while the weights are on their way.
-  constexpr int NCH = MM_WAVES * MM_SPW * 16 / 64;   // pieces per lane and row at most
-  constexpr int NSC = MM_WAVES * MM_SPW * 8 * 16 / 512;  // (block, token) pairs per thread at most
+  constexpr int NCH = (TT::SB * 16 + 63) / 64;  // pieces per lane and row at most
+  constexpr int NSC = (TT::SB * 8 * 16 + 511) / 512;  // (block, token) pairs per thread at most
   const int cpr = Ks >> 4;
   mm_u4 va[2][NCH];
   float vs[NSC];
@@ -104,21 +179,17 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   for (int i = 0; i < NSC; ++i) {
     const int idx = min(tid + 512 * i, nb * 16 - 1), b = s_begin * 8 + (idx >> 4), t = idx & 15, tt = t < T ? t : 0;
     vs[i] = asc[(size_t)b * M + tt];
-    vu[i] = (int)absum[(size_t)(2 * b) * M + tt] + (int)absum[(size_t)(2 * b + 1) * M + tt];
+    if constexpr (TT::MIN) vu[i] = (int)absum[(size_t)(2 * b) * M + tt] + (int)absum[(size_t)(2 * b + 1) * M + tt];
   }
   __builtin_amdgcn_sched_barrier(0);
-  MmQ q0, q1, q2, q3, q4, q5, q6, q7;
+  MmQ<QT> q[D];
+  MmX<QT> xq;
   mm_u4 hq0, hq1;
   hload(hq0, u0);
   hload(hq1, u0 + 4);
-  qload(q0, min(u0 + 0, ulast));
-  qload(q1, min(u0 + 1, ulast));
-  qload(q2, min(u0 + 2, ulast));
-  qload(q3, min(u0 + 3, ulast));
-  qload(q4, min(u0 + 4, ulast));
-  qload(q5, min(u0 + 5, ulast));
-  qload(q6, min(u0 + 6, ulast));
-  qload(q7, min(u0 + 7, ulast));
+  xload(xq, u0);
+#pragma unroll
+  for (int k = 0; k < D; ++k) qload(q[k], min(u0 + k, ulast));
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int r2 = 0; r2 < 2; ++r2) {
@@ -136,60 +207,138 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     const int idx = min(tid + 512 * i, nb * 16 - 1), t = idx & 15;
     const float sa = t < T ? vs[i] : 0.0f;
     SA[idx] = sa;
-    U[idx] = sa * (float)vu[i];
+    if constexpr (TT::MIN) U[idx] = sa * (float)vu[i];
   }
   __syncthreads();
 
-  // the lane's places in the wave's LDS: piece p of row r of a superblock at 16-byte slot 16 p + (r ^ 2 p), so that the
-  // writes (a quarter wave: two rows' eight pieces) and the reads (half a wave: one piece of 16 rows, 8 bytes a lane)
-  // each go to all banks once
-  const int wp = lane & 7, wr = lane >> 3;
-  const int wa = (16 * wp + (wr ^ (2 * wp))) << 4, wb = wa ^ 128;
-  int rd[4];
+  // the lane's places in the wave's LDS.  Main plane: piece p of row r of a superblock at 16-byte slot 16 p + (r ^ 2 p)
+  // (Q8_0, 16 pieces a row: 16 p + (r ^ p)), so that the writes (a quarter wave: two rows' eight pieces, or one row's
+  // sixteen) and the reads (half a wave: one piece of 16 rows, 8 bytes a lane) each go to all banks once
+  int wq[NQ];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int i = 0; i < NQ; ++i) {
+    const int p = lane % LPRW, r = i * RPI + lane / LPRW;
+    wq[i] = (16 * p + (r ^ (LPRW == 8 ? 2 * p : p))) << 4;
+  }
+  constexpr int NC = QB / 32;  // 32-byte chunks of a row's superblock
+  int rd[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
     const int p = 2 * c + (g >> 1);
-    rd[c] = ((16 * p + (n16 ^ (2 * p))) << 4) + (g & 1) * 8;
+    rd[c] = ((16 * p + (n16 ^ (LPRW == 8 ? 2 * p : p))) << 4) + (g & 1) * 8;
   }
   const uint8_t* arow = A + n16 * Ks + (g & 1) * 8;
 
   // the products of one superblock (sbk: its index within the slice) of the lane's row, into acc
-  auto products = [&](const MmSb& h, int sbk, v4f& acc) {
-    const float d = f16_bits_to_f32(h.h.x), dmin = f16_bits_to_f32(h.h.x >> 16);
+  auto products = [&](const MmSb<QT>& h, int sbk, v4f& acc) {
     const int b0 = sbk * 8;
     long av[8];
     float4 sa4[8];
+    // the tokens' values and scales of the superblock's blocks (Q6_K: of four blocks at a time, for the registers)
+    auto tokens = [&](int from, int to) {
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      av[b] = *(const long*)(arow + ((sbk * 16 + ((2 * b + (g >> 1)) ^ n16)) << 4));
-      sa4[b] = *(const float4*)(SA + (b0 + b) * 16 + 4 * g);
+      for (int b = from; b < to; ++b) {
+        av[b] = *(const long*)(arow + ((sbk * 16 + ((2 * b + (g >> 1)) ^ n16)) << 4));
+        sa4[b] = *(const float4*)(SA + (b0 + b) * 16 + 4 * g);
+      }
+    };
+    if constexpr (QT != QT_Q6_K) tokens(0, 8);
+    if constexpr (Q45) {
+      const float d = f16_bits_to_f32(h.h.x), dmin = f16_bits_to_f32(h.h.x >> 16);
+      const float ua = U[(b0 + g) * 16 + n16], ub = U[(b0 + 4 + g) * 16 + n16];
+      int sc[8], mn[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) q4k_scales_pair(h.h.y, h.h.z, h.h.w, j, sc[2 * j], sc[2 * j + 1], mn[2 * j], mn[2 * j + 1]);
+      v4i I[8];
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const mm_u2 cw = h.c[b >> 1];
+        uint32_t w0 = ((b & 1) ? cw.x >> 4 : cw.x) & 0x0F0F0F0Fu, w1 = ((b & 1) ? cw.y >> 4 : cw.y) & 0x0F0F0F0Fu;
+        if constexpr (QT == QT_Q5_K) {
+          // the fifth bits: word H of the 16-byte unit the lane's 8 bytes lie in (unit 2 c + g / 2 of the superblock),
+          // whose bits 4 + k and k belong to the low and the high nibbles of the unit's word k; the lane's are words
+          // 2 (g & 1) and 2 (g & 1) + 1
+          const uint32_t H = (b >> 1) < 2 ? ((b >> 1) == 0 ? h.x[0].x : h.x[0].y) : ((b >> 1) == 2 ? h.x[1].x : h.x[1].y);
+          const int k0 = 2 * (g & 1);
+          if (b & 1) {
+            w0 |= (H << (4 - k0)) & 0x10101010u;
+            w1 |= (H << (3 - k0)) & 0x10101010u;
+          } else {
+            w0 |= (H >> k0) & 0x10101010u;
+            w1 |= (H >> (k0 + 1)) & 0x10101010u;
+          }
+        }
+        const long wv = (long)(((unsigned long)w1 << 32) | w0);
+        v4i z = {0, 0, 0, 0};
+        I[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wv, z, 0, 0, 0);
+      }
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const float ws = d * (float)sc[b];
+        acc[0] = fmaf((float)I[b][0], sa4[b].x * ws, acc[0]);
+        acc[1] = fmaf((float)I[b][1], sa4[b].y * ws, acc[1]);
+        acc[2] = fmaf((float)I[b][2], sa4[b].z * ws, acc[2]);
+        acc[3] = fmaf((float)I[b][3], sa4[b].w * ws, acc[3]);
+      }
+      // the min term of each half's four blocks, - sum_b (sa S)[t][b] (dmin mn)[n][b], as one f32 matrix instruction
+      const int m0 = g == 0 ? mn[0] : g == 1 ? mn[1] : g == 2 ? mn[2] : mn[3];
+      const int m1 = g == 0 ? mn[4] : g == 1 ? mn[5] : g == 2 ? mn[6] : mn[7];
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ua, -(dmin * (float)m0), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ub, -(dmin * (float)m1), acc, 0, 0, 0);
+    } else if constexpr (QT == QT_Q6_K) {
+      // block b = 4 n2 + hb of the superblock: the low (hb < 2) or high nibbles of ql bytes 64 n2 + 32 (hb & 1) + 0..31
+      // (chunk 2 n2 + (hb & 1)) with bits 2 hb, 2 hb + 1 of qh bytes 32 n2 + 0..31; scales 2 b and 2 b + 1 for its
+      // halves, which are the lanes g < 2 and g >= 2
+      const uint32_t keep_a = g < 2 ? 0xFCFCFCFCu : 0u, keep_b = g < 2 ? 0u : 0xFCFCFCFCu;
+      const float d = 0.25f * f16_bits_to_f32(h.d);
+      v4f part = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        if ((b & 3) == 0) {
+          __builtin_amdgcn_sched_barrier(0);
+          tokens(b, b + 4);
+        }
+        const int n2 = b >> 2, hb = b & 3;
+        const mm_u2 L = h.c[2 * n2 + (hb & 1)], H = h.x[n2];
+        uint32_t w[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          const uint32_t l = k ? L.y : L.x, hh = k ? H.y : H.x;
+          const uint32_t nib = hb < 2 ? l << 2 : l >> 2;                         // the nibble at bits 2..5
+          const uint32_t top = hb == 3 ? hh : hh << (6 - 2 * hb);                // the two high bits at 6..7
+          w[k] = (((nib & 0x3C3C3C3Cu) | (top & 0xC0C0C0C0u)) ^ 0x80808080u);   // 4 (q - 32) as int8
+        }
+        const long wa = (long)(((unsigned long)(w[1] & keep_a) << 32) | (w[0] & keep_a));
+        const long wb = (long)(((unsigned long)(w[1] & keep_b) << 32) | (w[0] & keep_b));
+        v4i z = {0, 0, 0, 0};
+        const v4i Ia = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wa, z, 0, 0, 0);
+        const v4i Ib = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wb, z, 0, 0, 0);
+        const uint32_t sw = b < 2 ? h.h.x : b < 4 ? h.h.y : b < 6 ? h.h.z : h.h.w;
+        // (the sums are below 2^23 in size -- 16 x 127 x 128 -- and the scales int8: 24-bit multiplies)
+        const int sca = (int)(signed char)(sw >> (16 * (b & 1))), scb = (int)(signed char)(sw >> (16 * (b & 1) + 8));
+        part[0] = fmaf((float)(__mul24(sca, Ia[0]) + __mul24(scb, Ib[0])), sa4[b].x, part[0]);
+        part[1] = fmaf((float)(__mul24(sca, Ia[1]) + __mul24(scb, Ib[1])), sa4[b].y, part[1]);
+        part[2] = fmaf((float)(__mul24(sca, Ia[2]) + __mul24(scb, Ib[2])), sa4[b].z, part[2]);
+        part[3] = fmaf((float)(__mul24(sca, Ia[3]) + __mul24(scb, Ib[3])), sa4[b].w, part[3]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(d, part[i], acc[i]);
+    } else {
+      // Q8_0: block b is bytes 32 b .. 32 b + 31 of the row's 256, its f16 scale entry b of the 16-byte header
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const mm_u2 cw = h.c[b];
+        const long wv = (long)(((unsigned long)cw.y << 32) | cw.x);
+        v4i z = {0, 0, 0, 0};
+        const v4i I = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wv, z, 0, 0, 0);
+        const uint32_t dw = b < 2 ? h.h.x : b < 4 ? h.h.y : b < 6 ? h.h.z : h.h.w;
+        const float d = f16_bits_to_f32((b & 1) ? dw >> 16 : dw);
+        acc[0] = fmaf((float)I[0], sa4[b].x * d, acc[0]);
+        acc[1] = fmaf((float)I[1], sa4[b].y * d, acc[1]);
+        acc[2] = fmaf((float)I[2], sa4[b].z * d, acc[2]);
+        acc[3] = fmaf((float)I[3], sa4[b].w * d, acc[3]);
+      }
     }
-    const float ua = U[(b0 + g) * 16 + n16], ub = U[(b0 + 4 + g) * 16 + n16];
-    int sc[8], mn[8];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) q4k_scales_pair(h.h.y, h.h.z, h.h.w, j, sc[2 * j], sc[2 * j + 1], mn[2 * j], mn[2 * j + 1]);
-    v4i I[8];
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      const mm_u2 cw = h.c[b >> 1];
-      const uint32_t w0 = ((b & 1) ? cw.x >> 4 : cw.x) & 0x0F0F0F0Fu, w1 = ((b & 1) ? cw.y >> 4 : cw.y) & 0x0F0F0F0Fu;
-      const long wv = (long)(((unsigned long)w1 << 32) | w0);
-      v4i z = {0, 0, 0, 0};
-      I[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wv, z, 0, 0, 0);
-    }
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-      const float ws = d * (float)sc[b];
-      acc[0] = fmaf((float)I[b][0], sa4[b].x * ws, acc[0]);
-      acc[1] = fmaf((float)I[b][1], sa4[b].y * ws, acc[1]);
-      acc[2] = fmaf((float)I[b][2], sa4[b].z * ws, acc[2]);
-      acc[3] = fmaf((float)I[b][3], sa4[b].w * ws, acc[3]);
-    }
-    // the min term of each half's four blocks, - sum_b (sa S)[t][b] (dmin mn)[n][b], as one f32 matrix instruction
-    const int m0 = g == 0 ? mn[0] : g == 1 ? mn[1] : g == 2 ? mn[2] : mn[3];
-    const int m1 = g == 0 ? mn[4] : g == 1 ? mn[5] : g == 2 ? mn[6] : mn[7];
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ua, -(dmin * (float)m0), acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ub, -(dmin * (float)m1), acc, 0, 0, 0);
   };
 
   // lane (n16, g) holds tokens 4 g .. 4 g + 3 of row n16 of a group
@@ -219,17 +368,34 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
 
   const int gf = group_of(min(u0, ulast));  // the stretch's first group
   v4f acc = {0.0f, 0.0f, 0.0f, 0.0f}, ph = acc, pt = acc;  // running sums; the cut group at the head, at the tail
-  auto sbstep = [&](MmQ& q, int u, int j) {
+  // unit u: its rows out of qq through the wave's LDS, qq refilled with the unit D on (past the stretch the last unit
+  // again: the same loads on every path), the products
+  auto sbstep = [&](MmQ<QT>& qq, int u, int j) {
     if (u < u1) {
-      *(mm_u4*)(WQ + wa) = q.a;
-      *(mm_u4*)(WQ + wb) = q.b;
-    }
-    qload(q, min(u + MM2_D, ulast));
-    if (u < u1) {
-      MmSb s;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) s.c[c] = *(const mm_u2*)(WQ + rd[c]);
+      for (int i = 0; i < NQ; ++i) *(mm_u4*)(WQ + wq[i]) = qq.r[i];
+    }
+    qload(qq, min(u + D, ulast));
+    if (u < u1) {
+      MmSb<QT> s;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) s.c[c] = *(const mm_u2*)(WQ + rd[c]);
       s.h = *(const mm_u4*)(WH + ((j * 16 + n16) << 4));
+      if constexpr (QT == QT_Q5_K) {
+        // words g / 2, 2 + g / 2, 4 + g / 2, 6 + g / 2 of the row's 8 words of fifth bits
+        const uint8_t* xr = WX + (j * 16 + n16) * 32 + 4 * (g >> 1);
+        s.x[0].x = *(const uint32_t*)(xr);
+        s.x[0].y = *(const uint32_t*)(xr + 8);
+        s.x[1].x = *(const uint32_t*)(xr + 16);
+        s.x[1].y = *(const uint32_t*)(xr + 24);
+      }
+      if constexpr (QT == QT_Q6_K) {
+        // bytes 32 n2 + 8 g .. + 7 of the row's 64 bytes of qh (16-byte pieces XOR-ed with r / 4 against conflicts)
+        const uint8_t* xr = WX + (j * 16 + n16) * 64 + (g & 1) * 8;
+        s.x[0] = *(const mm_u2*)(xr + ((((g >> 1)) ^ (n16 >> 2)) << 4));
+        s.x[1] = *(const mm_u2*)(xr + (((2 + (g >> 1)) ^ (n16 >> 2)) << 4));
+        s.d = *(const uint32_t*)(WD + ((j * 16 + n16) << 2));
+      }
       const int gl = group_of(u), sb = u - gl * sbs;
       products(s, sb, acc);
       if (sb == sbs - 1 || u == u1 - 1) {  // the group ends here, or the stretch does
@@ -240,20 +406,30 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
       }
     }
   };
+  // a batch of four units' headers (and second plane) into the wave's LDS, the next ones asked for
+  auto batch = [&](mm_u4& hq, int ub_next_h, int ub_next_x) {
+    *(mm_u4*)(WH + ((g * 16 + n16) << 4)) = hq;
+    hload(hq, ub_next_h);
+    if constexpr (TT::XB > 0) {
+      constexpr int PU = TT::XB / 16, RX = 64 / (4 * PU);
+#pragma unroll
+      for (int i = 0; i < PU; ++i) {
+        const int row = i * RX + lane / (4 * PU), j = (lane % (4 * PU)) / PU, p = lane % PU;
+        const int pp = QT == QT_Q6_K ? p ^ (row >> 2) : p;
+        *(mm_u4*)(WX + (j * 16 + row) * TT::XB + pp * 16) = xq.r[i];
+      }
+    }
+    if constexpr (TT::DPL) *(uint32_t*)(WD + ((g * 16 + n16) << 2)) = xq.d;
+    if constexpr (TT::XB > 0 || TT::DPL) xload(xq, ub_next_x);
+  };
 #pragma unroll 1
   for (int u = u0; u < u1; u += 8) {
-    *(mm_u4*)(WH + ((g * 16 + n16) << 4)) = hq0;
-    hload(hq0, u + 8);
-    sbstep(q0, u + 0, 0);
-    sbstep(q1, u + 1, 1);
-    sbstep(q2, u + 2, 2);
-    sbstep(q3, u + 3, 3);
-    *(mm_u4*)(WH + ((g * 16 + n16) << 4)) = hq1;
-    hload(hq1, u + 12);
-    sbstep(q4, u + 4, 0);
-    sbstep(q5, u + 5, 1);
-    sbstep(q6, u + 6, 2);
-    sbstep(q7, u + 7, 3);
+    batch(hq0, u + 8, u + 4);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) sbstep(q[k % D], u + k, k);
+    batch(hq1, u + 12, u + 8);
+#pragma unroll
+    for (int k = 4; k < 8; ++k) sbstep(q[k % D], u + k, k - 4);
   }
 
   // the cut groups: the partial sums into the wave's own LDS (two slots of [16 tokens][16 rows]), one meeting, then the
@@ -270,7 +446,7 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     for (int w = 0; w <= wave; ++w) {
       const int a0 = w * units / MM_WAVES, a1 = (w + 1) * units / MM_WAVES;
       if (a1 > a0 && a1 > gf * sbs && a0 < (gf + 1) * sbs) {
-        const float* pw = (const float*)(WB + w * 3072) + (group_of(a0) == gf ? 0 : 256);
+        const float* pw = (const float*)(WB + w * LL::WSZ) + (group_of(a0) == gf ? 0 : 256);
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] += pw[(4 * g + i) * 16 + n16];
       }
@@ -279,25 +455,36 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   }
 }
 
-// Superblocks [s_begin, s_end) of K, in slices of at most 24 that the work-group takes one after the other.  With more
-// than one slice the sums of a work-group's groups wait in LDS for the last slice (up to MM_GA groups a work-group);
+// Superblocks [s_begin, s_end) of K, in slices that the work-group takes one after the other.  With more than one slice
+// the sums of a work-group's groups wait in LDS for the last slice (as many groups as the type's LDS leaves room for);
 // with more groups than that a later slice adds to what the work-group itself has stored in C (other waves of it, as
 // the stretches fall: the meetings between the slices order those stores and loads within the work-group).
-#define MM_GA 12
-
-extern "C" __global__ __launch_bounds__(512, 1) void gemv_mm__QT12(
-    const uint8_t* __restrict__ raw, int N, int K, const uint32_t* tabs, const signed char* __restrict__ aq,
-    const float* __restrict__ asc, const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off,
-    int accumulate, int s_begin, int s_end) {
-  // tokens 24 x (4096 + 1024) bytes at most, 3 KiB per wave, 1 KiB per group of sums
-  __shared__ __attribute__((aligned(16))) uint8_t lds[MM_WAVES * MM_SPW * 5120 + MM_WAVES * 3072 + MM_GA * 1024];
-  const int all = s_end - s_begin, slices = (all + MM_WAVES * MM_SPW - 1) / (MM_WAVES * MM_SPW);
+template <int QT>
+__device__ inline void mm_kernel(uint8_t* lds, const uint8_t* __restrict__ raw, int N, int K,
+                                 const signed char* __restrict__ aq, const float* __restrict__ asc,
+                                 const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off, int accumulate,
+                                 int s_begin, int s_end) {
+  constexpr int SB = MmT<QT>::SB;
+  const int all = s_end - s_begin, slices = (all + SB - 1) / SB;
   const int groups = (N + 15) >> 4, gd = (int)gridDim.x;
   const int ng = (int)((long)(blockIdx.x + 1) * groups / gd) - (int)((long)blockIdx.x * groups / gd);
-  float* GA = slices > 1 && ng <= MM_GA ? (float*)(lds + MM_WAVES * MM_SPW * 5120 + MM_WAVES * 3072) : nullptr;
+  float* GA = slices > 1 && ng <= MmL<QT>::GA ? (float*)(lds + SB * MmL<QT>::TOK + MM_WAVES * MmL<QT>::WSZ) : nullptr;
   for (int sl = 0; sl < slices; ++sl) {
     if (sl) __syncthreads();  // (the tokens and partial sums of the slice before have been read)
-    mm_slice(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, GA ? accumulate : (accumulate || sl),
-             s_begin + all * sl / slices, s_begin + all * (sl + 1) / slices, GA, sl == 0, sl == slices - 1);
+    mm_slice<QT>(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, GA ? accumulate : (accumulate || sl),
+                 s_begin + all * sl / slices, s_begin + all * (sl + 1) / slices, GA, sl == 0, sl == slices - 1);
   }
 }
+
+#define MM_KERNEL(QTV)                                                                                                  \
+  extern "C" __global__ __launch_bounds__(512, 1) void gemv_mm__QT##QTV(                                                \
+      const uint8_t* __restrict__ raw, int N, int K, const uint32_t* tabs, const signed char* __restrict__ aq,          \
+      const float* __restrict__ asc, const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off,       \
+      int accumulate, int s_begin, int s_end) {                                                                         \
+    __shared__ __attribute__((aligned(16))) uint8_t lds[MmL<QTV>::LDS];                                                 \
+    mm_kernel<QTV>(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, s_begin, s_end);                    \
+  }
+MM_KERNEL(12)
+MM_KERNEL(13)
+MM_KERNEL(14)
+MM_KERNEL(8)

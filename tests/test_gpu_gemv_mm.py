@@ -1,4 +1,4 @@
-"""gemv_mm: the Q4_K matrix-vector form for a few tokens on the matrix pipe.  The engine takes it for 9-16 tokens in a
+"""gemv_mm: the matrix-vector form for a few tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0).  The engine takes it for 9-16 tokens in a
 16-row chunk, for 5-8 tokens, and for 3-4 tokens whose activations do not fit the LDS of the dot-product kernels; every
 case here lands on it.  Against the double-accumulated dequantized reference (1e-3 as max|err| / max|ref| per token
 row), with unit scales against the exact integer sums, with K in one slice and in several (later slices accumulate),
@@ -28,12 +28,11 @@ CASES = [(7, 100, 256), (8, 1000, 5120), (9, 333, 2048), (13, 4097, 1024), (16, 
          (8, 53000, 6400)]
 
 
-@pytest.mark.parametrize("T,N,K", CASES)
-def test_gemv_mm_parity(eng, T, N, K):
-    print(f"gemv_mm T={T} N={N} K={K}", flush=True)
-    W = make_weights(az.Q4_K, N, K, seed=800 + T)
+def _parity(eng, qt, T, N, K):
+    print(f"gemv_mm type={qt} T={T} N={N} K={K}", flush=True)
+    W = make_weights(qt, N, K, seed=800 + T)
     x = make_acts(T, K, seed=801 + T, outliers=True)
-    w = eng.make_weight(az.Q4_K, N, K, W)
+    w = eng.make_weight(qt, N, K, W)
     xb = az.Runtime.from_numpy(x)
     eng.quantize(xb, K, K, 16, T)
     rows = T if T <= 8 else 16
@@ -41,7 +40,7 @@ def test_gemv_mm_parity(eng, T, N, K):
     eng.matmul("mm", w, 16, cb, N, 0, 0)
     y = cb.read(np.float32, rows * N).reshape(rows, N)
     aq, asc, _ = quantize_padded(x, 16)
-    ref = orc.matmul_ref(az.Q4_K, W, N, K, aq[:T], asc)
+    ref = orc.matmul_ref(qt, W, N, K, aq[:T], asc)
     assert np.isfinite(y).all()
     assert rel_err_rows(y[:T], ref).max() <= 1e-3
     if rows > T:
@@ -57,12 +56,30 @@ def test_gemv_mm_parity(eng, T, N, K):
     w.free()
 
 
+@pytest.mark.parametrize("T,N,K", CASES)
+def test_gemv_mm_parity(eng, T, N, K):
+    _parity(eng, az.Q4_K, T, N, K)
+
+
+# the other types of the matrix-pipe form: a slice of K, several slices (22 / 20 / 24 superblocks at most for Q5_K / Q6_K /
+# Q8_0), rows that do not fill a group, work-groups with several groups, more groups than wait in LDS
+CASES_TYPES = [(8, 100, 256), (16, 333, 2048), (13, 1000, 5120), (7, 129, 17408), (16, 5120, 6400), (9, 17408, 1024),
+               (8, 53000, 6400)]
+
+
+@pytest.mark.parametrize("T,N,K", CASES_TYPES)
+@pytest.mark.parametrize("qt", [az.Q5_K, az.Q6_K, az.Q8_0])
+def test_gemv_mm_parity_types(eng, qt, T, N, K):
+    _parity(eng, qt, T, N, K)
+
+
 @pytest.mark.parametrize("T,N,K", [(8, 48, 512), (16, 37, 7168)])
-def test_gemv_mm_unit_scales_exact(eng, T, N, K):
+@pytest.mark.parametrize("qt", [az.Q4_K, az.Q5_K, az.Q6_K])
+def test_gemv_mm_unit_scales_exact(eng, qt, T, N, K):
     """All scales 1: the f32 output is the exact integer sum (partial sums stay below 2^24)."""
-    W, wi = unit_scale_weights(az.Q4_K, N, K, seed=820)
+    W, wi = unit_scale_weights(qt, N, K, seed=820)
     x = unit_scale_acts(T, K, seed=821)
-    w = eng.make_weight(az.Q4_K, N, K, W)
+    w = eng.make_weight(qt, N, K, W)
     xb = az.Runtime.from_numpy(x)
     eng.quantize(xb, K, K, 16, T)
     rows = T if T <= 8 else 16
