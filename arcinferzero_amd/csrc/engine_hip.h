@@ -462,7 +462,8 @@ class Engine {
     // the dot-product kernels (5120 x 17408, 4 tokens: 41 against 88 us).  Not with two-pass inputs (their second half
     // goes through the kernels below).  ARCZ_GEMV_MM=0: off.
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
-    const bool mm_type = w.type == GGML_Q4_K || w.type == GGML_Q5_K || w.type == GGML_Q6_K || w.type == GGML_Q8_0;
+    const bool mm_type = w.type == GGML_Q4_K || w.type == GGML_Q5_K || w.type == GGML_Q6_K || w.type == GGML_Q8_0 ||
+                         w.type == GGML_Q4_0 || w.type == GGML_IQ4_XS;
     const bool mm_ok = !mm_off && !q2mm_ && mm_type && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;

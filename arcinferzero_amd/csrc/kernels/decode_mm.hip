@@ -1,4 +1,5 @@
-// "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0).
+// "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0,
+// Q4_0, IQ4_XS).
 //
 // From a handful of tokens on, the dot-product GEMVs are bound by their vector ALU work (eight v_dot4 per token and
 // 16-byte unit), not by memory, and past eight tokens the engine had only the prefill GEMM with its 64-token tiles.
@@ -8,7 +9,8 @@
 //   res += (sa[t][b] * (d[n] * sc[n][b])) * (float)I[t][n][b]  -  (sa[t][b] * (float)S[t][b]) * (dmin[n] * mn[n][b])
 // with S the sum of the block's 32 int8 activations, for Q6_K (two int8 sub-scales per block, :457-464, 485)
 //   res += d[n] * sa[t][b] * (float)(sc0[n][b] * I0[t][n][b] + sc1[n][b] * I1[t][n][b])
-// and for Q8_0 (:445-447)  res += (sa[t][b] * d[n][b]) * (float)I[t][n][b].  The weights are read once, as in the GEMVs.
+// and for Q8_0 (:445-447), Q4_0 and IQ4_XS (one scale per block)  res += (sa[t][b] * d[n][b]) * (float)I[t][n][b].  The
+// weights are read once, as in the GEMVs.
 //
 // Tokens.  A work-group of 8 waves stages superblocks [s_begin, s_end) of the tokens in LDS -- int8 rows, and per block
 // the 16 tokens' sa and (where the type has a min term) sa * S -- and keeps them for all its weight rows.  K in slices
@@ -53,6 +55,8 @@ template <> struct MmT<QT_Q4_K> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN =
 template <> struct MmT<QT_Q5_K> { enum { SB = 22, QB = 128, D = 4, XB = 32, MIN = 1, DPL = 0 }; };
 template <> struct MmT<QT_Q6_K> { enum { SB = 20, QB = 128, D = 4, XB = 64, MIN = 0, DPL = 1 }; };
 template <> struct MmT<QT_Q8_0> { enum { SB = 24, QB = 256, D = 4, XB = 0, MIN = 0, DPL = 0 }; };
+template <> struct MmT<QT_Q4_0> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 0, DPL = 0 }; };
+template <> struct MmT<QT_IQ4_XS> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 0, DPL = 0 }; };
 // LDS: per superblock of a slice 4096 bytes of tokens and 512 of sa (512 more of sa * S); per wave the main plane's rows
 // of one superblock, 1 KiB of headers, the second plane's four superblocks, 256 bytes of d; then 1 KiB per group whose
 // sums wait for the last slice (as many as fit, 12 at most)
@@ -69,7 +73,8 @@ template <int QT> struct MmL {
 template <int QT> struct MmQ { mm_u4 r[MmT<QT>::QB / 64]; };  // the lane's 16-byte pieces of a superblock of 16 rows
 template <int QT> struct MmX { mm_u4 r[MmT<QT>::XB / 16 > 0 ? MmT<QT>::XB / 16 : 1]; uint32_t d; };  // of four superblocks' second plane
 // a superblock as the products take it: the lane's 8 bytes of each 32-byte chunk of the main plane, the header
-template <int QT> struct MmSb { mm_u2 c[MmT<QT>::QB / 32]; mm_u4 h; mm_u2 x[2]; uint32_t d; };
+// (Q4_0 and IQ4_XS: of each 16-byte block)
+template <int QT> struct MmSb { mm_u2 c[QT == QT_Q4_0 || QT == QT_IQ4_XS ? 8 : MmT<QT>::QB / 32]; mm_u4 h; mm_u2 x[2]; uint32_t d; };
 
 // one slice of K, superblocks [s_begin, s_end): at most MmT<QT>::SB of them
 template <int QT>
@@ -81,6 +86,8 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   using LL = MmL<QT>;
   constexpr int QB = TT::QB, NQ = QB / 64, D = TT::D, LPRW = QB / 16, RPI = 64 / LPRW;
   constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
+  constexpr bool B16 = QT == QT_Q4_0 || QT == QT_IQ4_XS;  // a block is 16 bytes: low nibbles values 0..15, high 16..31
+  constexpr int HB = QT == QT_IQ4_XS ? 8 : 16;            // bytes of a row's superblock in the header plane
   const int tid = threadIdx.x, lane = tid & 63, n16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (a scalar: what follows from it is scalar arithmetic)
   const int nsb = K >> 8, sbs = s_end - s_begin, Ks = sbs * 256, nb = sbs * 8;
@@ -100,8 +107,12 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   } else if constexpr (QT == QT_Q6_K) {
     const PlanesQ6K pl = planes_q6k((size_t)N, nsb);
     o_hdr = pl.sc; o_x = pl.qh; o_d = pl.d;
-  } else {
+  } else if constexpr (QT == QT_Q8_0) {
     o_hdr = planes_q80((size_t)N, nsb).d;
+  } else if constexpr (QT == QT_Q4_0) {
+    o_hdr = planes_q40((size_t)N, nsb).d;
+  } else {
+    o_hdr = planes_iq4xs((size_t)N, nsb).hdr;
   }
   const uint8_t* qs = raw;
   const uint8_t* hd = raw + o_hdr;
@@ -133,7 +144,12 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     const int u = min(ub + g, ulast);
     const int gl = group_of(u), sb = u - gl * sbs;
     const int r = min((gb0 + gl) * 16 + n16, N - 1);
-    h = *(const mm_u4*)(hd + ((size_t)r * nsb + s_begin + sb) * 16);
+    if constexpr (HB == 16) {
+      h = *(const mm_u4*)(hd + ((size_t)r * nsb + s_begin + sb) * 16);
+    } else {
+      const mm_u2 h2 = *(const mm_u2*)(hd + ((size_t)r * nsb + s_begin + sb) * 8);
+      h = mm_u4{h2.x, h2.y, 0, 0};
+    }
   };
   // the second plane of units ub .. ub + 3: a row's XB bytes of a unit are XB / 16 lanes' pieces, whole lines where the
   // four units are superblocks of one group; Q6_K's d with the header's lanes
@@ -220,11 +236,13 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     const int p = lane % LPRW, r = i * RPI + lane / LPRW;
     wq[i] = (16 * p + (r ^ (LPRW == 8 ? 2 * p : p))) << 4;
   }
-  constexpr int NC = QB / 32;  // 32-byte chunks of a row's superblock
+  // (the lane's 8 bytes: bytes 8 g .. of each 32-byte chunk; for the 16-byte blocks bytes 8 (g & 1) .. of each block,
+  //  whose low nibbles are the values of lanes g < 2 and whose high nibbles those of g >= 2)
+  constexpr int NC = B16 ? 8 : QB / 32;
   int rd[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
-    const int p = 2 * c + (g >> 1);
+    const int p = B16 ? c : 2 * c + (g >> 1);
     rd[c] = ((16 * p + (n16 ^ (LPRW == 8 ? 2 * p : p))) << 4) + (g & 1) * 8;
   }
   const uint8_t* arow = A + n16 * Ks + (g & 1) * 8;
@@ -323,6 +341,36 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] = fmaf(d, part[i], acc[i]);
+    } else if constexpr (B16) {
+      // block b is the 16 bytes 16 b .. of the row's 128; Q4_0: value nibble - 8, f16 scale entry b of the header;
+      // IQ4_XS: the table's value of the nibble, d in the header's first half word and a 6-bit scale - 32 per block (low
+      // four bits in the second word, high two in the upper half of the first)
+      const int sh = 4 * (g >> 1);
+      const float d4 = f16_bits_to_f32(h.h.x);
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const mm_u2 cw = h.c[b];
+        uint32_t w0, w1;
+        float d;
+        if constexpr (QT == QT_Q4_0) {
+          w0 = q40_vals(cw.x >> sh);
+          w1 = q40_vals(cw.y >> sh);
+          const uint32_t dw = b < 2 ? h.h.x : b < 4 ? h.h.y : b < 6 ? h.h.z : h.h.w;
+          d = f16_bits_to_f32((b & 1) ? dw >> 16 : dw);
+        } else {
+          w0 = iq4_lookup(cw.x >> sh);
+          w1 = iq4_lookup(cw.y >> sh);
+          const int ls = (int)(((h.h.y >> (4 * b)) & 0xFu) | ((((h.h.x >> 16) >> (2 * b)) & 3u) << 4)) - 32;
+          d = d4 * (float)ls;
+        }
+        const long wv = (long)(((unsigned long)w1 << 32) | w0);
+        v4i z = {0, 0, 0, 0};
+        const v4i I = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wv, z, 0, 0, 0);
+        acc[0] = fmaf((float)I[0], sa4[b].x * d, acc[0]);
+        acc[1] = fmaf((float)I[1], sa4[b].y * d, acc[1]);
+        acc[2] = fmaf((float)I[2], sa4[b].z * d, acc[2]);
+        acc[3] = fmaf((float)I[3], sa4[b].w * d, acc[3]);
+      }
     } else {
       // Q8_0: block b is bytes 32 b .. 32 b + 31 of the row's 256, its f16 scale entry b of the 16-byte header
 #pragma unroll
@@ -488,3 +536,5 @@ MM_KERNEL(12)
 MM_KERNEL(13)
 MM_KERNEL(14)
 MM_KERNEL(8)
+MM_KERNEL(2)
+MM_KERNEL(23)
