@@ -135,7 +135,7 @@ def bench_decode(az, qtype, N, K, T, launches, copies):
     x = az.gen_normal(4, (T, K))
     xb = az.Runtime.from_numpy(x)
     eng.quantize(xb, K, K, 16, T)
-    cb = az.Runtime.alloc(T * N * 4)
+    cb = az.Runtime.alloc((T if T <= 8 else 16) * N * 4)   # (9-16 tokens: a chunk of 16 rows)
     def round_of_copies():   # warm-up: every buffer in turn
         for i in range(copies):
             eng.matmul("gemv", ws[i], 16, cb, N, 0, 0)
@@ -444,8 +444,13 @@ def main():
         log(f"[bench] decode T=2: {d2}")
         dgu = bench_gemv_gu(az, az.Q4_K, 17408, 5120, 200, 4)
         log(f"[bench] decode gate + up in one launch: {dgu}")
+        # a batch of 8 tokens (the matrix-pipe GEMV): the headline matrix, and the Q6_K down projection's shape
+        d8 = bench_decode(az, az.Q4_K, 17408, 5120, 8, 200, 8)
+        log(f"[bench] decode T=8: {d8}")
+        d86 = bench_decode(az, az.Q6_K, 5120, 17408, 8, 200, 6)
+        log(f"[bench] decode T=8 Q6_K: {d86}")
         out["decode"] = {"Q4_K_17408x5120_T1": d1, "Q4_K_5120x17408_T2": d2, "Q4_K_gate_up_2x17408x5120_T1": dgu,
-                         "hbm_peak_GBps": PEAK_HBM_GBS}
+                         "Q4_K_17408x5120_T8": d8, "Q6_K_5120x17408_T8": d86, "hbm_peak_GBps": PEAK_HBM_GBS}
     if not args.no_extras:
         az.self_check()
         c1, _ = bench_gemm_config(az, az.Q8_0, 4096, 4096, 512, 50, 31)
