@@ -273,16 +273,26 @@ class Engine {
   // zero/engine.h:1404-1440): a work-group per row of the chunk, or -- a pass of 1-8 tokens -- the valid rows only,
   // their superblocks over several work-groups (the GEMVs read nothing else).
   static bool wide_rows(int T) { return T <= 8; }
+  // the 16-rows-a-work-group forms: one-pass engines, chunks of at least 256 rows in multiples of 16, rows of up to
+  // kmax values (the kernels' R16_KMAX_NORM and R16_KMAX)
+  bool rows16(int K, int Mp, int T, int kmax) const {
+    static const bool off = getenv("ARCZ_PROD_R16") && atoi(getenv("ARCZ_PROD_R16")) == 0;
+    return !off && !q2mm_ && !wide_rows(T) && Mp % 16 == 0 && Mp >= 256 && K <= kmax;
+  }
   void rmsnorm_quant(cl_mem x, int row_off, cl_mem w, int K, int Mp, int T, int act32, float eps, cl_mem hout = nullptr) {
     check_chunk(K, Mp, T);
     if (!act32 && q2mm_) throw std::runtime_error("rmsnorm_quant: two-pass inputs take per-32 activation scales (act32)");
     if (row_off < 0 || arcz_mem_size(x) < (size_t)(row_off + T) * K * 4 || arcz_mem_size(w) < (size_t)K * 4 ||
         (hout && arcz_mem_size(hout) < (size_t)Mp * K * 4))
       throw std::runtime_error("rmsnorm_quant: a buffer is too small for " + std::to_string(T) + " rows of " + std::to_string(K));
-    cl_kernel k = kernel("ops", q2_defs_, "rmsnorm_quant");
+    // (chunks: 16 rows a work-group, their scales and sums written in pieces of 16 rows; ARCZ_PROD_R16=0: a row a
+    //  work-group)
+    const bool r16 = rows16(K, Mp, T, 16384);
+    cl_kernel k = r16 ? kernel("ops", "", "rmsnorm_quant_r16") : kernel("ops", q2_defs_, "rmsnorm_quant");
     int wh = hout ? 1 : 0;
     set_args(k, 0, x, row_off, w, K, Mp, T, eps, aq_, asc_, absum_, hout, wh, act32);
     size_t gws[2] = {256, (size_t)Mp}, lws[2] = {256, 1};
+    if (r16) gws[1] = (size_t)Mp / 16;
     if (wide_rows(T)) {
       gws[0] = 256 * (size_t)((K / 256 + 15) / 16);
       gws[1] = (size_t)T;
@@ -295,9 +305,11 @@ class Engine {
     check_chunk(F, Mp, T);
     if (!act32 && q2mm_) throw std::runtime_error("swiglu_quant: two-pass inputs take per-32 activation scales (act32)");
     if (arcz_mem_size(gu) < (size_t)T * F * (fused ? 1 : 2) * 4) throw std::runtime_error("swiglu_quant: gu is too small");
-    cl_kernel k = kernel("ops", q2_defs_, "swiglu_quant");
+    const bool r16 = rows16(F, Mp, T, 20480);
+    cl_kernel k = r16 ? kernel("ops", "", "swiglu_quant_r16") : kernel("ops", q2_defs_, "swiglu_quant");
     set_args(k, 0, gu, F, Mp, T, aq_, asc_, absum_, act32, fused, gelu);
     size_t gws[2] = {256, (size_t)Mp}, lws[2] = {256, 1};
+    if (r16) gws[1] = (size_t)Mp / 16;
     if (wide_rows(T)) {
       gws[0] = 256 * (size_t)((F / 256 + 15) / 16);
       gws[1] = (size_t)T;

@@ -25,6 +25,8 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "quant_rows", nullptr, "piiiipppi", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "rmsnorm_quant", nullptr, "pipiiifppppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "swiglu_quant", nullptr, "piiipppiii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
+    {"ops", "rmsnorm_quant_r16", nullptr, "pipiiifppppii", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "swiglu_quant_r16", nullptr, "piiipppiii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "add_norm_quant", nullptr, "pppiffpiipppii", {nullptr}, {{"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"Q2_AB", 0, false}, {nullptr, 0, false}}, 256},
     {"ops", "act_usum", nullptr, "ppip", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "q4k_wscales", nullptr, "pziip", {nullptr}, {{nullptr, 0, false}}, 256},

@@ -374,6 +374,14 @@ extern "C" __global__ __launch_bounds__(256) void q4k_wscales_bf16(const uint8_t
   }
 }
 
+// silu(g) = g / (1 + exp(-g)) (reference zero/kernels/ops.cl:33) or the tanh form of gelu.  The exponential and the
+// reciprocal are the hardware's (v_exp_f32 on -g log2 e, v_rcp_f32: an ulp or two each) instead of the library's
+// sequences of about 25 instructions an element, which were a third of the SwiGLU kernel's time.
+__device__ inline float act_gate(float g, int gelu) {
+  if (gelu) return 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)));
+  return g * __frcp_rn(1.0f + __expf(-g));
+}
+
 // swiglu_quant: y = silu(gate) * up (or the tanh form of gelu(gate) * up) from rows [gate(F) | up(F)], or the row as it
 // is when the matmul before has fused the product (`fused`), quantized with K = F (reference zero/kernels/ops.cl:
 // 271-315, same arguments; silu(x) = x / (1 + exp(-x)), ops.cl:33).  grid (256 * G, rows), local (256, 1).
@@ -415,16 +423,173 @@ extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __re
           const float uv[4] = {uv4[h][i].x, uv4[h][i].y, uv4[h][i].z, uv4[h][i].w};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const float g = v[4 * i + j];
-            const float a = gelu ? 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)))
-                                 : g / (1.0f + expf(-g));
-            v[4 * i + j] = a * uv[j];
+            v[4 * i + j] = act_gate(v[4 * i + j], gelu) * uv[j];
           }
         }
       }
       store_row_quant(v, s, lane16, m, M, F, act32, aq, asc, absum, q2_aq, q2_sc, q2_ab);
     }
   }
+}
+
+// ---- the fused producers over chunks of many rows: a work-group takes 16 consecutive rows one after the other and
+// keeps their scales and sums in LDS, [block][16 rows], so that the token-minor arrays are written in pieces of 16
+// rows (64 and 32 bytes) instead of one element per block and row from a work-group per row, whose 480 scattered
+// stores a row were most of that form's memory transactions.  One-pass engines, M a multiple of 16, rows of up to
+// R16_KMAX (R16_KMAX_NORM) values.
+#define R16_KMAX 20480      // swiglu_quant_r16 (80 KiB of LDS: two work-groups a compute unit)
+#define R16_KMAX_NORM 16384 // rmsnorm_quant_r16 (64 KiB, and the row sum's four floats)
+template <int KMAX> struct R16Stage {
+  float sc[KMAX / 32 * 16];
+  short sum[KMAX / 16 * 16];
+};
+// a thread's 16 values of superblock s of row r of the 16: quantized, the int8 values stored, scale and sum staged
+template <int KMAX>
+__device__ inline void r16_quant(R16Stage<KMAX>& st, const float* v, int s, int lane16, int r, int m, int K, int act32,
+                                 signed char* __restrict__ aq) {
+  const float amax = block_amax(v, act32);
+  uint4 pk;
+  int sum;
+  quant16(v, amax, pk, sum, nullptr);
+  *(uint4*)(aq + (size_t)m * K + s * 256 + 16 * lane16) = pk;
+  st.sum[(s * 16 + lane16) * 16 + r] = (short)sum;
+  if (act32) {
+    if ((lane16 & 1) == 0) st.sc[(s * 8 + (lane16 >> 1)) * 16 + r] = amax / 127.0f;
+  } else if (lane16 == 0) {
+    st.sc[s * 16 + r] = amax / 127.0f;
+  }
+}
+// the staged scales and sums of rows m0 .. m0 + 15 out to asc [blocks][M] and absum [K / 16][M]
+template <int KMAX>
+__device__ inline void r16_flush(const R16Stage<KMAX>& st, int m0, int M, int K, int act32, float* __restrict__ asc,
+                                 short* __restrict__ absum) {
+  __syncthreads();
+  const int nb = act32 ? K >> 5 : K >> 8;
+  for (int i = threadIdx.x; i < nb * 16; i += 256) asc[(size_t)(i >> 4) * M + m0 + (i & 15)] = st.sc[i];
+  for (int i = threadIdx.x; i < (K >> 4) * 8; i += 256)
+    *(uint32_t*)(absum + (size_t)(i >> 3) * M + m0 + 2 * (i & 7)) = *(const uint32_t*)(st.sum + (i >> 3) * 16 + 2 * (i & 7));
+}
+
+// rmsnorm_quant over 16 rows a work-group: grid (256, M / 16).  A row stays in registers between its sum of squares
+// and its quantization, and the next row's loads are in flight meanwhile.
+extern "C" __global__ __launch_bounds__(256, 2) void rmsnorm_quant_r16(const float* __restrict__ x, int row_off,
+                                                                       const float* __restrict__ w, int K, int M,
+                                                                       int M_valid, float eps, signed char* __restrict__ aq,
+                                                                       float* __restrict__ asc, short* __restrict__ absum,
+                                                                       float* __restrict__ hout, int write_h, int act32) {
+  __shared__ float red[4];
+  __shared__ R16Stage<R16_KMAX_NORM> st;
+  const int m0 = blockIdx.y * 16;
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4, nsb = K >> 8;
+  constexpr int MAXU = R16_KMAX_NORM / 4096;  // superblocks a thread holds
+  auto load = [&](float4 (&xv)[MAXU][4], int m) {
+    const bool valid = m < M_valid;
+    const float* xr = x + (size_t)((valid ? m : 0) + row_off) * K;
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+      const int sb = sub + 16 * u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        xv[u][i] = valid && sb < nsb ? *(const float4*)(xr + sb * 256 + 16 * lane16 + 4 * i) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  };
+  auto work = [&](const float4 (&xv)[MAXU][4], int r) {
+    const int m = m0 + r;
+    float ss = 0.0f;
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ss += xv[u][i].x * xv[u][i].x;
+        ss += xv[u][i].y * xv[u][i].y;
+        ss += xv[u][i].z * xv[u][i].z;
+        ss += xv[u][i].w * xv[u][i].w;
+      }
+    ss = group_sum(ss, red);
+    const float rs = rsqrtf(ss / (float)K + eps);
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+      const int sb = sub + 16 * u;
+      if (sb >= nsb) break;  // (the same for the 16 threads of a superblock)
+      const int base = sb * 256 + 16 * lane16;
+      float v[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 f = xv[u][i], g = *(const float4*)(w + base + 4 * i);
+        v[4 * i] = f.x * rs * g.x; v[4 * i + 1] = f.y * rs * g.y; v[4 * i + 2] = f.z * rs * g.z; v[4 * i + 3] = f.w * rs * g.w;
+      }
+      if (write_h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          *(float4*)(hout + (size_t)m * K + base + 4 * i) = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+      r16_quant(st, v, sb, lane16, r, m, K, act32, aq);
+    }
+  };
+  float4 xa[MAXU][4], xb[MAXU][4];
+  load(xa, m0);
+#pragma unroll 1
+  for (int r = 0; r < 16; r += 2) {
+    load(xb, m0 + r + 1);
+    work(xa, r);
+    load(xa, min(m0 + r + 2, m0 + 15));  // (after the last pair: row 15 again, not used)
+    work(xb, r + 1);
+  }
+  r16_flush(st, m0, M, K, act32, asc, absum);
+}
+
+// swiglu_quant over 16 rows a work-group: grid (256, M / 16).
+extern "C" __global__ __launch_bounds__(256, 2) void swiglu_quant_r16(const float* __restrict__ gu, int F, int M, int M_valid,
+                                                                      signed char* __restrict__ aq, float* __restrict__ asc,
+                                                                      short* __restrict__ absum, int act32, int fused,
+                                                                      int gelu) {
+  __shared__ R16Stage<R16_KMAX> st;
+  const int m0 = blockIdx.y * 16;
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4, nsb = F >> 8;
+  // (the units of work: superblock s of row r, row-major over the 16 rows, dealt to the 16 groups of threads in turn --
+  //  by rows alone 20 superblocks would keep four groups busy twice and twelve once; the loads of a thread's next unit
+  //  are in flight while it works on the current one)
+  const int units = 16 * nsb, total = (units - sub + 15) / 16;
+  struct Unit { float4 g[4], u[4]; int r, s; };
+  auto load = [&](Unit& t, int j) {
+    const int i = sub + 16 * min(j, total - 1);   // (past the end: the last again, not used)
+    t.r = i / nsb;
+    t.s = i - t.r * nsb;
+    const bool in = m0 + t.r < M_valid;
+    const float* gr = gu + (size_t)(in ? m0 + t.r : 0) * (fused ? F : 2 * F) + t.s * 256 + 16 * lane16;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      t.g[k] = in ? *(const float4*)(gr + 4 * k) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      t.u[k] = in && !fused ? *(const float4*)(gr + F + 4 * k) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  };
+  auto work = [&](const Unit& t) {
+    float v[16];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[4 * k] = t.g[k].x; v[4 * k + 1] = t.g[k].y; v[4 * k + 2] = t.g[k].z; v[4 * k + 3] = t.g[k].w;
+    }
+    if (m0 + t.r < M_valid && !fused) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float uv[4] = {t.u[k].x, t.u[k].y, t.u[k].z, t.u[k].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[4 * k + j] = act_gate(v[4 * k + j], gelu) * uv[j];
+      }
+    }
+    r16_quant(st, v, t.s, lane16, t.r, m0 + t.r, F, act32, aq);
+  };
+  if (total > 0) {
+    Unit a, b;
+    load(a, 0);
+#pragma unroll 1
+    for (int j = 0; j < total; j += 2) {
+      load(b, j + 1);
+      work(a);
+      load(a, j + 2);
+      if (j + 1 < total) work(b);
+    }
+  }
+  r16_flush(st, m0, M, F, act32, asc, absum);
 }
 
 // softcap_rows: C[t][off + n] = cap * tanh(C[t][off + n] / cap) over N columns of the launch's rows (the output head of

@@ -90,6 +90,59 @@ def test_swiglu_quant(eng, T, Mp, F, gelu):
     gb.free(); vb.free()
 
 
+@pytest.mark.parametrize("T,Mp,K,act32", [(256, 256, 16384, 1), (300, 320, 5120, 1), (250, 256, 4096, 0), (1000, 1024, 256, 0)])
+def test_producers_16_rows_a_work_group(rt, T, Mp, K, act32):
+    """Chunks of at least 256 rows go through the forms that take 16 rows a work-group and write scales and sums in
+    pieces of 16 rows: the same bits as the plain quantizer on the f32 rows (RMS norm: on the rows the kernel itself
+    wrote out), per-32 and per-256 scales, rows past T as zeros, the longest rows each form takes."""
+    print(f"producers r16 T={T} Mp={Mp} K={K} act32={act32}", flush=True)
+    eng = az.Engine(Mp, max(K, 256))
+    try:
+        B = 32 if act32 else 256
+        def read(K):
+            return (eng.aq.read(np.int8, Mp * K).reshape(Mp, K), eng.asc.read(np.float32, Mp * K // B).reshape(K // B, Mp),
+                    eng.absum.read(np.int16, Mp * K // 16).reshape(K // 16, Mp))
+        x = make_acts(T, K, seed=330 + T, outliers=True)
+        w = (1.0 + 0.1 * az.gen_normal(331, (K,))).astype(np.float32)
+        xb, wb = az.Runtime.from_numpy(x), az.Runtime.from_numpy(w)
+        hb = az.Runtime.alloc(Mp * K * 4).fill(0xFFFFFFFF)
+        poison(eng)
+        eng.rmsnorm_quant(xb, 0, wb, K, Mp, T, 1e-6, hout=hb, act32=act32)
+        h = hb.read(np.float32, Mp * K).reshape(Mp, K)
+        x64 = x.astype(np.float64)
+        ref = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + 1e-6) * w.astype(np.float64)
+        assert np.abs(h[:T] - ref).max() <= 1e-6 * np.abs(ref).max() and not h[T:].any()
+        aq, asc, absum = read(K)
+        raq, rasc, rabsum = orc.quantize_act(np.ascontiguousarray(h), act32=bool(act32))
+        assert np.array_equal(aq, raq) and np.array_equal(asc.view(np.uint32), rasc.view(np.uint32)) and np.array_equal(absum, rabsum)
+        # SwiGLU on rows taken as they are (the fused form) and on gate | up
+        vb = az.Runtime.from_numpy(np.ascontiguousarray(h[:T]))
+        poison(eng)
+        eng.swiglu_quant(vb, K, Mp, T, fused=1, act32=act32)
+        aq2, asc2, absum2 = read(K)
+        assert np.array_equal(aq2, raq) and np.array_equal(asc2.view(np.uint32), rasc.view(np.uint32)) and np.array_equal(absum2, rabsum)
+        F = K // 2
+        if F % 256 == 0:
+            gb = az.Runtime.from_numpy(x)          # rows [gate(F) | up(F)]
+            poison(eng)
+            eng.swiglu_quant(gb, F, Mp, T, fused=0, act32=act32)
+            g, u = x[:, :F].astype(np.float64), x[:, F:].astype(np.float64)
+            v = pad_rows((g / (1.0 + np.exp(-g)) * u).astype(np.float32), Mp)
+            vaq, vasc, vabsum = orc.quantize_act(v, act32=bool(act32))
+            gaq = eng.aq.read(np.int8, Mp * F).reshape(Mp, F)
+            gasc = eng.asc.read(np.float32, Mp * F // B).reshape(F // B, Mp)
+            gabsum = eng.absum.read(np.int16, Mp * F // 16).reshape(F // 16, Mp)
+            assert np.abs(gasc - vasc).max() <= 1e-6 * np.abs(vasc).max()
+            d = np.abs(gaq.astype(np.int32) - vaq.astype(np.int32))
+            assert d.max() <= 1 and (d != 0).mean() <= 1e-3
+            assert np.array_equal(gabsum.T.reshape(Mp, F // 16), gaq.astype(np.int32).reshape(Mp, F // 16, 16).sum(axis=2))
+            gb.free()
+        for b in (xb, wb, hb, vb):
+            b.free()
+    finally:
+        eng.close()
+
+
 def test_producer_feeds_matmul(eng):
     """rmsnorm_quant -> GEMV and GEMM: the matmul of the normalized rows, against the oracle on the GPU's own int8 rows."""
     from common import make_weights, rel_err_rows
