@@ -112,6 +112,7 @@ class Engine {
   cl_mem wsv_ = nullptr;
   size_t wsv_bytes_ = 0;
   int cur_act32_ = 1;
+  bool a256_ = false;  // inside a matmul on the per-32 expansion of per-256 scales
   // Two-pass matmul inputs (zero/engine.h:1034-1075 q2_init, the mode of the reference's Gemma 4 and Qwen3 models):
   // every producer also quantizes what its int8 values miss, v - q * scale, the same way, into the second half of the
   // three buffers, and every matmul runs a second time over that half, accumulating (matmul below).
@@ -228,7 +229,8 @@ class Engine {
     if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
     w.raw = buf(pb, planes.data());
     if ((type == GGML_Q4_K || type == GGML_Q5_K) && rows == (size_t)N) {  // (room for its rows' scale vectors, gemm_dense)
-      const size_t need = (size_t)N * (K / 32) * 20 + 4096;  // (4 + 4 bytes a block and row, or 4 + 16: the bf16 pieces)
+      // (with per-256 activation scales also d, an f32 per superblock and row: half a byte more per block and row)
+      const size_t need = (size_t)N * (K / 32) * 21 + 4096;  // (4 + 4 bytes a block and row, or 4 + 16: the bf16 pieces)
       if (need > wsv_bytes_) {
         if (wsv_) release(wsv_);
         wsv_ = nullptr;
@@ -373,13 +375,16 @@ class Engine {
       run("asc_expand", k, 1, &g1, &l1);
       const cl_mem s0 = asc_;
       asc_ = asc_rep_;
+      a256_ = true;
       try {
         matmul1(name, w, Mp, C, ldc, c_off, acc, true);
       } catch (...) {
         asc_ = s0;
+        a256_ = false;
         throw;
       }
       asc_ = s0;
+      a256_ = false;
       return;
     }
     // (the output head with a logit soft cap and two-pass inputs: the cap applies to the sum of both passes, so both
@@ -688,17 +693,21 @@ class Engine {
     // for 17408 x 5120; pays from the shortest chunks this path takes: ARCZ_Q4_AU=1 never, ARCZ_Q4_AU2_MIN=n from n
     // token rows on)
     static const int au2_min = getenv("ARCZ_Q4_AU2_MIN") ? atoi(getenv("ARCZ_Q4_AU2_MIN")) : 256;
-    const bool au2 = au && q4_au >= 2 && Mp >= au2_min && N % 4 == 0 && (size_t)N * (K / 32) * 20 + 4096 <= wsv_bytes_;
+    const bool au2 = au && q4_au >= 2 && Mp >= au2_min && N % 4 == 0 && (size_t)N * (K / 32) * 21 + 4096 <= wsv_bytes_;
     // ... and, Q4_K, the min term's operands as bf16 pieces (-DAU=3: 20 bytes per block and row to write, 56 MB,
     // about 15 us, for 17408 x 5120; us per launch at that shape against the -DAU=2 form, both with their pre-passes:
     // 512 tokens 199 / 210, 1024 313 / 331, 2048 545 / 577, 8192 2062 / 2121; ARCZ_Q4_AU=2 never, ARCZ_Q4_AU3_MIN=n
     // from n token rows on)
     static const int au3_min = getenv("ARCZ_Q4_AU3_MIN") ? atoi(getenv("ARCZ_Q4_AU3_MIN")) : 256;
     const bool au3 = au2 && q4_au >= 3 && w.type == GGML_Q4_K && Mp >= au3_min;
+    // ... and, when the chunk's activation scales are per 256 values (act32 = 0: asc_ is their per-32 expansion), the
+    // form that adds a superblock's block sums up as integers (-DAU=4; ARCZ_Q4_A256=0: the per-32 form on the expansion)
+    static const bool a256_off = getenv("ARCZ_Q4_A256") && atoi(getenv("ARCZ_Q4_A256")) == 0;
+    const bool au4 = au3 && a256_ && !a256_off;
     cl_kernel k = q8_small  ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
                   : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")
                   : q4_wide ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64", "gemm")
-                  : au      ? kernel("gemm", "-DQTYPE=" + std::to_string(w.type) + (au3 ? " -DACT32 -DAU=3" : au2 ? " -DACT32 -DAU=2" : " -DACT32 -DAU"), "gemm")
+                  : au      ? kernel("gemm", "-DQTYPE=" + std::to_string(w.type) + (au4 ? " -DACT32 -DAU=4" : au3 ? " -DACT32 -DAU=3" : au2 ? " -DACT32 -DAU=2" : " -DACT32 -DAU"), "gemm")
                             : gemm_kernel(w.type, false);
     // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
     //  registers over the whole of K.  The reference splits rows longer than 8192 into 17-superblock pieces for its
@@ -719,7 +728,7 @@ class Engine {
     }
     cl_mem sums = absum_;
     if (au2) {
-      cl_kernel kw = kernel("ops", "", au3 ? "q4k_wscales_bf16" : "q4k_wscales");
+      cl_kernel kw = kernel("ops", "", au4 ? "q4k_wscales_int" : au3 ? "q4k_wscales_bf16" : "q4k_wscales");
       size_t hdr = planes_q4k((size_t)N, K / 256).hdr;
       int NN = N, nsb2 = K / 256;
       set_args(kw, 0, w.raw, hdr, NN, nsb2, wsv_);

@@ -32,6 +32,7 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "q4k_wscales", nullptr, "pziip", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "act_usum_bf16", nullptr, "ppip", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "q4k_wscales_bf16", nullptr, "pziip", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"ops", "q4k_wscales_int", nullptr, "pziip", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "asc_expand", nullptr, "ppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "softcap_rows", nullptr, "piiif", {nullptr}, {{nullptr, 0, false}}, 0},
     {"ops", "fill32", nullptr, "piz", {nullptr}, {{nullptr, 0, false}}, 256},

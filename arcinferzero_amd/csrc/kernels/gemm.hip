@@ -431,6 +431,9 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   constexpr bool Q5 = QT == QT_Q5_K;
   constexpr bool BF = PRE >= 3;
   static_assert(!(BF && Q5), "the bf16 min-term form is built for Q4_K");
+  // PRE = 4: the activations' scales are per 256 (the chunk's asc holds each eight times): a superblock's block sums
+  // are added up as integers, sc * I per block in a 24-bit multiply-add, and meet the f32 scales once per superblock
+  constexpr bool A256 = PRE == 4;
   // the scale vectors of a stage: f32 per block and token / row (2 KB each), or, BF: sa, ws as before, then the min
   // term's operands, 8 bytes per block and token (4 KB) and 16 per block and row (8 KB): a stage of 40 KB
   constexpr int oSA = G3_SA, oWS = BF ? G3_SA + 2048 : G3_WS, oU = BF ? G3_SA + 4096 : G3_U, oV = BF ? G3_SA + 8192 : G3_V;
@@ -488,6 +491,10 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   const uint8_t* fbase = wave < 2 ? (const uint8_t*)asc + (size_t)s_begin * 8 * M * 4 : (const uint8_t*)wsv + (size_t)s_begin * 8 * N * 4;
   const uint32_t fstep = 16u * (uint32_t)(wave < 2 ? M : N);  // (bytes of four blocks' f32 entries)
   uint32_t foff = wave < 2 ? soff : roff;
+  // A256: wave 1 brings, in the place of sa of blocks 2 and 3, the superblock's d[n] (f32 [K / 256][N] behind the other
+  // two parts of wsv), rows n0 + 4 (l % 32) .. + 3
+  const uint8_t* dbase = (const uint8_t*)wsv + (size_t)(K >> 5) * N * 20 + (size_t)s_begin * N * 4;
+  uint32_t doff = ((uint32_t)n0 + 4u * (lane & 31)) * 4u;
   const uint8_t* ubase = (const uint8_t*)au + ((size_t)s_begin * 8 + wave) * M * 8;
   uint32_t uoff = ((uint32_t)m0 + 2u * lane) * 8u;
   const uint8_t* vbase = (const uint8_t*)wsv + (size_t)(K >> 5) * N * 4 + ((size_t)s_begin * 8 + wave) * N * 16;
@@ -526,8 +533,13 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
       g3_dma16(wbase + (size_t)st * 64 + woff[piece - 4], base + G3_WQ + (wave * 2 + piece - 4) * 1024);
     } else if constexpr (BF) {
       if (piece == 6) {
-        asm volatile("" : "+v"(foff));
-        g3_dma16(fbase + (size_t)st * fstep + foff, base + (wave < 2 ? oSA : oWS) + (wave & 1) * 1024);
+        if (A256 && wave == 1) {
+          asm volatile("" : "+v"(doff));
+          g3_dma16(dbase + (size_t)(st >> 1) * N * 4 + doff, base + oSA + 1024);
+        } else {
+          asm volatile("" : "+v"(foff));
+          g3_dma16(fbase + (size_t)st * fstep + foff, base + (wave < 2 ? oSA : oWS) + (wave & 1) * 1024);
+        }
       } else if (piece == 7) {
         asm volatile("" : "+v"(uoff));
         g3_dma16(ubase + (size_t)st * 4 * M * 8 + uoff, base + oU + wave * 1024);
@@ -655,6 +667,64 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
       for (int i = 0; i < 16; ++i) z[i] = 0;
       I[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[ms], w16[ns], z, 0, 0, 0);
     };
+    if constexpr (A256) {
+      // One row tile (ns) at a time, its two token tiles' integer sums J over the step's four blocks in registers: a
+      // block's weights are decoded once, its sum is sc * I in a 24-bit multiply-add (|I| <= 32 x 127 x 15, sc <= 63), and
+      // the four blocks' total meets the f32 scales once, as (sa[t] d[n]) tiles from the outer-product instruction.
+      // The next step's loads go out one per product.  Then the min term as in the -DAU=3 form.
+      const float dop = ((const float*)(Sb + oSA + 1024))[wn * 64 + lane];
+      int piece = 0;
+#pragma unroll
+      for (int ns = 0; ns < 2; ++ns) {
+        v16i Jt[2];
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) Jt[ms][i] = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          if ((b & 1) == 0) ld_wraw(b >> 1, ns);
+          dec_w(b, ns);
+          const int scn = ((const int*)(Sb + oWS))[b * 128 + wn * 64 + ns * 32 + l32];
+#pragma unroll
+          for (int ms = 0; ms < 2; ++ms) {
+            ld_a(b, ms);
+            mfma_i(ms, ns, ms);
+            if (piece < 10) dma_piece(next ? st + 1 : st, (st + 1) & 1, piece);
+            ++piece;
+          }
+#pragma unroll
+          for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) Jt[ms][i] = __mul24(I[ms][i], scn) + Jt[ms][i];
+        }
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) {
+          const float sa256 = ((const float*)(Sb + oSA))[wm * 64 + ms * 32 + l32];
+          v32f zf;
+#pragma unroll
+          for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+          const v32f Pd = __builtin_amdgcn_mfma_f32_32x32x1f32(sa256, dop, zf, 0, 0, 0);
+#pragma unroll
+          for (int i = 0; i < 16; ++i) res[ms][ns][i] = __builtin_fmaf((float)Jt[ms][i], Pd[16 * ns + i], res[ms][ns][i]);
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < 4; b += 2) {
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) {
+          const uint2 e = ((const uint2*)(Sb + oU))[(b + g) * 128 + wm * 64 + ms * 32 + l32];
+          uopb[ms] = v4u{e.x, e.x, e.x, e.y};
+        }
+#pragma unroll
+        for (int ns = 0; ns < 2; ++ns) vopb[ns] = *(const v4u*)(Sb + oV + ((b + g) * 128 + wn * 64 + ns * 32 + l32) * 16);
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+          for (int ns = 0; ns < 2; ++ns)
+            res[ms][ns] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(uopb[ms]), as_bf16x8(vopb[ns]), res[ms][ns], 0, 0, 0);
+      }
+    } else {
     ld_wraw(0, 0); ld_wraw(0, 1); ld_a(0, 0); ld_a(0, 1); ld_sa(0, 0); ld_sa(0, 1); ld_ws(0);
     dec_w(0, 0); dec_w(0, 1);
     mfma_p(0);
@@ -719,6 +789,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    }  // (!A256)
     if (next) {
       store_scales(sr, st + 1, (st + 1) & 1);
       __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -2072,6 +2143,19 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_AU3(
   tile_of(blockIdx.x, mt, nt, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   gemm3_body<false, QT_Q4_K, 3>(raw, aq, asc, nullptr, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                                min(BM, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au, (const float*)wsv);
+}
+// -DAU=4: the -DAU=3 form for chunks whose activation scales are per 256 values (asc holds each eight times): wsv holds
+// the integer sub-block scales as int32 [K / 32][N], the min term's pieces as before, then d as f32 [K / 256][N]
+// (q4k_wscales_int).
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_AU4(
+    const uint8_t* raw, const uint8_t* au, const signed char* aq, const float* asc, const short* wsv, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  gemm3_body<false, QT_Q4_K, 4>(raw, aq, asc, nullptr, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
                                 min(BM, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au, (const float*)wsv);
 }
 // (tiles of at most 64 slots: the engine builds the tile list for that size)

@@ -432,6 +432,33 @@ extern "C" __global__ __launch_bounds__(256) void swiglu_quant(const float* __re
   }
 }
 
+// q4k_wscales_int: the row side for chunks with per-256 activation scales (the prefill GEMM's -DAU=4 form): the 6-bit
+// sub-block scales as int32 [K / 32][N], the min term's bf16 pieces as q4k_wscales_bf16 writes them, and behind those
+// (20 bytes per block and row in) d as f32 [K / 256][N].  Grid as q4k_wscales.
+extern "C" __global__ __launch_bounds__(256) void q4k_wscales_int(const uint8_t* __restrict__ raw, size_t hdr_off, int N, int nsb,
+                                                                  float* __restrict__ wsv) {
+  const int n = blockIdx.x * 256 + threadIdx.x, sb = blockIdx.y;
+  if (n >= N) return;
+  const uint4 h = *(const uint4*)(raw + hdr_off + ((size_t)n * nsb + sb) * 16);
+  const float d = f16_bits_to_f32(h.x), dmin = f16_bits_to_f32(h.x >> 16);
+  int* ws = (int*)wsv + (size_t)sb * 8 * N + n;
+  uint4* v = (uint4*)(wsv + (size_t)nsb * 8 * N) + (size_t)sb * 8 * N + n;
+  wsv[(size_t)nsb * 8 * N * 5 + (size_t)sb * N + n] = d;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    int sc[2], mn[2];
+    q4k_scales_pair(h.y, h.z, h.w, j, sc[0], sc[1], mn[0], mn[1]);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      ws[(size_t)(2 * j + q) * N] = sc[q];
+      uint32_t w0, w1;
+      split3(-(dmin * (float)mn[q]), w0, w1);
+      const uint32_t v1 = w0 & 0xFFFFu, v2 = w0 >> 16, v3 = w1;
+      v[(size_t)(2 * j + q) * N] = make_uint4(v1 | v1 << 16, v2 | v2 << 16, v3 | v3 << 16, w0);
+    }
+  }
+}
+
 // ---- the fused producers over chunks of many rows: a work-group takes 16 consecutive rows one after the other and
 // keeps their scales and sums in LDS, [block][16 rows], so that the token-minor arrays are written in pieces of 16
 // rows (64 and 32 bytes) instead of one element per block and row from a work-group per row, whose 480 scattered

@@ -180,6 +180,45 @@ def test_per_256_activation_scales(eng, qtype, T, Mp, N, K):
     w.free()
 
 
+@pytest.mark.parametrize("T,Mp,N,K,acc", [(1100, 1104, 392, 512, 0), (1030, 1040, 640, 768, 1), (760, 768, 520, 1024, 2),
+                                          (2050, 2064, 136, 256, 1), (300, 384, 388, 5120, 0)])
+def test_gemm_per_256_scales_integer_sums(rt, T, Mp, N, K, acc):
+    """act32 = 0 on chunks of at least 256 token rows of Q4_K: the form of the 128 x 128 kernel that adds a superblock's
+    block sums up as integers (sc * I) and applies sa * d once per four blocks.  Against the double-accumulated
+    reference with the one scale on each of a superblock's eight blocks, the three epilogues, partly empty last tiles,
+    run to run."""
+    print(f"per-256 integer sums T={T} Mp={Mp} N={N} K={K} acc={acc}", flush=True)
+    eng = az.Engine(Mp, K)
+    W = make_weights(az.Q4_K, N, K, seed=75)
+    x = make_acts(T, K, seed=76, outliers=True)
+    c0 = np.random.default_rng(77).standard_normal((Mp, N)).astype(np.float32)
+    w = eng.make_weight(az.Q4_K, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, Mp, T, act32=0)
+    ys = []
+    for _ in range(2):
+        cb = az.Runtime.alloc(Mp * N * 4)
+        cb.write(c0) if acc else cb.fill(0xFFFFFFFF)
+        eng.matmul("test", w, Mp, cb, N, 0, acc, act32=False)
+        ys.append(cb.read(np.float32, Mp * N).reshape(Mp, N))
+        cb.free()
+    xb.free(); w.free(); eng.close()
+    assert np.array_equal(ys[0].view(np.uint32), ys[1].view(np.uint32))
+    xp = np.zeros((Mp, K), np.float32)
+    xp[:T] = x
+    raq, rasc, _ = orc.quantize_act(xp, act32=False)
+    ref = orc.matmul_ref(az.Q4_K, W, N, K, raq[:T], np.ascontiguousarray(np.repeat(rasc, 8, axis=0)[:, :T]))
+    if acc == 1:
+        ref = ref + c0[:T]
+    elif acc == 2:
+        g = c0[:T].astype(np.float64)
+        ref = ref * (g / (1.0 + np.exp(-g)))
+    y = ys[0][:T]
+    assert np.isfinite(y).all() and mixed_err(y, ref) <= TOL
+    if acc == 0:
+        assert not ys[0][T:].any()
+
+
 @pytest.mark.parametrize("qtype", [az.Q4_K, az.Q5_K])
 @pytest.mark.parametrize("T,Mp,N,K,acc", [(1100, 1104, 392, 512, 0), (1100, 1104, 390, 512, 0), (1030, 1040, 640, 768, 1),
                                           (760, 768, 520, 1024, 2), (1200, 1216, 132, 256, 0),
