@@ -230,7 +230,8 @@ __device__ __forceinline__ void gemm2_body(const uint8_t* __restrict__ raw, cons
                                   int m0, int rows_valid, int n0, const int* __restrict__ rowmap, int use_map,
                                   const float* __restrict__ rowscale, int use_scale) {
   __shared__ Gemm2Lds L;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // (a scalar: what follows from it alone is scalar arithmetic)
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
@@ -439,7 +440,8 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   constexpr int oSA = G3_SA, oWS = BF ? G3_SA + 2048 : G3_WS, oU = BF ? G3_SA + 4096 : G3_U, oV = BF ? G3_SA + 8192 : G3_V;
   constexpr int STAGE = BF ? G3_SA + 16384 : Q5 ? G3_STAGE + 2048 : G3_STAGE, QH = G3_STAGE;  // (Q5_K: the fifth bits behind the scale vectors)
   __shared__ alignas(16) uint8_t lds[2 * STAGE];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // (a scalar: the DMA destinations and bases that follow from it are scalar arithmetic)
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
@@ -858,7 +860,7 @@ __device__ __forceinline__ bool store_tile64(uint8_t* lds, const v16f (&res)[2],
                                              int accumulate, int m0, int rows_valid, int n0, int N,
                                              const float* __restrict__ rowscale, int use_scale) {
   if (n0 + BN > N || ((ldc | c_off) & 3) != 0 || ((uintptr_t)C & 15) != 0) return false;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l32 = lane & 31, g = lane >> 5;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), l32 = lane & 31, g = lane >> 5;
   float* rs = (float*)lds;
   uint8_t* tl = lds + 256;
   if (use_scale && t < G6_BM) rs[t] = t < rows_valid ? rowscale[m0 + t] : 0.0f;
@@ -907,7 +909,7 @@ __device__ __forceinline__ bool store_tile64(uint8_t* lds, const v16f (&res)[2],
 __device__ __forceinline__ void store_tile64_quant(uint8_t* lds, const v16f (&hv)[2], float* __restrict__ H, int F, int m0,
                                                    int rows_valid, int n0, int S, signed char* __restrict__ hq,
                                                    float* __restrict__ hsc, short* __restrict__ hbs) {
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l32 = lane & 31, g = lane >> 5;
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), l32 = lane & 31, g = lane >> 5;
   uint8_t* tl = lds + 256;
   float* lasc = (float*)(lds + 256 + 64 * 528);       // [4][64]
   short* lsum = (short*)(lds + 256 + 64 * 528 + 1024);  // [8][64]
@@ -961,7 +963,8 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
                                   size_t rows_total = 0, size_t row_base = 0, const int* __restrict__ rowmap = nullptr,
                                   int use_map = 0, const float* __restrict__ rowscale = nullptr, int use_scale = 0) {
   __shared__ alignas(16) uint8_t lds[2 * G6_STAGE];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // (a scalar: what follows from it alone is scalar arithmetic)
   const int l32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const PlanesQ6K pl = planes_q6k(TILES ? rows_total : (size_t)N, nsb);
@@ -989,7 +992,7 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
   // scales: threads 0-63 prepare token t (the step's 4 activation scales: one per thread and block -> 4 threads a
   // token would do; here thread t takes token t % 64, block t / 64); every thread prepares weight row t / 2: the four
   // sub-scales 4 (t % 2) .. + 3 of the step, and (t % 2 == 0) the row's d.
-  const int r_s = t & 63, b_s = t >> 6;
+  const int r_s = t & 63, b_s = wave;
   const bool tok_valid = r_s < rows_valid;
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
@@ -1183,7 +1186,8 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
   constexpr bool Q5 = QT == QT_Q5_K;
   constexpr int STAGE = Q5 ? G4_STAGE + 2048 : G4_STAGE, QH = G4_STAGE;
   __shared__ alignas(16) uint8_t lds[2 * STAGE];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // (a scalar: what follows from it alone is scalar arithmetic)
   const int l32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const PlanesQ4K pl = planes_q4k(rows_total, nsb);
@@ -1205,7 +1209,7 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
   const uint8_t* qbase = raw + pl.qh + (row_base * nsb + s_begin) * 32;  // Q5_K: row 64 wave + lane, waves 0 and 1
   uint32_t qoff = (uint32_t)min(n0 + (wave & 1) * 64 + lane, N - 1) * (uint32_t)nsb * 32u;
   // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t / 2, block pair t % 2
-  const int r_s = t & 63, b_s = t >> 6;
+  const int r_s = t & 63, b_s = wave;
   const bool tok_valid = r_s < rows_valid;
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
@@ -1452,7 +1456,7 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
   }
   const size_t wrow0 = pl.qs + row_base * nsb * 128;
   // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t % 128 of gate (t < 128) or up
-  const int r_s = t & 63, b_s = t >> 6;
+  const int r_s = t & 63, b_s = wave;
   const bool tok_valid = r_s < rows_valid;
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int row_s = t & 127, x_s = wave >> 1;
@@ -1724,7 +1728,7 @@ __device__ __forceinline__ void gemm8_body(const uint8_t* __restrict__ raw, cons
   const signed char* abase = aq + (size_t)s_begin * 256;
   const uint8_t* wbase = raw + pl.qs + (size_t)s_begin * 256;
   // scales: thread t prepares token t % 64, block t / 64 of the step, and weight row t / 2, blocks 2 (t % 2) + {0, 1}
-  const int r_s = t & 63, b_s = t >> 6;
+  const int r_s = t & 63, b_s = wave;
   const bool tok_valid = r_s < rows_valid;
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
