@@ -22,7 +22,7 @@ PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
 # HBM bytes one launch of the headline GEMM moves, from two counter runs of this script (FETCH_SIZE x 2.0 KiB read,
 # WRITE_SIZE x 1.0 KiB written, the factors calibrated on the 2 GiB copy in the same runs): 2745.3 MB + 570.4 MB
-GEMM_HBM_BYTES_PER_LAUNCH = 3.316e9
+GEMM_HBM_BYTES_PER_LAUNCH = 3.313e9
 
 
 def log(*a):
