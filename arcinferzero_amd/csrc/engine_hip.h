@@ -470,18 +470,18 @@ class Engine {
       throw std::runtime_error(std::string("matmul ") + name + ": the output does not fit C");
     int a = acc;
     cl_mem tabs = tabs_;  // (the reference's codebook tables; IQ3_S's kernels read theirs from it)
-    // A few tokens of Q4_K, Q5_K, Q6_K, Q8_0, Q4_0 or IQ4_XS: the matrix-vector form on the matrix pipe (gemv_mm; it
+    // A few tokens, any weight type: the matrix-vector form on the matrix pipe (gemv_mm; it
     // takes K in slices of the tokens that fit LDS).  It takes 9-16 tokens in chunks of 16 rows (what the reference pads
     // them to, zero/engine.h:522; the rows from T on come out as zeros, as the GEMM writes them: Q4_K 21 against 95 us at
     // 17408 x 5120), and 3-8 tokens where it is the faster one: from 5 on always (us at the settled clock, 8 tokens,
     // against the dot-product kernels, 17408 x 5120: Q4_K 20.8 / 27.6, Q5_K 21.5 / 30.5, Q6_K 31.0 / 33.1, Q8_0 23.7 /
-    // 31.4, Q4_0 20.2 / 27.7, IQ4_XS 23.4 / 31.0; with 4 tokens 20.5 / 18.9, 21.4 / 20.7, 30.8 / 23.2, 23.6 / 20.1,
+    // 31.4, Q4_0 20.2 / 27.7, IQ4_XS 23.4 / 31.0, IQ3_S 26.4 / 32.9; with 4 tokens 20.5 / 18.9, 21.4 / 20.7, 30.8 / 23.2, 23.6 / 20.1,
     // 20.4 / 17.1, 23.3 / 20.0: not taken; ARCZ_GEMV_MM_MIN: the first count it takes), 3 and 4 when the tokens do not
     // fit the LDS of the dot-product kernels (5120 x 17408, 4 tokens: Q4_K 34 against 88 us, Q5_K 42 against 97).  Not
     // with two-pass inputs (their second half goes through the kernels below).  ARCZ_GEMV_MM=0: off.
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
     const bool mm_type = w.type == GGML_Q4_K || w.type == GGML_Q5_K || w.type == GGML_Q6_K || w.type == GGML_Q8_0 ||
-                         w.type == GGML_Q4_0 || w.type == GGML_IQ4_XS;
+                         w.type == GGML_Q4_0 || w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S;
     const bool mm_ok = !mm_off && !q2mm_ && mm_type && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;

@@ -1,5 +1,5 @@
 // "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0,
-// Q4_0, IQ4_XS).
+// Q4_0, IQ4_XS, IQ3_S).
 //
 // From a handful of tokens on, the dot-product GEMVs are bound by their vector ALU work (eight v_dot4 per token and
 // 16-byte unit), not by memory, and past eight tokens the engine had only the prefill GEMM with its 64-token tiles.
@@ -57,16 +57,22 @@ template <> struct MmT<QT_Q6_K> { enum { SB = 20, QB = 128, D = 4, XB = 64, MIN 
 template <> struct MmT<QT_Q8_0> { enum { SB = 24, QB = 256, D = 4, XB = 0, MIN = 0, DPL = 0 }; };
 template <> struct MmT<QT_Q4_0> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 0, DPL = 0 }; };
 template <> struct MmT<QT_IQ4_XS> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 0, DPL = 0 }; };
+// (IQ3_S: the main plane is the 8 index bytes per block, the second the sign bits, the header the ninth bits and scale
+//  nibbles, 12 bytes; the codebook, 2 KiB, sits behind the groups' sums in LDS)
+template <> struct MmT<QT_IQ3_S> { enum { SB = 22, QB = 64, D = 8, XB = 32, MIN = 0, DPL = 1 }; };
 // LDS: per superblock of a slice 4096 bytes of tokens and 512 of sa (512 more of sa * S); per wave the main plane's rows
 // of one superblock, 1 KiB of headers, the second plane's four superblocks, 256 bytes of d; then 1 KiB per group whose
 // sums wait for the last slice (as many as fit, 12 at most)
 template <int QT> struct MmL {
   static constexpr int TOK = 4096 + 512 + (MmT<QT>::MIN ? 512 : 0);
-  static constexpr int WQ = MmT<QT>::QB * 16, WH = 1024, WX = MmT<QT>::XB * 64, WD = MmT<QT>::DPL ? 256 : 0;
+  static constexpr int WQ = MmT<QT>::QB * 16 < 2048 ? 2048 : MmT<QT>::QB * 16;  // (also the wave's two partial sums: 2 KiB)
+  static constexpr int WH = 1024, WX = MmT<QT>::XB * 64, WD = MmT<QT>::DPL ? 256 : 0;
+  static constexpr int GRID = QT == QT_IQ3_S ? 2048 : 0;
   static constexpr int WSZ = WQ + WH + WX + WD;
-  static constexpr int FREE = (MM_LDS_MAX - MmT<QT>::SB * TOK - MM_WAVES * WSZ) / 1024;
+  static constexpr int FREE = (MM_LDS_MAX - MmT<QT>::SB * TOK - MM_WAVES * WSZ - GRID) / 1024;
   static constexpr int GA = FREE < 12 ? FREE : 12;
-  static constexpr int LDS = MmT<QT>::SB * TOK + MM_WAVES * WSZ + GA * 1024;
+  static constexpr int OGRID = MmT<QT>::SB * TOK + MM_WAVES * WSZ + GA * 1024;
+  static constexpr int LDS = OGRID + GRID;
   static_assert(GA >= 1, "no room for the groups' sums");
 };
 
@@ -74,7 +80,14 @@ template <int QT> struct MmQ { mm_u4 r[MmT<QT>::QB / 64]; };  // the lane's 16-b
 template <int QT> struct MmX { mm_u4 r[MmT<QT>::XB / 16 > 0 ? MmT<QT>::XB / 16 : 1]; uint32_t d; };  // of four superblocks' second plane
 // a superblock as the products take it: the lane's 8 bytes of each 32-byte chunk of the main plane, the header
 // (Q4_0 and IQ4_XS: of each 16-byte block)
-template <int QT> struct MmSb { mm_u2 c[QT == QT_Q4_0 || QT == QT_IQ4_XS ? 8 : MmT<QT>::QB / 32]; mm_u4 h; mm_u2 x[2]; uint32_t d; };
+// (IQ3_S: c[b].x the lane's two index bytes of block b, sg the row's eight words of sign bits)
+template <int QT> struct MmSb {
+  mm_u2 c[QT == QT_Q4_0 || QT == QT_IQ4_XS || QT == QT_IQ3_S ? 8 : MmT<QT>::QB / 32];
+  mm_u4 h;
+  mm_u2 x[2];
+  uint32_t d;
+  mm_u4 sg[QT == QT_IQ3_S ? 2 : 1];
+};
 
 // one slice of K, superblocks [s_begin, s_end): at most MmT<QT>::SB of them
 template <int QT>
@@ -87,7 +100,8 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   constexpr int QB = TT::QB, NQ = QB / 64, D = TT::D, LPRW = QB / 16, RPI = 64 / LPRW;
   constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
   constexpr bool B16 = QT == QT_Q4_0 || QT == QT_IQ4_XS;  // a block is 16 bytes: low nibbles values 0..15, high 16..31
-  constexpr int HB = QT == QT_IQ4_XS ? 8 : 16;            // bytes of a row's superblock in the header plane
+  constexpr int HB = QT == QT_IQ4_XS ? 8 : QT == QT_IQ3_S ? 12 : 16;  // bytes of a row's superblock in the header plane
+  constexpr bool I3 = QT == QT_IQ3_S;
   const int tid = threadIdx.x, lane = tid & 63, n16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (a scalar: what follows from it is scalar arithmetic)
   const int nsb = K >> 8, sbs = s_end - s_begin, Ks = sbs * 256, nb = sbs * 8;
@@ -111,6 +125,9 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     o_hdr = planes_q80((size_t)N, nsb).d;
   } else if constexpr (QT == QT_Q4_0) {
     o_hdr = planes_q40((size_t)N, nsb).d;
+  } else if constexpr (I3) {
+    const PlanesIQ3S pl = planes_iq3s((size_t)N, nsb);
+    o_hdr = pl.hd; o_x = pl.sg; o_d = pl.d;
   } else {
     o_hdr = planes_iq4xs((size_t)N, nsb).hdr;
   }
@@ -146,6 +163,9 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     const int r = min((gb0 + gl) * 16 + n16, N - 1);
     if constexpr (HB == 16) {
       h = *(const mm_u4*)(hd + ((size_t)r * nsb + s_begin + sb) * 16);
+    } else if constexpr (HB == 12) {
+      const uint32_t* hp = (const uint32_t*)(hd + ((size_t)r * nsb + s_begin + sb) * 12);
+      h = mm_u4{hp[0], hp[1], hp[2], 0};
     } else {
       const mm_u2 h2 = *(const mm_u2*)(hd + ((size_t)r * nsb + s_begin + sb) * 8);
       h = mm_u4{h2.x, h2.y, 0, 0};
@@ -234,16 +254,18 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
 #pragma unroll
   for (int i = 0; i < NQ; ++i) {
     const int p = lane % LPRW, r = i * RPI + lane / LPRW;
-    wq[i] = (16 * p + (r ^ (LPRW == 8 ? 2 * p : p))) << 4;
+    wq[i] = I3 ? r * 64 + ((p ^ (r >> 2)) << 4) : (16 * p + (r ^ (LPRW == 8 ? 2 * p : p))) << 4;
   }
   // (the lane's 8 bytes: bytes 8 g .. of each 32-byte chunk; for the 16-byte blocks bytes 8 (g & 1) .. of each block,
   //  whose low nibbles are the values of lanes g < 2 and whose high nibbles those of g >= 2)
-  constexpr int NC = B16 ? 8 : QB / 32;
+  // (IQ3_S: the row's 64 index bytes lie together, 16-byte pieces XOR-ed with row / 4; the lane's are bytes 8 b + 2 g, + 1)
+  constexpr int NC = B16 || I3 ? 8 : QB / 32;
   int rd[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const int p = B16 ? c : 2 * c + (g >> 1);
-    rd[c] = ((16 * p + (n16 ^ (LPRW == 8 ? 2 * p : p))) << 4) + (g & 1) * 8;
+    rd[c] = I3 ? n16 * 64 + (((c >> 1) ^ (n16 >> 2)) << 4) + 8 * (c & 1) + 2 * g
+               : ((16 * p + (n16 ^ (LPRW == 8 ? 2 * p : p))) << 4) + (g & 1) * 8;
   }
   const uint8_t* arow = A + n16 * Ks + (g & 1) * 8;
 
@@ -341,6 +363,29 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] = fmaf(d, part[i], acc[i]);
+    } else if constexpr (I3) {
+      // block b: indices 2 g and 2 g + 1 of its eight (a byte each and a ninth bit from byte b of the header) name
+      // codebook words of four magnitudes, the signs are bits 8 g .. 8 g + 7 of the block's word; scale 1 + 2 x nibble b
+      // of the header's third word, times d (reference src/quants.h IQ3_S, zero/kernels/decode.cl:183-478)
+      const uint32_t* grid = (const uint32_t*)(lds + LL::OGRID);
+      const float d3 = f16_bits_to_f32(h.d);
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const uint32_t q16 = h.c[b].x;
+        const uint32_t n9 = (b < 4 ? h.h.x : h.h.y) >> (8 * (b & 3) + 2 * g);
+        const uint32_t g0 = grid[(q16 & 0xFFu) | ((n9 & 1u) << 8)], g1 = grid[((q16 >> 8) & 0xFFu) | ((n9 & 2u) << 7)];
+        const uint32_t sw = b < 4 ? h.sg[0][b & 3] : h.sg[1][b & 3];
+        const uint32_t s8 = sw >> (8 * g);
+        const uint32_t w0 = iq3s_signed4(g0, s8 & 0xFu), w1 = iq3s_signed4(g1, (s8 >> 4) & 0xFu);
+        const long wv = (long)(((unsigned long)w1 << 32) | w0);
+        v4i z = {0, 0, 0, 0};
+        const v4i I = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wv, z, 0, 0, 0);
+        const float d = d3 * (float)(1 + 2 * (int)((h.h.z >> (4 * b)) & 0xFu));
+        acc[0] = fmaf((float)I[0], sa4[b].x * d, acc[0]);
+        acc[1] = fmaf((float)I[1], sa4[b].y * d, acc[1]);
+        acc[2] = fmaf((float)I[2], sa4[b].z * d, acc[2]);
+        acc[3] = fmaf((float)I[3], sa4[b].w * d, acc[3]);
+      }
     } else if constexpr (B16) {
       // block b is the 16 bytes 16 b .. of the row's 128; Q4_0: value nibble - 8, f16 scale entry b of the header;
       // IQ4_XS: the table's value of the nibble, d in the header's first half word and a 6-bit scale - 32 per block (low
@@ -426,8 +471,16 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     qload(qq, min(u + D, ulast));
     if (u < u1) {
       MmSb<QT> s;
+      if constexpr (I3) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) s.c[c] = *(const mm_u2*)(WQ + rd[c]);
+        for (int c = 0; c < NC; ++c) s.c[c] = mm_u2{(uint32_t) * (const unsigned short*)(WQ + rd[c]), 0u};
+        s.sg[0] = *(const mm_u4*)(WX + (j * 16 + n16) * 32);
+        s.sg[1] = *(const mm_u4*)(WX + (j * 16 + n16) * 32 + 16);
+        s.d = *(const uint32_t*)(WD + ((j * 16 + n16) << 2));
+      } else {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) s.c[c] = *(const mm_u2*)(WQ + rd[c]);
+      }
       s.h = *(const mm_u4*)(WH + ((j * 16 + n16) << 4));
       if constexpr (QT == QT_Q5_K) {
         // words g / 2, 2 + g / 2, 4 + g / 2, 6 + g / 2 of the row's 8 words of fifth bits
@@ -511,12 +564,15 @@ template <int QT>
 __device__ inline void mm_kernel(uint8_t* lds, const uint8_t* __restrict__ raw, int N, int K,
                                  const signed char* __restrict__ aq, const float* __restrict__ asc,
                                  const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off, int accumulate,
-                                 int s_begin, int s_end) {
+                                 int s_begin, int s_end, const uint32_t* __restrict__ tabs) {
   constexpr int SB = MmT<QT>::SB;
   const int all = s_end - s_begin, slices = (all + SB - 1) / SB;
   const int groups = (N + 15) >> 4, gd = (int)gridDim.x;
   const int ng = (int)((long)(blockIdx.x + 1) * groups / gd) - (int)((long)blockIdx.x * groups / gd);
   float* GA = slices > 1 && ng <= MmL<QT>::GA ? (float*)(lds + SB * MmL<QT>::TOK + MM_WAVES * MmL<QT>::WSZ) : nullptr;
+  if constexpr (QT == QT_IQ3_S) {  // (the codebook: the first 512 words of the tables; the first slice's meeting orders it)
+    for (int i = threadIdx.x; i < 512; i += 512) ((uint32_t*)(lds + MmL<QT>::OGRID))[i] = tabs[i];
+  }
   for (int sl = 0; sl < slices; ++sl) {
     if (sl) __syncthreads();  // (the tokens and partial sums of the slice before have been read)
     mm_slice<QT>(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, GA ? accumulate : (accumulate || sl),
@@ -530,7 +586,7 @@ __device__ inline void mm_kernel(uint8_t* lds, const uint8_t* __restrict__ raw, 
       const float* __restrict__ asc, const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off,       \
       int accumulate, int s_begin, int s_end) {                                                                         \
     __shared__ __attribute__((aligned(16))) uint8_t lds[MmL<QTV>::LDS];                                                 \
-    mm_kernel<QTV>(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, s_begin, s_end);                    \
+    mm_kernel<QTV>(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, s_begin, s_end, tabs);              \
   }
 MM_KERNEL(12)
 MM_KERNEL(13)
@@ -538,3 +594,4 @@ MM_KERNEL(14)
 MM_KERNEL(8)
 MM_KERNEL(2)
 MM_KERNEL(23)
+MM_KERNEL(21)
