@@ -487,8 +487,43 @@ class Engine {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
       rd_bytes += raw_bytes(w);
       cl_kernel k = kernel("decode", "-DQT=" + std::to_string(w.type), "gemv_mm");
-      const size_t groups = (size_t)(N + 15) / 16;
-      size_t g1 = std::min<size_t>(groups, (size_t)arcz_device_cus()) * 512, l1 = 512;
+      const size_t groups = (size_t)(N + 15) / 16, cus = (size_t)arcz_device_cus();
+      // Rows longer than the tokens' LDS holds (slices of sb_max superblocks): K is shared out over `ny` work-groups
+      // per run of groups, each staging its piece of the tokens once, and gemv_mm_reduce adds the pieces -- inside one
+      // work-group the slices are staged one after the other, and 320 groups on 256 work-groups leave a quarter of them
+      // two groups and the rest one (8 tokens, us: 5120 x 17408 Q4_K 34.4 -> 22.6, Q6_K 58.0 -> 32.1, Q8_0 34.4 -> 25.7;
+      // 17408 x 17408 Q4_K 60.7 -> 44.9; 40960 x 8192 Q4_K 60.9 -> 46.7, Q8_0 69.1 -> 72.5).  Up to 12 groups a compute
+      // unit (ARCZ_GEMV_MM_SK=n: n, 0: never); beyond that, and when the workspace is not to be had, the kernel walks
+      // the slices itself.
+      static const int sk_env = getenv("ARCZ_GEMV_MM_SK") ? atoi(getenv("ARCZ_GEMV_MM_SK")) : -1;
+      static const bool sk_off = sk_env == 0;
+      const size_t sk_groups = (size_t)(sk_env > 0 ? sk_env : 12) * cus;
+      const int nsb = K / 256;
+      const int sb_max = w.type == GGML_Q6_K ? 20 : w.type == GGML_Q5_K || w.type == GGML_IQ3_S ? 22 : 24;  // (the kernels' MmT<QT>::SB)
+      const int ny = (nsb + sb_max - 1) / sb_max;
+      const size_t need = (size_t)ny * 16 * N * 4;
+      cl_mem ws = noalloc_ ? arcz_scratch_mem() : sk_ws_;
+      if (!sk_off && ny >= 2 && groups <= sk_groups && (!noalloc_ || need <= arcz_mem_size(ws))) {
+        if (!noalloc_ && need > sk_ws_bytes_) {
+          if (sk_ws_) release(sk_ws_);
+          sk_ws_ = nullptr;
+          sk_ws_bytes_ = 0;
+          sk_ws_ = buf(need);
+          sk_ws_bytes_ = need;
+          ws = sk_ws_;
+        }
+        int zero = 0, ldw = N, s1 = nsb;
+        set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, ws, ldw, zero, zero, zero, s1);
+        size_t g2[2] = {std::min<size_t>(groups, std::max<size_t>(cus / (size_t)ny, 1)) * 512, (size_t)ny}, l2[2] = {512, 1};
+        run(name, k, 2, g2, l2);
+        cl_kernel kr = kernel("decode", "", "gemv_mm_reduce");
+        int rows = T > 8 ? 16 : T, nyy = ny;
+        set_args(kr, 0, ws, nyy, C, rows, N, ldc, c_off, a);
+        size_t g3 = ((size_t)rows * N + 255) / 256 * 256, l3 = 256;
+        run(name, kr, 1, &g3, &l3);
+        return;
+      }
+      size_t g1 = std::min<size_t>(groups, cus) * 512, l1 = 512;
       set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, T, C, ldc, c_off, a, 0, K / 256);
       run(name, k, 1, &g1, &l1);
     };

@@ -47,6 +47,7 @@ static const KernelSpec kKernelTable[] = {
     {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "LPR", "PF", "TB", nullptr},
      {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
+    {"decode", "gemv_mm_reduce", nullptr, "pipiiiii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"decode", "gemv_mm", nullptr, "piippppiipiiiii", {"QT", nullptr}, {{nullptr, 0, false}}, 512},
     {"decode", "moe_gateup_q", "ROUTE", "ppiipppippppipppppppiiipp", {"QT", "GROWS", "TM", "QUANT", "ROUTE", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 512},
     {"decode", "moe_gateup_q", "QUANT", "ppiipppippppippp", {"QT", "GROWS", "TM", "QUANT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 512},

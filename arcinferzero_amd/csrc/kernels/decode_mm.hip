@@ -586,7 +586,11 @@ __device__ inline void mm_kernel(uint8_t* lds, const uint8_t* __restrict__ raw, 
       const float* __restrict__ asc, const short* __restrict__ absum, int M, int T, float* C, int ldc, int c_off,       \
       int accumulate, int s_begin, int s_end) {                                                                         \
     __shared__ __attribute__((aligned(16))) uint8_t lds[MmL<QTV>::LDS];                                                 \
-    mm_kernel<QTV>(lds, raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, s_begin, s_end, tabs);              \
+    /* gridDim.y > 1: K shared out over the work-groups (x, y), y-th of gridDim.y even pieces of the superblocks, the    \
+       partial sums into plane y of C, here a workspace [gridDim.y][16][ldc] that gemv_mm_reduce adds up */              \
+    const int ny = (int)gridDim.y, y = (int)blockIdx.y, all = s_end - s_begin;                                          \
+    mm_kernel<QTV>(lds, raw, N, K, aq, asc, absum, M, T, C + (size_t)y * 16 * ldc, ldc, c_off, accumulate,              \
+                   s_begin + all * y / ny, s_begin + all * (y + 1) / ny, tabs);                                         \
   }
 MM_KERNEL(12)
 MM_KERNEL(13)
@@ -595,3 +599,16 @@ MM_KERNEL(8)
 MM_KERNEL(2)
 MM_KERNEL(23)
 MM_KERNEL(21)
+
+// gemv_mm_reduce: C[t][c_off + n] (=, +=) the sum over the ny planes of ws [ny][16][N], plane 0 first, for the `rows`
+// token rows a launch stores.  grid: ceil(rows * N / 256) work-groups of 256.
+extern "C" __global__ __launch_bounds__(256) void gemv_mm_reduce(const float* __restrict__ ws, int ny, float* C, int rows, int N,
+                                                                 int ldc, int c_off, int accumulate) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= rows * N) return;
+  const int t = i / N, n = i - t * N;
+  float v = ws[(size_t)t * N + n];
+  for (int y = 1; y < ny; ++y) v += ws[((size_t)y * 16 + t) * N + n];
+  float* cp = C + (size_t)t * ldc + c_off + n;
+  *cp = accumulate ? *cp + v : v;
+}

@@ -25,7 +25,8 @@ CASES = [(7, 100, 256), (8, 1000, 5120), (9, 333, 2048), (13, 4097, 1024), (16, 
          (3, 77, 17408), (6, 300, 17408), (12, 129, 17408), (5, 200, 5120), (4, 5120, 17408),
          # rounds of one, two and four waves a group, then the rest spread wider
          (7, 33000, 256), (16, 20000, 1024), (8, 17408, 512), (11, 17408, 5120),
-         # several slices of K: the sums wait in LDS, or (13 groups to a work-group) are added to C slice by slice
+         # several slices of K inside the kernel (more than 12 groups a compute unit: K is not shared out over
+         # work-groups): the sums wait in LDS, or (13 groups to a work-group) are added to C slice by slice
          (8, 53000, 6400)]
 
 
@@ -63,7 +64,8 @@ def test_gemv_mm_parity(eng, T, N, K):
 
 
 # the other types of the matrix-pipe form: a slice of K, several slices (22 / 20 / 24 superblocks at most for Q5_K / Q6_K /
-# Q8_0), rows that do not fill a group, work-groups with several groups, more groups than wait in LDS
+# Q8_0; shared out over work-groups with a reduce behind them, or -- the last case -- walked inside the kernel), rows
+# that do not fill a group, work-groups with several groups, more groups than wait in LDS
 CASES_TYPES = [(8, 100, 256), (16, 333, 2048), (13, 1000, 5120), (7, 129, 17408), (16, 5120, 6400), (9, 17408, 1024),
                (8, 53000, 6400)]
 
