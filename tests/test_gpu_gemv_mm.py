@@ -76,6 +76,38 @@ def test_gemv_mm_parity_types(eng, qt, T, N, K):
     _parity(eng, qt, T, N, K)
 
 
+@pytest.mark.parametrize("qt,T,N,K", [(az.Q4_K, 7, 200, 1024), (az.Q4_K, 12, 130, 17408), (az.Q6_K, 16, 96, 6400),
+                                      (az.Q8_0, 5, 333, 8192)])
+def test_gemv_mm_into_a_wider_output(eng, qt, T, N, K):
+    """The output as columns [c_off, c_off + N) of rows of ldc values, stored and accumulated: nothing outside them is
+    touched (K within a slice, and shared out over work-groups with the reduce behind them)."""
+    print(f"gemv_mm wide output type={qt} T={T} N={N} K={K}", flush=True)
+    ldc, c_off = N + 24, 8
+    W = make_weights(qt, N, K, seed=840 + T)
+    x = make_acts(T, K, seed=841 + T, outliers=True)
+    w = eng.make_weight(qt, N, K, W)
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, 16, T)
+    rows = T if T <= 8 else 16
+    c0 = np.random.default_rng(842).standard_normal((rows, ldc)).astype(np.float32)
+    cb = az.Runtime.alloc(rows * ldc * 4)
+    aq, asc, _ = quantize_padded(x, 16)
+    ref = orc.matmul_ref(qt, W, N, K, aq[:T], asc)
+    for acc in (0, 1):
+        cb.write(c0)
+        eng.matmul("mm", w, 16, cb, ldc, c_off, acc)
+        y = cb.read(np.float32, rows * ldc).reshape(rows, ldc)
+        assert np.array_equal(y[:, :c_off], c0[:, :c_off]) and np.array_equal(y[:, c_off + N:], c0[:, c_off + N:])
+        want = ref + (c0[:T, c_off:c_off + N] if acc else 0.0)
+        assert rel_err_rows(y[:T, c_off:c_off + N], want).max() <= 1e-3
+        if rows > T:
+            pad = y[T:, c_off:c_off + N]
+            assert np.array_equal(pad, c0[T:, c_off:c_off + N]) if acc else not pad.any()
+    for b in (cb, xb):
+        b.free()
+    w.free()
+
+
 @pytest.mark.parametrize("T,N,K", [(8, 48, 512), (16, 37, 7168)])
 @pytest.mark.parametrize("qt", [az.Q4_K, az.Q5_K, az.Q6_K, az.Q4_0, az.IQ4_XS, az.IQ3_S])
 def test_gemv_mm_unit_scales_exact(eng, qt, T, N, K):
