@@ -169,9 +169,12 @@ def _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp):
         print(f"  down + combine on the GPU's int8 h: rel err {err2.max():.2e}")
         assert err2.max() <= 1e-3
         # The whole layer against the oracle's own two stages: every token whose int8 h equals the oracle's
-        same = ~np.isin(np.arange(T), np.nonzero((hq[inv] != orc.moe_quant(href)[0]).any(axis=1))[0] // NU)
-        print(f"  tokens with an int8 h one step from the oracle's: {int((~same).sum())}")
-        assert (~same).sum() <= max(1, T // 20)
+        dq = hq[inv].astype(np.int32) - orc.moe_quant(href)[0].astype(np.int32)
+        same = ~np.isin(np.arange(T), np.nonzero(dq.any(axis=1))[0] // NU)
+        print(f"  int8 h values one step from the oracle's: {int((dq != 0).sum())} of {dq.size}, in {int((~same).sum())} tokens")
+        # (a value of h within an ulp or two of a rounding boundary, or a block whose largest value is: a few in a million,
+        #  never more than one step)
+        assert np.abs(dq).max() <= 1 and (dq != 0).sum() <= 4 + dq.size // 10000
         assert err[same].max(initial=0.0) <= 1e-3
         if T >= 17:
             # the tile passes keep the down projection's weighted rows in y [S][E]: each expert's slots against the
