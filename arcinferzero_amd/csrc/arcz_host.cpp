@@ -13,6 +13,8 @@
 #include "kernels/common.h"
 #define GGML_TYPE_Q4_0 2u  // (GGUF type id, src/gguf.h:19)
 #define GGML_TYPE_IQ3_S 21u  // (src/gguf.h:22)
+#define GGML_TYPE_IQ4_NL 20u  // (src/gguf.h:21)
+#define GGML_TYPE_MXFP4 39u  // (src/gguf.h:23)
 
 namespace {
 
@@ -115,7 +117,8 @@ extern "C" {
 
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
-  return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : type == GGML_TYPE_IQ3_S ? u * 110 : 0;
+  return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : type == GGML_TYPE_IQ3_S ? u * 110
+         : type == GGML_TYPE_IQ4_NL ? u * 144 : type == GGML_TYPE_MXFP4 ? u * 136 : 0;
 }
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) { return raw_planes_bytes((int)type, rows, K / 256); }
 // The IQ3_S codebook as the kernels take it: 512 words, byte j of a word = magnitude j of the entry (1, 3, ..., 15).
@@ -219,9 +222,24 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
       }
     return 0;
   }
-  if (type == GGML_TYPE_Q4_0) {
-    // eight 18-byte blocks (f16 d, 16 bytes of nibbles: low = elements 0..15, high = 16..31, value = nibble - 8;
-    // reference src/quants.h:136-148) -> 128 bytes of nibbles and 8 scales per superblock
+  if (type == GGML_TYPE_MXFP4) {
+    // eight 17-byte blocks (E8M0 scale byte, 16 bytes of nibbles: low = elements 0..15, high = 16..31, each an E2M1
+    // code; reference src/quants.h:520-530) -> 128 bytes of nibbles and 8 scale bytes per superblock
+    const PlanesMXFP4 pl = planes_mxfp4(rows, nsb);
+    memset(dst + pl.e + u * 8, 0, raw_planes_bytes(QT_MXFP4, rows, nsb) - (pl.e + u * 8));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i)
+      for (int b = 0; b < 8; ++b) {
+        const uint8_t* blk = src + i * 136 + 17 * b;
+        dst[pl.e + i * 8 + b] = blk[0];
+        memcpy(dst + pl.qs + i * 128 + 16 * b, blk + 1, 16);
+      }
+    return 0;
+  }
+  if (type == GGML_TYPE_Q4_0 || type == GGML_TYPE_IQ4_NL) {
+    // eight 18-byte blocks (f16 d, 16 bytes of nibbles: low = elements 0..15, high = 16..31; Q4_0: value = nibble - 8,
+    // IQ4_NL: the nibble's entry of the IQ4 table; reference src/quants.h:136-148, 594-606) -> 128 bytes of nibbles and
+    // 8 scales per superblock
     const PlanesQ40 pl = planes_q40(rows, nsb);
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < u; ++i)
@@ -517,7 +535,70 @@ static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) 
   }
 }
 
-// Quantizes f32 rows to `type` (2, 8, 12, 13, 14, 21, 23).  0 or -1.
+// f32 rows -> GGUF IQ4_NL blocks (18 bytes per 32 values; reference src/quants.h:594-606): d = (the value of largest
+// magnitude) / -127, which that value then decodes to exactly; every value takes the nearest entry of the table.  An
+// input generator for tests: no search over scales as a real quantizer would make.
+static void arcz_quantize_iq4_nl(const float* src, size_t N, int K, uint8_t* out) {
+  static const int kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < (int64_t)(N * (size_t)(K / 32)); ++b) {
+    const float* v = src + b * 32;
+    float amax = 0.0f, mx = 0.0f;
+    for (int i = 0; i < 32; ++i)
+      if (std::fabs(v[i]) > amax) { amax = std::fabs(v[i]); mx = v[i]; }
+    uint8_t* blk = out + b * 18;
+    const uint16_t dh = f32_to_f16(mx / -127.0f);
+    const float d = f16_to_f32(dh), id = d != 0.0f ? 1.0f / d : 0.0f;
+    memcpy(blk, &dh, 2);
+    memset(blk + 2, 0, 16);
+    for (int i = 0; i < 32; ++i) {
+      const float x = v[i] * id;
+      int best = 0;
+      float be = 1e30f;
+      for (int c = 0; c < 16; ++c) {
+        const float e = std::fabs(x - (float)kv[c]);
+        if (e < be) { be = e; best = c; }
+      }
+      blk[2 + (i & 15)] |= (uint8_t)(best << (4 * (i >> 4)));
+    }
+  }
+}
+
+// f32 rows -> GGUF MXFP4 blocks (17 bytes per 32 values; reference src/quants.h:495-503, 520-530): the scale byte e is
+// the smallest with amax <= 12 * 2^(e - 128) (12 = the table's largest entry), every value takes the nearest of
+// +-{0, 1, 2, 3, 4, 6, 8, 12} * 2^(e - 128).  An input generator for tests.
+static void arcz_quantize_mxfp4(const float* src, size_t N, int K, uint8_t* out) {
+  static const int kv[8] = {0, 1, 2, 3, 4, 6, 8, 12};
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < (int64_t)(N * (size_t)(K / 32)); ++b) {
+    const float* v = src + b * 32;
+    float amax = 0.0f;
+    for (int i = 0; i < 32; ++i) amax = std::fmax(amax, std::fabs(v[i]));
+    int e = 0;
+    if (amax > 0.0f) {
+      int ex;
+      const float m = std::frexp(amax / 12.0f, &ex);  // amax / 12 = m 2^ex, 0.5 <= m < 1
+      e = std::min(254, std::max(0, (m == 0.5f ? ex - 1 : ex) + 128));
+    }
+    uint8_t* blk = out + b * 17;
+    blk[0] = (uint8_t)e;
+    memset(blk + 1, 0, 16);
+    const float id = std::ldexp(1.0f, 128 - e);
+    for (int i = 0; i < 32; ++i) {
+      const float x = std::fabs(v[i]) * id;
+      int best = 0;
+      float be = 1e30f;
+      for (int c = 0; c < 8; ++c) {
+        const float er = std::fabs(x - (float)kv[c]);
+        if (er < be) { be = er; best = c; }
+      }
+      if (v[i] < 0.0f && best) best |= 8;
+      blk[1 + (i & 15)] |= (uint8_t)(best << (4 * (i >> 4)));
+    }
+  }
+}
+
+// Quantizes f32 rows to `type` (2, 8, 12, 13, 14, 20, 21, 23, 39).  0 or -1.
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
   if (K <= 0 || K % 256) return -1;
   if (type == GGML_TYPE_Q4_0) arcz_quantize_q4_0(src, N, K, out);
@@ -527,6 +608,8 @@ int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t
   else if (type == QT_Q6_K) arcz_quantize_q6_k(src, N, K, out);
   else if (type == QT_IQ4_XS) arcz_quantize_iq4_xs(src, N, K, out);
   else if (type == GGML_TYPE_IQ3_S) arcz_quantize_iq3_s(src, N, K, out);
+  else if (type == GGML_TYPE_IQ4_NL) arcz_quantize_iq4_nl(src, N, K, out);
+  else if (type == GGML_TYPE_MXFP4) arcz_quantize_mxfp4(src, N, K, out);
   else return -1;
   return 0;
 }

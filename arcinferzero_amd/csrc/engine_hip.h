@@ -22,6 +22,8 @@
 #define GGML_Q5_K 13u
 #define GGML_Q6_K 14u
 #define GGML_IQ4_XS 23u
+#define GGML_IQ4_NL 20u
+#define GGML_MXFP4 39u
 
 extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
 extern "C" size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
@@ -40,7 +42,7 @@ struct GpuWeight {
 
 inline const char* ggml_type_name(uint32_t t) {
   return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : t == GGML_IQ4_XS ? "IQ4_XS"
-         : t == GGML_Q4_0 ? "Q4_0" : t == GGML_IQ3_S ? "IQ3_S" : "?";
+         : t == GGML_Q4_0 ? "Q4_0" : t == GGML_IQ3_S ? "IQ3_S" : t == GGML_IQ4_NL ? "IQ4_NL" : t == GGML_MXFP4 ? "MXFP4" : "?";
 }
 
 class Engine {
@@ -210,7 +212,7 @@ class Engine {
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
     if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS &&
-        type != GGML_IQ3_S)
+        type != GGML_IQ3_S && type != GGML_IQ4_NL && type != GGML_MXFP4)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
     if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))
@@ -481,7 +483,8 @@ class Engine {
     // with two-pass inputs (their second half goes through the kernels below).  ARCZ_GEMV_MM=0: off.
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
     const bool mm_type = w.type == GGML_Q4_K || w.type == GGML_Q5_K || w.type == GGML_Q6_K || w.type == GGML_Q8_0 ||
-                         w.type == GGML_Q4_0 || w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S;
+                         w.type == GGML_Q4_0 || w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S || w.type == GGML_IQ4_NL ||
+                         w.type == GGML_MXFP4;
     const bool mm_ok = !mm_off && !q2mm_ && mm_type && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
@@ -576,7 +579,7 @@ class Engine {
         // 17408 x 5120: 20.2 against 25.7 with one; three or four per unit are slower everywhere).
         static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
         static const int wgs_env = getenv("ARCZ_GEMV_WGS") ? atoi(getenv("ARCZ_GEMV_WGS")) : 0;
-        const bool codebook = w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S;
+        const bool codebook = w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S || w.type == GGML_IQ4_NL || w.type == GGML_MXFP4;
         const int wpc = wpc_env > 0 ? wpc_env : bt == 512 || (tb == 1 && !codebook) ? 1 : 2;
         size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * wpc);
         if (wgs_env > 0) wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)wgs_env);
@@ -1108,15 +1111,17 @@ inline std::string engine_self_check() {
           wq[b * 32 + i] = q;
         }
       }
-    } else if (type == GGML_Q4_0) {
+    } else if (type == GGML_Q4_0 || type == GGML_IQ4_NL || type == GGML_MXFP4) {
+      static const int fp4[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+      const int hb = type == GGML_MXFP4 ? 1 : 2;  // bytes of a block's scale: E8M0 128 = 2^0, or f16 1.0
       for (int b = 0; b < 8; ++b) {
-        uint8_t* p = blk + 18 * b;
-        p[0] = 0x00; p[1] = 0x3C;  // f16 1.0
+        uint8_t* p = blk + (16 + hb) * b;
+        if (hb == 1) { p[0] = 128; } else { p[0] = 0x00; p[1] = 0x3C; }
         for (int i = 0; i < 16; ++i) {
           const int lo = (int)(next() & 15u), hi = (int)(next() & 15u);
-          p[2 + i] = (uint8_t)(lo | hi << 4);
-          wq[b * 32 + i] = lo - 8;
-          wq[b * 32 + 16 + i] = hi - 8;
+          p[hb + i] = (uint8_t)(lo | hi << 4);
+          wq[b * 32 + i] = type == GGML_Q4_0 ? lo - 8 : type == GGML_IQ4_NL ? iq4[lo] : fp4[lo];
+          wq[b * 32 + 16 + i] = type == GGML_Q4_0 ? hi - 8 : type == GGML_IQ4_NL ? iq4[hi] : fp4[hi];
         }
       }
     } else if (type == GGML_Q4_K || type == GGML_Q5_K) {
@@ -1178,7 +1183,7 @@ inline std::string engine_self_check() {
     cl_mem c0 = e.buf((size_t)M * N * 4), c1 = e.buf((size_t)M * N * 4);
     std::vector<float> y0((size_t)M * N), y1((size_t)M * N), cinit((size_t)M * N);
     for (auto& v : cinit) v = (float)((int)(next() % 9u) - 4);  // small integers: sums with them stay exact
-    for (uint32_t type : {GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ4_XS, GGML_Q4_0}) {
+    for (uint32_t type : {GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ4_XS, GGML_Q4_0, GGML_IQ4_NL, GGML_MXFP4}) {
       const size_t rb = arcz_gguf_bytes(type, 1, K), sbb = rb / (size_t)(K / 256);
       std::vector<uint8_t> w((size_t)N * rb);
       std::vector<int> wq((size_t)N * K);

@@ -17,8 +17,10 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 #define QT_Q4_K 12
 #define QT_Q5_K 13
 #define QT_Q6_K 14
+#define QT_IQ4_NL 20
 #define QT_IQ3_S 21
 #define QT_IQ4_XS 23
+#define QT_MXFP4 39
 
 // ---- device weight layout ("raw planes").  A matrix of R rows x K columns (K % 256 == 0, nsb = K / 256) is held
 // as separate planes, each row-major over (row, superblock), so that every field is 16-byte aligned and a wave's
@@ -41,6 +43,10 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 //   Q4_0 : qs  [R][nsb][128]  (the sixteen nibble bytes of each of the superblock's eight 32-value blocks, as GGUF: byte
 //                              j of block b = element 32b+j low nibble, 32b+16+j high nibble; value = nibble - 8),
 //          d   [R][nsb][8] (f16: the eight blocks' scales).  144 bytes per 256 values, as GGUF's eight 18-byte blocks.
+//   IQ4_NL: as Q4_0; value = the nibble's entry of the IQ4_XS table.
+//   MXFP4: qs  [R][nsb][128]  (as Q4_0; a nibble is an E2M1 code: sign | 3 bits naming 0, 1, 2, 3, 4, 6, 8, 12, the
+//                              doubled magnitudes), e [R][nsb][8] (the eight blocks' E8M0 scale bytes: value =
+//                              2^(e - 128) * the table's entry).  136 bytes per 256 values, as GGUF's eight 17-byte blocks.
 //   IQ3_S: qs  [R][nsb][64]   (the low bytes of the 64 codebook indices: 8 per 32-value block, each naming 4 magnitudes),
 //          sg  [R][nsb][32]   (sign bits: 4 bytes per block, bit e of the block's 32 = element e is negative),
 //          hd  [R][nsb][12]   (8 bytes of ninth index bits, bit g of byte b = index g of block b; 4 bytes of scale nibbles,
@@ -54,6 +60,7 @@ struct PlanesQ80 { size_t qs, d; };
 struct PlanesIQ4XS { size_t qs, hdr; };
 struct PlanesQ40 { size_t qs, d; };
 struct PlanesIQ3S { size_t qs, sg, hd, d; };
+struct PlanesMXFP4 { size_t qs, e; };
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 __host__ __device__ inline PlanesQ4K planes_q4k(size_t rows, int nsb) {
@@ -90,6 +97,12 @@ __host__ __device__ inline PlanesQ40 planes_q40(size_t rows, int nsb) {
   p.d = rows * (size_t)nsb * 128;
   return p;
 }
+__host__ __device__ inline PlanesMXFP4 planes_mxfp4(size_t rows, int nsb) {
+  PlanesMXFP4 p;
+  p.qs = 0;
+  p.e = rows * (size_t)nsb * 128;
+  return p;
+}
 __host__ __device__ inline PlanesIQ3S planes_iq3s(size_t rows, int nsb) {
   PlanesIQ3S p;
   const size_t u = rows * (size_t)nsb;
@@ -102,7 +115,8 @@ __host__ __device__ inline PlanesIQ3S planes_iq3s(size_t rows, int nsb) {
 __host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb) {
   const size_t u = rows * (size_t)nsb;
   if (qt == QT_IQ3_S) return align16(u * 110);
-  if (qt == QT_Q4_0) return u * 144;
+  if (qt == QT_Q4_0 || qt == QT_IQ4_NL) return u * 144;
+  if (qt == QT_MXFP4) return align16(u * 136);
   if (qt == QT_Q4_K) return u * 144;
   if (qt == QT_Q5_K) return u * 176;
   if (qt == QT_Q6_K) return align16(u * 208 + u * 2);
@@ -152,6 +166,41 @@ __device__ inline uint32_t iq4_lookup(uint32_t c) {
 // Q4_0: four nibbles, one in the low nibble of each byte of c (the other bits ignored), to the four int8 values
 // nibble - 8, without borrows between bytes.
 __device__ inline uint32_t q40_vals(uint32_t c) { return (((c & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
+
+// MXFP4: four E2M1 codes, one in the low nibble of each byte of c, to the four int8 values of the format's table of
+// doubled magnitudes (0 1 2 3 4 6 8 12, bit 3 = negative; reference src/quants.h:497): one byte permute for the
+// magnitudes, then a byte is negated as (x ^ 0xFF) + 1 -- no carry leaves a byte, a negated 0 being 0x00 + 0x100's
+// low byte only when x = 0, where the carry is masked off below.
+__device__ inline uint32_t mxfp4_lookup(uint32_t c) {
+  const uint32_t mag = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, c & 0x07070707u);
+  const uint32_t neg = (c >> 3) & 0x01010101u;                 // 1 in every byte to negate
+  const uint32_t nz = ((mag + 0x7F7F7F7Fu) >> 7) & 0x01010101u;  // 1 in every byte whose magnitude is not 0
+  const uint32_t m = neg & nz;
+  return (mag ^ (m * 0xFFu)) + m;
+}
+
+// The types whose block is 16 bytes of nibbles and one scale (Q4_0, IQ4_NL, MXFP4) share every kernel path: the nibbles'
+// values by the type's rule, the scale an f16 (Q4_0, IQ4_NL) or an E8M0 byte (MXFP4).
+__host__ __device__ constexpr bool qt_nib16(int qt) { return qt == QT_Q4_0 || qt == QT_IQ4_NL || qt == QT_MXFP4; }
+template <int QT>
+__device__ inline uint32_t nib_vals(uint32_t c) {
+  if constexpr (QT == QT_IQ4_NL) return iq4_lookup(c);
+  else if constexpr (QT == QT_MXFP4) return mxfp4_lookup(c);
+  else return q40_vals(c);
+}
+// (the scale plane lies where Q4_0's does, behind the nibbles: planes_q40(rows, nsb).d; an entry is 2 bytes or 1)
+#define NIB16_SCALE_BYTES(QT) ((QT) == QT_MXFP4 ? 1 : 2)
+// 2^(e - 128) of an E8M0 scale byte (e = 0, 1: the f32 subnormals 2^-128, 2^-127; reference src/quants.h:498-503)
+__device__ inline float e8m0_half(uint32_t e) {
+  e &= 0xFFu;
+  return __builtin_bit_cast(float, e < 2 ? 0x00200000u << e : (e - 1) << 23);
+}
+// scale of block `blk` (counted over the whole plane) of a nibble type
+template <int QT>
+__device__ inline float nib16_scale(const uint8_t* plane, size_t blk) {
+  if constexpr (QT == QT_MXFP4) return e8m0_half(plane[blk]);
+  else return f16_bits_to_f32(*(const unsigned short*)(plane + blk * 2));
+}
 
 // IQ3_S: four magnitudes (bytes of a codebook entry g) with the four sign bits s4 (bit j: byte j is negative) applied:
 // the bits are spread to the bytes' low bits by one multiply, and a byte is negated as (x ^ 0xFF) + 1 -- no carry

@@ -186,9 +186,9 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
         }
       }
     }
-  } else if constexpr (QT == QT_Q4_0) {
+  } else if constexpr (qt_nib16(QT)) {
     const PlanesQ40 pl = planes_q40(plane_rows, nsb);
-    const int ib = hl & 7;  // a unit is one 32-block: low nibbles = its elements 0..15, high = 16..31, value = nibble - 8
+    const int ib = hl & 7;  // a unit is one 32-block: low nibbles = its elements 0..15, high = 16..31, value by the type's rule (nibble - 8, or a table entry)
     for (int u = hl; u < units; u += 32) {
       const int sb = u >> 3;
       const int e1 = sb * 256 + 32 * ib;
@@ -206,18 +206,18 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
         const size_t n = rows[r];
         const uint8_t* rb = r < SPLIT ? raw : raw2;
         const uint4 w = *(const uint4*)(rb + pl.qs + n * nsb * 128 + (size_t)u * 16);
-        const float d = f16_bits_to_f32(*(const unsigned short*)(rb + pl.d + (n * nsb * 8 + u) * 2));
+        const float d = nib16_scale<QT>(rb + pl.d, n * nsb * 8 + u);
         const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int t = 0; t < TB; ++t) if (t < nt) {
-          int i1 = dot4(q40_vals(ww[0]), a1[t].x, 0);
-          i1 = dot4(q40_vals(ww[1]), a1[t].y, i1);
-          i1 = dot4(q40_vals(ww[2]), a1[t].z, i1);
-          i1 = dot4(q40_vals(ww[3]), a1[t].w, i1);
-          i1 = dot4(q40_vals(ww[0] >> 4), a2[t].x, i1);
-          i1 = dot4(q40_vals(ww[1] >> 4), a2[t].y, i1);
-          i1 = dot4(q40_vals(ww[2] >> 4), a2[t].z, i1);
-          i1 = dot4(q40_vals(ww[3] >> 4), a2[t].w, i1);
+          int i1 = dot4(nib_vals<QT>(ww[0]), a1[t].x, 0);
+          i1 = dot4(nib_vals<QT>(ww[1]), a1[t].y, i1);
+          i1 = dot4(nib_vals<QT>(ww[2]), a1[t].z, i1);
+          i1 = dot4(nib_vals<QT>(ww[3]), a1[t].w, i1);
+          i1 = dot4(nib_vals<QT>(ww[0] >> 4), a2[t].x, i1);
+          i1 = dot4(nib_vals<QT>(ww[1] >> 4), a2[t].y, i1);
+          i1 = dot4(nib_vals<QT>(ww[2] >> 4), a2[t].z, i1);
+          i1 = dot4(nib_vals<QT>(ww[3] >> 4), a2[t].w, i1);
           acc[r][t] += sa[t] * d * (float)i1;   // (the 32-block in one conversion, as the reference's gemv: decode.cl:1003)
         }
       }
@@ -366,6 +366,8 @@ GEMV_ALL(13)
 GEMV_ALL(14)
 GEMV_ALL(23)
 GEMV_ALL(2)
+GEMV_ALL(20)
+GEMV_ALL(39)
 GEMV_ALL(21)
 
 // ---- the experts of a pass of a few tokens (the reference's per-tile kernels moe_gateup_q / moe_down_q,
@@ -649,6 +651,8 @@ MOE_DECODE_FUSED_INST(13)
 MOE_DECODE_FUSED_INST(14)
 MOE_DECODE_FUSED_INST(23)
 MOE_DECODE_FUSED_INST(2)
+MOE_DECODE_FUSED_INST(20)
+MOE_DECODE_FUSED_INST(39)
 MOE_DECODE_FUSED_INST(21)
 
 #define MOE_DECODE_INST(QT, TM)                                                                                      \
@@ -671,6 +675,8 @@ MOE_DECODE_ALL(13)
 MOE_DECODE_ALL(14)
 MOE_DECODE_ALL(23)
 MOE_DECODE_ALL(2)
+MOE_DECODE_ALL(20)
+MOE_DECODE_ALL(39)
 MOE_DECODE_ALL(21)
 
 // expand_iq3s: the IQ3_S planes of `rows` rows to Q6_K planes of the same rows, value for value -- the same f16 d, the

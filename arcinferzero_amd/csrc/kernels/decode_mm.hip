@@ -56,6 +56,8 @@ template <> struct MmT<QT_Q5_K> { enum { SB = 22, QB = 128, D = 4, XB = 32, MIN 
 template <> struct MmT<QT_Q6_K> { enum { SB = 20, QB = 128, D = 4, XB = 64, MIN = 0, DPL = 1 }; };
 template <> struct MmT<QT_Q8_0> { enum { SB = 24, QB = 256, D = 4, XB = 0, MIN = 0, DPL = 0 }; };
 template <> struct MmT<QT_Q4_0> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 0, DPL = 0 }; };
+template <> struct MmT<QT_IQ4_NL> : MmT<QT_Q4_0> {};
+template <> struct MmT<QT_MXFP4> : MmT<QT_Q4_0> {};
 template <> struct MmT<QT_IQ4_XS> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 0, DPL = 0 }; };
 // (IQ3_S: the main plane is the 8 index bytes per block, the second the sign bits, the header the ninth bits and scale
 //  nibbles, 12 bytes; the codebook, 2 KiB, sits behind the groups' sums in LDS)
@@ -79,10 +81,10 @@ template <int QT> struct MmL {
 template <int QT> struct MmQ { mm_u4 r[MmT<QT>::QB / 64]; };  // the lane's 16-byte pieces of a superblock of 16 rows
 template <int QT> struct MmX { mm_u4 r[MmT<QT>::XB / 16 > 0 ? MmT<QT>::XB / 16 : 1]; uint32_t d; };  // of four superblocks' second plane
 // a superblock as the products take it: the lane's 8 bytes of each 32-byte chunk of the main plane, the header
-// (Q4_0 and IQ4_XS: of each 16-byte block)
+// (Q4_0, IQ4_NL, MXFP4 and IQ4_XS: of each 16-byte block)
 // (IQ3_S: c[b].x the lane's two index bytes of block b, sg the row's eight words of sign bits)
 template <int QT> struct MmSb {
-  mm_u2 c[QT == QT_Q4_0 || QT == QT_IQ4_XS || QT == QT_IQ3_S ? 8 : MmT<QT>::QB / 32];
+  mm_u2 c[qt_nib16(QT) || QT == QT_IQ4_XS || QT == QT_IQ3_S ? 8 : MmT<QT>::QB / 32];
   mm_u4 h;
   mm_u2 x[2];
   uint32_t d;
@@ -99,8 +101,8 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   using LL = MmL<QT>;
   constexpr int QB = TT::QB, NQ = QB / 64, D = TT::D, LPRW = QB / 16, RPI = 64 / LPRW;
   constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
-  constexpr bool B16 = QT == QT_Q4_0 || QT == QT_IQ4_XS;  // a block is 16 bytes: low nibbles values 0..15, high 16..31
-  constexpr int HB = QT == QT_IQ4_XS ? 8 : QT == QT_IQ3_S ? 12 : 16;  // bytes of a row's superblock in the header plane
+  constexpr bool B16 = qt_nib16(QT) || QT == QT_IQ4_XS;  // a block is 16 bytes: low nibbles values 0..15, high 16..31
+  constexpr int HB = QT == QT_IQ4_XS || QT == QT_MXFP4 ? 8 : QT == QT_IQ3_S ? 12 : 16;  // bytes of a row's superblock in the header plane
   constexpr bool I3 = QT == QT_IQ3_S;
   const int tid = threadIdx.x, lane = tid & 63, n16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (a scalar: what follows from it is scalar arithmetic)
@@ -123,8 +125,8 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     o_hdr = pl.sc; o_x = pl.qh; o_d = pl.d;
   } else if constexpr (QT == QT_Q8_0) {
     o_hdr = planes_q80((size_t)N, nsb).d;
-  } else if constexpr (QT == QT_Q4_0) {
-    o_hdr = planes_q40((size_t)N, nsb).d;
+  } else if constexpr (qt_nib16(QT)) {
+    o_hdr = planes_q40((size_t)N, nsb).d;  // (MXFP4: its scale bytes, at the same place)
   } else if constexpr (I3) {
     const PlanesIQ3S pl = planes_iq3s((size_t)N, nsb);
     o_hdr = pl.hd; o_x = pl.sg; o_d = pl.d;
@@ -387,7 +389,8 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
         acc[3] = fmaf((float)I[3], sa4[b].w * d, acc[3]);
       }
     } else if constexpr (B16) {
-      // block b is the 16 bytes 16 b .. of the row's 128; Q4_0: value nibble - 8, f16 scale entry b of the header;
+      // block b is the 16 bytes 16 b .. of the row's 128; Q4_0: value nibble - 8, f16 scale entry b of the header (IQ4_NL:
+      // the table's value; MXFP4: its table's, and a scale byte);
       // IQ4_XS: the table's value of the nibble, d in the header's first half word and a 6-bit scale - 32 per block (low
       // four bits in the second word, high two in the upper half of the first)
       const int sh = 4 * (g >> 1);
@@ -397,9 +400,13 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
         const mm_u2 cw = h.c[b];
         uint32_t w0, w1;
         float d;
-        if constexpr (QT == QT_Q4_0) {
-          w0 = q40_vals(cw.x >> sh);
-          w1 = q40_vals(cw.y >> sh);
+        if constexpr (QT == QT_MXFP4) {  // (the header: the eight blocks' scale bytes)
+          w0 = mxfp4_lookup(cw.x >> sh);
+          w1 = mxfp4_lookup(cw.y >> sh);
+          d = e8m0_half((b < 4 ? h.h.x : h.h.y) >> (8 * (b & 3)));
+        } else if constexpr (qt_nib16(QT)) {
+          w0 = nib_vals<QT>(cw.x >> sh);
+          w1 = nib_vals<QT>(cw.y >> sh);
           const uint32_t dw = b < 2 ? h.h.x : b < 4 ? h.h.y : b < 6 ? h.h.z : h.h.w;
           d = f16_bits_to_f32((b & 1) ? dw >> 16 : dw);
         } else {
@@ -597,6 +604,8 @@ MM_KERNEL(13)
 MM_KERNEL(14)
 MM_KERNEL(8)
 MM_KERNEL(2)
+MM_KERNEL(20)
+MM_KERNEL(39)
 MM_KERNEL(23)
 MM_KERNEL(21)
 

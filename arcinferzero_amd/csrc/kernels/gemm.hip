@@ -111,7 +111,7 @@ __device__ __forceinline__ void step_load(StepRegs<QT>& r, const Gemm2Lds& L, co
     const uint2 h = *(const uint2*)(raw + pl.hdr + ((row_base + n) * nsb + s) * 8);
     r.h.x = h.x;
     r.h.y = h.y;
-  } else if constexpr (QT == QT_Q4_0) {
+  } else if constexpr (qt_nib16(QT)) {
     const PlanesQ40 pl = planes_q40(rows_total, nsb);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -120,8 +120,11 @@ __device__ __forceinline__ void step_load(StepRegs<QT>& r, const Gemm2Lds& L, co
       r.w[i] = *(const g2_u4*)(raw + pl.qs + ((row_base + n) * nsb + s) * 128 + 64 * hh + 16 * c);
     }
     const int n = min(n0 + (t >> 1), N - 1);
-    // (the f16 scales of blocks 4 hh + 2 (t & 1) and the next)
-    r.h.x = *(const uint32_t*)(raw + pl.d + (((row_base + n) * nsb + s) * 8 + 4 * hh + 2 * (t & 1)) * 2);
+    // (the scales of blocks 4 hh + 2 (t & 1) and the next: two f16, or -- MXFP4 -- two bytes)
+    if constexpr (QT == QT_MXFP4)
+      r.h.x = *(const unsigned short*)(raw + pl.d + ((row_base + n) * nsb + s) * 8 + 4 * hh + 2 * (t & 1));
+    else
+      r.h.x = *(const uint32_t*)(raw + pl.d + (((row_base + n) * nsb + s) * 8 + 4 * hh + 2 * (t & 1)) * 2);
   } else {
     const PlanesQ80 pl = planes_q80(rows_total, nsb);
 #pragma unroll
@@ -200,17 +203,22 @@ __device__ __forceinline__ void step_store(const StepRegs<QT>& r, Gemm2Lds& L, i
       const int ls = (int)(((r.h.y >> (4 * ib)) & 0xFu) | ((((r.h.x >> 16) >> (2 * ib)) & 3u) << 4)) - 32;
       L.ws[2 * p + k][row] = d * (float)ls;
     }
-  } else if constexpr (QT == QT_Q4_0) {
+  } else if constexpr (qt_nib16(QT)) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {  // block 4 hh + c of the superblock: 16 bytes -> its 32 values, nibble - 8
+    for (int i = 0; i < 2; ++i) {  // block 4 hh + c of the superblock: 16 bytes -> its 32 values (nibble - 8, or the table's)
       const int id = t + 256 * i, row = id >> 2, c = id & 3;
       const g2_u4 w = r.w[i];
-      *(uint4*)&L.wq[row][32 * c] = make_uint4(q40_vals(w.x), q40_vals(w.y), q40_vals(w.z), q40_vals(w.w));
-      *(uint4*)&L.wq[row][32 * c + 16] = make_uint4(q40_vals(w.x >> 4), q40_vals(w.y >> 4), q40_vals(w.z >> 4), q40_vals(w.w >> 4));
+      *(uint4*)&L.wq[row][32 * c] = make_uint4(nib_vals<QT>(w.x), nib_vals<QT>(w.y), nib_vals<QT>(w.z), nib_vals<QT>(w.w));
+      *(uint4*)&L.wq[row][32 * c + 16] = make_uint4(nib_vals<QT>(w.x >> 4), nib_vals<QT>(w.y >> 4), nib_vals<QT>(w.z >> 4), nib_vals<QT>(w.w >> 4));
     }
     const int row = t >> 1, p = t & 1;
-    L.ws[2 * p][row] = f16_bits_to_f32(r.h.x);
-    L.ws[2 * p + 1][row] = f16_bits_to_f32(r.h.x >> 16);
+    if constexpr (QT == QT_MXFP4) {
+      L.ws[2 * p][row] = e8m0_half(r.h.x);
+      L.ws[2 * p + 1][row] = e8m0_half(r.h.x >> 8);
+    } else {
+      L.ws[2 * p][row] = f16_bits_to_f32(r.h.x);
+      L.ws[2 * p + 1][row] = f16_bits_to_f32(r.h.x >> 16);
+    }
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1920,6 +1928,11 @@ GEMM2_TILES_INST(23)
 // Q4_0: the same body (nibbles to values as they are stored to LDS, a block's f16 scale as Q8_0's)
 GEMM2_INST(2)
 GEMM2_TILES_INST(2)
+// IQ4_NL, MXFP4: Q4_0's path with the nibbles through the types' tables (MXFP4: a block's scale from its E8M0 byte)
+GEMM2_INST(20)
+GEMM2_TILES_INST(20)
+GEMM2_INST(39)
+GEMM2_TILES_INST(39)
 // Q4_K -DBM=64: 64 tokens x 256 rows per work-group (grid ceil(N / 256) * ceil(M / 64) work-groups), K from 0
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
@@ -2039,6 +2052,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_B
   }
 GEMM2_SPLITK_INST(23)
 GEMM2_SPLITK_INST(2)
+GEMM2_SPLITK_INST(20)
+GEMM2_SPLITK_INST(39)
 // (Q5_K: the DMA-staged body, as Q4_K)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE13_ACT321_BM128_BN128_SPLITK1(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,

@@ -17,6 +17,8 @@
  *   orc_act_residual                    PARITY UNPINNED (no reference CPU twin, no vector); identities and bounds only
  *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
  *   IQ4_XS decode                       closed-form block; live comparison with the compiled reference header
+ *   IQ4_NL, MXFP4 decode                closed-form blocks (every code, every E8M0 exponent); live comparison with the
+ *                                       compiled reference header
  *   IQ3_S decode (and its grid table)   closed-form block; golden vectors (tests/golden/ref_vectors_types2.npz) and live
  *                                       comparison with the compiled reference header over every grid index
  *   Q5_K decode                         closed-form block; golden vectors (tests/golden/ref_vectors_q5k.npz) and live
@@ -42,7 +44,11 @@
 #define ORC_Q4_0 2u
 #define ORC_Q8_0 8u
 /* Q4_0 is Q8_0 with q - 8 in four bits (src/quants.h:136): everything after the decode treats the two alike */
-#define ORC_Q8LIKE(t) ((t) == ORC_Q8_0 || (t) == ORC_Q4_0)
+/* IQ4_NL and MXFP4 are Q4_0 with a table of 16 values in the place of q - 8 (and MXFP4 a power-of-two scale byte in the
+ * place of the f16 one): src/quants.h:520-530, 594-606 */
+#define ORC_IQ4_NL 20u
+#define ORC_MXFP4 39u
+#define ORC_Q8LIKE(t) ((t) == ORC_Q8_0 || (t) == ORC_Q4_0 || (t) == ORC_IQ4_NL || (t) == ORC_MXFP4)
 #define ORC_Q4_K 12u
 #define ORC_Q5_K 13u
 #define ORC_Q45(t) ((t) == ORC_Q4_K || (t) == ORC_Q5_K) /* d, dmin, 6-bit scales and mins */
@@ -109,6 +115,8 @@ int orc_sb_bytes(uint32_t type) {
   switch (type) {
     case ORC_Q8_0: return 34 * 8;
     case ORC_Q4_0: return 18 * 8;
+    case ORC_IQ4_NL: return 18 * 8;
+    case ORC_MXFP4: return 17 * 8;
     case ORC_Q4_K: return 144;
     case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
@@ -253,6 +261,33 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
       const uint8_t* blk = p + 34 * b;
       o->d8[b] = orc_fp16_to_f32(rd16(blk));
       for (int i = 0; i < 32; ++i) o->q[32 * b + i] = (int8_t)blk[2 + i];
+    }
+    return 0;
+  }
+  if (type == ORC_IQ4_NL) { /* 8 blocks of 18 bytes: f16 d, low nibbles = elements 0..15, high = 16..31, each a code of
+                               the IQ4 table (src/quants.h:594-606) */
+    for (int b = 0; b < 8; ++b) {
+      const uint8_t* blk = p + 18 * b;
+      o->d8[b] = orc_fp16_to_f32(rd16(blk));
+      for (int i = 0; i < 16; ++i) {
+        o->q[32 * b + i] = iq4_values[blk[2 + i] & 0xF];
+        o->q[32 * b + 16 + i] = iq4_values[blk[2 + i] >> 4];
+      }
+    }
+    return 0;
+  }
+  if (type == ORC_MXFP4) { /* 8 blocks of 17 bytes: E8M0 scale byte e, then the nibbles as above, each an E2M1 code whose
+                              doubled value is in the table; value = 2^(e - 128) * table[code] (src/quants.h:495-503,
+                              520-530; e = 0 and 1 give the f32 subnormals 2^-128 and 2^-127) */
+    static const int8_t mxfp4_values[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+    for (int b = 0; b < 8; ++b) {
+      const uint8_t* blk = p + 17 * b;
+      const uint32_t bits = blk[0] < 2 ? 0x00200000u << blk[0] : (uint32_t)(blk[0] - 1) << 23;
+      memcpy(&o->d8[b], &bits, 4);
+      for (int i = 0; i < 16; ++i) {
+        o->q[32 * b + i] = mxfp4_values[blk[1 + i] & 0xF];
+        o->q[32 * b + 16 + i] = mxfp4_values[blk[1 + i] >> 4];
+      }
     }
     return 0;
   }

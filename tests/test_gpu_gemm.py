@@ -150,7 +150,7 @@ def test_startup_self_check(rt):
     az.self_check()
 
 
-@pytest.mark.parametrize("qtype", [az.Q4_K, az.Q6_K, az.Q8_0, az.Q4_0])
+@pytest.mark.parametrize("qtype", [az.Q4_K, az.Q6_K, az.Q8_0, az.Q4_0, az.IQ4_NL, az.MXFP4])
 @pytest.mark.parametrize("T,Mp,N,K", [(1, 16, 264, 1024), (5, 16, 136, 512), (100, 112, 272, 768), (64, 64, 130, 4096)])
 def test_per_256_activation_scales(eng, qtype, T, Mp, N, K):
     """act32 = 0: one activation scale per superblock (the reference's quant_store16 with act32 = 0, zero/kernels/ops.cl:

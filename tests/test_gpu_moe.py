@@ -83,6 +83,9 @@ def test_routing_and_sort(rt, NE, NU, T, tm):
                                                    (az.Q4_K, 8, 2, 256, 768, 3, 16), (az.Q4_K, 128, 8, 2048, 768, 8, 16),
                                                    (az.Q8_0, 4, 2, 256, 512, 1, 16), (az.Q6_K, 6, 3, 512, 256, 5, 16),
                                                    (az.Q5_K, 8, 2, 512, 256, 7, 16), (az.IQ4_XS, 4, 2, 256, 512, 4, 16),
+                                                   # IQ4_NL and MXFP4 experts: small passes and tile passes
+                                                   (az.IQ4_NL, 4, 2, 256, 512, 1, 16), (az.IQ4_NL, 4, 2, 256, 512, 150, 160),
+                                                   (az.MXFP4, 4, 2, 256, 512, 4, 16), (az.MXFP4, 6, 2, 512, 256, 40, 48),
                                                    # IQ3_S experts (uploaded as Q6_K planes): one token and a tile pass
                                                    (az.IQ3_S, 4, 2, 256, 512, 1, 16), (az.IQ3_S, 6, 2, 512, 256, 40, 48),
                                                    # 9-16 tokens: still the matrix-vector form, the routing kernel's waves

@@ -99,7 +99,12 @@ def test_repack_planes_layout(qtype):
         sb = W.reshape(u, 136)
         assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 8:]) and np.array_equal(P[u * 128:u * 136].reshape(u, 8), sb[:, :8])
         assert not P[u * 136:].any() and P.size % 16 == 0
-    elif qtype == az.Q4_0:
+    elif qtype == az.MXFP4:
+        blk = W.reshape(u, 8, 17)                                            # eight 17-byte blocks: E8M0 byte, 16 nibble bytes
+        assert P.size == (W.size + 15) // 16 * 16
+        assert np.array_equal(P[:u * 128].reshape(u, 8, 16), blk[:, :, 1:]) and np.array_equal(P[u * 128:u * 136].reshape(u, 8), blk[:, :, 0])
+        assert not P[u * 136:].any()
+    elif qtype in (az.Q4_0, az.IQ4_NL):
         blk = W.reshape(u, 8, 18)                                            # eight 18-byte blocks: f16 d, 16 nibble bytes
         assert P.size == W.size == u * 144
         assert np.array_equal(P[:u * 128].reshape(u, 8, 16), blk[:, :, 2:]) and np.array_equal(P[u * 128:].reshape(u, 8, 2), blk[:, :, :2])
@@ -121,7 +126,8 @@ def test_q8_0_quantizer_is_the_reference_one():
     assert np.array_equal(az.quantize_rows(az.Q8_0, w), orc.quantize_rows_q8_0(w))
 
 
-@pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q5_K, 0.04), (az.Q6_K, 0.02), (az.Q8_0, 0.006), (az.IQ4_XS, 0.09)])
+@pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q5_K, 0.04), (az.Q6_K, 0.02), (az.Q8_0, 0.006), (az.IQ4_XS, 0.09),
+                                       (az.IQ4_NL, 0.10), (az.MXFP4, 0.15)])
 def test_block_makers_make_valid_close_blocks(qtype, rel):
     """The Q4_K / Q5_K / Q6_K block makers are input generators (the reference has none): valid fields and a round-trip
     error of the size the bit width allows."""

@@ -323,6 +323,76 @@ def test_q40_vs_compiled_reference():
     assert np.array_equal((qs * dd).reshape(16, 512), orc.dequant_rows(az.Q4_0, a, 16, 512))
 
 
+def _e8m0_half(e):
+    """2^(e - 128) in f32, e = 0 and 1 being subnormals (src/quants.h:498-503)."""
+    return np.float32(np.ldexp(1.0, int(e) - 128))
+
+
+def test_iq4_nl_and_mxfp4_closed_form():
+    """IQ4_NL (src/quants.h:594-606): f16 d times the nibble's entry of the IQ4 table; MXFP4 (src/quants.h:495-503,
+    520-530): 2^(e - 128) times the doubled E2M1 magnitude of the nibble.  Blocks made by hand with every code in both
+    nibble positions, power-of-two and zero scales, and every E8M0 exponent (0 and 1: f32 subnormals; 255: 2^127)."""
+    from common import IQ4_VALUES, MXFP4_VALUES
+    K = 256
+    blk = np.zeros((8, 18), np.uint8)
+    exp = np.zeros(K, np.float32)
+    for b in range(8):
+        d = [0.0, 0.25, -0.5, 2.0, 1.0, -1.0, 0.0078125, 4.0][b]
+        blk[b, 0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+        for i in range(16):
+            c0, c1 = (i + b) % 16, (5 * i + 3 * b + 1) % 16
+            blk[b, 2 + i] = c0 | (c1 << 4)
+            exp[32 * b + i] = np.float32(d) * np.float32(IQ4_VALUES[c0])
+            exp[32 * b + 16 + i] = np.float32(d) * np.float32(IQ4_VALUES[c1])
+    assert np.array_equal(orc.dequant_rows(az.IQ4_NL, blk.reshape(-1), 1, K)[0], exp)
+    # MXFP4: all 256 exponents over 32 superblocks, every code in both positions
+    K = 256 * 32
+    blk = np.zeros((256, 17), np.uint8)
+    exp = np.zeros(K, np.float32)
+    for b in range(256):
+        blk[b, 0] = b
+        for i in range(16):
+            c0, c1 = (i + b) % 16, (7 * i + b + 3) % 16
+            blk[b, 1 + i] = c0 | (c1 << 4)
+            with np.errstate(over="ignore"):             # (e = 255: 2^127 times 4 and more is inf, in the oracle too)
+                exp[32 * b + i] = _e8m0_half(b) * np.float32(MXFP4_VALUES[c0])
+                exp[32 * b + 16 + i] = _e8m0_half(b) * np.float32(MXFP4_VALUES[c1])
+    got = orc.dequant_rows(az.MXFP4, blk.reshape(-1), 1, K)[0]
+    assert np.array_equal(got.view(np.uint32) & 0x7FFFFFFF, exp.view(np.uint32) & 0x7FFFFFFF)   # (-0.0 from the codes 8)
+    assert np.array_equal(got, exp)
+    # the integer fields the dot products see, and one scale per 32-block
+    q, isc, imn, d, dmin = orc.decode_row_fields(az.MXFP4, blk[:8].reshape(-1), 256)
+    assert np.array_equal(isc, np.ones(16)) and not imn.any() and not dmin.any()
+    assert np.array_equal(d, [_e8m0_half(b) for b in range(8)])
+    assert np.array_equal(q.reshape(8, 32)[:, :16], MXFP4_VALUES[blk[:8, 1:] & 15])
+
+
+@pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
+@pytest.mark.parametrize("qtype", [az.IQ4_NL, az.MXFP4])
+def test_iq4_nl_and_mxfp4_vs_compiled_reference(qtype):
+    """The oracle's decode of generated blocks and of blocks of random bytes (IQ4_NL: finite f16 scales) against the
+    compiled reference header's dequant_row, bit for bit; and the device planes against the reference's own GPU form
+    of a superblock (src/quants.h gpu_raw_sb: the eight scales, then the eight blocks' nibble bytes)."""
+    N, K = 16, 512
+    nsb, hb = K // 256, 1 if qtype == az.MXFP4 else 2
+    W = az.gen_weights(qtype, 7, N, K, 0.02)
+    R = np.random.default_rng(9).integers(0, 256, size=W.size, dtype=np.uint8)
+    if qtype == az.IQ4_NL:
+        R.reshape(-1, 18)[:, 1] &= 0x7B
+    for blocks in (W, R):
+        a, b = orc.dequant_rows(qtype, blocks, N, K), orc.dequant_rows(qtype, blocks, N, K, lib=orc.ref)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    planes = az.repack_planes(qtype, N, K, W)
+    u = N * nsb
+    rsb = int(orc.ref.ref_raw_padded_sb_bytes(qtype))
+    assert rsb == 128 + 8 * hb
+    raw = np.zeros(rsb, np.uint8)
+    for i in range(u):
+        orc.ref.ref_gpu_raw_sb(qtype, orc.ptr(W[i * (16 + hb) * 8:]), orc.ptr(raw))
+        assert np.array_equal(raw[:8 * hb], planes[u * 128 + i * 8 * hb:u * 128 + (i + 1) * 8 * hb])
+        assert np.array_equal(raw[8 * hb:], planes[i * 128:(i + 1) * 128])
+
+
 # ---------------------------------------------------------------- quantizers
 def test_quantize_act_golden():
     for a32 in (1, 0):
