@@ -168,15 +168,14 @@ __device__ inline uint32_t iq4_lookup(uint32_t c) {
 __device__ inline uint32_t q40_vals(uint32_t c) { return (((c & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
 
 // MXFP4: four E2M1 codes, one in the low nibble of each byte of c, to the four int8 values of the format's table of
-// doubled magnitudes (0 1 2 3 4 6 8 12, bit 3 = negative; reference src/quants.h:497): one byte permute for the
-// magnitudes, then a byte is negated as (x ^ 0xFF) + 1 -- no carry leaves a byte, a negated 0 being 0x00 + 0x100's
-// low byte only when x = 0, where the carry is masked off below.
+// doubled values (0 1 2 3 4 6 8 12 | 0 -1 -2 -3 -4 -6 -8 -12; reference src/quants.h:497): a byte permute per table
+// half, the code's bit 3 picks between them (as iq4_lookup).
 __device__ inline uint32_t mxfp4_lookup(uint32_t c) {
-  const uint32_t mag = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, c & 0x07070707u);
-  const uint32_t neg = (c >> 3) & 0x01010101u;                 // 1 in every byte to negate
-  const uint32_t nz = ((mag + 0x7F7F7F7Fu) >> 7) & 0x01010101u;  // 1 in every byte whose magnitude is not 0
-  const uint32_t m = neg & nz;
-  return (mag ^ (m * 0xFFu)) + m;
+  const uint32_t sel = c & 0x07070707u;
+  const uint32_t lo = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);  // codes 0-7
+  const uint32_t hi = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);  // codes 8-15
+  const uint32_t m = ((c >> 3) & 0x01010101u) * 0xFFu;
+  return (hi & m) | (lo & ~m);
 }
 
 // The types whose block is 16 bytes of nibbles and one scale (Q4_0, IQ4_NL, MXFP4) share every kernel path: the nibbles'
