@@ -1,5 +1,5 @@
 // "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0,
-// Q4_0, IQ4_XS, IQ3_S).
+// Q4_0, IQ4_NL, MXFP4, IQ4_XS, IQ3_S).
 //
 // From a handful of tokens on, the dot-product GEMVs are bound by their vector ALU work (eight v_dot4 per token and
 // 16-byte unit), not by memory, and past eight tokens the engine had only the prefill GEMM with its 64-token tiles.
@@ -9,7 +9,7 @@
 //   res += (sa[t][b] * (d[n] * sc[n][b])) * (float)I[t][n][b]  -  (sa[t][b] * (float)S[t][b]) * (dmin[n] * mn[n][b])
 // with S the sum of the block's 32 int8 activations, for Q6_K (two int8 sub-scales per block, :457-464, 485)
 //   res += d[n] * sa[t][b] * (float)(sc0[n][b] * I0[t][n][b] + sc1[n][b] * I1[t][n][b])
-// and for Q8_0 (:445-447), Q4_0 and IQ4_XS (one scale per block)  res += (sa[t][b] * d[n][b]) * (float)I[t][n][b].  The
+// and for Q8_0 (:445-447), Q4_0, IQ4_NL, MXFP4 and IQ4_XS (one scale per block)  res += (sa[t][b] * d[n][b]) * (float)I[t][n][b].  The
 // weights are read once, as in the GEMVs.
 //
 // Tokens.  A work-group of 8 waves stages superblocks [s_begin, s_end) of the tokens in LDS -- int8 rows, and per block

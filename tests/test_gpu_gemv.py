@@ -108,7 +108,8 @@ def test_gemv_accumulate_and_offset(eng):
 
 
 @pytest.mark.parametrize("qtype,F,K", [(az.Q4_K, 17408, 5120), (az.Q4_K, 264, 512), (az.Q6_K, 1024, 2048), (az.Q8_0, 512, 1024),
-                                       (az.Q5_K, 776, 2560), (az.IQ4_XS, 128, 17408)])
+                                       (az.Q5_K, 776, 2560), (az.IQ4_XS, 128, 17408), (az.Q4_0, 520, 1024), (az.IQ3_S, 264, 2048),
+                                       (az.IQ4_NL, 1032, 1536), (az.MXFP4, 136, 5120)])
 def test_gemv_gu_equals_two_launches(eng, qtype, F, K):
     """Gate and up of one token in one launch (zero/engine.h:1124-1146): rows [0, F) of gate, then of up at C + F, bit
     for bit what the two launches give; and the cases that are not taken."""
@@ -146,7 +147,8 @@ def test_gemv_gu_equals_two_launches(eng, qtype, F, K):
 
 
 @pytest.mark.parametrize("qtype,N,K,T", [(az.Q6_K, 1000, 512, 1), (az.Q4_K, 264, 512, 3), (az.Q8_0, 300, 17408, 2),
-                                         (az.Q6_K, 520, 17408, 5), (az.Q4_K, 264, 1024, 8)])
+                                         (az.Q6_K, 520, 17408, 5), (az.Q4_K, 264, 1024, 8), (az.IQ4_NL, 300, 768, 2),
+                                         (az.MXFP4, 264, 17408, 4), (az.Q4_0, 100, 512, 1), (az.IQ3_S, 200, 1024, 6)])
 def test_gemv_softcap_output_head(eng, qtype, N, K, T):
     """The output head's soft cap (the reference's -DSOFTCAP=c, zero/kernels/decode.cl:882-886, 1029-1031): the GEMVs
     write c * tanh(v / c), then add C when accumulating.  LDS-staged and global-memory kernels, 1-8 tokens."""

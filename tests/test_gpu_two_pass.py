@@ -9,7 +9,7 @@ import pytest
 
 import arcinferzero_amd as az
 import oracle_lib as orc
-from common import TYPES, TYPE_NAMES, make_acts, make_weights, pad_rows, rel_err_rows
+from common import ALL_TYPES, TYPES, TYPE_NAMES, make_acts, make_weights, pad_rows, rel_err_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -67,7 +67,7 @@ def test_fused_producers_residual(eng, T, Mp, K):
 
 
 @pytest.mark.parametrize("T,Mp", [(1, 16), (2, 16), (5, 16), (100, 112)])
-@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_matmul_two_pass(eng, qtype, T, Mp):
     N, K = 320, 2048
     print(f"two-pass matmul {TYPE_NAMES[qtype]} T={T} Mp={Mp} N={N} K={K}", flush=True)
