@@ -9,7 +9,7 @@ import os
 
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ3_S, IQ4_XS, MXFP4 = 2, 8, 12, 13, 14, 20, 21, 23, 39  # GGUF type ids
+Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ3_S, IQ4_XS, MXFP4 = 2, 8, 11, 12, 13, 14, 20, 21, 23, 39  # GGUF type ids
 
 lib_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libarcz_hip.so")
 if not os.path.exists(lib_path):

@@ -14,6 +14,7 @@
 #define GGML_TYPE_Q4_0 2u  // (GGUF type id, src/gguf.h:19)
 #define GGML_TYPE_IQ3_S 21u  // (src/gguf.h:22)
 #define GGML_TYPE_IQ4_NL 20u  // (src/gguf.h:21)
+#define GGML_TYPE_Q3_K 11u  // (src/gguf.h:20)
 #define GGML_TYPE_MXFP4 39u  // (src/gguf.h:23)
 
 namespace {
@@ -118,7 +119,7 @@ extern "C" {
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
   return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : type == GGML_TYPE_IQ3_S ? u * 110
-         : type == GGML_TYPE_IQ4_NL ? u * 144 : type == GGML_TYPE_MXFP4 ? u * 136 : 0;
+         : type == GGML_TYPE_IQ4_NL ? u * 144 : type == GGML_TYPE_MXFP4 ? u * 136 : type == GGML_TYPE_Q3_K ? u * 110 : 0;
 }
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) { return raw_planes_bytes((int)type, rows, K / 256); }
 // The IQ3_S codebook as the kernels take it: 512 words, byte j of a word = magnitude j of the entry (1, 3, ..., 15).
@@ -171,6 +172,27 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
         }
         memcpy(dst + pl.qh + i * 32, H, 32);
       }
+    }
+    return 0;
+  }
+  if (type == GGML_TYPE_Q3_K) {
+    // 110 bytes per superblock (hmask[32], qs[64], sixteen 6-bit scales in 12 bytes, f16 d; reference
+    // src/quants.h:465-494) written out as Q6_K planes, value for value: q6 = (q3 - 4) + 32, int8 sub-scale =
+    // scale - 32, the same d
+    const PlanesQ6K pl = planes_q6k(rows, nsb);
+    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_Q6_K, rows, nsb) - (pl.d + u * 2));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i) {
+      const uint8_t *p = src + i * 110, *hm = p, *qs = p + 32, *sc = p + 96;
+      int q[256];
+      for (int b = 0; b < 8; ++b)
+        for (int e = 0; e < 32; ++e)
+          q[32 * b + e] = ((qs[32 * (b / 4) + e] >> (2 * (b % 4))) & 3) + (((hm[e] >> b) & 1) ? 4 : 0) - 4 + 32;
+      q6k_pack(q, dst + pl.ql + i * 128, dst + pl.qh + i * 64);
+      for (int k = 0; k < 16; ++k)
+        dst[pl.sc + i * 16 + k] =
+            (uint8_t)(int8_t)((int)(((sc[k & 7] >> (4 * (k >> 3))) & 0xF) | (((sc[8 + (k & 3)] >> (2 * (k >> 2))) & 3) << 4)) - 32);
+      memcpy(dst + pl.d + i * 2, p + 108, 2);
     }
     return 0;
   }
@@ -535,6 +557,42 @@ static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) 
   }
 }
 
+// f32 rows -> GGUF Q3_K superblocks (110 bytes per 256 values; reference src/quants.h:465-494): per 16 values a step
+// (the value of largest magnitude) / -4, which that value then decodes to exactly; d = the largest |step| / 31 (fp16),
+// the 6-bit scale round(step / d) + 32; each value the nearest of -4..3 steps.  An input generator for tests.
+static void arcz_quantize_q3_k(const float* src, size_t N, int K, uint8_t* out) {
+  const int64_t nsbt = (int64_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < nsbt; ++s) {
+    const float* v = src + s * 256;
+    uint8_t* p = out + s * 110;
+    memset(p, 0, 110);
+    float step[16], smax = 0;
+    for (int b = 0; b < 16; ++b) {
+      float amax = 0, mx = 0;
+      for (int i = 0; i < 16; ++i)
+        if (std::fabs(v[16 * b + i]) > amax) { amax = std::fabs(v[16 * b + i]); mx = v[16 * b + i]; }
+      step[b] = mx / -4.0f;
+      smax = std::fmax(smax, std::fabs(step[b]));
+    }
+    const uint16_t dh = f32_to_f16(smax / 31.0f);
+    const float d = f16_to_f32(dh);
+    memcpy(p + 108, &dh, 2);
+    for (int b = 0; b < 16; ++b) {
+      const int sc = d > 0 ? std::min(31, std::max(-32, (int)std::lrintf(step[b] / d))) : 0, s6 = sc + 32;
+      p[96 + (b & 7)] |= (uint8_t)((s6 & 0xF) << (4 * (b >> 3)));
+      p[104 + (b & 3)] |= (uint8_t)((s6 >> 4) << (2 * (b >> 2)));
+      const float sd = d * (float)sc, inv = sd != 0 ? 1.0f / sd : 0.0f;
+      for (int i = 0; i < 16; ++i) {
+        const int e = 16 * b + i, blk = e >> 5, el = e & 31;
+        const int q = std::min(3, std::max(-4, (int)std::lrintf(v[e] * inv))) + 4;  // 0..7
+        p[32 + 32 * (blk / 4) + el] |= (uint8_t)((q & 3) << (2 * (blk % 4)));
+        if (q & 4) p[el] |= (uint8_t)(1u << blk);
+      }
+    }
+  }
+}
+
 // f32 rows -> GGUF IQ4_NL blocks (18 bytes per 32 values; reference src/quants.h:594-606): d = (the value of largest
 // magnitude) / -127, which that value then decodes to exactly; every value takes the nearest entry of the table.  An
 // input generator for tests: no search over scales as a real quantizer would make.
@@ -598,7 +656,7 @@ static void arcz_quantize_mxfp4(const float* src, size_t N, int K, uint8_t* out)
   }
 }
 
-// Quantizes f32 rows to `type` (2, 8, 12, 13, 14, 20, 21, 23, 39).  0 or -1.
+// Quantizes f32 rows to `type` (2, 8, 11, 12, 13, 14, 20, 21, 23, 39).  0 or -1.
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
   if (K <= 0 || K % 256) return -1;
   if (type == GGML_TYPE_Q4_0) arcz_quantize_q4_0(src, N, K, out);
@@ -608,6 +666,7 @@ int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t
   else if (type == QT_Q6_K) arcz_quantize_q6_k(src, N, K, out);
   else if (type == QT_IQ4_XS) arcz_quantize_iq4_xs(src, N, K, out);
   else if (type == GGML_TYPE_IQ3_S) arcz_quantize_iq3_s(src, N, K, out);
+  else if (type == GGML_TYPE_Q3_K) arcz_quantize_q3_k(src, N, K, out);
   else if (type == GGML_TYPE_IQ4_NL) arcz_quantize_iq4_nl(src, N, K, out);
   else if (type == GGML_TYPE_MXFP4) arcz_quantize_mxfp4(src, N, K, out);
   else return -1;

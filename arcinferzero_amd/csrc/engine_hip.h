@@ -23,6 +23,7 @@
 #define GGML_Q6_K 14u
 #define GGML_IQ4_XS 23u
 #define GGML_IQ4_NL 20u
+#define GGML_Q3_K 11u
 #define GGML_MXFP4 39u
 
 extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
@@ -212,7 +213,7 @@ class Engine {
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
     if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS &&
-        type != GGML_IQ3_S && type != GGML_IQ4_NL && type != GGML_MXFP4)
+        type != GGML_IQ3_S && type != GGML_IQ4_NL && type != GGML_MXFP4 && type != GGML_Q3_K)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
     if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))
@@ -230,6 +231,7 @@ class Engine {
     std::vector<uint8_t> planes(pb);
     if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
     w.raw = buf(pb, planes.data());
+    if (type == GGML_Q3_K) w.type = GGML_Q6_K;  // (written out as Q6_K planes, value for value: a Q6_K matrix from here on)
     if ((type == GGML_Q4_K || type == GGML_Q5_K) && rows == (size_t)N) {  // (room for its rows' scale vectors, gemm_dense)
       // (with per-256 activation scales also d, an f32 per superblock and row: half a byte more per block and row)
       const size_t need = (size_t)N * (K / 32) * 21 + 4096;  // (4 + 4 bytes a block and row, or 4 + 16: the bf16 pieces)

@@ -14,6 +14,7 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 // GGUF type ids (reference src/gguf.h:18-22)
 #define QT_Q4_0 2
 #define QT_Q8_0 8
+#define QT_Q3_K 11
 #define QT_Q4_K 12
 #define QT_Q5_K 13
 #define QT_Q6_K 14
@@ -43,6 +44,9 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 //   Q4_0 : qs  [R][nsb][128]  (the sixteen nibble bytes of each of the superblock's eight 32-value blocks, as GGUF: byte
 //                              j of block b = element 32b+j low nibble, 32b+16+j high nibble; value = nibble - 8),
 //          d   [R][nsb][8] (f16: the eight blocks' scales).  144 bytes per 256 values, as GGUF's eight 18-byte blocks.
+//   Q3_K : no planes of its own: a matrix of this type is written out as Q6_K planes when it is uploaded, value for
+//          value (the 3-bit value - 4 as q - 32 in six bits, the 6-bit scale - 32 as the int8 sub-scale, the same f16
+//          d), and every kernel sees a Q6_K matrix: 210 bytes per 256 values on the device for GGUF's 110.
 //   IQ4_NL: as Q4_0; value = the nibble's entry of the IQ4_XS table.
 //   MXFP4: qs  [R][nsb][128]  (as Q4_0; a nibble is an E2M1 code: sign | 3 bits naming 0, 1, 2, 3, 4, 6, 8, 12, the
 //                              doubled magnitudes), e [R][nsb][8] (the eight blocks' E8M0 scale bytes: value =
@@ -119,7 +123,7 @@ __host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb)
   if (qt == QT_MXFP4) return align16(u * 136);
   if (qt == QT_Q4_K) return u * 144;
   if (qt == QT_Q5_K) return u * 176;
-  if (qt == QT_Q6_K) return align16(u * 208 + u * 2);
+  if (qt == QT_Q6_K || qt == QT_Q3_K) return align16(u * 208 + u * 2);
   if (qt == QT_Q8_0) return u * 272;
   if (qt == QT_IQ4_XS) return align16(u * 136);
   return 0;

@@ -17,6 +17,7 @@
  *   orc_act_residual                    PARITY UNPINNED (no reference CPU twin, no vector); identities and bounds only
  *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
  *   IQ4_XS decode                       closed-form block; live comparison with the compiled reference header
+ *   Q3_K decode                         closed-form block; live comparison with the compiled reference header
  *   IQ4_NL, MXFP4 decode                closed-form blocks (every code, every E8M0 exponent); live comparison with the
  *                                       compiled reference header
  *   IQ3_S decode (and its grid table)   closed-form block; golden vectors (tests/golden/ref_vectors_types2.npz) and live
@@ -56,7 +57,8 @@
 #define ORC_IQ4_XS 23u
 /* one int scale per 16 (Q6_K) or per 32 values (IQ4_XS: the same one for both halves), kept in sc6[], and no mins */
 #define ORC_IQ3_S 21u
-#define ORC_IQLIKE(t) ((t) == ORC_IQ4_XS || (t) == ORC_IQ3_S) /* q[] holds the signed value itself */
+#define ORC_Q3_K 11u /* 3-bit values - 4 with a 6-bit scale - 32 per 16 of them: q[] and sc6[] as the IQ types' */
+#define ORC_IQLIKE(t) ((t) == ORC_IQ4_XS || (t) == ORC_IQ3_S || (t) == ORC_Q3_K) /* q[] holds the signed value itself */
 #define ORC_Q6LIKE(t) ((t) == ORC_Q6_K || ORC_IQLIKE(t))
 
 /* ---------------------------------------------------------------- fp16 (src/quants.h:17-52) */
@@ -122,6 +124,7 @@ int orc_sb_bytes(uint32_t type) {
     case ORC_Q6_K: return 210;
     case ORC_IQ4_XS: return 136;
     case ORC_IQ3_S: return 110;
+    case ORC_Q3_K: return 110;
     default: return 0;
   }
 }
@@ -262,6 +265,20 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
       o->d8[b] = orc_fp16_to_f32(rd16(blk));
       for (int i = 0; i < 32; ++i) o->q[32 * b + i] = (int8_t)blk[2 + i];
     }
+    return 0;
+  }
+  if (type == ORC_Q3_K) { /* 110 bytes: hmask[32] (bit b of byte e: the third bit of element e of 32-block b), qs[64]
+                             (two bits of element e of block b: byte 32 (b / 4) + e, bits 2 (b % 4)), 12 bytes of sixteen
+                             6-bit scales (scale i: low nibble i / 8 of byte i % 8, top two bits: bits 2 (i / 4) of byte
+                             8 + i % 4), f16 d; value = d * (scale - 32) * (q - 4), q the three bits
+                             (src/quants.h:465-494) */
+    const uint8_t *hm = p, *qs = p + 32, *sc = p + 96;
+    o->d = orc_fp16_to_f32(rd16(p + 108));
+    for (int i = 0; i < 16; ++i)
+      o->sc6[i] = (int)(((sc[i & 7] >> (4 * (i >> 3))) & 0xF) | (((sc[8 + (i & 3)] >> (2 * (i >> 2))) & 3) << 4)) - 32;
+    for (int b = 0; b < 8; ++b)
+      for (int e = 0; e < 32; ++e)
+        o->q[32 * b + e] = (int16_t)(((qs[32 * (b / 4) + e] >> (2 * (b % 4))) & 3) + (((hm[e] >> b) & 1) ? 4 : 0) - 4);
     return 0;
   }
   if (type == ORC_IQ4_NL) { /* 8 blocks of 18 bytes: f16 d, low nibbles = elements 0..15, high = 16..31, each a code of

@@ -8,14 +8,14 @@ import oracle_lib as orc
 import os
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS, Q4_0, IQ3_S = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K, az.IQ4_XS, az.Q4_0, az.IQ3_S
-IQ4_NL, MXFP4 = az.IQ4_NL, az.MXFP4
+IQ4_NL, MXFP4, Q3_K = az.IQ4_NL, az.MXFP4, az.Q3_K
 TYPES = (Q8_0, Q4_K, Q6_K, Q5_K, IQ4_XS)
-ALL_TYPES = TYPES + (Q4_0, IQ3_S, IQ4_NL, MXFP4)     # with the types the golden files of the first five do not cover
+ALL_TYPES = TYPES + (Q4_0, IQ3_S, IQ4_NL, MXFP4, Q3_K)     # with the types the golden files of the first five do not cover
 # the IQ3_S codebook as the compiled reference decodes it (a golden vector): 512 entries of four magnitudes
 IQ3S_GRID = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors_types2.npz"))[
     "iq3s_grid_dequant"].reshape(512, 4).astype(np.int64)
 TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS", az.IQ3_S: "IQ3_S", az.Q4_0: "Q4_0",
-              az.IQ4_NL: "IQ4_NL", az.MXFP4: "MXFP4"}
+              az.IQ4_NL: "IQ4_NL", az.MXFP4: "MXFP4", az.Q3_K: "Q3_K"}
 IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64)
 MXFP4_VALUES = np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.int64)   # (src/quants.h:497)
 
@@ -98,6 +98,17 @@ def unit_scale_weights(qtype, N, K, seed):
         blk[..., 0:2] = one
         blk[..., 2:] = (q[..., :16] | (q[..., 16:] << 4)).astype(np.uint8)
         return blk.reshape(-1), (q - 8).reshape(N, K)
+    if qtype == Q3_K:
+        # d = 1, every 6-bit scale 33 (- 32 = 1): low nibbles 1, high two bits 2; values = the three bits - 4
+        q = rng.integers(0, 8, size=(N, nsb, 8, 32), dtype=np.int64)               # [block][element]
+        blk = np.zeros((N, nsb, 110), np.uint8)
+        blk[..., 96:104] = 0x11
+        blk[..., 104:108] = 0xAA
+        blk[..., 108:110] = one
+        for b in range(8):
+            blk[..., 32 + 32 * (b // 4):64 + 32 * (b // 4)] |= ((q[..., b, :] & 3) << (2 * (b % 4))).astype(np.uint8)
+            blk[..., 0:32] |= ((q[..., b, :] >> 2) << b).astype(np.uint8)
+        return blk.reshape(-1), (q - 4).reshape(N, K)
     if qtype == IQ4_NL:
         c = rng.integers(0, 16, size=(N, nsb * 8, 32), dtype=np.int64)
         blk = np.zeros((N, nsb * 8, 18), np.uint8)

@@ -109,7 +109,7 @@ def test_gemv_accumulate_and_offset(eng):
 
 @pytest.mark.parametrize("qtype,F,K", [(az.Q4_K, 17408, 5120), (az.Q4_K, 264, 512), (az.Q6_K, 1024, 2048), (az.Q8_0, 512, 1024),
                                        (az.Q5_K, 776, 2560), (az.IQ4_XS, 128, 17408), (az.Q4_0, 520, 1024), (az.IQ3_S, 264, 2048),
-                                       (az.IQ4_NL, 1032, 1536), (az.MXFP4, 136, 5120)])
+                                       (az.IQ4_NL, 1032, 1536), (az.MXFP4, 136, 5120), (az.Q3_K, 264, 1024)])
 def test_gemv_gu_equals_two_launches(eng, qtype, F, K):
     """Gate and up of one token in one launch (zero/engine.h:1124-1146): rows [0, F) of gate, then of up at C + F, bit
     for bit what the two launches give; and the cases that are not taken."""

@@ -99,6 +99,13 @@ def test_repack_planes_layout(qtype):
         sb = W.reshape(u, 136)
         assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 8:]) and np.array_equal(P[u * 128:u * 136].reshape(u, 8), sb[:, :8])
         assert not P[u * 136:].any() and P.size % 16 == 0
+    elif qtype == az.Q3_K:
+        # written out as Q6_K planes, value for value: put back together as Q6_K rows, they decode to the same floats
+        assert P.size == az.planes_bytes(az.Q6_K, rows, K) and az.gguf_bytes(qtype, rows, K) == u * 110
+        g6 = np.concatenate([P[:u * 128].reshape(u, 128), P[u * 128:u * 192].reshape(u, 64), P[u * 192:u * 208].reshape(u, 16),
+                             P[u * 208:u * 210].reshape(u, 2)], axis=1).reshape(-1)
+        assert np.array_equal(orc.dequant_rows(az.Q6_K, g6, rows, K).view(np.uint32), orc.dequant_rows(qtype, W, rows, K).view(np.uint32))
+        assert not P[u * 210:].any()
     elif qtype == az.MXFP4:
         blk = W.reshape(u, 8, 17)                                            # eight 17-byte blocks: E8M0 byte, 16 nibble bytes
         assert P.size == (W.size + 15) // 16 * 16
@@ -127,7 +134,7 @@ def test_q8_0_quantizer_is_the_reference_one():
 
 
 @pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q5_K, 0.04), (az.Q6_K, 0.02), (az.Q8_0, 0.006), (az.IQ4_XS, 0.09),
-                                       (az.IQ4_NL, 0.10), (az.MXFP4, 0.15)])
+                                       (az.IQ4_NL, 0.10), (az.MXFP4, 0.15), (az.Q3_K, 0.25)])
 def test_block_makers_make_valid_close_blocks(qtype, rel):
     """The Q4_K / Q5_K / Q6_K block makers are input generators (the reference has none): valid fields and a round-trip
     error of the size the bit width allows."""

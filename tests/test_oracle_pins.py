@@ -367,6 +367,39 @@ def test_iq4_nl_and_mxfp4_closed_form():
     assert np.array_equal(q.reshape(8, 32)[:, :16], MXFP4_VALUES[blk[:8, 1:] & 15])
 
 
+def test_q3_k_closed_form():
+    """Q3_K (src/quants.h:465-494): a superblock made by hand -- every 3-bit value in every block, sixteen different
+    6-bit scales on both sides of 32, d a power of two -- decodes to d * (scale - 32) * (q - 4)."""
+    K = 256
+    blk = np.zeros(110, np.uint8)
+    blk[108:110] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    sc = [(7 * i + 3) % 64 for i in range(16)]
+    for i, s6 in enumerate(sc):
+        blk[96 + (i & 7)] |= (s6 & 0xF) << (4 * (i >> 3))
+        blk[104 + (i & 3)] |= (s6 >> 4) << (2 * (i >> 2))
+    exp = np.zeros(K, np.float32)
+    for b in range(8):
+        for e in range(32):
+            q = (3 * e + 5 * b + 1) % 8
+            blk[32 + 32 * (b // 4) + e] |= (q & 3) << (2 * (b % 4))
+            blk[e] |= (q >> 2) << b
+            exp[32 * b + e] = np.float32(0.5) * np.float32(sc[2 * b + e // 16] - 32) * np.float32(q - 4)
+    assert np.array_equal(orc.dequant_rows(az.Q3_K, blk, 1, K)[0], exp)
+    q, isc, imn, d, dmin = orc.decode_row_fields(az.Q3_K, blk, K)
+    assert np.array_equal(isc, np.array(sc) - 32) and not imn.any() and q.min() == -4 and q.max() == 3
+
+
+@pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
+def test_q3_k_vs_compiled_reference():
+    N, K = 16, 512
+    W = az.gen_weights(az.Q3_K, 7, N, K, 0.02)
+    R = np.random.default_rng(9).integers(0, 256, size=W.size, dtype=np.uint8)
+    R.reshape(-1, 110)[:, 109] &= 0x7B                      # finite f16 d
+    for blocks in (W, R):
+        a, b = orc.dequant_rows(az.Q3_K, blocks, N, K), orc.dequant_rows(az.Q3_K, blocks, N, K, lib=orc.ref)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 @pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
 @pytest.mark.parametrize("qtype", [az.IQ4_NL, az.MXFP4])
 def test_iq4_nl_and_mxfp4_vs_compiled_reference(qtype):
