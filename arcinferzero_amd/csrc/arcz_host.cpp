@@ -176,22 +176,33 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
     return 0;
   }
   if (type == GGML_TYPE_Q3_K) {
-    // 110 bytes per superblock (hmask[32], qs[64], sixteen 6-bit scales in 12 bytes, f16 d; reference
-    // src/quants.h:465-494) written out as Q6_K planes, value for value: q6 = (q3 - 4) + 32, int8 sub-scale =
-    // scale - 32, the same d
-    const PlanesQ6K pl = planes_q6k(rows, nsb);
-    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_Q6_K, rows, nsb) - (pl.d + u * 2));
+    // 110 bytes per superblock (hmask[32]: bit b of byte e = the third bit of element e of block b; qs[64]: byte
+    // 32 (b / 4) + e, bits 2 (b % 4): its low two; sixteen 6-bit scales in 12 bytes; f16 d -- reference
+    // src/quants.h:465-494) -> a block's bits together: two words of bit pairs, a word of third bits, a 12-bit entry of
+    // its two scales (layout: kernels/common.h)
+    const PlanesIQ3S pl = planes_iq3s(rows, nsb);
+    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_Q3_K, rows, nsb) - (pl.d + u * 2));
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < u; ++i) {
       const uint8_t *p = src + i * 110, *hm = p, *qs = p + 32, *sc = p + 96;
-      int q[256];
-      for (int b = 0; b < 8; ++b)
-        for (int e = 0; e < 32; ++e)
-          q[32 * b + e] = ((qs[32 * (b / 4) + e] >> (2 * (b % 4))) & 3) + (((hm[e] >> b) & 1) ? 4 : 0) - 4 + 32;
-      q6k_pack(q, dst + pl.ql + i * 128, dst + pl.qh + i * 64);
-      for (int k = 0; k < 16; ++k)
-        dst[pl.sc + i * 16 + k] =
-            (uint8_t)(int8_t)((int)(((sc[k & 7] >> (4 * (k >> 3))) & 0xF) | (((sc[8 + (k & 3)] >> (2 * (k >> 2))) & 3) << 4)) - 32);
+      for (int b = 0; b < 8; ++b) {
+        uint32_t D[2] = {0, 0}, H = 0;
+        for (int j = 0; j < 32; ++j) {
+          const uint32_t q2 = (qs[32 * (b / 4) + j] >> (2 * (b % 4))) & 3u, hb = (hm[j] >> b) & 1u;
+          D[j >> 4] |= q2 << (8 * (j & 3) + 2 * ((j & 15) >> 2));
+          H |= hb << (8 * (j & 3) + (j >> 2));
+        }
+        memcpy(dst + pl.qs + i * 64 + b * 8, D, 8);
+        memcpy(dst + pl.sg + i * 32 + b * 4, &H, 4);
+      }
+      uint8_t hd[12] = {0};
+      for (int k = 0; k < 16; ++k) {  // scale k: 6 bits at bit 6 k of the 96
+        const uint32_t s6 = ((sc[k & 7] >> (4 * (k >> 3))) & 0xFu) | (((sc[8 + (k & 3)] >> (2 * (k >> 2))) & 3u) << 4);
+        const int bit = 6 * k;
+        hd[bit >> 3] |= (uint8_t)(s6 << (bit & 7));
+        if ((bit & 7) > 2) hd[(bit >> 3) + 1] |= (uint8_t)(s6 >> (8 - (bit & 7)));
+      }
+      memcpy(dst + pl.hd + i * 12, hd, 12);
       memcpy(dst + pl.d + i * 2, p + 108, 2);
     }
     return 0;

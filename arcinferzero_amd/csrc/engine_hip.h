@@ -43,7 +43,7 @@ struct GpuWeight {
 
 inline const char* ggml_type_name(uint32_t t) {
   return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : t == GGML_IQ4_XS ? "IQ4_XS"
-         : t == GGML_Q4_0 ? "Q4_0" : t == GGML_IQ3_S ? "IQ3_S" : t == GGML_IQ4_NL ? "IQ4_NL" : t == GGML_MXFP4 ? "MXFP4" : "?";
+         : t == GGML_Q4_0 ? "Q4_0" : t == GGML_IQ3_S ? "IQ3_S" : t == GGML_IQ4_NL ? "IQ4_NL" : t == GGML_MXFP4 ? "MXFP4" : t == GGML_Q3_K ? "Q3_K" : "?";
 }
 
 class Engine {
@@ -75,18 +75,19 @@ class Engine {
     tabs_ = buf(sizeof grid, grid);
   }
   cl_mem tabs_ = nullptr;
-  // IQ3_S in the GEMM forms (prefill chunks, expert tiles): the matrix is first written out as Q6_K planes, value for
+  // IQ3_S and Q3_K in the GEMM forms (prefill chunks, expert tiles): the matrix is first written out as Q6_K planes, value for
   // value, into xw_ -- the place of the reference's decode pass in front of its GEMM (zero/engine.h:1205-1250) -- and
   // the Q6_K kernels run on that.  xw_ is sized when such a weight is uploaded (the largest one), never in a matmul.
   cl_mem xw_ = nullptr;
   size_t xw_bytes_ = 0;
   GpuWeight gemm_form(const char* name, const GpuWeight& w) {
-    if (w.type != GGML_IQ3_S) return w;
+    if (w.type != GGML_IQ3_S && w.type != GGML_Q3_K) return w;
     const size_t need = raw_planes_bytes(QT_Q6_K, w.rows, w.K / 256);
     if (need > xw_bytes_) throw std::logic_error("gemm_form: the expansion buffer is smaller than the weight");
-    cl_kernel k = kernel("decode", "", "expand_iq3s");
+    cl_kernel k = kernel("decode", "", w.type == GGML_Q3_K ? "expand_q3k" : "expand_iq3s");
     int rows = (int)w.rows, nsb = w.K / 256;
-    set_args(k, 0, w.raw, xw_, tabs_, rows, nsb);
+    if (w.type == GGML_Q3_K) set_args(k, 0, w.raw, xw_, rows, nsb);
+    else set_args(k, 0, w.raw, xw_, tabs_, rows, nsb);
     size_t g1 = ((size_t)rows * nsb + 15) / 16 * 256, l1 = 256;
     run(name, k, 1, &g1, &l1);
     GpuWeight x = w;
@@ -231,7 +232,6 @@ class Engine {
     std::vector<uint8_t> planes(pb);
     if (arcz_repack_planes(type, rows, K, data, planes.data()) != 0) throw std::runtime_error("make_weight: repack failed");
     w.raw = buf(pb, planes.data());
-    if (type == GGML_Q3_K) w.type = GGML_Q6_K;  // (written out as Q6_K planes, value for value: a Q6_K matrix from here on)
     if ((type == GGML_Q4_K || type == GGML_Q5_K) && rows == (size_t)N) {  // (room for its rows' scale vectors, gemm_dense)
       // (with per-256 activation scales also d, an f32 per superblock and row: half a byte more per block and row)
       const size_t need = (size_t)N * (K / 32) * 21 + 4096;  // (4 + 4 bytes a block and row, or 4 + 16: the bf16 pieces)
@@ -243,7 +243,7 @@ class Engine {
         wsv_bytes_ = need;
       }
     }
-    if (type == GGML_IQ3_S) {  // (room for its GEMM form)
+    if (type == GGML_IQ3_S || type == GGML_Q3_K) {  // (room for its GEMM form)
       const size_t need = raw_planes_bytes(QT_Q6_K, rows, K / 256);
       if (need > xw_bytes_) {
         if (xw_) release(xw_);
@@ -1036,7 +1036,8 @@ class Engine {
     // 64-slot tiles as well -- else 128
     bool t64 = false;
     for (int i = 0; i < 3; ++i)
-      t64 = t64 || L.ex[i].type == GGML_Q4_K || L.ex[i].type == GGML_Q5_K || L.ex[i].type == GGML_Q6_K || L.ex[i].type == GGML_IQ3_S;
+      t64 = t64 || L.ex[i].type == GGML_Q4_K || L.ex[i].type == GGML_Q5_K || L.ex[i].type == GGML_Q6_K || L.ex[i].type == GGML_IQ3_S ||
+            L.ex[i].type == GGML_Q3_K;
     const int tm = t64 ? 64 : 128;
     moe_route(L, rl, ldl, T, tm);
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)

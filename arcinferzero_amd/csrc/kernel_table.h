@@ -55,6 +55,7 @@ static const KernelSpec kKernelTable[] = {
     {"decode", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", "GROWS", "TM", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "moe_down_q", nullptr, "piipppipppp", {"QT", "GROWS", "TM", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "expand_iq3s", nullptr, "pppii", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"decode", "expand_q3k", nullptr, "ppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"decode", "gemv_v", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt_v", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     // ---- gemm

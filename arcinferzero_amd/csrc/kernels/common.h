@@ -44,9 +44,15 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 //   Q4_0 : qs  [R][nsb][128]  (the sixteen nibble bytes of each of the superblock's eight 32-value blocks, as GGUF: byte
 //                              j of block b = element 32b+j low nibble, 32b+16+j high nibble; value = nibble - 8),
 //          d   [R][nsb][8] (f16: the eight blocks' scales).  144 bytes per 256 values, as GGUF's eight 18-byte blocks.
-//   Q3_K : no planes of its own: a matrix of this type is written out as Q6_K planes when it is uploaded, value for
-//          value (the 3-bit value - 4 as q - 32 in six bits, the 6-bit scale - 32 as the int8 sub-scale, the same f16
-//          d), and every kernel sees a Q6_K matrix: 210 bytes per 256 values on the device for GGUF's 110.
+//   Q3_K : the planes of IQ3_S in size and place (planes_iq3s), regrouped from GGUF's hmask / qs / scales so that a
+//          32-value block's bits lie together and four values come out of a word with a shift and a mask:
+//          qs  [R][nsb][64]   (block b: words D0, D1 at bytes 8 b: value j of the block's first / second 16 in byte
+//                              j % 4, bits 2 (j / 4) and the next: its low two bits),
+//          sg  [R][nsb][32]   (block b: the word of third bits, value j (0..31) at bit 8 (j % 4) + j / 4),
+//          hd  [R][nsb][12]   (eight 12-bit entries, entry b at bit 12 b: the 6-bit scales of the block's first and
+//                              second 16 values, s | s' << 6, 32 not yet subtracted),
+//          d   [R][nsb]       (f16).  110 bytes per 256 values, as GGUF (src/quants.h:465-494).
+//          value = d * (scale - 32) * (the three bits - 4).
 //   IQ4_NL: as Q4_0; value = the nibble's entry of the IQ4_XS table.
 //   MXFP4: qs  [R][nsb][128]  (as Q4_0; a nibble is an E2M1 code: sign | 3 bits naming 0, 1, 2, 3, 4, 6, 8, 12, the
 //                              doubled magnitudes), e [R][nsb][8] (the eight blocks' E8M0 scale bytes: value =
@@ -118,12 +124,12 @@ __host__ __device__ inline PlanesIQ3S planes_iq3s(size_t rows, int nsb) {
 }
 __host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb) {
   const size_t u = rows * (size_t)nsb;
-  if (qt == QT_IQ3_S) return align16(u * 110);
+  if (qt == QT_IQ3_S || qt == QT_Q3_K) return align16(u * 110);
   if (qt == QT_Q4_0 || qt == QT_IQ4_NL) return u * 144;
   if (qt == QT_MXFP4) return align16(u * 136);
   if (qt == QT_Q4_K) return u * 144;
   if (qt == QT_Q5_K) return u * 176;
-  if (qt == QT_Q6_K || qt == QT_Q3_K) return align16(u * 208 + u * 2);
+  if (qt == QT_Q6_K) return align16(u * 208 + u * 2);
   if (qt == QT_Q8_0) return u * 272;
   if (qt == QT_IQ4_XS) return align16(u * 136);
   return 0;
@@ -170,6 +176,20 @@ __device__ inline uint32_t iq4_lookup(uint32_t c) {
 // Q4_0: four nibbles, one in the low nibble of each byte of c (the other bits ignored), to the four int8 values
 // nibble - 8, without borrows between bytes.
 __device__ inline uint32_t q40_vals(uint32_t c) { return (((c & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
+
+// Q3_K (device form): the four int8 values 4 k .. 4 k + 3 (k = 0..7) of a 32-value block from its words of low bits
+// (D = D0 for k < 4, D1 above) and third bits H: the three bits - 4, no borrow between bytes.
+__device__ inline uint32_t q3k_vals(uint32_t D, uint32_t H, int k) {
+  const uint32_t v = ((D >> (2 * (k & 3))) & 0x03030303u) | (((H >> k) & 0x01010101u) << 2);
+  return ((v | 0x80808080u) - 0x04040404u) ^ 0x80808080u;
+}
+// ... and the block's two scales - 32 from the header's three words (entry b at bit 12 b of the 96)
+__device__ inline void q3k_scales(uint32_t s0, uint32_t s1, uint32_t s2, int b, int& sc0, int& sc1) {
+  int a0, a1, m0, m1;
+  q4k_scales_pair(s0, s1, s2, b >> 1, a0, a1, m0, m1);  // entries 2 (b / 2) and the next: (a0, m0), (a1, m1)
+  sc0 = ((b & 1) ? a1 : a0) - 32;
+  sc1 = ((b & 1) ? m1 : m0) - 32;
+}
 
 // MXFP4: four E2M1 codes, one in the low nibble of each byte of c, to the four int8 values of the format's table of
 // doubled values (0 1 2 3 4 6 8 12 | 0 -1 -2 -3 -4 -6 -8 -12; reference src/quants.h:497): a byte permute per table

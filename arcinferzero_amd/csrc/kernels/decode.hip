@@ -138,6 +138,52 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
         }
       }
     }
+  } else if constexpr (QT == QT_Q3_K) {
+    // a unit is one 32-value block: two words of low bit pairs, a word of third bits, two 6-bit scales (one per 16
+    // values) out of the superblock's 12-byte header; value = d * (scale - 32) * (bits - 4), the two halves' sums
+    // weighted in integers as Q6_K's (zero/kernels/decode.cl:203-222 for the fields, :1000-1003 for the formula)
+    const PlanesIQ3S pl = planes_iq3s(plane_rows, nsb);
+    const int ib = hl & 7;
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 3;
+      const int e1 = sb * 256 + 32 * ib;
+      uint4 a1[TB], a2[TB];
+      float sa[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
+        a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
+        a2[t] = *(const uint4*)(aq + (size_t)tt * K + e1 + 16);
+        sa[t] = asc[(size_t)(e1 >> 5) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const size_t n = rows[r];
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
+        const size_t rs = n * nsb + sb;
+        const uint2 q = *(const uint2*)(rb + pl.qs + rs * 64 + ib * 8);
+        const uint32_t H = *(const uint32_t*)(rb + pl.sg + rs * 32 + ib * 4);
+        const uint32_t* hp = (const uint32_t*)(rb + pl.hd + rs * 12);
+        int sc0, sc1;
+        q3k_scales(hp[0], hp[1], hp[2], ib, sc0, sc1);
+        const float d = f16_bits_to_f32(*(const unsigned short*)(rb + pl.d + rs * 2));
+        uint32_t w[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) w[k] = q3k_vals(k < 4 ? q.x : q.y, H, k);
+#pragma unroll
+        for (int t = 0; t < TB; ++t) if (t < nt) {
+          int i1 = dot4(w[0], a1[t].x, 0);
+          i1 = dot4(w[1], a1[t].y, i1);
+          i1 = dot4(w[2], a1[t].z, i1);
+          i1 = dot4(w[3], a1[t].w, i1);
+          int i2 = dot4(w[4], a2[t].x, 0);
+          i2 = dot4(w[5], a2[t].y, i2);
+          i2 = dot4(w[6], a2[t].z, i2);
+          i2 = dot4(w[7], a2[t].w, i2);
+          acc[r][t] += sa[t] * d * (float)(sc0 * i1 + sc1 * i2);
+        }
+      }
+    }
   } else if constexpr (QT == QT_IQ3_S) {
     // a unit is one 32-value block: 8 codebook indices (9 bits: a byte and a bit of the block's ninth-bit byte), 32
     // sign bits, one 4-bit scale s; value = +-(1, 3, ..., 15), sub-scale 1 + 2 s (zero/kernels/decode.cl:400-414)
@@ -366,6 +412,7 @@ GEMV_ALL(13)
 GEMV_ALL(14)
 GEMV_ALL(23)
 GEMV_ALL(2)
+GEMV_ALL(11)
 GEMV_ALL(20)
 GEMV_ALL(39)
 GEMV_ALL(21)
@@ -651,6 +698,7 @@ MOE_DECODE_FUSED_INST(13)
 MOE_DECODE_FUSED_INST(14)
 MOE_DECODE_FUSED_INST(23)
 MOE_DECODE_FUSED_INST(2)
+MOE_DECODE_FUSED_INST(11)
 MOE_DECODE_FUSED_INST(20)
 MOE_DECODE_FUSED_INST(39)
 MOE_DECODE_FUSED_INST(21)
@@ -675,6 +723,7 @@ MOE_DECODE_ALL(13)
 MOE_DECODE_ALL(14)
 MOE_DECODE_ALL(23)
 MOE_DECODE_ALL(2)
+MOE_DECODE_ALL(11)
 MOE_DECODE_ALL(20)
 MOE_DECODE_ALL(39)
 MOE_DECODE_ALL(21)
@@ -713,6 +762,41 @@ extern "C" __global__ __launch_bounds__(256) void expand_iq3s(const uint8_t* __r
     const uint32_t sb = raw[pi.hd + rs * 12 + 8 + j];
     const uint32_t s0 = 1 + 2 * (sb & 0xFu), s1 = 1 + 2 * (sb >> 4);
     *(uint32_t*)(out + po.sc + rs * 16 + 4 * j) = s0 | (s0 << 8) | (s1 << 16) | (s1 << 24);
+  }
+  if (n == 1 && j == 0) *(unsigned short*)(out + po.d + rs * 2) = *(const unsigned short*)(raw + pi.d + rs * 2);
+}
+
+// expand_q3k: the Q3_K planes of `rows` rows to Q6_K planes of the same rows, value for value -- the same f16 d, the
+// 6-bit scales - 32 as the int8 sub-scales, q = value + 32 in six bits -- for the prefill GEMM and the expert-tile GEMM,
+// as expand_iq3s.  Thread (superblock, n, j) makes the words ql[64 n + 4 j ..], ql[64 n + 32 + 4 j ..] and
+// qh[32 n + 4 j ..]: the values 4 j .. 4 j + 3 of blocks 4 n .. 4 n + 3.  grid: ceil(rows * nsb / 16) work-groups of 256.
+extern "C" __global__ __launch_bounds__(256) void expand_q3k(const uint8_t* __restrict__ raw, uint8_t* __restrict__ out, int rows,
+                                                             int nsb) {
+  const size_t total = (size_t)rows * nsb;
+  const size_t rs = (size_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (rs >= total) return;
+  const PlanesIQ3S pi = planes_iq3s((size_t)rows, nsb);
+  const PlanesQ6K po = planes_q6k((size_t)rows, nsb);
+  const int n = (threadIdx.x >> 3) & 1, j = threadIdx.x & 7;
+  uint32_t q[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int ib = 4 * n + k;
+    const uint32_t D = *(const uint32_t*)(raw + pi.qs + rs * 64 + ib * 8 + 4 * (j >> 2));
+    const uint32_t H = *(const uint32_t*)(raw + pi.sg + rs * 32 + ib * 4);
+    const uint32_t v = q3k_vals(D, H, j);
+    q[k] = ((v & 0x7F7F7F7Fu) + 0x20202020u) ^ (v & 0x80808080u);  // value + 32 in every byte, no carry between bytes
+  }
+  const uint32_t lo = 0x0F0F0F0Fu, two = 0x03030303u;
+  *(uint32_t*)(out + po.ql + rs * 128 + 64 * n + 4 * j) = (q[0] & lo) | ((q[2] & lo) << 4);
+  *(uint32_t*)(out + po.ql + rs * 128 + 64 * n + 32 + 4 * j) = (q[1] & lo) | ((q[3] & lo) << 4);
+  *(uint32_t*)(out + po.qh + rs * 64 + 32 * n + 4 * j) =
+      ((q[0] >> 4) & two) | (((q[1] >> 4) & two) << 2) | (((q[2] >> 4) & two) << 4) | (((q[3] >> 4) & two) << 6);
+  if (n == 0) {  // sub-scales 2 j, 2 j + 1: block j's two
+    const uint32_t* hp = (const uint32_t*)(raw + pi.hd + rs * 12);
+    int sc0, sc1;
+    q3k_scales(hp[0], hp[1], hp[2], j, sc0, sc1);
+    *(unsigned short*)(out + po.sc + rs * 16 + 2 * j) = (unsigned short)((uint32_t)(sc0 & 0xFF) | ((uint32_t)(sc1 & 0xFF) << 8));
   }
   if (n == 1 && j == 0) *(unsigned short*)(out + po.d + rs * 2) = *(const unsigned short*)(raw + pi.d + rs * 2);
 }

@@ -30,8 +30,7 @@ void arcz_engine_destroy(arcz_engine* e);
 
 /* make_weight + upload_padded (zero/engine_load.h:84-130, 157-196): N rows of K values as GGUF blocks of `type`
  * (2 = Q4_0, 8 = Q8_0, 11 = Q3_K, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K, 20 = IQ4_NL, 21 = IQ3_S, 23 = IQ4_XS, 39 = MXFP4),
- * regrouped into the device layout -- every type in its own form, the GGUF byte count; Q3_K alone is written out as
- * Q6_K planes, value for value -- and uploaded. */
+ * regrouped into the device layout -- every type in its own form, the GGUF byte count -- and uploaded. */
 arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, const void* gguf, size_t bytes);
 /* The same from a tensor of an open GGUF file (upload of zero/engine_load.h:84-196): a matrix (dims K, N) or an expert
  * tensor (dims K, N, experts) of type Q4_0 / Q8_0 / Q3_K / Q4_K / Q5_K / Q6_K / IQ4_NL / IQ3_S / IQ4_XS / MXFP4, by name;

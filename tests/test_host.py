@@ -100,12 +100,25 @@ def test_repack_planes_layout(qtype):
         assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 8:]) and np.array_equal(P[u * 128:u * 136].reshape(u, 8), sb[:, :8])
         assert not P[u * 136:].any() and P.size % 16 == 0
     elif qtype == az.Q3_K:
-        # written out as Q6_K planes, value for value: put back together as Q6_K rows, they decode to the same floats
-        assert P.size == az.planes_bytes(az.Q6_K, rows, K) and az.gguf_bytes(qtype, rows, K) == u * 110
-        g6 = np.concatenate([P[:u * 128].reshape(u, 128), P[u * 128:u * 192].reshape(u, 64), P[u * 192:u * 208].reshape(u, 16),
-                             P[u * 208:u * 210].reshape(u, 2)], axis=1).reshape(-1)
-        assert np.array_equal(orc.dequant_rows(az.Q6_K, g6, rows, K).view(np.uint32), orc.dequant_rows(qtype, W, rows, K).view(np.uint32))
-        assert not P[u * 210:].any()
+        # a block's bits together: words D0, D1 of bit pairs (value j of a half in byte j % 4, bits 2 (j / 4)), a word of
+        # third bits (value j at bit 8 (j % 4) + j / 4), eight 12-bit header entries of two 6-bit scales, d; put back
+        # together they must give the oracle's fields
+        sb = W.reshape(u, 110)
+        assert P.size == (W.size + 15) // 16 * 16
+        D = P[:u * 64].view(np.uint32).reshape(u, 8, 2).astype(np.int64)
+        H = P[u * 64:u * 96].view(np.uint32).reshape(u, 8).astype(np.int64)
+        j = np.arange(32)
+        q = (((D[:, :, j >> 4] >> (8 * (j & 3) + 2 * ((j & 15) >> 2))) & 3) | (((H[:, :, None] >> (8 * (j & 3) + (j >> 2))) & 1) << 2)) - 4
+        hd = P[u * 96:u * 108].reshape(u, 12)
+        bits = np.zeros(u, dtype=object)
+        for k in range(12):
+            bits = bits + (hd[:, k].astype(object) << (8 * k))
+        sc = np.array([[((int(bits[i]) >> (6 * k)) & 63) - 32 for k in range(16)] for i in range(u)])
+        for r in range(rows):
+            wq, isc, imn, d, dmin = orc.decode_row_fields(qtype, W[r * nsb * 110:(r + 1) * nsb * 110], K)
+            assert np.array_equal(q[r * nsb:(r + 1) * nsb].reshape(K), wq)
+            assert np.array_equal(sc[r * nsb:(r + 1) * nsb].reshape(K // 16), isc)
+        assert np.array_equal(P[u * 108:u * 110].reshape(u, 2), sb[:, 108:110]) and not P[u * 110:].any()
     elif qtype == az.MXFP4:
         blk = W.reshape(u, 8, 17)                                            # eight 17-byte blocks: E8M0 byte, 16 nibble bytes
         assert P.size == (W.size + 15) // 16 * 16
