@@ -486,7 +486,7 @@ class Engine {
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
     const bool mm_type = w.type == GGML_Q4_K || w.type == GGML_Q5_K || w.type == GGML_Q6_K || w.type == GGML_Q8_0 ||
                          w.type == GGML_Q4_0 || w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S || w.type == GGML_IQ4_NL ||
-                         w.type == GGML_MXFP4;
+                         w.type == GGML_MXFP4 || w.type == GGML_Q3_K;
     const bool mm_ok = !mm_off && !q2mm_ && mm_type && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
@@ -504,7 +504,7 @@ class Engine {
       static const bool sk_off = sk_env == 0;
       const size_t sk_groups = (size_t)(sk_env > 0 ? sk_env : 12) * cus;
       const int nsb = K / 256;
-      const int sb_max = w.type == GGML_Q6_K ? 20 : w.type == GGML_Q5_K || w.type == GGML_IQ3_S ? 22 : 24;  // (the kernels' MmT<QT>::SB)
+      const int sb_max = w.type == GGML_Q6_K ? 20 : w.type == GGML_Q5_K || w.type == GGML_IQ3_S || w.type == GGML_Q3_K ? 22 : 24;  // (the kernels' MmT<QT>::SB)
       const int ny = (nsb + sb_max - 1) / sb_max;
       const size_t need = (size_t)ny * 16 * N * 4;
       cl_mem ws = noalloc_ ? arcz_scratch_mem() : sk_ws_;

@@ -1,5 +1,5 @@
 // "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0,
-// Q4_0, IQ4_NL, MXFP4, IQ4_XS, IQ3_S).
+// Q4_0, IQ4_NL, MXFP4, IQ4_XS, IQ3_S, Q3_K).
 //
 // From a handful of tokens on, the dot-product GEMVs are bound by their vector ALU work (eight v_dot4 per token and
 // 16-byte unit), not by memory, and past eight tokens the engine had only the prefill GEMM with its 64-token tiles.
@@ -62,6 +62,8 @@ template <> struct MmT<QT_IQ4_XS> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN
 // (IQ3_S: the main plane is the 8 index bytes per block, the second the sign bits, the header the ninth bits and scale
 //  nibbles, 12 bytes; the codebook, 2 KiB, sits behind the groups' sums in LDS)
 template <> struct MmT<QT_IQ3_S> { enum { SB = 22, QB = 64, D = 8, XB = 32, MIN = 0, DPL = 1 }; };
+// (Q3_K: planes of the same sizes -- 8 bytes of bit pairs per block, the words of third bits, 12 bytes of scales)
+template <> struct MmT<QT_Q3_K> : MmT<QT_IQ3_S> {};
 // LDS: per superblock of a slice 4096 bytes of tokens and 512 of sa (512 more of sa * S); per wave the main plane's rows
 // of one superblock, 1 KiB of headers, the second plane's four superblocks, 256 bytes of d; then 1 KiB per group whose
 // sums wait for the last slice (as many as fit, 12 at most)
@@ -84,11 +86,11 @@ template <int QT> struct MmX { mm_u4 r[MmT<QT>::XB / 16 > 0 ? MmT<QT>::XB / 16 :
 // (Q4_0, IQ4_NL, MXFP4 and IQ4_XS: of each 16-byte block)
 // (IQ3_S: c[b].x the lane's two index bytes of block b, sg the row's eight words of sign bits)
 template <int QT> struct MmSb {
-  mm_u2 c[qt_nib16(QT) || QT == QT_IQ4_XS || QT == QT_IQ3_S ? 8 : MmT<QT>::QB / 32];
+  mm_u2 c[qt_nib16(QT) || QT == QT_IQ4_XS || QT == QT_IQ3_S || QT == QT_Q3_K ? 8 : MmT<QT>::QB / 32];
   mm_u4 h;
   mm_u2 x[2];
   uint32_t d;
-  mm_u4 sg[QT == QT_IQ3_S ? 2 : 1];
+  mm_u4 sg[QT == QT_IQ3_S || QT == QT_Q3_K ? 2 : 1];
 };
 
 // one slice of K, superblocks [s_begin, s_end): at most MmT<QT>::SB of them
@@ -102,8 +104,9 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   constexpr int QB = TT::QB, NQ = QB / 64, D = TT::D, LPRW = QB / 16, RPI = 64 / LPRW;
   constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
   constexpr bool B16 = qt_nib16(QT) || QT == QT_IQ4_XS;  // a block is 16 bytes: low nibbles values 0..15, high 16..31
-  constexpr int HB = QT == QT_IQ4_XS || QT == QT_MXFP4 ? 8 : QT == QT_IQ3_S ? 12 : 16;  // bytes of a row's superblock in the header plane
-  constexpr bool I3 = QT == QT_IQ3_S;
+  constexpr int HB = QT == QT_IQ4_XS || QT == QT_MXFP4 ? 8 : QT == QT_IQ3_S || QT == QT_Q3_K ? 12 : 16;  // bytes of a row's superblock in the header plane
+  constexpr bool I3 = QT == QT_IQ3_S || QT == QT_Q3_K;  // (the two types of these plane sizes)
+  constexpr bool K3 = QT == QT_Q3_K;
   const int tid = threadIdx.x, lane = tid & 63, n16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (a scalar: what follows from it is scalar arithmetic)
   const int nsb = K >> 8, sbs = s_end - s_begin, Ks = sbs * 256, nb = sbs * 8;
@@ -266,7 +269,8 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const int p = B16 ? c : 2 * c + (g >> 1);
-    rd[c] = I3 ? n16 * 64 + (((c >> 1) ^ (n16 >> 2)) << 4) + 8 * (c & 1) + 2 * g
+    rd[c] = K3 ? n16 * 64 + (((c >> 1) ^ (n16 >> 2)) << 4) + 8 * (c & 1) + 4 * (g >> 1)  // (Q3_K: the word of the lane's half)
+            : I3 ? n16 * 64 + (((c >> 1) ^ (n16 >> 2)) << 4) + 8 * (c & 1) + 2 * g
                : ((16 * p + (n16 ^ (LPRW == 8 ? 2 * p : p))) << 4) + (g & 1) * 8;
   }
   const uint8_t* arow = A + n16 * Ks + (g & 1) * 8;
@@ -365,6 +369,32 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] = fmaf(d, part[i], acc[i]);
+    } else if constexpr (K3) {
+      // block b: the lane's eight values 8 g .. 8 g + 7 are the fields 2 g and 2 g + 1 of the block's bit words; the
+      // block's two 16-value halves have a scale each, so, as for Q6_K, two products with the other half's lanes zeroed
+      // (values 0..15 are the lanes g < 2) and sc0 * I0 + sc1 * I1 in integers (zero/kernels/decode.cl:203-222)
+      const float d3 = f16_bits_to_f32(h.d);
+      v4f part = {0.0f, 0.0f, 0.0f, 0.0f};
+      const uint32_t keep0 = g < 2 ? 0xFFFFFFFFu : 0u, keep1 = ~keep0;
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const uint32_t D = h.c[b].x;
+        const uint32_t H = b < 4 ? h.sg[0][b & 3] : h.sg[1][b & 3];
+        const uint32_t w0 = q3k_vals(D, H, 2 * g), w1 = q3k_vals(D, H, 2 * g + 1);
+        const long wa = (long)(((unsigned long)(w1 & keep0) << 32) | (w0 & keep0));
+        const long wb = (long)(((unsigned long)(w1 & keep1) << 32) | (w0 & keep1));
+        v4i z = {0, 0, 0, 0};
+        const v4i Ia = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wa, z, 0, 0, 0);
+        const v4i Ib = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wb, z, 0, 0, 0);
+        int sca, scb;
+        q3k_scales(h.h.x, h.h.y, h.h.z, b, sca, scb);
+        part[0] = fmaf((float)(__mul24(sca, Ia[0]) + __mul24(scb, Ib[0])), sa4[b].x, part[0]);
+        part[1] = fmaf((float)(__mul24(sca, Ia[1]) + __mul24(scb, Ib[1])), sa4[b].y, part[1]);
+        part[2] = fmaf((float)(__mul24(sca, Ia[2]) + __mul24(scb, Ib[2])), sa4[b].z, part[2]);
+        part[3] = fmaf((float)(__mul24(sca, Ia[3]) + __mul24(scb, Ib[3])), sa4[b].w, part[3]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(d3, part[i], acc[i]);
     } else if constexpr (I3) {
       // block b: indices 2 g and 2 g + 1 of its eight (a byte each and a ninth bit from byte b of the header) name
       // codebook words of four magnitudes, the signs are bits 8 g .. 8 g + 7 of the block's word; scale 1 + 2 x nibble b
@@ -480,7 +510,8 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
       MmSb<QT> s;
       if constexpr (I3) {
 #pragma unroll
-        for (int c = 0; c < NC; ++c) s.c[c] = mm_u2{(uint32_t) * (const unsigned short*)(WQ + rd[c]), 0u};
+        for (int c = 0; c < NC; ++c)
+          s.c[c] = mm_u2{K3 ? *(const uint32_t*)(WQ + rd[c]) : (uint32_t) * (const unsigned short*)(WQ + rd[c]), 0u};
         s.sg[0] = *(const mm_u4*)(WX + (j * 16 + n16) * 32);
         s.sg[1] = *(const mm_u4*)(WX + (j * 16 + n16) * 32 + 16);
         s.d = *(const uint32_t*)(WD + ((j * 16 + n16) << 2));
@@ -604,6 +635,7 @@ MM_KERNEL(13)
 MM_KERNEL(14)
 MM_KERNEL(8)
 MM_KERNEL(2)
+MM_KERNEL(11)
 MM_KERNEL(20)
 MM_KERNEL(39)
 MM_KERNEL(23)

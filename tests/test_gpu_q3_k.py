@@ -1,6 +1,6 @@
 """Q3_K weights (reference src/quants.h:465-494: d * (scale - 32) * (three bits - 4), a 6-bit scale per 16 values).  The
 device holds them at the GGUF byte count (110 bytes per 256 values), a block's bits regrouped so that four values leave
-a word with a shift and a mask.  The GEMVs (1-8 tokens) decode them in registers; the GEMM forms first write the matrix
+a word with a shift and a mask.  The GEMVs (chunks of 16 rows) decode them in registers; the GEMM forms first write the matrix
 out as Q6_K planes, value for value (same d, the scales - 32 as the int8 sub-scales, q = value + 32), and run the Q6_K
 kernels on that -- so a chunk of more than 16 rows is bit for bit what the same matrix uploaded as Q6_K superblocks
 gives, and the shorter ones equal it to float rounding.  All against the double-accumulated reference on the Q3_K rows
@@ -61,7 +61,7 @@ def test_q3_k_matmul(rt, T, Mp, N, K):
         assert rel_err_rows(ys[0], ref).max() <= 1e-3
         if Mp > 16:
             assert np.array_equal(ys[0].view(np.uint32), ys[1].view(np.uint32))
-        else:   # (a chunk of 16 rows of a Q6_K matrix takes the matrix-pipe GEMV, which Q3_K does not have)
+        else:
             assert rel_err_rows(ys[0], ys[1]).max() <= 2e-5
         assert az.planes_bytes(az.Q3_K, N, K) == (az.gguf_bytes(az.Q3_K, N, K) + 15) // 16 * 16 == (N * K // 256 * 110 + 15) // 16 * 16
         assert az.lib.arcz_mem_size(az.lib.arcz_weight_raw(w3.h)) == az.planes_bytes(az.Q3_K, N, K)   # 3.44 bits a weight on the device
