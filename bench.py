@@ -167,6 +167,26 @@ def bench_decode(az, qtype, N, K, T, launches, copies):
             "distinct_weight_MB": copies * az.gguf_bytes(qtype, N, K) / 1e6}
 
 
+def bench_types(az, N=17408, K=5120):
+    """Every weight type on the headline matrix: GEMV over 1, 2, 8 and 16 tokens (cycling through distinct weight
+    buffers, as bench_decode) and the prefill GEMM at 2048 tokens.  Not part of the default run (--types)."""
+    names = {az.Q4_0: "Q4_0", az.Q8_0: "Q8_0", az.Q3_K: "Q3_K", az.Q4_K: "Q4_K", az.Q5_K: "Q5_K", az.Q6_K: "Q6_K",
+             az.IQ4_NL: "IQ4_NL", az.IQ3_S: "IQ3_S", az.IQ4_XS: "IQ4_XS", az.MXFP4: "MXFP4"}
+    out = {}
+    for qt, name in names.items():
+        copies = 6
+        row = {"gguf_MB": az.gguf_bytes(qt, N, K) / 1e6, "device_MB": az.planes_bytes(qt, N, K) / 1e6}
+        for T in (1, 2, 8, 16):
+            d = bench_decode(az, qt, N, K, T, 200, copies)
+            row[f"T{T}_us"] = d["kernel_us"]
+            row[f"T{T}_frac_hbm_peak"] = d["frac_hbm_peak"]
+        r, _ = bench_gemm_config(az, qt, N, K, 2048, 5, 61)
+        row["M2048_ms"], row["M2048_TOPS"] = r["ms"], r["TOPS"]
+        out[name] = row
+        log(f"[bench] {name} {N}x{K}: {row}")
+    return out
+
+
 def bench_gemv_gu(az, qtype, F, K, launches, copies):
     """Gate and up of one token in one launch (Engine::gemv_gu), over `copies` distinct pairs of matrices in turn."""
     eng = az.Engine(16, K)
@@ -407,6 +427,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode GEMV extras")
+    ap.add_argument("--types", action="store_true",
+                    help="only the table of all weight types on the headline matrix (one JSON line, key weight_types)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the other configurations (Q8_0 GEMM, Q6_K output head, MoE layer) and the machine probes")
     args = ap.parse_args()
@@ -416,6 +438,9 @@ def main():
     import arcinferzero_amd as az
     az.Runtime.init(0)
     log(f"[bench] {az.Runtime.device_name()}, {az.Runtime.cus()} CUs")
+    if args.types:
+        print(json.dumps({"weight_types": bench_types(az)}))
+        return
     M, N, K, qtype = 8192, 17408, 5120, az.Q4_K
     pre, W = bench_prefill(az, args.steps, args.warmup, M, N, K, qtype)
     log(f"[bench] prefill: {pre}")
