@@ -82,6 +82,7 @@ _sig("arcz_gguf_find", C.c_long, _p, C.c_char_p)
 _sig("arcz_ggml_block_info", _i, _u32, C.POINTER(_i), C.POINTER(_i))
 _sig("arcz_weight_free", _i, _p, _p)
 _sig("arcz_weight_raw", _p, _p)
+_sig("arcz_weight_k", C.c_int, _p)
 _sig("arcz_engine_quantize", _i, _p, _p, _i, _i, _i, _i, _i)
 _sig("arcz_engine_rmsnorm_quant", _i, _p, _p, _i, _p, _i, _i, _i, _i, C.c_float, _p)
 _sig("arcz_engine_add_norm_quant", _i, _p, _p, _p, _p, _i, _i, _i, C.c_float, _p, _i, _i, C.c_float)
@@ -406,7 +407,7 @@ class Engine:
         h = lib.arcz_weight_upload(self.h, qtype, N, K, _np_ptr(gguf), gguf.nbytes)
         if not h:
             raise ArczError(-100, lib.arcz_engine_error().decode())
-        return Weight(self, h, qtype, N, K)
+        return Weight(self, h, qtype, N, lib.arcz_weight_k(h))     # (K rounded up when the rows were padded)
 
     def make_weight_gguf(self, gguf, name):
         """A matrix of an open GgufFile, by name, as it lies in the file."""
@@ -414,7 +415,7 @@ class Engine:
         if not h:
             raise ArczError(-100, lib.arcz_engine_error().decode())
         t = gguf.tensor(gguf.find(name))
-        return Weight(self, h, t["type"], t["dims"][1], t["dims"][0])
+        return Weight(self, h, t["type"], t["dims"][1], lib.arcz_weight_k(h))
 
     def make_moe_layer_gguf(self, gguf, gate, up, down, NU):
         h = lib.arcz_moe_layer_upload_gguf(self.h, gguf.h, gate.encode(), up.encode(), down.encode(), NU)

@@ -108,6 +108,7 @@ int arcz_weight_free(arcz_engine* e, arcz_weight* w) {
   return r;
 }
 arcz_mem* arcz_weight_raw(const arcz_weight* w) { return w ? w->w.raw : nullptr; }
+int arcz_weight_k(const arcz_weight* w) { return w ? w->w.K : 0; }
 int arcz_weight_set_softcap(arcz_weight* w, float cap) {
   if (!w || !(cap >= 0.0f)) return ARCZ_E_ENGINE;
   w->w.softcap = cap;

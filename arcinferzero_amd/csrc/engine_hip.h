@@ -216,7 +216,25 @@ class Engine {
     if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS &&
         type != GGML_IQ3_S && type != GGML_IQ4_NL && type != GGML_MXFP4 && type != GGML_Q3_K)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
-    if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N) throw std::runtime_error("make_weight: K must be a multiple of 256");
+    // Rows of a 32-value-block type that end inside a superblock (K a multiple of 32, not of 256) are padded with zero
+    // blocks to whole superblocks, as the reference's loader pads them (zero/engine_load.h:371-387 load_w_pad with
+    // src/quants.h:661-671: scale bytes 0, so the added elements decode to 0): the weight then has K rounded up, and
+    // the activations it meets are rows of that length whose tail is zero.
+    std::vector<uint8_t> padded;
+    const bool blk32 = type == GGML_Q8_0 || type == GGML_Q4_0 || type == GGML_IQ4_NL || type == GGML_MXFP4;
+    if (blk32 && K > 0 && K % 256 && K % 32 == 0 && N > 0 && rows % (size_t)N == 0) {
+      const int Kp = (K + 255) / 256 * 256;
+      const size_t bb = arcz_gguf_bytes(type, 1, 256) / 8, rb = (size_t)(K / 32) * bb, prb = (size_t)(Kp / 32) * bb;
+      if (nbytes != rows * rb)
+        throw std::runtime_error("make_weight: " + std::to_string(nbytes) + " bytes given, " + std::to_string(rows * rb) + " expected");
+      padded.assign(rows * prb, 0);
+      for (size_t r = 0; r < rows; ++r) memcpy(&padded[r * prb], data + r * rb, rb);
+      data = padded.data();
+      nbytes = padded.size();
+      K = Kp;
+    }
+    if (K <= 0 || K % 256 || N <= 0 || rows % (size_t)N)
+      throw std::runtime_error("make_weight: K must be a multiple of 256 (of 32 for Q8_0, Q4_0, IQ4_NL and MXFP4, whose rows are padded)");
     if ((uint64_t)N * (uint64_t)(K / 256) * 256 >= (1ull << 32))
       throw std::runtime_error("make_weight: a matrix of " + std::to_string(N) + " x " + std::to_string(K) + " is too large for 32-bit row offsets");
     if (nbytes != arcz_gguf_bytes(type, rows, K))

@@ -40,6 +40,11 @@ arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, c
                                            const char* down, int NU);
 int arcz_weight_free(arcz_engine* e, arcz_weight* w);
 arcz_mem* arcz_weight_raw(const arcz_weight* w);
+/* The row length the matmuls see: K, or -- Q8_0, Q4_0, IQ4_NL, MXFP4 rows of a K that is a multiple of 32 but not of
+ * 256 -- K rounded up to whole superblocks, the rows having been padded with zero blocks as the reference's loader
+ * pads them (zero/engine_load.h:371-387, src/quants.h:661-671).  The activations of such a matmul are rows of that
+ * length whose tail is zero. */
+int arcz_weight_k(const arcz_weight* w);
 /* Marks w as the output head of a model with final-logit soft-capping (the reference's lm_head_ with hp.softcap,
  * zero/engine.h:984-990; kernel epilogue -DSOFTCAP=c, zero/kernels/decode.cl:882-886): arcz_engine_matmul over 1-8
  * tokens writes c * tanh(v / c) (then adds C when accumulating); with two-pass inputs both passes run without the cap

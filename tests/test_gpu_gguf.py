@@ -6,7 +6,7 @@ import pytest
 import arcinferzero_amd as az
 import gguf_writer as gw
 import oracle_lib as orc
-from common import make_acts, make_weights, quantize_padded, rel_err_rows
+from common import TYPE_NAMES, make_acts, make_weights, quantize_padded, rel_err_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -75,5 +75,46 @@ def test_moe_layer_from_gguf(rt, tmp_path):
         ref, _ = orc.moe_layer(qt, Wg, Wu, Wd, NE, NU, E, F, aq[:T], asc, logits)
         assert rel_err_rows(out, ref).max() <= 1e-3
         lb.free(); ob.free()
+    finally:
+        eng.close()
+
+
+@pytest.mark.parametrize("qtype,N,K,T,Mp", [(az.Q8_0, 200, 640, 1, 16), (az.MXFP4, 136, 2880, 3, 16), (az.IQ4_NL, 64, 96, 12, 16),
+                                            (az.Q4_0, 300, 2880, 100, 112), (az.MXFP4, 520, 2880, 300, 304)])
+def test_rows_that_end_inside_a_superblock(rt, qtype, N, K, T, Mp):
+    """Rows of a 32-value-block type whose K is a multiple of 32 but not of 256 (the reference's 640-wide shared expert;
+    MXFP4 matrices of 2880 columns): the upload pads them with zero blocks to whole superblocks, as the reference's
+    loader does (zero/engine_load.h:371-387, src/quants.h:661-671), the weight reports the rounded-up K, and the
+    product with activation rows of that length whose tail is zero equals the double-accumulated reference on the
+    unpadded rows."""
+    print(f"padded rows {TYPE_NAMES[qtype]} N={N} K={K} T={T}", flush=True)
+    Kp = (K + 255) // 256 * 256
+    bb = az.gguf_bytes(qtype, 1, 256) // 8                          # bytes of a 32-value block
+    full = make_weights(qtype, N, Kp, seed=470).reshape(N, Kp // 32, bb)
+    W = np.ascontiguousarray(full[:, :K // 32]).reshape(-1)         # rows of K values as a file would hold them
+    eng = az.Engine(Mp, Kp)
+    try:
+        w = eng.make_weight(qtype, N, K, W)
+        assert w.K == Kp and az.lib.arcz_mem_size(az.lib.arcz_weight_raw(w.h)) == az.planes_bytes(qtype, N, Kp)
+        x = np.zeros((T, Kp), np.float32)
+        x[:, :K] = make_acts(T, K, seed=471, outliers=True)
+        xb = az.Runtime.from_numpy(x)
+        eng.quantize(xb, Kp, Kp, Mp, T)
+        rows = T if T <= 8 else Mp
+        cb = az.Runtime.alloc(rows * N * 4).fill(0xFFFFFFFF)
+        eng.matmul("padded", w, Mp, cb, N, 0, 0)
+        y = cb.read(np.float32, rows * N).reshape(rows, N)[:T]
+        zero_tail = full.copy()
+        zero_tail[:, K // 32:] = 0                                   # what the device holds: zero blocks behind the rows
+        aq, asc, _ = quantize_padded(x, Mp)
+        ref = orc.matmul_ref(qtype, zero_tail.reshape(-1), N, Kp, aq[:T], asc)
+        assert np.isfinite(y).all() and rel_err_rows(y, ref).max() <= 1e-3
+        # ... which is the product over the first K columns alone
+        assert np.abs(orc.dequant_rows(qtype, zero_tail.reshape(-1), N, Kp)[:, K:]).max() == 0.0
+        with pytest.raises(az.ArczError):
+            eng.make_weight(az.Q4_K, N, K, W)                       # superblock types: whole superblocks only
+        for b in (cb, xb):
+            b.free()
+        w.free()
     finally:
         eng.close()
