@@ -9,7 +9,7 @@ import os
 
 import numpy as np
 
-Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ3_S, IQ4_XS, MXFP4 = 2, 8, 11, 12, 13, 14, 20, 21, 23, 39  # GGUF type ids
+Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ3_XXS, IQ4_NL, IQ3_S, IQ4_XS, MXFP4 = 2, 8, 11, 12, 13, 14, 18, 20, 21, 23, 39  # GGUF type ids
 
 lib_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libarcz_hip.so")
 if not os.path.exists(lib_path):
@@ -95,6 +95,7 @@ _sig("arcz_engine_asc", _p, _p)
 _sig("arcz_engine_absum", _p, _p)
 _sig("arcz_engine_matmul", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
 _sig("arcz_iq3s_grid", None, _p)
+_sig("arcz_iq3xxs_grid", None, _p)
 _sig("arcz_weight_set_softcap", _i, _p, C.c_float)
 _sig("arcz_engine_gemv_gu", _i, _p, _p, _p, _i, _p)
 _sig("arcz_engine_matmul_noalloc", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)

@@ -15,6 +15,7 @@
 #define GGML_TYPE_IQ3_S 21u  // (src/gguf.h:22)
 #define GGML_TYPE_IQ4_NL 20u  // (src/gguf.h:21)
 #define GGML_TYPE_Q3_K 11u  // (src/gguf.h:20)
+#define GGML_TYPE_IQ3_XXS 18u  // (src/gguf.h:21)
 #define GGML_TYPE_MXFP4 39u  // (src/gguf.h:23)
 
 namespace {
@@ -53,6 +54,36 @@ struct Iq3sGrid {
   }
 };
 const Iq3sGrid kIq3s;
+
+// The IQ3_XXS codebook (ggml's iq3xxs_grid, a constant of the GGUF format; the reference carries it in src/iq_tables.h):
+// 256 entries of four magnitudes out of 4, 12, ..., 52, 62, three hex digits an entry, magnitude j its bits 3 j .. 3 j + 2
+// as an index into that list.
+const char kIq3xxsCodes[] =
+"00000200400900b00f01001201902203b03d04104304804a05105505805a06106c07808008208408909009209909b09f"
+"0a90af0bd0c10c70c80ca0d50f810b11f12412f13b13d14114715a16a19d1b41c81cc1ce1e31f120120320820a211213"
+"21821a21c22722824024224925025228128328828a2912982ba2c02c22d02d92e62f63013053283503543663793853d2"
+"3e040040240940b41041241641942244144344544844a45145847347747848048248948f49049249f4a04ad4c14c84cc"
+"4f84fc51d52b54355756157c5c15c35ce5e560160860a61161362863563a6406426506596646666816836886956aa6ba"
+"6c96db71872773a74074675276d78c79e7b37db7f080480f81d81f82b82f87c89089f8a08b08b68c78e5904929934955"
+"9639789c59c89ca9d8a0aa21a38a40a46a56a6da8ca9aabaac2aebb08b13b17b3ab42b59ba8bd4be2c14c24c26c34c51"
+"c71c8fcb4cd8cded24d45d6ad9bdc3dd1e03e05e07e08e1ae2ae56e60e8aea5eaaec0ecdedbef0f11f21f40f42f54f98";
+struct Iq3xxsGrid {
+  uint8_t m[256][4];
+  Iq3xxsGrid() {
+    for (int i = 0; i < 256; ++i) {
+      int c = 0;
+      for (int k = 0; k < 3; ++k) {
+        const char ch = kIq3xxsCodes[3 * i + k];
+        c = c * 16 + (ch <= '9' ? ch - '0' : ch - 'a' + 10);
+      }
+      for (int j = 0; j < 4; ++j) {
+        const int x = (c >> (3 * j)) & 7;
+        m[i][j] = (uint8_t)(x == 7 ? 62 : 4 + 8 * x);
+      }
+    }
+  }
+};
+const Iq3xxsGrid kIq3xxs;
 
 // 256 six-bit values (0..63) into the ql / qh bytes of a Q6_K superblock (reference src/quants.h:115-134 read backwards)
 void q6k_pack(const int* q, uint8_t* ql, uint8_t* qh) {
@@ -119,13 +150,19 @@ extern "C" {
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K) {
   const size_t u = rows * (size_t)(K / 256);
   return type == QT_Q4_K ? u * 144 : type == QT_Q5_K ? u * 176 : type == QT_Q6_K ? u * 210 : type == QT_Q8_0 ? u * 272 : type == GGML_TYPE_Q4_0 ? u * 144 : type == QT_IQ4_XS ? u * 136 : type == GGML_TYPE_IQ3_S ? u * 110
-         : type == GGML_TYPE_IQ4_NL ? u * 144 : type == GGML_TYPE_MXFP4 ? u * 136 : type == GGML_TYPE_Q3_K ? u * 110 : 0;
+         : type == GGML_TYPE_IQ4_NL ? u * 144 : type == GGML_TYPE_MXFP4 ? u * 136 : type == GGML_TYPE_Q3_K ? u * 110 : type == GGML_TYPE_IQ3_XXS ? u * 98 : 0;
 }
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K) { return raw_planes_bytes((int)type, rows, K / 256); }
 // The IQ3_S codebook as the kernels take it: 512 words, byte j of a word = magnitude j of the entry (1, 3, ..., 15).
 void arcz_iq3s_grid(uint32_t* out) {
   for (int i = 0; i < 512; ++i)
     out[i] = (uint32_t)kIq3s.m[i][0] | ((uint32_t)kIq3s.m[i][1] << 8) | ((uint32_t)kIq3s.m[i][2] << 16) | ((uint32_t)kIq3s.m[i][3] << 24);
+}
+
+// The IQ3_XXS codebook as the kernels take it: 256 words, byte j of a word = magnitude j of the entry.
+void arcz_iq3xxs_grid(uint32_t* out) {
+  for (int i = 0; i < 256; ++i)
+    out[i] = (uint32_t)kIq3xxs.m[i][0] | ((uint32_t)kIq3xxs.m[i][1] << 8) | ((uint32_t)kIq3xxs.m[i][2] << 16) | ((uint32_t)kIq3xxs.m[i][3] << 24);
 }
 
 // GGUF rows -> device planes (layout: kernels/common.h).  0 or -1 (unsupported type / K).
@@ -172,6 +209,20 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
         }
         memcpy(dst + pl.qh + i * 32, H, 32);
       }
+    }
+    return 0;
+  }
+  if (type == GGML_TYPE_IQ3_XXS) {
+    // 98 bytes per superblock (f16 d, 64 index bytes, 8 words of sign codes and scales; reference
+    // src/quants.h:220-239) -> the three fields as planes
+    const PlanesIQ3XXS pl = planes_iq3xxs(rows, nsb);
+    memset(dst + pl.d + u * 2, 0, raw_planes_bytes(QT_IQ3_XXS, rows, nsb) - (pl.d + u * 2));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < u; ++i) {
+      const uint8_t* p = src + i * 98;
+      memcpy(dst + pl.d + i * 2, p, 2);
+      memcpy(dst + pl.qs + i * 64, p + 2, 64);
+      memcpy(dst + pl.ss + i * 32, p + 66, 32);
     }
     return 0;
   }
@@ -568,6 +619,60 @@ static void arcz_quantize_q4_0(const float* src, size_t N, int K, uint8_t* out) 
   }
 }
 
+// f32 rows -> GGUF IQ3_XXS superblocks (98 bytes per 256 values; reference src/quants.h:220-239): per 32-block a step
+// amax / 62 (the codebook's largest magnitude), d / 4 = max step / 31 (d an fp16), the scale s the nearest of 0..15 to
+// (step / (d / 4) - 1) / 2; each 4 values take the codebook entry nearest to their magnitudes (all 256 tried); of each 8
+// values the signs as a 7-bit code whose parity is the eighth's -- where the eight signs are an odd number of minus
+// signs, the value of smallest magnitude changes its sign.  An input generator for tests.
+static void arcz_quantize_iq3_xxs(const float* src, size_t N, int K, uint8_t* out) {
+  const int64_t nsbt = (int64_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+  for (int64_t s = 0; s < nsbt; ++s) {
+    const float* v = src + s * 256;
+    uint8_t* p = out + s * 98;
+    memset(p, 0, 98);
+    float step[8], smax = 0;
+    for (int b = 0; b < 8; ++b) {
+      float amax = 0;
+      for (int i = 0; i < 32; ++i) amax = std::fmax(amax, std::fabs(v[32 * b + i]));
+      step[b] = amax / 62.0f;
+      smax = std::fmax(smax, step[b]);
+    }
+    const uint16_t dh = f32_to_f16(4.0f * smax / 31.0f);
+    const float d4 = f16_to_f32(dh) / 4.0f;
+    memcpy(p, &dh, 2);
+    for (int b = 0; b < 8; ++b) {
+      const int sn = d4 > 0 ? std::min(15, std::max(0, (int)std::lrintf((step[b] / d4 - 1.0f) * 0.5f))) : 0;
+      const float sd = d4 * (float)(1 + 2 * sn), inv = sd > 0 ? 1.0f / sd : 0.0f;
+      uint32_t a = (uint32_t)sn << 28;
+      for (int l = 0; l < 4; ++l) {
+        uint32_t sg = 0;
+        int least = 0;
+        for (int j = 0; j < 8; ++j) {
+          const float x = v[32 * b + 8 * l + j];
+          if (x < 0) sg |= 1u << j;
+          if (std::fabs(x) < std::fabs(v[32 * b + 8 * l + least])) least = j;
+        }
+        if (__builtin_popcount(sg) & 1) sg ^= 1u << least;
+        a |= (sg & 127u) << (7 * l);
+        for (int h = 0; h < 2; ++h) {
+          float m[4];
+          for (int j = 0; j < 4; ++j) m[j] = std::fabs(v[32 * b + 8 * l + 4 * h + j]) * inv;
+          int best = 0;
+          float bd = 1e30f;
+          for (int i = 0; i < 256; ++i) {
+            float e = 0;
+            for (int j = 0; j < 4; ++j) e += (m[j] - (float)kIq3xxs.m[i][j]) * (m[j] - (float)kIq3xxs.m[i][j]);
+            if (e < bd) { bd = e; best = i; }
+          }
+          p[2 + 8 * b + 2 * l + h] = (uint8_t)best;
+        }
+      }
+      memcpy(p + 66 + 4 * b, &a, 4);
+    }
+  }
+}
+
 // f32 rows -> GGUF Q3_K superblocks (110 bytes per 256 values; reference src/quants.h:465-494): per 16 values a step
 // (the value of largest magnitude) / -4, which that value then decodes to exactly; d = the largest |step| / 31 (fp16),
 // the 6-bit scale round(step / d) + 32; each value the nearest of -4..3 steps.  An input generator for tests.
@@ -667,7 +772,7 @@ static void arcz_quantize_mxfp4(const float* src, size_t N, int K, uint8_t* out)
   }
 }
 
-// Quantizes f32 rows to `type` (2, 8, 11, 12, 13, 14, 20, 21, 23, 39).  0 or -1.
+// Quantizes f32 rows to `type` (2, 8, 11, 12, 13, 14, 18, 20, 21, 23, 39).  0 or -1.
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out) {
   if (K <= 0 || K % 256) return -1;
   if (type == GGML_TYPE_Q4_0) arcz_quantize_q4_0(src, N, K, out);
@@ -678,6 +783,7 @@ int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t
   else if (type == QT_IQ4_XS) arcz_quantize_iq4_xs(src, N, K, out);
   else if (type == GGML_TYPE_IQ3_S) arcz_quantize_iq3_s(src, N, K, out);
   else if (type == GGML_TYPE_Q3_K) arcz_quantize_q3_k(src, N, K, out);
+  else if (type == GGML_TYPE_IQ3_XXS) arcz_quantize_iq3_xxs(src, N, K, out);
   else if (type == GGML_TYPE_IQ4_NL) arcz_quantize_iq4_nl(src, N, K, out);
   else if (type == GGML_TYPE_MXFP4) arcz_quantize_mxfp4(src, N, K, out);
   else return -1;

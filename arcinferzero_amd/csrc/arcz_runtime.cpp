@@ -82,7 +82,7 @@ extern "C" {
 
 // the code objects, linked in by kernel_blobs.S
 extern const unsigned char arcz_blob_ops[], arcz_blob_decode[], arcz_blob_decode_q80[], arcz_blob_decode_q40[], arcz_blob_decode_q4k[],
-    arcz_blob_decode_q5k[], arcz_blob_decode_q6k[], arcz_blob_decode_iq4xs[], arcz_blob_decode_iq3s[], arcz_blob_decode_iq4nl[], arcz_blob_decode_mxfp4[], arcz_blob_decode_q3k[], arcz_blob_decode_mm[], arcz_blob_gemm[], arcz_blob_moe[];
+    arcz_blob_decode_q5k[], arcz_blob_decode_q6k[], arcz_blob_decode_iq4xs[], arcz_blob_decode_iq3s[], arcz_blob_decode_iq4nl[], arcz_blob_decode_mxfp4[], arcz_blob_decode_q3k[], arcz_blob_decode_iq3xxs[], arcz_blob_decode_mm[], arcz_blob_gemm[], arcz_blob_moe[];
 
 static std::vector<const unsigned char*> blobs_of(const std::string& which);
 
@@ -293,7 +293,7 @@ int arcz_fill(arcz_mem* dst, const void* pattern, size_t ps, size_t offset, size
 
 static std::vector<const unsigned char*> blobs_of(const std::string& which) {
   if (which == "ops") return {arcz_blob_ops};
-  if (which == "decode") return {arcz_blob_decode, arcz_blob_decode_q80, arcz_blob_decode_q40, arcz_blob_decode_q4k, arcz_blob_decode_q5k, arcz_blob_decode_q6k, arcz_blob_decode_iq4xs, arcz_blob_decode_iq3s, arcz_blob_decode_iq4nl, arcz_blob_decode_mxfp4, arcz_blob_decode_q3k, arcz_blob_decode_mm};
+  if (which == "decode") return {arcz_blob_decode, arcz_blob_decode_q80, arcz_blob_decode_q40, arcz_blob_decode_q4k, arcz_blob_decode_q5k, arcz_blob_decode_q6k, arcz_blob_decode_iq4xs, arcz_blob_decode_iq3s, arcz_blob_decode_iq4nl, arcz_blob_decode_mxfp4, arcz_blob_decode_q3k, arcz_blob_decode_iq3xxs, arcz_blob_decode_mm};
   if (which == "gemm") return {arcz_blob_gemm};
   if (which == "moe") return {arcz_blob_moe};
   return {};

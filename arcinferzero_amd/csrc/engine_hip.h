@@ -24,11 +24,13 @@
 #define GGML_IQ4_XS 23u
 #define GGML_IQ4_NL 20u
 #define GGML_Q3_K 11u
+#define GGML_IQ3_XXS 18u
 #define GGML_MXFP4 39u
 
 extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
 extern "C" size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
 extern "C" void arcz_iq3s_grid(uint32_t* out);
+extern "C" void arcz_iq3xxs_grid(uint32_t* out);
 
 // (zero/engine.h:27-34) raw = the device planes of all `rows` rows (an expert tensor holds n_expert * N rows)
 struct GpuWeight {
@@ -39,11 +41,13 @@ struct GpuWeight {
   // > 0: this matrix is the output head of a model with final-logit soft-capping (the reference's lm_head_ with
   // hp.softcap, zero/engine.h:984-990): the GEMVs (1-8 tokens) write c * tanh(v / c)
   float softcap = 0.0f;
+  // the planes hold half the values (IQ3_XXS written out as Q6_K planes for the GEMM forms): the kernels' -DHD forms
+  bool half_d = false;
 };
 
 inline const char* ggml_type_name(uint32_t t) {
   return t == GGML_Q8_0 ? "Q8_0" : t == GGML_Q4_K ? "Q4_K" : t == GGML_Q5_K ? "Q5_K" : t == GGML_Q6_K ? "Q6_K" : t == GGML_IQ4_XS ? "IQ4_XS"
-         : t == GGML_Q4_0 ? "Q4_0" : t == GGML_IQ3_S ? "IQ3_S" : t == GGML_IQ4_NL ? "IQ4_NL" : t == GGML_MXFP4 ? "MXFP4" : t == GGML_Q3_K ? "Q3_K" : "?";
+         : t == GGML_Q4_0 ? "Q4_0" : t == GGML_IQ3_S ? "IQ3_S" : t == GGML_IQ4_NL ? "IQ4_NL" : t == GGML_MXFP4 ? "MXFP4" : t == GGML_Q3_K ? "Q3_K" : t == GGML_IQ3_XXS ? "IQ3_XXS" : "?";
 }
 
 class Engine {
@@ -70,8 +74,9 @@ class Engine {
     sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
     sk_ws_ = buf(sk_ws_bytes_);
     // the codebook tables the kernels take as `tabs` (the reference's tabs_, zero/engine_setup.h): IQ3_S's 512 entries
-    uint32_t grid[512];
+    uint32_t grid[512 + 256];  // (and IQ3_XXS's 256 behind them)
     arcz_iq3s_grid(grid);
+    arcz_iq3xxs_grid(grid + 512);
     tabs_ = buf(sizeof grid, grid);
   }
   cl_mem tabs_ = nullptr;
@@ -81,10 +86,10 @@ class Engine {
   cl_mem xw_ = nullptr;
   size_t xw_bytes_ = 0;
   GpuWeight gemm_form(const char* name, const GpuWeight& w) {
-    if (w.type != GGML_IQ3_S && w.type != GGML_Q3_K) return w;
+    if (w.type != GGML_IQ3_S && w.type != GGML_Q3_K && w.type != GGML_IQ3_XXS) return w;
     const size_t need = raw_planes_bytes(QT_Q6_K, w.rows, w.K / 256);
     if (need > xw_bytes_) throw std::logic_error("gemm_form: the expansion buffer is smaller than the weight");
-    cl_kernel k = kernel("decode", "", w.type == GGML_Q3_K ? "expand_q3k" : "expand_iq3s");
+    cl_kernel k = kernel("decode", "", w.type == GGML_Q3_K ? "expand_q3k" : w.type == GGML_IQ3_XXS ? "expand_iq3xxs" : "expand_iq3s");
     int rows = (int)w.rows, nsb = w.K / 256;
     if (w.type == GGML_Q3_K) set_args(k, 0, w.raw, xw_, rows, nsb);
     else set_args(k, 0, w.raw, xw_, tabs_, rows, nsb);
@@ -92,6 +97,7 @@ class Engine {
     run(name, k, 1, &g1, &l1);
     GpuWeight x = w;
     x.type = GGML_Q6_K;
+    x.half_d = w.type == GGML_IQ3_XXS;
     x.raw = xw_;
     return x;
   }
@@ -214,7 +220,7 @@ class Engine {
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
     if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS &&
-        type != GGML_IQ3_S && type != GGML_IQ4_NL && type != GGML_MXFP4 && type != GGML_Q3_K)
+        type != GGML_IQ3_S && type != GGML_IQ4_NL && type != GGML_MXFP4 && type != GGML_Q3_K && type != GGML_IQ3_XXS)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
     // Rows of a 32-value-block type that end inside a superblock (K a multiple of 32, not of 256) are padded with zero
     // blocks to whole superblocks, as the reference's loader pads them (zero/engine_load.h:371-387 load_w_pad with
@@ -261,7 +267,7 @@ class Engine {
         wsv_bytes_ = need;
       }
     }
-    if (type == GGML_IQ3_S || type == GGML_Q3_K) {  // (room for its GEMM form)
+    if (type == GGML_IQ3_S || type == GGML_Q3_K || type == GGML_IQ3_XXS) {  // (room for its GEMM form)
       const size_t need = raw_planes_bytes(QT_Q6_K, rows, K / 256);
       if (need > xw_bytes_) {
         if (xw_) release(xw_);
@@ -504,7 +510,7 @@ class Engine {
     static const bool mm_off = getenv("ARCZ_GEMV_MM") && atoi(getenv("ARCZ_GEMV_MM")) == 0;
     const bool mm_type = w.type == GGML_Q4_K || w.type == GGML_Q5_K || w.type == GGML_Q6_K || w.type == GGML_Q8_0 ||
                          w.type == GGML_Q4_0 || w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S || w.type == GGML_IQ4_NL ||
-                         w.type == GGML_MXFP4 || w.type == GGML_Q3_K;
+                         w.type == GGML_MXFP4 || w.type == GGML_Q3_K || w.type == GGML_IQ3_XXS;
     const bool mm_ok = !mm_off && !q2mm_ && mm_type && a <= 1 && w.softcap <= 0.0f;  // (gemv_mm has no soft cap)
     auto gemv_mm = [&] {
       int N = w.N, K = w.K, M = Mp, T = cur_T_;
@@ -522,7 +528,7 @@ class Engine {
       static const bool sk_off = sk_env == 0;
       const size_t sk_groups = (size_t)(sk_env > 0 ? sk_env : 12) * cus;
       const int nsb = K / 256;
-      const int sb_max = w.type == GGML_Q6_K ? 20 : w.type == GGML_Q5_K || w.type == GGML_IQ3_S || w.type == GGML_Q3_K ? 22 : 24;  // (the kernels' MmT<QT>::SB)
+      const int sb_max = w.type == GGML_Q6_K ? 20 : w.type == GGML_Q5_K || w.type == GGML_IQ3_S || w.type == GGML_Q3_K || w.type == GGML_IQ3_XXS ? 22 : 24;  // (the kernels' MmT<QT>::SB)
       const int ny = (nsb + sb_max - 1) / sb_max;
       const size_t need = (size_t)ny * 16 * N * 4;
       cl_mem ws = noalloc_ ? arcz_scratch_mem() : sk_ws_;
@@ -577,11 +583,11 @@ class Engine {
       // the kernel's token slots: T rounded up, or -- both halves of two-pass inputs in one launch -- 2 T rounded up
       auto lds_of = [&](int slots) { return (size_t)slots * tok_bytes + (wpr > 1 ? (size_t)16 * g * wpr * slots * 4 : 0); };  // (16: the kernels' GEMV_FLUSH)
       const int tb2 = T == 1 ? 2 : T == 2 ? 4 : 8;
-      const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= (w.type == GGML_IQ3_S ? 65536 - 2048 : 65536);
+      const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= (w.type == GGML_IQ3_S || w.type == GGML_IQ3_XXS ? 65536 - 2048 : 65536);
       const int tbl = q2f ? tb2 : T <= 2 ? T : T <= 4 ? 4 : 8;
       const size_t lds = lds_of(tbl);
       // (IQ3_S: 2 KiB of the work-group's LDS hold the codebook)
-      const size_t lds_max = w.type == GGML_IQ3_S ? 65536 - 2048 : 65536;
+      const size_t lds_max = w.type == GGML_IQ3_S || w.type == GGML_IQ3_XXS ? 65536 - 2048 : 65536;
       const bool fits = !force_v && lpr && lds <= lds_max;
       static const int mm_min = getenv("ARCZ_GEMV_MM_MIN") ? atoi(getenv("ARCZ_GEMV_MM_MIN")) : 5;
       if (mm_ok && T >= 3 && (T >= mm_min || !fits)) {
@@ -599,7 +605,8 @@ class Engine {
         // 17408 x 5120: 20.2 against 25.7 with one; three or four per unit are slower everywhere).
         static const int wpc_env = getenv("ARCZ_GEMV_WPC") ? atoi(getenv("ARCZ_GEMV_WPC")) : 0;
         static const int wgs_env = getenv("ARCZ_GEMV_WGS") ? atoi(getenv("ARCZ_GEMV_WGS")) : 0;
-        const bool codebook = w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S || w.type == GGML_IQ4_NL || w.type == GGML_MXFP4;
+        const bool codebook = w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S || w.type == GGML_IQ4_NL || w.type == GGML_MXFP4 ||
+                              w.type == GGML_IQ3_XXS;
         const int wpc = wpc_env > 0 ? wpc_env : bt == 512 || (tb == 1 && !codebook) ? 1 : 2;
         size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * wpc);
         if (wgs_env > 0) wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)wgs_env);
@@ -653,7 +660,7 @@ class Engine {
     if (!lpr) return false;
     const int gr = 256 / lpr, wpr = lpr > 64 ? lpr / 64 : 1;
     const size_t lds = (size_t)tok_bytes + (wpr > 1 ? (size_t)16 * gr * wpr * 4 : 0);
-    if (lds > (g.type == GGML_IQ3_S ? 65536u - 2048u : 65536u) || N % gr) return false;
+    if (lds > (g.type == GGML_IQ3_S || g.type == GGML_IQ3_XXS ? 65536u - 2048u : 65536u) || N % gr) return false;
     if (arcz_mem_size(C) < (size_t)2 * N * 4) throw std::runtime_error("gemv_gu: the output does not fit C");
     rd_bytes += raw_bytes(g) + raw_bytes(u);
     const int pf = (units + lpr - 1) / lpr;
@@ -718,7 +725,7 @@ class Engine {
           ws = sk_ws_;
         }
         cl_kernel k = kernel("gemm", std::string("-DQTYPE=") + std::to_string(w.type) + " -DACT32 -DBM=" + std::to_string(bm) +
-                                         " -DBN=128 -DSPLITK", "gemm");
+                                         " -DBN=128 -DSPLITK" + (w.half_d ? " -DHDS" : ""), "gemm");
         cl_mem unused = nullptr;
         int zero = 0, one = 1, ldw = N, s1 = nsb;
         set_args(k, 0, w.raw, unused, aq_, asc_, absum_, ws, M, N, K, ldw, zero, zero, one, zero, s1);
@@ -766,7 +773,7 @@ class Engine {
                   : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")
                   : q4_wide ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64", "gemm")
                   : au      ? kernel("gemm", "-DQTYPE=" + std::to_string(w.type) + (au4 ? " -DACT32 -DAU=4" : au3 ? " -DACT32 -DAU=3" : au2 ? " -DACT32 -DAU=2" : " -DACT32 -DAU"), "gemm")
-                            : gemm_kernel(w.type, false);
+                            : gemm_kernel(w.type, false, 0, w.half_d);
     // (ARCZ_GEMM_SPLIT: superblocks per split-K piece, 0 = one pass, the default here: a work-group keeps its sums in
     //  registers over the whole of K.  The reference splits rows longer than 8192 into 17-superblock pieces for its
     //  cache, zero/engine.h:1236-1250; pieces after the first accumulate into C and are not bit-identical to one pass.)
@@ -801,9 +808,10 @@ class Engine {
     }
   }
   // (zero/engine_setup.h:384-420 gemm_kernel / moe_gemm_kernel)
-  cl_kernel gemm_kernel(uint32_t qtype, bool tiles, int ne = 0) {
+  cl_kernel gemm_kernel(uint32_t qtype, bool tiles, int ne = 0, bool half_d = false) {
     std::string defs = "-DQTYPE=" + std::to_string(qtype) + " -DACT32";
     if (tiles) defs += " -DMOE_TILES -DNE=" + std::to_string(ne);
+    if (half_d) defs += tiles ? " -DHDT" : " -DHD";
     return kernel("gemm", defs, "gemm");
   }
 
@@ -914,7 +922,7 @@ class Engine {
     for (int i = part; i < (part == 0 ? 2 : 3); ++i) {
       const int N = i == 2 ? E : F, K = i == 2 ? F : E;
       const GpuWeight wx = gemm_form(i == 2 ? "moe_down" : "moe_gateup", L.ex[i]);
-      cl_kernel k = gemm_kernel(wx.type, true, NE);
+      cl_kernel k = gemm_kernel(wx.type, true, NE, wx.half_d);
       int M = i == 2 ? slots_ : Mp, NN = N, KK = K, ldc = N, acc = i == 1 ? 2 : 0, e0 = 0, e1 = NE, um = i == 2 ? 0 : 1,
           us = i == 2 ? 1 : 0;
       cl_mem unused = nullptr;
@@ -1055,7 +1063,7 @@ class Engine {
     bool t64 = false;
     for (int i = 0; i < 3; ++i)
       t64 = t64 || L.ex[i].type == GGML_Q4_K || L.ex[i].type == GGML_Q5_K || L.ex[i].type == GGML_Q6_K || L.ex[i].type == GGML_IQ3_S ||
-            L.ex[i].type == GGML_Q3_K;
+            L.ex[i].type == GGML_Q3_K || L.ex[i].type == GGML_IQ3_XXS;
     const int tm = t64 ? 64 : 128;
     moe_route(L, rl, ldl, T, tm);
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)

@@ -20,6 +20,7 @@
     BLOB arcz_blob_decode_iq4nl, "decode_iq4nl.hsaco"
     BLOB arcz_blob_decode_mxfp4, "decode_mxfp4.hsaco"
     BLOB arcz_blob_decode_q3k, "decode_q3k.hsaco"
+    BLOB arcz_blob_decode_iq3xxs, "decode_iq3xxs.hsaco"
     BLOB arcz_blob_decode_mm, "decode_mm.hsaco"
     BLOB arcz_blob_gemm, "gemm.hsaco"
     BLOB arcz_blob_moe, "moe.hsaco"

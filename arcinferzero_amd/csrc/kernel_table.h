@@ -14,7 +14,7 @@ struct KernelSpec {
   const char* name;
   const char* requires_def;  // this entry is taken only when the -D string holds this name (nullptr: always)
   const char* args;
-  const char* variant[6];  // nullptr-terminated
+  const char* variant[8];  // nullptr-terminated
   HiddenDef hidden[6];     // {nullptr} terminated
   int local_x;             // threads per work-group the kernel is written for (0 = any)
 };
@@ -56,9 +56,15 @@ static const KernelSpec kKernelTable[] = {
     {"decode", "moe_down_q", nullptr, "piipppipppp", {"QT", "GROWS", "TM", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"decode", "expand_iq3s", nullptr, "pppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"decode", "expand_q3k", nullptr, "ppii", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"decode", "expand_iq3xxs", nullptr, "pppii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"decode", "gemv_v", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt_v", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     // ---- gemm
+    // (-DHDT / -DHDS / -DHD: the Q6_K kernels on planes that hold half the values -- IQ3_XXS written out as Q6_K)
+    {"gemm", "gemm", "HDT", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", "HDT", nullptr},
+     {{"NE", 0, true}, {nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "HDS", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", "HDS", nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "HD", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "HD", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", "MOE_TILES", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm", "SPLITK", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", nullptr}, {{nullptr, 0, false}}, 256},

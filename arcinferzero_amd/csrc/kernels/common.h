@@ -18,6 +18,7 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 #define QT_Q4_K 12
 #define QT_Q5_K 13
 #define QT_Q6_K 14
+#define QT_IQ3_XXS 18
 #define QT_IQ4_NL 20
 #define QT_IQ3_S 21
 #define QT_IQ4_XS 23
@@ -44,6 +45,11 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 //   Q4_0 : qs  [R][nsb][128]  (the sixteen nibble bytes of each of the superblock's eight 32-value blocks, as GGUF: byte
 //                              j of block b = element 32b+j low nibble, 32b+16+j high nibble; value = nibble - 8),
 //          d   [R][nsb][8] (f16: the eight blocks' scales).  144 bytes per 256 values, as GGUF's eight 18-byte blocks.
+//   IQ3_XXS: qs [R][nsb][64]  (eight codebook indices per 32-value block, a byte each, each naming 4 magnitudes of
+//                              4, 12, ..., 52, 62), ss [R][nsb][8] words (block b: four 7-bit sign codes -- the signs of 8
+//                              values, the eighth making their number even -- and in the top nibble the scale s),
+//          d   [R][nsb]       (f16).  value = d / 4 * (1 + 2 s) * the signed magnitude.  98 bytes per 256 values, as
+//          GGUF (src/quants.h:220-239).
 //   Q3_K : the planes of IQ3_S in size and place (planes_iq3s), regrouped from GGUF's hmask / qs / scales so that a
 //          32-value block's bits lie together and four values come out of a word with a shift and a mask:
 //          qs  [R][nsb][64]   (block b: words D0, D1 at bytes 8 b: value j of the block's first / second 16 in byte
@@ -71,6 +77,7 @@ struct PlanesIQ4XS { size_t qs, hdr; };
 struct PlanesQ40 { size_t qs, d; };
 struct PlanesIQ3S { size_t qs, sg, hd, d; };
 struct PlanesMXFP4 { size_t qs, e; };
+struct PlanesIQ3XXS { size_t qs, ss, d; };
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 __host__ __device__ inline PlanesQ4K planes_q4k(size_t rows, int nsb) {
@@ -113,6 +120,14 @@ __host__ __device__ inline PlanesMXFP4 planes_mxfp4(size_t rows, int nsb) {
   p.e = rows * (size_t)nsb * 128;
   return p;
 }
+__host__ __device__ inline PlanesIQ3XXS planes_iq3xxs(size_t rows, int nsb) {
+  PlanesIQ3XXS p;
+  const size_t u = rows * (size_t)nsb;
+  p.qs = 0;
+  p.ss = u * 64;
+  p.d = u * 96;
+  return p;
+}
 __host__ __device__ inline PlanesIQ3S planes_iq3s(size_t rows, int nsb) {
   PlanesIQ3S p;
   const size_t u = rows * (size_t)nsb;
@@ -125,6 +140,7 @@ __host__ __device__ inline PlanesIQ3S planes_iq3s(size_t rows, int nsb) {
 __host__ __device__ inline size_t raw_planes_bytes(int qt, size_t rows, int nsb) {
   const size_t u = rows * (size_t)nsb;
   if (qt == QT_IQ3_S || qt == QT_Q3_K) return align16(u * 110);
+  if (qt == QT_IQ3_XXS) return align16(u * 98);
   if (qt == QT_Q4_0 || qt == QT_IQ4_NL) return u * 144;
   if (qt == QT_MXFP4) return align16(u * 136);
   if (qt == QT_Q4_K) return u * 144;
@@ -176,6 +192,13 @@ __device__ inline uint32_t iq4_lookup(uint32_t c) {
 // Q4_0: four nibbles, one in the low nibble of each byte of c (the other bits ignored), to the four int8 values
 // nibble - 8, without borrows between bytes.
 __device__ inline uint32_t q40_vals(uint32_t c) { return (((c & 0x0F0F0F0Fu) | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
+
+// IQ3_XXS: the sign bits of values 8 l .. 8 l + 7 of a block from its word a: the 7-bit code at bit 7 l, and as the
+// eighth bit the code's parity (ggml's ksigns_iq2xs, which the reference carries as a table: src/iq_tables.h).
+__device__ inline uint32_t iq3xxs_signs8(uint32_t a, int l) {
+  const uint32_t c = (a >> (7 * l)) & 127u;
+  return c | ((__builtin_popcount(c) & 1u) << 7);
+}
 
 // Q3_K (device form): the four int8 values 4 k .. 4 k + 3 (k = 0..7) of a 32-value block from its words of low bits
 // (D = D0 for k < 4, D1 above) and third bits H: the three bits - 4, no borrow between bytes.

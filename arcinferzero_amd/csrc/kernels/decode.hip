@@ -22,10 +22,20 @@ template <int QT> struct UnitsPerSb { static constexpr int v = QT == QT_Q8_0 ? 1
 
 // IQ3_S: the codebook (512 entries of four magnitudes 1, 3, ..., 15, one per byte; ggml's iq3s_grid) in LDS, copied from
 // the kernels' `tabs` argument once per work-group, before anything else (every thread of the work-group calls this).
+// IQ3_XXS: its 256 entries (magnitudes 4, 12, ..., 52, 62; ggml's iq3xxs_grid) lie behind those in `tabs` and take the
+// array's first 256 words.
 __shared__ uint32_t iq3s_grid_lds[512];
 __device__ inline void iq3s_grid_init(const uint32_t* __restrict__ tabs) {
   for (int i = threadIdx.x; i < 512; i += blockDim.x) iq3s_grid_lds[i] = tabs[i];
   __syncthreads();
+}
+template <int QT>
+__device__ inline void grid_init(const uint32_t* __restrict__ tabs) {
+  if constexpr (QT == QT_IQ3_S) iq3s_grid_init(tabs);
+  if constexpr (QT == QT_IQ3_XXS) {
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) iq3s_grid_lds[i] = tabs[512 + i];
+    __syncthreads();
+  }
 }
 
 // acc[r][t] += the products of plane rows rows[r] (absolute rows of planes that hold `plane_rows` rows) with the token
@@ -135,6 +145,54 @@ __device__ __forceinline__ void gemv_acc(const uint8_t* __restrict__ raw, size_t
           i2 = dot4(w2[3], a2[t].w, i2);
           acc[r][t] += sa1[t] * d * (float)(sc1 * i1);
           acc[r][t] += sa2[t] * d * (float)(sc2 * i2);
+        }
+      }
+    }
+  } else if constexpr (QT == QT_IQ3_XXS) {
+    // a unit is one 32-value block: 8 codebook indices (a byte each) and a word of four 7-bit sign codes and the 4-bit
+    // scale s; value = d / 4 * (1 + 2 s) * the signed magnitude (zero/kernels/decode.cl:183-478, src/quants.h:220-239)
+    const PlanesIQ3XXS pl = planes_iq3xxs(plane_rows, nsb);
+    const int ib = hl & 7;
+    for (int u = hl; u < units; u += 32) {
+      const int sb = u >> 3;
+      const int e1 = sb * 256 + 32 * ib;
+      uint4 a1[TB], a2[TB];
+      float sa[TB];
+#pragma unroll
+      for (int t = 0; t < TB; ++t) if (t < nt) {
+        const int tt = tok[t];
+        a1[t] = *(const uint4*)(aq + (size_t)tt * K + e1);
+        a2[t] = *(const uint4*)(aq + (size_t)tt * K + e1 + 16);
+        sa[t] = asc[(size_t)(e1 >> 5) * M + tt];
+      }
+#pragma unroll
+      for (int r = 0; r < GROWS; ++r) {
+        const size_t n = rows[r];
+        const uint8_t* rb = r < SPLIT ? raw : raw2;
+        const size_t rs = n * nsb + sb;
+        const uint2 q = *(const uint2*)(rb + pl.qs + rs * 64 + ib * 8);
+        const uint32_t a = *(const uint32_t*)(rb + pl.ss + rs * 32 + ib * 4);
+        const int sc = 1 + 2 * (int)(a >> 28);
+        const float d = 0.25f * f16_bits_to_f32(*(const unsigned short*)(rb + pl.d + rs * 2));
+        uint32_t w[8];
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+          const uint32_t s8 = iq3xxs_signs8(a, l);
+          const uint32_t qq = l < 2 ? q.x : q.y;
+          w[2 * l] = iq3s_signed4(iq3s_grid_lds[(qq >> (16 * (l & 1))) & 0xFFu], s8 & 0xFu);
+          w[2 * l + 1] = iq3s_signed4(iq3s_grid_lds[(qq >> (16 * (l & 1) + 8)) & 0xFFu], s8 >> 4);
+        }
+#pragma unroll
+        for (int t = 0; t < TB; ++t) if (t < nt) {
+          int i1 = dot4(w[0], a1[t].x, 0);
+          i1 = dot4(w[1], a1[t].y, i1);
+          i1 = dot4(w[2], a1[t].z, i1);
+          i1 = dot4(w[3], a1[t].w, i1);
+          i1 = dot4(w[4], a2[t].x, i1);
+          i1 = dot4(w[5], a2[t].y, i1);
+          i1 = dot4(w[6], a2[t].z, i1);
+          i1 = dot4(w[7], a2[t].w, i1);
+          acc[r][t] += sa[t] * d * (float)(sc * i1);
         }
       }
     }
@@ -386,7 +444,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
   extern "C" __global__ __launch_bounds__(256) void gemv_v__QT##QT##_GROWS##GROWS(                                      \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
       const short* absum, int M, float* C, int c_off, int accumulate, float softcap) {                                \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     gemv_body<QT, 1, GROWS>(raw, N, K, aq, asc, absum, M, 1, C, 0, c_off, accumulate, (size_t)N, softcap);           \
   }
 
@@ -395,7 +453,7 @@ __device__ inline void gemv_body(const uint8_t* __restrict__ raw, int N, int K, 
   extern "C" __global__ __launch_bounds__(256) void gemv_mt_v__QT##QT##_GROWS##GROWS##_TB##TB(                          \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* aq, const float* asc,               \
       const short* absum, int M, int T, float* C, int ldc, int c_off, int accumulate, float softcap) {                \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     gemv_body<QT, TB, GROWS>(raw, N, K, aq, asc, absum, M, T, C, ldc, c_off, accumulate, (size_t)N, softcap);        \
   }
 
@@ -412,6 +470,7 @@ GEMV_ALL(13)
 GEMV_ALL(14)
 GEMV_ALL(23)
 GEMV_ALL(2)
+GEMV_ALL(18)
 GEMV_ALL(11)
 GEMV_ALL(20)
 GEMV_ALL(39)
@@ -666,21 +725,21 @@ __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, in
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
       short* hbs, int NE) {                                                                                           \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     moe_gateup_quant_rows<QT, 1>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM2_QUANT1(                         \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,     \
       short* hbs, int NE) {                                                                                           \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     moe_gateup_quant_rows<QT, 2>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE, S, hq, hsc, hbs);              \
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(512) void moe_gateup_q__QT##QT##_GROWS4_TM1_QUANT1_ROUTE1(                  \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, int* tiles, int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc, short* hbs,     \
       const float* logits, float* sgate, float* swt, int* inv, int NU, int ldl, int T, int* ids, float* wts, int NE) { \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     MoeRouteArgs ra;                                                                                                  \
     ra.logits = logits; ra.sgate = sgate; ra.swt = swt; ra.tiles_out = tiles; ra.stok_out = stok; ra.inv = inv;       \
     ra.NU = NU; ra.ldl = ldl; ra.T = T; ra.ids = ids; ra.wts = wts;                                                   \
@@ -689,7 +748,7 @@ __device__ inline void moe_down1_rows(const uint8_t* __restrict__ raw, int N, in
   extern "C" __global__ __launch_bounds__(256) void moe_down1_q__QT##QT##_GROWS4(                                     \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
       const int* tiles, const float* swt, float* x, const short* hbs, const int* inv, int NU, int NE) {              \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     moe_down1_rows<QT, 4>(raw, N, K, hq, hsc, hbs, S, tiles, swt, x, inv, NU, NE);                                   \
   }
 MOE_DECODE_FUSED_INST(8)
@@ -698,6 +757,7 @@ MOE_DECODE_FUSED_INST(13)
 MOE_DECODE_FUSED_INST(14)
 MOE_DECODE_FUSED_INST(23)
 MOE_DECODE_FUSED_INST(2)
+MOE_DECODE_FUSED_INST(18)
 MOE_DECODE_FUSED_INST(11)
 MOE_DECODE_FUSED_INST(20)
 MOE_DECODE_FUSED_INST(39)
@@ -707,13 +767,13 @@ MOE_DECODE_FUSED_INST(21)
   extern "C" __global__ __launch_bounds__(256) void moe_gateup_q__QT##QT##_GROWS2_TM##TM(                             \
       const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc, \
       int M, const int* tiles, const int* stok, float* h, const short* absum, int NE) {                              \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     moe_gateup_rows<QT, TM, 2>(rg, ru, F, K, aq, asc, absum, M, tiles, stok, h, NE);                                 \
   }                                                                                                                   \
   extern "C" __global__ __launch_bounds__(256) void moe_down_q__QT##QT##_GROWS2_TM##TM(                               \
       const uint8_t* raw, int N, int K, const uint32_t* tabs, const signed char* hq, const float* hsc, int S,         \
       const int* tiles, const float* swt, float* y, const short* hbs, int NE) {                                      \
-    if (QT == QT_IQ3_S) iq3s_grid_init(tabs);                                                                         \
+    grid_init<QT>(tabs);                                                                                           \
     moe_down_rows<QT, TM, 2>(raw, N, K, hq, hsc, hbs, S, tiles, swt, y, NE);                                         \
   }
 #define MOE_DECODE_ALL(QT) MOE_DECODE_INST(QT, 1) MOE_DECODE_INST(QT, 2) MOE_DECODE_INST(QT, 4) MOE_DECODE_INST(QT, 8)
@@ -723,6 +783,7 @@ MOE_DECODE_ALL(13)
 MOE_DECODE_ALL(14)
 MOE_DECODE_ALL(23)
 MOE_DECODE_ALL(2)
+MOE_DECODE_ALL(18)
 MOE_DECODE_ALL(11)
 MOE_DECODE_ALL(20)
 MOE_DECODE_ALL(39)
@@ -797,6 +858,42 @@ extern "C" __global__ __launch_bounds__(256) void expand_q3k(const uint8_t* __re
     int sc0, sc1;
     q3k_scales(hp[0], hp[1], hp[2], j, sc0, sc1);
     *(unsigned short*)(out + po.sc + rs * 16 + 2 * j) = (unsigned short)((uint32_t)(sc0 & 0xFF) | ((uint32_t)(sc1 & 0xFF) << 8));
+  }
+  if (n == 1 && j == 0) *(unsigned short*)(out + po.d + rs * 2) = *(const unsigned short*)(raw + pi.d + rs * 2);
+}
+
+// expand_iq3xxs: the IQ3_XXS planes of `rows` rows to Q6_K planes of the same rows that hold HALF the values -- the
+// magnitudes are even, so q = value / 2 + 32 fits six bits; the int8 sub-scale 1 + 2 s for both halves of a block; and
+// d / 4, which an f16 cannot always hold, as d unchanged: the Q6_K GEMM kernels that run on these planes (-DHD, -DHDS,
+// -DHDT) halve their factor of d -- as expand_iq3s.  Thread (superblock, n, j) makes the words ql[64 n + 4 j ..],
+// ql[64 n + 32 + 4 j ..] and qh[32 n + 4 j ..]: the values 4 j .. 4 j + 3 of blocks 4 n .. 4 n + 3, one codebook entry per
+// block.  grid: ceil(rows * nsb / 16) work-groups of 256.
+extern "C" __global__ __launch_bounds__(256) void expand_iq3xxs(const uint8_t* __restrict__ raw, uint8_t* __restrict__ out,
+                                                                const uint32_t* __restrict__ tabs, int rows, int nsb) {
+  grid_init<QT_IQ3_XXS>(tabs);
+  const size_t total = (size_t)rows * nsb;
+  const size_t rs = (size_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (rs >= total) return;
+  const PlanesIQ3XXS pi = planes_iq3xxs((size_t)rows, nsb);
+  const PlanesQ6K po = planes_q6k((size_t)rows, nsb);
+  const int n = (threadIdx.x >> 3) & 1, j = threadIdx.x & 7;
+  uint32_t q[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int ib = 4 * n + k;
+    const uint32_t a = *(const uint32_t*)(raw + pi.ss + rs * 32 + ib * 4);
+    const uint32_t s4 = (iq3xxs_signs8(a, j >> 1) >> (4 * (j & 1))) & 0xFu;
+    const uint32_t v = iq3s_signed4(iq3s_grid_lds[raw[pi.qs + rs * 64 + ib * 8 + j]] >> 1, s4);  // (magnitudes halved: 2 .. 31)
+    q[k] = ((v & 0x7F7F7F7Fu) + 0x20202020u) ^ (v & 0x80808080u);  // value + 32 in every byte, no carry between bytes
+  }
+  const uint32_t lo = 0x0F0F0F0Fu, two = 0x03030303u;
+  *(uint32_t*)(out + po.ql + rs * 128 + 64 * n + 4 * j) = (q[0] & lo) | ((q[2] & lo) << 4);
+  *(uint32_t*)(out + po.ql + rs * 128 + 64 * n + 32 + 4 * j) = (q[1] & lo) | ((q[3] & lo) << 4);
+  *(uint32_t*)(out + po.qh + rs * 64 + 32 * n + 4 * j) =
+      ((q[0] >> 4) & two) | (((q[1] >> 4) & two) << 2) | (((q[2] >> 4) & two) << 4) | (((q[3] >> 4) & two) << 6);
+  if (n == 0) {  // sub-scales 2 j, 2 j + 1: block j's, the same for both of its halves
+    const uint32_t sc = 1u + 2u * (*(const uint32_t*)(raw + pi.ss + rs * 32 + j * 4) >> 28);
+    *(unsigned short*)(out + po.sc + rs * 16 + 2 * j) = (unsigned short)(sc | (sc << 8));
   }
   if (n == 1 && j == 0) *(unsigned short*)(out + po.d + rs * 2) = *(const unsigned short*)(raw + pi.d + rs * 2);
 }

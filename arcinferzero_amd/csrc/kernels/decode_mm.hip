@@ -1,5 +1,5 @@
 // "decode" module, part: gemv_mm, the matrix-vector form for 3..16 tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0,
-// Q4_0, IQ4_NL, MXFP4, IQ4_XS, IQ3_S, Q3_K).
+// Q4_0, IQ4_NL, MXFP4, IQ4_XS, IQ3_S, Q3_K, IQ3_XXS).
 //
 // From a handful of tokens on, the dot-product GEMVs are bound by their vector ALU work (eight v_dot4 per token and
 // 16-byte unit), not by memory, and past eight tokens the engine had only the prefill GEMM with its 64-token tiles.
@@ -64,6 +64,8 @@ template <> struct MmT<QT_IQ4_XS> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN
 template <> struct MmT<QT_IQ3_S> { enum { SB = 22, QB = 64, D = 8, XB = 32, MIN = 0, DPL = 1 }; };
 // (Q3_K: planes of the same sizes -- 8 bytes of bit pairs per block, the words of third bits, 12 bytes of scales)
 template <> struct MmT<QT_Q3_K> : MmT<QT_IQ3_S> {};
+// (IQ3_XXS: the index bytes and the blocks' words of sign codes and scales likewise; no header plane)
+template <> struct MmT<QT_IQ3_XXS> : MmT<QT_IQ3_S> {};
 // LDS: per superblock of a slice 4096 bytes of tokens and 512 of sa (512 more of sa * S); per wave the main plane's rows
 // of one superblock, 1 KiB of headers, the second plane's four superblocks, 256 bytes of d; then 1 KiB per group whose
 // sums wait for the last slice (as many as fit, 12 at most)
@@ -71,7 +73,7 @@ template <int QT> struct MmL {
   static constexpr int TOK = 4096 + 512 + (MmT<QT>::MIN ? 512 : 0);
   static constexpr int WQ = MmT<QT>::QB * 16 < 2048 ? 2048 : MmT<QT>::QB * 16;  // (also the wave's two partial sums: 2 KiB)
   static constexpr int WH = 1024, WX = MmT<QT>::XB * 64, WD = MmT<QT>::DPL ? 256 : 0;
-  static constexpr int GRID = QT == QT_IQ3_S ? 2048 : 0;
+  static constexpr int GRID = QT == QT_IQ3_S ? 2048 : QT == QT_IQ3_XXS ? 1024 : 0;
   static constexpr int WSZ = WQ + WH + WX + WD;
   static constexpr int FREE = (MM_LDS_MAX - MmT<QT>::SB * TOK - MM_WAVES * WSZ - GRID) / 1024;
   static constexpr int GA = FREE < 12 ? FREE : 12;
@@ -86,11 +88,11 @@ template <int QT> struct MmX { mm_u4 r[MmT<QT>::XB / 16 > 0 ? MmT<QT>::XB / 16 :
 // (Q4_0, IQ4_NL, MXFP4 and IQ4_XS: of each 16-byte block)
 // (IQ3_S: c[b].x the lane's two index bytes of block b, sg the row's eight words of sign bits)
 template <int QT> struct MmSb {
-  mm_u2 c[qt_nib16(QT) || QT == QT_IQ4_XS || QT == QT_IQ3_S || QT == QT_Q3_K ? 8 : MmT<QT>::QB / 32];
+  mm_u2 c[qt_nib16(QT) || QT == QT_IQ4_XS || QT == QT_IQ3_S || QT == QT_Q3_K || QT == QT_IQ3_XXS ? 8 : MmT<QT>::QB / 32];
   mm_u4 h;
   mm_u2 x[2];
   uint32_t d;
-  mm_u4 sg[QT == QT_IQ3_S || QT == QT_Q3_K ? 2 : 1];
+  mm_u4 sg[QT == QT_IQ3_S || QT == QT_Q3_K || QT == QT_IQ3_XXS ? 2 : 1];
 };
 
 // one slice of K, superblocks [s_begin, s_end): at most MmT<QT>::SB of them
@@ -104,9 +106,9 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
   constexpr int QB = TT::QB, NQ = QB / 64, D = TT::D, LPRW = QB / 16, RPI = 64 / LPRW;
   constexpr bool Q45 = QT == QT_Q4_K || QT == QT_Q5_K;
   constexpr bool B16 = qt_nib16(QT) || QT == QT_IQ4_XS;  // a block is 16 bytes: low nibbles values 0..15, high 16..31
-  constexpr int HB = QT == QT_IQ4_XS || QT == QT_MXFP4 ? 8 : QT == QT_IQ3_S || QT == QT_Q3_K ? 12 : 16;  // bytes of a row's superblock in the header plane
-  constexpr bool I3 = QT == QT_IQ3_S || QT == QT_Q3_K;  // (the two types of these plane sizes)
-  constexpr bool K3 = QT == QT_Q3_K;
+  constexpr int HB = QT == QT_IQ3_XXS ? 0 : QT == QT_IQ4_XS || QT == QT_MXFP4 ? 8 : QT == QT_IQ3_S || QT == QT_Q3_K ? 12 : 16;  // bytes of a row's superblock in the header plane
+  constexpr bool I3 = QT == QT_IQ3_S || QT == QT_Q3_K || QT == QT_IQ3_XXS;  // (the types of these plane sizes)
+  constexpr bool K3 = QT == QT_Q3_K, X3 = QT == QT_IQ3_XXS;
   const int tid = threadIdx.x, lane = tid & 63, n16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (a scalar: what follows from it is scalar arithmetic)
   const int nsb = K >> 8, sbs = s_end - s_begin, Ks = sbs * 256, nb = sbs * 8;
@@ -130,6 +132,9 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     o_hdr = planes_q80((size_t)N, nsb).d;
   } else if constexpr (qt_nib16(QT)) {
     o_hdr = planes_q40((size_t)N, nsb).d;  // (MXFP4: its scale bytes, at the same place)
+  } else if constexpr (X3) {
+    const PlanesIQ3XXS pl = planes_iq3xxs((size_t)N, nsb);
+    o_hdr = 0; o_x = pl.ss; o_d = pl.d;  // (no header plane)
   } else if constexpr (I3) {
     const PlanesIQ3S pl = planes_iq3s((size_t)N, nsb);
     o_hdr = pl.hd; o_x = pl.sg; o_d = pl.d;
@@ -166,7 +171,9 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
     const int u = min(ub + g, ulast);
     const int gl = group_of(u), sb = u - gl * sbs;
     const int r = min((gb0 + gl) * 16 + n16, N - 1);
-    if constexpr (HB == 16) {
+    if constexpr (HB == 0) {
+      h = mm_u4{0u, 0u, 0u, 0u};
+    } else if constexpr (HB == 16) {
       h = *(const mm_u4*)(hd + ((size_t)r * nsb + s_begin + sb) * 16);
     } else if constexpr (HB == 12) {
       const uint32_t* hp = (const uint32_t*)(hd + ((size_t)r * nsb + s_begin + sb) * 12);
@@ -369,6 +376,27 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] = fmaf(d, part[i], acc[i]);
+    } else if constexpr (X3) {
+      // block b: indices 2 g and 2 g + 1 of its eight (a byte each) name codebook words of four magnitudes; the signs of
+      // the lane's eight values are the block's sign code g, the scale the top nibble of that word; d / 4
+      // (reference src/quants.h:220-239, zero/kernels/decode.cl:183-478)
+      const uint32_t* grid = (const uint32_t*)(lds + LL::OGRID);
+      const float d3 = 0.25f * f16_bits_to_f32(h.d);
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const uint32_t q16 = h.c[b].x;
+        const uint32_t a = b < 4 ? h.sg[0][b & 3] : h.sg[1][b & 3];
+        const uint32_t s8 = iq3xxs_signs8(a, g);
+        const uint32_t w0 = iq3s_signed4(grid[q16 & 0xFFu], s8 & 0xFu), w1 = iq3s_signed4(grid[(q16 >> 8) & 0xFFu], s8 >> 4);
+        const long wv = (long)(((unsigned long)w1 << 32) | w0);
+        v4i z = {0, 0, 0, 0};
+        const v4i I = __builtin_amdgcn_mfma_i32_16x16x32_i8(av[b], wv, z, 0, 0, 0);
+        const float d = d3 * (float)(1 + 2 * (int)(a >> 28));
+        acc[0] = fmaf((float)I[0], sa4[b].x * d, acc[0]);
+        acc[1] = fmaf((float)I[1], sa4[b].y * d, acc[1]);
+        acc[2] = fmaf((float)I[2], sa4[b].z * d, acc[2]);
+        acc[3] = fmaf((float)I[3], sa4[b].w * d, acc[3]);
+      }
     } else if constexpr (K3) {
       // block b: the lane's eight values 8 g .. 8 g + 7 are the fields 2 g and 2 g + 1 of the block's bit words; the
       // block's two 16-value halves have a scale each, so, as for Q6_K, two products with the other half's lanes zeroed
@@ -608,6 +636,9 @@ __device__ inline void mm_kernel(uint8_t* lds, const uint8_t* __restrict__ raw, 
   const int groups = (N + 15) >> 4, gd = (int)gridDim.x;
   const int ng = (int)((long)(blockIdx.x + 1) * groups / gd) - (int)((long)blockIdx.x * groups / gd);
   float* GA = slices > 1 && ng <= MmL<QT>::GA ? (float*)(lds + SB * MmL<QT>::TOK + MM_WAVES * MmL<QT>::WSZ) : nullptr;
+  if constexpr (QT == QT_IQ3_XXS) {  // (its codebook: the 256 words behind IQ3_S's)
+    for (int i = threadIdx.x; i < 256; i += 512) ((uint32_t*)(lds + MmL<QT>::OGRID))[i] = tabs[512 + i];
+  }
   if constexpr (QT == QT_IQ3_S) {  // (the codebook: the first 512 words of the tables; the first slice's meeting orders it)
     for (int i = threadIdx.x; i < 512; i += 512) ((uint32_t*)(lds + MmL<QT>::OGRID))[i] = tabs[i];
   }
@@ -635,6 +666,7 @@ MM_KERNEL(13)
 MM_KERNEL(14)
 MM_KERNEL(8)
 MM_KERNEL(2)
+MM_KERNEL(18)
 MM_KERNEL(11)
 MM_KERNEL(20)
 MM_KERNEL(39)

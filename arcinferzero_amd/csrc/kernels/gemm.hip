@@ -964,7 +964,9 @@ __device__ __forceinline__ void store_tile64_quant(uint8_t* lds, const v16f (&hv
 
 // TILES: one expert tile -- the planes hold rows_total rows, the expert's N rows start at row_base, slot r of the tile
 // reads token row rowmap[m0 + r] (use_map) and its results are scaled by rowscale[m0 + r] (use_scale).
-template <bool TILES = false>
+// HD: the planes hold half the values (IQ3_XXS written out as Q6_K planes: its magnitudes, up to 62, are even and
+// enter halved, and d / 4, which an f16 cannot always hold, becomes d with half the factor here).
+template <bool TILES = false, bool HD = false>
 __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
                                   int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0,
@@ -1026,7 +1028,7 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
     uint8_t* base = lds + stage * G6_STAGE;
     ((float*)(base + G6_SA))[b_s * 64 + r_s] = tok_valid ? r.sa : 0.0f;
     ((uint32_t*)(base + G6_SC))[(t >> 1) * 2 + p_s] = r.sc;
-    if (p_s == 0) ((float*)(base + G6_D))[t >> 1] = 0.25f * f16_bits_to_f32(r.d);  // (the weights enter as 4 (q - 32))
+    if (p_s == 0) ((float*)(base + G6_D))[t >> 1] = (HD ? 0.125f : 0.25f) * f16_bits_to_f32(r.d);  // (the weights enter as 4 (q - 32))
   };
 
   // ---- operand addresses of this lane (bytes from a stage's start)
@@ -2037,6 +2039,18 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_B
   gemm6_body<false>(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny, s_begin + ns * (y + 1) / ny,
              m0, min(G6_BM, M - m0), n0);
 }
+// (... -DHDS: the planes hold half the values, gemm6_body<..., HD>)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_BN128_SPLITK1_HDS1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
+  gemm6_body<false, true>(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
+                          s_begin + ns * (y + 1) / ny, m0, min(G6_BM, M - m0), n0);
+}
 // (Q5_K, IQ4_XS -DBM=128 -DBN=128 -DSPLITK: the register-staged body's tiles)
 #define GEMM2_SPLITK_INST(QT)                                                                                        \
   extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE##QT##_ACT321_BM128_BN128_SPLITK1(                  \
@@ -2213,6 +2227,27 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321(
   tile_of(blockIdx.x, mt, nt, tm, tn);
   const int m0 = tm * G6_BM, n0 = tn * BN;
   gemm6_body<false>(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
+}
+// (-DHD, -DHDT below: the planes hold half the values, gemm6_body<..., HD>)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_HD1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  gemm6_body<false, true>(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
+}
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_MOE_TILES1_HDT1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
+    int use_map, const float* rowscale, int use_scale, int NE) {
+  int ti, chunk;
+  if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;
+  ti += tstart[e0];
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm6_body<true, true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, r0, min(nr, G6_BM), chunk * BN,
+                         (size_t)NE * N, (size_t)e * N, rowmap, use_map, rowscale, use_scale);
 }
 // (Q6_K experts: the dense kernel's body over tiles of at most 64 slots -- the engine builds the list for that size)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_MOE_TILES1(

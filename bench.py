@@ -171,7 +171,7 @@ def bench_types(az, N=17408, K=5120):
     """Every weight type on the headline matrix: GEMV over 1, 2, 8 and 16 tokens (cycling through distinct weight
     buffers, as bench_decode) and the prefill GEMM at 2048 tokens.  Not part of the default run (--types)."""
     names = {az.Q4_0: "Q4_0", az.Q8_0: "Q8_0", az.Q3_K: "Q3_K", az.Q4_K: "Q4_K", az.Q5_K: "Q5_K", az.Q6_K: "Q6_K",
-             az.IQ4_NL: "IQ4_NL", az.IQ3_S: "IQ3_S", az.IQ4_XS: "IQ4_XS", az.MXFP4: "MXFP4"}
+             az.IQ3_XXS: "IQ3_XXS", az.IQ4_NL: "IQ4_NL", az.IQ3_S: "IQ3_S", az.IQ4_XS: "IQ4_XS", az.MXFP4: "MXFP4"}
     out = {}
     for qt, name in names.items():
         copies = 6

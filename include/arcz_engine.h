@@ -29,11 +29,12 @@ arcz_engine* arcz_engine_create(int max_chunk, int max_k);
 void arcz_engine_destroy(arcz_engine* e);
 
 /* make_weight + upload_padded (zero/engine_load.h:84-130, 157-196): N rows of K values as GGUF blocks of `type`
- * (2 = Q4_0, 8 = Q8_0, 11 = Q3_K, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K, 20 = IQ4_NL, 21 = IQ3_S, 23 = IQ4_XS, 39 = MXFP4),
+ * (2 = Q4_0, 8 = Q8_0, 11 = Q3_K, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K, 18 = IQ3_XXS, 20 = IQ4_NL, 21 = IQ3_S, 23 = IQ4_XS,
+ * 39 = MXFP4),
  * regrouped into the device layout -- every type in its own form, the GGUF byte count -- and uploaded. */
 arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, const void* gguf, size_t bytes);
 /* The same from a tensor of an open GGUF file (upload of zero/engine_load.h:84-196): a matrix (dims K, N) or an expert
- * tensor (dims K, N, experts) of type Q4_0 / Q8_0 / Q3_K / Q4_K / Q5_K / Q6_K / IQ4_NL / IQ3_S / IQ4_XS / MXFP4, by name;
+ * tensor (dims K, N, experts) of type Q4_0 / Q8_0 / Q3_K / Q4_K / Q5_K / Q6_K / IQ3_XXS / IQ4_NL / IQ3_S / IQ4_XS / MXFP4, by name;
  * NULL + arcz_engine_error() when it is missing, of another type or shape.  The MoE layer: its three expert tensors (gate and up [NE][F][E], down [NE][E][F]). */
 arcz_weight* arcz_weight_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* name);
 arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* gate, const char* up,
@@ -171,6 +172,8 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, u
 /* The IQ3_S codebook (ggml's iq3s_grid, src/iq_tables.h:297) as the kernels take it in their `tabs` argument: 512 words,
  * byte j of a word = magnitude j of the entry (1, 3, ..., 15). */
 void arcz_iq3s_grid(uint32_t* out512);
+/* ... and IQ3_XXS's: 256 words (ggml's iq3xxs_grid, the reference's src/iq_tables.h). */
+void arcz_iq3xxs_grid(uint32_t* out256);
 /* quantize_rows_q8_0 (src/quants.h:429-442) and this library's own Q4_K / Q5_K / Q6_K / IQ4_XS / IQ3_S / IQ4_NL / MXFP4 block makers (input generators). */
 int arcz_quantize_rows(uint32_t type, const float* src, size_t N, int K, uint8_t* out);
 void arcz_gen_normal(uint64_t seed, size_t n, float mean, float std, float* out);

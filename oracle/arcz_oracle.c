@@ -17,6 +17,8 @@
  *   orc_act_residual                    PARITY UNPINNED (no reference CPU twin, no vector); identities and bounds only
  *   orc_quantize_rows_q4_0, Q4_0 decode  closed-form blocks; live comparison with the compiled reference header
  *   IQ4_XS decode                       closed-form block; live comparison with the compiled reference header
+ *   IQ3_XXS decode (and its grid table) closed-form block; live comparison with the compiled reference header over every
+ *                                       grid index and on blocks of random bytes
  *   Q3_K decode                         closed-form block; live comparison with the compiled reference header
  *   IQ4_NL, MXFP4 decode                closed-form blocks (every code, every E8M0 exponent); live comparison with the
  *                                       compiled reference header
@@ -58,7 +60,8 @@
 /* one int scale per 16 (Q6_K) or per 32 values (IQ4_XS: the same one for both halves), kept in sc6[], and no mins */
 #define ORC_IQ3_S 21u
 #define ORC_Q3_K 11u /* 3-bit values - 4 with a 6-bit scale - 32 per 16 of them: q[] and sc6[] as the IQ types' */
-#define ORC_IQLIKE(t) ((t) == ORC_IQ4_XS || (t) == ORC_IQ3_S || (t) == ORC_Q3_K) /* q[] holds the signed value itself */
+#define ORC_IQ3_XXS 18u
+#define ORC_IQLIKE(t) ((t) == ORC_IQ4_XS || (t) == ORC_IQ3_S || (t) == ORC_Q3_K || (t) == ORC_IQ3_XXS) /* q[] holds the signed value itself */
 #define ORC_Q6LIKE(t) ((t) == ORC_Q6_K || ORC_IQLIKE(t))
 
 /* ---------------------------------------------------------------- fp16 (src/quants.h:17-52) */
@@ -125,6 +128,7 @@ int orc_sb_bytes(uint32_t type) {
     case ORC_IQ4_XS: return 136;
     case ORC_IQ3_S: return 110;
     case ORC_Q3_K: return 110;
+    case ORC_IQ3_XXS: return 98;
     default: return 0;
   }
 }
@@ -171,6 +175,29 @@ static const char iq3s_codes[] =
 "a51a5aa7aa80a89a93a98a9eaabac2ac7ac8ad7ae4ae9af5afbb01b04b10b1ab26b4ab56b69b6bba2bc2bc4bd2c09c0b"
 "c0dc19c1bc30c40c50c57c74c8ac9cca2cadcb2cb8cc0ccccd1ce0d15d23d32d40d43d5cd70d85da0dc9dcbe00e04e07"
 "e10e12e1ee20e2ce32e42e49e54e63e65e81e84e88e8ee91e98ea9ec2edaeddeebf01f05f0bf10f28f52f62f82f99fc0";
+/* The IQ3_XXS codebook (ggml's iq3xxs_grid, a constant of the GGUF format; the reference carries it in
+ * src/iq_tables.h): 256 entries of four magnitudes out of 4, 12, 20, 28, 36, 44, 52, 62, here three hex digits an
+ * entry, magnitude j its bits 3 j .. 3 j + 2 as an index into that list. */
+static const char iq3xxs_codes[] =
+"00000200400900b00f01001201902203b03d04104304804a05105505805a06106c07808008208408909009209909b09f"
+"0a90af0bd0c10c70c80ca0d50f810b11f12412f13b13d14114715a16a19d1b41c81cc1ce1e31f120120320820a211213"
+"21821a21c22722824024224925025228128328828a2912982ba2c02c22d02d92e62f63013053283503543663793853d2"
+"3e040040240940b41041241641942244144344544844a45145847347747848048248948f49049249f4a04ad4c14c84cc"
+"4f84fc51d52b54355756157c5c15c35ce5e560160860a61161362863563a6406426506596646666816836886956aa6ba"
+"6c96db71872773a74074675276d78c79e7b37db7f080480f81d81f82b82f87c89089f8a08b08b68c78e5904929934955"
+"9639789c59c89ca9d8a0aa21a38a40a46a56a6da8ca9aabaac2aebb08b13b17b3ab42b59ba8bd4be2c14c24c26c34c51"
+"c71c8fcb4cd8cded24d45d6ad9bdc3dd1e03e05e07e08e1ae2ae56e60e8aea5eaaec0ecdedbef0f11f21f40f42f54f98";
+static void iq3xxs_entry(int idx, int out[4]) {
+  int c = 0;
+  for (int k = 0; k < 3; ++k) {
+    const char ch = iq3xxs_codes[3 * idx + k];
+    c = c * 16 + (ch <= '9' ? ch - '0' : ch - 'a' + 10);
+  }
+  for (int j = 0; j < 4; ++j) {
+    const int i = (c >> (3 * j)) & 7;
+    out[j] = i == 7 ? 62 : 4 + 8 * i;
+  }
+}
 static void iq3s_entry(int idx, int out[4]) {
   int c = 0;
   for (int k = 0; k < 3; ++k) {
@@ -264,6 +291,30 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
       const uint8_t* blk = p + 34 * b;
       o->d8[b] = orc_fp16_to_f32(rd16(blk));
       for (int i = 0; i < 32; ++i) o->q[32 * b + i] = (int8_t)blk[2 + i];
+    }
+    return 0;
+  }
+  if (type == ORC_IQ3_XXS) { /* 98 bytes: f16 d, qs[64] (a codebook index per 4 values), then per 32-block a word: four
+                                7-bit sign codes (code l: the signs of values 8 l .. 8 l + 7, the eighth bit the
+                                parity of the seven -- ggml's ksigns_iq2xs) and in the top nibble the scale s;
+                                value = d / 4 * (1 + 2 s) * the signed magnitude (src/quants.h:220-239) */
+    o->d = orc_fp16_to_f32(rd16(p)) / 4;
+    const uint8_t *qs = p + 2, *ss = p + 66;
+    for (int ib = 0; ib < 8; ++ib) {
+      uint32_t a;
+      memcpy(&a, ss + 4 * ib, 4);
+      o->sc6[2 * ib] = o->sc6[2 * ib + 1] = 1 + 2 * (int)(a >> 28);
+      for (int l = 0; l < 4; ++l) {
+        uint32_t sg = (a >> (7 * l)) & 127u, par = sg;
+        par ^= par >> 4; par ^= par >> 2; par ^= par >> 1;
+        sg |= (par & 1u) << 7;
+        for (int h = 0; h < 2; ++h) {
+          int m[4];
+          iq3xxs_entry(qs[8 * ib + 2 * l + h], m);
+          for (int j = 0; j < 4; ++j)
+            o->q[32 * ib + 8 * l + 4 * h + j] = (int16_t)(((sg >> (4 * h + j)) & 1) ? -m[j] : m[j]);
+        }
+      }
     }
     return 0;
   }

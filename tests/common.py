@@ -8,14 +8,17 @@ import oracle_lib as orc
 import os
 
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS, Q4_0, IQ3_S = az.Q8_0, az.Q4_K, az.Q5_K, az.Q6_K, az.IQ4_XS, az.Q4_0, az.IQ3_S
-IQ4_NL, MXFP4, Q3_K = az.IQ4_NL, az.MXFP4, az.Q3_K
+IQ4_NL, MXFP4, Q3_K, IQ3_XXS = az.IQ4_NL, az.MXFP4, az.Q3_K, az.IQ3_XXS
 TYPES = (Q8_0, Q4_K, Q6_K, Q5_K, IQ4_XS)
-ALL_TYPES = TYPES + (Q4_0, IQ3_S, IQ4_NL, MXFP4, Q3_K)     # with the types the golden files of the first five do not cover
+ALL_TYPES = TYPES + (Q4_0, IQ3_S, IQ4_NL, MXFP4, Q3_K, IQ3_XXS)     # with the types the golden files of the first five do not cover
 # the IQ3_S codebook as the compiled reference decodes it (a golden vector): 512 entries of four magnitudes
 IQ3S_GRID = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors_types2.npz"))[
     "iq3s_grid_dequant"].reshape(512, 4).astype(np.int64)
 TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS", az.IQ3_S: "IQ3_S", az.Q4_0: "Q4_0",
-              az.IQ4_NL: "IQ4_NL", az.MXFP4: "MXFP4", az.Q3_K: "Q3_K"}
+              az.IQ4_NL: "IQ4_NL", az.MXFP4: "MXFP4", az.Q3_K: "Q3_K", az.IQ3_XXS: "IQ3_XXS"}
+# ... and the IQ3_XXS codebook likewise: 256 entries of four magnitudes
+IQ3XXS_GRID = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors_types3.npz"))[
+    "iq3xxs_grid_dequant"].reshape(256, 4).astype(np.int64)
 IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64)
 MXFP4_VALUES = np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.int64)   # (src/quants.h:497)
 
@@ -98,6 +101,23 @@ def unit_scale_weights(qtype, N, K, seed):
         blk[..., 0:2] = one
         blk[..., 2:] = (q[..., :16] | (q[..., 16:] << 4)).astype(np.uint8)
         return blk.reshape(-1), (q - 8).reshape(N, K)
+    if qtype == IQ3_XXS:
+        # d = 4 (d / 4 = 1), every scale nibble 0 (1 + 2 s = 1): values = the codebook's magnitudes with the signs of
+        # random 7-bit codes, the eighth sign their parity
+        idx = rng.integers(0, 256, size=(N, nsb, 8, 8), dtype=np.int64)            # [block][group of 4]
+        code = rng.integers(0, 128, size=(N, nsb, 8, 4), dtype=np.int64)           # [block][group of 8]
+        par = np.zeros_like(code)
+        for k in range(7):
+            par ^= (code >> k) & 1
+        sg8 = code | (par << 7)
+        sg = ((sg8[..., None] >> np.arange(8)) & 1).reshape(N, nsb, 8, 32)         # sign bit per value
+        blk = np.zeros((N, nsb, 98), np.uint8)
+        blk[..., 0:2] = np.frombuffer(np.float16(4.0).tobytes(), np.uint8)
+        blk[..., 2:66] = idx.astype(np.uint8).reshape(N, nsb, 64)
+        words = (code << (7 * np.arange(4))).sum(axis=-1).astype(np.uint32)        # [N][nsb][8]
+        blk[..., 66:98] = words.view(np.uint8).reshape(N, nsb, 32)
+        vals = IQ3XXS_GRID[idx].reshape(N, nsb, 8, 32) * (1 - 2 * sg)
+        return blk.reshape(-1), vals.reshape(N, K)
     if qtype == Q3_K:
         # d = 1, every 6-bit scale 33 (- 32 = 1): low nibbles 1, high two bits 2; values = the three bits - 4
         q = rng.integers(0, 8, size=(N, nsb, 8, 32), dtype=np.int64)               # [block][element]

@@ -1,5 +1,5 @@
 """gemv_mm: the matrix-vector form for a few tokens on the matrix pipe (Q4_K, Q5_K, Q6_K, Q8_0, Q4_0,
-IQ4_XS, IQ3_S, IQ4_NL, MXFP4, Q3_K).  The engine takes it for 9-16 tokens in a
+IQ4_XS, IQ3_S, IQ4_NL, MXFP4, Q3_K, IQ3_XXS).  The engine takes it for 9-16 tokens in a
 16-row chunk, for 5-8 tokens, and for 3-4 tokens whose activations do not fit the LDS of the dot-product kernels; every
 case here lands on it.  Against the double-accumulated dequantized reference (1e-3 as max|err| / max|ref| per token
 row), with unit scales against the exact integer sums, with K in one slice and in several (later slices accumulate),
@@ -71,7 +71,7 @@ CASES_TYPES = [(8, 100, 256), (16, 333, 2048), (13, 1000, 5120), (7, 129, 17408)
 
 
 @pytest.mark.parametrize("T,N,K", CASES_TYPES)
-@pytest.mark.parametrize("qt", [az.Q5_K, az.Q6_K, az.Q8_0, az.Q4_0, az.IQ4_XS, az.IQ3_S, az.IQ4_NL, az.MXFP4, az.Q3_K])
+@pytest.mark.parametrize("qt", [az.Q5_K, az.Q6_K, az.Q8_0, az.Q4_0, az.IQ4_XS, az.IQ3_S, az.IQ4_NL, az.MXFP4, az.Q3_K, az.IQ3_XXS])
 def test_gemv_mm_parity_types(eng, qt, T, N, K):
     _parity(eng, qt, T, N, K)
 
@@ -109,7 +109,7 @@ def test_gemv_mm_into_a_wider_output(eng, qt, T, N, K):
 
 
 @pytest.mark.parametrize("T,N,K", [(8, 48, 512), (16, 37, 7168)])
-@pytest.mark.parametrize("qt", [az.Q4_K, az.Q5_K, az.Q6_K, az.Q4_0, az.IQ4_XS, az.IQ3_S, az.IQ4_NL, az.MXFP4, az.Q3_K])
+@pytest.mark.parametrize("qt", [az.Q4_K, az.Q5_K, az.Q6_K, az.Q4_0, az.IQ4_XS, az.IQ3_S, az.IQ4_NL, az.MXFP4, az.Q3_K, az.IQ3_XXS])
 def test_gemv_mm_unit_scales_exact(eng, qt, T, N, K):
     """All scales 1: the f32 output is the exact integer sum (partial sums stay below 2^24)."""
     W, wi = unit_scale_weights(qt, N, K, seed=820)

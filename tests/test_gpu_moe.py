@@ -86,7 +86,9 @@ def test_routing_and_sort(rt, NE, NU, T, tm):
                                                    # IQ4_NL and MXFP4 experts: small passes and tile passes
                                                    (az.IQ4_NL, 4, 2, 256, 512, 1, 16), (az.IQ4_NL, 4, 2, 256, 512, 150, 160),
                                                    (az.MXFP4, 4, 2, 256, 512, 4, 16), (az.MXFP4, 6, 2, 512, 256, 40, 48),
-                                                   # Q3_K experts (uploaded as Q6_K planes)
+                                                   # IQ3_XXS experts
+                                                   (az.IQ3_XXS, 4, 2, 256, 512, 2, 16), (az.IQ3_XXS, 6, 2, 512, 256, 40, 48),
+                                                   # Q3_K experts
                                                    (az.Q3_K, 4, 2, 256, 512, 3, 16), (az.Q3_K, 6, 2, 512, 256, 70, 80),
                                                    # IQ3_S experts (uploaded as Q6_K planes): one token and a tile pass
                                                    (az.IQ3_S, 4, 2, 256, 512, 1, 16), (az.IQ3_S, 6, 2, 512, 256, 40, 48),

@@ -1,4 +1,4 @@
-"""Seeded random cases over everything a matmul call can vary at once: the ten weight types, 1 to 2047 tokens in
+"""Seeded random cases over everything a matmul call can vary at once: the eleven weight types, 1 to 2047 tokens in
 chunks with and without an empty group of 16 rows, 1 to 40000 weight rows, K of 1 to 68 superblocks, an output wider
 than the matrix (ldc > N) at a column offset, the three epilogues (store, add to C, SwiGLU on the gate in C), per-32
 and per-256 activation scales.  Each case against the double-accumulated dequantized reference (1e-3), the columns of

@@ -99,6 +99,11 @@ def test_repack_planes_layout(qtype):
         sb = W.reshape(u, 136)
         assert np.array_equal(P[:u * 128].reshape(u, 128), sb[:, 8:]) and np.array_equal(P[u * 128:u * 136].reshape(u, 8), sb[:, :8])
         assert not P[u * 136:].any() and P.size % 16 == 0
+    elif qtype == az.IQ3_XXS:
+        sb = W.reshape(u, 98)                                                # d, 64 index bytes, 8 words of sign codes and scales
+        assert P.size == (W.size + 15) // 16 * 16
+        assert np.array_equal(P[:u * 64].reshape(u, 64), sb[:, 2:66]) and np.array_equal(P[u * 64:u * 96].reshape(u, 32), sb[:, 66:98])
+        assert np.array_equal(P[u * 96:u * 98].reshape(u, 2), sb[:, :2]) and not P[u * 98:].any()
     elif qtype == az.Q3_K:
         # a block's bits together: words D0, D1 of bit pairs (value j of a half in byte j % 4, bits 2 (j / 4)), a word of
         # third bits (value j at bit 8 (j % 4) + j / 4), eight 12-bit header entries of two 6-bit scales, d; put back
@@ -147,7 +152,7 @@ def test_q8_0_quantizer_is_the_reference_one():
 
 
 @pytest.mark.parametrize("qtype,rel", [(az.Q4_K, 0.08), (az.Q5_K, 0.04), (az.Q6_K, 0.02), (az.Q8_0, 0.006), (az.IQ4_XS, 0.09),
-                                       (az.IQ4_NL, 0.10), (az.MXFP4, 0.15), (az.Q3_K, 0.25)])
+                                       (az.IQ4_NL, 0.10), (az.MXFP4, 0.15), (az.Q3_K, 0.25), (az.IQ3_XXS, 0.25)])
 def test_block_makers_make_valid_close_blocks(qtype, rel):
     """The Q4_K / Q5_K / Q6_K block makers are input generators (the reference has none): valid fields and a round-trip
     error of the size the bit width allows."""

@@ -14,6 +14,7 @@ from common import TYPES, make_acts, make_weights, rel_err_rows, unit_scale_acts
 
 G = dict(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz")))
 G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_types2.npz")))
+G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_types3.npz")))
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = 8, 12, 13, 14, 23
 NAMES = {Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k", Q8_0: "q80", IQ4_XS: "iq4xs"}
 
@@ -365,6 +366,50 @@ def test_iq4_nl_and_mxfp4_closed_form():
     assert np.array_equal(isc, np.ones(16)) and not imn.any() and not dmin.any()
     assert np.array_equal(d, [_e8m0_half(b) for b in range(8)])
     assert np.array_equal(q.reshape(8, 32)[:, :16], MXFP4_VALUES[blk[:8, 1:] & 15])
+
+
+@pytest.mark.parametrize("name,qtype", [("q3k", az.Q3_K), ("iq3xxs", az.IQ3_XXS), ("iq4nl", az.IQ4_NL), ("mxfp4", az.MXFP4)])
+def test_further_types_golden(name, qtype):
+    """The compiled reference's decode of blocks of random bytes (tests/golden/ref_vectors_types3.npz), bit for bit."""
+    got = orc.dequant_rows(qtype, G[name + "_raw"], 4, 512)
+    assert np.array_equal(got.view(np.uint32), G[name + "_dequant"].view(np.uint32))
+
+
+def test_iq3xxs_closed_form_and_whole_codebook():
+    """IQ3_XXS (src/quants.h:220-239): groups of four magnitudes by 8-bit codebook index, the signs of 8 values as a
+    7-bit code whose parity is the eighth, the scale in the top nibble of the block's word; value = d / 4 * (1 + 2 s) *
+    the signed magnitude.  A block made by hand from codebook entries written out here; then blocks that name entries
+    0..255 in order with d / 4 = 1, scale 1 and no signs (golden): every entry of the codebook, and the product's own
+    copy of it as its kernels take it."""
+    known = {0: (4, 4, 4, 4), 1: (20, 4, 4, 4), 2: (36, 4, 4, 4), 3: (12, 12, 4, 4), 255: (4, 28, 52, 62)}
+    idxs = list(known)
+    K = 256
+    blk = np.zeros(98, np.uint8)
+    d = 0.5
+    blk[0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+    sn = [0, 15, 7, 8, 1, 14, 3, 12]
+    exp = np.zeros(K, np.float32)
+    for b in range(8):
+        a = sn[b] << 28
+        for l in range(4):
+            code = (37 * b + 11 * l + 5) % 128
+            a |= code << (7 * l)
+            sg = code | ((bin(code).count("1") & 1) << 7)
+            for h in range(2):
+                idx = idxs[(3 * b + 2 * l + h) % len(idxs)]
+                blk[2 + 8 * b + 2 * l + h] = idx
+                for j in range(4):
+                    neg = (sg >> (4 * h + j)) & 1
+                    exp[32 * b + 8 * l + 4 * h + j] = np.float32(d / 4) * np.float32(1 + 2 * sn[b]) * np.float32(-known[idx][j] if neg else known[idx][j])
+        blk[66 + 4 * b:70 + 4 * b] = np.frombuffer(np.uint32(a).tobytes(), np.uint8)
+    assert np.array_equal(orc.dequant_rows(az.IQ3_XXS, blk, 1, K)[0], exp)
+    got = orc.dequant_rows(az.IQ3_XXS, G["iq3xxs_grid_raw"], 1, 1024)
+    assert np.array_equal(got, G["iq3xxs_grid_dequant"])
+    v = got.reshape(256, 4)
+    assert set(np.unique(v)) == {4.0, 12.0, 20.0, 28.0, 36.0, 44.0, 52.0, 62.0} and len({tuple(r) for r in v}) == 256
+    grid = np.zeros(256, np.uint32)
+    az.lib.arcz_iq3xxs_grid(grid.ctypes.data_as(C.c_void_p))
+    assert np.array_equal(grid.view(np.uint8).reshape(256, 4), v.astype(np.uint8))
 
 
 def test_q3_k_closed_form():
