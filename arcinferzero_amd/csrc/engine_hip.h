@@ -41,8 +41,9 @@ struct GpuWeight {
   // > 0: this matrix is the output head of a model with final-logit soft-capping (the reference's lm_head_ with
   // hp.softcap, zero/engine.h:984-990): the GEMVs (1-8 tokens) write c * tanh(v / c)
   float softcap = 0.0f;
-  // the planes hold half the values (IQ3_XXS written out as Q6_K planes for the GEMM forms): the kernels' -DHD forms
-  bool half_d = false;
+  // Q6_K planes written out from a type with one scale per 32 values, for the GEMM forms (the kernels' -DHD forms):
+  // 2 = the two sub-scales of a block are equal (IQ3_S), 1 = moreover the planes hold half the values (IQ3_XXS)
+  int half_d = 0;
 };
 
 inline const char* ggml_type_name(uint32_t t) {
@@ -97,7 +98,7 @@ class Engine {
     run(name, k, 1, &g1, &l1);
     GpuWeight x = w;
     x.type = GGML_Q6_K;
-    x.half_d = w.type == GGML_IQ3_XXS;
+    x.half_d = w.type == GGML_IQ3_XXS ? 1 : w.type == GGML_IQ3_S ? 2 : 0;
     x.raw = xw_;
     return x;
   }
@@ -725,7 +726,7 @@ class Engine {
           ws = sk_ws_;
         }
         cl_kernel k = kernel("gemm", std::string("-DQTYPE=") + std::to_string(w.type) + " -DACT32 -DBM=" + std::to_string(bm) +
-                                         " -DBN=128 -DSPLITK" + (w.half_d ? " -DHDS" : ""), "gemm");
+                                         " -DBN=128 -DSPLITK" + (w.half_d ? " -DHDS=" + std::to_string(w.half_d) : std::string()), "gemm");
         cl_mem unused = nullptr;
         int zero = 0, one = 1, ldw = N, s1 = nsb;
         set_args(k, 0, w.raw, unused, aq_, asc_, absum_, ws, M, N, K, ldw, zero, zero, one, zero, s1);
@@ -808,10 +809,10 @@ class Engine {
     }
   }
   // (zero/engine_setup.h:384-420 gemm_kernel / moe_gemm_kernel)
-  cl_kernel gemm_kernel(uint32_t qtype, bool tiles, int ne = 0, bool half_d = false) {
+  cl_kernel gemm_kernel(uint32_t qtype, bool tiles, int ne = 0, int half_d = 0) {
     std::string defs = "-DQTYPE=" + std::to_string(qtype) + " -DACT32";
     if (tiles) defs += " -DMOE_TILES -DNE=" + std::to_string(ne);
-    if (half_d) defs += tiles ? " -DHDT" : " -DHD";
+    if (half_d) defs += (tiles ? " -DHDT=" : " -DHD=") + std::to_string(half_d);
     return kernel("gemm", defs, "gemm");
   }
 

@@ -60,7 +60,7 @@ static const KernelSpec kKernelTable[] = {
     {"decode", "gemv_v", nullptr, "piippppipii", {"QT", "GROWS", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt_v", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     // ---- gemm
-    // (-DHDT / -DHDS / -DHD: the Q6_K kernels on planes that hold half the values -- IQ3_XXS written out as Q6_K)
+    // (-DHDT / -DHDS / -DHD = 1 or 2: the Q6_K kernels on planes written out from IQ3_XXS or IQ3_S)
     {"gemm", "gemm", "HDT", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", "HDT", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm", "HDS", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", "HDS", nullptr}, {{nullptr, 0, false}}, 256},

@@ -964,15 +964,19 @@ __device__ __forceinline__ void store_tile64_quant(uint8_t* lds, const v16f (&hv
 
 // TILES: one expert tile -- the planes hold rows_total rows, the expert's N rows start at row_base, slot r of the tile
 // reads token row rowmap[m0 + r] (use_map) and its results are scaled by rowscale[m0 + r] (use_scale).
-// HD: the planes hold half the values (IQ3_XXS written out as Q6_K planes: its magnitudes, up to 62, are even and
-// enter halved, and d / 4, which an f16 cannot always hold, becomes d with half the factor here).
-template <bool TILES = false, bool HD = false>
+// HD != 0: planes written out from a type with one scale per 32 values (IQ3_S, IQ3_XXS), so a block's two int8 sub-scales
+// are equal: one product per block over all 32 values instead of two over 16, and sc * I in the place of
+// sc0 * I0 + sc1 * I1.  HD == 1: the planes moreover hold half the values (IQ3_XXS: its magnitudes, up to 62, are even
+// and enter halved, and d / 4, which an f16 cannot always hold, becomes d with half the factor here).
+template <bool TILES = false, int HD = 0>
 __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, float* __restrict__ C, int M, int N, int K, int ldc,
                                   int c_off, int accumulate, int s_begin, int s_end, int m0, int rows_valid, int n0,
                                   size_t rows_total = 0, size_t row_base = 0, const int* __restrict__ rowmap = nullptr,
                                   int use_map = 0, const float* __restrict__ rowscale = nullptr, int use_scale = 0) {
-  __shared__ alignas(16) uint8_t lds[2 * G6_STAGE];
+  // (HD != 0: in the place of d and the sub-scale bytes, 1.5 KiB, the four blocks' f32 row scales d * sc: 2 KiB)
+  constexpr int STAGE = HD != 0 ? G6_D + 2048 : G6_STAGE;
+  __shared__ alignas(16) uint8_t lds[2 * STAGE];
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // (a scalar: what follows from it alone is scalar arithmetic)
   const int l32 = lane & 31, g = lane >> 5;
@@ -1008,7 +1012,7 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
 
   auto dma_step = [&](int st, int stage) {
-    uint8_t* base = lds + stage * G6_STAGE;
+    uint8_t* base = lds + stage * STAGE;
     const signed char* ab = abase + (size_t)st * 128;
     const uint8_t* lb = lbase + (size_t)st * 64;
     const uint8_t* hb = hbase + (size_t)st * 32;
@@ -1025,10 +1029,17 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
     r.d = *(const unsigned short*)(raw + pl.d + ((row_base + n_s) * nsb + sb) * 2);
   };
   auto store_scales = [&](const G6ScaleRegs& r, int stage) {
-    uint8_t* base = lds + stage * G6_STAGE;
+    uint8_t* base = lds + stage * STAGE;
     ((float*)(base + G6_SA))[b_s * 64 + r_s] = tok_valid ? r.sa : 0.0f;
-    ((uint32_t*)(base + G6_SC))[(t >> 1) * 2 + p_s] = r.sc;
-    if (p_s == 0) ((float*)(base + G6_D))[t >> 1] = (HD ? 0.125f : 0.25f) * f16_bits_to_f32(r.d);  // (the weights enter as 4 (q - 32))
+    if constexpr (HD != 0) {
+      // blocks 2 p_s and 2 p_s + 1 of the step: their scale (the first of the two equal sub-scale bytes) times d
+      const float dq = (HD == 1 ? 0.125f : 0.25f) * f16_bits_to_f32(r.d);  // (the weights enter as 4 (q - 32))
+      ((float*)(base + G6_D))[(2 * p_s) * 128 + (t >> 1)] = dq * (float)(int)(signed char)(r.sc & 0xFFu);
+      ((float*)(base + G6_D))[(2 * p_s + 1) * 128 + (t >> 1)] = dq * (float)(int)(signed char)((r.sc >> 16) & 0xFFu);
+    } else {
+      ((uint32_t*)(base + G6_SC))[(t >> 1) * 2 + p_s] = r.sc;
+      if (p_s == 0) ((float*)(base + G6_D))[t >> 1] = 0.25f * f16_bits_to_f32(r.d);  // (the weights enter as 4 (q - 32))
+    }
   };
 
   // ---- operand addresses of this lane (bytes from a stage's start)
@@ -1058,7 +1069,7 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
 
 #pragma unroll 1
   for (int st = 0; st < steps; ++st) {
-    const uint8_t* Sb = lds + (st & 1) * G6_STAGE;
+    const uint8_t* Sb = lds + (st & 1) * STAGE;
     const bool next = st + 1 < steps;
     if (next) {
       dma_step(st + 1, (st + 1) & 1);
@@ -1066,16 +1077,21 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
     }
     // raw weights of the lane's row for the whole step: low nibbles of blocks (0, 2) and (1, 3), high bits of all four
     const v4i ql0 = *(const v4i*)(Sb + ol[0]), ql1 = *(const v4i*)(Sb + ol[1]), qh = *(const v4i*)(Sb + oh);
-    const uint2 scw = *(const uint2*)(Sb + G6_SC + (wave * 32 + l32) * 8);
-    const float dop = ((const float*)(Sb + G6_D))[wave * 32 + l32];
+    uint2 scw = {0u, 0u};
+    float dop = 0.0f;
+    if constexpr (HD == 0) {
+      scw = *(const uint2*)(Sb + G6_SC + (wave * 32 + l32) * 8);
+      dop = ((const float*)(Sb + G6_D))[wave * 32 + l32];
+    }
     v4i a16[2][2], w0[2], w1[2];  // [buffer][ms]; [buffer]
-    float saop[2];
+    float saop[2], wsop[2];
     v32f P[2];
     v16i I0[2], I1[2];
     auto ld_a = [&](int b, int buf) {
       a16[buf][0] = *(const v4i*)(Sb + oa[b]);
       a16[buf][1] = *(const v4i*)(Sb + oa[b] + 32 * 128);
       saop[buf] = ((const float*)(Sb + G6_SA))[b * 64 + lane];
+      wsop[buf] = HD != 0 ? ((const float*)(Sb + G6_D))[b * 128 + wave * 32 + l32] : dop;  // (HD: the block's row scale)
     };
     auto dec_w = [&](int b, int buf) {
 #pragma unroll
@@ -1084,22 +1100,26 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
         const uint32_t nib = (b >> 1) ? (lw >> 2) & 0x3C3C3C3Cu : (lw << 2) & 0x3C3C3C3Cu;
         const uint32_t top = b == 3 ? hw & 0xC0C0C0C0u : (hw << (6 - 2 * b)) & 0xC0C0C0C0u;
         const uint32_t w = (nib | top) ^ 0x80808080u;
-        w0[buf][i] = (int)(w & keep0);
-        w1[buf][i] = (int)(w & keep1);
+        if constexpr (HD != 0) {
+          w0[buf][i] = (int)w;
+        } else {
+          w0[buf][i] = (int)(w & keep0);
+          w1[buf][i] = (int)(w & keep1);
+        }
       }
     };
     auto mfma_p = [&](int buf) {
       v32f zf;
 #pragma unroll
       for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
-      P[buf] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[buf], dop, zf, 0, 0, 0);
+      P[buf] = __builtin_amdgcn_mfma_f32_32x32x1f32(saop[buf], wsop[buf], zf, 0, 0, 0);
     };
     auto mfma_i = [&](int buf, int ms, int slot) {
       v16i z;
 #pragma unroll
       for (int i = 0; i < 16; ++i) z[i] = 0;
       I0[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[buf][ms], w0[buf], z, 0, 0, 0);
-      I1[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[buf][ms], w1[buf], z, 0, 0, 0);
+      if constexpr (HD == 0) I1[slot] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[buf][ms], w1[buf], z, 0, 0, 0);
     };
     ld_a(0, 0);
     dec_w(0, 0);
@@ -1125,7 +1145,7 @@ __device__ __forceinline__ void gemm6_body(const uint8_t* __restrict__ raw, cons
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int j = __mul24(sc0, I0[slot][i]) + __mul24(sc1, I1[slot][i]);
+          const int j = HD != 0 ? I0[slot][i] : __mul24(sc0, I0[slot][i]) + __mul24(sc1, I1[slot][i]);
           res[ms][i] = __builtin_fmaf((float)j, P[buf][16 * ms + i], res[ms][i]);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -2039,18 +2059,21 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_B
   gemm6_body<false>(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny, s_begin + ns * (y + 1) / ny,
              m0, min(G6_BM, M - m0), n0);
 }
-// (... -DHDS: the planes hold half the values, gemm6_body<..., HD>)
-extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_BN128_SPLITK1_HDS1(
-    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
-    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
-  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
-  int tm, tn;
-  tile_of(blockIdx.x, mt, nt, tm, tn);
-  const int m0 = tm * G6_BM, n0 = tn * BN;
-  const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;
-  gemm6_body<false, true>(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,
-                          s_begin + ns * (y + 1) / ny, m0, min(G6_BM, M - m0), n0);
-}
+// (... -DHDS=1 / 2: planes written out from IQ3_XXS / IQ3_S, gemm6_body<..., HD>)
+#define GEMM6_HDS_INST(HDV)                                                                                          \
+  extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_BM64_BN128_SPLITK1_HDS##HDV(               \
+      const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum,      \
+      float* C, int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {        \
+    const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;                                                   \
+    int tm, tn;                                                                                                       \
+    tile_of(blockIdx.x, mt, nt, tm, tn);                                                                              \
+    const int m0 = tm * G6_BM, n0 = tn * BN;                                                                          \
+    const int ns = s_end - s_begin, y = blockIdx.y, ny = gridDim.y;                                                   \
+    gemm6_body<false, HDV>(raw, aq, asc, C + (size_t)y * M * ldc, M, N, K, ldc, 0, 0, s_begin + ns * y / ny,           \
+                           s_begin + ns * (y + 1) / ny, m0, min(G6_BM, M - m0), n0);                                   \
+  }
+GEMM6_HDS_INST(1)
+GEMM6_HDS_INST(2)
 // (Q5_K, IQ4_XS -DBM=128 -DBN=128 -DSPLITK: the register-staged body's tiles)
 #define GEMM2_SPLITK_INST(QT)                                                                                        \
   extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE##QT##_ACT321_BM128_BN128_SPLITK1(                  \
@@ -2228,27 +2251,31 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321(
   const int m0 = tm * G6_BM, n0 = tn * BN;
   gemm6_body<false>(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
 }
-// (-DHD, -DHDT below: the planes hold half the values, gemm6_body<..., HD>)
-extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_HD1(
-    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
-    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
-  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
-  int tm, tn;
-  tile_of(blockIdx.x, mt, nt, tm, tn);
-  const int m0 = tm * G6_BM, n0 = tn * BN;
-  gemm6_body<false, true>(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0), n0);
-}
-extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_MOE_TILES1_HDT1(
-    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
-    int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
-    int use_map, const float* rowscale, int use_scale, int NE) {
-  int ti, chunk;
-  if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;
-  ti += tstart[e0];
-  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-  gemm6_body<true, true>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, r0, min(nr, G6_BM), chunk * BN,
-                         (size_t)NE * N, (size_t)e * N, rowmap, use_map, rowscale, use_scale);
-}
+// (-DHD=1 / 2, -DHDT=1 / 2: planes written out from IQ3_XXS / IQ3_S, gemm6_body<..., HD>)
+#define GEMM6_HD_INST(HDV)                                                                                           \
+  extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_HD##HDV(                                   \
+      const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum,      \
+      float* C, int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {        \
+    const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;                                                   \
+    int tm, tn;                                                                                                       \
+    tile_of(blockIdx.x, mt, nt, tm, tn);                                                                              \
+    const int m0 = tm * G6_BM, n0 = tn * BN;                                                                          \
+    gemm6_body<false, HDV>(raw, aq, asc, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, m0, min(G6_BM, M - m0),   \
+                           n0);                                                                                       \
+  }                                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_MOE_TILES1_HDT##HDV(                       \
+      const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum,      \
+      float* C, int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1,    \
+      const int* rowmap, int use_map, const float* rowscale, int use_scale, int NE) {                                 \
+    int ti, chunk;                                                                                                    \
+    if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;                                          \
+    ti += tstart[e0];                                                                                                 \
+    const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];                                  \
+    gemm6_body<true, HDV>(raw, aq, asc, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, r0, min(nr, G6_BM), chunk * BN,     \
+                          (size_t)NE * N, (size_t)e * N, rowmap, use_map, rowscale, use_scale);                       \
+  }
+GEMM6_HD_INST(1)
+GEMM6_HD_INST(2)
 // (Q6_K experts: the dense kernel's body over tiles of at most 64 slots -- the engine builds the list for that size)
 extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE14_ACT321_MOE_TILES1(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
