@@ -83,6 +83,7 @@ _sig("arcz_ggml_block_info", _i, _u32, C.POINTER(_i), C.POINTER(_i))
 _sig("arcz_weight_free", _i, _p, _p)
 _sig("arcz_weight_raw", _p, _p)
 _sig("arcz_weight_k", C.c_int, _p)
+_sig("arcz_moe_layer_dims", C.c_int, _p, C.POINTER(C.c_int), C.POINTER(C.c_int))
 _sig("arcz_engine_quantize", _i, _p, _p, _i, _i, _i, _i, _i)
 _sig("arcz_engine_rmsnorm_quant", _i, _p, _p, _i, _p, _i, _i, _i, _i, C.c_float, _p)
 _sig("arcz_engine_add_norm_quant", _i, _p, _p, _p, _p, _i, _i, _i, C.c_float, _p, _i, _i, C.c_float)
@@ -423,7 +424,9 @@ class Engine:
         if not h:
             raise ArczError(-100, lib.arcz_engine_error().decode())
         t = gguf.tensor(gguf.find(gate))
-        return MoeLayer(self, h, t["dims"][2], NU, t["dims"][0], t["dims"][1])
+        Ep, Fp = C.c_int(), C.c_int()
+        lib.arcz_moe_layer_dims(h, C.byref(Ep), C.byref(Fp))
+        return MoeLayer(self, h, t["dims"][2], NU, Ep.value, Fp.value)
 
     def quantize(self, x, ldx, K, Mp, T, act32=1):
         _check(lib.arcz_engine_quantize(self.h, x.h, ldx, K, Mp, T, act32), engine=True)
@@ -489,11 +492,14 @@ class Engine:
 
     def make_moe_layer(self, qtype, gate, up, down, NE, NU, E, F):
         g, u, d = (np.ascontiguousarray(a, dtype=np.uint8) for a in (gate, up, down))
-        assert g.size == gguf_bytes(qtype, NE * F, E) and u.size == g.size and d.size == gguf_bytes(qtype, NE * E, F)
+        if E % 256 == 0 and F % 256 == 0:
+            assert g.size == gguf_bytes(qtype, NE * F, E) and u.size == g.size and d.size == gguf_bytes(qtype, NE * E, F)
         h = lib.arcz_moe_layer_upload(self.h, qtype, _np_ptr(g), _np_ptr(u), _np_ptr(d), NE, NU, E, F)
         if not h:
             raise ArczError(-100, lib.arcz_engine_error().decode())
-        return MoeLayer(self, h, NE, NU, E, F)
+        Ep, Fp = C.c_int(), C.c_int()
+        lib.arcz_moe_layer_dims(h, C.byref(Ep), C.byref(Fp))       # (E and F rounded up where the tensors were padded)
+        return MoeLayer(self, h, NE, NU, Ep.value, Fp.value)
 
     def layer_moe(self, L, logits, ldl, x, T, Mp, sh=None):
         if sh is None:

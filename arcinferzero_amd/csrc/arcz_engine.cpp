@@ -87,13 +87,26 @@ arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, c
         if (dims[0] > (1u << 30) || dims[1] > (1u << 30) || dims[2] > 65536)  // (before they become ints)
           throw std::runtime_error(std::string("tensor ") + gate + ": dimensions out of range");
         const int Ed = (int)dims[0], F = (int)dims[1], NE = (int)dims[2];
-        E.moe_alloc(NE, NU, Ed, F);
-        L->L.NE = NE; L->L.NU = NU; L->L.E = Ed; L->L.F = F;
-        L->L.ex[0] = weight_from_gguf(E, g, gate, &ne[0]);
-        L->L.ex[1] = weight_from_gguf(E, g, up, &ne[1]);
-        L->L.ex[2] = weight_from_gguf(E, g, down, &ne[2]);
-        if (ne[1] != NE || ne[2] != NE || L->L.ex[1].N != F || L->L.ex[1].K != Ed || L->L.ex[2].N != Ed || L->L.ex[2].K != F)
-          throw std::runtime_error("the expert tensors' shapes do not belong to one layer");
+        // the three tensors as they lie in the file: shapes checked here, rows and columns padded in make_moe_layer
+        uint32_t types[3];
+        const uint8_t* data[3];
+        const char* names[3] = {gate, up, down};
+        for (int i = 0; i < 3; ++i) {
+          const long it = arcz_gguf_find(g, names[i]);
+          if (it < 0) throw std::runtime_error(std::string("missing tensor ") + names[i]);
+          uint32_t ndi = 0;
+          uint64_t di[8], nb = 0;
+          const void* p = nullptr;
+          arcz_gguf_tensor(g, (size_t)it, nullptr, &types[i], &ndi, di, &p, &nb);
+          const uint64_t k = i == 2 ? (uint64_t)F : (uint64_t)Ed, n = i == 2 ? (uint64_t)Ed : (uint64_t)F;
+          if (ndi != 3 || di[0] != k || di[1] != n || di[2] != (uint64_t)NE)
+            throw std::runtime_error("the expert tensors' shapes do not belong to one layer");
+          int blk = 0, bytes = 0;
+          if (!arcz_ggml_block_info(types[i], &blk, &bytes) || k % (uint64_t)blk || nb != (uint64_t)NE * n * (k / (uint64_t)blk) * (uint64_t)bytes)
+            throw std::runtime_error(std::string("tensor ") + names[i] + ": its bytes do not match its shape");
+          data[i] = (const uint8_t*)p;
+        }
+        L->L = E.make_moe_layer(types, data, NE, NU, Ed, F);
       }) != ARCZ_OK) {
     delete L;
     return nullptr;
@@ -182,6 +195,12 @@ arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void*
     return nullptr;
   }
   return L;
+}
+int arcz_moe_layer_dims(const arcz_moe_layer* L, int* E, int* F) {
+  if (!L) return ARCZ_E_ENGINE;
+  if (E) *E = L->L.E;
+  if (F) *F = L->L.F;
+  return ARCZ_OK;
 }
 int arcz_engine_layer_moe(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp) {
   return guarded([&] { e->e->layer_moe(L->L, logits, ldl, x, T, Mp); });

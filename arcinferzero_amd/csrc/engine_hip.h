@@ -872,15 +872,48 @@ class Engine {
     CL_CHECK(clEnqueueFillBuffer(cl_.queue, mcount_, &zero, 4, 0, nchunks * NE * 4, 0, nullptr, nullptr));
   }
 
+  // NE matrices of N rows x K values -> NE matrices of Np rows x Kp values, the added rows and the added blocks of a
+  // row zero bytes (every type decodes them to zeros).  K != Kp: the 32-value-block types only (make_weight).
+  static std::vector<uint8_t> pad_expert_tensor(uint32_t type, const uint8_t* src, int NE, int N, int K, int Np, int Kp) {
+    const bool blk32 = type == GGML_Q8_0 || type == GGML_Q4_0 || type == GGML_IQ4_NL || type == GGML_MXFP4;
+    if (K != Kp && (!blk32 || K % 32)) throw std::runtime_error("make_moe_layer: rows of " + std::to_string(K) + " values of this type cannot be padded");
+    const size_t bb = arcz_gguf_bytes(type, 1, 256) / 8;  // (bytes of 32 values; used for the block types only)
+    const size_t rb = K != Kp ? (size_t)(K / 32) * bb : arcz_gguf_bytes(type, 1, K);
+    const size_t prb = K != Kp ? (size_t)(Kp / 32) * bb : rb;
+    std::vector<uint8_t> out((size_t)NE * Np * prb, 0);
+    for (int e = 0; e < NE; ++e)
+      for (int n = 0; n < N; ++n) memcpy(&out[((size_t)e * Np + n) * prb], src + ((size_t)e * N + n) * rb, rb);
+    return out;
+  }
+  // The three expert tensors of a layer: gate and up [NE][F][E], down [NE][E][F], each of its own type.  E and F that are
+  // not whole superblocks (the reference's Gemma 4 layers with F = 704, MXFP4 layers of 2880 x 2880) are padded to them,
+  // rows and columns, with zeros, as the reference's loader pads (zero/engine_load.h:371-387): the layer then has the
+  // rounded-up E and F -- the activations and the residual rows it works on are that wide, their tails zero -- and the
+  // added rows of gate and up give h = silu(0) * 0 = 0 for the added columns of down.
+  MoeLayer make_moe_layer(const uint32_t type[3], const uint8_t* const data[3], int NE, int NU, int E, int F) {
+    if (NE <= 0 || E <= 0 || F <= 0) throw std::runtime_error("make_moe_layer: bad shape");
+    const int Ep = (E + 255) / 256 * 256, Fp = (F + 255) / 256 * 256;
+    std::vector<uint8_t> pad[3];
+    const uint8_t* d[3] = {data[0], data[1], data[2]};
+    if (Ep != E || Fp != F) {
+      pad[0] = pad_expert_tensor(type[0], data[0], NE, F, E, Fp, Ep);
+      pad[1] = pad_expert_tensor(type[1], data[1], NE, F, E, Fp, Ep);
+      pad[2] = pad_expert_tensor(type[2], data[2], NE, E, F, Ep, Fp);
+      for (int i = 0; i < 3; ++i) d[i] = pad[i].data();
+    }
+    moe_alloc(NE, NU, Ep, Fp);
+    MoeLayer L;
+    L.NE = NE; L.NU = NU; L.E = Ep; L.F = Fp;
+    L.ex[0] = make_weight(type[0], d[0], arcz_gguf_bytes(type[0], (size_t)NE * Fp, Ep), Fp, Ep, (size_t)NE * Fp);
+    L.ex[1] = make_weight(type[1], d[1], arcz_gguf_bytes(type[1], (size_t)NE * Fp, Ep), Fp, Ep, (size_t)NE * Fp);
+    L.ex[2] = make_weight(type[2], d[2], arcz_gguf_bytes(type[2], (size_t)NE * Ep, Fp), Ep, Fp, (size_t)NE * Ep);
+    return L;
+  }
   MoeLayer make_moe_layer(uint32_t type, const uint8_t* gate, const uint8_t* up, const uint8_t* down, int NE, int NU,
                           int E, int F) {
-    moe_alloc(NE, NU, E, F);
-    MoeLayer L;
-    L.NE = NE; L.NU = NU; L.E = E; L.F = F;
-    L.ex[0] = make_weight(type, gate, arcz_gguf_bytes(type, (size_t)NE * F, E), F, E, (size_t)NE * F);
-    L.ex[1] = make_weight(type, up, arcz_gguf_bytes(type, (size_t)NE * F, E), F, E, (size_t)NE * F);
-    L.ex[2] = make_weight(type, down, arcz_gguf_bytes(type, (size_t)NE * E, F), E, F, (size_t)NE * E);
-    return L;
+    const uint32_t types[3] = {type, type, type};
+    const uint8_t* const data[3] = {gate, up, down};
+    return make_moe_layer(types, data, NE, NU, E, F);
   }
 
   // routing -> slots grouped by expert -> tiles (zero/engine_moe.h:95-134).  rl: router logits [T][ldl] f32.

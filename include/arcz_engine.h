@@ -127,6 +127,11 @@ arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void*
                                       int NE, int NU, int E, int F);
 /* Engine::layer_moe (zero/engine_moe.h:8-361, standard experts, no shared expert): x[t] += sum_k w_k expert_k(h[t]) for
  * the T tokens whose quantized h is the current activation chunk; logits: router logits [T][ldl] f32. */
+/* The hidden and FFN widths the layer works with: E and F, or -- where they are not whole superblocks (multiples of
+ * 256) -- E and F rounded up, the tensors having been padded with zero rows and zero blocks as the reference's loader
+ * pads them (zero/engine_load.h:371-387; columns: Q8_0, Q4_0, IQ4_NL and MXFP4 only).  The activations and the rows of
+ * x are then that wide, their tails zero. */
+int arcz_moe_layer_dims(const arcz_moe_layer* L, int* E, int* F);
 int arcz_engine_layer_moe(arcz_engine* e, arcz_moe_layer* L, arcz_mem* logits, int ldl, arcz_mem* x, int T, int Mp);
 /* The same with the shared expert's term (moe_combine's sgate * sh, zero/kernels/moe.cl:344-352): sh [T][E] f32 is the
  * shared expert's output for the chunk (computed by the caller with arcz_engine_matmul, as zero/engine_moe.h:66-84

@@ -305,3 +305,50 @@ def test_moe_layer_with_shared_expert_term(rt, qtype, T, Mp):
             b.free()
     finally:
         eng.close()
+
+
+@pytest.mark.parametrize("qtype,NE,NU,E,F,T,Mp", [(az.MXFP4, 4, 2, 352, 160, 3, 16), (az.MXFP4, 4, 2, 352, 160, 70, 80),
+                                                   (az.Q8_0, 6, 3, 512, 96, 40, 48), (az.IQ4_NL, 4, 2, 2880, 2880, 5, 16)])
+def test_moe_layer_of_widths_that_are_not_whole_superblocks(rt, qtype, NE, NU, E, F, T, Mp):
+    """Expert tensors whose hidden or FFN width is not a multiple of 256 (the reference's Gemma 4 layers with F = 704;
+    MXFP4 layers of 2880 x 2880): the upload pads rows and columns with zeros to whole superblocks, as the reference's
+    loader pads (zero/engine_load.h:371-387), the layer reports the rounded-up widths, and on activations and residual
+    rows of those widths whose tails are zero it gives, bit for bit, what the same tensors padded by hand give -- a
+    layer of whole superblocks, which the other tests hold to the oracle."""
+    print(f"moe layer padded {TYPE_NAMES[qtype]} NE={NE} NU={NU} E={E} F={F} T={T}", flush=True)
+    Ep, Fp = (E + 255) // 256 * 256, (F + 255) // 256 * 256
+    bb = az.gguf_bytes(qtype, 1, 256) // 8
+    def cut(seed, N, K, Np, Kp):
+        """[NE][Np][Kp] generated, then the rows and blocks past N and K zeroed: the padded tensor and the one a file holds."""
+        full = make_weights(qtype, NE * Np, Kp, seed=seed).reshape(NE, Np, Kp // 32, bb).copy()
+        full[:, N:] = 0
+        full[:, :, K // 32:] = 0
+        return full.reshape(-1), np.ascontiguousarray(full[:, :N, :K // 32]).reshape(-1)
+    Gp, G = cut(1, F, E, Fp, Ep)
+    Up, U = cut(2, F, E, Fp, Ep)
+    Dp, D = cut(3, E, F, Ep, Fp)
+    eng = az.Engine(Mp, max(Ep, Fp))
+    try:
+        x = np.zeros((T, Ep), np.float32)
+        x[:, :E] = make_acts(T, E, seed=4)
+        x0 = np.zeros((T, Ep), np.float32)
+        x0[:, :E] = az.gen_normal(9, (T, E))
+        logits = np.random.default_rng(5).standard_normal((T, NE)).astype(np.float32)
+        xb, lb = az.Runtime.from_numpy(x), az.Runtime.from_numpy(logits)
+        eng.quantize(xb, Ep, Ep, Mp, T)
+        outs = []
+        for tensors, dims in (((G, U, D), (E, F)), ((Gp, Up, Dp), (Ep, Fp))):
+            L = eng.make_moe_layer(qtype, *tensors, NE, NU, *dims)
+            assert (L.E, L.F) == (Ep, Fp)
+            ob = az.Runtime.from_numpy(x0)
+            eng.layer_moe(L, lb, NE, ob, T, Mp)
+            outs.append(ob.read(np.float32, T * Ep).reshape(T, Ep))
+            ob.free()
+        assert np.isfinite(outs[0]).all() and np.abs(outs[0] - x0).max() > 0
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+        assert np.array_equal(outs[0][:, E:], x0[:, E:])            # the padding columns of x: nothing added
+        with pytest.raises(az.ArczError):
+            eng.make_moe_layer(az.Q4_K, G, U, D, NE, NU, E, F)       # superblock types: whole superblocks only
+        xb.free(); lb.free()
+    finally:
+        eng.close()
