@@ -10,6 +10,7 @@ import os
 import numpy as np
 
 Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ3_XXS, IQ4_NL, IQ3_S, IQ4_XS, MXFP4 = 2, 8, 11, 12, 13, 14, 18, 20, 21, 23, 39  # GGUF type ids
+Q2_0, AR4_128 = 42, 0x41523447   # (uploaded as Q4_0 blocks of the same values)
 
 lib_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libarcz_hip.so")
 if not os.path.exists(lib_path):
@@ -119,6 +120,7 @@ _sig("arcz_engine_rd_bytes", _u64, _p)
 _sig("arcz_gguf_bytes", _z, _u32, _z, _i)
 _sig("arcz_planes_bytes", _z, _u32, _z, _i)
 _sig("arcz_repack_planes", _i, _u32, _z, _i, _p, _p)
+_sig("arcz_relayout_q4_0", _z, _u32, _z, _i, _p, _p)
 _sig("arcz_quantize_rows", _i, _u32, _p, _z, _i, _p)
 _sig("arcz_gen_normal", None, _u64, _z, C.c_float, C.c_float, _p)
 _sig("arcz_gen_weights", _i, _u32, _u64, _z, _i, C.c_float, _p)
@@ -204,6 +206,16 @@ class GgufFile:
 # ---------------------------------------------------------------- host helpers (no GPU)
 def gguf_bytes(qtype, rows, K):
     return lib.arcz_gguf_bytes(qtype, rows, K)
+
+
+def relayout_q4_0(qtype, rows, K, src):
+    """AR4_128 / Q2_0 rows as Q4_0 blocks of the same values (what make_weight does with them first)."""
+    src = np.ascontiguousarray(src, dtype=np.uint8)
+    if src.size != lib.arcz_relayout_q4_0(qtype, rows, K, None, None) or src.size == 0:
+        raise ValueError("relayout_q4_0: type, K or byte count do not fit")
+    out = np.empty(rows * (K // 32) * 18, np.uint8)
+    lib.arcz_relayout_q4_0(qtype, rows, K, _np_ptr(src), _np_ptr(out))
+    return out
 
 
 def planes_bytes(qtype, rows, K):
@@ -387,6 +399,11 @@ class MoeLayer:
     def __init__(self, eng, h, NE, NU, E, F):
         self.eng, self.h, self.NE, self.NU, self.E, self.F = eng, h, NE, NU, E, F
 
+    def free(self):
+        if self.h:
+            lib.arcz_moe_layer_free(self.eng.h, self.h)
+            self.h = None
+
 
 class Engine:
     """The matmul dispatch of the reference's Engine for one GPU (zero/engine.h:936-1251, zero/engine_moe.h)."""
@@ -492,7 +509,10 @@ class Engine:
 
     def make_moe_layer(self, qtype, gate, up, down, NE, NU, E, F):
         g, u, d = (np.ascontiguousarray(a, dtype=np.uint8) for a in (gate, up, down))
-        if E % 256 == 0 and F % 256 == 0:
+        if qtype in (Q2_0, AR4_128):
+            assert g.size == lib.arcz_relayout_q4_0(qtype, NE * F, E, None, None) and u.size == g.size
+            assert d.size == lib.arcz_relayout_q4_0(qtype, NE * E, F, None, None) and g.size and d.size
+        elif E % 256 == 0 and F % 256 == 0:
             assert g.size == gguf_bytes(qtype, NE * F, E) and u.size == g.size and d.size == gguf_bytes(qtype, NE * E, F)
         h = lib.arcz_moe_layer_upload(self.h, qtype, _np_ptr(g), _np_ptr(u), _np_ptr(d), NE, NU, E, F)
         if not h:

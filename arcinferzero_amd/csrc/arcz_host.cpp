@@ -17,6 +17,8 @@
 #define GGML_TYPE_Q3_K 11u  // (src/gguf.h:20)
 #define GGML_TYPE_IQ3_XXS 18u  // (src/gguf.h:21)
 #define GGML_TYPE_MXFP4 39u  // (src/gguf.h:23)
+#define GGML_TYPE_Q2_0 42u   // (src/gguf.h:30)
+#define GGML_TYPE_AR4_128 0x41523447u  // (src/gguf.h:29)
 
 namespace {
 
@@ -335,6 +337,51 @@ int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* src, ui
     return 0;
   }
   return -1;
+}
+
+// Two types that share Q4_0's arithmetic -- one f16 scale times a small integer -- written out as Q4_0 blocks, value
+// for value: AR4_128 (blocks of 128: f16 d, then four runs of 16 nibble bytes arranged as Q4_0's, value d * (q - 8);
+// reference src/quants.h:531-542) gives each of its four runs the block's d; Q2_0 (blocks of 64: f16 d, 64 2-bit codes,
+// element j in bits 2 (j % 4) of byte j / 4, value d * (q - 1); src/quants.h:607-616) becomes two blocks of nibbles
+// q + 7.  K in whole source blocks; dst holds rows * K / 32 blocks of 18 bytes.  Bytes per 256 values: 132 and 72
+// in the file, 144 as written here.  Returns the bytes of the source it read, 0 for another type or a K that does not fit.
+size_t arcz_relayout_q4_0(uint32_t type, size_t rows, int K, const uint8_t* src, uint8_t* dst) {
+  if (K <= 0) return 0;
+  if (type == GGML_TYPE_AR4_128) {
+    if (K % 128) return 0;
+    const int64_t nb = (int64_t)rows * (K / 128);
+    if (!dst) return (size_t)nb * 66;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < nb; ++i) {
+      const uint8_t* b = src + i * 66;
+      for (int c = 0; c < 4; ++c) {
+        uint8_t* o = dst + (i * 4 + c) * 18;
+        memcpy(o, b, 2);
+        memcpy(o + 2, b + 2 + 16 * c, 16);
+      }
+    }
+    return (size_t)nb * 66;
+  }
+  if (type == GGML_TYPE_Q2_0) {
+    if (K % 64) return 0;
+    const int64_t nb = (int64_t)rows * (K / 64);
+    if (!dst) return (size_t)nb * 18;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < nb; ++i) {
+      const uint8_t* b = src + i * 18;
+      for (int c = 0; c < 2; ++c) {
+        uint8_t* o = dst + (i * 2 + c) * 18;
+        memcpy(o, b, 2);
+        for (int j = 0; j < 16; ++j) {
+          const int e0 = 32 * c + j, e1 = e0 + 16;
+          const int q0 = (b[2 + e0 / 4] >> (2 * (e0 % 4))) & 3, q1 = (b[2 + e1 / 4] >> (2 * (e1 % 4))) & 3;
+          o[2 + j] = (uint8_t)((q0 + 7) | ((q1 + 7) << 4));
+        }
+      }
+    }
+    return (size_t)nb * 18;
+  }
+  return 0;
 }
 
 // n values ~ N(mean, std): SplitMix64 -> two uniforms -> Box-Muller in f32, element i from the stream position i / 2

@@ -26,8 +26,11 @@
 #define GGML_Q3_K 11u
 #define GGML_IQ3_XXS 18u
 #define GGML_MXFP4 39u
+#define GGML_Q2_0 42u
+#define GGML_AR4_128 0x41523447u
 
 extern "C" int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* out);
+extern "C" size_t arcz_relayout_q4_0(uint32_t type, size_t rows, int K, const uint8_t* src, uint8_t* dst);
 extern "C" size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
 extern "C" void arcz_iq3s_grid(uint32_t* out);
 extern "C" void arcz_iq3xxs_grid(uint32_t* out);
@@ -218,8 +221,25 @@ class Engine {
 
   // ---- weights (zero/engine_load.h:84-130 upload_padded, :157-196 make_weight): the GGUF rows regrouped into the
   // device planes on the host, then one upload.  rows = N for a matrix, n_expert * N for an expert tensor.
+  // AR4_128 and Q2_0 tensors become Q4_0 ones with the same values (arcz_relayout_q4_0): every kernel then sees Q4_0,
+  // at 144 bytes per 256 values where the file has 132 and 72.  (The reference keeps both in kernels of their own,
+  // zero/kernels/decode.cl PER32; the values and the arithmetic on them are the same.)
+  static bool as_q4_0(uint32_t& type, const uint8_t*& data, size_t& nbytes, size_t rows, int K, std::vector<uint8_t>& hold) {
+    if (type != GGML_AR4_128 && type != GGML_Q2_0) return false;
+    const size_t want = arcz_relayout_q4_0(type, rows, K, nullptr, nullptr);
+    if (!want) throw std::runtime_error("make_weight: K = " + std::to_string(K) + " is not whole blocks of this type (128 for AR4_128, 64 for Q2_0)");
+    if (nbytes != want) throw std::runtime_error("make_weight: " + std::to_string(nbytes) + " bytes given, " + std::to_string(want) + " expected");
+    hold.resize(rows * (size_t)(K / 32) * 18);
+    arcz_relayout_q4_0(type, rows, K, data, hold.data());
+    type = GGML_Q4_0;
+    data = hold.data();
+    nbytes = hold.size();
+    return true;
+  }
   GpuWeight make_weight(uint32_t type, const uint8_t* data, size_t nbytes, int N, int K, size_t rows = 0) {
     if (rows == 0) rows = (size_t)N;
+    std::vector<uint8_t> as40;
+    if (K > 0 && N > 0) as_q4_0(type, data, nbytes, rows, K, as40);
     if (type != GGML_Q4_0 && type != GGML_Q8_0 && type != GGML_Q4_K && type != GGML_Q5_K && type != GGML_Q6_K && type != GGML_IQ4_XS &&
         type != GGML_IQ3_S && type != GGML_IQ4_NL && type != GGML_MXFP4 && type != GGML_Q3_K && type != GGML_IQ3_XXS)
       throw std::runtime_error(std::string("unsupported weight type ") + std::to_string(type));
@@ -890,15 +910,22 @@ class Engine {
   // rows and columns, with zeros, as the reference's loader pads (zero/engine_load.h:371-387): the layer then has the
   // rounded-up E and F -- the activations and the residual rows it works on are that wide, their tails zero -- and the
   // added rows of gate and up give h = silu(0) * 0 = 0 for the added columns of down.
-  MoeLayer make_moe_layer(const uint32_t type[3], const uint8_t* const data[3], int NE, int NU, int E, int F) {
+  MoeLayer make_moe_layer(const uint32_t type_in[3], const uint8_t* const data[3], int NE, int NU, int E, int F) {
     if (NE <= 0 || E <= 0 || F <= 0) throw std::runtime_error("make_moe_layer: bad shape");
     const int Ep = (E + 255) / 256 * 256, Fp = (F + 255) / 256 * 256;
-    std::vector<uint8_t> pad[3];
+    std::vector<uint8_t> pad[3], as40[3];
+    uint32_t type[3] = {type_in[0], type_in[1], type_in[2]};
     const uint8_t* d[3] = {data[0], data[1], data[2]};
+    for (int i = 0; i < 3; ++i) {  // (AR4_128, Q2_0: as Q4_0 blocks first, see as_q4_0)
+      const size_t rows = (size_t)NE * (i == 2 ? E : F);
+      const int K = i == 2 ? F : E;
+      size_t nb = arcz_relayout_q4_0(type[i], rows, K, nullptr, nullptr);
+      if (type[i] == GGML_AR4_128 || type[i] == GGML_Q2_0) as_q4_0(type[i], d[i], nb, rows, K, as40[i]);
+    }
     if (Ep != E || Fp != F) {
-      pad[0] = pad_expert_tensor(type[0], data[0], NE, F, E, Fp, Ep);
-      pad[1] = pad_expert_tensor(type[1], data[1], NE, F, E, Fp, Ep);
-      pad[2] = pad_expert_tensor(type[2], data[2], NE, E, F, Ep, Fp);
+      pad[0] = pad_expert_tensor(type[0], d[0], NE, F, E, Fp, Ep);
+      pad[1] = pad_expert_tensor(type[1], d[1], NE, F, E, Fp, Ep);
+      pad[2] = pad_expert_tensor(type[2], d[2], NE, E, F, Ep, Fp);
       for (int i = 0; i < 3; ++i) d[i] = pad[i].data();
     }
     moe_alloc(NE, NU, Ep, Fp);

@@ -31,10 +31,12 @@ void arcz_engine_destroy(arcz_engine* e);
 /* make_weight + upload_padded (zero/engine_load.h:84-130, 157-196): N rows of K values as GGUF blocks of `type`
  * (2 = Q4_0, 8 = Q8_0, 11 = Q3_K, 12 = Q4_K, 13 = Q5_K, 14 = Q6_K, 18 = IQ3_XXS, 20 = IQ4_NL, 21 = IQ3_S, 23 = IQ4_XS,
  * 39 = MXFP4),
- * regrouped into the device layout -- every type in its own form, the GGUF byte count -- and uploaded. */
+ * regrouped into the device layout -- every type in its own form, the GGUF byte count -- and uploaded.  Two more types,
+ * 42 = Q2_0 (K a multiple of 64) and 0x41523447 = AR4_128 (K a multiple of 128), are taken as Q4_0: written out as Q4_0
+ * blocks of the same values first (arcz_relayout_q4_0), so on the device they take Q4_0's bytes, not the file's. */
 arcz_weight* arcz_weight_upload(arcz_engine* e, uint32_t type, int N, int K, const void* gguf, size_t bytes);
 /* The same from a tensor of an open GGUF file (upload of zero/engine_load.h:84-196): a matrix (dims K, N) or an expert
- * tensor (dims K, N, experts) of type Q4_0 / Q8_0 / Q3_K / Q4_K / Q5_K / Q6_K / IQ3_XXS / IQ4_NL / IQ3_S / IQ4_XS / MXFP4, by name;
+ * tensor (dims K, N, experts) of type Q4_0 / Q8_0 / Q3_K / Q4_K / Q5_K / Q6_K / IQ3_XXS / IQ4_NL / IQ3_S / IQ4_XS / MXFP4 (or Q2_0 / AR4_128, as above), by name;
  * NULL + arcz_engine_error() when it is missing, of another type or shape.  The MoE layer: its three expert tensors (gate and up [NE][F][E], down [NE][E][F]). */
 arcz_weight* arcz_weight_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* name);
 arcz_moe_layer* arcz_moe_layer_upload_gguf(arcz_engine* e, const arcz_gguf* g, const char* gate, const char* up,
@@ -174,6 +176,11 @@ uint64_t arcz_engine_rd_bytes(arcz_engine* e);
 size_t arcz_gguf_bytes(uint32_t type, size_t rows, int K);
 size_t arcz_planes_bytes(uint32_t type, size_t rows, int K);
 int arcz_repack_planes(uint32_t type, size_t rows, int K, const uint8_t* gguf, uint8_t* planes);
+/* AR4_128 (0x41523447) and Q2_0 (42) rows (src/quants.h:531-542, 607-616) written out as Q4_0 blocks with the same
+ * values (d * (q - 8) with the 128-block's d; d * ((q + 7) - 8)): what make_weight does with these two types before
+ * anything else.  K in whole source blocks (128, 64); dst: rows * K / 32 * 18 bytes, or NULL to ask for the count only.
+ * Returns the source bytes (rows * K / 128 * 66, rows * K / 64 * 18), 0 for another type or a K that does not fit. */
+size_t arcz_relayout_q4_0(uint32_t type, size_t rows, int K, const uint8_t* src, uint8_t* dst);
 /* The IQ3_S codebook (ggml's iq3s_grid, src/iq_tables.h:297) as the kernels take it in their `tabs` argument: 512 words,
  * byte j of a word = magnitude j of the entry (1, 3, ..., 15). */
 void arcz_iq3s_grid(uint32_t* out512);

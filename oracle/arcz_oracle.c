@@ -22,6 +22,9 @@
  *   Q3_K decode                         closed-form block; live comparison with the compiled reference header
  *   IQ4_NL, MXFP4 decode                closed-form blocks (every code, every E8M0 exponent); live comparison with the
  *                                       compiled reference header
+ *   AR4_128, Q2_0 decode                closed-form blocks (every code at every position); golden vectors
+ *                                       (tests/golden/ref_vectors_types4.npz) and live comparison with the compiled
+ *                                       reference header
  *   IQ3_S decode (and its grid table)   closed-form block; golden vectors (tests/golden/ref_vectors_types2.npz) and live
  *                                       comparison with the compiled reference header over every grid index
  *   Q5_K decode                         closed-form block; golden vectors (tests/golden/ref_vectors_q5k.npz) and live
@@ -51,7 +54,12 @@
  * place of the f16 one): src/quants.h:520-530, 594-606 */
 #define ORC_IQ4_NL 20u
 #define ORC_MXFP4 39u
-#define ORC_Q8LIKE(t) ((t) == ORC_Q8_0 || (t) == ORC_Q4_0 || (t) == ORC_IQ4_NL || (t) == ORC_MXFP4)
+/* AR4_128 is Q4_0 with one f16 scale for four 32-blocks; Q2_0 has 64-blocks of 2-bit codes q, value d * (q - 1):
+ * src/quants.h:531-542, 607-616 */
+#define ORC_AR4_128 0x41523447u
+#define ORC_Q2_0 42u
+#define ORC_Q8LIKE(t) \
+  ((t) == ORC_Q8_0 || (t) == ORC_Q4_0 || (t) == ORC_IQ4_NL || (t) == ORC_MXFP4 || (t) == ORC_AR4_128 || (t) == ORC_Q2_0)
 #define ORC_Q4_K 12u
 #define ORC_Q5_K 13u
 #define ORC_Q45(t) ((t) == ORC_Q4_K || (t) == ORC_Q5_K) /* d, dmin, 6-bit scales and mins */
@@ -122,6 +130,8 @@ int orc_sb_bytes(uint32_t type) {
     case ORC_Q4_0: return 18 * 8;
     case ORC_IQ4_NL: return 18 * 8;
     case ORC_MXFP4: return 17 * 8;
+    case ORC_AR4_128: return 66 * 2;
+    case ORC_Q2_0: return 18 * 4;
     case ORC_Q4_K: return 144;
     case ORC_Q5_K: return 176;
     case ORC_Q6_K: return 210;
@@ -355,6 +365,30 @@ int orc_decode_sb(uint32_t type, const uint8_t* p, orc_sb* o) {
       for (int i = 0; i < 16; ++i) {
         o->q[32 * b + i] = mxfp4_values[blk[1 + i] & 0xF];
         o->q[32 * b + 16 + i] = mxfp4_values[blk[1 + i] >> 4];
+      }
+    }
+    return 0;
+  }
+  if (type == ORC_AR4_128) { /* 2 blocks of 66 bytes: f16 d, then four runs of 16 bytes, each the nibbles of 32 elements
+                                as Q4_0 holds them, q - 8 (src/quants.h:531-542) */
+    for (int b = 0; b < 8; ++b) {
+      const uint8_t* blk = p + 66 * (b / 4);
+      o->d8[b] = orc_fp16_to_f32(rd16(blk));
+      for (int i = 0; i < 16; ++i) {
+        o->q[32 * b + i] = (int16_t)((blk[2 + 16 * (b % 4) + i] & 0xF) - 8);
+        o->q[32 * b + 16 + i] = (int16_t)((blk[2 + 16 * (b % 4) + i] >> 4) - 8);
+      }
+    }
+    return 0;
+  }
+  if (type == ORC_Q2_0) { /* 4 blocks of 18 bytes: f16 d, then 64 2-bit codes, element j in bits 2 (j % 4) of byte j / 4,
+                             q - 1 (src/quants.h:607-616) */
+    for (int b = 0; b < 8; ++b) {
+      const uint8_t* blk = p + 18 * (b / 2);
+      o->d8[b] = orc_fp16_to_f32(rd16(blk));
+      for (int i = 0; i < 32; ++i) {
+        const int j = 32 * (b % 2) + i;
+        o->q[32 * b + i] = (int16_t)(((blk[2 + j / 4] >> (2 * (j % 4))) & 3) - 1);
       }
     }
     return 0;

@@ -10,7 +10,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ3_XXS, IQ4_NL, IQ3_S, IQ4_XS, MXFP4 = 2, 8, 11, 12, 13, 14, 18, 20, 21, 23, 39
-SB_BYTES = {Q4_0: 144, Q8_0: 272, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ3_S: 110, IQ4_XS: 136, IQ4_NL: 144, MXFP4: 136, Q3_K: 110, IQ3_XXS: 98}
+Q2_0, AR4_128 = 42, 0x41523447
+SB_BYTES = {Q2_0: 72, AR4_128: 132, Q4_0: 144, Q8_0: 272, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ3_S: 110, IQ4_XS: 136, IQ4_NL: 144, MXFP4: 136, Q3_K: 110, IQ3_XXS: 98}
 
 _p, _i = C.c_void_p, C.c_int
 

@@ -15,6 +15,7 @@ from common import TYPES, make_acts, make_weights, rel_err_rows, unit_scale_acts
 G = dict(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz")))
 G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_types2.npz")))
 G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_types3.npz")))
+G.update(np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors_types4.npz")))
 Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = 8, 12, 13, 14, 23
 NAMES = {Q4_K: "q4k", Q5_K: "q5k", Q6_K: "q6k", Q8_0: "q80", IQ4_XS: "iq4xs"}
 
@@ -469,6 +470,89 @@ def test_iq4_nl_and_mxfp4_vs_compiled_reference(qtype):
         orc.ref.ref_gpu_raw_sb(qtype, orc.ptr(W[i * (16 + hb) * 8:]), orc.ptr(raw))
         assert np.array_equal(raw[:8 * hb], planes[u * 128 + i * 8 * hb:u * 128 + (i + 1) * 8 * hb])
         assert np.array_equal(raw[8 * hb:], planes[i * 128:(i + 1) * 128])
+
+
+def _ar4_q20_by_hand():
+    """One superblock of each type written field by field, with the values it must decode to: every code in every
+    position class (AR4_128: low and high nibble of every byte of a run; Q2_0: each of the four 2-bit slots of a byte),
+    scales of both signs, zero and a subnormal."""
+    ar = np.zeros((2, 66), np.uint8)
+    ar_exp = np.zeros(256, np.float32)
+    for b, d in enumerate([-0.75, 6.103515625e-05 / 4]):                  # (the second: an f16 subnormal)
+        ar[b, 0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+        for c in range(4):
+            for j in range(16):
+                lo, hi = (j + 3 * c + b) % 16, (7 * j + c + 5 * b + 2) % 16
+                ar[b, 2 + 16 * c + j] = lo | (hi << 4)
+                ar_exp[128 * b + 32 * c + j] = np.float32(np.float16(d)) * np.float32(lo - 8)
+                ar_exp[128 * b + 32 * c + 16 + j] = np.float32(np.float16(d)) * np.float32(hi - 8)
+    q2 = np.zeros((4, 18), np.uint8)
+    q2_exp = np.zeros(256, np.float32)
+    for b, d in enumerate([0.5, -3.0, 0.0, 1024.0]):
+        q2[b, 0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+        for j in range(64):
+            q = (j + j // 4 + b) % 4
+            q2[b, 2 + j // 4] |= q << (2 * (j % 4))
+            q2_exp[64 * b + j] = np.float32(d) * np.float32(q - 1)
+    return ar.reshape(-1), ar_exp, q2.reshape(-1), q2_exp
+
+
+def test_ar4_128_and_q2_0_closed_form_and_golden():
+    """AR4_128 (src/quants.h:531-542): the 128-block's f16 d times (nibble - 8), four runs of 16 bytes laid out as
+    Q4_0's; Q2_0 (src/quants.h:607-616): the 64-block's f16 d times (code - 1), element j in bits 2 (j % 4) of byte
+    j / 4.  By hand, then the compiled reference's decode of blocks of random bytes, bit for bit."""
+    ar, ar_exp, q2, q2_exp = _ar4_q20_by_hand()
+    assert np.array_equal(orc.dequant_rows(orc.AR4_128, ar, 1, 256)[0], ar_exp)
+    assert np.array_equal(orc.dequant_rows(orc.Q2_0, q2, 1, 256)[0], q2_exp)
+    q, isc, imn, d, dmin = orc.decode_row_fields(orc.Q2_0, q2, 256)
+    assert np.array_equal(isc, np.ones(16)) and not imn.any() and not dmin.any()
+    assert np.array_equal(d, np.repeat(np.float32([0.5, -3.0, 0.0, 1024.0]), 2)) and q.min() == -1 and q.max() == 2
+    for name, qtype in (("ar4128", orc.AR4_128), ("q20", orc.Q2_0)):
+        got = orc.dequant_rows(qtype, G[name + "_raw"], 4, 512)
+        assert np.array_equal(got.view(np.uint32), G[name + "_dequant"].view(np.uint32))
+
+
+@pytest.mark.skipif(orc.ref is None, reason="oracle/_ref is not built (no reference tree here)")
+@pytest.mark.parametrize("qtype", [orc.AR4_128, orc.Q2_0])
+def test_ar4_128_and_q2_0_vs_compiled_reference(qtype):
+    """Blocks of random bytes (finite f16 scales) through the oracle and the compiled reference header, bit for bit."""
+    N, K = 8, 1024
+    nb = orc.SB_BYTES[qtype] // (2 if qtype == orc.AR4_128 else 4)
+    R = np.random.default_rng(11).integers(0, 256, size=(N * K // 256 * orc.SB_BYTES[qtype] // nb, nb), dtype=np.uint8)
+    R[:, 1] &= 0x7B
+    a, b = orc.dequant_rows(qtype, R.reshape(-1), N, K), orc.dequant_rows(qtype, R.reshape(-1), N, K, lib=orc.ref)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_relayout_q4_0_keeps_every_value():
+    """The library writes AR4_128 and Q2_0 rows out as Q4_0 blocks before it uploads them: the Q4_0 decode of what it
+    writes is the decode of the source, bit for bit (by hand, golden blocks, random bytes), and K that is not whole
+    source blocks, another type or a wrong byte count are refused."""
+    ar, ar_exp, q2, q2_exp = _ar4_q20_by_hand()
+    assert np.array_equal(orc.dequant_rows(az.Q4_0, az.relayout_q4_0(az.AR4_128, 1, 256, ar), 1, 256)[0], ar_exp)
+    assert np.array_equal(orc.dequant_rows(az.Q4_0, az.relayout_q4_0(az.Q2_0, 1, 256, q2), 1, 256)[0], q2_exp)
+    for name, qtype in (("ar4128", az.AR4_128), ("q20", az.Q2_0)):
+        out = az.relayout_q4_0(qtype, 4, 512, G[name + "_raw"])
+        assert out.size == 4 * 16 * 18
+        assert np.array_equal(orc.dequant_rows(az.Q4_0, out, 4, 512).view(np.uint32), G[name + "_dequant"].view(np.uint32))
+    # rows that end inside a superblock: 3 rows of 384 (AR4_128) and of 320 (Q2_0) values
+    rng = np.random.default_rng(5)
+    for qtype, K, blk, nbytes in ((az.AR4_128, 384, 128, 66), (az.Q2_0, 320, 64, 18)):
+        raw = rng.integers(0, 256, size=(3 * K // blk, nbytes), dtype=np.uint8)
+        raw[:, 1] &= 0x7B
+        out = az.relayout_q4_0(qtype, 3, K, raw.reshape(-1)).reshape(3, K // 32 * 18)
+        for r in range(3):     # (each row alone, padded with zero blocks to 512 for the oracle's whole superblocks)
+            src = np.zeros(512 // blk * nbytes, np.uint8)
+            src[:K // blk * nbytes] = raw.reshape(3, -1)[r]
+            dst = np.zeros(16 * 18, np.uint8)
+            dst[:K // 32 * 18] = out[r]
+            assert np.array_equal(orc.dequant_rows(az.Q4_0, dst, 1, 512), orc.dequant_rows(qtype, src, 1, 512))
+    for bad in (lambda: az.relayout_q4_0(az.AR4_128, 1, 192, np.zeros(99, np.uint8)),
+                lambda: az.relayout_q4_0(az.Q2_0, 1, 96, np.zeros(27, np.uint8)),
+                lambda: az.relayout_q4_0(az.Q4_0, 1, 256, np.zeros(144, np.uint8)),
+                lambda: az.relayout_q4_0(az.Q2_0, 2, 128, np.zeros(71, np.uint8))):
+        with pytest.raises(ValueError):
+            bad()
 
 
 # ---------------------------------------------------------------- quantizers
