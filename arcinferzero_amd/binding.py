@@ -61,6 +61,12 @@ _sig("arcz_event_elapsed_ms", C.c_double, _p, _p)
 _sig("arcz_set_fake_oom", None, C.c_long)
 _sig("arcz_set_oom_hook", None, _p)
 _sig("arcz_launch_count", _u64)
+_sig("arcz_record_begin", _i)
+_sig("arcz_record_end", _i, _p)
+_sig("arcz_recording", _i)
+_sig("arcz_list_run", _i, _p)
+_sig("arcz_list_launches", _u64, _p)
+_sig("arcz_list_free", _i, _p)
 _sig("arcz_engine_error", C.c_char_p)
 _sig("arcz_engine_create", _p, _i, _i)
 _sig("arcz_engine_destroy", None, _p)
@@ -378,6 +384,37 @@ class Runtime:
     @staticmethod
     def event_release(e):
         lib.arcz_event_release(e)
+
+    @staticmethod
+    def record(fn):
+        """Records the kernel launches that fn() makes into a LaunchList (nothing runs meanwhile).  fn must have run
+        once before, so that every buffer it needs exists: allocation, copies and waits are refused while recording.
+        If fn raises, the recording is dropped and the exception goes on."""
+        _check(lib.arcz_record_begin())
+        try:
+            fn()
+        except BaseException:
+            lib.arcz_record_end(None)
+            raise
+        h = C.c_void_p()
+        _check(lib.arcz_record_end(C.byref(h)))
+        return LaunchList(h)
+
+
+class LaunchList:
+    """A recorded sequence of kernel launches (arcz_record_begin / arcz_record_end), submitted as one."""
+
+    def __init__(self, h):
+        self.h = h
+        self.launches = lib.arcz_list_launches(h)
+
+    def run(self):
+        _check(lib.arcz_list_run(self.h))
+
+    def free(self):
+        if self.h:
+            _check(lib.arcz_list_free(self.h))
+            self.h = None
 
 
 # ---------------------------------------------------------------- engine (include/arcz_engine.h)

@@ -34,6 +34,11 @@ struct arcz_event {
   hipEvent_t start, stop;
   bool pair;
 };
+struct arcz_list {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  uint64_t launches = 0;  // kernels recorded
+};
 
 namespace {
 struct Runtime {
@@ -51,6 +56,9 @@ struct Runtime {
   uint64_t launches = 0;
   std::string err;
   arcz_mem* scratch = nullptr;  // non-owning handle onto the device's static scratch array (arcz_scratch.hip)
+  bool recording = false;       // between arcz_record_begin and arcz_record_end: launches go into a list, not to the GPU
+  uint64_t rec_launches = 0;
+  std::set<arcz_list*> lists;
 };
 Runtime R;
 
@@ -68,6 +76,17 @@ int fail(int code, const char* fmt, ...) {
   do {                                                                                                      \
     hipError_t e_ = (x);                                                                                    \
     if (e_ != hipSuccess) return fail(ARCZ_E_DEVICE, "%s failed: %s", #x, hipGetErrorString(e_));           \
+  } while (0)
+
+// While a list is being recorded the stream takes nothing but kernel launches: what allocates, frees, copies to or from
+// the host, waits or times is refused, with the recording left as it is.
+#define NOT_WHILE_RECORDING(what, ret)                                                                       \
+  do {                                                                                                      \
+    if (R.recording) {                                                                                      \
+      fail(ARCZ_E_RECORDING, "%s while a launch list is being recorded (refused; run the sequence once before " \
+                             "recording it, so that every buffer it needs exists)", what);                  \
+      return ret;                                                                                           \
+    }                                                                                                       \
   } while (0)
 
 bool out_of_bounds(const char* what, const arcz_mem* b, size_t off, size_t n) {
@@ -140,7 +159,19 @@ arcz_mem* arcz_scratch_mem(void) { return R.up ? R.scratch : nullptr; }
 
 void arcz_shutdown(void) {
   if (!R.up) return;
+  if (R.recording) {  // (an open recording is dropped)
+    hipGraph_t g = nullptr;
+    if (hipStreamEndCapture(R.stream, &g) == hipSuccess && g) hipGraphDestroy(g);
+    (void)hipGetLastError();
+    R.recording = false;
+  }
   hipStreamSynchronize(R.stream);
+  for (arcz_list* l : R.lists) {
+    hipGraphExecDestroy(l->exec);
+    hipGraphDestroy(l->graph);
+    delete l;
+  }
+  R.lists.clear();
   for (auto& kv : R.kernels) delete kv.second;
   R.kernels.clear();
   for (auto& kv : R.modules)
@@ -166,6 +197,7 @@ size_t arcz_device_bytes(void) { return R.device_bytes; }
 
 arcz_mem* arcz_alloc(size_t bytes) {
   if (!R.up) { fail(ARCZ_E_DEVICE, "arcz_alloc before arcz_init"); return nullptr; }
+  NOT_WHILE_RECORDING("arcz_alloc", nullptr);
   const size_t n = bytes < 64 ? 64 : bytes;
   void* p = nullptr;
   hipError_t e = hipSuccess;
@@ -202,6 +234,7 @@ int arcz_free(arcz_mem* m) {
   if (!m) return ARCZ_OK;
   if (m == R.scratch) return fail(ARCZ_E_ARG_VALUE, "arcz_free of the library's static scratch");
   if (!R.mems.count(m)) return fail(ARCZ_E_ARG_VALUE, "arcz_free of a handle that is not live");
+  if (m->owner) NOT_WHILE_RECORDING("arcz_free", ARCZ_E_RECORDING);
   if (m->owner) {
     // (the caller frees views before their parents, zero/engine.h:251-252; a view that is still live would name freed
     //  memory: refused, nothing is freed)
@@ -222,6 +255,7 @@ void* arcz_mem_ptr(const arcz_mem* m) { return m && R.mems.count(const_cast<arcz
 int arcz_h2d(arcz_mem* dst, size_t offset, const void* src, size_t bytes) {
   if (out_of_bounds("write", dst, offset, bytes)) return ARCZ_E_BOUNDS;
   if (!bytes) return ARCZ_OK;
+  NOT_WHILE_RECORDING("arcz_h2d", ARCZ_E_RECORDING);
   HIP_TRY(hipMemcpyAsync(dst->ptr + offset, src, bytes, hipMemcpyHostToDevice, R.stream));
   HIP_TRY(hipStreamSynchronize(R.stream));
   return ARCZ_OK;
@@ -229,6 +263,7 @@ int arcz_h2d(arcz_mem* dst, size_t offset, const void* src, size_t bytes) {
 int arcz_d2h(void* dst, const arcz_mem* src, size_t offset, size_t bytes) {
   if (out_of_bounds("read", src, offset, bytes)) return ARCZ_E_BOUNDS;
   if (!bytes) return ARCZ_OK;
+  NOT_WHILE_RECORDING("arcz_d2h", ARCZ_E_RECORDING);
   HIP_TRY(hipMemcpyAsync(dst, src->ptr + offset, bytes, hipMemcpyDeviceToHost, R.stream));
   HIP_TRY(hipStreamSynchronize(R.stream));
   return ARCZ_OK;
@@ -237,6 +272,7 @@ int arcz_d2d(arcz_mem* dst, size_t dst_offset, const arcz_mem* src, size_t src_o
   if (out_of_bounds("copy (source)", src, src_offset, bytes) || out_of_bounds("copy (destination)", dst, dst_offset, bytes))
     return ARCZ_E_BOUNDS;
   if (!bytes) return ARCZ_OK;
+  NOT_WHILE_RECORDING("arcz_d2d", ARCZ_E_RECORDING);
   HIP_TRY(hipMemcpyAsync(dst->ptr + dst_offset, src->ptr + src_offset, bytes, hipMemcpyDeviceToDevice, R.stream));
   return ARCZ_OK;
 }
@@ -245,6 +281,7 @@ int arcz_d2d(arcz_mem* dst, size_t dst_offset, const arcz_mem* src, size_t src_o
 // full rate; allocated, never registered over existing memory.
 void* arcz_host_alloc(size_t bytes) {
   if (!R.up) { fail(ARCZ_E_DEVICE, "arcz_host_alloc before arcz_init"); return nullptr; }
+  NOT_WHILE_RECORDING("arcz_host_alloc", nullptr);
   void* p = nullptr;
   const hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault);
   if (e != hipSuccess || !p) {
@@ -256,6 +293,7 @@ void* arcz_host_alloc(size_t bytes) {
 }
 int arcz_host_free(void* p) {
   if (!p) return ARCZ_OK;
+  NOT_WHILE_RECORDING("arcz_host_free", ARCZ_E_RECORDING);
   HIP_TRY(hipHostFree(p));
   return ARCZ_OK;
 }
@@ -281,7 +319,12 @@ int arcz_fill(arcz_mem* dst, const void* pattern, size_t ps, size_t offset, size
     void* params[3] = {&p, &v, &n};
     const unsigned blocks = (unsigned)((n + 255) / 256);
     HIP_TRY(hipModuleLaunchKernel(k->fn, blocks, 1, 1, 256, 1, 1, 0, R.stream, params, nullptr));
+    if (R.recording) {  // (recorded as the kernel it is; nothing to wait for)
+      ++R.rec_launches;
+      return ARCZ_OK;
+    }
   } else {
+    NOT_WHILE_RECORDING("arcz_fill of a range that is not whole words", ARCZ_E_RECORDING);  // (no memset nodes in a list)
     if (ps == 1) HIP_TRY(hipMemsetAsync(dst->ptr + offset, (int)(v & 0xFF), bytes, R.stream));
     else HIP_TRY(hipMemsetD16Async((hipDeviceptr_t)(dst->ptr + offset), (unsigned short)(v & 0xFFFF), bytes / 2, R.stream));
   }
@@ -442,6 +485,7 @@ int arcz_launch(arcz_kernel* k, unsigned dim, const size_t* global, const size_t
   }
   for (size_t h = 0; h < k->hidden.size(); ++h) params[nargs + h] = &k->hidden[h];
   arcz_event* ev = nullptr;
+  if (event) NOT_WHILE_RECORDING("arcz_launch with an event", ARCZ_E_RECORDING);
   if (event) {
     ev = new arcz_event{nullptr, nullptr, true};
     HIP_TRY(hipEventCreate(&ev->start));
@@ -455,7 +499,8 @@ int arcz_launch(arcz_kernel* k, unsigned dim, const size_t* global, const size_t
     return fail(ARCZ_E_DEVICE, "launch of %s (global %u x %u x %u, local %u x %u x %u) failed: %s", k->symbol.c_str(),
                 gs[0], gs[1], gs[2], ls[0], ls[1], ls[2], hipGetErrorString(e));
   }
-  ++R.launches;
+  if (R.recording) ++R.rec_launches;  // (it runs when the list runs)
+  else ++R.launches;
   if (ev) {
     HIP_TRY(hipEventRecord(ev->stop, R.stream));
     *event = ev;
@@ -465,6 +510,7 @@ int arcz_launch(arcz_kernel* k, unsigned dim, const size_t* global, const size_t
 
 int arcz_sync(void) {
   if (!R.up) return fail(ARCZ_E_DEVICE, "arcz_sync before arcz_init");
+  NOT_WHILE_RECORDING("arcz_sync", ARCZ_E_RECORDING);
   HIP_TRY(hipStreamSynchronize(R.stream));
   return ARCZ_OK;
 }
@@ -484,6 +530,7 @@ void arcz_event_release(arcz_event* e) {
 }
 arcz_event* arcz_event_record(void) {
   if (!R.up) return nullptr;
+  NOT_WHILE_RECORDING("arcz_event_record", nullptr);
   arcz_event* ev = new arcz_event{nullptr, nullptr, false};
   if (hipEventCreate(&ev->start) != hipSuccess || hipEventRecord(ev->start, R.stream) != hipSuccess) {
     delete ev;
@@ -497,6 +544,67 @@ double arcz_event_elapsed_ms(arcz_event* start, arcz_event* stop) {
   float ms = 0;
   if (hipEventElapsedTime(&ms, start->start, stop->start) != hipSuccess) return -1.0;
   return ms;
+}
+
+// ---- recorded launch lists.  The reference can record its kernels into regular command lists and hand the GPU a
+// whole list at a time (ARC_BATCH, zero/clrt.h:170-265: 700 small kernels took 2.56 us each appended one by one and
+// 0.66 us replayed from a list); here the stream is captured into a HIP graph.  Between begin and end arcz_launch
+// (and a whole-word arcz_fill) add to the list and nothing reaches the GPU; the list then runs as one submission, as
+// often as wanted, on the same buffers with whatever they hold at that time.
+int arcz_record_begin(void) {
+  if (!R.up) return fail(ARCZ_E_DEVICE, "arcz_record_begin before arcz_init");
+  NOT_WHILE_RECORDING("arcz_record_begin", ARCZ_E_RECORDING);
+  // (thread-local mode: calls of other threads that are unsafe under capture do not break this one)
+  HIP_TRY(hipStreamBeginCapture(R.stream, hipStreamCaptureModeThreadLocal));
+  R.recording = true;
+  R.rec_launches = 0;
+  return ARCZ_OK;
+}
+int arcz_record_end(arcz_list** out) {
+  if (out) *out = nullptr;
+  if (!R.up || !R.recording) return fail(ARCZ_E_RECORDING, "arcz_record_end without arcz_record_begin");
+  R.recording = false;
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture(R.stream, &g);
+  if (e != hipSuccess || !g) {
+    (void)hipGetLastError();
+    return fail(ARCZ_E_DEVICE, "the recording did not end in a list: %s", hipGetErrorString(e));
+  }
+  if (!out || R.rec_launches == 0) {  // (abandoned, or empty: nothing to keep)
+    hipGraphDestroy(g);
+    return out ? fail(ARCZ_E_RECORDING, "nothing was recorded") : ARCZ_OK;
+  }
+  hipGraphExec_t x = nullptr;
+  e = hipGraphInstantiate(&x, g, nullptr, nullptr, 0);
+  if (e != hipSuccess || !x) {
+    (void)hipGetLastError();
+    hipGraphDestroy(g);
+    return fail(ARCZ_E_DEVICE, "the recorded list does not instantiate: %s", hipGetErrorString(e));
+  }
+  arcz_list* l = new arcz_list{g, x, R.rec_launches};
+  R.lists.insert(l);
+  *out = l;
+  return ARCZ_OK;
+}
+int arcz_recording(void) { return R.recording ? 1 : 0; }
+int arcz_list_run(arcz_list* l) {
+  if (!R.up || !l || !R.lists.count(l)) return fail(ARCZ_E_ARG_VALUE, "arcz_list_run of a handle that is not a live list");
+  NOT_WHILE_RECORDING("arcz_list_run", ARCZ_E_RECORDING);
+  HIP_TRY(hipGraphLaunch(l->exec, R.stream));
+  R.launches += l->launches;
+  return ARCZ_OK;
+}
+uint64_t arcz_list_launches(const arcz_list* l) { return l && R.lists.count(const_cast<arcz_list*>(l)) ? l->launches : 0; }
+int arcz_list_free(arcz_list* l) {
+  if (!l) return ARCZ_OK;
+  if (!R.lists.count(l)) return fail(ARCZ_E_ARG_VALUE, "arcz_list_free of a handle that is not a live list");
+  NOT_WHILE_RECORDING("arcz_list_free", ARCZ_E_RECORDING);
+  HIP_TRY(hipStreamSynchronize(R.stream));  // (a run of it may still be in flight)
+  hipGraphExecDestroy(l->exec);
+  hipGraphDestroy(l->graph);
+  R.lists.erase(l);
+  delete l;
+  return ARCZ_OK;
 }
 
 void arcz_set_oom_hook(int (*hook)(void)) { R.oom_hook = hook; }

@@ -27,6 +27,7 @@ extern "C" {
 #define ARCZ_E_ARG_VALUE (-50)     /* CL_INVALID_ARG_VALUE: a pointer argument that is no live buffer */
 #define ARCZ_E_ARG_SIZE (-51)      /* CL_INVALID_ARG_SIZE (clrt.h:900-903) */
 #define ARCZ_E_WORK_GROUP (-54)    /* CL_INVALID_WORK_GROUP_SIZE: global not a multiple of local (clrt.h:973-981) */
+#define ARCZ_E_RECORDING (-59)     /* CL_INVALID_OPERATION: a call that a launch list being recorded cannot hold, or a list call out of place */
 #define ARCZ_E_GLOBAL_SIZE (-63)   /* CL_INVALID_GLOBAL_WORK_SIZE: a size past 32 bits (clrt.h:943-947) */
 
 typedef struct arcz_mem arcz_mem;       /* the reference's cl_mem = ZMem {ptr, size, owner} (clrt.h:41-46) */
@@ -98,6 +99,23 @@ void arcz_event_release(arcz_event* e);
 /* Timestamps on the stream without a launch of their own: a pair brackets any sequence of launches. */
 arcz_event* arcz_event_record(void);
 double arcz_event_elapsed_ms(arcz_event* start, arcz_event* stop);
+
+/* Recorded launch lists: the reference's ARC_BATCH (clrt.h:170-265 -- kernels recorded into regular command lists and
+ * handed to the GPU a list at a time instead of one by one), here a HIP graph captured from the stream.  Between
+ * arcz_record_begin and arcz_record_end, arcz_launch without an event (and arcz_fill of whole words, which is a kernel)
+ * add to the list and nothing runs; every call that allocates, frees, copies, waits or times returns
+ * ARCZ_E_RECORDING (NULL where it returns a handle) and leaves the recording as it is -- so run a sequence once
+ * before recording it, so that every buffer it needs exists.  arcz_record_end(NULL) drops the recording.
+ * arcz_list_run submits the whole list (in stream order with everything else); it works on the buffers named when it
+ * was recorded, with what they hold when it runs, so new input goes into the same buffers.  A list must be freed
+ * before the buffers it names. */
+typedef struct arcz_list arcz_list;
+int arcz_record_begin(void);
+int arcz_record_end(arcz_list** out);
+int arcz_recording(void);
+int arcz_list_run(arcz_list* l);
+uint64_t arcz_list_launches(const arcz_list* l);
+int arcz_list_free(arcz_list* l);
 
 /* zrt::oom_hook (clrt.h:148-168): called when an allocation fails; returns nonzero if it freed something. */
 void arcz_set_oom_hook(int (*hook)(void));
