@@ -167,6 +167,46 @@ def bench_decode(az, qtype, N, K, T, launches, copies):
             "distinct_weight_MB": copies * az.gguf_bytes(qtype, N, K) / 1e6}
 
 
+def bench_launch_list(az, N=2048, layers=32, reps=40):
+    """A decode-like chain of small launches -- `layers` times (quantize one token, GEMV N x N Q4_K) -- issued launch
+    by launch and as one recorded list (arcz_record_begin / arcz_list_run): device time per launch, both ways."""
+    eng = az.Engine(16, N)
+    W = az.gen_weights(az.Q4_K, 9, N, N, 0.02)
+    ws = [eng.make_weight(az.Q4_K, N, N, W) for _ in range(4)]
+    bufs = [az.Runtime.from_numpy(az.gen_normal(10, (1, N))), az.Runtime.alloc(N * 4)]
+
+    def step():
+        for i in range(layers):
+            eng.quantize(bufs[i % 2], N, N, 16, 1)
+            eng.matmul("chain", ws[i % 4], 16, bufs[(i + 1) % 2], N, 0, 0)
+
+    def timed(fn):
+        settle(az, fn)
+        e0 = az.Runtime.event()
+        for _ in range(reps):
+            fn()
+        e1 = az.Runtime.event()
+        az.Runtime.sync()
+        ms = az.Runtime.elapsed_ms(e0, e1)
+        az.Runtime.event_release(e0)
+        az.Runtime.event_release(e1)
+        return ms
+
+    step()
+    lst = az.Runtime.record(step)
+    n = lst.launches
+    eager_ms, list_ms = timed(step), timed(lst.run)
+    lst.free()
+    for w in ws:
+        w.free()
+    for b in bufs:
+        b.free()
+    eng.close()
+    return {"launches_per_step": int(n), "eager_us_per_launch": eager_ms / reps / n * 1e3,
+            "list_us_per_launch": list_ms / reps / n * 1e3, "eager_us_per_step": eager_ms / reps * 1e3,
+            "list_us_per_step": list_ms / reps * 1e3, "shape": [N, N], "layers": layers}
+
+
 def bench_types(az, N=17408, K=5120):
     """Every weight type on the headline matrix: GEMV over 1, 2, 8 and 16 tokens (cycling through distinct weight
     buffers, as bench_decode) and the prefill GEMM at 2048 tokens.  Not part of the default run (--types)."""
@@ -474,7 +514,9 @@ def main():
         log(f"[bench] decode T=8: {d8}")
         d86 = bench_decode(az, az.Q6_K, 5120, 17408, 8, 200, 6)
         log(f"[bench] decode T=8 Q6_K: {d86}")
-        out["decode"] = {"Q4_K_17408x5120_T1": d1, "Q4_K_5120x17408_T2": d2, "Q4_K_gate_up_2x17408x5120_T1": dgu,
+        dll = bench_launch_list(az)
+        log(f"[bench] chain of small launches, eager and as a recorded list: {dll}")
+        out["decode"] = {"launch_list_chain_Q4_K_2048x2048_T1": dll, "Q4_K_17408x5120_T1": d1, "Q4_K_5120x17408_T2": d2, "Q4_K_gate_up_2x17408x5120_T1": dgu,
                          "Q4_K_17408x5120_T8": d8, "Q6_K_5120x17408_T8": d86, "hbm_peak_GBps": PEAK_HBM_GBS}
     if not args.no_extras:
         az.self_check()
