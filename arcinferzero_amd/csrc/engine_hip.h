@@ -588,7 +588,12 @@ class Engine {
       // The main kernels stage the tokens' activations in LDS (gemv / gemv_mt); when T tokens of K values do not fit
       // the 64 KiB a launch may ask for, the kernels that read them from global memory take over (gemv_v / gemv_mt_v).
       const int ups = w.type == GGML_Q8_0 ? 16 : 8, units = K / 256 * ups;
-      const int tok_bytes = (w.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (w.type == GGML_Q4_K || w.type == GGML_Q5_K ? 8 : 4));
+      // (a token's bytes in LDS: 16 values and a scale per unit and part; Q4_K / Q5_K: the scale times the block sum
+      //  beside it; Q6_K in the one-token kernel: the 16 values' sum)
+      auto tokb = [&](int slots) {
+        const bool wide = w.type == GGML_Q4_K || w.type == GGML_Q5_K || (w.type == GGML_Q6_K && slots == 1);
+        return (w.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (wide ? 8 : 4));
+      };
       static const int force_v = getenv("ARCZ_GEMV_V") ? atoi(getenv("ARCZ_GEMV_V")) : 0;
       // lanes per row: the fewest of 32 / 64 / 128 / 256 that leave a lane at most 6 sixteen-byte units of a row
       static const int force_lpr = getenv("ARCZ_GEMV_LPR") ? atoi(getenv("ARCZ_GEMV_LPR")) : 0;
@@ -602,7 +607,7 @@ class Engine {
       const int bt = lpr >= 128 && (T == 2 || (T == 1 && bt_env == 512)) && !q2_fuse_ && bt_env != 256 ? 512 : 256;
       const int g = lpr ? bt / lpr : 1, wpr = lpr > 64 ? lpr / 64 : 1;
       // the kernel's token slots: T rounded up, or -- both halves of two-pass inputs in one launch -- 2 T rounded up
-      auto lds_of = [&](int slots) { return (size_t)slots * tok_bytes + (wpr > 1 ? (size_t)16 * g * wpr * slots * 4 : 0); };  // (16: the kernels' GEMV_FLUSH)
+      auto lds_of = [&](int slots) { return (size_t)slots * tokb(slots) + (wpr > 1 ? (size_t)16 * g * wpr * slots * 4 : 0); };  // (16: the kernels' GEMV_FLUSH)
       const int tb2 = T == 1 ? 2 : T == 2 ? 4 : 8;
       const bool q2f = q2_fuse_ && T <= 4 && lpr && lds_of(tb2) <= (w.type == GGML_IQ3_S || w.type == GGML_IQ3_XXS ? 65536 - 2048 : 65536);
       const int tbl = q2f ? tb2 : T <= 2 ? T : T <= 4 ? 4 : 8;
@@ -674,7 +679,7 @@ class Engine {
                                ", the matrices take " + std::to_string(Mp) + " x " + std::to_string(g.K));
     const int N = g.N, K = g.K;
     const int ups = g.type == GGML_Q8_0 ? 16 : 8, units = K / 256 * ups;
-    const int tok_bytes = (g.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (g.type == GGML_Q4_K || g.type == GGML_Q5_K ? 8 : 4));
+    const int tok_bytes = (g.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (g.type == GGML_Q4_K || g.type == GGML_Q5_K || g.type == GGML_Q6_K ? 8 : 4));
     int lpr = 0;
     for (int l : {32, 64, 128, 256})
       if (!lpr && (units + l - 1) / l <= 6) lpr = l;
