@@ -591,7 +591,8 @@ class Engine {
       // (a token's bytes in LDS: 16 values and a scale per unit and part; Q4_K / Q5_K: the scale times the block sum
       //  beside it; Q6_K in the one-token kernel: the 16 values' sum)
       auto tokb = [&](int slots) {
-        const bool wide = w.type == GGML_Q4_K || w.type == GGML_Q5_K || (w.type == GGML_Q6_K && slots == 1);
+        const bool wide = w.type == GGML_Q4_K || w.type == GGML_Q5_K ||
+                          ((w.type == GGML_Q6_K || w.type == GGML_Q3_K) && slots == 1);
         return (w.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (wide ? 8 : 4));
       };
       static const int force_v = getenv("ARCZ_GEMV_V") ? atoi(getenv("ARCZ_GEMV_V")) : 0;
@@ -679,7 +680,7 @@ class Engine {
                                ", the matrices take " + std::to_string(Mp) + " x " + std::to_string(g.K));
     const int N = g.N, K = g.K;
     const int ups = g.type == GGML_Q8_0 ? 16 : 8, units = K / 256 * ups;
-    const int tok_bytes = (g.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (g.type == GGML_Q4_K || g.type == GGML_Q5_K || g.type == GGML_Q6_K ? 8 : 4));
+    const int tok_bytes = (g.type == GGML_Q8_0 ? 1 : 2) * units * (16 + (g.type == GGML_Q4_K || g.type == GGML_Q5_K || g.type == GGML_Q6_K || g.type == GGML_Q3_K ? 8 : 4));
     int lpr = 0;
     for (int l : {32, 64, 128, 256})
       if (!lpr && (units + l - 1) / l <= 6) lpr = l;
