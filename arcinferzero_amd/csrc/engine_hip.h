@@ -634,7 +634,14 @@ class Engine {
         static const int wgs_env = getenv("ARCZ_GEMV_WGS") ? atoi(getenv("ARCZ_GEMV_WGS")) : 0;
         const bool codebook = w.type == GGML_IQ4_XS || w.type == GGML_IQ3_S || w.type == GGML_IQ4_NL || w.type == GGML_MXFP4 ||
                               w.type == GGML_IQ3_XXS;
-        const int wpc = wpc_env > 0 ? wpc_env : bt == 512 || (tb == 1 && !codebook) ? 1 : 2;
+        // (Q6_K, one token, since its kernel takes the - 32 off the sums: two work-groups a unit are ahead on matrices
+        //  of layer size -- 17408 x 5120 16.4 -> 15.9 us, 5120 x 17408 16.3 -> 15.9, 8192 x 8192 12.8 -> 12.3 -- and
+        //  behind on the 151936 x 5120 output head, 106.3 -> 110.3)
+        // (Q3_K, one token: two everywhere -- 17408 x 5120 11.6 -> 10.7 us, 5120 x 17408 13.5 -> 11.3, 4096 x 4096
+        //  5.0 -> 4.6; Q5_K and Q8_0 measured beside it stay at one: 12.8 -> 13.1 and 16.9 -> 17.1)
+        const bool q6_mid = (w.type == GGML_Q6_K && tb == 1 && (size_t)N * (size_t)K <= ((size_t)1 << 28)) ||
+                            (w.type == GGML_Q3_K && tb == 1);
+        const int wpc = wpc_env > 0 ? wpc_env : bt == 512 || (tb == 1 && !codebook && !q6_mid) ? 1 : 2;
         size_t wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)arcz_device_cus() * wpc);
         if (wgs_env > 0) wgs = std::min<size_t>((size_t)(N + g - 1) / g, (size_t)wgs_env);
         const std::string defs = "-DQT=" + std::to_string(w.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" +
