@@ -507,6 +507,35 @@ class Engine {
     return w.N <= 4096 ? 1 : 2;
   }
 
+  // The LDS-staged GEMVs' -DSCHED: how the rows of a launch of `wgs` work-groups of `g` rows a pass are dealt out (the
+  // kernels would work it out themselves, in their first microsecond).  Whole rounds << 10 | rows of the one shorter
+  // pass that every work-group gets of the rows left over -- when that is at least half a pass; else whole passes for
+  // the first work-groups -- and, for two matrices in one launch, whole rounds << 10 | work-groups with a pass more.
+  // Bit 30: the weight stream is read with non-temporal loads -- measured to pay from about 40 MB of matrix on (one
+  // token, us with / without: Q4_K 17408 x 5120 10.0 / 10.4, Q8_0 15.5 / 16.4; 8192 x 8192 8.6 / 8.5, 4096 x 4096
+  // 4.7 / 4.55), but not for one token over rows of 128 lanes and more (Q4_K 5120 x 17408: 11.15 / 10.9; two tokens,
+  // in work-groups of 512: 12.65 / 13.2).  ARCZ_GEMV_NT=0 / 1: never / always.
+  // `short_tail`: the rows left over go out as one short pass a work-group (one and two tokens of the types decoded
+  // without a table -- GemvLds<QT>::short_tail: Q4_K one token 17408 x 5120 on 256 work-groups, 4 rows each, 10.6 ->
+  // 10.5 us; Q6_K on 512, 2 rows each, 15.9 -> 14.8); otherwise as whole passes for the first work-groups (a short pass
+  // still issues a whole pass's loads and takes a whole pass's time in the kernels bound by their arithmetic: IQ3_XXS
+  // 12.1 -> 12.4 us, Q4_K four tokens 18.6 -> 20.8 with it).
+  static int gemv_sched(int rows, int g, size_t wgs, bool two_matrices, size_t bytes, bool long_rows_one_token,
+                        bool short_tail = false) {
+    static const int nt_env = getenv("ARCZ_GEMV_NT") ? atoi(getenv("ARCZ_GEMV_NT")) : -1;
+    const bool nt = nt_env >= 0 ? nt_env != 0 : bytes >= ((size_t)40 << 20) && !long_rows_one_token;
+    const int ntb = nt ? 1 << 30 : 0;
+    const int nw = (int)wgs;
+    if (two_matrices) {
+      const int npass = (rows + g - 1) / g;
+      return ((npass / nw) << 10) | (npass % nw) | ntb;
+    }
+    const int full = rows / (g * nw);
+    int tail = (rows - full * g * nw + nw - 1) / nw;
+    if (!short_tail || tail == 0) tail = g;
+    return (full << 10) | tail | ntb;
+  }
+
   void matmul1(const char* name, const GpuWeight& w, int Mp, cl_mem C, int ldc, int c_off, int acc, bool act32) {
     if (!w.raw) throw std::runtime_error(std::string("matmul ") + name + ": the weight is not loaded");
     if (cur_T_ <= 0 || w.K != cur_K_ || Mp != cur_Mp_)
@@ -649,7 +678,7 @@ class Engine {
                                  (bt == 512 ? " -DBT=512" : "") + " -DLDS=" +
                                  std::to_string(lds) +
                                  (q2f ? " -DQ2_AQ=" + std::to_string(q2_aq_) + " -DQ2_SC=" + std::to_string(q2_sc_ / 4) : std::string()) +
-                                 head_defs(w);
+                                 head_defs(w) + " -DSCHED=" + std::to_string(gemv_sched(N, g, wgs, false, raw_bytes(w), lpr >= 128 && tb == 1 && bt == 256, !codebook && tb <= 2));
         cl_kernel k = kernel("decode", defs, tb == 1 ? "gemv" : "gemv_mt");
         int ld1 = T == 1 ? 0 : ldc;  // (one token: C is the row itself)
         if (tb == 1) set_args(k, 0, w.raw, N, K, tabs, aq_, asc_, absum_, M, C, c_off, a);
@@ -698,14 +727,15 @@ class Engine {
     if (arcz_mem_size(C) < (size_t)2 * N * 4) throw std::runtime_error("gemv_gu: the output does not fit C");
     rd_bytes += raw_bytes(g) + raw_bytes(u);
     const int pf = (units + lpr - 1) / lpr;
+    static const int gu_wpc = getenv("ARCZ_GEMV_GU_WPC") ? atoi(getenv("ARCZ_GEMV_GU_WPC")) : 1;  // (17.6 against 18.2 us with two)
+    const size_t wgs = std::min<size_t>((size_t)2 * N / gr, (size_t)arcz_device_cus() * gu_wpc);
     const std::string defs = "-DQT=" + std::to_string(g.type) + " -DLPR=" + std::to_string(lpr) + " -DPF=" + std::to_string(pf) +
-                             " -DLDS=" + std::to_string(lds) + " -DGU2";
+                             " -DLDS=" + std::to_string(lds) + " -DGU2 -DSCHED=" +
+                             std::to_string(gemv_sched(2 * N, gr, wgs, true, raw_bytes(g) + raw_bytes(u), lpr >= 128));
     cl_kernel k = kernel("decode", defs, "gemv");
     cl_mem tabs = tabs_;
     int NN = N, KK = K, M = Mp, c_off = 0, a = 0;
     set_args(k, 0, g.raw, NN, KK, tabs, aq_, asc_, absum_, M, C, c_off, a, u.raw);
-    static const int gu_wpc = getenv("ARCZ_GEMV_GU_WPC") ? atoi(getenv("ARCZ_GEMV_GU_WPC")) : 1;  // (17.6 against 18.2 us with two)
-    const size_t wgs = std::min<size_t>((size_t)2 * N / gr, (size_t)arcz_device_cus() * gu_wpc);
     size_t g1 = wgs * 256, l1 = 256;
     run("gemm_gate_up", k, 1, &g1, &l1);
     return true;

@@ -40,13 +40,17 @@ static const KernelSpec kKernelTable[] = {
     {"ops", "read_probe", nullptr, "pzp", {nullptr}, {{nullptr, 0, false}}, 256},
     {"ops", "mfma_probe", nullptr, "pi", {nullptr}, {{nullptr, 0, false}}, 256},
     // ---- decode
-    {"decode", "gemv", "GU2", "piippppipiip", {"QT", "LPR", "PF", "GU2", nullptr}, {{"LDS", 0, true}, {nullptr, 0, false}}, 256},
-    {"decode", "gemv", "BT", "piippppipii", {"QT", "LPR", "PF", "BT", nullptr}, {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 512},
+    // (-DSCHED=n: the LDS-staged GEMVs' row schedule for the launch's grid, worked out by the launcher -- see
+    //  gemv_lds.inc; left out, the kernel works it out itself)
+    {"decode", "gemv", "GU2", "piippppipiip", {"QT", "LPR", "PF", "GU2", nullptr}, {{"LDS", 0, true}, {"SCHED", -1, false}, {nullptr, 0, false}}, 256},
+    {"decode", "gemv", "BT", "piippppipii", {"QT", "LPR", "PF", "BT", nullptr},
+     {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {"SCHED", -1, false}, {nullptr, 0, false}}, 512},
     {"decode", "gemv_mt", "BT", "piippppiipiii", {"QT", "LPR", "PF", "TB", "BT", nullptr},
-     {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 512},
-    {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr}, {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
+     {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {"SCHED", -1, false}, {nullptr, 0, false}}, 512},
+    {"decode", "gemv", nullptr, "piippppipii", {"QT", "LPR", "PF", nullptr},
+     {{"LDS", 0, true}, {"SOFTCAP", 0, false}, {"SCHED", -1, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mt", nullptr, "piippppiipiii", {"QT", "LPR", "PF", "TB", nullptr},
-     {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
+     {{"LDS", 0, true}, {"Q2_AQ", 0, false}, {"Q2_SC", 0, false}, {"SOFTCAP", 0, false}, {"SCHED", -1, false}, {nullptr, 0, false}}, 256},
     {"decode", "gemv_mm_reduce", nullptr, "pipiiiii", {nullptr}, {{nullptr, 0, false}}, 256},
     {"decode", "gemv_mm", nullptr, "piippppiipiiiii", {"QT", nullptr}, {{nullptr, 0, false}}, 512},
     {"decode", "moe_gateup_q", "ROUTE", "ppiipppippppipppppppiiipp", {"QT", "GROWS", "TM", "QUANT", "ROUTE", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 512},

@@ -180,3 +180,45 @@ def test_gemv_softcap_output_head(eng, qtype, N, K, T):
     for b in (plain, capped, capped_acc, xb):
         b.free()
     w.free()
+
+
+def _sched(rows, g, wgs):
+    """Engine::gemv_sched for one matrix: whole rounds << 10 | rows of the last, shorter pass."""
+    full = rows // (g * wgs)
+    tail = (rows - full * g * wgs + wgs - 1) // wgs or g   # (Q4_K, one or two tokens: a short last pass whatever its size)
+    return (full << 10) | tail
+
+
+@pytest.mark.parametrize("N,K,T", [(1000, 1024, 1), (1001, 1024, 2), (2176, 2048, 1), (333, 5120, 1), (96, 17408, 2)])
+def test_gemv_row_schedule(eng, N, K, T):
+    """The LDS-staged GEMV deals its rows out by the grid it is launched with; the schedule comes from the launcher
+    (-DSCHED) or, left out, from the kernel's own arithmetic.  Whatever the grid and whoever works the schedule out, every
+    row is computed once, by the same lanes in the same order: the output equals the engine's launch bit for bit."""
+    qtype, Mp = az.Q4_K, 16
+    print(f"gemv schedule N={N} K={K} T={T}", flush=True)
+    W = make_weights(qtype, N, K, seed=5)
+    x = make_acts(T, K, seed=6)
+    ref = run_gemv(eng, qtype, W, N, K, x, Mp)
+    units = K // 256 * 8
+    lpr = next(l for l in (32, 64, 128, 256) if (units + l - 1) // l <= 6)
+    pf, g, wpr = (units + lpr - 1) // lpr, 256 // lpr, max(1, lpr // 64)
+    lds = T * 2 * units * 24 + (16 * g * wpr * T * 4 if wpr > 1 else 0)
+    raw = az.Runtime.from_numpy(az.repack_planes(qtype, N, K, W))
+    xb = az.Runtime.from_numpy(x)
+    eng.quantize(xb, K, K, Mp, T)
+    cb = az.Runtime.alloc(T * N * 4)
+    npass = (N + g - 1) // g
+    for wgs in sorted({1, 3, min(37, npass), max(1, npass // 2), npass}):
+        for given in (0, 1, 2):   # the kernel's own schedule; the launcher's; the launcher's with non-temporal weight loads
+            defs = f"-DQT={qtype} -DLPR={lpr} -DPF={pf}" + (f" -DTB={T}" if T > 1 else "") + f" -DLDS={lds}"
+            if given:
+                defs += f" -DSCHED={_sched(N, g, wgs) | ((1 << 30) if given == 2 else 0)}"
+            k = az.Runtime.kernel("decode", defs, "gemv" if T == 1 else "gemv_mt")
+            cb.fill(0xFFFFFFFF)
+            args = [raw, N, K, None, eng.aq, eng.asc, eng.absum, Mp]
+            args += [cb, 0, 0] if T == 1 else [T, cb, N, 0, 0]
+            az.Runtime.launch(k, (wgs * 256,), (256,), args)
+            y = cb.read(np.float32, T * N).reshape(T, N)
+            assert np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (wgs, given)
+    for b in (raw, xb, cb):
+        b.free()
