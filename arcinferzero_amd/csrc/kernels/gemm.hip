@@ -397,6 +397,11 @@ __device__ inline v8bf as_bf16x8(v4u v) { return __builtin_bit_cast(v8bf, v); }
 #define G3_WS (G3_SA + 4096)
 #define G3_V (G3_SA + 6144)
 
+// A result leaves for good: non-temporal stores keep the output (570 MB for 8192 tokens x 17408 rows, more than every
+// cache) from displacing the operands that the neighbouring tiles still read (8192 tokens: 707 -> 717 TOP/s).  (Not for
+// the expert tiles' y rows, which moe_combine reads right back: 56 -> 62 us there.)
+__device__ inline void st_stream(float* p, float v) { __builtin_nontemporal_store(v, p); }
+
 __device__ inline void g3_dma16(const void* src, uint8_t* lds_wave_base) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                    (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
@@ -827,7 +832,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
           const float gt = *cp;
           v *= gt / (1.0f + __expf(-gt));
         }
-        *cp = v;
+        st_stream(cp, v);
       }
     }
 }
@@ -1893,7 +1898,12 @@ __device__ __forceinline__ void gemm8_body(const uint8_t* __restrict__ raw, cons
 
 // Tile of work-group `id` out of mt x nt tiles.  XCDs take work-groups in turn (id % 8), each running 64 at a time:
 // those 64 are made an 8 x 8 block of tiles when both tile counts are multiples of 8 and the blocks share out evenly
-// over the 8 XCDs; token tiles fastest otherwise.
+// over the 8 XCDs.  Any other shape: the tiles are put in the order "panels of 8 token tiles; within a panel row tile
+// by row tile" and that list is cut into 8 runs, one per XCD (XCD x's j-th work-group takes the j-th tile of run x), so
+// that the 64 tiles an XCD works on are 8 token tiles x 8 row tiles whose successors keep the same token tiles: the
+// panel's activations stay in the XCD's L2 while the weight rows stream through it once per panel.  (Token tiles
+// fastest over the whole grid, as it was, gave every XCD 4 token tiles x 16 row tiles and every row tile to all 8 XCDs:
+// the 151936 x 5120 Q6_K head at 2048 tokens read 6.9 GB from memory for 0.65 GB of input.)
 __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
   if ((mt & 7) == 0 && (nt & 7) == 0 && (((mt >> 3) * (nt >> 3)) & 7) == 0) {  // (whole 8 x 8 blocks, 8 XCDs' worth)
     const int x = id & 7, q = id >> 3;
@@ -1902,8 +1912,11 @@ __device__ inline void tile_of(int id, int mt, int nt, int& tm, int& tn) {
     tm = (st % smt) * 8 + (within & 7);
     tn = (st / smt) * 8 + (within >> 3);
   } else {
-    tm = id % mt;
-    tn = id / mt;
+    const int total = mt * nt, x = id & 7, j = id >> 3;
+    const int L = x * (total >> 3) + min(x, total & 7) + j;  // (XCD y has total / 8 tiles, one more if y < total % 8)
+    const int panel = L / (8 * nt), rem = L - panel * 8 * nt, pw = min(8, mt - panel * 8);
+    tn = rem / pw;
+    tm = panel * 8 + rem - tn * pw;
   }
 }
 
