@@ -89,6 +89,7 @@ _sig("arcz_gguf_find", C.c_long, _p, C.c_char_p)
 _sig("arcz_ggml_block_info", _i, _u32, C.POINTER(_i), C.POINTER(_i))
 _sig("arcz_weight_free", _i, _p, _p)
 _sig("arcz_weight_raw", _p, _p)
+_sig("arcz_mem_listed", C.c_int, _p)
 _sig("arcz_weight_k", C.c_int, _p)
 _sig("arcz_moe_layer_dims", C.c_int, _p, C.POINTER(C.c_int), C.POINTER(C.c_int))
 _sig("arcz_engine_quantize", _i, _p, _p, _i, _i, _i, _i, _i)

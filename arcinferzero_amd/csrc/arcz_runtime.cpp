@@ -38,6 +38,7 @@ struct arcz_list {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
   uint64_t launches = 0;  // kernels recorded
+  std::set<arcz_mem*> owners;  // the allocations its kernels' buffer arguments lie in: not to be freed while it lives
 };
 
 namespace {
@@ -57,6 +58,7 @@ struct Runtime {
   std::string err;
   arcz_mem* scratch = nullptr;  // non-owning handle onto the device's static scratch array (arcz_scratch.hip)
   bool recording = false;       // between arcz_record_begin and arcz_record_end: launches go into a list, not to the GPU
+  std::set<arcz_mem*> rec_owners;  // ... and the allocations their buffer arguments lie in
   uint64_t rec_launches = 0;
   std::set<arcz_list*> lists;
 };
@@ -240,6 +242,9 @@ int arcz_free(arcz_mem* m) {
     //  memory: refused, nothing is freed)
     for (const arcz_mem* v : R.mems)
       if (v->parent == m) return fail(ARCZ_E_ARG_VALUE, "arcz_free of a buffer that still has live views");
+    // (a recorded list keeps the device addresses of the buffers its kernels were given: it would read and write
+    //  freed memory.  Refused, nothing is freed: free the list first)
+    if (arcz_mem_listed(m)) return fail(ARCZ_E_ARG_VALUE, "arcz_free of a buffer that a live launch list names");
     HIP_TRY(hipStreamSynchronize(R.stream));
     HIP_TRY(hipFree(m->ptr));
     R.device_bytes -= m->size;
@@ -249,6 +254,13 @@ int arcz_free(arcz_mem* m) {
   return ARCZ_OK;
 }
 
+int arcz_mem_listed(const arcz_mem* m) {
+  if (!m || !R.mems.count(const_cast<arcz_mem*>(m))) return 0;
+  arcz_mem* o = m->owner ? const_cast<arcz_mem*>(m) : m->parent;
+  for (const arcz_list* l : R.lists)
+    if (l->owners.count(o)) return 1;
+  return 0;
+}
 size_t arcz_mem_size(const arcz_mem* m) { return m && R.mems.count(const_cast<arcz_mem*>(m)) ? m->size : 0; }
 void* arcz_mem_ptr(const arcz_mem* m) { return m && R.mems.count(const_cast<arcz_mem*>(m)) ? m->ptr : nullptr; }
 
@@ -321,6 +333,7 @@ int arcz_fill(arcz_mem* dst, const void* pattern, size_t ps, size_t offset, size
     HIP_TRY(hipModuleLaunchKernel(k->fn, blocks, 1, 1, 256, 1, 1, 0, R.stream, params, nullptr));
     if (R.recording) {  // (recorded as the kernel it is; nothing to wait for)
       ++R.rec_launches;
+      R.rec_owners.insert(dst->owner ? dst : dst->parent);
       return ARCZ_OK;
     }
   } else {
@@ -479,6 +492,7 @@ int arcz_launch(arcz_kernel* k, unsigned dim, const size_t* global, const size_t
         if (!R.mems.count(m))
           return fail(ARCZ_E_ARG_VALUE, "%s: argument %u is not a live buffer", k->symbol.c_str(), i);
         memcpy(store[i], &m->ptr, 8);
+        if (R.recording) R.rec_owners.insert(m->owner ? m : m->parent);
       }
     }
     params[i] = store[i];
@@ -558,6 +572,7 @@ int arcz_record_begin(void) {
   HIP_TRY(hipStreamBeginCapture(R.stream, hipStreamCaptureModeThreadLocal));
   R.recording = true;
   R.rec_launches = 0;
+  R.rec_owners.clear();
   return ARCZ_OK;
 }
 int arcz_record_end(arcz_list** out) {
@@ -581,7 +596,8 @@ int arcz_record_end(arcz_list** out) {
     hipGraphDestroy(g);
     return fail(ARCZ_E_DEVICE, "the recorded list does not instantiate: %s", hipGetErrorString(e));
   }
-  arcz_list* l = new arcz_list{g, x, R.rec_launches};
+  arcz_list* l = new arcz_list{g, x, R.rec_launches, R.rec_owners};
+  R.rec_owners.clear();
   R.lists.insert(l);
   *out = l;
   return ARCZ_OK;

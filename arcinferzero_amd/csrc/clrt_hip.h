@@ -71,10 +71,28 @@ inline void check(int err, const char* what, const char* file, int line) {
 }  // namespace arcz
 #define CL_CHECK(x) arcz::check((x), #x, __FILE__, __LINE__)
 
+// zrt::oom_throws (zero/clrt.h:148-168, 474-487): what an allocation does once the out-of-memory hook has given up --
+// the reference never hands a failed allocation back to its caller: it ends the process with the sizes that say why,
+// or, while this thread-local switch is set (a model being placed that the caller can still load elsewhere), throws.
+namespace zrt {
+inline thread_local bool oom_throws = false;
+}  // namespace zrt
+
 inline cl_int clFinish(cl_command_queue) { return arcz_sync(); }
 inline cl_int clFlush(cl_command_queue) { return CL_SUCCESS; }
 inline cl_mem clCreateBuffer(cl_context, cl_mem_flags flags, size_t n, void* host, cl_int* err) {
   cl_mem m = arcz_alloc(n);
+  // (out of memory -- the hook was called and could free nothing more, or there is none -- as against a call before
+  //  arcz_init or inside a recording, which come back as errors: told apart by the runtime's message)
+  if (!m && strncmp(arcz_last_error(), "allocation of", 13) == 0) {
+    char msg[256];
+    snprintf(msg, sizeof msg, "device allocation of %.1f MB failed (%.2f GiB allocated): %s", n / 1e6,
+             arcz_device_bytes() / 1073741824.0, arcz_last_error());
+    if (zrt::oom_throws) throw std::runtime_error(msg);
+    fprintf(stderr, "arcz: %s\n", msg);
+    fflush(stderr);
+    _Exit(1);
+  }
   cl_int e = m ? CL_SUCCESS : ARCZ_E_OOM;
   if (m && (flags & CL_MEM_COPY_HOST_PTR) && host) e = arcz_h2d(m, 0, host, n);
   if (err) *err = e;

@@ -75,6 +75,13 @@ class Engine {
     // the short-chunk GEMM's workspace, sized once for the most its launch rule can ask for (below: pieces x tiles
     // within two work-groups per compute unit, tiles of at most 128 x 128 f32), so that no matmul allocates or frees
     sk_force_ = getenv("ARCZ_Q4_SPLITK") ? atoi(getenv("ARCZ_Q4_SPLITK")) : -1;
+    // the expert layer's launch-rule switches, read when the engine is made (a one-token layer is 16 us: nothing of
+    // the environment is looked up per call)
+    moe_dec_off_ = getenv("ARCZ_MOE_DECODE") && atoi(getenv("ARCZ_MOE_DECODE")) == 0;
+    moe_dec_max_ = getenv("ARCZ_MOE_DECODE_MAX") ? atoi(getenv("ARCZ_MOE_DECODE_MAX")) : 16;
+    moe_tmd_ = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
+    moe_fuse_off_ = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
+    moe_qfuse_off_ = getenv("ARCZ_MOE_QFUSE") && atoi(getenv("ARCZ_MOE_QFUSE")) == 0;
     sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
     sk_ws_ = buf(sk_ws_bytes_);
     // the codebook tables the kernels take as `tabs` (the reference's tabs_, zero/engine_setup.h): IQ3_S's 512 entries
@@ -139,6 +146,7 @@ class Engine {
     // (checked before anything is changed: a refusal leaves the engine as it was)
     if (on && (size_t)max_chunk * max_k >= (1ull << 31))
       throw std::invalid_argument("two-pass mode: a chunk of max_chunk x max_k values must stay below 2 GiB");
+    for (cl_mem m : {aq_, asc_, absum_}) not_listed(m, "set_two_pass (the activation buffers are made anew)");
     for (cl_mem* v : {&aq2_, &asc2_, &absum2_})
       if (*v) { release(*v); *v = nullptr; }
     release(aq_); release(asc_); release(absum_);
@@ -182,10 +190,18 @@ class Engine {
     mems_.push_back(m);
     return m;
   }
+  // A recorded launch list keeps the device addresses its kernels were given, the engine's own workspaces among them:
+  // a buffer that a live list names is not freed or replaced (the list would read and write freed memory).  The call
+  // that wanted to throws, with the engine as it was; free the list first.
+  static void not_listed(cl_mem m, const char* what) {
+    if (m && arcz_mem_listed(m))
+      throw std::runtime_error(std::string(what) + ": a recorded launch list names this buffer (free the list first)");
+  }
   void release(cl_mem m) {
+    not_listed(m, "release");
+    CL_CHECK(clReleaseMemObject(m));
     auto it = std::find(mems_.begin(), mems_.end(), m);
     if (it != mems_.end()) mems_.erase(it);
-    CL_CHECK(clReleaseMemObject(m));
   }
 
   // (zero/engine_setup.h:317-362) one kernel object per (source, -D string, name)
@@ -748,6 +764,8 @@ class Engine {
   cl_mem sk_ws_ = nullptr;
   size_t sk_ws_bytes_ = 0;
   int sk_force_ = -1;  // ARCZ_Q4_SPLITK: 0 = never share K out, n >= 2: n pieces, -1 = the rule below
+  bool moe_dec_off_ = false, moe_fuse_off_ = false, moe_qfuse_off_ = false;  // ARCZ_MOE_DECODE / _FUSE / _QFUSE = 0
+  int moe_dec_max_ = 16, moe_tmd_ = 0;                                      // ARCZ_MOE_DECODE_MAX, ARCZ_MOE_TMD
   void gemm_dense(const char* name, const GpuWeight& w0, int Mp, cl_mem C, int ldc, int c_off, int a) {
     const GpuWeight w = gemm_form(name, w0);
     int M = Mp, N = w.N, K = w.K;
@@ -1054,17 +1072,17 @@ class Engine {
     // work-groups (128 us a layer at 128 experts x 768 x 2048; ARCZ_MOE_DECODE=0 brings that back).  At 128 x 8 experts
     // the two forms meet at 24 tokens (170 us); 16 tokens take 112 against 137 us (ARCZ_MOE_DECODE_MAX moves the limit).
     // (the four switches of this function are read at every call, so that a test can set them)
-    const bool dec_off = getenv("ARCZ_MOE_DECODE") && atoi(getenv("ARCZ_MOE_DECODE")) == 0;
-    const int dec_max = getenv("ARCZ_MOE_DECODE_MAX") ? atoi(getenv("ARCZ_MOE_DECODE_MAX")) : 16;
+    const bool dec_off = moe_dec_off_;
+    const int dec_max = moe_dec_max_;
     if (!dec_off && T <= dec_max && T * NU <= 512) {
       const int NE = L.NE;
       // (one-slot tiles at every count: eight tokens' 64 pairs hit about 50 experts, so a tile of 8 slots holds 1.3 on
       //  average, and the one-slot kernels are the light ones: 71 us a layer against 113 with 8-slot tiles, 45 against
       //  60 for four tokens; ARCZ_MOE_TMD=2|4|8 sets larger tiles)
-      const int tmd_env = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
+      const int tmd_env = moe_tmd_;
       const int tmd = T > 1 && (tmd_env == 2 || tmd_env == 4 || tmd_env == 8) ? tmd_env : 1;
       size_t tiles_max;
-      const bool fuse_off = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
+      const bool fuse_off = moe_fuse_off_;
       // one or two tokens, everything fused: the gate/up kernel routes the tokens itself (no routing launch: 2 launches
       // a layer; the kernel takes up to 8 tokens, but every work-group routes all of them, and from 4 tokens on the
       // routing launch is the cheaper way: 36.6 against 35.7 us at 4, 65.5 against 56.4 at 8)
@@ -1178,7 +1196,7 @@ class Engine {
       // zero/engine_moe.h:300-330): h = silu(gate) * up into mh_
       // ... and, when F is whole tiles of 128 rows, the expert inputs' quantization in the same kernel's epilogue
       // (-DQUANT=1: hq / hsc / hbs as moe_quant_sums makes them, bit for bit; ARCZ_MOE_QFUSE=0: the separate launch)
-      quant_fused = F % 128 == 0 && !(getenv("ARCZ_MOE_QFUSE") && atoi(getenv("ARCZ_MOE_QFUSE")) == 0);
+      quant_fused = F % 128 == 0 && !moe_qfuse_off_;
       cl_kernel k = kernel("gemm", std::string(quant_fused ? "-DQT=12 -DQUANT=1 -DNE=" : "-DQT=12 -DNE=") + std::to_string(L.NE), "moe_gateup_q");
       int FF = F, KK = E, MM = Mp, S = slots_;
       cl_mem tabs = nullptr;

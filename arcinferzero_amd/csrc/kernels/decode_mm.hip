@@ -53,7 +53,9 @@ typedef uint32_t mm_u4 __attribute__((ext_vector_type(4)));
 template <int QT> struct MmT;
 template <> struct MmT<QT_Q4_K> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 1, DPL = 0 }; };
 template <> struct MmT<QT_Q5_K> { enum { SB = 22, QB = 128, D = 4, XB = 32, MIN = 1, DPL = 0 }; };
-template <> struct MmT<QT_Q6_K> { enum { SB = 20, QB = 128, D = 4, XB = 64, MIN = 0, DPL = 1 }; };
+// (Q6_K: two -- with four the kernel needed 270 registers and kept 14 of them in scratch memory, 60 bytes a lane written
+//  and read back per superblock: 8 tokens at 17408 x 5120 31.1 -> 24.5 us)
+template <> struct MmT<QT_Q6_K> { enum { SB = 20, QB = 128, D = 2, XB = 64, MIN = 0, DPL = 1 }; };
 template <> struct MmT<QT_Q8_0> { enum { SB = 24, QB = 256, D = 4, XB = 0, MIN = 0, DPL = 0 }; };
 template <> struct MmT<QT_Q4_0> { enum { SB = 24, QB = 128, D = 8, XB = 0, MIN = 0, DPL = 0 }; };
 template <> struct MmT<QT_IQ4_NL> : MmT<QT_Q4_0> {};
@@ -164,7 +166,9 @@ __device__ inline void mm_slice(uint8_t* lds, const uint8_t* __restrict__ raw, i
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
       const uint32_t rel = (uint32_t)min(i * RPI + lane / LPRW, N - 1 - g0);
-      q.r[i] = *(const mm_u4*)(base + (__umul24(rel, row_stride) + piece_off));
+      // (the main plane is read once per launch: non-temporal, so that the caches keep the tokens and the small planes
+      //  -- 8 tokens, us: Q4_K 17408 x 5120 21.1 -> 20.5, 151936 x 5120 100 -> 96, Q8_0 155 -> 139)
+      q.r[i] = __builtin_nontemporal_load((const mm_u4*)(base + (__umul24(rel, row_stride) + piece_off)));
     }
   };
   auto hload = [&](mm_u4& h, int ub) {  // the headers of units ub .. ub + 3 (past the stretch: its last)

@@ -108,7 +108,9 @@ double arcz_event_elapsed_ms(arcz_event* start, arcz_event* stop);
  * before recording it, so that every buffer it needs exists.  arcz_record_end(NULL) drops the recording.
  * arcz_list_run submits the whole list (in stream order with everything else); it works on the buffers named when it
  * was recorded, with what they hold when it runs, so new input goes into the same buffers.  A list must be freed
- * before the buffers it names. */
+ * before the buffers it names: arcz_free of an allocation that a live list names (directly or through a view) is
+ * refused with ARCZ_E_ARG_VALUE and frees nothing.  arcz_mem_listed: 1 if a live list names the buffer's allocation
+ * (what the owner of internal workspaces asks before it replaces one). */
 typedef struct arcz_list arcz_list;
 int arcz_record_begin(void);
 int arcz_record_end(arcz_list** out);
@@ -116,6 +118,7 @@ int arcz_recording(void);
 int arcz_list_run(arcz_list* l);
 uint64_t arcz_list_launches(const arcz_list* l);
 int arcz_list_free(arcz_list* l);
+int arcz_mem_listed(const arcz_mem* m);
 
 /* zrt::oom_hook (clrt.h:148-168): called when an allocation fails; returns nonzero if it freed something. */
 void arcz_set_oom_hook(int (*hook)(void));

@@ -5,6 +5,7 @@
 // exit status (0 = every check held).
 #include <cstdint>
 #include <cstdio>
+#include <cstring>
 #include <vector>
 
 #include "clrt_hip.h"
@@ -65,6 +66,22 @@ int main() {
     thrown = true;
   }
   EXPECT(thrown);
+  // an allocation that fails after the out-of-memory hook has given up throws while zrt::oom_throws is set (it ends
+  // the process otherwise, as the reference's does): the runtime's test switch makes the next allocation fail
+  arcz_set_fake_oom(1);
+  zrt::oom_throws = true;
+  thrown = false;
+  try {
+    clCreateBuffer(cl.ctx, CL_MEM_READ_WRITE, 1 << 20, nullptr, &err);
+  } catch (const std::runtime_error& e) {
+    thrown = strstr(e.what(), "device allocation of") != nullptr;
+  }
+  arcz_set_fake_oom(0);
+  zrt::oom_throws = false;
+  EXPECT(thrown);
+  cl_mem after = clCreateBuffer(cl.ctx, CL_MEM_READ_WRITE, 1 << 20, nullptr, &err);
+  EXPECT(after && err == CL_SUCCESS);
+  CL_CHECK(clReleaseMemObject(after));
   clReleaseKernel(k);
   clReleaseKernel(kd);
   clReleaseProgram(p);

@@ -106,6 +106,8 @@ def test_an_expert_layer_step_as_a_list(rt):
             step()
             want = ob.read(np.float32, T * E)
             assert np.abs(want).max() > 0 and np.array_equal(y.view(np.uint32), want.view(np.uint32)), f"replay {i}"
+        lst.free()   # (a list before the buffers it names)
+        lst = None
         L.free()
         for b in (xb, lb, ob):
             b.free()
@@ -160,4 +162,49 @@ def test_what_a_list_cannot_hold_is_refused(rt):
             m.free()
         w.free()
     finally:
+        eng.close()
+
+
+def test_a_list_keeps_the_buffers_it_names(rt):
+    """A list holds the device addresses of the buffers its kernels were given -- the caller's and the engine's own
+    workspaces (a chunk of 256 token rows over a Q4_K matrix reads the ready-made scale vectors).  While the list lives
+    none of them is freed or replaced: the call that would have to is refused and leaves everything as it was, the list
+    still replays on valid memory, and once the list is freed the same calls go through."""
+    T = Mp = 256
+    N, K = 512, 1024
+    eng = az.Engine(Mp, 2048)
+    lst = None
+    try:
+        w = eng.make_weight(az.Q4_K, N, K, make_weights(az.Q4_K, N, K, seed=41))
+        xb = az.Runtime.from_numpy(make_acts(T, K, seed=42))
+        cb = az.Runtime.alloc(Mp * N * 4).fill(0)
+
+        def step():
+            eng.quantize(xb, K, K, Mp, T)
+            eng.matmul("listed", w, Mp, cb, N, 0, 0)
+
+        step()
+        ref = cb.read(np.float32, Mp * N).copy()
+        lst = az.Runtime.record(step)
+        assert az.lib.arcz_mem_listed(cb.h) == 1 and az.lib.arcz_mem_listed(xb.h) == 1
+        with pytest.raises(az.ArczError):        # the caller's output buffer
+            cb.free()
+        with pytest.raises(az.ArczError):        # a larger Q4_K matrix would replace the workspace of scale vectors
+            eng.make_weight(az.Q4_K, 4 * N, 2 * K, make_weights(az.Q4_K, 4 * N, 2 * K, seed=43))
+        with pytest.raises(az.ArczError):        # the activation buffers are made anew when the mode changes
+            eng.two_pass(True)
+        cb.fill(0xFFFFFFFF)
+        lst.run()
+        assert np.array_equal(cb.read(np.float32, Mp * N).view(np.uint32), ref.view(np.uint32))
+        lst.free()
+        lst = None
+        assert az.lib.arcz_mem_listed(cb.h) == 0
+        w2 = eng.make_weight(az.Q4_K, 4 * N, 2 * K, make_weights(az.Q4_K, 4 * N, 2 * K, seed=43))
+        w2.free()
+        for b in (xb, cb):
+            b.free()
+        w.free()
+    finally:
+        if lst is not None:
+            lst.free()
         eng.close()

@@ -106,8 +106,8 @@ def test_moe_layer_vs_oracle(rt, qtype, NE, NU, E, F, T, Mp):
 @pytest.mark.parametrize("qtype,NE,NU,E,F,T", [(az.Q4_K, 16, 4, 512, 256, 7), (az.Q6_K, 8, 3, 256, 256, 2),
                                                (az.Q5_K, 128, 8, 512, 256, 1)])
 def test_moe_small_pass_other_forms(rt, monkeypatch, env, qtype, NE, NU, E, F, T):
-    """The earlier forms of a small pass, which the launch-rule switches bring back (the engine reads them at every
-    call): larger tiles, the five-launch form, the tile GEMMs.  Same checks as the default form."""
+    """The earlier forms of a small pass, which the launch-rule switches bring back (an engine reads them when it is
+    made): larger tiles, the five-launch form, the tile GEMMs.  Same checks as the default form."""
     for k, v in env.items():
         monkeypatch.setenv(k, v)
     _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, 16)

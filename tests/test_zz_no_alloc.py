@@ -9,7 +9,8 @@ import numpy as np
 import pytest
 
 import arcinferzero_amd as az
-from common import make_acts, make_weights
+import oracle_lib as orc
+from common import make_acts, make_weights, quantize_padded, rel_err_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -54,6 +55,50 @@ def test_noalloc_equals_matmul_two_calls_in_a_row(rt):
             print(f"noalloc type {qtype} N={N} K={K} T={T}", flush=True)
             ya, yb, b0, b1 = both(eng, qtype, N, K, T, Mp, seed=50 + T)
             assert np.array_equal(ya, yb) and b0 == b1
+    finally:
+        eng.close()
+
+
+def _free_device_bytes():
+    """hipMemGetInfo's free bytes, asked of the HIP runtime the library itself runs on."""
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+@pytest.mark.parametrize("qtype,N,K,T,Mp", [(az.Q6_K, 1040, 6144, 12, 16),    # gemv_mm, K shared out: partial sums in the scratch
+                                            (az.Q4_K, 1040, 7168, 7, 16),
+                                            (az.Q4_K, 2176, 5120, 128, 128),  # the short-chunk GEMM's partial tiles
+                                            (az.Q4_K, 264, 1024, 1, 16)])
+def test_noalloc_as_the_first_call_of_a_fresh_engine(rt, qtype, N, K, T, Mp):
+    """No ordinary matmul has run before it on this engine (no kernel object of the form exists yet, no workspace has
+    been touched): the result is held to the oracle, and the device's free memory is what it was before the call."""
+    print(f"noalloc first call type {qtype} N={N} K={K} T={T}", flush=True)
+    eng = az.Engine(Mp, 8192)
+    try:
+        W = make_weights(qtype, N, K, seed=77)
+        w = eng.make_weight(qtype, N, K, W)
+        x = make_acts(T, K, seed=78, outliers=True)
+        xb = az.Runtime.from_numpy(x)
+        rows = Mp if T > 8 else T
+        cb = az.Runtime.alloc(rows * N * 4).fill(0xFFFFFFFF)
+        eng.quantize(xb, K, K, Mp, T)
+        az.Runtime.sync()
+        free0, bytes0 = _free_device_bytes(), az.lib.arcz_device_bytes()
+        eng.matmul_noalloc("first", w, Mp, cb, N, 0, 0)
+        az.Runtime.sync()
+        assert _free_device_bytes() == free0 and az.lib.arcz_device_bytes() == bytes0
+        y = cb.read(np.float32, rows * N).reshape(rows, N)[:T]
+        aq, asc, _ = quantize_padded(x, Mp)
+        ref = orc.matmul_ref(qtype, W, N, K, aq[:T], asc)
+        assert np.isfinite(y).all() and rel_err_rows(y, ref).max() <= 1e-3
+        ca = az.Runtime.alloc(rows * N * 4).fill(0xFFFFFFFF)
+        eng.matmul("plain", w, Mp, ca, N, 0, 0)                 # and the ordinary entry point gives the same bits
+        assert np.array_equal(ca.read(np.uint32, rows * N).reshape(rows, N)[:T], y.view(np.uint32))
+        for b in (ca, cb, xb):
+            b.free()
+        w.free()
     finally:
         eng.close()
 
