@@ -108,7 +108,7 @@ _sig("arcz_iq3xxs_grid", None, _p)
 _sig("arcz_weight_set_softcap", _i, _p, C.c_float)
 _sig("arcz_engine_gemv_gu", _i, _p, _p, _p, _i, _p)
 _sig("arcz_engine_matmul_noalloc", _i, _p, C.c_char_p, _p, _i, _p, _i, _i, _i, _i)
-_sig("arcz_moe_layer_upload", _p, _p, _u32, _p, _p, _p, _i, _i, _i, _i)
+_sig("arcz_moe_layer_upload", _p, _p, _u32, _p, _z, _p, _z, _p, _z, _i, _i, _i, _i)
 _sig("arcz_engine_layer_moe", _i, _p, _p, _p, _i, _p, _i, _i)
 _sig("arcz_engine_moe_route", _i, _p, _p, _p, _i, _i, _i)
 _sig("arcz_engine_layer_moe_sh", _i, _p, _p, _p, _i, _p, _i, _i, _p)
@@ -547,12 +547,8 @@ class Engine:
 
     def make_moe_layer(self, qtype, gate, up, down, NE, NU, E, F):
         g, u, d = (np.ascontiguousarray(a, dtype=np.uint8) for a in (gate, up, down))
-        if qtype in (Q2_0, AR4_128):
-            assert g.size == lib.arcz_relayout_q4_0(qtype, NE * F, E, None, None) and u.size == g.size
-            assert d.size == lib.arcz_relayout_q4_0(qtype, NE * E, F, None, None) and g.size and d.size
-        elif E % 256 == 0 and F % 256 == 0:
-            assert g.size == gguf_bytes(qtype, NE * F, E) and u.size == g.size and d.size == gguf_bytes(qtype, NE * E, F)
-        h = lib.arcz_moe_layer_upload(self.h, qtype, _np_ptr(g), _np_ptr(u), _np_ptr(d), NE, NU, E, F)
+        # (the library checks the byte counts against the type and the shape, padded shapes included)
+        h = lib.arcz_moe_layer_upload(self.h, qtype, _np_ptr(g), g.size, _np_ptr(u), u.size, _np_ptr(d), d.size, NE, NU, E, F)
         if not h:
             raise ArczError(-100, lib.arcz_engine_error().decode())
         Ep, Fp = C.c_int(), C.c_int()

@@ -185,10 +185,20 @@ int arcz_engine_matmul_noalloc(arcz_engine* e, const char* name, arcz_weight* w,
   });
 }
 
-arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, const void* up, const void* down,
-                                      int NE, int NU, int E, int F) {
+arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, size_t gate_bytes, const void* up,
+                                      size_t up_bytes, const void* down, size_t down_bytes, int NE, int NU, int E, int F) {
   arcz_moe_layer* L = new arcz_moe_layer;
   if (guarded([&] {
+        // (the tensors are read for NE x rows x K values of the type: fewer bytes than that would be read past their end)
+        int blk = 0, bb = 0;
+        if (!arcz_ggml_block_info(type, &blk, &bb) || NE <= 0 || E <= 0 || F <= 0 || E % blk || F % blk)
+          throw std::runtime_error("moe layer upload: type " + std::to_string(type) + " with E = " + std::to_string(E) +
+                                   ", F = " + std::to_string(F));
+        const size_t want_gu = (size_t)NE * F * (size_t)(E / blk) * bb, want_d = (size_t)NE * E * (size_t)(F / blk) * bb;
+        if (gate_bytes != want_gu || up_bytes != want_gu || down_bytes != want_d)
+          throw std::runtime_error("moe layer upload: the tensors hold " + std::to_string(gate_bytes) + " / " +
+                                   std::to_string(up_bytes) + " / " + std::to_string(down_bytes) + " bytes, the shape takes " +
+                                   std::to_string(want_gu) + " / " + std::to_string(want_gu) + " / " + std::to_string(want_d));
         L->L = e->e->make_moe_layer(type, (const uint8_t*)gate, (const uint8_t*)up, (const uint8_t*)down, NE, NU, E, F);
       }) != ARCZ_OK) {
     delete L;

@@ -455,7 +455,10 @@ class Engine {
     // (the output head with a logit soft cap and two-pass inputs: the cap applies to the sum of both passes, so both
     //  run without it and softcap_rows caps the sum; zero/engine.h:1081-1110)
     const bool cap = q2mm_ && w.softcap > 0.0f;
-    if (cap && cur_T_ > 8) throw std::logic_error("two-pass output head over more than 8 rows (no softcap there)");
+    // (only the GEMVs of 1-8 tokens cap their results -- the reference's engine never runs a head over more rows,
+    //  zero/engine.h:984-990; a caller of this boundary might, and would get uncapped logits without a word)
+    if (w.softcap > 0.0f && cur_T_ > 8)
+      throw std::logic_error(std::string("matmul ") + name + ": a matrix with a logit soft cap over more than 8 token rows (only the GEMVs cap)");
     q2_nocap_ = cap;
     q2_fuse_ = q2mm_ && !fuse_off && !q2_nofuse_ && cur_T_ <= 4;
     q2_fused_ = false;

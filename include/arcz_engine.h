@@ -124,9 +124,11 @@ int arcz_engine_gemv_gu(arcz_engine* e, arcz_weight* g, arcz_weight* u, int Mp, 
 int arcz_engine_matmul_noalloc(arcz_engine* e, const char* name, arcz_weight* w, int Mp, arcz_mem* C, int ldc, int c_off,
                                int acc, int act32);
 
-/* Expert tensors of one MoE layer: gate, up [NE][F][E] and down [NE][E][F] as GGUF blocks of `type`. */
-arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, const void* up, const void* down,
-                                      int NE, int NU, int E, int F);
+/* Expert tensors of one MoE layer: gate, up [NE][F][E] and down [NE][E][F] as GGUF blocks of `type`, with the bytes the
+ * caller holds of each: a tensor whose byte count is not what its type and shape come to (rows x K / block x block
+ * bytes) is refused before anything is read (NULL + arcz_engine_error()). */
+arcz_moe_layer* arcz_moe_layer_upload(arcz_engine* e, uint32_t type, const void* gate, size_t gate_bytes, const void* up,
+                                      size_t up_bytes, const void* down, size_t down_bytes, int NE, int NU, int E, int F);
 /* Engine::layer_moe (zero/engine_moe.h:8-361, standard experts, no shared expert): x[t] += sum_k w_k expert_k(h[t]) for
  * the T tokens whose quantized h is the current activation chunk; logits: router logits [T][ldl] f32. */
 /* The hidden and FFN widths the layer works with: E and F, or -- where they are not whole superblocks (multiples of

@@ -182,6 +182,27 @@ def test_gemv_softcap_output_head(eng, qtype, N, K, T):
     w.free()
 
 
+@pytest.mark.parametrize("T,Mp", [(9, 16), (12, 16), (16, 16)])
+def test_softcap_head_over_more_than_eight_rows_is_refused(eng, T, Mp):
+    """Only the GEMVs of 1-8 tokens apply a matrix's logit soft cap: a capped matrix over more token rows is an error,
+    not a matmul with uncapped results (one-pass engines too)."""
+    N, K = 264, 512
+    w = eng.make_weight(az.Q4_K, N, K, make_weights(az.Q4_K, N, K, seed=84))
+    w.set_softcap(30.0)
+    xb = az.Runtime.from_numpy(make_acts(T, K, seed=85))
+    eng.quantize(xb, K, K, Mp, T)
+    cb = az.Runtime.alloc(Mp * N * 4).fill(0)
+    with pytest.raises(az.ArczError) as e:
+        eng.matmul("head", w, Mp, cb, N, 0, 0)
+    assert "soft cap" in str(e.value) and not cb.read(np.uint32, Mp * N).any()
+    w.set_softcap(0.0)
+    eng.matmul("head", w, Mp, cb, N, 0, 0)          # without the cap the same call goes through
+    assert np.isfinite(cb.read(np.float32, Mp * N)).all()
+    for b in (xb, cb):
+        b.free()
+    w.free()
+
+
 def _sched(rows, g, wgs):
     """Engine::gemv_sched for one matrix: whole rounds << 10 | rows of the last, shorter pass."""
     full = rows // (g * wgs)

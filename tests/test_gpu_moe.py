@@ -352,3 +352,28 @@ def test_moe_layer_of_widths_that_are_not_whole_superblocks(rt, qtype, NE, NU, E
         xb.free(); lb.free()
     finally:
         eng.close()
+
+
+def test_moe_layer_upload_checks_the_tensors_byte_counts(rt):
+    """An expert tensor with fewer (or more) bytes than its type and shape come to is refused before anything is read,
+    for whole-superblock widths and for the padded ones alike."""
+    for qtype, NE, E, F in [(az.Q4_K, 4, 512, 256), (az.Q8_0, 4, 640, 352)]:
+        eng = az.Engine(16, 1024)   # (an engine takes one expert geometry)
+        try:
+            Wg = make_weights(qtype, NE * F, E, seed=1) if E % 256 == 0 else np.zeros(NE * F * (E // 32) * 34, np.uint8)
+            Wd = make_weights(qtype, NE * E, F, seed=3) if F % 256 == 0 else np.zeros(NE * E * (F // 32) * 34, np.uint8)
+            for bad in ("gate", "up", "down"):
+                g, u, d = Wg, Wg.copy(), Wd
+                if bad == "gate":
+                    g = g[:-34]
+                elif bad == "up":
+                    u = np.concatenate([u, u[:34]])
+                else:
+                    d = d[: d.size // 2]
+                with pytest.raises(az.ArczError) as e:
+                    eng.make_moe_layer(qtype, g, u, d, NE, 2, E, F)
+                assert "bytes" in str(e.value)
+            L = eng.make_moe_layer(qtype, Wg, Wg.copy(), Wd, NE, 2, E, F)
+            L.free()
+        finally:
+            eng.close()
