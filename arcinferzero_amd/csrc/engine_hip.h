@@ -82,6 +82,8 @@ class Engine {
     moe_tmd_ = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
     moe_fuse_off_ = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
     moe_qfuse_off_ = getenv("ARCZ_MOE_QFUSE") && atoi(getenv("ARCZ_MOE_QFUSE")) == 0;
+    q4_wm_ = getenv("ARCZ_Q4_WM") ? atoi(getenv("ARCZ_Q4_WM")) : 2;
+    q4_wm_min_ = getenv("ARCZ_Q4_WM_MIN") ? atoi(getenv("ARCZ_Q4_WM_MIN")) : 2048;
     sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
     sk_ws_ = buf(sk_ws_bytes_);
     // the codebook tables the kernels take as `tabs` (the reference's tabs_, zero/engine_setup.h): IQ3_S's 512 entries
@@ -769,6 +771,7 @@ class Engine {
   int sk_force_ = -1;  // ARCZ_Q4_SPLITK: 0 = never share K out, n >= 2: n pieces, -1 = the rule below
   bool moe_dec_off_ = false, moe_fuse_off_ = false, moe_qfuse_off_ = false;  // ARCZ_MOE_DECODE / _FUSE / _QFUSE = 0
   int moe_dec_max_ = 16, moe_tmd_ = 0;                                      // ARCZ_MOE_DECODE_MAX, ARCZ_MOE_TMD
+  int q4_wm_ = 2, q4_wm_min_ = 2048;                                        // ARCZ_Q4_WM, ARCZ_Q4_WM_MIN
   void gemm_dense(const char* name, const GpuWeight& w0, int Mp, cl_mem C, int ldc, int c_off, int a) {
     const GpuWeight w = gemm_form(name, w0);
     int M = Mp, N = w.N, K = w.K;
@@ -854,7 +857,13 @@ class Engine {
     // form that adds a superblock's block sums up as integers (-DAU=4; ARCZ_Q4_A256=0: the per-32 form on the expansion)
     static const bool a256_off = getenv("ARCZ_Q4_A256") && atoi(getenv("ARCZ_Q4_A256")) == 0;
     const bool au4 = au3 && a256_ && !a256_off;
-    cl_kernel k = q8_small  ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
+    // ... in tiles of 256 tokens x 128 rows, work-groups of 512 threads (ARCZ_Q4_WM=4, read when the engine is made; from
+    // ARCZ_Q4_WM_MIN token rows on).  Not the default: ms per launch at 17408 x 5120 against the 128 x 128 tiles, same
+    // box, 8192 tokens 2.13 / 2.12, 4096 1.107 / 1.06, 2048 0.613 / 0.552 -- one work-group of 8 waves a compute unit
+    // meets at one barrier where two of 4 waves overlap each other's waits, and 256-token tiles fill the last round worse.
+    const bool wm4 = au3 && !au4 && q4_wm_ == 4 && Mp >= q4_wm_min_;
+    cl_kernel k = wm4       ? kernel("gemm", "-DQTYPE=12 -DACT32 -DAU=3 -DWM=4", "gemm")
+                  : q8_small ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
                   : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")
                   : q4_wide ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64", "gemm")
                   : au      ? kernel("gemm", "-DQTYPE=" + std::to_string(w.type) + (au4 ? " -DACT32 -DAU=4" : au3 ? " -DACT32 -DAU=3" : au2 ? " -DACT32 -DAU=2" : " -DACT32 -DAU"), "gemm")
@@ -865,10 +874,11 @@ class Engine {
     static const int sk_sb = getenv("ARCZ_GEMM_SPLIT") ? std::max(0, atoi(getenv("ARCZ_GEMM_SPLIT"))) : 0;
     const int nsb = K / 256, splits = a != 2 && sk_sb > 0 ? (nsb + sk_sb - 1) / sk_sb : 1, rgroup = 1;
     cl_mem unused = nullptr;
-    const int bm = w.type == GGML_Q6_K || q8_small || q4_wide || q4_small ? 64 : 128;  // token rows of a work-group's tile
+    const int bm = wm4 ? 256 : w.type == GGML_Q6_K || q8_small || q4_wide || q4_small ? 64 : 128;  // token rows of a work-group's tile
     const int bn = q4_wide && !q4_small ? 256 : 128;
     const size_t tiles = (size_t)((Mp + bm - 1) / bm) * ((N + bn - 1) / bn);
-    size_t gws[1] = {tiles * 256}, lws[1] = {256};
+    const size_t wg = wm4 ? 512 : 256;
+    size_t gws[1] = {tiles * wg}, lws[1] = {wg};
     if (au) {
       cl_kernel ku = kernel("ops", "", au3 ? "act_usum_bf16" : "act_usum");
       set_args(ku, 0, asc_, absum_, M, au_);

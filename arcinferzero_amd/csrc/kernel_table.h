@@ -73,6 +73,7 @@ static const KernelSpec kKernelTable[] = {
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm", "SPLITK", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", "BN", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "WM", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "AU", "WM", nullptr}, {{nullptr, 0, false}}, 512},
     {"gemm", "gemm", "AU", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "AU", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", "BM", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},

@@ -431,8 +431,11 @@ struct G3ScaleRegs {
 // ready-made: au[K / 32][M] entries (u1 | u2 << 16, u3 | u3 << 16), and behind ws in wsv v[K / 32][N] entries
 // (v1 v1, v2 v2, v3 v3, v1 v2); a lane's token-side operand is the words (x, x, x, y) of its entry, its row-side
 // operand the entry as it lies.  M even, 1 KB and 2 KB past the arrays' ends readable.  A stage is 40 KB.
-template <bool TILES, int QT = QT_Q4_K, int PRE = 0>  // (only the dense form is instantiated: over expert tiles,
-                                                     //  with their short K, the register-staged body measured faster)
+// WM: the work-group's waves along the token rows, two rows of waves each way: 2 = 128 tokens x 128 rows in 4 waves, 4
+// (PRE = 3 only) = 256 tokens x 128 rows in 8 waves of 64 x 64 -- one work-group a compute unit instead of two, the
+// step's weight rows and row-side scale vectors brought into LDS once for 256 tokens instead of once for each 128.
+template <bool TILES, int QT = QT_Q4_K, int PRE = 0, int WM = 2>  // (only the dense form is instantiated: over expert tiles,
+                                                                 //  with their short K, the register-staged body measured faster)
 __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
                                   int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
@@ -448,10 +451,15 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   // PRE = 4: the activations' scales are per 256 (the chunk's asc holds each eight times): a superblock's block sums
   // are added up as integers, sc * I per block in a 24-bit multiply-add, and meet the f32 scales once per superblock
   constexpr bool A256 = PRE == 4;
+  static_assert(WM == 2 || (WM == 4 && PRE == 3), "the 256-token tile is built for the -DAU=3 form");
+  constexpr int BMT = 64 * WM;        // token rows of the tile
+  constexpr int NWI = 4 / WM;         // weight-row DMA instructions a wave and step (16 rows each)
+  constexpr int oWQ = BMT * 128;      // the packed weight rows, behind the int8 token rows
   // the scale vectors of a stage: f32 per block and token / row (2 KB each), or, BF: sa, ws as before, then the min
   // term's operands, 8 bytes per block and token (4 KB) and 16 per block and row (8 KB): a stage of 40 KB
-  constexpr int oSA = G3_SA, oWS = BF ? G3_SA + 2048 : G3_WS, oU = BF ? G3_SA + 4096 : G3_U, oV = BF ? G3_SA + 8192 : G3_V;
-  constexpr int STAGE = BF ? G3_SA + 16384 : Q5 ? G3_STAGE + 2048 : G3_STAGE, QH = G3_STAGE;  // (Q5_K: the fifth bits behind the scale vectors)
+  constexpr int oSA = oWQ + 8192, oWS = BF ? oSA + 16 * BMT : G3_WS, oU = BF ? oWS + 2048 : G3_U, oV = BF ? oU + 32 * BMT : G3_V;
+  constexpr int STAGE = BF ? oV + 8192 : Q5 ? G3_STAGE + 2048 : G3_STAGE, QH = G3_STAGE;  // (Q5_K: the fifth bits behind the scale vectors)
+  static_assert(WM != 2 || (oWQ == G3_WQ && oSA == G3_SA && (!BF || STAGE == G3_SA + 16384)), "the 128-token layout");
   __shared__ alignas(16) uint8_t lds[2 * STAGE];
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // (a scalar: the DMA destinations and bases that follow from it are scalar arithmetic)
@@ -468,15 +476,15 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   // lane / 8 lands at chunk lane % 8, so the lane names source chunk (lane % 8) ^ (R % 8).  Weights: 2 instructions a
   // wave, 16 rows each; row R = (2 wave + i) 16 + lane / 4, source chunk (lane % 4) ^ ((R / 2) % 4).
   // (per-lane parts as 32-bit byte offsets from bases that are the same for the whole wave and advance with the step)
-  uint32_t aoff[4], woff[2];
+  uint32_t aoff[4], woff[NWI];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int R = (wave * 4 + i) * 8 + (lane >> 3);
     aoff[i] = (uint32_t)token_row(R) * (uint32_t)K + 16u * ((lane & 7) ^ (lane >> 3));
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int R = (wave * 2 + i) * 16 + (lane >> 2);
+  for (int i = 0; i < NWI; ++i) {
+    const int R = (wave * NWI + i) * 16 + (lane >> 2);
     const int n = min(n0 + R, N - 1);
     woff[i] = (uint32_t)n * (uint32_t)nsb * 128u + 16u * ((lane & 3) ^ ((lane >> 3) & 3));
   }
@@ -503,17 +511,26 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
   // BF: waves 0 and 1 bring sa (asc), waves 2 and 3 d * sc (the f32 half of wsv), two blocks each as above; then wave w
   // the min term's operands of block w of the step: 128 token entries of 8 bytes (au: one instruction, lane l tokens
   // 2 l, 2 l + 1) and 128 row entries of 16 bytes (behind the f32 half of wsv: two instructions, lane l row 64 i + l)
-  const uint8_t* fbase = wave < 2 ? (const uint8_t*)asc + (size_t)s_begin * 8 * M * 4 : (const uint8_t*)wsv + (size_t)s_begin * 8 * N * 4;
-  const uint32_t fstep = 16u * (uint32_t)(wave < 2 ? M : N);  // (bytes of four blocks' f32 entries)
-  uint32_t foff = wave < 2 ? soff : roff;
+  // (WM = 4: waves 0-3 bring sa of block w for the tile's 256 tokens, lane l the tokens 4 l .. + 3; waves 4 and 5 -- and 6
+  //  and 7 once more, to the same place -- d * sc of blocks (0, 1) and (2, 3))
+  const bool f_tok = WM == 4 ? wave < 4 : wave < 2;
+  const uint8_t* fbase = f_tok ? (const uint8_t*)asc + (size_t)s_begin * 8 * M * 4 : (const uint8_t*)wsv + (size_t)s_begin * 8 * N * 4;
+  const uint32_t fstep = 16u * (uint32_t)(f_tok ? M : N);  // (bytes of four blocks' f32 entries)
+  uint32_t foff = WM == 4 ? (f_tok ? ((uint32_t)wave * (uint32_t)M + (uint32_t)m0 + 4u * lane) * 4u : roff) : (wave < 2 ? soff : roff);
+  const int fdst = WM == 4 ? (f_tok ? oSA + wave * 1024 : oWS + (wave & 1) * 1024) : ((wave < 2 ? oSA : oWS) + (wave & 1) * 1024);
   // A256: wave 1 brings, in the place of sa of blocks 2 and 3, the superblock's d[n] (f32 [K / 256][N] behind the other
   // two parts of wsv), rows n0 + 4 (l % 32) .. + 3
   const uint8_t* dbase = (const uint8_t*)wsv + (size_t)(K >> 5) * N * 20 + (size_t)s_begin * N * 4;
   uint32_t doff = ((uint32_t)n0 + 4u * (lane & 31)) * 4u;
-  const uint8_t* ubase = (const uint8_t*)au + ((size_t)s_begin * 8 + wave) * M * 8;
-  uint32_t uoff = ((uint32_t)m0 + 2u * lane) * 8u;
-  const uint8_t* vbase = (const uint8_t*)wsv + (size_t)(K >> 5) * N * 4 + ((size_t)s_begin * 8 + wave) * N * 16;
-  uint32_t voff = ((uint32_t)n0 + lane) * 16u;
+  // (the min term's operands: WM = 2, wave w brings block w -- 128 token entries in one instruction, 128 row entries in
+  //  two; WM = 4, wave w brings block w / 2: the token entries 128 (w % 2) + 2 l, + 1 and the row entries 64 (w % 2) + l)
+  const int mblk = WM == 4 ? wave >> 1 : wave;
+  const uint8_t* ubase = (const uint8_t*)au + ((size_t)s_begin * 8 + mblk) * M * 8;
+  uint32_t uoff = ((uint32_t)m0 + (WM == 4 ? 128u * (wave & 1) : 0u) + 2u * lane) * 8u;
+  const int udst = WM == 4 ? oU + mblk * 2048 + (wave & 1) * 1024 : oU + wave * 1024;
+  const uint8_t* vbase = (const uint8_t*)wsv + (size_t)(K >> 5) * N * 4 + ((size_t)s_begin * 8 + mblk) * N * 16;
+  uint32_t voff = ((uint32_t)n0 + (WM == 4 ? 64u * (wave & 1) : 0u) + lane) * 16u;
+  const int vdst = WM == 4 ? oV + mblk * 2048 + (wave & 1) * 1024 : oV + wave * 2048;
 
   auto dma_step = [&](int st, int stage) {  // st: half-superblock steps from s_begin
     uint8_t* base = lds + stage * STAGE;
@@ -543,24 +560,24 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
     if (piece < 4) {
       asm volatile("" : "+v"(aoff[piece]));
       g3_dma16(abase + (size_t)st * 128 + aoff[piece], base + (wave * 4 + piece) * 1024);
-    } else if (piece < 6) {
+    } else if (piece < 4 + NWI) {
       asm volatile("" : "+v"(woff[piece - 4]));
-      g3_dma16(wbase + (size_t)st * 64 + woff[piece - 4], base + G3_WQ + (wave * 2 + piece - 4) * 1024);
+      g3_dma16(wbase + (size_t)st * 64 + woff[piece - 4], base + oWQ + (wave * NWI + piece - 4) * 1024);
     } else if constexpr (BF) {
-      if (piece == 6) {
+      if (piece == 4 + NWI) {
         if (A256 && wave == 1) {
           asm volatile("" : "+v"(doff));
           g3_dma16(dbase + (size_t)(st >> 1) * N * 4 + doff, base + oSA + 1024);
         } else {
           asm volatile("" : "+v"(foff));
-          g3_dma16(fbase + (size_t)st * fstep + foff, base + (wave < 2 ? oSA : oWS) + (wave & 1) * 1024);
+          g3_dma16(fbase + (size_t)st * fstep + foff, base + fdst);
         }
-      } else if (piece == 7) {
+      } else if (piece == 5 + NWI) {
         asm volatile("" : "+v"(uoff));
-        g3_dma16(ubase + (size_t)st * 4 * M * 8 + uoff, base + oU + wave * 1024);
-      } else if (piece < 10) {
+        g3_dma16(ubase + (size_t)st * 4 * M * 8 + uoff, base + udst);
+      } else if (piece < 6 + 2 * NWI) {  // (WM = 2: two instructions for the wave's 128 row entries; WM = 4: one for its 64)
         asm volatile("" : "+v"(voff));
-        g3_dma16(vbase + (size_t)st * 4 * N * 16 + voff + (piece - 8) * 1024, base + oV + wave * 2048 + (piece - 8) * 1024);
+        g3_dma16(vbase + (size_t)st * 4 * N * 16 + voff + (piece - 6 - NWI) * 1024, base + vdst + (piece - 6 - NWI) * 1024);
       }
     } else if (piece == 6) {
       asm volatile("" : "+v"(soff));
@@ -615,7 +632,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
 #pragma unroll
   for (int b = 0; b < 4; ++b) oa[b] = (wm * 64 + l32) * 128 + (((2 * b + g) ^ (l32 & 7)) * 16);
 #pragma unroll
-  for (int jj = 0; jj < 2; ++jj) ow[jj] = G3_WQ + (wn * 64 + l32) * 64 + (((2 * jj + g) ^ ((l32 >> 1) & 3)) * 16);
+  for (int jj = 0; jj < 2; ++jj) ow[jj] = oWQ + (wn * 64 + l32) * 64 + (((2 * jj + g) ^ ((l32 >> 1) & 3)) * 16);
 
   v16f res[2][2];
 #pragma unroll
@@ -625,12 +642,13 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
 #pragma unroll
       for (int i = 0; i < 16; ++i) res[ms][ns][i] = 0.0f;
 
+  constexpr int NPIECE = BF ? 6 + 2 * NWI : 10;  // the DMA instructions of a wave and step (the forms below BF: up to 9, Q5_K's included)
   const int steps = 2 * (s_end - s_begin);
   G3ScaleRegs sr;
   if (steps > 0) {
     if constexpr (AU) {
 #pragma unroll
-      for (int p = 0; p < 10; ++p) dma_piece(0, 0, p);
+      for (int p = 0; p < NPIECE; ++p) dma_piece(0, 0, p);
     } else {
       dma_step(0, 0);
     }
@@ -668,7 +686,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
           w16[ns][i] = (b & 1) ? (int)(((uint32_t)wraw[ns][i] >> 4) & 0x0F0F0F0Fu) : (int)((uint32_t)wraw[ns][i] & 0x0F0F0F0Fu);
       }
     };
-    auto ld_sa = [&](int b, int ms) { saop[ms] = ((const float*)(Sb + oSA))[b * 128 + wm * 64 + ms * 32 + l32]; };
+    auto ld_sa = [&](int b, int ms) { saop[ms] = ((const float*)(Sb + oSA))[b * BMT + wm * 64 + ms * 32 + l32]; };
     auto ld_ws = [&](int b) { wsop = ((const float*)(Sb + oWS))[b * 128 + wn * 64 + lane]; };
     auto mfma_p = [&](int ms) {
       v32f zf;
@@ -751,7 +769,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
 #pragma unroll
         for (int ms = 0; ms < 2; ++ms) {
           if constexpr (BF) {  // slots (u1 u2 | u1 u2 | u1 u2 | u3 u3) against the row side's (v1 v1 | v2 v2 | v3 v3 | v1 v2)
-            const uint2 e = ((const uint2*)(Sb + oU))[(b + g) * 128 + wm * 64 + ms * 32 + l32];
+            const uint2 e = ((const uint2*)(Sb + oU))[(b + g) * BMT + wm * 64 + ms * 32 + l32];
             uopb[ms] = v4u{e.x, e.x, e.x, e.y};
           } else {
             uop[ms] = ((const float*)(Sb + oU))[(b + g) * 128 + wm * 64 + ms * 32 + l32];
@@ -789,7 +807,7 @@ __device__ __forceinline__ void gemm3_body(const uint8_t* __restrict__ raw, cons
         }
         if constexpr (AU) {  // the next step's loads, one instruction per phase over the first nine (no branch: the
                              //  last step brings its own stage once more, into the stage nobody reads)
-          if (4 * b + tile < (BF ? 10 : 9)) dma_piece(next ? st + 1 : st, (st + 1) & 1, 4 * b + tile);
+          if (4 * b + tile < (BF ? NPIECE : 9)) dma_piece(next ? st + 1 : st, (st + 1) & 1, 4 * b + tile);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -2213,6 +2231,17 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_AU3(
   const int m0 = tm * BM, n0 = tn * BN;
   gemm3_body<false, QT_Q4_K, 3>(raw, aq, asc, nullptr, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
                                 min(BM, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au, (const float*)wsv);
+}
+// -DAU=3 -DWM=4: the same in tiles of 256 tokens x 128 rows, work-groups of 512 threads (gemm3_body's WM).
+extern "C" __global__ __launch_bounds__(512, 2) void gemm__QTYPE12_ACT321_AU3_WM4(
+    const uint8_t* raw, const uint8_t* au, const signed char* aq, const float* asc, const short* wsv, float* C,
+    int M, int N, int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + 255) / 256, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * 256, n0 = tn * BN;
+  gemm3_body<false, QT_Q4_K, 3, 4>(raw, aq, asc, nullptr, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                                   min(256, M - m0), n0, nullptr, 0, nullptr, 0, (const float*)au, (const float*)wsv);
 }
 // -DAU=4: the -DAU=3 form for chunks whose activation scales are per 256 values (asc holds each eight times): wsv holds
 // the integer sub-block scales as int32 [K / 32][N], the min term's pieces as before, then d as f32 [K / 256][N]

@@ -246,3 +246,24 @@ def test_gemm_ready_made_scale_vectors(rt, qtype, T, Mp, N, K, acc):
         g = c0[:T].astype(np.float64)
         ref = ref * (g / (1.0 + np.exp(-g)))
     assert np.isfinite(y).all() and mixed_err(y, ref) <= TOL
+
+
+@pytest.mark.parametrize("T,Mp,N,K,acc", [(1100, 1104, 392, 512, 0), (1030, 1040, 640, 768, 1), (760, 768, 520, 1024, 2),
+                                          (300, 304, 132, 256, 0), (2050, 2064, 136, 256, 1)])
+def test_gemm_tiles_of_256_tokens(rt, monkeypatch, T, Mp, N, K, acc):
+    """The Q4_K kernel in tiles of 256 tokens x 128 rows, work-groups of 8 waves (ARCZ_Q4_WM=4, which an engine reads
+    when it is made; not the default launch): the same arithmetic in the same order as the 128 x 128 kernel, so the same
+    bits, on chunks whose last tiles are partly empty, with the three epilogues."""
+    print(f"256-token tiles T={T} Mp={Mp} N={N} K={K} acc={acc}", flush=True)
+    W = make_weights(az.Q4_K, N, K, seed=91)
+    x = make_acts(T, K, seed=92, outliers=True)
+    c0 = np.random.default_rng(93).standard_normal((Mp, N)).astype(np.float32)
+    eng = az.Engine(Mp, K)
+    want = run_gemm(eng, az.Q4_K, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
+    eng.close()
+    monkeypatch.setenv("ARCZ_Q4_WM", "4")
+    monkeypatch.setenv("ARCZ_Q4_WM_MIN", "256")
+    eng = az.Engine(Mp, K)
+    y = run_gemm(eng, az.Q4_K, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
+    eng.close()
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
