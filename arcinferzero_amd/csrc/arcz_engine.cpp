@@ -225,8 +225,7 @@ int arcz_moe_layer_set_routing(arcz_engine* e, arcz_moe_layer* L, const float* e
 int arcz_moe_layer_free(arcz_engine* e, arcz_moe_layer* L) {
   if (!L) return ARCZ_OK;
   const int r = guarded([&] {
-    for (int i = 0; i < 3; ++i) e->e->free_weight(L->L.ex[i]);
-    e->e->set_moe_routing(L->L, nullptr, nullptr, 1.0f);
+    e->e->free_moe_layer(L->L);
   });
   delete L;
   return r;

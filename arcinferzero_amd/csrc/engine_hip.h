@@ -82,6 +82,7 @@ class Engine {
     moe_tmd_ = getenv("ARCZ_MOE_TMD") ? atoi(getenv("ARCZ_MOE_TMD")) : 0;
     moe_fuse_off_ = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
     moe_qfuse_off_ = getenv("ARCZ_MOE_QFUSE") && atoi(getenv("ARCZ_MOE_QFUSE")) == 0;
+    moe_pre_ = getenv("ARCZ_MOE_PRE") ? atoi(getenv("ARCZ_MOE_PRE")) != 0 : false;
     q4_wm_ = getenv("ARCZ_Q4_WM") ? atoi(getenv("ARCZ_Q4_WM")) : 2;
     q4_wm_min_ = getenv("ARCZ_Q4_WM_MIN") ? atoi(getenv("ARCZ_Q4_WM_MIN")) : 2048;
     sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
@@ -772,6 +773,7 @@ class Engine {
   bool moe_dec_off_ = false, moe_fuse_off_ = false, moe_qfuse_off_ = false;  // ARCZ_MOE_DECODE / _FUSE / _QFUSE = 0
   int moe_dec_max_ = 16, moe_tmd_ = 0;                                      // ARCZ_MOE_DECODE_MAX, ARCZ_MOE_TMD
   int q4_wm_ = 2, q4_wm_min_ = 2048;                                        // ARCZ_Q4_WM, ARCZ_Q4_WM_MIN
+  bool moe_pre_ = false;                                                    // ARCZ_MOE_PRE
   void gemm_dense(const char* name, const GpuWeight& w0, int Mp, cl_mem C, int ldc, int c_off, int a) {
     const GpuWeight w = gemm_form(name, w0);
     int M = Mp, N = w.N, K = w.K;
@@ -919,6 +921,10 @@ class Engine {
     // a bias (-DROUTE_DS -DRSCALE)
     cl_mem escale = nullptr, ebias = nullptr;
     float rscale = 1.0f;
+    // Q4_K tensors, when the engine was made with ARCZ_MOE_PRE=1: the rows' scale vectors ws | v (q4k_wscales over the
+    // tensor as one matrix of NE * rows: 8 bytes per 32 weights on top of the 18 of the planes), which the tile kernels
+    // of a chunk of many tokens then take by DMA instead of unpacking the 6-bit scales per tile and step
+    cl_mem wsv[3] = {nullptr, nullptr, nullptr};
     bool variant() const { return escale || ebias; }
     std::string route_defs() const {
       if (ebias) {
@@ -940,7 +946,7 @@ class Engine {
   // buffers of the layer (zero/engine_alloc.h:109-159): sized for max_chunk tokens
   cl_mem mids_ = nullptr, mwts_ = nullptr, sgate_ = nullptr, mcount_ = nullptr, moffs_ = nullptr, mcursor_ = nullptr,
          mtiles_ = nullptr, mtstart_ = nullptr, stok_ = nullptr, swt_ = nullptr, minv_ = nullptr, mh_ = nullptr,
-         mhq_ = nullptr, mhsc_ = nullptr, mhbs_ = nullptr, my_ = nullptr;
+         mhq_ = nullptr, mhsc_ = nullptr, mhbs_ = nullptr, my_ = nullptr, mhu_ = nullptr;
   // The pair list is sorted in chunks of moe_tpc_ tokens (at most 512 pairs): counters [chunks][NE]
   int moe_tpc_ = 0;
   int moe_chunks(int T) const { return (T + moe_tpc_ - 1) / moe_tpc_; }
@@ -962,6 +968,7 @@ class Engine {
     mtiles_ = buf((1 + 3 * (S + NE)) * 4); mtstart_ = buf((size_t)(NE + 1) * 4);
     stok_ = buf(S * 4); swt_ = buf(S * 4); minv_ = buf(S * 4);
     mh_ = buf(S * F * 4); mhq_ = buf(S * F); mhsc_ = buf(S * (F / 32) * 4); mhbs_ = buf(S * (F / 16) * 2); my_ = buf(S * E * 4);
+    if (moe_pre_) mhu_ = buf(S * (F / 32) * 4 + 1024);  // (sa * S of the experts' inputs, act_usum over mhsc_ / mhbs_)
     const uint32_t zero = 0;
     CL_CHECK(clEnqueueFillBuffer(cl_.queue, mcount_, &zero, 4, 0, nchunks * NE * 4, 0, nullptr, nullptr));
   }
@@ -1008,7 +1015,30 @@ class Engine {
     L.ex[0] = make_weight(type[0], d[0], arcz_gguf_bytes(type[0], (size_t)NE * Fp, Ep), Fp, Ep, (size_t)NE * Fp);
     L.ex[1] = make_weight(type[1], d[1], arcz_gguf_bytes(type[1], (size_t)NE * Fp, Ep), Fp, Ep, (size_t)NE * Fp);
     L.ex[2] = make_weight(type[2], d[2], arcz_gguf_bytes(type[2], (size_t)NE * Ep, Fp), Ep, Fp, (size_t)NE * Ep);
+    if (moe_pre_ && mhu_)
+      for (int i = 0; i < 3; ++i) {
+        if (L.ex[i].type != GGML_Q4_K) continue;
+        const size_t rows = L.ex[i].rows;
+        const int K = L.ex[i].K, nsb = K / 256;
+        if (rows * (size_t)(K / 32) >= (1ull << 30)) continue;  // (the kernels form these offsets in 32 bits)
+        // (+ 4096: the last expert's last tile reads whole 128-row pieces)
+        L.wsv[i] = buf(rows * (size_t)(K / 32) * 8 + 4096);
+        cl_kernel kw = kernel("ops", "", "q4k_wscales");
+        size_t hdr = planes_q4k(rows, nsb).hdr;
+        int NN = (int)rows, nsb2 = nsb;
+        set_args(kw, 0, L.ex[i].raw, hdr, NN, nsb2, L.wsv[i]);
+        size_t g2[2] = {(rows + 255) / 256 * 256, (size_t)nsb}, l2[2] = {256, 1};
+        run("q4k_wscales", kw, 2, g2, l2);
+      }
     return L;
+  }
+  void free_moe_layer(MoeLayer& L) {
+    for (int i = 0; i < 3; ++i) {
+      free_weight(L.ex[i]);
+      if (L.wsv[i]) release(L.wsv[i]);
+      L.wsv[i] = nullptr;
+    }
+    set_moe_routing(L, nullptr, nullptr, 1.0f);
   }
   MoeLayer make_moe_layer(uint32_t type, const uint8_t* gate, const uint8_t* up, const uint8_t* down, int NE, int NU,
                           int E, int F) {
@@ -1019,18 +1049,24 @@ class Engine {
 
   // routing -> slots grouped by expert -> tiles (zero/engine_moe.h:95-134).  rl: router logits [T][ldl] f32.
   // tm: slots per tile.
-  void moe_route(const MoeLayer& L, cl_mem rl, int ldl, int T, int tm) {
+  // usum (plain routing only): the routing launch also writes au_ = sa * S of the current chunk's rows of K values.
+  void moe_route(const MoeLayer& L, cl_mem rl, int ldl, int T, int tm, bool usum = false) {
     const int NE = L.NE, NU = L.NU, n = T * NU;
     if (T <= 0 || T > max_chunk || ldl < NE || arcz_mem_size(rl) < ((size_t)(T - 1) * ldl + NE) * 4)
       throw std::runtime_error("moe_route: router logits do not fit");
     const std::string defs = "-DNE=" + std::to_string(NE) + " -DNU=" + std::to_string(NU) + " -DTM=" + std::to_string(tm) +
                              " -DNPART=" + std::to_string(moe_tpc_) + " -DNCH=" + std::to_string(moe_chunks(T));
     {
-      cl_kernel k = kernel("moe", defs + L.route_defs(), "moe_route");
+      if (usum && L.variant()) throw std::logic_error("moe_route: the routing variants do not write the sums");
+      cl_kernel k = kernel("moe", defs + (usum ? " -DUSUM=1" : L.route_defs()), "moe_route");
       int NR = ldl, TT = T;
       set_args(k, 0, rl, NR, TT, mids_, mwts_, sgate_, mcount_);
       if (L.escale) set_args(k, 7, L.escale);  // (zero/engine_moe.h:114-115)
       if (L.ebias) set_args(k, 7, L.ebias);
+      if (usum) {
+        int MM = cur_Mp_, nblk = cur_K_ / 32;
+        set_args(k, 7, asc_, absum_, MM, au_, nblk);
+      }
       size_t g1 = (size_t)(T + 3) / 4 * 256, l1 = 256;
       run("moe_route", k, 1, &g1, &l1);
     }
@@ -1052,17 +1088,26 @@ class Engine {
   // The experts of a chunk through the tile GEMM (zero/engine_moe.h:433-470 moe_gemm, without its decode pass: the
   // kernel decodes the raw rows itself): part 0 = gate, then up with the fused SwiGLU into mh_; part 2 = down,
   // routing-weighted, into my_.
-  void moe_gemm(const MoeLayer& L, int part, int Mp, size_t max_tiles) {
+  void moe_gemm(const MoeLayer& L, int part, int Mp, size_t max_tiles, int n_slots = 0) {
     const int E = L.E, F = L.F, NE = L.NE;
     for (int i = part; i < (part == 0 ? 2 : 3); ++i) {
       const int N = i == 2 ? E : F, K = i == 2 ? F : E;
       const GpuWeight wx = gemm_form(i == 2 ? "moe_down" : "moe_gateup", L.ex[i]);
-      cl_kernel k = gemm_kernel(wx.type, true, NE, wx.half_d);
+      const bool pre = i == 2 && L.wsv[2] && n_slots != 0;
+      cl_kernel k = pre ? kernel("gemm", "-DQTYPE=12 -DACT32 -DMOE_TILES -DPRE=1 -DNE=" + std::to_string(NE), "gemm")
+                        : gemm_kernel(wx.type, true, NE, wx.half_d);
       int M = i == 2 ? slots_ : Mp, NN = N, KK = K, ldc = N, acc = i == 1 ? 2 : 0, e0 = 0, e1 = NE, um = i == 2 ? 0 : 1,
           us = i == 2 ? 1 : 0;
       cl_mem unused = nullptr;
+      if (pre && n_slots > 0) {  // sa * S of the n_slots expert inputs (n_slots < 0: the gate / up kernel wrote them)
+        cl_kernel ku = kernel("ops", "", "act_usum");
+        set_args(ku, 0, mhsc_, mhbs_, M, mhu_);
+        size_t g2[2] = {(size_t)(n_slots + 255) / 256 * 256, (size_t)(K / 32)}, l2[2] = {256, 1};
+        run("act_usum", ku, 2, g2, l2);
+      }
       set_args(k, 0, wx.raw, unused, i == 2 ? mhq_ : aq_, i == 2 ? mhsc_ : asc_, i == 2 ? mhbs_ : absum_, i == 2 ? my_ : mh_, M, NN, KK,
                ldc, acc, mtiles_, mtstart_, e0, e1, stok_, um, swt_, us);
+      if (pre) set_args(k, 19, mhu_, L.wsv[2]);
       // (tile work-groups in a multiple of 8: the kernels deal tiles to the XCDs in runs of the expert-sorted list)
       size_t gws[2] = {(size_t)(N + 127) / 128 * 256, (max_tiles + 7) / 8 * 8}, lws[2] = {256, 1};
       run(i == 2 ? "moe_down" : "moe_gateup", k, 2, gws, lws);
@@ -1200,7 +1245,11 @@ class Engine {
       t64 = t64 || L.ex[i].type == GGML_Q4_K || L.ex[i].type == GGML_Q5_K || L.ex[i].type == GGML_Q6_K || L.ex[i].type == GGML_IQ3_S ||
             L.ex[i].type == GGML_Q3_K || L.ex[i].type == GGML_IQ3_XXS;
     const int tm = t64 ? 64 : 128;
-    moe_route(L, rl, ldl, T, tm);
+    // (the ready-made scale vectors: gate and up Q4_K with the quantizing epilogue; the token side's sa * S then comes
+    //  from the routing launch, or from a launch of its own with the routing variants)
+    const bool pre_gu = L.ex[0].type == GGML_Q4_K && L.ex[1].type == GGML_Q4_K && F % 128 == 0 && !moe_qfuse_off_ &&
+                        L.wsv[0] && L.wsv[1];
+    moe_route(L, rl, ldl, T, tm, pre_gu && !L.variant());
     // the tile count is only known on the GPU: launch for the most tiles possible (zero/engine_moe.h:153)
     const size_t max_tiles = (size_t)(n + tm - 1) / tm + std::min(n, L.NE);
     bool quant_fused = false;
@@ -1210,10 +1259,20 @@ class Engine {
       // ... and, when F is whole tiles of 128 rows, the expert inputs' quantization in the same kernel's epilogue
       // (-DQUANT=1: hq / hsc / hbs as moe_quant_sums makes them, bit for bit; ARCZ_MOE_QFUSE=0: the separate launch)
       quant_fused = F % 128 == 0 && !moe_qfuse_off_;
-      cl_kernel k = kernel("gemm", std::string(quant_fused ? "-DQT=12 -DQUANT=1 -DNE=" : "-DQT=12 -DNE=") + std::to_string(L.NE), "moe_gateup_q");
+      const bool pre = pre_gu;
+      cl_kernel k = kernel("gemm", std::string(pre ? "-DQT=12 -DQUANT=1 -DPRE=1 -DNE=" : quant_fused ? "-DQT=12 -DQUANT=1 -DNE=" : "-DQT=12 -DNE=") + std::to_string(L.NE), "moe_gateup_q");
       int FF = F, KK = E, MM = Mp, S = slots_;
       cl_mem tabs = nullptr;
-      if (quant_fused)
+      if (pre && L.variant()) {  // sa * S of the chunk's tokens
+        cl_kernel ku = kernel("ops", "", "act_usum");
+        set_args(ku, 0, asc_, absum_, MM, au_);
+        size_t g2[2] = {(size_t)(Mp + 255) / 256 * 256, (size_t)(E / 32)}, l2[2] = {256, 1};
+        run("act_usum", ku, 2, g2, l2);
+      }
+      if (pre)
+        set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_, S, mhq_, mhsc_, mhbs_,
+                 au_, L.wsv[0], L.wsv[1], L.wsv[2] ? mhu_ : nullptr);
+      else if (quant_fused)
         set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_, S, mhq_, mhsc_, mhbs_);
       else
         set_args(k, 0, L.ex[0].raw, L.ex[1].raw, FF, KK, tabs, aq_, asc_, MM, mtiles_, stok_, mh_, absum_);
@@ -1230,7 +1289,7 @@ class Engine {
       size_t gws[2] = {(size_t)256 * (F / 256), (size_t)(n + 63) / 64}, lws[2] = {256, 1};
       run("moe_quant", k, 2, gws, lws);
     }
-    moe_gemm(L, 2, Mp, max_tiles);
+    moe_gemm(L, 2, Mp, max_tiles, pre_gu ? -1 : n);  // (-1: mhu_ is written already)
     {
       cl_kernel k = kernel("moe", "-DNE=" + std::to_string(L.NE) + " -DNU=" + std::to_string(NU), "moe_combine");
       int EE = E;

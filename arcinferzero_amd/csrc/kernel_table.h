@@ -65,6 +65,9 @@ static const KernelSpec kKernelTable[] = {
     {"decode", "gemv_mt_v", nullptr, "piippppiipiii", {"QT", "GROWS", "TB", nullptr}, {{"SOFTCAP", 0, false}, {nullptr, 0, false}}, 256},
     // ---- gemm
     // (-DHDT / -DHDS / -DHD = 1 or 2: the Q6_K kernels on planes written out from IQ3_XXS or IQ3_S)
+    // (-DPRE=1: the Q4_K tile kernels with the scale vectors ready-made, two more buffers behind the plain form's)
+    {"gemm", "gemm", "PRE", "ppppppiiiiippiipipipp", {"QTYPE", "ACT32", "MOE_TILES", "PRE", nullptr},
+     {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm", "HDT", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", "HDT", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm", "HDS", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", "HDS", nullptr}, {{nullptr, 0, false}}, 256},
@@ -81,9 +84,11 @@ static const KernelSpec kKernelTable[] = {
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm_simple", nullptr, "ppppppiiiiiiiii", {"QTYPE", "ACT32", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "splitk_reduce", nullptr, "pipiiiii", {nullptr}, {{nullptr, 0, false}}, 256},
+    {"gemm", "moe_gateup_q", "PRE", "ppiipppippppippppppp", {"QT", "QUANT", "PRE", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "moe_gateup_q", "QUANT", "ppiipppippppippp", {"QT", "QUANT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "moe_gateup_q", nullptr, "ppiipppipppp", {"QT", nullptr}, {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     // ---- moe
+    {"moe", "moe_route", "USUM", "piippppppipi", {"USUM", nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_route", "ESCALE", "piippppp", {"ESCALE", nullptr}, {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {nullptr, 0, false}}, 256},
     {"moe", "moe_route", "ROUTE_DS", "piippppp", {"ROUTE_DS", nullptr},
      {{"NE", 0, true}, {"NU", 0, true}, {"NPART", 1, false}, {"RSCALE", 0x3F800000, false}, {nullptr, 0, false}}, 256},

@@ -402,6 +402,11 @@ __device__ inline v8bf as_bf16x8(v4u v) { return __builtin_bit_cast(v8bf, v); }
 // the expert tiles' y rows, which moe_combine reads right back: 56 -> 62 us there.)
 __device__ inline void st_stream(float* p, float v) { __builtin_nontemporal_store(v, p); }
 
+// (the 4-byte form: lane l's word lands at base + 4 l -- a gather of one value per lane)
+__device__ inline void g3_dma4(const void* src, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 4, 0, 0);
+}
 __device__ inline void g3_dma16(const void* src, uint8_t* lds_wave_base) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                    (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
@@ -939,7 +944,8 @@ __device__ __forceinline__ bool store_tile64(uint8_t* lds, const v16f (&res)[2],
 // rows only (F a multiple of 128).
 __device__ __forceinline__ void store_tile64_quant(uint8_t* lds, const v16f (&hv)[2], float* __restrict__ H, int F, int m0,
                                                    int rows_valid, int n0, int S, signed char* __restrict__ hq,
-                                                   float* __restrict__ hsc, short* __restrict__ hbs) {
+                                                   float* __restrict__ hsc, short* __restrict__ hbs,
+                                                   float* __restrict__ hu = nullptr) {
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), l32 = lane & 31, g = lane >> 5;
   uint8_t* tl = lds + 256;
   float* lasc = (float*)(lds + 256 + 64 * 528);       // [4][64]
@@ -977,6 +983,9 @@ __device__ __forceinline__ void store_tile64_quant(uint8_t* lds, const v16f (&hv
   {
     const int b = t >> 6, r = t & 63;
     if (r < rows_valid) hsc[((size_t)(n0 >> 5) + b) * S + m0 + r] = lasc[b * 64 + r];
+    // (hu [F/32][S]: scale times the block's sum, what act_usum would make of hsc and hbs, for the down kernel's PRE form)
+    if (hu && r < rows_valid)
+      hu[((size_t)(n0 >> 5) + b) * S + m0 + r] = lasc[b * 64 + r] * (float)((int)lsum[2 * b * 64 + r] + (int)lsum[(2 * b + 1) * 64 + r]);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int hb = b + 4 * i;
@@ -1229,13 +1238,21 @@ struct G4ScaleRegs {
 // TWO = false: tiles of at most 32 slots; the second slot tile, whose scales would all be zero, is left out (half
 // the matrix and vector instructions of a step).
 // QT = Q5_K: as in the 128 x 128 body, a step's fifth bits (16 bytes a row) by one more DMA of the first two waves.
-template <bool TWO = true, int QT = QT_Q4_K>
+// PRE: the four scale vectors of a step come ready-made and go into LDS by DMA like the int8 rows, as in the dense
+// kernel's -DAU=2 form: the token side from asc itself and au[K / 32][M] = sa * S (act_usum), a value per slot gathered
+// by 4-byte DMA (a slot's token is wherever the routing put it); the row side from wsv = ws[K / 32][rows_total] (d * sc)
+// followed by v[K / 32][rows_total] (-(dmin * mn)), made once per tensor when it is uploaded (q4k_wscales: 8 bytes per
+// 32 weights).  The same expressions as the kernel's own preparation, so the same bits; what leaves the step loop is,
+// per thread, four loads, the 6-bit unpack, eight conversions and products, six LDS stores and their wait.
+template <bool TWO = true, int QT = QT_Q4_K, bool PRE = false>
 __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, const signed char* __restrict__ aq,
                                   const float* __restrict__ asc, const short* __restrict__ absum, float* __restrict__ C,
                                   int M, int N, int K, int ldc, int c_off, int accumulate, int s_begin, int s_end,
                                   size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
                                   const int* __restrict__ rowmap, int use_map, const float* __restrict__ rowscale,
-                                  int use_scale) {
+                                  int use_scale, const float* __restrict__ au = nullptr,
+                                  const float* __restrict__ wsv = nullptr) {
+  static_assert(!PRE || QT == QT_Q4_K, "the ready-made scale vectors are built for Q4_K");
   constexpr bool Q5 = QT == QT_Q5_K;
   constexpr int STAGE = Q5 ? G4_STAGE + 2048 : G4_STAGE, QH = G4_STAGE;
   __shared__ alignas(16) uint8_t lds[2 * STAGE];
@@ -1266,6 +1283,14 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
   const bool tok_valid = r_s < rows_valid;
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
+  // PRE: wave w brings sa and sa * S of block w of the step for the 64 slots (lane l: slot l's token), and one of the
+  // four row-side pieces of 1 KB: waves 0 and 1 d * sc of blocks (0, 1) and (2, 3), waves 2 and 3 -(dmin * mn) of the
+  // same -- lane l the rows 4 (l % 32) .. + 3 of block 2 (w % 2) + l / 32
+  uint32_t toff = (uint32_t)token_row(lane) * 4u;
+  const uint8_t* tbase = (const uint8_t*)asc + ((size_t)s_begin * 8 + wave) * M * 4;
+  const uint8_t* ubase = (const uint8_t*)au + ((size_t)s_begin * 8 + wave) * M * 4;
+  const uint8_t* rbase = (const uint8_t*)wsv + ((wave < 2 ? (size_t)0 : (size_t)(K >> 5) * rows_total) + (size_t)s_begin * 8 * rows_total) * 4;
+  uint32_t roff = ((uint32_t)(2 * (wave & 1) + (lane >> 5)) * (uint32_t)rows_total + (uint32_t)row_base + (uint32_t)n0 + 4u * (lane & 31)) * 4u;
 
   auto dma_step = [&](int st, int stage) {
     uint8_t* base = lds + stage * STAGE;
@@ -1279,9 +1304,16 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
       asm volatile("" : "+v"(qoff));
       if (wave < 2) g3_dma16(qbase + (size_t)st * 16 + qoff, base + QH + wave * 1024);
     }
+    if constexpr (PRE) {
+      asm volatile("" : "+v"(toff), "+v"(roff));
+      g3_dma4(tbase + (size_t)st * 4 * M * 4 + toff, base + G4_SA + wave * 256);
+      g3_dma4(ubase + (size_t)st * 4 * M * 4 + toff, base + G4_U + wave * 256);
+      g3_dma16(rbase + (size_t)st * 4 * rows_total * 4 + roff, base + (wave < 2 ? G4_WS : G4_V) + (wave & 1) * 1024);
+    }
   };
   // (loads only: anything computed from them here would make the wave wait for the whole step's traffic)
   auto load_scales = [&](G4ScaleRegs& r, int st) {
+    if constexpr (PRE) return;
     const int blk = s_begin * 8 + st * 4 + b_s;
     r.sa = (asc + (size_t)blk * M)[m_s];
     r.bs[0] = (absum + (size_t)(2 * blk) * M)[m_s];
@@ -1289,6 +1321,7 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
     r.h = *(const uint4*)(raw + pl.hdr + ((row_base + n_s) * nsb + s_begin + (st >> 1)) * 16);
   };
   auto store_scales = [&](const G4ScaleRegs& r, int st, int stage) {
+    if constexpr (PRE) return;
     uint8_t* base = lds + stage * STAGE;
     const float sa = tok_valid ? r.sa : 0.0f;
     ((float*)(base + G4_SA))[b_s * 64 + r_s] = sa;
@@ -1477,14 +1510,19 @@ struct GuScaleRegs {
 
 // GU: the two streams are gate and up of an expert (rows n0.. of both tensors, h = silu(gate) * up); otherwise they are
 // rows n0.. and n0 + 128.. of one matrix and each gets the plain epilogue (a 64 x 256 tile of a dense product).
-template <bool GU, bool QUANT = false>
+// PRE: the scale vectors ready-made, by DMA (gemm4_body's PRE): au[K / 32][M] = sa * S, and per tensor
+// ws[K / 32][rows_total] followed by v[K / 32][rows_total] (wsg for gate's, wsu for up's).
+template <bool GU, bool QUANT = false, bool PRE = false>
 __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
                                     const signed char* __restrict__ aq, const float* __restrict__ asc,
                                     const short* __restrict__ absum, float* __restrict__ H, int M, int N, int K,
                                     size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
                                     const int* __restrict__ rowmap, int ldc, int c_off, int accumulate, int S = 0,
                                     signed char* __restrict__ hq = nullptr, float* __restrict__ hsc = nullptr,
-                                    short* __restrict__ hbs = nullptr) {
+                                    short* __restrict__ hbs = nullptr, const float* __restrict__ au = nullptr,
+                                    const float* __restrict__ wsg = nullptr, const float* __restrict__ wsu = nullptr,
+                                    float* __restrict__ hu = nullptr) {
+  static_assert(!PRE || GU, "the ready-made scale vectors are wired for the gate / up form");
   __shared__ alignas(16) uint8_t lds[2 * GU_STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
@@ -1514,6 +1552,15 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int row_s = t & 127, x_s = wave >> 1;
   const uint8_t* hsrc = (x_s ? ru : rg) + pl.hdr + (row_base + min(nx[x_s] + row_s, N - 1)) * nsb * 16;
+  // PRE: wave w brings sa and sa * S of block w of the step for the 64 slots (lane l: slot l's token), and for stream
+  // w / 2 (gate, up) d * sc and -(dmin * mn) of blocks 2 (w % 2), + 1: lane l the rows 4 (l % 32) .. + 3 of block
+  // 2 (w % 2) + l / 32
+  uint32_t toff = (uint32_t)token_row(lane) * 4u;
+  const uint8_t* tbase = (const uint8_t*)asc + (size_t)wave * M * 4;
+  const uint8_t* ubase = (const uint8_t*)au + (size_t)wave * M * 4;
+  const uint8_t* rbase = (const uint8_t*)((wave >> 1) ? wsu : wsg);
+  const size_t vpart = (size_t)(K >> 5) * rows_total * 4;  // (from a tensor's d * sc to its -(dmin * mn), in bytes)
+  uint32_t roff = ((uint32_t)(2 * (wave & 1) + (lane >> 5)) * (uint32_t)rows_total + (uint32_t)row_base + (uint32_t)n0 + 4u * (lane & 31)) * 4u;
 
   auto dma_step = [&](int st, int stage) {
     uint8_t* base = lds + stage * GU_STAGE;
@@ -1530,8 +1577,17 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
 #pragma unroll
       for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[x][i], base + (x ? GU_WQ1 : GU_WQ0) + (wave * 2 + i) * 1024);
     }
+    if constexpr (PRE) {
+      asm volatile("" : "+v"(toff), "+v"(roff));
+      g3_dma4(tbase + (size_t)st * 4 * M * 4 + toff, base + GU_SA + wave * 256);
+      g3_dma4(ubase + (size_t)st * 4 * M * 4 + toff, base + GU_U + wave * 256);
+      const uint8_t* rb = rbase + (size_t)st * 4 * rows_total * 4 + roff;
+      g3_dma16(rb, base + ((wave >> 1) ? GU_WS1 : GU_WS0) + (wave & 1) * 1024);
+      g3_dma16(rb + vpart, base + ((wave >> 1) ? GU_V1 : GU_V0) + (wave & 1) * 1024);
+    }
   };
   auto load_scales = [&](GuScaleRegs& r, int st) {
+    if constexpr (PRE) return;
     const int blk = st * 4 + b_s;
     r.sa = (asc + (size_t)blk * M)[m_s];
     r.bs[0] = (absum + (size_t)(2 * blk) * M)[m_s];
@@ -1539,6 +1595,7 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
     r.h = *(const uint4*)(hsrc + (size_t)(st >> 1) * 16);
   };
   auto store_scales = [&](const GuScaleRegs& r, int st, int stage) {
+    if constexpr (PRE) return;
     uint8_t* base = lds + stage * GU_STAGE;
     const float sa = tok_valid ? r.sa : 0.0f;
     ((float*)(base + GU_SA))[b_s * 64 + r_s] = sa;
@@ -1685,7 +1742,7 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
         hv[ms][i] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
       }
     if constexpr (QUANT) {
-      store_tile64_quant(lds, hv, H, N, m0, rows_valid, n0, S, hq, hsc, hbs);
+      store_tile64_quant(lds, hv, H, N, m0, rows_valid, n0, S, hq, hsc, hbs, hu);
       return;
     }
     if (store_tile64(lds, hv, H, N, 0, 0, m0, rows_valid, n0, N, nullptr, 0)) return;
@@ -1749,6 +1806,20 @@ extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12_QUANT1(
   const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
   gemm4gu_body<true, true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), chunk * BN,
                            stok, 0, 0, 0, S, hq, hsc, hbs);
+}
+
+// -DQUANT=1 -DPRE=1: the same with the scale vectors ready-made (gemm4gu_body's PRE): au [K/32][M] from act_usum, wsg
+// and wsu the two tensors' ws | v from q4k_wscales (made when the layer is uploaded); hu [F/32][S] (may be null): the
+// expert inputs' sa * S, written by the quantizing epilogue for the down kernel's -DPRE=1 form.
+extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12_QUANT1_PRE1(
+    const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc,
+    int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,
+    short* hbs, const float* au, const float* wsg, const float* wsu, float* hu, int NE) {
+  int ti, chunk;
+  if (!moe_tile_of(tiles[0], gridDim.x, ti, chunk)) return;
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm4gu_body<true, true, true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM),
+                                 chunk * BN, stok, 0, 0, 0, S, hq, hsc, hbs, au, wsg, wsu, hu);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -2267,6 +2338,21 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TI
   const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
   gemm4_body<true>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N, (size_t)e * N, r0,
                    min(nr, G6_BM), chunk * BN, rowmap, use_map, rowscale, use_scale);
+}
+
+// -DPRE=1: the scale vectors ready-made (gemm4_body's PRE): au [K/32][M] from act_usum over the slots' scales and sums,
+// wsv the tensor's ws | v from q4k_wscales (made when the layer is uploaded)
+extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TILES1_PRE1(
+    const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
+    int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
+    int use_map, const float* rowscale, int use_scale, const float* au, const float* wsv, int NE) {
+  int ti, chunk;
+  if (!moe_tile_of(tstart[e1] - tstart[e0], gridDim.x, ti, chunk)) return;
+  ti += tstart[e0];
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm4_body<true, QT_Q4_K, true>(raw, aq, asc, absum, C, M, N, K, ldc, 0, accumulate, 0, K >> 8, (size_t)NE * N,
+                                  (size_t)e * N, r0, min(nr, G6_BM), chunk * BN, rowmap, use_map, rowscale, use_scale, au,
+                                  wsv);
 }
 
 // (Q5_K experts: the same body, one tile of at most 64 slots per work-group)

@@ -113,15 +113,59 @@ def test_moe_small_pass_other_forms(rt, monkeypatch, env, qtype, NE, NU, E, F, T
     _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, 16)
 
 
-@pytest.mark.parametrize("env", [{}, {"ARCZ_MOE_QFUSE": "0"}])
+@pytest.mark.parametrize("env", [{}, {"ARCZ_MOE_QFUSE": "0"}, {"ARCZ_MOE_PRE": "1"}, {"ARCZ_MOE_PRE": "1", "ARCZ_MOE_QFUSE": "0"}])
 @pytest.mark.parametrize("NE,NU,E,F,T,Mp", [(16, 4, 512, 256, 300, 304), (8, 2, 256, 512, 70, 80), (8, 3, 256, 768, 90, 96)])
 def test_moe_tile_pass_quantization_forms(rt, monkeypatch, env, NE, NU, E, F, T, Mp):
     """Q4_K experts, a tile pass: the expert inputs quantized in the gate/up kernel's epilogue (F a multiple of 128, the
-    default) and by the separate launch (ARCZ_MOE_QFUSE=0): the layer checks hold
-    for both, among them hq / hsc / hbs bit for bit what the quantizer makes of the GPU's own h."""
+    default) and by the separate launch (ARCZ_MOE_QFUSE=0), and the tile kernels on ready-made scale vectors
+    (ARCZ_MOE_PRE=1; with ARCZ_MOE_QFUSE=0 only the down kernel, its token side from a launch of its own): the layer
+    checks hold for all, among them hq / hsc / hbs bit for bit what the quantizer makes of the GPU's own h."""
     for k, v in env.items():
         monkeypatch.setenv(k, v)
     _moe_layer_vs_oracle(az.Q4_K, NE, NU, E, F, T, Mp)
+
+
+@pytest.mark.parametrize("variant", [None, "escale"])
+@pytest.mark.parametrize("NE,NU,E,F,T,Mp", [(16, 4, 512, 256, 300, 304), (128, 8, 2048, 768, 520, 528), (8, 2, 256, 512, 17, 32)])
+def test_moe_ready_made_scale_vectors_change_no_bit(rt, monkeypatch, variant, NE, NU, E, F, T, Mp):
+    """ARCZ_MOE_PRE=1 (read when the engine is made): the Q4_K tile kernels take d * sc, -(dmin * mn) and sa * S from
+    buffers made beforehand -- the rows' at upload, the tokens' by the routing launch (by a launch of its own with a
+    routing variant) and by the gate / up kernel's epilogue -- instead of forming them per tile and step.  The same
+    expressions: the layer's output, h, its int8 form and y are the plain engine's, bit for bit."""
+    print(f"moe PRE NE={NE} NU={NU} E={E} F={F} T={T} {variant}", flush=True)
+    Wg, Wu, Wd = (make_weights(az.Q4_K, NE * n, k, seed=s) for n, k, s in ((F, E, 1), (F, E, 2), (E, F, 3)))
+    x = make_acts(T, E, seed=4)
+    logits = np.random.default_rng(5).standard_normal((T, NE)).astype(np.float32)
+    x0 = az.gen_normal(9, (T, E))
+    escale = (0.5 + np.random.default_rng(6).random(NE)).astype(np.float32)
+    got = []
+    for pre in ("0", "1"):
+        monkeypatch.setenv("ARCZ_MOE_PRE", pre)
+        eng = az.Engine(Mp, max(E, F))
+        try:
+            L = eng.make_moe_layer(az.Q4_K, Wg, Wu, Wd, NE, NU, E, F)
+            if variant:
+                eng.set_moe_routing(L, escale=escale)
+            xb, lb = az.Runtime.from_numpy(x), az.Runtime.from_numpy(logits)
+            outs = []
+            for rep in range(2):          # (the second call: on buffers the first has used)
+                ob = az.Runtime.from_numpy(x0)
+                eng.quantize(xb, E, E, Mp, T)
+                eng.layer_moe(L, lb, NE, ob, T, Mp)
+                outs.append(ob.read(np.float32, T * E).copy())
+                ob.free()
+            assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+            S, n = eng.moe_slots, T * NU
+            used = np.sort(eng.moe_buffer("inv").read(np.int32, n))
+            got.append((outs[0], eng.moe_buffer("h").read(np.float32, S * F).reshape(S, F)[used].copy(),
+                        eng.moe_buffer("hq").read(np.int8, S * F).reshape(S, F)[used].copy(),
+                        eng.moe_buffer("y").read(np.float32, S * E).reshape(S, E)[used].copy()))
+            L.free(); xb.free(); lb.free()
+        finally:
+            eng.close()
+    assert np.isfinite(got[0][0]).all() and np.abs(got[0][0] - x0.reshape(-1)).max() > 0
+    for a, b in zip(got[0], got[1]):
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
 
 
 def _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, Mp):
