@@ -83,7 +83,7 @@ class Engine {
     moe_fuse_off_ = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
     moe_qfuse_off_ = getenv("ARCZ_MOE_QFUSE") && atoi(getenv("ARCZ_MOE_QFUSE")) == 0;
     moe_pre_ = getenv("ARCZ_MOE_PRE") ? atoi(getenv("ARCZ_MOE_PRE")) != 0 : false;
-    q4_wm_ = getenv("ARCZ_Q4_WM") ? atoi(getenv("ARCZ_Q4_WM")) : 2;
+    q4_wm_ = getenv("ARCZ_Q4_WM") ? atoi(getenv("ARCZ_Q4_WM")) : 0;
     q4_wm_min_ = getenv("ARCZ_Q4_WM_MIN") ? atoi(getenv("ARCZ_Q4_WM_MIN")) : 2048;
     sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
     sk_ws_ = buf(sk_ws_bytes_);
@@ -772,7 +772,7 @@ class Engine {
   int sk_force_ = -1;  // ARCZ_Q4_SPLITK: 0 = never share K out, n >= 2: n pieces, -1 = the rule below
   bool moe_dec_off_ = false, moe_fuse_off_ = false, moe_qfuse_off_ = false;  // ARCZ_MOE_DECODE / _FUSE / _QFUSE = 0
   int moe_dec_max_ = 16, moe_tmd_ = 0;                                      // ARCZ_MOE_DECODE_MAX, ARCZ_MOE_TMD
-  int q4_wm_ = 2, q4_wm_min_ = 2048;                                        // ARCZ_Q4_WM, ARCZ_Q4_WM_MIN
+  int q4_wm_ = 0, q4_wm_min_ = 2048;                                        // ARCZ_Q4_WM (0: by rule), ARCZ_Q4_WM_MIN (of =4)
   bool moe_pre_ = false;                                                    // ARCZ_MOE_PRE
   void gemm_dense(const char* name, const GpuWeight& w0, int Mp, cl_mem C, int ldc, int c_off, int a) {
     const GpuWeight w = gemm_form(name, w0);
@@ -864,6 +864,38 @@ class Engine {
     // box, 8192 tokens 2.13 / 2.12, 4096 1.107 / 1.06, 2048 0.613 / 0.552 -- one work-group of 8 waves a compute unit
     // meets at one barrier where two of 4 waves overlap each other's waits, and 256-token tiles fill the last round worse.
     const bool wm4 = au3 && !au4 && q4_wm_ == 4 && Mp >= q4_wm_min_;
+    // ... or in tiles of 64 tokens x 128 rows on f32 scale vectors, work-groups of 168 registers, three a compute unit.
+    // In the steady state the smaller tile loses (8192 tokens at 17408 x 5120: 681 against 727 TOP/s: each step's
+    // row-side traffic and scale tiles serve half the products), but a short chunk is a few rounds of work-groups and
+    // smaller ones fill the last round better: ms per launch, 64 x 128 against 128 x 128, at 17408 x 5120: 256 tokens
+    // 0.108 / 0.131, 384 0.142 / 0.131, 768 0.230 / 0.243, 1024 0.290 / 0.302, 1536 0.423 / 0.415, 2048 0.546 / 0.530;
+    // 5120 x 17408 x 1024 0.329 / 0.390; 5120 x 5120 x 1024 0.104 / 0.124, x 2048 0.169 / 0.187.  The rule: at most 2.2
+    // rounds of the large tiles, and not a little over one round of the small ones.  ARCZ_Q4_WM=1 always, =2 never.
+    bool t64 = au2 && !au4 && w.type == GGML_Q4_K && (q4_wm_ == 1 || q4_wm_ == 0);
+    if (t64 && q4_wm_ == 0) {
+      const double cus = (double)arcz_device_cus();
+      const double r128 = (double)((Mp + 127) / 128) * ((N + 127) / 128) / (2.0 * cus);
+      const double r64 = (double)((Mp + 63) / 64) * ((N + 127) / 128) / (3.0 * cus);
+      t64 = r128 <= 2.2 && !(r64 > 1.0 && r64 <= 1.2);
+    }
+    if (t64) {
+      cl_kernel ku = kernel("ops", "", "act_usum");
+      set_args(ku, 0, asc_, absum_, M, au_);
+      size_t g2[2] = {(size_t)(M + 255) / 256 * 256, (size_t)(K / 32)}, l2[2] = {256, 1};
+      run("act_usum", ku, 2, g2, l2);
+      cl_kernel kw = kernel("ops", "", "q4k_wscales");
+      size_t hdr = planes_q4k((size_t)N, K / 256).hdr;
+      int NN = N, nsb2 = K / 256;
+      set_args(kw, 0, w.raw, hdr, NN, nsb2, wsv_);
+      size_t g3[2] = {(size_t)(N + 255) / 256 * 256, (size_t)(K / 256)};
+      run("q4k_wscales", kw, 2, g3, l2);
+      cl_kernel k = kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128 -DPRE64=1", "gemm");
+      int rgroup = 1, s0 = 0, s1 = K / 256;
+      set_args(k, 0, w.raw, au_, aq_, asc_, wsv_, C, M, N, K, ldc, c_off, a, rgroup, s0, s1);
+      size_t gws[1] = {(size_t)((Mp + 63) / 64) * ((N + 127) / 128) * 256}, lws[1] = {256};
+      run(name, k, 1, gws, lws);
+      return;
+    }
     cl_kernel k = wm4       ? kernel("gemm", "-DQTYPE=12 -DACT32 -DAU=3 -DWM=4", "gemm")
                   : q8_small ? kernel("gemm", "-DQTYPE=8 -DACT32 -DBM=64", "gemm")
                   : q4_small ? kernel("gemm", "-DQTYPE=12 -DACT32 -DBM=64 -DBN=128", "gemm")

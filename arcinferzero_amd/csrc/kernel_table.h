@@ -68,6 +68,7 @@ static const KernelSpec kKernelTable[] = {
     // (-DPRE=1: the Q4_K tile kernels with the scale vectors ready-made, two more buffers behind the plain form's)
     {"gemm", "gemm", "PRE", "ppppppiiiiippiipipipp", {"QTYPE", "ACT32", "MOE_TILES", "PRE", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
+    {"gemm", "gemm", "PRE64", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "PRE64", nullptr}, {{nullptr, 0, false}}, 256},
     {"gemm", "gemm", "HDT", "ppppppiiiiippiipipi", {"QTYPE", "ACT32", "MOE_TILES", "HDT", nullptr},
      {{"NE", 0, true}, {nullptr, 0, false}}, 256},
     {"gemm", "gemm", "HDS", "ppppppiiiiiiiii", {"QTYPE", "ACT32", "BM", "BN", "SPLITK", "HDS", nullptr}, {{nullptr, 0, false}}, 256},

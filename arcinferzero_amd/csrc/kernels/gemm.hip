@@ -2080,6 +2080,18 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_BM64_B
   gemm4_body(raw, aq, asc, absum, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0, min(G6_BM, M - m0),
              n0, nullptr, 0, nullptr, 0);
 }
+// -DPRE64=1: the same tiles on ready-made scale vectors (gemm4_body's PRE; the arguments of the -DAU=2 kernel: au in the
+// place of the unused plane pointer, wsv = ws | v in the place of the block sums), three work-groups a compute unit
+extern "C" __global__ __launch_bounds__(256, 3) void gemm__QTYPE12_ACT321_BM64_BN128_PRE641(
+    const uint8_t* raw, const float* au, const signed char* aq, const float* asc, const float* wsv, float* C, int M, int N,
+    int K, int ldc, int c_off, int accumulate, int rgroup, int s_begin, int s_end) {
+  const int mt = (M + G6_BM - 1) / G6_BM, nt = (N + BN - 1) / BN;
+  int tm, tn;
+  tile_of(blockIdx.x, mt, nt, tm, tn);
+  const int m0 = tm * G6_BM, n0 = tn * BN;
+  gemm4_body<true, QT_Q4_K, true>(raw, aq, asc, nullptr, C, M, N, K, ldc, c_off, accumulate, s_begin, s_end, (size_t)N, 0, m0,
+                                  min(G6_BM, M - m0), n0, nullptr, 0, nullptr, 0, au, wsv);
+}
 // The same with K shared out over gridDim.y work-groups per tile (-DSPLITK): work-group (x, y) takes the y-th of
 // gridDim.y even pieces of superblocks [s_begin, s_end) and stores its partial tile in slice y of C, here a workspace
 // [gridDim.y][M][ldc] (c_off and accumulate apply in splitk_reduce, which adds the slices in order).  A chunk of 64
@@ -2341,8 +2353,10 @@ extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TI
 }
 
 // -DPRE=1: the scale vectors ready-made (gemm4_body's PRE): au [K/32][M] from act_usum over the slots' scales and sums,
-// wsv the tensor's ws | v from q4k_wscales (made when the layer is uploaded)
-extern "C" __global__ __launch_bounds__(256, 2) void gemm__QTYPE12_ACT321_MOE_TILES1_PRE1(
+// wsv the tensor's ws | v from q4k_wscales (made when the layer is uploaded).  Without the scale registers the body fits
+// 168 registers, three work-groups a compute unit (one register spilled outside the loop): the down projection of 32768
+// slots x 768 -> 2048 in 0.220 ms against 0.247 with two (the plain form spills six at that size and gains nothing).
+extern "C" __global__ __launch_bounds__(256, 3) void gemm__QTYPE12_ACT321_MOE_TILES1_PRE1(
     const uint8_t* raw, const uint8_t* wh_unused, const signed char* aq, const float* asc, const short* absum, float* C,
     int M, int N, int K, int ldc, int accumulate, const int* tiles, const int* tstart, int e0, int e1, const int* rowmap,
     int use_map, const float* rowscale, int use_scale, const float* au, const float* wsv, int NE) {

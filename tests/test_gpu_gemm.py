@@ -223,13 +223,14 @@ def test_gemm_per_256_scales_integer_sums(rt, T, Mp, N, K, acc):
 @pytest.mark.parametrize("T,Mp,N,K,acc", [(1100, 1104, 392, 512, 0), (1100, 1104, 390, 512, 0), (1030, 1040, 640, 768, 1),
                                           (760, 768, 520, 1024, 2), (1200, 1216, 132, 256, 0),
                                           (2100, 2112, 392, 512, 0), (2050, 2064, 136, 256, 1), (2048, 2048, 256, 768, 2)])
-def test_gemm_ready_made_scale_vectors(rt, qtype, T, Mp, N, K, acc):
+def test_gemm_ready_made_scale_vectors(rt, monkeypatch, qtype, T, Mp, N, K, acc):
     """The 128 x 128 Q4_K / Q5_K kernel whose scale vectors are written by small kernels in front of it (token side: sa and
     sa * S; row side, from 256 token rows on when N is a multiple of 4: d * sc and -(dmin * mn), for Q4_K with the min
     term's factors as bf16 pieces for the matrix instruction) and go into LDS by DMA:
     chunks whose last token tile and last row tile are partly empty, so that the whole-row reads run into the next
     block's entries and past the arrays' ends; the three epilogues.  Against the oracle, and run to run."""
     print(f"ready-made scales {TYPE_NAMES[qtype]} T={T} Mp={Mp} N={N} K={K} acc={acc}", flush=True)
+    monkeypatch.setenv("ARCZ_Q4_WM", "2")   # (the 128 x 128 tiles also where the launch rule would take 64 x 128)
     eng = az.Engine(Mp, K)            # (an engine of exactly this chunk: the arrays end where the chunk ends)
     W = make_weights(qtype, N, K, seed=71)
     x = make_acts(T, K, seed=72, outliers=True)
@@ -258,6 +259,7 @@ def test_gemm_tiles_of_256_tokens(rt, monkeypatch, T, Mp, N, K, acc):
     W = make_weights(az.Q4_K, N, K, seed=91)
     x = make_acts(T, K, seed=92, outliers=True)
     c0 = np.random.default_rng(93).standard_normal((Mp, N)).astype(np.float32)
+    monkeypatch.setenv("ARCZ_Q4_WM", "2")
     eng = az.Engine(Mp, K)
     want = run_gemm(eng, az.Q4_K, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
     eng.close()
@@ -267,3 +269,32 @@ def test_gemm_tiles_of_256_tokens(rt, monkeypatch, T, Mp, N, K, acc):
     y = run_gemm(eng, az.Q4_K, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
     eng.close()
     assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("wm", ["1", "0"])
+@pytest.mark.parametrize("T,Mp,N,K,acc", [(1100, 1104, 392, 512, 0), (1100, 1104, 390, 512, 0), (1030, 1040, 640, 768, 1),
+                                          (760, 768, 520, 1024, 2), (300, 304, 132, 256, 0), (257, 260, 1000, 2048, 0),
+                                          (2050, 2064, 136, 256, 1)])
+def test_gemm_tiles_of_64_tokens_on_ready_made_scales(rt, monkeypatch, wm, T, Mp, N, K, acc):
+    """The Q4_K kernel in tiles of 64 tokens x 128 rows that takes all four scale vectors ready-made -- the launch
+    rule's choice for chunks of a few rounds of work-groups (ARCZ_Q4_WM=0, the default; =1 always, =2 never; read when
+    an engine is made) -- on chunks whose last tiles are partly empty, so that the whole-row reads run into the next
+    block's entries and past the arrays' ends, with the three epilogues.  Against the oracle, and run to run."""
+    print(f"64-token tiles T={T} Mp={Mp} N={N} K={K} acc={acc} ARCZ_Q4_WM={wm}", flush=True)
+    W = make_weights(az.Q4_K, N, K, seed=91)
+    x = make_acts(T, K, seed=92, outliers=True)
+    c0 = np.random.default_rng(93).standard_normal((Mp, N)).astype(np.float32)
+    monkeypatch.setenv("ARCZ_Q4_WM", wm)
+    eng = az.Engine(Mp, K)            # (an engine of exactly this chunk: the arrays end where the chunk ends)
+    y = run_gemm(eng, az.Q4_K, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
+    y2 = run_gemm(eng, az.Q4_K, W, N, K, x, Mp, acc=acc, c_init=c0 if acc else None)[:T]
+    eng.close()
+    assert np.array_equal(y.view(np.uint32), y2.view(np.uint32))
+    aq, asc, _ = quantize_padded(x, Mp)
+    ref = orc.matmul_ref(az.Q4_K, W, N, K, aq[:T], np.ascontiguousarray(asc[:, :T]))
+    if acc == 1:
+        ref = ref + c0[:T]
+    elif acc == 2:
+        g = c0[:T].astype(np.float64)
+        ref = ref * (g / (1.0 + np.exp(-g)))
+    assert np.isfinite(y).all() and mixed_err(y, ref) <= TOL
