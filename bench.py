@@ -21,8 +21,9 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, published
 # HBM bytes one launch of the headline GEMM moves, from two counter runs of this script (FETCH_SIZE x 2.0 KiB read,
-# WRITE_SIZE x 1.0 KiB written, the factors calibrated on the 2 GiB copy in the same runs): 2745.3 MB + 570.4 MB
-GEMM_HBM_BYTES_PER_LAUNCH = 3.313e9
+# WRITE_SIZE x 1.0 KiB written, the factors calibrated on the 2 GiB copy in the same runs): 1,338,862 KiB x 2 = 2742.0 MB
+# read + 557,056 KiB = 570.4 MB written
+GEMM_HBM_BYTES_PER_LAUNCH = 3.312e9
 
 
 def log(*a):
@@ -288,11 +289,21 @@ def bench_gemm_config(az, qtype, N, K, M, launches, seed, W=None):
             "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS}, W
 
 
-def bench_moe(az, launches):
+def bench_moe(az, launches, ready_made=True):
     """The MoE configuration (configs[4] of the benchmark definition): 128 experts, top-8, 4096 tokens, hidden 2048, expert FFN 768, Q4_K; the whole layer
-    (route, sort, gate/up tile GEMM with SwiGLU, expert-input quantization, down tile GEMM, combine) per launch."""
+    (route, sort, gate/up tile GEMM with SwiGLU, expert-input quantization, down tile GEMM, combine) per launch.
+    ready_made=False: an engine made with ARCZ_MOE_PRE=0 (the tile kernels form their scale vectors per tile and step
+    instead of taking them ready-made from 8 more bytes per 32 expert weights)."""
     NE, NU, T, E, F, qt = 128, 8, 4096, 2048, 768, az.Q4_K
-    eng = az.Engine(T, E)
+    before = os.environ.get("ARCZ_MOE_PRE")
+    os.environ["ARCZ_MOE_PRE"] = "1" if ready_made else "0"
+    try:
+        eng = az.Engine(T, E)   # (reads the switch here)
+    finally:
+        if before is None:
+            del os.environ["ARCZ_MOE_PRE"]
+        else:
+            os.environ["ARCZ_MOE_PRE"] = before
     Wg = az.gen_weights(qt, 21, NE * F, E, 0.02)
     Wu = az.gen_weights(qt, 22, NE * F, E, 0.02)
     Wd = az.gen_weights(qt, 23, NE * E, F, 0.02)
@@ -493,7 +504,14 @@ def main():
                                "quantized to int8 per 32 in the step, out 8192x17408 f32 (configs[1] of the benchmark definition)",
                    "M": M, "N": N, "K": K, "step": "quant_rows + gemm"},
         "roofline": {"bound": "mfma", "achieved": pre["kernel_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": pre["kernel_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_HBM_BYTES_PER_LAUNCH,
+                     "frac": pre["kernel_tops"] / PEAK_INT8_TOPS,
+                     # what the vector unit allows whatever the matrix unit does: per 32 x 32 x 32 int8 product (32
+                     # cycles of the matrix unit at the published peak) a lane converts 16 int32 sums and multiplies
+                     # them into 16 f32 accumulators with the block's scale tile: 32 vector instructions x 4 cycles
+                     "ceiling_frac": 0.25,
+                     "ceiling": "per-32 scales: 2 vector instructions (int32 -> f32, fma with the scale tile) per "
+                                "accumulator and block = 128 vector cycles per 32-cycle matrix instruction",
+                     "traffic": GEMM_HBM_BYTES_PER_LAUNCH,
                      "traffic_source": "profiles/bench_hbm_traffic_fetch_write.txt (counter runs of this script; "
                                        "a constant here, not read in this run)",
                      "kernel": "gemm__QTYPE12_ACT321_AU3",
@@ -536,6 +554,8 @@ def main():
         log(f"[bench] Q5_K 17408x5120: {out['other_configs']['Q5_K_17408x5120_T1']} {r5}")
         out["other_configs"]["MoE_128x8_T4096_E2048_F768_Q4_K"] = bench_moe(az, 5)
         log(f"[bench] MoE: {out['other_configs']['MoE_128x8_T4096_E2048_F768_Q4_K']}")
+        out["other_configs"]["MoE_128x8_T4096_E2048_F768_Q4_K_scales_in_kernel"] = bench_moe(az, 5, ready_made=False)
+        log(f"[bench] MoE, ARCZ_MOE_PRE=0: {out['other_configs']['MoE_128x8_T4096_E2048_F768_Q4_K_scales_in_kernel']}")
         out["other_configs"]["MoE_128x8_E2048_F768_Q4_K_decode"] = bench_moe_decode(az, 50)
         log(f"[bench] MoE decode: {out['other_configs']['MoE_128x8_E2048_F768_Q4_K_decode']}")
         out["producers_8192x5120"] = bench_producers(az, M, K)

@@ -113,13 +113,14 @@ def test_moe_small_pass_other_forms(rt, monkeypatch, env, qtype, NE, NU, E, F, T
     _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, 16)
 
 
-@pytest.mark.parametrize("env", [{}, {"ARCZ_MOE_QFUSE": "0"}, {"ARCZ_MOE_PRE": "1"}, {"ARCZ_MOE_PRE": "1", "ARCZ_MOE_QFUSE": "0"}])
+@pytest.mark.parametrize("env", [{}, {"ARCZ_MOE_QFUSE": "0"}, {"ARCZ_MOE_PRE": "0"}, {"ARCZ_MOE_PRE": "0", "ARCZ_MOE_QFUSE": "0"}])
 @pytest.mark.parametrize("NE,NU,E,F,T,Mp", [(16, 4, 512, 256, 300, 304), (8, 2, 256, 512, 70, 80), (8, 3, 256, 768, 90, 96)])
 def test_moe_tile_pass_quantization_forms(rt, monkeypatch, env, NE, NU, E, F, T, Mp):
     """Q4_K experts, a tile pass: the expert inputs quantized in the gate/up kernel's epilogue (F a multiple of 128, the
-    default) and by the separate launch (ARCZ_MOE_QFUSE=0), and the tile kernels on ready-made scale vectors
-    (ARCZ_MOE_PRE=1; with ARCZ_MOE_QFUSE=0 only the down kernel, its token side from a launch of its own): the layer
-    checks hold for all, among them hq / hsc / hbs bit for bit what the quantizer makes of the GPU's own h."""
+    default) and by the separate launch (ARCZ_MOE_QFUSE=0); the tile kernels on ready-made scale vectors (the default;
+    with ARCZ_MOE_QFUSE=0 only the down kernel, its token side from a launch of its own) and forming them per tile and
+    step (ARCZ_MOE_PRE=0): the layer checks hold for all, among them hq / hsc / hbs bit for bit what the quantizer
+    makes of the GPU's own h."""
     for k, v in env.items():
         monkeypatch.setenv(k, v)
     _moe_layer_vs_oracle(az.Q4_K, NE, NU, E, F, T, Mp)
@@ -128,7 +129,7 @@ def test_moe_tile_pass_quantization_forms(rt, monkeypatch, env, NE, NU, E, F, T,
 @pytest.mark.parametrize("variant", [None, "escale"])
 @pytest.mark.parametrize("NE,NU,E,F,T,Mp", [(16, 4, 512, 256, 300, 304), (128, 8, 2048, 768, 520, 528), (8, 2, 256, 512, 17, 32)])
 def test_moe_ready_made_scale_vectors_change_no_bit(rt, monkeypatch, variant, NE, NU, E, F, T, Mp):
-    """ARCZ_MOE_PRE=1 (read when the engine is made): the Q4_K tile kernels take d * sc, -(dmin * mn) and sa * S from
+    """Unless ARCZ_MOE_PRE=0 (read when the engine is made) the Q4_K tile kernels take d * sc, -(dmin * mn) and sa * S from
     buffers made beforehand -- the rows' at upload, the tokens' by the routing launch (by a launch of its own with a
     routing variant) and by the gate / up kernel's epilogue -- instead of forming them per tile and step.  The same
     expressions: the layer's output, h, its int8 form and y are the plain engine's, bit for bit."""
