@@ -1782,6 +1782,179 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
   }
 }
 
+// The gate / up tile on ready-made scale vectors in steps of 64 values (one 32-byte group of a row: two blocks), for
+// three work-groups a compute unit: a stage is 17 KB instead of 34 (the quantizing epilogue's 36 KB set the array), and
+// one scale tile and one pair of product tiles are live at a time -- the streams take turns inside a block -- so that the
+// body stays within 168 registers.  The same products, scale tiles and min-term instructions in the same order per
+// accumulator as gemm4gu_body (block 2s, the min term of blocks 2s and 2s + 1, block 2s + 1): the same bits.
+// Stage: the 64 slots' int8 values [64][64] (16-byte piece c of row r at piece c ^ ((r / 4) % 4)), the two streams'
+// packed rows [128][32] (piece c of row r at c ^ ((r / 8) % 2)), sa and sa * S [2][64], and per stream d * sc and
+// -(dmin * mn) [2][128].  A wave brings per step: a quarter of the slots' rows, its 32 rows of both streams, one of
+// the four token-side vectors (4-byte DMA, a lane a slot) and one of the four row-side vectors.
+#define G5_STAGE 17408
+#define G5_WQ0 4096
+#define G5_WQ1 8192
+#define G5_SA 12288
+#define G5_U 12800
+#define G5_WS0 13312
+#define G5_V0 14336
+#define G5_WS1 15360
+#define G5_V1 16384
+#define G5_LDS 36352  // (store_tile64_quant: 256 + 64 * 528 + 1024 + 1024)
+__device__ __forceinline__ void gemm5gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
+                                             const signed char* __restrict__ aq, const float* __restrict__ asc,
+                                             float* __restrict__ H, int M, int N, int K, size_t rows_total, size_t row_base,
+                                             int m0, int rows_valid, int n0, const int* __restrict__ rowmap, int S,
+                                             signed char* __restrict__ hq, float* __restrict__ hsc, short* __restrict__ hbs,
+                                             const float* __restrict__ au, const float* __restrict__ wsg,
+                                             const float* __restrict__ wsu, float* __restrict__ hu) {
+  static_assert(2 * G5_STAGE <= G5_LDS, "two stages fit the epilogue's array");
+  __shared__ alignas(16) uint8_t lds[G5_LDS];
+  const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int l32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8;
+  const PlanesQ4K pl = planes_q4k(rows_total, nsb);
+  auto token_row = [&](int r) { return rowmap[m0 + (r < rows_valid ? r : 0)]; };  // slots past the tile read its first
+
+  // ---- what this lane fetches each step
+  const int Ra = 16 * wave + (lane >> 2), Rw = 32 * wave + (lane >> 1);
+  uint32_t aoff = (uint32_t)token_row(Ra) * (uint32_t)K + 16u * ((lane & 3) ^ ((Ra >> 2) & 3));
+  uint32_t woff = (uint32_t)min(n0 + Rw, N - 1) * (uint32_t)nsb * 128u + 16u * ((lane & 1) ^ ((Rw >> 3) & 1));
+  const uint8_t* wg0 = rg + pl.qs + row_base * nsb * 128;
+  const uint8_t* wu0 = ru + pl.qs + row_base * nsb * 128;
+  // token side: waves 0, 1 sa of blocks 0, 1; waves 2, 3 sa * S of blocks 0, 1.  Row side: wave w vector w of
+  // (gate d * sc, gate -(dmin * mn), up d * sc, up -(dmin * mn)): lane l the rows 4 (l % 32) .. + 3 of block l / 32
+  uint32_t toff = (uint32_t)token_row(lane) * 4u;
+  const uint8_t* tbase = (const uint8_t*)(wave < 2 ? asc : au) + (size_t)(wave & 1) * M * 4;
+  const uint8_t* rbase = (const uint8_t*)((wave >> 1) ? wsu : wsg) + ((wave & 1) ? (size_t)(K >> 5) * rows_total * 4 : (size_t)0);
+  uint32_t roff = ((uint32_t)(lane >> 5) * (uint32_t)rows_total + (uint32_t)row_base + (uint32_t)n0 + 4u * (lane & 31)) * 4u;
+
+  auto dma_step = [&](int st, int stage) {
+    uint8_t* base = lds + stage * G5_STAGE;
+    asm volatile("" : "+v"(aoff), "+v"(woff), "+v"(toff), "+v"(roff));  // (addresses formed here, not kept over the loop)
+    g3_dma16(aq + (size_t)st * 64 + aoff, base + wave * 1024);
+    g3_dma16(wg0 + (size_t)st * 32 + woff, base + G5_WQ0 + wave * 1024);
+    g3_dma16(wu0 + (size_t)st * 32 + woff, base + G5_WQ1 + wave * 1024);
+    g3_dma4(tbase + (size_t)st * 2 * M * 4 + toff, base + G5_SA + wave * 256);
+    g3_dma16(rbase + (size_t)st * 2 * rows_total * 4 + roff, base + G5_WS0 + wave * 1024);
+  };
+
+  // ---- operand addresses of this lane (bytes from a stage's start)
+  int oa[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) oa[b] = l32 * 64 + (((2 * b + g) ^ ((l32 >> 2) & 3)) * 16);
+  const int ow = (wave * 32 + l32) * 32 + ((g ^ ((l32 >> 3) & 1)) * 16);
+
+  v16f res[2][2];  // [gate / up][slot tile]
+#pragma unroll
+  for (int x = 0; x < 2; ++x)
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) res[x][ms][i] = 0.0f;
+
+  const int steps = 4 * nsb;
+  dma_step(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's part of the stage has landed
+  __syncthreads();
+
+  // TWO = false: a tile of at most 32 slots; its second slot tile, all padding, is left out (half the products and
+  // their sums).  Two loops, chosen once per tile: with the choice as a branch inside one loop the compiler kept both
+  // forms' values live and spilled 20 registers.
+  auto loop = [&](auto two_c) {
+    constexpr bool TWO = decltype(two_c)::value;
+#pragma unroll 1
+    for (int st = 0; st < steps; ++st) {
+      const uint8_t* Sb = lds + (st & 1) * G5_STAGE;
+      if (st + 1 < steps) dma_step(st + 1, (st + 1) & 1);
+      // (every operand of the step is read here, in one go: the reads' latency is paid once a step, not once a block
+      //  and stream)
+      v4i wr[2];
+      wr[0] = *(const v4i*)(Sb + G5_WQ0 + ow);
+      wr[1] = *(const v4i*)(Sb + G5_WQ1 + ow);
+      v4i a16s[2][2];
+      float saops[2], wsops[2][2];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        a16s[b][0] = *(const v4i*)(Sb + oa[b]);
+        if constexpr (TWO) a16s[b][1] = *(const v4i*)(Sb + oa[b] + 32 * 64);
+        saops[b] = ((const float*)(Sb + G5_SA))[b * 64 + lane];
+#pragma unroll
+        for (int x = 0; x < 2; ++x) wsops[b][x] = ((const float*)(Sb + (x ? G5_WS1 : G5_WS0)))[b * 128 + wave * 32 + l32];
+      }
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const v4i* a16 = a16s[b];
+        const float saop = saops[b];
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+          const float wsop = wsops[b][x];
+          v4i w16;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t v = (uint32_t)wr[x][i];
+            w16[i] = (int)(b ? (v >> 4) & 0x0F0F0F0Fu : v & 0x0F0F0F0Fu);
+          }
+          v32f zf;
+#pragma unroll
+          for (int i = 0; i < 32; ++i) zf[i] = 0.0f;
+          v16i z;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) z[i] = 0;
+          const v32f P = __builtin_amdgcn_mfma_f32_32x32x1f32(saop, wsop, zf, 0, 0, 0);
+          const v16i I0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[0], w16, z, 0, 0, 0);
+          v16i I1;
+          if constexpr (TWO) I1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a16[1], w16, z, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int i = 0; i < 16; ++i) res[x][0][i] = __builtin_fmaf((float)I0[i], P[i], res[x][0][i]);
+          if constexpr (TWO) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) res[x][1][i] = __builtin_fmaf((float)I1[i], P[16 + i], res[x][1][i]);
+          }
+          if (b == 0) {  // min term of the step's two blocks: lane half g supplies block g
+            const float vop = ((const float*)(Sb + (x ? G5_V1 : G5_V0)))[g * 128 + wave * 32 + l32];
+#pragma unroll
+            for (int ms = 0; ms < (TWO ? 2 : 1); ++ms) {
+              const float uop = ((const float*)(Sb + G5_U))[g * 64 + ms * 32 + l32];
+              res[x][ms] = __builtin_amdgcn_mfma_f32_32x32x2f32(uop, vop, res[x][ms], 0, 0, 0);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      asm volatile("" : "+v"(res[0][0]), "+v"(res[0][1]), "+v"(res[1][0]), "+v"(res[1][1]));
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+    }
+  };
+  if (rows_valid > 32) loop(std::true_type{});
+  else loop(std::false_type{});
+
+  // ---- epilogue: lane = row n of the stream, accumulator i = slot 8 * (i / 4) + 4 * g + i % 4
+  v16f hv[2];
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float gt = res[0][ms][i];
+      hv[ms][i] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
+    }
+  store_tile64_quant(lds, hv, H, N, m0, rows_valid, n0, S, hq, hsc, hbs, hu);
+}
+
+// -DQUANT=1 -DPRE=2: moe_gateup_q__QT12_QUANT1_PRE1's arguments, the body above
+extern "C" __global__ __launch_bounds__(256, 3) void moe_gateup_q__QT12_QUANT1_PRE2(
+    const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc,
+    int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,
+    short* hbs, const float* au, const float* wsg, const float* wsu, float* hu, int NE) {
+  int ti, chunk;
+  if (!moe_tile_of(tiles[0], gridDim.x, ti, chunk)) return;
+  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
+  gemm5gu_body(rg, ru, aq, asc, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), chunk * BN, stok, S, hq, hsc,
+               hbs, au, wsg, wsu, hu);
+}
+
 // moe_gateup_q: arguments as the reference's (zero/kernels/decode_moe.cl:92-94) -- the two raw expert tensors
 // [NE][F][K], the tile list (tiles of at most 64 slots), stok = the token row of every slot, h [slots][F] -- and, as its
 // extra arguments, the activations' sums per 16 values.  grid (ceil(F / 128) * 256, tile work-groups: the most tiles
