@@ -776,7 +776,9 @@ class Engine {
   int q4_wm_ = 0, q4_wm_min_ = 2048;                                        // ARCZ_Q4_WM (0: by rule), ARCZ_Q4_WM_MIN (of =4)
   bool moe_pre_ = true;                                                     // ARCZ_MOE_PRE (0: off)
   // ARCZ_MOE_GU=1: the gate / up tile kernel on ready-made scale vectors in steps of 128 values, two work-groups a
-  // compute unit; 2 (the default): in steps of 64, three a compute unit (0.401 -> 0.369 ms at 4096 tokens, same bits)
+  // compute unit; 2 (the default): in steps of 64, three a compute unit (0.401 -> 0.369 ms at 4096 tokens, same bits).
+  // (The down projection's kernel in that form -- 121 registers, four work-groups a compute unit -- was built and measured
+  // equal to its three-a-unit form in steps of 128: 0.2275 against 0.2255 ms; not kept.)
   int moe_gu_ = 2;
   void gemm_dense(const char* name, const GpuWeight& w0, int Mp, cl_mem C, int ldc, int c_off, int a) {
     const GpuWeight w = gemm_form(name, w0);
