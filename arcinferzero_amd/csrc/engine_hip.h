@@ -83,7 +83,6 @@ class Engine {
     moe_fuse_off_ = getenv("ARCZ_MOE_FUSE") && atoi(getenv("ARCZ_MOE_FUSE")) == 0;
     moe_qfuse_off_ = getenv("ARCZ_MOE_QFUSE") && atoi(getenv("ARCZ_MOE_QFUSE")) == 0;
     moe_pre_ = getenv("ARCZ_MOE_PRE") ? atoi(getenv("ARCZ_MOE_PRE")) != 0 : true;
-    moe_gu_ = getenv("ARCZ_MOE_GU") ? atoi(getenv("ARCZ_MOE_GU")) : 2;
     q4_wm_ = getenv("ARCZ_Q4_WM") ? atoi(getenv("ARCZ_Q4_WM")) : 0;
     q4_wm_min_ = getenv("ARCZ_Q4_WM_MIN") ? atoi(getenv("ARCZ_Q4_WM_MIN")) : 2048;
     sk_ws_bytes_ = (size_t)2 * (size_t)arcz_device_cus() * 128 * 128 * 4;
@@ -775,11 +774,10 @@ class Engine {
   int moe_dec_max_ = 16, moe_tmd_ = 0;                                      // ARCZ_MOE_DECODE_MAX, ARCZ_MOE_TMD
   int q4_wm_ = 0, q4_wm_min_ = 2048;                                        // ARCZ_Q4_WM (0: by rule), ARCZ_Q4_WM_MIN (of =4)
   bool moe_pre_ = true;                                                     // ARCZ_MOE_PRE (0: off)
-  // ARCZ_MOE_GU=1: the gate / up tile kernel on ready-made scale vectors in steps of 128 values, two work-groups a
-  // compute unit; 2 (the default): in steps of 64, three a compute unit (0.401 -> 0.369 ms at 4096 tokens, same bits).
-  // (The down projection's kernel in that form -- 121 registers, four work-groups a compute unit -- was built and measured
-  // equal to its three-a-unit form in steps of 128: 0.2275 against 0.2255 ms; not kept.)
-  int moe_gu_ = 2;
+  // (The gate / up tile kernel on ready-made scale vectors runs in steps of 64 values, three work-groups a compute unit:
+  // 0.401 -> 0.369 ms at 4096 tokens against the same in steps of 128 at two a unit, same bits.  The down projection's
+  // kernel in that form -- 121 registers, four work-groups a compute unit -- was built and measured equal to its
+  // three-a-unit form in steps of 128: 0.2275 against 0.2255 ms; not kept.)
   void gemm_dense(const char* name, const GpuWeight& w0, int Mp, cl_mem C, int ldc, int c_off, int a) {
     const GpuWeight w = gemm_form(name, w0);
     int M = Mp, N = w.N, K = w.K;
@@ -1301,7 +1299,7 @@ class Engine {
       // (-DQUANT=1: hq / hsc / hbs as moe_quant_sums makes them, bit for bit; ARCZ_MOE_QFUSE=0: the separate launch)
       quant_fused = F % 128 == 0 && !moe_qfuse_off_;
       const bool pre = pre_gu;
-      cl_kernel k = kernel("gemm", std::string(pre ? (moe_gu_ == 2 ? "-DQT=12 -DQUANT=1 -DPRE=2 -DNE=" : "-DQT=12 -DQUANT=1 -DPRE=1 -DNE=") : quant_fused ? "-DQT=12 -DQUANT=1 -DNE=" : "-DQT=12 -DNE=") + std::to_string(L.NE), "moe_gateup_q");
+      cl_kernel k = kernel("gemm", std::string(pre ? "-DQT=12 -DQUANT=1 -DPRE=2 -DNE=" : quant_fused ? "-DQT=12 -DQUANT=1 -DNE=" : "-DQT=12 -DNE=") + std::to_string(L.NE), "moe_gateup_q");
       int FF = F, KK = E, MM = Mp, S = slots_;
       cl_mem tabs = nullptr;
       if (pre && L.variant()) {  // sa * S of the chunk's tokens

@@ -1285,7 +1285,9 @@ __device__ __forceinline__ void gemm4_body(const uint8_t* __restrict__ raw, cons
   const int n_s = min(n0 + (t >> 1), N - 1), p_s = t & 1;
   // PRE: wave w brings sa and sa * S of block w of the step for the 64 slots (lane l: slot l's token), and one of the
   // four row-side pieces of 1 KB: waves 0 and 1 d * sc of blocks (0, 1) and (2, 3), waves 2 and 3 -(dmin * mn) of the
-  // same -- lane l the rows 4 (l % 32) .. + 3 of block 2 (w % 2) + l / 32
+  // same -- lane l the rows 4 (l % 32) .. + 3 of block 2 (w % 2) + l / 32.  (A layout of wsv with a step's vectors of a
+  // row side by side -- one run of 4 KB a step instead of eight pieces of 512 bytes rows_total * 4 bytes apart -- was
+  // built and measured the same: 0.705-0.72 ms a layer either way.)
   uint32_t toff = (uint32_t)token_row(lane) * 4u;
   const uint8_t* tbase = (const uint8_t*)asc + ((size_t)s_begin * 8 + wave) * M * 4;
   const uint8_t* ubase = (const uint8_t*)au + ((size_t)s_begin * 8 + wave) * M * 4;
@@ -1510,19 +1512,14 @@ struct GuScaleRegs {
 
 // GU: the two streams are gate and up of an expert (rows n0.. of both tensors, h = silu(gate) * up); otherwise they are
 // rows n0.. and n0 + 128.. of one matrix and each gets the plain epilogue (a 64 x 256 tile of a dense product).
-// PRE: the scale vectors ready-made, by DMA (gemm4_body's PRE): au[K / 32][M] = sa * S, and per tensor
-// ws[K / 32][rows_total] followed by v[K / 32][rows_total] (wsg for gate's, wsu for up's).
-template <bool GU, bool QUANT = false, bool PRE = false>
+template <bool GU, bool QUANT = false>
 __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, const uint8_t* __restrict__ ru,
                                     const signed char* __restrict__ aq, const float* __restrict__ asc,
                                     const short* __restrict__ absum, float* __restrict__ H, int M, int N, int K,
                                     size_t rows_total, size_t row_base, int m0, int rows_valid, int n0,
                                     const int* __restrict__ rowmap, int ldc, int c_off, int accumulate, int S = 0,
                                     signed char* __restrict__ hq = nullptr, float* __restrict__ hsc = nullptr,
-                                    short* __restrict__ hbs = nullptr, const float* __restrict__ au = nullptr,
-                                    const float* __restrict__ wsg = nullptr, const float* __restrict__ wsu = nullptr,
-                                    float* __restrict__ hu = nullptr) {
-  static_assert(!PRE || GU, "the ready-made scale vectors are wired for the gate / up form");
+                                    short* __restrict__ hbs = nullptr) {
   __shared__ alignas(16) uint8_t lds[2 * GU_STAGE];
   const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int l32 = lane & 31, g = lane >> 5;
@@ -1552,16 +1549,6 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
   const uint32_t m_s = (uint32_t)token_row(r_s);
   const int row_s = t & 127, x_s = wave >> 1;
   const uint8_t* hsrc = (x_s ? ru : rg) + pl.hdr + (row_base + min(nx[x_s] + row_s, N - 1)) * nsb * 16;
-  // PRE: wave w brings sa and sa * S of block w of the step for the 64 slots (lane l: slot l's token), and for stream
-  // w / 2 (gate, up) d * sc and -(dmin * mn) of blocks 2 (w % 2), + 1: lane l the rows 4 (l % 32) .. + 3 of block
-  // 2 (w % 2) + l / 32
-  uint32_t toff = (uint32_t)token_row(lane) * 4u;
-  const uint8_t* tbase = (const uint8_t*)asc + (size_t)wave * M * 4;
-  const uint8_t* ubase = (const uint8_t*)au + (size_t)wave * M * 4;
-  const uint8_t* rbase = (const uint8_t*)((wave >> 1) ? wsu : wsg);
-  const size_t vpart = (size_t)(K >> 5) * rows_total * 4;  // (from a tensor's d * sc to its -(dmin * mn), in bytes)
-  uint32_t roff = ((uint32_t)(2 * (wave & 1) + (lane >> 5)) * (uint32_t)rows_total + (uint32_t)row_base + (uint32_t)n0 + 4u * (lane & 31)) * 4u;
-
   auto dma_step = [&](int st, int stage) {
     uint8_t* base = lds + stage * GU_STAGE;
     const signed char* ab = aq + (size_t)st * 128;
@@ -1577,17 +1564,8 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
 #pragma unroll
       for (int i = 0; i < 2; ++i) g3_dma16(wb + woff[x][i], base + (x ? GU_WQ1 : GU_WQ0) + (wave * 2 + i) * 1024);
     }
-    if constexpr (PRE) {
-      asm volatile("" : "+v"(toff), "+v"(roff));
-      g3_dma4(tbase + (size_t)st * 4 * M * 4 + toff, base + GU_SA + wave * 256);
-      g3_dma4(ubase + (size_t)st * 4 * M * 4 + toff, base + GU_U + wave * 256);
-      const uint8_t* rb = rbase + (size_t)st * 4 * rows_total * 4 + roff;
-      g3_dma16(rb, base + ((wave >> 1) ? GU_WS1 : GU_WS0) + (wave & 1) * 1024);
-      g3_dma16(rb + vpart, base + ((wave >> 1) ? GU_V1 : GU_V0) + (wave & 1) * 1024);
-    }
   };
   auto load_scales = [&](GuScaleRegs& r, int st) {
-    if constexpr (PRE) return;
     const int blk = st * 4 + b_s;
     r.sa = (asc + (size_t)blk * M)[m_s];
     r.bs[0] = (absum + (size_t)(2 * blk) * M)[m_s];
@@ -1595,7 +1573,6 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
     r.h = *(const uint4*)(hsrc + (size_t)(st >> 1) * 16);
   };
   auto store_scales = [&](const GuScaleRegs& r, int st, int stage) {
-    if constexpr (PRE) return;
     uint8_t* base = lds + stage * GU_STAGE;
     const float sa = tok_valid ? r.sa : 0.0f;
     ((float*)(base + GU_SA))[b_s * 64 + r_s] = sa;
@@ -1742,7 +1719,7 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
         hv[ms][i] = res[1][ms][i] * (gt / (1.0f + __expf(-gt)));
       }
     if constexpr (QUANT) {
-      store_tile64_quant(lds, hv, H, N, m0, rows_valid, n0, S, hq, hsc, hbs, hu);
+      store_tile64_quant(lds, hv, H, N, m0, rows_valid, n0, S, hq, hsc, hbs);
       return;
     }
     if (store_tile64(lds, hv, H, N, 0, 0, m0, rows_valid, n0, N, nullptr, 0)) return;
@@ -1783,7 +1760,7 @@ __device__ __forceinline__ void gemm4gu_body(const uint8_t* __restrict__ rg, con
 }
 
 // The gate / up tile on ready-made scale vectors in steps of 64 values (one 32-byte group of a row: two blocks), for
-// three work-groups a compute unit: a stage is 17 KB instead of 34 (the quantizing epilogue's 36 KB set the array), and
+// three work-groups a compute unit: a stage is 17 KB where gemm4gu_body's is 34 (the quantizing epilogue's 36 KB set the array), and
 // one scale tile and one pair of product tiles are live at a time -- the streams take turns inside a block -- so that the
 // body stays within 168 registers.  The same products, scale tiles and min-term instructions in the same order per
 // accumulator as gemm4gu_body (block 2s, the min term of blocks 2s and 2s + 1, block 2s + 1): the same bits.
@@ -1943,7 +1920,9 @@ __device__ __forceinline__ void gemm5gu_body(const uint8_t* __restrict__ rg, con
   store_tile64_quant(lds, hv, H, N, m0, rows_valid, n0, S, hq, hsc, hbs, hu);
 }
 
-// -DQUANT=1 -DPRE=2: moe_gateup_q__QT12_QUANT1_PRE1's arguments, the body above
+// -DQUANT=1 -DPRE=2: the -DQUANT=1 kernel's arguments and, behind them, au [K/32][M] = sa * S of the chunk's tokens, the
+// two tensors' ws | v from q4k_wscales (made when the layer is uploaded), and hu
+// [F/32][S] (may be null): the expert inputs' sa * S, written by the quantizing epilogue for the down kernel's -DPRE=1 form
 extern "C" __global__ __launch_bounds__(256, 3) void moe_gateup_q__QT12_QUANT1_PRE2(
     const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc,
     int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,
@@ -1979,20 +1958,6 @@ extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12_QUANT1(
   const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
   gemm4gu_body<true, true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM), chunk * BN,
                            stok, 0, 0, 0, S, hq, hsc, hbs);
-}
-
-// -DQUANT=1 -DPRE=1: the same with the scale vectors ready-made (gemm4gu_body's PRE): au [K/32][M] from act_usum, wsg
-// and wsu the two tensors' ws | v from q4k_wscales (made when the layer is uploaded); hu [F/32][S] (may be null): the
-// expert inputs' sa * S, written by the quantizing epilogue for the down kernel's -DPRE=1 form.
-extern "C" __global__ __launch_bounds__(256, 2) void moe_gateup_q__QT12_QUANT1_PRE1(
-    const uint8_t* rg, const uint8_t* ru, int F, int K, const uint32_t* tabs, const signed char* aq, const float* asc,
-    int M, const int* tiles, const int* stok, float* h, const short* absum, int S, signed char* hq, float* hsc,
-    short* hbs, const float* au, const float* wsg, const float* wsu, float* hu, int NE) {
-  int ti, chunk;
-  if (!moe_tile_of(tiles[0], gridDim.x, ti, chunk)) return;
-  const int e = tiles[1 + 3 * ti], r0 = tiles[2 + 3 * ti], nr = tiles[3 + 3 * ti];
-  gemm4gu_body<true, true, true>(rg, ru, aq, asc, absum, h, M, F, K, (size_t)NE * F, (size_t)e * F, r0, min(nr, G6_BM),
-                                 chunk * BN, stok, 0, 0, 0, S, hq, hsc, hbs, au, wsg, wsu, hu);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -26,6 +26,8 @@ const char* arcz_engine_error(void);
 /* Engine::Engine + alloc_buffers (zero/engine.h:268, zero/engine_alloc.h:4-41): activation buffers for chunks of up
  * to max_chunk token rows of up to max_k values (aq int8 [M][K], asc f32 [K/32][M], absum int16 [K/16][M]). */
 arcz_engine* arcz_engine_create(int max_chunk, int max_k);
+/* Frees the engine's buffers -- except those that a live recorded launch list still names (arcz_mem_listed): these stay
+ * allocated until the process ends, so that the list never replays on freed memory.  Free lists before their engine. */
 void arcz_engine_destroy(arcz_engine* e);
 
 /* make_weight + upload_padded (zero/engine_load.h:84-130, 157-196): N rows of K values as GGUF blocks of `type`

@@ -113,15 +113,13 @@ def test_moe_small_pass_other_forms(rt, monkeypatch, env, qtype, NE, NU, E, F, T
     _moe_layer_vs_oracle(qtype, NE, NU, E, F, T, 16)
 
 
-@pytest.mark.parametrize("env", [{}, {"ARCZ_MOE_QFUSE": "0"}, {"ARCZ_MOE_PRE": "0"}, {"ARCZ_MOE_PRE": "0", "ARCZ_MOE_QFUSE": "0"},
-                                 {"ARCZ_MOE_GU": "1"}])
+@pytest.mark.parametrize("env", [{}, {"ARCZ_MOE_QFUSE": "0"}, {"ARCZ_MOE_PRE": "0"}, {"ARCZ_MOE_PRE": "0", "ARCZ_MOE_QFUSE": "0"}])
 @pytest.mark.parametrize("NE,NU,E,F,T,Mp", [(16, 4, 512, 256, 300, 304), (8, 2, 256, 512, 70, 80), (8, 3, 256, 768, 90, 96)])
 def test_moe_tile_pass_quantization_forms(rt, monkeypatch, env, NE, NU, E, F, T, Mp):
     """Q4_K experts, a tile pass: the expert inputs quantized in the gate/up kernel's epilogue (F a multiple of 128, the
     default) and by the separate launch (ARCZ_MOE_QFUSE=0); the tile kernels on ready-made scale vectors (the default;
-    with ARCZ_MOE_QFUSE=0 only the down kernel, its token side from a launch of its own; ARCZ_MOE_GU=1: the gate / up
-    kernel in steps of 128 values instead of 64) and forming them per tile and step (ARCZ_MOE_PRE=0): the layer checks
-    hold for all, among them hq / hsc / hbs bit for bit what the quantizer
+    with ARCZ_MOE_QFUSE=0 only the down kernel, its token side from a launch of its own) and forming them per tile and
+    step (ARCZ_MOE_PRE=0): the layer checks hold for all, among them hq / hsc / hbs bit for bit what the quantizer
     makes of the GPU's own h."""
     for k, v in env.items():
         monkeypatch.setenv(k, v)
@@ -134,8 +132,8 @@ def test_moe_ready_made_scale_vectors_change_no_bit(rt, monkeypatch, variant, NE
     """Unless ARCZ_MOE_PRE=0 (read when the engine is made) the Q4_K tile kernels take d * sc, -(dmin * mn) and sa * S from
     buffers made beforehand -- the rows' at upload, the tokens' by the routing launch (by a launch of its own with a
     routing variant) and by the gate / up kernel's epilogue -- instead of forming them per tile and step, the gate / up
-    kernel in steps of 64 values (the default) or of 128 (ARCZ_MOE_GU=1).  The same expressions in the same order: the
-    layer's output, h, its int8 form and y are the plain engine's, bit for bit."""
+    kernel in steps of 64 values instead of 128.  The same expressions in the same order: the layer's output, h, its
+    int8 form and y are the plain engine's, bit for bit."""
     print(f"moe PRE NE={NE} NU={NU} E={E} F={F} T={T} {variant}", flush=True)
     Wg, Wu, Wd = (make_weights(az.Q4_K, NE * n, k, seed=s) for n, k, s in ((F, E, 1), (F, E, 2), (E, F, 3)))
     x = make_acts(T, E, seed=4)
@@ -143,9 +141,8 @@ def test_moe_ready_made_scale_vectors_change_no_bit(rt, monkeypatch, variant, NE
     x0 = az.gen_normal(9, (T, E))
     escale = (0.5 + np.random.default_rng(6).random(NE)).astype(np.float32)
     got = []
-    for pre, gu in (("0", "2"), ("1", "2"), ("1", "1")):
+    for pre in ("0", "1"):
         monkeypatch.setenv("ARCZ_MOE_PRE", pre)
-        monkeypatch.setenv("ARCZ_MOE_GU", gu)
         eng = az.Engine(Mp, max(E, F))
         try:
             L = eng.make_moe_layer(az.Q4_K, Wg, Wu, Wd, NE, NU, E, F)
