@@ -320,7 +320,8 @@ def bench_moe(az, launches, ready_made=True):
     ob = az.Runtime.alloc(T * E * 4).fill(0)
     eng.quantize(xb, E, E, T, T)
     settle(az, lambda: eng.layer_moe(L, lb, NE, ob, T, T))
-    eng.profile(True)
+    # the layer's time: launches back to back between two events, no event pair around each kernel (a pair costs 2.5-3 us,
+    # and the layer is six kernels) ...
     e0 = az.Runtime.event()
     for _ in range(launches):
         eng.layer_moe(L, lb, NE, ob, T, T)
@@ -329,6 +330,11 @@ def bench_moe(az, launches, ready_made=True):
     ms = az.Runtime.elapsed_ms(e0, e1) / launches
     az.Runtime.event_release(e0)
     az.Runtime.event_release(e1)
+    # ... and, right behind them, the same launches again with the per-kernel events, for the parts
+    eng.profile(True)
+    for _ in range(launches):
+        eng.layer_moe(L, lb, NE, ob, T, T)
+    az.Runtime.sync()
     eng.profile_collect()
     parts = {}
     for name in ("moe_route", "moe_scan", "moe_scatter", "moe_gateup", "moe_quant", "moe_down", "moe_combine"):
