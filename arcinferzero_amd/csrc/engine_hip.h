@@ -960,9 +960,8 @@ class Engine {
     // Q4_K tensors (ARCZ_MOE_PRE=0 when the engine is made: none): the rows' scale vectors ws | v (q4k_wscales over the
     // tensor as one matrix of NE * rows: 8 bytes per 32 weights on top of the 18 of the planes), which the tile kernels
     // of a chunk of many tokens then take by DMA instead of unpacking the 6-bit scales per tile and step.  A layer of
-    // 128 experts x 768 x 2048 at 4096 tokens, same process, launches alternating: 0.802 -> 0.735 ms (gate / up 0.430 ->
-    // 0.400, down 0.256 -> 0.209: without the scale registers its kernel fits three work-groups a compute unit) for
-    // 151 MB on top of the layer's 340.
+    // 128 experts x 768 x 2048 at 4096 tokens: 0.80 -> 0.70 ms (gate / up 0.430 -> 0.375, down 0.256 -> 0.212: without
+    // the scale registers both tile kernels fit three work-groups a compute unit) for 151 MB on top of the layer's 340.
     cl_mem wsv[3] = {nullptr, nullptr, nullptr};
     bool variant() const { return escale || ebias; }
     std::string route_defs() const {

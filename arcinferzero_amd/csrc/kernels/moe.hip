@@ -34,9 +34,9 @@ extern "C" __global__ __launch_bounds__(256) void moe_route(const float* __restr
                                                             int NE, int NU, int NPART) {
   moe_route_body(logits, ldl, T, ids, wts, sgate, counts, NE, NU, NPART, RouteVariant());
 }
-// -DUSUM=1: the work-group also writes au[b][t] = sa * S (ops.hip's act_usum: the same expression, the same bits) of
-// its four tokens for the nblk 32-blocks of their quantized rows -- asc [nblk][M], absum [2 nblk][M] -- which the
-// expert tile kernels' -DPRE=1 form takes by DMA; no launch of its own for 12 bytes in and 4 out per token and block.
+// -DUSUM=1: the launch also writes au[b][m] = sa * S (ops.hip's act_usum: the same expression, the same bits) for the nblk
+// 32-blocks of the chunk's M quantized rows -- asc [nblk][M], absum [2 nblk][M] -- which the expert tile kernels' ready-made
+// forms take by DMA; no launch of its own for 12 bytes in and 4 out per token and block.
 extern "C" __global__ __launch_bounds__(256) void moe_route__USUM1(const float* __restrict__ logits, int ldl, int T,
                                                                    int* __restrict__ ids, float* __restrict__ wts,
                                                                    float* __restrict__ sgate, int* __restrict__ counts,
@@ -44,13 +44,16 @@ extern "C" __global__ __launch_bounds__(256) void moe_route__USUM1(const float* 
                                                                    const short* __restrict__ absum, int M,
                                                                    float* __restrict__ au, int nblk, int NE, int NU,
                                                                    int NPART) {
-  {
-    const int m = blockIdx.x * 4 + (threadIdx.x & 3);
-    if (m < T)
-      for (int b = threadIdx.x >> 2; b < nblk; b += 64) {
-        const float sa = asc[(size_t)b * M + m];
-        au[(size_t)b * M + m] = sa * (float)((int)absum[(size_t)(2 * b) * M + m] + (int)absum[(size_t)(2 * b + 1) * M + m]);
-      }
+  {  // (the nblk x M entries dealt to the work-groups in runs of consecutive tokens of a block: whole lines read and written;
+     //  by the work-group's own four tokens the launch took 23 us instead of 11)
+    const size_t total = (size_t)nblk * M;
+    const size_t per = ((total + gridDim.x - 1) / gridDim.x + 255) / 256 * 256;
+    const size_t e1 = min(total, (size_t)(blockIdx.x + 1) * per);
+    for (size_t e = (size_t)blockIdx.x * per + threadIdx.x; e < e1; e += 256) {
+      const size_t b = e / M, m = e - b * M;
+      const float sa = asc[e];
+      au[e] = sa * (float)((int)absum[(2 * b) * M + m] + (int)absum[(2 * b + 1) * M + m]);
+    }
   }
   moe_route_body(logits, ldl, T, ids, wts, sgate, counts, NE, NU, NPART, RouteVariant());
 }
