@@ -1167,7 +1167,7 @@ class Engine {
     // moe_route_small for more) instead of the 64-slot tile GEMMs, which for one token walked K alone in 8 x 6
     // work-groups (128 us a layer at 128 experts x 768 x 2048; ARCZ_MOE_DECODE=0 brings that back).  At 128 x 8 experts
     // the two forms meet at 24 tokens (170 us); 16 tokens take 112 against 137 us (ARCZ_MOE_DECODE_MAX moves the limit).
-    // (the four switches of this function are read at every call, so that a test can set them)
+    // (the switches of this function are read when the engine is made: a test sets them before it makes its engine)
     const bool dec_off = moe_dec_off_;
     const int dec_max = moe_dec_max_;
     if (!dec_off && T <= dec_max && T * NU <= 512) {
