@@ -871,16 +871,22 @@ class Engine {
     // ... or in tiles of 64 tokens x 128 rows on f32 scale vectors, work-groups of 168 registers, three a compute unit.
     // In the steady state the smaller tile loses (8192 tokens at 17408 x 5120: 681 against 727 TOP/s: each step's
     // row-side traffic and scale tiles serve half the products), but a short chunk is a few rounds of work-groups and
-    // smaller ones fill the last round better: ms per launch, 64 x 128 against 128 x 128, at 17408 x 5120: 256 tokens
-    // 0.108 / 0.131, 384 0.142 / 0.131, 768 0.230 / 0.243, 1024 0.290 / 0.302, 1536 0.423 / 0.415, 2048 0.546 / 0.530;
-    // 5120 x 17408 x 1024 0.329 / 0.390; 5120 x 5120 x 1024 0.104 / 0.124, x 2048 0.169 / 0.187.  The rule: at most 2.2
-    // rounds of the large tiles, and not a little over one round of the small ones.  ARCZ_Q4_WM=1 always, =2 never.
+    // which tile fills its last round better decides: ms per launch, 64 x 128 against 128 x 128, at 17408 x 5120: 256
+    // tokens 0.108 / 0.132, 384 0.143 / 0.132, 512 0.170 / 0.193, 768 0.230 / 0.243, 1024 0.291 / 0.302, 2048 0.550 /
+    // 0.535; 5120 x 17408 x 1024 0.331 / 0.393, x 1536 0.449 / 0.406; 8192 x 8192 x 768 0.166 / 0.194, x 1024 0.221 /
+    // 0.204.  The rule prices both in rounds of the large tiles (two work-groups a compute unit): a full round of the
+    // small ones (three a unit, 3/4 of the work at 681 / 727 of the rate) 0.8; a last round in which every compute unit
+    // has at most one large tile 0.5, else 1; at most one small tile 0.30, at most two 0.48, else 0.8 -- fitted to a
+    // sweep of nine matrices x twelve chunk lengths, where it picks the slower tile by more than 2 % in one case of 103.
+    // ARCZ_Q4_WM=1 always, =2 never.
     bool t64 = au2 && !au4 && w.type == GGML_Q4_K && (q4_wm_ == 1 || q4_wm_ == 0);
     if (t64 && q4_wm_ == 0) {
-      const double cus = (double)arcz_device_cus();
-      const double r128 = (double)((Mp + 127) / 128) * ((N + 127) / 128) / (2.0 * cus);
-      const double r64 = (double)((Mp + 63) / 64) * ((N + 127) / 128) / (3.0 * cus);
-      t64 = r128 <= 2.2 && !(r64 > 1.0 && r64 <= 1.2);
+      const size_t cus = (size_t)arcz_device_cus(), nt = (size_t)(N + 127) / 128;
+      const size_t t128 = (size_t)((Mp + 127) / 128) * nt, s128 = 2 * cus, r128 = t128 % s128;
+      const size_t t64n = (size_t)((Mp + 63) / 64) * nt, s64 = 3 * cus, r64 = t64n % s64;
+      const double c128 = (double)(t128 / s128) + (r128 == 0 ? 0.0 : 2 * r128 <= s128 ? 0.5 : 1.0);
+      const double c64 = 0.8 * (double)(t64n / s64) + (r64 == 0 ? 0.0 : 3 * r64 <= s64 ? 0.30 : 3 * r64 <= 2 * s64 ? 0.48 : 0.8);
+      t64 = c64 < 0.97 * c128;
     }
     if (t64) {
       cl_kernel ku = kernel("ops", "", "act_usum");
